@@ -1,0 +1,63 @@
+"""Builds libbreccia_kv.so (HIP, gfx950) in-tree with hipcc.
+
+Usage: ``python -m breccia_amd.build`` or ``breccia_amd.build.build()``.  The library is
+written next to this file so that it travels with the source tree.
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(HERE, "build")
+LIB = os.path.join(HERE, "libbreccia_kv.so")
+
+SOURCES = ["allocator.cpp", "api.hip", "kv_move.hip", "decode_attn.hip"]
+ARCH = "gfx950"
+# Packed-FP32 VALU forms are switched off for every kernel in this library.
+HIP_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def _hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found: cannot build libbreccia_kv.so")
+    return exe
+
+
+def _run(cmd: list[str]) -> None:
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    err = "\n".join(l for l in proc.stderr.splitlines() if noise not in l)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s\n%s" % (" ".join(cmd), proc.stdout, err))
+    if err.strip():
+        sys.stderr.write(err + "\n")
+
+
+def build(verbose: bool = False) -> str:
+    """Compile every source for gfx950 and link the shared library.  Returns its path."""
+    os.makedirs(OBJ, exist_ok=True)
+    hipcc = _hipcc()
+    objs = []
+    for src in SOURCES:
+        obj = os.path.join(OBJ, os.path.splitext(src)[0] + ".o")
+        cmd = [hipcc] + HIP_FLAGS + ["-I", os.path.join(HERE, "..", "include"), "-c",
+                                     os.path.join(CSRC, src), "-o", obj]
+        if verbose:
+            print(" ".join(cmd))
+        _run(cmd)
+        objs.append(obj)
+    cmd = [hipcc, "-shared", "-fPIC", "--offload-arch=" + ARCH] + objs + ["-o", LIB]
+    if verbose:
+        print(" ".join(cmd))
+    _run(cmd)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

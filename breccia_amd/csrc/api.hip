@@ -1,0 +1,910 @@
+// C ABI of libbreccia_kv.so: argument checking, the pool object, block-table
+// mirroring, and the launches.  Every range violation is reported here, on the host,
+// before anything reaches the GPU (the reference's contract, crates/breccia-kernels/
+// src/qsa/mod.rs:1108-1116).
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <unordered_map>
+
+#include "bkv_internal.hpp"
+
+namespace bkv {
+
+static thread_local std::string g_last_error;
+
+void set_error(const std::string& msg) { g_last_error = msg; }
+
+bkv_status fail(bkv_status st, const std::string& msg) {
+    g_last_error = msg;
+    return st;
+}
+
+bkv_status hip_fail(hipError_t e, const char* what) {
+    g_last_error = std::string(what) + " failed: " + hipGetErrorString(e);
+    (void)hipGetLastError();
+    return BKV_ERR_HIP;
+}
+
+static std::string sfmt(const char* f, long long a = 0, long long b = 0, long long c = 0,
+                        long long d = 0) {
+    char buf[320];
+    std::snprintf(buf, sizeof buf, f, a, b, c, d);
+    return buf;
+}
+
+static bkv_status from_alloc(AllocErr e, const std::string& msg) {
+    switch (e) {
+        case AllocErr::Ok: return BKV_OK;
+        case AllocErr::Invalid: return fail(BKV_ERR_INVALID, msg);
+        case AllocErr::Range: return fail(BKV_ERR_RANGE, msg);
+        case AllocErr::NoPages: return fail(BKV_ERR_NO_PAGES, msg);
+        default: return fail(BKV_ERR_STATE, msg);
+    }
+}
+
+static inline hipStream_t S(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---- parameter ring ---------------------------------------------------------------
+bkv_status ring_upload(bkv_pool* p, const void* host_src, size_t bytes, hipStream_t stream,
+                       void** dev_out, int* slot_out) {
+    ParamRing& r = p->ring;
+    if (bytes > ParamRing::kSlotBytes)
+        return fail(BKV_ERR_INVALID, "internal: parameter list larger than a ring slot");
+    const int slot = r.next;
+    r.next = (r.next + 1) % ParamRing::kSlots;
+    if (r.used[slot]) BKV_HIP(hipEventSynchronize(r.ev[slot]));
+    uint8_t* h = r.host + (size_t)slot * ParamRing::kSlotBytes;
+    uint8_t* d = r.dev + (size_t)slot * ParamRing::kSlotBytes;
+    std::memcpy(h, host_src, bytes);
+    BKV_HIP(hipMemcpyAsync(d, h, bytes, hipMemcpyHostToDevice, stream));
+    *dev_out = d;
+    *slot_out = slot;
+    return BKV_OK;
+}
+
+bkv_status ring_done(bkv_pool* p, int slot, hipStream_t stream) {
+    BKV_HIP(hipEventRecord(p->ring.ev[slot], stream));
+    p->ring.used[slot] = true;
+    return BKV_OK;
+}
+
+bkv_status flush_tables(bkv_pool* p, hipStream_t stream) {
+    std::vector<TableUpdate>& pend = p->alloc->pending();
+    if (pend.empty()) return BKV_OK;
+    if (p->host_only) {
+        pend.clear();
+        return BKV_OK;
+    }
+    // Keep the last value per offset: one launch applies updates in no fixed order.
+    std::unordered_map<int32_t, int32_t> last;
+    last.reserve(pend.size() * 2);
+    for (const TableUpdate& u : pend) last[u.offset] = u.value;
+    std::vector<TableUpdate> flat;
+    flat.reserve(last.size());
+    for (const auto& kv : last) flat.push_back(TableUpdate{kv.first, kv.second});
+    const size_t per_slot = ParamRing::kSlotBytes / sizeof(TableUpdate);
+    for (size_t at = 0; at < flat.size(); at += per_slot) {
+        const size_t n = std::min(per_slot, flat.size() - at);
+        void* dev;
+        int slot;
+        bkv_status st = ring_upload(p, flat.data() + at, n * sizeof(TableUpdate), stream, &dev, &slot);
+        if (st != BKV_OK) return st;
+        BKV_HIP(launch_table_scatter(p->table_dev, static_cast<const TableUpdate*>(dev), (int32_t)n,
+                                     stream));
+        st = ring_done(p, slot, stream);
+        if (st != BKV_OK) return st;
+    }
+    pend.clear();
+    return BKV_OK;
+}
+
+StageScope::StageScope(bkv_pool* p, int stage, hipStream_t stream) : p_(p), stream_(stream) {
+    StageTimer& t = p->timer;
+    if (!t.on) return;
+    auto take = [&t]() -> hipEvent_t {
+        if (!t.idle.empty()) {
+            hipEvent_t e = t.idle.back();
+            t.idle.pop_back();
+            return e;
+        }
+        hipEvent_t e = nullptr;
+        if (hipEventCreate(&e) != hipSuccess) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        return e;
+    };
+    hipEvent_t start = take();
+    hipEvent_t stop = take();
+    if (!start || !stop) return;
+    if (hipEventRecord(start, stream) != hipSuccess) {
+        (void)hipGetLastError();
+        return;
+    }
+    stop_ = stop;
+    t.open.push_back(StageTimer::Pair{stage, start, stop});
+}
+
+StageScope::~StageScope() {
+    if (stop_) {
+        if (hipEventRecord(stop_, stream_) != hipSuccess) (void)hipGetLastError();
+    }
+}
+
+bkv_status timer_collect(bkv_pool* p) {
+    StageTimer& t = p->timer;
+    for (const StageTimer::Pair& pr : t.open) {
+        BKV_HIP(hipEventSynchronize(pr.stop));
+        float ms = 0.0f;
+        BKV_HIP(hipEventElapsedTime(&ms, pr.start, pr.stop));
+        t.launches[pr.stage] += 1;
+        t.total_ms[pr.stage] += (double)ms;
+        t.idle.push_back(pr.start);
+        t.idle.push_back(pr.stop);
+    }
+    t.open.clear();
+    return BKV_OK;
+}
+
+static bkv_status need_device(const bkv_pool* p) {
+    if (!p) return fail(BKV_ERR_INVALID, "pool is NULL");
+    if (p->host_only)
+        return fail(BKV_ERR_NO_DEVICE, "this pool was created host-only: it has no device memory");
+    return BKV_OK;
+}
+
+static void destroy_device_side(bkv_pool* p) {
+    if (p->host_only) return;
+    (void)hipDeviceSynchronize();
+    if (p->slab) (void)hipFree(p->slab);
+    if (p->table_dev) (void)hipFree(p->table_dev);
+    if (p->part_o) (void)hipFree(p->part_o);
+    if (p->part_ml) (void)hipFree(p->part_ml);
+    if (p->ring.host) (void)hipHostFree(p->ring.host);
+    if (p->ring.dev) (void)hipFree(p->ring.dev);
+    for (int i = 0; i < ParamRing::kSlots; ++i)
+        if (p->ring.ev[i]) (void)hipEventDestroy(p->ring.ev[i]);
+    for (int i = 0; i < SwapStage::kHalves; ++i) {
+        if (p->stage.dev[i]) (void)hipFree(p->stage.dev[i]);
+        if (p->stage.ev_stream[i]) (void)hipEventDestroy(p->stage.ev_stream[i]);
+        if (p->stage.ev_side[i]) (void)hipEventDestroy(p->stage.ev_side[i]);
+    }
+    if (p->side_done) (void)hipEventDestroy(p->side_done);
+    if (p->side) (void)hipStreamDestroy(p->side);
+    for (const StageTimer::Pair& pr : p->timer.open) {
+        (void)hipEventDestroy(pr.start);
+        (void)hipEventDestroy(pr.stop);
+    }
+    for (hipEvent_t e : p->timer.idle) (void)hipEventDestroy(e);
+}
+
+}  // namespace bkv
+
+using namespace bkv;
+
+extern "C" {
+
+const char* bkv_last_error(void) { return g_last_error.c_str(); }
+const char* bkv_version(void) { return "breccia-kv 0.1 (gfx950)"; }
+
+bkv_status bkv_pool_create(const bkv_pool_desc* d, bkv_pool** out) {
+    if (!d || !out) return fail(BKV_ERR_INVALID, "pool_create: NULL argument");
+    *out = nullptr;
+    if (d->n_layers <= 0 || d->n_pages <= 0 || d->n_kv_head <= 0 || d->max_seqs <= 0 ||
+        d->max_pages_per_seq <= 0)
+        return fail(BKV_ERR_INVALID,
+                    "pool_create: n_layers, n_pages, n_kv_head, max_seqs and max_pages_per_seq "
+                    "must all be > 0 (a cache needs capacity > 0)");
+    if (d->head_dim <= 0 || d->head_dim % 32 != 0 || d->head_dim > 256)
+        return fail(BKV_ERR_INVALID, sfmt("pool_create: head_dim %lld must be a multiple of 32 "
+                                          "(the q8 block) and at most 256", d->head_dim));
+    if (d->page_cells != 16)
+        return fail(BKV_ERR_INVALID, sfmt("pool_create: page_cells %lld; pages are 16 cells",
+                                          d->page_cells));
+    if (d->layout < BKV_LAYOUT_F16 || d->layout > BKV_LAYOUT_I8H)
+        return fail(BKV_ERR_INVALID, sfmt("pool_create: unknown layout %lld", d->layout));
+    if ((int64_t)d->n_pages * d->page_cells >= (int64_t)1 << 31)
+        return fail(BKV_ERR_INVALID, "pool_create: n_pages * page_cells must stay below 2^31");
+
+    bkv_pool* p = new (std::nothrow) bkv_pool();
+    if (!p) return fail(BKV_ERR_NOMEM, "pool_create: out of host memory");
+    p->desc = *d;
+    p->host_only = (d->flags & BKV_POOL_HOST_ONLY) != 0;
+    Geom& g = p->g;
+    g.n_layers = d->n_layers, g.n_pages = d->n_pages, g.n_kv = d->n_kv_head, g.hd = d->head_dim;
+    g.page_cells = d->page_cells, g.layout = d->layout;
+    const uint32_t f16_row = (uint32_t)d->head_dim * 2u;
+    const uint32_t q8v_row = (uint32_t)(d->head_dim / 32) * 36u;
+    const uint32_t i8h_row = (uint32_t)d->head_dim + (uint32_t)(d->head_dim / 32) * 2u;
+    g.k_row_bytes = d->layout == BKV_LAYOUT_I8H ? i8h_row : f16_row;
+    g.v_row_bytes = d->layout == BKV_LAYOUT_F16 ? f16_row
+                    : d->layout == BKV_LAYOUT_Q8V ? q8v_row : i8h_row;
+    const uint64_t rows_per_page = (uint64_t)d->n_kv_head * (uint64_t)d->page_cells;
+    g.k_page_bytes = rows_per_page * g.k_row_bytes;
+    g.v_page_bytes = rows_per_page * g.v_row_bytes;
+    g.k_pool_bytes = g.k_page_bytes * (uint64_t)d->n_pages;
+    g.v_pool_bytes = g.v_page_bytes * (uint64_t)d->n_pages;
+    try {
+        p->alloc.reset(new PageAllocator(d->n_pages, d->page_cells, d->max_seqs,
+                                         d->max_pages_per_seq));
+    } catch (const std::bad_alloc&) {
+        delete p;
+        return fail(BKV_ERR_NOMEM, "pool_create: out of host memory for the block tables");
+    }
+    if (p->host_only) {
+        *out = p;
+        return BKV_OK;
+    }
+
+    auto bail = [&](bkv_status st) {
+        const std::string keep = g_last_error;
+        destroy_device_side(p);
+        delete p;
+        g_last_error = keep;
+        return st;
+    };
+#define BKV_TRY(call)                                                        \
+    do {                                                                     \
+        hipError_t e__ = (call);                                             \
+        if (e__ != hipSuccess) return bail(hip_fail(e__, #call));            \
+    } while (0)
+
+    int n_dev = 0;
+    if (hipGetDeviceCount(&n_dev) != hipSuccess || n_dev <= 0) {
+        (void)hipGetLastError();
+        p->host_only = true;  // nothing device-side to tear down
+        delete p;
+        return fail(BKV_ERR_NO_DEVICE, "pool_create: no HIP device is visible");
+    }
+    BKV_TRY(hipGetDevice(&p->device));
+    hipDeviceProp_t prop;
+    BKV_TRY(hipGetDeviceProperties(&prop, p->device));
+    p->n_cu = prop.multiProcessorCount;
+
+    const uint64_t layer_bytes = g.k_pool_bytes + g.v_pool_bytes;
+    BKV_TRY(hipMalloc(reinterpret_cast<void**>(&p->slab), layer_bytes * (uint64_t)d->n_layers));
+    for (int l = 0; l < d->n_layers; ++l) {
+        p->k_layer.push_back(p->slab + (uint64_t)l * layer_bytes);
+        p->v_layer.push_back(p->slab + (uint64_t)l * layer_bytes + g.k_pool_bytes);
+    }
+    BKV_TRY(launch_fill(p->slab, layer_bytes * (uint64_t)d->n_layers, 0u, nullptr));
+    const uint64_t table_bytes = (uint64_t)d->max_seqs * (uint64_t)d->max_pages_per_seq * 4u;
+    BKV_TRY(hipMalloc(reinterpret_cast<void**>(&p->table_dev), (table_bytes + 15u) & ~15ull));
+    BKV_TRY(launch_fill(p->table_dev, (table_bytes + 15u) & ~15ull, 0xffffffffu, nullptr));
+
+    p->max_wgs = 4096;
+    BKV_TRY(hipMalloc(reinterpret_cast<void**>(&p->part_o), (uint64_t)p->max_wgs * 8u * 256u * 4u));
+    BKV_TRY(hipMalloc(reinterpret_cast<void**>(&p->part_ml), (uint64_t)p->max_wgs * 8u * 2u * 4u));
+
+    BKV_TRY(hipHostMalloc(reinterpret_cast<void**>(&p->ring.host),
+                          ParamRing::kSlots * ParamRing::kSlotBytes, hipHostMallocDefault));
+    BKV_TRY(hipMalloc(reinterpret_cast<void**>(&p->ring.dev),
+                      ParamRing::kSlots * ParamRing::kSlotBytes));
+    for (int i = 0; i < ParamRing::kSlots; ++i)
+        BKV_TRY(hipEventCreateWithFlags(&p->ring.ev[i], hipEventDisableTiming));
+
+    const uint64_t swap_page = (g.k_page_bytes + g.v_page_bytes) * (uint64_t)d->n_layers;
+    p->stage.bytes = std::max<uint64_t>(32ull << 20, 4 * swap_page);
+    for (int i = 0; i < SwapStage::kHalves; ++i) {
+        BKV_TRY(hipMalloc(reinterpret_cast<void**>(&p->stage.dev[i]), p->stage.bytes));
+        BKV_TRY(hipEventCreateWithFlags(&p->stage.ev_stream[i], hipEventDisableTiming));
+        BKV_TRY(hipEventCreateWithFlags(&p->stage.ev_side[i], hipEventDisableTiming));
+    }
+    BKV_TRY(hipStreamCreateWithFlags(&p->side, hipStreamNonBlocking));
+    BKV_TRY(hipEventCreateWithFlags(&p->side_done, hipEventDisableTiming));
+    BKV_TRY(hipDeviceSynchronize());
+#undef BKV_TRY
+    *out = p;
+    return BKV_OK;
+}
+
+bkv_status bkv_pool_destroy(bkv_pool* p) {
+    if (!p) return fail(BKV_ERR_INVALID, "pool_destroy: NULL pool");
+    destroy_device_side(p);
+    delete p;
+    return BKV_OK;
+}
+
+bkv_status bkv_pool_reset(bkv_pool* p, void* stream) {
+    if (!p) return fail(BKV_ERR_INVALID, "pool_reset: NULL pool");
+    p->alloc->reset();
+    if (p->host_only) {
+        p->alloc->pending().clear();
+        return BKV_OK;
+    }
+    const uint64_t layer_bytes = p->g.k_pool_bytes + p->g.v_pool_bytes;
+    BKV_HIP(launch_fill(p->slab, layer_bytes * (uint64_t)p->g.n_layers, 0u, S(stream)));
+    return flush_tables(p, S(stream));
+}
+
+bkv_status bkv_pool_get_desc(const bkv_pool* p, bkv_pool_desc* out) {
+    if (!p || !out) return fail(BKV_ERR_INVALID, "pool_get_desc: NULL argument");
+    *out = p->desc;
+    return BKV_OK;
+}
+
+uint64_t bkv_pool_bytes(const bkv_pool* p) {
+    if (!p) return 0;
+    return (p->g.k_pool_bytes + p->g.v_pool_bytes) * (uint64_t)p->g.n_layers +
+           (uint64_t)p->desc.max_seqs * (uint64_t)p->desc.max_pages_per_seq * 4u;
+}
+
+uint64_t bkv_page_bytes(const bkv_pool* p, int which) {
+    if (!p) return 0;
+    return which ? p->g.v_page_bytes : p->g.k_page_bytes;
+}
+
+bkv_status bkv_pool_fill(bkv_pool* p, int byte, void* stream) {
+    bkv_status st = need_device(p);
+    if (st != BKV_OK) return st;
+    const uint32_t b = (uint32_t)(byte & 0xff);
+    const uint32_t word = b | (b << 8) | (b << 16) | (b << 24);
+    const uint64_t layer_bytes = p->g.k_pool_bytes + p->g.v_pool_bytes;
+    BKV_HIP(launch_fill(p->slab, layer_bytes * (uint64_t)p->g.n_layers, word, S(stream)));
+    return BKV_OK;
+}
+
+bkv_status bkv_pool_layer_ptr(const bkv_pool* p, int32_t layer, int which, void** dev_ptr,
+                              uint64_t* bytes) {
+    bkv_status st = need_device(p);
+    if (st != BKV_OK) return st;
+    if (layer < 0 || layer >= p->g.n_layers)
+        return fail(BKV_ERR_RANGE, sfmt("layer %lld is outside 0..%lld", layer, p->g.n_layers));
+    if (dev_ptr) *dev_ptr = which ? p->v_layer[(size_t)layer] : p->k_layer[(size_t)layer];
+    if (bytes) *bytes = which ? p->g.v_pool_bytes : p->g.k_pool_bytes;
+    return BKV_OK;
+}
+
+// ---- allocator ----------------------------------------------------------------------
+bkv_status bkv_seq_create(bkv_pool* p, int32_t* seq_out) {
+    if (!p || !seq_out) return fail(BKV_ERR_INVALID, "seq_create: NULL argument");
+    std::string err;
+    return from_alloc(p->alloc->seq_create(seq_out, err), err);
+}
+
+bkv_status bkv_seq_create_identity(bkv_pool* p, int32_t n_pages, int32_t* seq_out) {
+    if (!p || !seq_out) return fail(BKV_ERR_INVALID, "seq_create_identity: NULL argument");
+    std::string err;
+    return from_alloc(p->alloc->seq_create_identity(n_pages, seq_out, err), err);
+}
+
+bkv_status bkv_seq_fork(bkv_pool* p, int32_t parent, int64_t n_tokens, int32_t* child_out) {
+    if (!p || !child_out) return fail(BKV_ERR_INVALID, "seq_fork: NULL argument");
+    std::string err;
+    return from_alloc(p->alloc->seq_fork(parent, n_tokens, child_out, err), err);
+}
+
+bkv_status bkv_seq_free(bkv_pool* p, int32_t seq) {
+    if (!p) return fail(BKV_ERR_INVALID, "seq_free: NULL pool");
+    std::string err;
+    return from_alloc(p->alloc->seq_free(seq, err), err);
+}
+
+bkv_status bkv_seq_reserve(bkv_pool* p, int32_t seq, int64_t new_len, bkv_page_pair* cow,
+                           int32_t cow_cap, int32_t* n_cow) {
+    if (!p) return fail(BKV_ERR_INVALID, "seq_reserve: NULL pool");
+    std::string err;
+    static_assert(sizeof(PagePair) == sizeof(bkv_page_pair), "pair layouts must agree");
+    return from_alloc(p->alloc->seq_reserve(seq, new_len, reinterpret_cast<PagePair*>(cow), cow_cap,
+                                            n_cow, err),
+                      err);
+}
+
+bkv_status bkv_seq_truncate(bkv_pool* p, int32_t seq, int64_t new_len) {
+    if (!p) return fail(BKV_ERR_INVALID, "seq_truncate: NULL pool");
+    std::string err;
+    return from_alloc(p->alloc->seq_truncate(seq, new_len, err), err);
+}
+
+int64_t bkv_seq_len(const bkv_pool* p, int32_t seq) {
+    if (!p || !p->alloc->seq_valid(seq)) return -1;
+    return p->alloc->seq_len(seq);
+}
+int64_t bkv_seq_capacity(const bkv_pool* p, int32_t seq) {
+    if (!p || !p->alloc->seq_valid(seq)) return -1;
+    return p->alloc->seq_capacity(seq);
+}
+int32_t bkv_seq_n_pages(const bkv_pool* p, int32_t seq) {
+    if (!p || !p->alloc->seq_valid(seq)) return -1;
+    return p->alloc->seq_n_pages(seq);
+}
+const int32_t* bkv_seq_block_table(const bkv_pool* p, int32_t seq) {
+    if (!p || !p->alloc->seq_valid(seq)) return nullptr;
+    return p->alloc->seq_table(seq);
+}
+int32_t bkv_page_refcount(const bkv_pool* p, int32_t page) {
+    if (!p || page < 0 || page >= p->g.n_pages) return -1;
+    return p->alloc->refcount(page);
+}
+int32_t bkv_pool_free_pages(const bkv_pool* p) { return p ? p->alloc->free_pages() : -1; }
+
+bkv_status bkv_pool_set_free_order(bkv_pool* p, const int32_t* order, int32_t n) {
+    if (!p || (n > 0 && !order)) return fail(BKV_ERR_INVALID, "pool_set_free_order: NULL argument");
+    std::string err;
+    return from_alloc(p->alloc->set_free_order(order, n, err), err);
+}
+
+bkv_status bkv_pool_check(const bkv_pool* p) {
+    if (!p) return fail(BKV_ERR_INVALID, "pool_check: NULL pool");
+    std::string err;
+    if (!p->alloc->check(err)) return fail(BKV_ERR_STATE, "allocator invariant broken: " + err);
+    return BKV_OK;
+}
+
+// ---- append ------------------------------------------------------------------------
+bkv_status bkv_append(bkv_pool* p, int32_t layer, int32_t n_seqs, const int32_t* seqs,
+                      const int64_t* pos0, const int32_t* n_tokens, const float* k_dev,
+                      const float* v_dev, void* stream) {
+    if (!p) return fail(BKV_ERR_INVALID, "append: NULL pool");
+    if (layer < 0 || layer >= p->g.n_layers)
+        return fail(BKV_ERR_RANGE, sfmt("append: layer %lld is outside 0..%lld", layer,
+                                        p->g.n_layers));
+    if (n_seqs < 0 || n_seqs > BKV_MAX_BATCH)
+        return fail(BKV_ERR_INVALID, sfmt("append: %lld sequences in one call; the limit is %lld",
+                                          n_seqs, BKV_MAX_BATCH));
+    if (n_seqs > 0 && (!seqs || !pos0 || !n_tokens))
+        return fail(BKV_ERR_INVALID, "append: NULL sequence / position / token-count array");
+    AppendBatch b{};
+    int64_t src = 0;
+    int32_t max_tok = 0;
+    for (int i = 0; i < n_seqs; ++i) {
+        if (!p->alloc->seq_valid(seqs[i]))
+            return fail(BKV_ERR_RANGE, sfmt("append: sequence %lld is not live", seqs[i]));
+        if (n_tokens[i] < 0 || pos0[i] < 0)
+            return fail(BKV_ERR_RANGE, sfmt("append: entry %lld has pos0 %lld, n_tokens %lld", i,
+                                            pos0[i], n_tokens[i]));
+        const int64_t end = pos0[i] + n_tokens[i];
+        const int64_t cap = p->alloc->seq_capacity(seqs[i]);
+        if (end > cap)
+            return fail(BKV_ERR_RANGE,
+                        sfmt("append would write cells %lld..%lld of sequence %lld but it holds "
+                             "%lld (a write past the block table would land on an unmapped page)",
+                             pos0[i], end, seqs[i], cap));
+        if (n_tokens[i] > 0) {
+            const int32_t* row = p->alloc->seq_table(seqs[i]);
+            for (int64_t c = pos0[i] / p->g.page_cells; c <= (end - 1) / p->g.page_cells; ++c)
+                if (row[c] < 0)
+                    return fail(BKV_ERR_STATE, sfmt("append: logical page %lld of sequence %lld is "
+                                                    "swapped out", c, seqs[i]));
+        }
+        b.row[i] = seqs[i];
+        b.pos0[i] = (int32_t)pos0[i];
+        b.n_tok[i] = n_tokens[i];
+        b.src0[i] = (int32_t)src;
+        src += n_tokens[i];
+        max_tok = std::max(max_tok, n_tokens[i]);
+    }
+    b.n = n_seqs;
+    if (src > ((int64_t)1 << 30))
+        return fail(BKV_ERR_INVALID, "append: more than 2^30 tokens in one call");
+    bkv_status st = need_device(p);
+    if (st != BKV_OK) return st;
+    if (src == 0) return flush_tables(p, S(stream));
+    if (!k_dev || !v_dev || !aligned16(k_dev) || !aligned16(v_dev))
+        return fail(BKV_ERR_INVALID, "append: k/v device pointers must be non-NULL and 16-byte "
+                                     "aligned");
+    st = flush_tables(p, S(stream));
+    if (st != BKV_OK) return st;
+    {
+        StageScope timed(p, BKV_STAGE_APPEND, S(stream));
+        BKV_HIP(launch_append(p, layer, b, max_tok, k_dev, v_dev, S(stream)));
+    }
+    if (p->timer.open.size() > 8192) return timer_collect(p);
+    return BKV_OK;
+}
+
+// ---- decode attention ----------------------------------------------------------------
+bkv_status bkv_decode_attn(bkv_pool* p, int32_t layer, int32_t n, const int32_t* seqs,
+                           const int64_t* pos, int32_t n_q_head, const float* q_dev,
+                           const float* gate_dev, int64_t gate_seq_stride,
+                           int64_t gate_head_stride, float scale, float* out_dev, void* stream) {
+    if (!p) return fail(BKV_ERR_INVALID, "decode_attn: NULL pool");
+    if (layer < 0 || layer >= p->g.n_layers)
+        return fail(BKV_ERR_RANGE, sfmt("decode_attn: layer %lld is outside 0..%lld", layer,
+                                        p->g.n_layers));
+    if (n < 0 || n > BKV_MAX_BATCH)
+        return fail(BKV_ERR_INVALID, sfmt("decode_attn: %lld entries in one call; the limit is "
+                                          "%lld", n, BKV_MAX_BATCH));
+    if (n_q_head <= 0 || n_q_head % p->g.n_kv != 0 || n_q_head / p->g.n_kv > BKV_MAX_HEAD_GROUP)
+        return fail(BKV_ERR_INVALID,
+                    sfmt("decode_attn: %lld q heads over %lld kv heads (need a whole group of at "
+                         "most %lld)", n_q_head, p->g.n_kv, BKV_MAX_HEAD_GROUP));
+    if (p->g.hd != 256)
+        return fail(BKV_ERR_INVALID, sfmt("decode_attn is built for head_dim 256, pool has %lld",
+                                          p->g.hd));
+    if (p->g.layout != BKV_LAYOUT_F16)
+        return fail(BKV_ERR_INVALID, "decode_attn: only the f16 K/V layout is built");
+    if (n > 0 && (!seqs || !pos)) return fail(BKV_ERR_INVALID, "decode_attn: NULL seqs / pos");
+    AttnBatch b{};
+    for (int i = 0; i < n; ++i) {
+        if (!p->alloc->seq_valid(seqs[i]))
+            return fail(BKV_ERR_RANGE, sfmt("decode_attn: sequence %lld is not live", seqs[i]));
+        const int64_t cap = p->alloc->seq_capacity(seqs[i]);
+        if (pos[i] < 0 || pos[i] >= cap)
+            return fail(BKV_ERR_RANGE, sfmt("decode_attn: position %lld of sequence %lld is "
+                                            "outside its %lld addressable cells", pos[i], seqs[i],
+                                            cap));
+        if (!p->alloc->seq_resident(seqs[i], pos[i] + 1))
+            return fail(BKV_ERR_STATE, sfmt("decode_attn: sequence %lld has swapped-out pages "
+                                            "below position %lld", seqs[i], pos[i]));
+        b.row[i] = seqs[i];
+        b.pos[i] = (int32_t)pos[i];
+    }
+    b.n = n;
+    bkv_status st = need_device(p);
+    if (st != BKV_OK) return st;
+    if (n == 0) return BKV_OK;
+    if (!q_dev || !out_dev || !aligned16(q_dev) || !aligned16(out_dev))
+        return fail(BKV_ERR_INVALID, "decode_attn: q/out device pointers must be non-NULL and "
+                                     "16-byte aligned");
+    st = flush_tables(p, S(stream));
+    if (st != BKV_OK) return st;
+    plan_attn(p, n_q_head, b);
+    AttnArgs a;
+    a.n_q_head = n_q_head;
+    a.q = q_dev;
+    a.gate = gate_dev;
+    a.gate_seq_stride = gate_seq_stride;
+    a.gate_head_stride = gate_head_stride;
+    a.scale = scale;
+    a.out = out_dev;
+    BKV_HIP(launch_decode_attn(p, layer, b, a, S(stream)));
+    if (p->timer.open.size() > 8192) return timer_collect(p);
+    return BKV_OK;
+}
+
+// ---- page copy -------------------------------------------------------------------------
+bkv_status bkv_page_copy(bkv_pool* p, const bkv_page_pair* pairs, int32_t n_pairs, void* stream) {
+    if (!p) return fail(BKV_ERR_INVALID, "page_copy: NULL pool");
+    if (n_pairs < 0 || (n_pairs > 0 && !pairs))
+        return fail(BKV_ERR_INVALID, "page_copy: bad pair list");
+    std::vector<int32_t> dsts;
+    dsts.reserve((size_t)n_pairs);
+    for (int i = 0; i < n_pairs; ++i) {
+        if (pairs[i].src < 0 || pairs[i].src >= p->g.n_pages || pairs[i].dst < 0 ||
+            pairs[i].dst >= p->g.n_pages)
+            return fail(BKV_ERR_RANGE, sfmt("page_copy: pair %lld (%lld -> %lld) is outside the "
+                                            "%lld-page pool", i, pairs[i].src, pairs[i].dst,
+                                            p->g.n_pages));
+        dsts.push_back(pairs[i].dst);
+    }
+    std::sort(dsts.begin(), dsts.end());
+    if (std::adjacent_find(dsts.begin(), dsts.end()) != dsts.end())
+        return fail(BKV_ERR_INVALID, "page_copy: a destination page appears twice");
+    bkv_status st = need_device(p);
+    if (st != BKV_OK) return st;
+    const int32_t per_launch = std::min<int32_t>(
+        (int32_t)(ParamRing::kSlotBytes / sizeof(bkv_page_pair)), 65535 / (p->g.n_layers * 2));
+    if (per_launch <= 0) return fail(BKV_ERR_INVALID, "page_copy: too many layers for one launch");
+    for (int32_t at = 0; at < n_pairs; at += per_launch) {
+        const int32_t n = std::min(per_launch, n_pairs - at);
+        void* dev;
+        int slot;
+        st = ring_upload(p, pairs + at, (size_t)n * sizeof(bkv_page_pair), S(stream), &dev, &slot);
+        if (st != BKV_OK) return st;
+        {
+            StageScope timed(p, BKV_STAGE_PAGE_COPY, S(stream));
+            BKV_HIP(launch_page_copy(p, static_cast<const bkv_page_pair*>(dev), n, S(stream)));
+        }
+        st = ring_done(p, slot, S(stream));
+        if (st != BKV_OK) return st;
+    }
+    return BKV_OK;
+}
+
+// ---- swap --------------------------------------------------------------------------------
+uint64_t bkv_swap_page_bytes(const bkv_pool* p) {
+    if (!p) return 0;
+    return (p->g.k_page_bytes + p->g.v_page_bytes) * (uint64_t)p->g.n_layers;
+}
+
+bkv_status bkv_host_alloc(bkv_pool* p, uint64_t bytes, void** host_out) {
+    bkv_status st = need_device(p);
+    if (st != BKV_OK) return st;
+    if (!host_out || bytes == 0) return fail(BKV_ERR_INVALID, "host_alloc: bad argument");
+    void* h = nullptr;
+    const hipError_t e = hipHostMalloc(&h, bytes, hipHostMallocDefault);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(BKV_ERR_NOMEM, sfmt("host_alloc: hipHostMalloc of %lld bytes of pinned host "
+                                        "memory failed: ", (long long)bytes) +
+                                       hipGetErrorString(e));
+    }
+    *host_out = h;
+    return BKV_OK;
+}
+
+bkv_status bkv_host_free(bkv_pool* p, void* host) {
+    bkv_status st = need_device(p);
+    if (st != BKV_OK) return st;
+    if (!host) return BKV_OK;
+    BKV_HIP(hipHostFree(host));
+    return BKV_OK;
+}
+
+static bkv_status swap_move(bkv_pool* p, const int32_t* pages, int32_t n, uint8_t* host, bool out,
+                            hipStream_t stream) {
+    const uint64_t slab = bkv_swap_page_bytes(p);
+    const int32_t per_chunk = (int32_t)std::min<uint64_t>(
+        std::min<uint64_t>(p->stage.bytes / slab, ParamRing::kSlotBytes / 4),
+        (uint64_t)(65535 / (p->g.n_layers * 2)));
+    if (per_chunk <= 0) return fail(BKV_ERR_INVALID, "swap: a page slab exceeds the staging buffer");
+    for (int32_t at = 0; at < n; at += per_chunk) {
+        const int32_t m = std::min(per_chunk, n - at);
+        SwapStage& sg = p->stage;
+        const int h = sg.next;
+        sg.next = (sg.next + 1) % SwapStage::kHalves;
+        uint8_t* hostp = host + (uint64_t)at * slab;
+        void* pages_dev;
+        int slot;
+        if (out) {
+            BKV_HIP(hipStreamWaitEvent(stream, sg.ev_side[h], 0));
+            bkv_status st = ring_upload(p, pages + at, (size_t)m * 4, stream, &pages_dev, &slot);
+            if (st != BKV_OK) return st;
+            BKV_HIP(launch_page_stage(p, static_cast<const int32_t*>(pages_dev), m, sg.dev[h], 1,
+                                      stream));
+            st = ring_done(p, slot, stream);
+            if (st != BKV_OK) return st;
+            BKV_HIP(hipEventRecord(sg.ev_stream[h], stream));
+            BKV_HIP(hipStreamWaitEvent(p->side, sg.ev_stream[h], 0));
+            BKV_HIP(hipMemcpyAsync(hostp, sg.dev[h], (uint64_t)m * slab, hipMemcpyDeviceToHost,
+                                   p->side));
+            BKV_HIP(hipEventRecord(sg.ev_side[h], p->side));
+        } else {
+            BKV_HIP(hipStreamWaitEvent(p->side, sg.ev_stream[h], 0));
+            BKV_HIP(hipMemcpyAsync(sg.dev[h], hostp, (uint64_t)m * slab, hipMemcpyHostToDevice,
+                                   p->side));
+            BKV_HIP(hipEventRecord(sg.ev_side[h], p->side));
+            BKV_HIP(hipStreamWaitEvent(stream, sg.ev_side[h], 0));
+            bkv_status st = ring_upload(p, pages + at, (size_t)m * 4, stream, &pages_dev, &slot);
+            if (st != BKV_OK) return st;
+            BKV_HIP(launch_page_stage(p, static_cast<const int32_t*>(pages_dev), m, sg.dev[h], 0,
+                                      stream));
+            st = ring_done(p, slot, stream);
+            if (st != BKV_OK) return st;
+            BKV_HIP(hipEventRecord(sg.ev_stream[h], stream));
+        }
+    }
+    BKV_HIP(hipEventRecord(p->side_done, p->side));
+    p->side_used = true;
+    return BKV_OK;
+}
+
+static bkv_status check_pages(const bkv_pool* p, const int32_t* pages, int32_t n, const void* host,
+                              const char* who) {
+    if (n < 0 || (n > 0 && (!pages || !host)))
+        return fail(BKV_ERR_INVALID, std::string(who) + ": bad page list or host buffer");
+    for (int i = 0; i < n; ++i)
+        if (pages[i] < 0 || pages[i] >= p->g.n_pages)
+            return fail(BKV_ERR_RANGE, std::string(who) + sfmt(": page %lld (entry %lld) is outside "
+                                                               "the %lld-page pool", pages[i], i,
+                                                               p->g.n_pages));
+    return BKV_OK;
+}
+
+bkv_status bkv_swap_out(bkv_pool* p, const int32_t* pages, int32_t n, void* pinned_host,
+                        void* stream) {
+    if (!p) return fail(BKV_ERR_INVALID, "swap_out: NULL pool");
+    bkv_status st = check_pages(p, pages, n, pinned_host, "swap_out");
+    if (st != BKV_OK) return st;
+    st = need_device(p);
+    if (st != BKV_OK) return st;
+    if (n == 0) return BKV_OK;
+    return swap_move(p, pages, n, static_cast<uint8_t*>(pinned_host), true, S(stream));
+}
+
+bkv_status bkv_swap_in(bkv_pool* p, const int32_t* pages, int32_t n, const void* pinned_host,
+                       void* stream) {
+    if (!p) return fail(BKV_ERR_INVALID, "swap_in: NULL pool");
+    bkv_status st = check_pages(p, pages, n, pinned_host, "swap_in");
+    if (st != BKV_OK) return st;
+    std::vector<int32_t> sorted(pages, pages + n);
+    std::sort(sorted.begin(), sorted.end());
+    if (std::adjacent_find(sorted.begin(), sorted.end()) != sorted.end())
+        return fail(BKV_ERR_INVALID, "swap_in: a destination page appears twice");
+    st = need_device(p);
+    if (st != BKV_OK) return st;
+    if (n == 0) return BKV_OK;
+    return swap_move(p, pages, n, const_cast<uint8_t*>(static_cast<const uint8_t*>(pinned_host)),
+                     false, S(stream));
+}
+
+bkv_status bkv_swap_wait(bkv_pool* p) {
+    bkv_status st = need_device(p);
+    if (st != BKV_OK) return st;
+    BKV_HIP(hipStreamSynchronize(p->side));
+    return BKV_OK;
+}
+
+bkv_status bkv_swap_fence(bkv_pool* p, void* stream) {
+    bkv_status st = need_device(p);
+    if (st != BKV_OK) return st;
+    if (p->side_used) BKV_HIP(hipStreamWaitEvent(S(stream), p->side_done, 0));
+    return BKV_OK;
+}
+
+bkv_status bkv_seq_evict(bkv_pool* p, int32_t seq, int32_t lp0, int32_t n, void* pinned_host,
+                         void* stream) {
+    if (!p) return fail(BKV_ERR_INVALID, "seq_evict: NULL pool");
+    if (n > 0 && !pinned_host) return fail(BKV_ERR_INVALID, "seq_evict: NULL host buffer");
+    if (!p->host_only) {
+        // The device copy reads the pages through ids taken before they are freed.
+        bkv_status st = flush_tables(p, S(stream));
+        if (st != BKV_OK) return st;
+    }
+    std::vector<int32_t> phys;
+    std::string err;
+    const AllocErr e = p->alloc->seq_detach_pages(seq, lp0, n, phys, err);
+    if (e != AllocErr::Ok) return from_alloc(e, err);
+    if (p->host_only || n == 0) return BKV_OK;
+    return swap_move(p, phys.data(), n, static_cast<uint8_t*>(pinned_host), true, S(stream));
+}
+
+bkv_status bkv_seq_restore(bkv_pool* p, int32_t seq, int32_t lp0, int32_t n,
+                           const void* pinned_host, void* stream) {
+    if (!p) return fail(BKV_ERR_INVALID, "seq_restore: NULL pool");
+    if (n > 0 && !pinned_host) return fail(BKV_ERR_INVALID, "seq_restore: NULL host buffer");
+    std::vector<int32_t> phys;
+    std::string err;
+    const AllocErr e = p->alloc->seq_attach_pages(seq, lp0, n, phys, err);
+    if (e != AllocErr::Ok) return from_alloc(e, err);
+    if (p->host_only || n == 0) return BKV_OK;
+    bkv_status st = swap_move(p, phys.data(), n,
+                              const_cast<uint8_t*>(static_cast<const uint8_t*>(pinned_host)), false,
+                              S(stream));
+    if (st != BKV_OK) return st;
+    return flush_tables(p, S(stream));
+}
+
+// ---- gather ------------------------------------------------------------------------------
+bkv_status bkv_gather(bkv_pool* p, int32_t layer, int32_t seq, int64_t cell0, int64_t n,
+                      float* k_out_dev, float* v_out_dev, void* stream) {
+    if (!p) return fail(BKV_ERR_INVALID, "gather: NULL pool");
+    if (layer < 0 || layer >= p->g.n_layers)
+        return fail(BKV_ERR_RANGE, sfmt("gather: layer %lld is outside 0..%lld", layer,
+                                        p->g.n_layers));
+    if (!p->alloc->seq_valid(seq))
+        return fail(BKV_ERR_RANGE, sfmt("gather: sequence %lld is not live", seq));
+    if (cell0 < 0 || n < 0 || cell0 + n > p->alloc->seq_capacity(seq))
+        return fail(BKV_ERR_RANGE, sfmt("gather: cells %lld..%lld are outside the sequence's %lld",
+                                        cell0, cell0 + n, p->alloc->seq_capacity(seq)));
+    if (n > 0) {
+        const int32_t* row = p->alloc->seq_table(seq);
+        for (int64_t c = cell0 / p->g.page_cells; c <= (cell0 + n - 1) / p->g.page_cells; ++c)
+            if (row[c] < 0)
+                return fail(BKV_ERR_STATE, sfmt("gather: logical page %lld is swapped out", c));
+    }
+    bkv_status st = need_device(p);
+    if (st != BKV_OK) return st;
+    if (n == 0) return BKV_OK;
+    if (!k_out_dev || !v_out_dev) return fail(BKV_ERR_INVALID, "gather: NULL output");
+    st = flush_tables(p, S(stream));
+    if (st != BKV_OK) return st;
+    BKV_HIP(launch_gather(p, layer, seq, cell0, n, k_out_dev, v_out_dev, S(stream)));
+    return BKV_OK;
+}
+
+// ---- per-kernel timing ---------------------------------------------------------------
+bkv_status bkv_timing_enable(bkv_pool* p, int on) {
+    bkv_status st = need_device(p);
+    if (st != BKV_OK) return st;
+    if (!on && p->timer.on) {
+        st = timer_collect(p);
+        if (st != BKV_OK) return st;
+    }
+    p->timer.on = on != 0;
+    return BKV_OK;
+}
+
+bkv_status bkv_timing_reset(bkv_pool* p) {
+    bkv_status st = need_device(p);
+    if (st != BKV_OK) return st;
+    st = timer_collect(p);
+    if (st != BKV_OK) return st;
+    for (int i = 0; i < BKV_STAGE_COUNT; ++i) {
+        p->timer.launches[i] = 0;
+        p->timer.total_ms[i] = 0.0;
+    }
+    return BKV_OK;
+}
+
+bkv_status bkv_timing_read(bkv_pool* p, int stage, uint64_t* launches, double* total_ms) {
+    bkv_status st = need_device(p);
+    if (st != BKV_OK) return st;
+    if (stage < 0 || stage >= BKV_STAGE_COUNT)
+        return fail(BKV_ERR_RANGE, sfmt("timing_read: stage %lld is outside 0..%lld", stage,
+                                        BKV_STAGE_COUNT));
+    st = timer_collect(p);
+    if (st != BKV_OK) return st;
+    if (launches) *launches = p->timer.launches[stage];
+    if (total_ms) *total_ms = p->timer.total_ms[stage];
+    return BKV_OK;
+}
+
+// ---- device plumbing ------------------------------------------------------------------
+bkv_status bkv_dev_alloc(uint64_t bytes, void** dev_out) {
+    if (!dev_out) return fail(BKV_ERR_INVALID, "dev_alloc: NULL out pointer");
+    BKV_HIP(hipMalloc(dev_out, bytes ? bytes : 16));
+    return BKV_OK;
+}
+bkv_status bkv_dev_free(void* dev) {
+    if (dev) BKV_HIP(hipFree(dev));
+    return BKV_OK;
+}
+bkv_status bkv_memcpy_h2d(void* dev, const void* host, uint64_t bytes, void* stream) {
+    BKV_HIP(hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, S(stream)));
+    return BKV_OK;
+}
+bkv_status bkv_memcpy_d2h(void* host, const void* dev, uint64_t bytes, void* stream) {
+    BKV_HIP(hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, S(stream)));
+    return BKV_OK;
+}
+bkv_status bkv_stream_create(void** stream_out) {
+    if (!stream_out) return fail(BKV_ERR_INVALID, "stream_create: NULL out pointer");
+    hipStream_t s;
+    BKV_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    *stream_out = s;
+    return BKV_OK;
+}
+bkv_status bkv_stream_destroy(void* stream) {
+    if (stream) BKV_HIP(hipStreamDestroy(S(stream)));
+    return BKV_OK;
+}
+bkv_status bkv_stream_sync(void* stream) {
+    BKV_HIP(hipStreamSynchronize(S(stream)));
+    return BKV_OK;
+}
+bkv_status bkv_device_sync(void) {
+    BKV_HIP(hipDeviceSynchronize());
+    return BKV_OK;
+}
+bkv_status bkv_event_create(void** event_out) {
+    if (!event_out) return fail(BKV_ERR_INVALID, "event_create: NULL out pointer");
+    hipEvent_t e;
+    BKV_HIP(hipEventCreate(&e));
+    *event_out = e;
+    return BKV_OK;
+}
+bkv_status bkv_event_destroy(void* event) {
+    if (event) BKV_HIP(hipEventDestroy(reinterpret_cast<hipEvent_t>(event)));
+    return BKV_OK;
+}
+bkv_status bkv_event_record(void* event, void* stream) {
+    BKV_HIP(hipEventRecord(reinterpret_cast<hipEvent_t>(event), S(stream)));
+    return BKV_OK;
+}
+bkv_status bkv_event_sync(void* event) {
+    BKV_HIP(hipEventSynchronize(reinterpret_cast<hipEvent_t>(event)));
+    return BKV_OK;
+}
+bkv_status bkv_event_elapsed_ms(void* start, void* stop, float* ms_out) {
+    if (!ms_out) return fail(BKV_ERR_INVALID, "event_elapsed_ms: NULL out pointer");
+    BKV_HIP(hipEventElapsedTime(ms_out, reinterpret_cast<hipEvent_t>(start),
+                                reinterpret_cast<hipEvent_t>(stop)));
+    return BKV_OK;
+}
+bkv_status bkv_device_info(char* name_out, int32_t name_cap, int32_t* cu_out,
+                           uint64_t* mem_bytes_out) {
+    int dev = 0;
+    BKV_HIP(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    BKV_HIP(hipGetDeviceProperties(&prop, dev));
+    if (name_out && name_cap > 0) {
+        std::snprintf(name_out, (size_t)name_cap, "%s (%s)", prop.name, prop.gcnArchName);
+    }
+    if (cu_out) *cu_out = prop.multiProcessorCount;
+    if (mem_bytes_out) *mem_bytes_out = prop.totalGlobalMem;
+    return BKV_OK;
+}
+bkv_status bkv_copy_probe(void* dst_dev, const void* src_dev, uint64_t bytes, void* stream) {
+    if (!dst_dev || !src_dev || !aligned16(dst_dev) || !aligned16(src_dev) || bytes % 16)
+        return fail(BKV_ERR_INVALID, "copy_probe: pointers and size must be 16-byte multiples");
+    BKV_HIP(launch_copy_probe(dst_dev, src_dev, bytes, S(stream)));
+    return BKV_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,170 @@
+// Internal declarations shared by the translation units of libbreccia_kv.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "../../include/breccia_kv.h"
+#include "allocator.hpp"
+
+namespace bkv {
+
+// ---- error plumbing ---------------------------------------------------------
+void set_error(const std::string& msg);
+bkv_status fail(bkv_status st, const std::string& msg);
+bkv_status hip_fail(hipError_t e, const char* what);
+
+#define BKV_HIP(call)                                                 \
+    do {                                                              \
+        hipError_t e__ = (call);                                      \
+        if (e__ != hipSuccess) return ::bkv::hip_fail(e__, #call);    \
+    } while (0)
+
+// ---- geometry ----------------------------------------------------------------
+struct Geom {
+    int32_t n_layers, n_pages, n_kv, hd, page_cells, layout;
+    // bytes of one (page, kv head, cell) row and of one whole page, per pool
+    uint32_t k_row_bytes, v_row_bytes;
+    uint64_t k_page_bytes, v_page_bytes;
+    uint64_t k_pool_bytes, v_pool_bytes;  // one layer
+};
+
+// Pinned-host + device slot pairs for argument lists too long for kernel
+// arguments (page-pair lists, block-table updates).  A slot is reused only after
+// the event recorded behind its last consumer has completed.
+struct ParamRing {
+    static constexpr int kSlots = 32;
+    static constexpr size_t kSlotBytes = 64 * 1024;
+    uint8_t* host = nullptr;
+    uint8_t* dev = nullptr;
+    hipEvent_t ev[kSlots] = {};
+    bool used[kSlots] = {};
+    int next = 0;
+};
+
+// Event pairs around individual kernels while timing is enabled.
+struct StageTimer {
+    struct Pair {
+        int stage;
+        hipEvent_t start, stop;
+    };
+    bool on = false;
+    std::vector<Pair> open;       // recorded, not yet read
+    std::vector<hipEvent_t> idle; // events to reuse
+    uint64_t launches[BKV_STAGE_COUNT] = {};
+    double total_ms[BKV_STAGE_COUNT] = {};
+};
+
+struct SwapStage {
+    static constexpr int kHalves = 2;
+    uint8_t* dev[kHalves] = {nullptr, nullptr};
+    uint64_t bytes = 0;             // per half
+    hipEvent_t ev_stream[kHalves] = {};  // last use on a caller stream
+    hipEvent_t ev_side[kHalves] = {};    // last use on the side stream
+    int next = 0;
+};
+
+}  // namespace bkv
+
+struct bkv_pool {
+    bkv_pool_desc desc{};
+    bkv::Geom g{};
+    std::unique_ptr<bkv::PageAllocator> alloc;
+    bool host_only = false;
+    int device = 0;
+    int n_cu = 0;
+
+    uint8_t* slab = nullptr;  // every layer's K and V pool, one allocation
+    std::vector<uint8_t*> k_layer, v_layer;
+    int32_t* table_dev = nullptr;  // [max_seqs][max_pages_per_seq]
+
+    // split-K workspace: partial (m, l) and O per work-group
+    float* part_o = nullptr;
+    float* part_ml = nullptr;
+    int32_t max_wgs = 0;
+
+    bkv::ParamRing ring;
+    bkv::StageTimer timer;
+    bkv::SwapStage stage;
+    hipStream_t side = nullptr;
+    hipEvent_t side_done = nullptr;
+    bool side_used = false;
+};
+
+namespace bkv {
+
+// Push pending block-table changes to the device arena on `stream`.
+bkv_status flush_tables(bkv_pool* p, hipStream_t stream);
+// Copy `bytes` of host data into a ring slot and enqueue its upload; returns the
+// device address the consumer kernel reads.  `done(stream)` must be called after
+// the consumer has been enqueued.
+bkv_status ring_upload(bkv_pool* p, const void* host_src, size_t bytes, hipStream_t stream,
+                       void** dev_out, int* slot_out);
+bkv_status ring_done(bkv_pool* p, int slot, hipStream_t stream);
+
+// RAII bracket: records a start event now and a stop event when it goes out of scope,
+// only while the pool's timer is on.
+class StageScope {
+public:
+    StageScope(bkv_pool* p, int stage, hipStream_t stream);
+    ~StageScope();
+
+private:
+    bkv_pool* p_;
+    hipStream_t stream_;
+    hipEvent_t stop_ = nullptr;
+};
+bkv_status timer_collect(bkv_pool* p);
+
+// ---- kernel launchers (each validates nothing: callers have checked) ---------
+struct AppendBatch {
+    int32_t n;
+    int32_t row[BKV_MAX_BATCH];      // block-table row of the sequence
+    int32_t pos0[BKV_MAX_BATCH];     // first cell
+    int32_t n_tok[BKV_MAX_BATCH];    // tokens of this sequence
+    int32_t src0[BKV_MAX_BATCH];     // first source row in k/v
+};
+hipError_t launch_append(const bkv_pool* p, int32_t layer, const AppendBatch& b, int32_t max_tok,
+                         const float* k, const float* v, hipStream_t stream);
+
+struct AttnBatch {
+    int32_t n;
+    int32_t row[BKV_MAX_BATCH];       // block-table row
+    int32_t pos[BKV_MAX_BATCH];       // last visible cell
+    int32_t wg_base[BKV_MAX_BATCH + 1];  // first work-group of the entry; [n] = total
+    int32_t splits[BKV_MAX_BATCH];    // page ranges the entry is cut into
+    int32_t pps[BKV_MAX_BATCH];       // pages per split
+};
+struct AttnArgs {
+    int32_t n_q_head;
+    const float* q;
+    const float* gate;
+    int64_t gate_seq_stride, gate_head_stride;
+    float scale;
+    float* out;
+};
+// Fills wg_base/splits/pps from row/pos; returns the total work-group count.
+int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b);
+hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, const AttnArgs& a,
+                              hipStream_t stream);
+// heads one wave carries for a given q-heads-per-kv-head group
+int32_t attn_heads_per_wave(int32_t group);
+
+hipError_t launch_page_copy(const bkv_pool* p, const bkv_page_pair* pairs_dev, int32_t n_pairs,
+                            hipStream_t stream);
+// Gather (to_stage=1) / scatter (to_stage=0) whole pages between the pools and a
+// contiguous staging buffer laid out [page][layer][K bytes | V bytes].
+hipError_t launch_page_stage(const bkv_pool* p, const int32_t* pages_dev, int32_t n_pages,
+                             uint8_t* stage, int to_stage, hipStream_t stream);
+hipError_t launch_gather(const bkv_pool* p, int32_t layer, int32_t row, int64_t cell0, int64_t n,
+                         float* k_out, float* v_out, hipStream_t stream);
+hipError_t launch_table_scatter(int32_t* table, const TableUpdate* upd_dev, int32_t n,
+                                hipStream_t stream);
+hipError_t launch_fill(void* dst, uint64_t bytes, uint32_t word, hipStream_t stream);
+hipError_t launch_copy_probe(void* dst, const void* src, uint64_t bytes, hipStream_t stream);
+
+}  // namespace bkv

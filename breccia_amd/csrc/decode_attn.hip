@@ -1,0 +1,474 @@
+// Paged decode attention for gfx950: one split-K online-softmax kernel and one merge
+// kernel.  Replaces the reference's four dispatches (scores -> softmax -> split
+// apply -> reduce: crates/breccia-kernels/shaders/qsa_attn_scores_small.comp,
+// ops_softmax.comp, qsa_attn_apply_split.comp, qsa_attn_apply_reduce.comp) and must
+// agree with its f64 CPU attend (crates/breccia-kernels/src/qsa/cpu.rs:197-246).
+//
+// Shape of the work: for one (sequence, kv head) every 512-byte f16 K row and V row
+// is read once and used by all q heads of the group -- a GEMV-shaped, HBM-bound
+// stream (about `group` flop per byte), so there is no MFMA here; the design goal
+// is to keep the VALU almost purely on FMAs while 16-byte row loads stay in flight.
+//
+// Work-group = 4 waves, all on one (entry, kv head, head chunk, page range).  A wave
+// owns whole pages (16 cells).  Lane l of a wave owns 8 consecutive head-dim elements
+// (l % 32) of the rows with parity l / 32, so one 16-byte load per lane covers two
+// rows and a page is 8 loads of K and 8 of V.  q (HG heads x 8 elements) and the
+// output accumulators (HG x 8) live in registers.
+//   scores: per row HG partial dots per lane -> transposed through LDS so that each
+//           lane finishes one (row, head) sum (no butterfly of selects)
+//   softmax: running max per head in base 2, per-lane partial denominators, the
+//           max is agreed across the 8..16 lanes of a head with three or four shuffles
+//   P.V   : probabilities go back through LDS (broadcast reads), FMAs straight from
+//           the f16 V registers
+// Partial (m, l, O) of the four waves are merged in LDS and written per work-group;
+// the merge kernel combines the splits and applies sigmoid(gate).
+#include "bkv_internal.hpp"
+
+namespace bkv {
+
+namespace {
+
+constexpr int kHd = 256;      // head_dim the kernel is built for
+constexpr int kPage = 16;     // cells per page
+constexpr int kWaves = 4;
+constexpr int kBlock = 64 * kWaves;
+constexpr float kLog2e = 1.4426950408889634f;
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+
+struct AttnKernelParams {
+    AttnBatch b;
+    const uint16_t* kpool;
+    const uint16_t* vpool;
+    const int32_t* tables;
+    const float* q;
+    float* part_o;
+    float* part_ml;
+    int32_t max_pages_per_seq;
+    int32_t n_kv, n_q, group, n_hc;
+    float scale_log2e;
+};
+
+__device__ __forceinline__ void wave_lds_sync() {
+    // LDS operations of one wave execute in order; this only stops the compiler from
+    // moving a lane's reads above other lanes' writes.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <int CTRL>
+__device__ __forceinline__ float dpp(float v) {
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+constexpr int kDppXor1 = 0xB1;  // quad_perm [1,0,3,2]
+constexpr int kDppXor2 = 0x4E;  // quad_perm [2,3,0,1]
+
+__device__ __forceinline__ float xor_max(float v, int mask) {
+    return fmaxf(v, __shfl_xor(v, mask, 64));
+}
+__device__ __forceinline__ float xor_sum(float v, int mask) { return v + __shfl_xor(v, mask, 64); }
+
+__device__ __forceinline__ half8 load_row8(const uint16_t* base, int idx) {
+    return __builtin_bit_cast(half8, reinterpret_cast<const uint4*>(base)[idx]);
+}
+
+// HG = q heads carried by one wave (8 or 4).
+template <int HG>
+__global__ __launch_bounds__(kBlock, 2) void decode_attn_f16_kernel(const AttnKernelParams P) {
+    constexpr int HQ = HG / 4;           // float4 groups of heads
+    constexpr int NB = HG / 4;           // score batches per page (8 float4 slots each)
+    constexpr int RP = 8 / NB;           // row pairs per batch
+    // xs: per wave 8 slots x 64 lanes of float4 = 8 KiB; reused for the final merge.
+    __shared__ f4 xs[kWaves][8 * 64];
+    __shared__ __attribute__((aligned(16))) float ps[kWaves][kPage][HG];
+    __shared__ __attribute__((aligned(16))) float alphas[kWaves][HG];
+    __shared__ float wave_m[kWaves][HG];
+    __shared__ float wave_l[kWaves][HG];
+
+    // ---- which (entry, kv head, head chunk, page range) ---------------------------
+    const int wg = blockIdx.x;
+    int e = 0;
+    while (e + 1 < P.b.n && wg >= P.b.wg_base[e + 1]) ++e;
+    const int local = wg - P.b.wg_base[e];
+    const int splits = P.b.splits[e];
+    const int per_hc = splits * P.n_kv;
+    const int hc = local / per_hc;
+    const int rem = local - hc * per_hc;
+    const int split = rem / P.n_kv;
+    const int kvh = rem - split * P.n_kv;
+    const int pos = P.b.pos[e];
+    const int n_pages = pos / kPage + 1;
+    const int pps = P.b.pps[e];
+    const int pg0 = split * pps;
+    const int pg1 = min(pg0 + pps, n_pages);
+    const int32_t* __restrict__ bt = P.tables + (size_t)P.b.row[e] * (size_t)P.max_pages_per_seq;
+
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int hw = lane >> 5;   // row parity this lane loads
+    const int dl = lane & 31;   // 8-element slice of the head dim
+
+    // ---- q slice (dead heads of a padded chunk stay zero) ---------------------------
+    float q[HG][8];
+#pragma unroll
+    for (int h = 0; h < HG; ++h) {
+        const int hl = hc * HG + h;
+        if (hl < P.group) {
+            const float* qp =
+                P.q + ((size_t)e * P.n_q + (size_t)kvh * P.group + hl) * kHd + dl * 8;
+            const float4 a = *reinterpret_cast<const float4*>(qp);
+            const float4 c = *reinterpret_cast<const float4*>(qp + 4);
+            q[h][0] = a.x, q[h][1] = a.y, q[h][2] = a.z, q[h][3] = a.w;
+            q[h][4] = c.x, q[h][5] = c.y, q[h][6] = c.z, q[h][7] = c.w;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) q[h][j] = 0.0f;
+        }
+    }
+
+    float o[HG][8];
+#pragma unroll
+    for (int h = 0; h < HG; ++h)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o[h][j] = 0.0f;
+
+    // ---- this lane's role when it finishes score sums ------------------------------
+    // part: which quarter of the 32 slices it adds; slot/rhw: which float4 slot and row
+    // parity; after the quad combine it keeps component `part`, i.e. one head.
+    const int part = lane & 3;
+    const int rslot = ((lane >> 4) << 1) | ((lane >> 2) & 1);
+    const int rhw = (lane >> 3) & 1;
+    const int my_head = (HG == 8) ? (lane & 7) : (lane & 3);
+    const int rbase = rslot * 64 + rhw * 32 + part * 8;
+    float m_run = -INFINITY;  // running max of this lane's head (base-2 logits)
+    float l_run = 0.0f;       // this lane's share of the denominator
+
+    const size_t page_elems = (size_t)P.n_kv * kPage * kHd;
+    const size_t head_off = (size_t)kvh * kPage * kHd;
+
+    int pg = pg0 + wave;
+    half8 kk[8], vv[8];
+    int32_t phys = 0;
+    if (pg < pg1) {
+        phys = bt[pg];
+        const uint16_t* kp = P.kpool + (size_t)phys * page_elems + head_off;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) kk[i] = load_row8(kp, i * 64 + lane);
+    }
+
+    while (pg < pg1) {
+        {
+            const uint16_t* vp = P.vpool + (size_t)phys * page_elems + head_off;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) vv[i] = load_row8(vp, i * 64 + lane);
+        }
+        const int pg_next = pg + kWaves;
+        int32_t phys_next = 0;
+        if (pg_next < pg1) phys_next = bt[pg_next];
+
+        // ---- scores: partial dots -> LDS transpose -> one (row, head) per lane ------
+        float sval[NB];
+#pragma unroll
+        for (int bch = 0; bch < NB; ++bch) {
+#pragma unroll
+            for (int ip = 0; ip < RP; ++ip) {
+                const int i = bch * RP + ip;
+                float s[HG];
+#pragma unroll
+                for (int h = 0; h < HG; ++h) {
+                    float acc = 0.0f;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) acc = fmaf((float)kk[i][j], q[h][j], acc);
+                    s[h] = acc;
+                }
+#pragma unroll
+                for (int hq = 0; hq < HQ; ++hq) {
+                    const int slot = (HG == 8) ? (ip * 2 + hq) : i;
+                    f4 w;
+                    w.x = s[hq * 4 + 0], w.y = s[hq * 4 + 1], w.z = s[hq * 4 + 2],
+                    w.w = s[hq * 4 + 3];
+                    xs[wave][slot * 64 + lane] = w;
+                }
+            }
+            wave_lds_sync();
+            f4 acc = xs[wave][rbase + (lane & 7)];
+#pragma unroll
+            for (int k = 1; k < 8; ++k) acc += xs[wave][rbase + ((k + lane) & 7)];
+            wave_lds_sync();
+            float r0 = acc.x + dpp<kDppXor1>(acc.x);
+            float r1 = acc.y + dpp<kDppXor1>(acc.y);
+            float r2 = acc.z + dpp<kDppXor1>(acc.z);
+            float r3 = acc.w + dpp<kDppXor1>(acc.w);
+            r0 += dpp<kDppXor2>(r0);
+            r1 += dpp<kDppXor2>(r1);
+            r2 += dpp<kDppXor2>(r2);
+            r3 += dpp<kDppXor2>(r3);
+            sval[bch] = part == 0 ? r0 : part == 1 ? r1 : part == 2 ? r2 : r3;
+        }
+
+        // K registers are free: start the next page's K rows.
+        if (pg_next < pg1) {
+            const uint16_t* kp = P.kpool + (size_t)phys_next * page_elems + head_off;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) kk[i] = load_row8(kp, i * 64 + lane);
+        }
+
+        // ---- online softmax for this lane's head -------------------------------------
+        float sv[NB];
+        int rowv[NB];
+        float pm = -INFINITY;
+#pragma unroll
+        for (int bch = 0; bch < NB; ++bch) {
+            const int i = (HG == 8) ? (bch * RP + (lane >> 4)) : rslot;
+            rowv[bch] = 2 * i + rhw;
+            const bool live = pg * kPage + rowv[bch] <= pos;
+            sv[bch] = live ? sval[bch] * P.scale_log2e : -INFINITY;
+            pm = fmaxf(pm, sv[bch]);
+        }
+        if (HG == 4) pm = xor_max(pm, 4);
+        pm = xor_max(pm, 8);
+        pm = xor_max(pm, 16);
+        pm = xor_max(pm, 32);
+        const float m_new = fmaxf(m_run, pm);
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        const bool changed = __builtin_amdgcn_ballot_w64(m_new > m_run) != 0;
+        float psum = 0.0f;
+#pragma unroll
+        for (int bch = 0; bch < NB; ++bch) {
+            const float pv = __builtin_amdgcn_exp2f(sv[bch] - m_new);
+            psum += pv;
+            ps[wave][rowv[bch]][my_head] = pv;
+        }
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+        if (changed && (lane >> 3) == 0 && (HG == 8 || (lane & 4) == 0))
+            alphas[wave][my_head] = alpha;
+        wave_lds_sync();
+
+        // ---- P.V ------------------------------------------------------------------
+        if (changed) {
+#pragma unroll
+            for (int h = 0; h < HG; ++h) {
+                const float a = alphas[wave][h];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) o[h][j] *= a;
+            }
+        }
+        if (pg == n_pages - 1) {
+            // Rows past `pos` may hold anything (even NaN): make them exact zeros.
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                if (pg * kPage + 2 * i + hw > pos) {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) vv[i][j] = (_Float16)0.0f;
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float pr[HG];
+            const f4* prow = reinterpret_cast<const f4*>(&ps[wave][2 * i + hw][0]);
+#pragma unroll
+            for (int hq = 0; hq < HQ; ++hq) {
+                const f4 t = prow[hq];
+                pr[hq * 4 + 0] = t.x, pr[hq * 4 + 1] = t.y, pr[hq * 4 + 2] = t.z,
+                            pr[hq * 4 + 3] = t.w;
+            }
+#pragma unroll
+            for (int h = 0; h < HG; ++h)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) o[h][j] = fmaf((float)vv[i][j], pr[h], o[h][j]);
+        }
+        wave_lds_sync();
+
+        pg = pg_next;
+        phys = phys_next;
+    }
+
+    // ---- wave totals ------------------------------------------------------------------
+    if (HG == 4) l_run = xor_sum(l_run, 4);
+    l_run = xor_sum(l_run, 8);
+    l_run = xor_sum(l_run, 16);
+    l_run = xor_sum(l_run, 32);
+    if ((lane >> 3) == 0 && (HG == 8 || (lane & 4) == 0)) {
+        wave_m[wave][my_head] = m_run;
+        wave_l[wave][my_head] = l_run;
+    }
+    float* ow = reinterpret_cast<float*>(&xs[wave][0]);  // [HG][256] floats = 8 KiB at HG 8
+#pragma unroll
+    for (int h = 0; h < HG; ++h) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o[h][j] += __shfl_xor(o[h][j], 32, 64);
+        if (hw == 0) {
+            f4 a, c;
+            a.x = o[h][0], a.y = o[h][1], a.z = o[h][2], a.w = o[h][3];
+            c.x = o[h][4], c.y = o[h][5], c.z = o[h][6], c.w = o[h][7];
+            reinterpret_cast<f4*>(ow + h * kHd + dl * 8)[0] = a;
+            reinterpret_cast<f4*>(ow + h * kHd + dl * 8)[1] = c;
+        }
+    }
+    __syncthreads();
+
+    // ---- merge the four waves; thread = head-dim element ----------------------------
+    const int d = threadIdx.x;
+#pragma unroll
+    for (int h = 0; h < HG; ++h) {
+        float mx = wave_m[0][h];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) mx = fmaxf(mx, wave_m[w][h]);
+        float acc = 0.0f, lsum = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            const float mw = wave_m[w][h];
+            const float f = mw == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(mw - mx);
+            acc = fmaf(f, reinterpret_cast<const float*>(&xs[w][0])[h * kHd + d], acc);
+            lsum = fmaf(f, wave_l[w][h], lsum);
+        }
+        P.part_o[((size_t)wg * HG + h) * kHd + d] = acc;
+        if (d == 0) {
+            P.part_ml[((size_t)wg * HG + h) * 2 + 0] = mx;
+            P.part_ml[((size_t)wg * HG + h) * 2 + 1] = lsum;
+        }
+    }
+}
+
+struct MergeParams {
+    AttnBatch b;
+    const float* part_o;
+    const float* part_ml;
+    const float* gate;
+    float* out;
+    int64_t gate_seq_stride, gate_head_stride;
+    int32_t n_kv, n_q, group, hg;
+};
+
+// One work-group per (entry, q head); thread = head-dim element.
+__global__ __launch_bounds__(kHd) void decode_attn_merge_kernel(const MergeParams P) {
+    const int e = blockIdx.x / P.n_q;
+    const int h = blockIdx.x % P.n_q;
+    const int kvh = h / P.group;
+    const int hl = h % P.group;
+    const int hc = hl / P.hg;
+    const int hh = hl % P.hg;
+    const int splits = P.b.splits[e];
+    const int wg0 = P.b.wg_base[e] + hc * splits * P.n_kv + kvh;
+    const int d = threadIdx.x;
+    float mx = -INFINITY;
+    for (int s = 0; s < splits; ++s) {
+        const size_t wg = (size_t)(wg0 + s * P.n_kv);
+        mx = fmaxf(mx, P.part_ml[(wg * P.hg + hh) * 2]);
+    }
+    float acc = 0.0f, lsum = 0.0f;
+    for (int s = 0; s < splits; ++s) {
+        const size_t wg = (size_t)(wg0 + s * P.n_kv);
+        const float ms = P.part_ml[(wg * P.hg + hh) * 2];
+        const float f = ms == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(ms - mx);
+        acc = fmaf(f, P.part_o[(wg * P.hg + hh) * kHd + d], acc);
+        lsum = fmaf(f, P.part_ml[(wg * P.hg + hh) * 2 + 1], lsum);
+    }
+    float r = lsum > 0.0f ? acc / lsum : 0.0f;
+    if (P.gate) {
+        const float g = P.gate[(size_t)e * P.gate_seq_stride + (size_t)h * P.gate_head_stride + d];
+        // sigmoid in the overflow-free form of the reference (qsa/cpu.rs:84-91)
+        float sg;
+        if (g >= 0.0f) {
+            sg = 1.0f / (1.0f + expf(-g));
+        } else {
+            const float t = expf(g);
+            sg = t / (1.0f + t);
+        }
+        r *= sg;
+    }
+    P.out[((size_t)e * P.n_q + h) * kHd + d] = r;
+}
+
+}  // namespace
+
+int32_t attn_heads_per_wave(int32_t group) { return group % 8 == 0 ? 8 : 4; }
+
+int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b) {
+    const int32_t n_kv = p->g.n_kv;
+    const int32_t group = n_q_head / n_kv;
+    const int32_t hg = attn_heads_per_wave(group);
+    const int32_t n_hc = (group + hg - 1) / hg;
+    const int64_t per_page = (int64_t)n_kv * n_hc;
+    int64_t total_pages = 0;
+    for (int i = 0; i < b.n; ++i) total_pages += b.pos[i] / kPage + 1;
+    // Two work-groups stay resident per CU (register budget); aim at one generation.
+    const int64_t target = (int64_t)(p->n_cu > 0 ? p->n_cu : 256) * 2;
+    int64_t pps = (total_pages * per_page + target - 1) / target;
+    pps = ((pps + kWaves - 1) / kWaves) * kWaves;
+    if (pps < kWaves) pps = kWaves;
+    for (;;) {
+        int64_t total = 0;
+        for (int i = 0; i < b.n; ++i) {
+            const int64_t pages = b.pos[i] / kPage + 1;
+            int64_t splits = (pages + pps - 1) / pps;
+            // even the ranges out inside the entry, keeping whole groups of kWaves pages
+            int64_t each = (pages + splits - 1) / splits;
+            each = ((each + kWaves - 1) / kWaves) * kWaves;
+            splits = (pages + each - 1) / each;
+            b.splits[i] = (int32_t)splits;
+            b.pps[i] = (int32_t)each;
+            b.wg_base[i] = (int32_t)total;
+            total += splits * per_page;
+        }
+        b.wg_base[b.n] = (int32_t)total;
+        if (total <= p->max_wgs) return (int32_t)total;
+        pps *= 2;
+    }
+}
+
+hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, const AttnArgs& a,
+                              hipStream_t stream) {
+    const int32_t n_kv = p->g.n_kv;
+    const int32_t group = a.n_q_head / n_kv;
+    const int32_t hg = attn_heads_per_wave(group);
+    AttnKernelParams kp;
+    kp.b = b;
+    kp.kpool = reinterpret_cast<const uint16_t*>(p->k_layer[(size_t)layer]);
+    kp.vpool = reinterpret_cast<const uint16_t*>(p->v_layer[(size_t)layer]);
+    kp.tables = p->table_dev;
+    kp.q = a.q;
+    kp.part_o = p->part_o;
+    kp.part_ml = p->part_ml;
+    kp.max_pages_per_seq = p->desc.max_pages_per_seq;
+    kp.n_kv = n_kv;
+    kp.n_q = a.n_q_head;
+    kp.group = group;
+    kp.n_hc = (group + hg - 1) / hg;
+    kp.scale_log2e = a.scale * kLog2e;
+    const int32_t total = b.wg_base[b.n];
+    {
+        StageScope timed(p, BKV_STAGE_ATTN_SPLIT, stream);
+        if (hg == 8)
+            decode_attn_f16_kernel<8><<<total, kBlock, 0, stream>>>(kp);
+        else
+            decode_attn_f16_kernel<4><<<total, kBlock, 0, stream>>>(kp);
+    }
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return err;
+
+    MergeParams mp;
+    mp.b = b;
+    mp.part_o = p->part_o;
+    mp.part_ml = p->part_ml;
+    mp.gate = a.gate;
+    mp.out = a.out;
+    mp.gate_seq_stride = a.gate_seq_stride;
+    mp.gate_head_stride = a.gate_head_stride;
+    mp.n_kv = n_kv;
+    mp.n_q = a.n_q_head;
+    mp.group = group;
+    mp.hg = hg;
+    {
+        StageScope timed(p, BKV_STAGE_ATTN_MERGE, stream);
+        decode_attn_merge_kernel<<<b.n * a.n_q_head, kHd, 0, stream>>>(mp);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace bkv

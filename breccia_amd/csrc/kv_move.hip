@@ -1,0 +1,487 @@
+// Byte-moving kernels of the paged-KV path for gfx950: K/V append through the block
+// table (three row encodings), copy-on-write page copy, page gather/scatter for the
+// host swap, a dequantising row gather for parity checks, and small utilities.
+// All of it is HBM-bound; the rules that matter are 16-byte accesses, whole-line
+// coalescing and several independent loads in flight per lane.
+#include "bkv_internal.hpp"
+
+namespace bkv {
+
+namespace {
+
+constexpr int kBlock = 256;
+
+// f32 -> binary16 code under the cache's storage rule
+// (crates/breccia-kernels/shaders/f16_storage.glsl:26-55, qsa/cpu.rs:23-53):
+// round-to-nearest-even like the hardware convert, except that every |x| < 2^-14
+// becomes a signed zero (no subnormals, even where rounding would reach 2^-14) and
+// NaN becomes a signed infinity.
+__device__ __forceinline__ uint32_t f16_store_bits(float x) {
+    const uint32_t b = __float_as_uint(x);
+    const uint32_t sign = (b >> 16) & 0x8000u;
+    const uint32_t mag = b & 0x7fffffffu;
+    const _Float16 h = static_cast<_Float16>(x);  // v_cvt_f16_f32, RNE, overflow -> inf
+    uint32_t code = static_cast<uint32_t>(__builtin_bit_cast(uint16_t, h));
+    if (mag < 0x38800000u) code = sign;
+    if (mag > 0x7f800000u) code = sign | 0x7c00u;
+    return code;
+}
+
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    return f16_store_bits(lo) | (f16_store_bits(hi) << 16);
+}
+
+// binary16 code -> f32 under the cache's load rule (f16_storage.glsl:58-69):
+// exponent field 0 reads as a signed zero.
+__device__ __forceinline__ float f16_load(uint32_t h) {
+    const uint32_t sign = (h & 0x8000u) << 16;
+    const uint32_t e = (h >> 10) & 0x1fu;
+    const uint32_t m = h & 0x3ffu;
+    if (e == 0) return __uint_as_float(sign);
+    if (e == 31) return __uint_as_float(sign | 0x7f800000u | (m << 13));
+    return __uint_as_float(sign | ((e + 112u) << 23) | (m << 13));
+}
+
+struct MoveGeom {
+    int32_t n_kv, hd, page_cells, max_pages_per_seq;
+};
+
+// ---- append, f16 rows ---------------------------------------------------------
+// One lane converts 8 consecutive elements of one (token, kv head) row of K and of V:
+// two 16-byte loads and one 16-byte store per pool.  grid.y = sequence of the call.
+__global__ __launch_bounds__(kBlock) void append_f16_kernel(AppendBatch b, MoveGeom g,
+                                                            uint16_t* __restrict__ kpool,
+                                                            uint16_t* __restrict__ vpool,
+                                                            const int32_t* __restrict__ tables,
+                                                            const float* __restrict__ k,
+                                                            const float* __restrict__ v) {
+    const int s = blockIdx.y;
+    const int lanes_per_tok = g.n_kv * g.hd / 8;
+    const int64_t unit = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const int64_t t = unit / lanes_per_tok;
+    if (t >= b.n_tok[s]) return;
+    const int r = (int)(unit % lanes_per_tok);  // 8-element group within [n_kv][hd]
+    const int kvh = (r * 8) / g.hd;
+    const int d0 = (r * 8) % g.hd;
+    const int64_t cell = (int64_t)b.pos0[s] + t;
+    const int32_t phys =
+        tables[(size_t)b.row[s] * (size_t)g.max_pages_per_seq + (size_t)(cell / g.page_cells)];
+    const int in_page = (int)(cell % g.page_cells);
+    const size_t row = ((size_t)phys * g.n_kv + kvh) * g.page_cells + in_page;
+    const size_t dst = row * (size_t)g.hd + d0;
+    const size_t src = ((size_t)b.src0[s] + (size_t)t) * (size_t)(g.n_kv * g.hd) + (size_t)r * 8;
+
+    const float4 k0 = *reinterpret_cast<const float4*>(k + src);
+    const float4 k1 = *reinterpret_cast<const float4*>(k + src + 4);
+    const float4 v0 = *reinterpret_cast<const float4*>(v + src);
+    const float4 v1 = *reinterpret_cast<const float4*>(v + src + 4);
+    uint4 ko, vo;
+    ko.x = pack2(k0.x, k0.y);
+    ko.y = pack2(k0.z, k0.w);
+    ko.z = pack2(k1.x, k1.y);
+    ko.w = pack2(k1.z, k1.w);
+    vo.x = pack2(v0.x, v0.y);
+    vo.y = pack2(v0.z, v0.w);
+    vo.z = pack2(v1.x, v1.y);
+    vo.w = pack2(v1.z, v1.w);
+    *reinterpret_cast<uint4*>(kpool + dst) = ko;
+    *reinterpret_cast<uint4*>(vpool + dst) = vo;
+}
+
+// q8_0 codes of 32 values (shaders/qsa_kv_append.comp:113-132, qsa/cpu.rs:65-82):
+// scale = amax/127 (1 if amax == 0), q = round-half-away(clamp(x/scale, +-127)).
+__device__ __forceinline__ void q8_block(const float (&x)[32], float scale, uint32_t (&w)[8]) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        uint32_t packed = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float t = x[j * 4 + i] / scale;
+            t = t < -127.0f ? -127.0f : t;
+            t = t > 127.0f ? 127.0f : t;
+            const int q = (int)roundf(t);
+            packed |= ((uint32_t)q & 0xffu) << (8 * i);
+        }
+        w[j] = packed;
+    }
+}
+
+__device__ __forceinline__ float amax32(const float (&x)[32]) {
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+        const float a = fabsf(x[i]);
+        amax = a > amax ? a : amax;
+    }
+    return amax;
+}
+
+__device__ __forceinline__ void load32(const float* p, float (&x)[32]) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float4 f = reinterpret_cast<const float4*>(p)[i];
+        x[i * 4 + 0] = f.x;
+        x[i * 4 + 1] = f.y;
+        x[i * 4 + 2] = f.z;
+        x[i * 4 + 3] = f.w;
+    }
+}
+
+// ---- append, reference q8_0-V rows: K f16, V [f32 scale][32 x i8] per 32 values ---
+// One lane per (token, kv head, 32-element block), as the reference shader does.
+__global__ __launch_bounds__(kBlock) void append_q8v_kernel(AppendBatch b, MoveGeom g,
+                                                            uint16_t* __restrict__ kpool,
+                                                            uint32_t* __restrict__ vpool,
+                                                            const int32_t* __restrict__ tables,
+                                                            const float* __restrict__ k,
+                                                            const float* __restrict__ v) {
+    const int s = blockIdx.y;
+    const int blocks = g.hd / 32;
+    const int lanes_per_tok = g.n_kv * blocks;
+    const int64_t unit = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const int64_t t = unit / lanes_per_tok;
+    if (t >= b.n_tok[s]) return;
+    const int r = (int)(unit % lanes_per_tok);
+    const int kvh = r / blocks;
+    const int blk = r % blocks;
+    const int64_t cell = (int64_t)b.pos0[s] + t;
+    const int32_t phys =
+        tables[(size_t)b.row[s] * (size_t)g.max_pages_per_seq + (size_t)(cell / g.page_cells)];
+    const int in_page = (int)(cell % g.page_cells);
+    const size_t row = ((size_t)phys * g.n_kv + kvh) * g.page_cells + in_page;
+    const size_t src = ((size_t)b.src0[s] + (size_t)t) * (size_t)(g.n_kv * g.hd) +
+                       (size_t)kvh * g.hd + (size_t)blk * 32;
+    float x[32];
+    load32(k + src, x);
+    uint4* kd = reinterpret_cast<uint4*>(kpool + row * (size_t)g.hd + (size_t)blk * 32);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        uint4 o;
+        o.x = pack2(x[i * 8 + 0], x[i * 8 + 1]);
+        o.y = pack2(x[i * 8 + 2], x[i * 8 + 3]);
+        o.z = pack2(x[i * 8 + 4], x[i * 8 + 5]);
+        o.w = pack2(x[i * 8 + 6], x[i * 8 + 7]);
+        kd[i] = o;
+    }
+    load32(v + src, x);
+    const float amax = amax32(x);
+    const float scale = amax > 0.0f ? amax / 127.0f : 1.0f;
+    uint32_t w[8];
+    q8_block(x, scale, w);
+    uint32_t* vd = vpool + (row * (size_t)blocks + (size_t)blk) * 9u;
+    vd[0] = __float_as_uint(scale);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) vd[1 + j] = w[j];
+}
+
+// ---- append, int8 K and V with f16 scales: row = [hd x i8][hd/32 x f16] -----------
+// The q8_0 rule with the scale stored through the cache's f16 encoding; a scale the
+// f16 rule would flush is raised to 2^-14.  (No reference counterpart.)
+__device__ __forceinline__ void i8h_block(const float* src, uint8_t* row_base, int hd, int blk) {
+    float x[32];
+    load32(src, x);
+    const float amax = amax32(x);
+    uint32_t hb;
+    if (amax > 0.0f) {
+        hb = f16_store_bits(amax / 127.0f);
+        if ((hb & 0x7fffu) == 0) hb = 0x0400u;
+    } else {
+        hb = 0x3c00u;
+    }
+    const float sh = f16_load(hb);
+    uint32_t w[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        uint32_t packed = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float t = x[j * 4 + i] / sh;
+            t = !(t >= -127.0f) ? -127.0f : t;
+            t = t > 127.0f ? 127.0f : t;
+            const int q = (int)roundf(t);
+            packed |= ((uint32_t)q & 0xffu) << (8 * i);
+        }
+        w[j] = packed;
+    }
+    uint4* qd = reinterpret_cast<uint4*>(row_base + (size_t)blk * 32);
+    qd[0] = make_uint4(w[0], w[1], w[2], w[3]);
+    qd[1] = make_uint4(w[4], w[5], w[6], w[7]);
+    *reinterpret_cast<uint16_t*>(row_base + hd + blk * 2) = (uint16_t)hb;
+}
+
+__global__ __launch_bounds__(kBlock) void append_i8h_kernel(AppendBatch b, MoveGeom g,
+                                                            uint8_t* __restrict__ kpool,
+                                                            uint8_t* __restrict__ vpool,
+                                                            const int32_t* __restrict__ tables,
+                                                            const float* __restrict__ k,
+                                                            const float* __restrict__ v) {
+    const int s = blockIdx.y;
+    const int blocks = g.hd / 32;
+    const int lanes_per_tok = g.n_kv * blocks * 2;  // K and V blocks
+    const int64_t unit = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const int64_t t = unit / lanes_per_tok;
+    if (t >= b.n_tok[s]) return;
+    int r = (int)(unit % lanes_per_tok);
+    const int which = r / (g.n_kv * blocks);
+    r %= g.n_kv * blocks;
+    const int kvh = r / blocks;
+    const int blk = r % blocks;
+    const int64_t cell = (int64_t)b.pos0[s] + t;
+    const int32_t phys =
+        tables[(size_t)b.row[s] * (size_t)g.max_pages_per_seq + (size_t)(cell / g.page_cells)];
+    const int in_page = (int)(cell % g.page_cells);
+    const size_t row = ((size_t)phys * g.n_kv + kvh) * g.page_cells + in_page;
+    const size_t src = ((size_t)b.src0[s] + (size_t)t) * (size_t)(g.n_kv * g.hd) +
+                       (size_t)kvh * g.hd + (size_t)blk * 32;
+    const size_t row_bytes = (size_t)g.hd + (size_t)blocks * 2;
+    i8h_block((which ? v : k) + src, (which ? vpool : kpool) + row * row_bytes, g.hd, blk);
+}
+
+// ---- whole-page moves -----------------------------------------------------------
+// Four independent 16-byte loads per lane, then four stores: one work-group moves up
+// to 16 KiB, which is one f16 K or V page.
+__device__ __forceinline__ void move_bytes16(const uint4* __restrict__ src, uint4* __restrict__ dst,
+                                             uint32_t n_vec, uint32_t base) {
+    uint4 r[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t idx = base + (uint32_t)i * kBlock + threadIdx.x;
+        if (idx < n_vec) r[i] = src[idx];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t idx = base + (uint32_t)i * kBlock + threadIdx.x;
+        if (idx < n_vec) dst[idx] = r[i];
+    }
+}
+
+struct PoolPtrs {
+    uint8_t* slab;
+    uint64_t layer_stride;  // bytes between consecutive layers
+    uint64_t v_offset;      // offset of a layer's V pool behind its K pool
+    uint64_t k_page_bytes, v_page_bytes;
+    int32_t n_layers;
+};
+
+// grid.y = pair * n_layers * 2 + layer * 2 + which; grid.x = 16 KiB chunk of the page.
+__global__ __launch_bounds__(kBlock) void page_copy_kernel(PoolPtrs pp,
+                                                           const bkv_page_pair* __restrict__ pairs) {
+    const uint32_t u = blockIdx.y;
+    const uint32_t which = u & 1u;
+    const uint32_t layer = (u >> 1) % (uint32_t)pp.n_layers;
+    const uint32_t pair = (u >> 1) / (uint32_t)pp.n_layers;
+    const uint64_t pb = which ? pp.v_page_bytes : pp.k_page_bytes;
+    const uint32_t n_vec = (uint32_t)(pb / 16);
+    const uint32_t base = blockIdx.x * (4u * kBlock);
+    if (base >= n_vec) return;
+    uint8_t* pool = pp.slab + (uint64_t)layer * pp.layer_stride + (which ? pp.v_offset : 0);
+    const bkv_page_pair pr = pairs[pair];
+    move_bytes16(reinterpret_cast<const uint4*>(pool + (uint64_t)pr.src * pb),
+                 reinterpret_cast<uint4*>(pool + (uint64_t)pr.dst * pb), n_vec, base);
+}
+
+// Staging layout: [page i][layer][K page bytes | V page bytes].
+__global__ __launch_bounds__(kBlock) void page_stage_kernel(PoolPtrs pp,
+                                                            const int32_t* __restrict__ pages,
+                                                            uint8_t* __restrict__ stage,
+                                                            int to_stage) {
+    const uint32_t u = blockIdx.y;
+    const uint32_t which = u & 1u;
+    const uint32_t layer = (u >> 1) % (uint32_t)pp.n_layers;
+    const uint32_t i = (u >> 1) / (uint32_t)pp.n_layers;
+    const uint64_t pb = which ? pp.v_page_bytes : pp.k_page_bytes;
+    const uint32_t n_vec = (uint32_t)(pb / 16);
+    const uint32_t base = blockIdx.x * (4u * kBlock);
+    if (base >= n_vec) return;
+    uint8_t* pool = pp.slab + (uint64_t)layer * pp.layer_stride + (which ? pp.v_offset : 0) +
+                    (uint64_t)pages[i] * pb;
+    const uint64_t slab_bytes = (pp.k_page_bytes + pp.v_page_bytes) * (uint64_t)pp.n_layers;
+    uint8_t* st = stage + (uint64_t)i * slab_bytes +
+                  (uint64_t)layer * (pp.k_page_bytes + pp.v_page_bytes) +
+                  (which ? pp.k_page_bytes : 0);
+    if (to_stage)
+        move_bytes16(reinterpret_cast<const uint4*>(pool), reinterpret_cast<uint4*>(st), n_vec, base);
+    else
+        move_bytes16(reinterpret_cast<const uint4*>(st), reinterpret_cast<uint4*>(pool), n_vec, base);
+}
+
+// ---- dequantising gather (parity / debugging; one lane per element) ---------------
+__global__ __launch_bounds__(kBlock) void gather_kernel(MoveGeom g, int layout,
+                                                        const uint8_t* __restrict__ kpool,
+                                                        const uint8_t* __restrict__ vpool,
+                                                        const int32_t* __restrict__ table_row,
+                                                        int64_t cell0, int64_t n,
+                                                        float* __restrict__ k_out,
+                                                        float* __restrict__ v_out) {
+    const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const int64_t total = n * g.n_kv * g.hd;
+    if (idx >= total) return;
+    const int d = (int)(idx % g.hd);
+    const int kvh = (int)((idx / g.hd) % g.n_kv);
+    const int64_t i = idx / ((int64_t)g.hd * g.n_kv);
+    const int64_t cell = cell0 + i;
+    const int32_t phys = table_row[cell / g.page_cells];
+    const size_t row = ((size_t)phys * g.n_kv + kvh) * g.page_cells + (size_t)(cell % g.page_cells);
+    float kv, vv;
+    if (layout == BKV_LAYOUT_I8H) {
+        const size_t rb = (size_t)g.hd + (size_t)(g.hd / 32) * 2;
+        const uint8_t* kr = kpool + row * rb;
+        const uint8_t* vr = vpool + row * rb;
+        const uint32_t ks = *reinterpret_cast<const uint16_t*>(kr + g.hd + (d / 32) * 2);
+        const uint32_t vs = *reinterpret_cast<const uint16_t*>(vr + g.hd + (d / 32) * 2);
+        kv = (float)(int8_t)kr[d] * f16_load(ks);
+        vv = (float)(int8_t)vr[d] * f16_load(vs);
+    } else {
+        kv = f16_load(reinterpret_cast<const uint16_t*>(kpool)[row * (size_t)g.hd + d]);
+        if (layout == BKV_LAYOUT_F16) {
+            vv = f16_load(reinterpret_cast<const uint16_t*>(vpool)[row * (size_t)g.hd + d]);
+        } else {
+            const uint32_t* w =
+                reinterpret_cast<const uint32_t*>(vpool) + (row * (size_t)(g.hd / 32) + d / 32) * 9u;
+            const int j = d % 32;
+            const int8_t q = (int8_t)((w[1 + j / 4] >> (8 * (j % 4))) & 0xffu);
+            vv = (float)q * __uint_as_float(w[0]);
+        }
+    }
+    k_out[idx] = kv;
+    v_out[idx] = vv;
+}
+
+__global__ __launch_bounds__(kBlock) void table_scatter_kernel(int32_t* __restrict__ table,
+                                                               const TableUpdate* __restrict__ upd,
+                                                               int32_t n) {
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    // Updates are applied in order of their index only within one launch when offsets
+    // are distinct; the host collapses repeated offsets before uploading.
+    if (i < n) table[upd[i].offset] = upd[i].value;
+}
+
+__global__ __launch_bounds__(kBlock) void fill_kernel(uint4* __restrict__ dst, uint64_t n_vec,
+                                                      uint32_t word) {
+    const uint4 w = make_uint4(word, word, word, word);
+    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n_vec;
+         i += (uint64_t)gridDim.x * kBlock)
+        dst[i] = w;
+}
+
+__global__ __launch_bounds__(kBlock) void copy_probe_kernel(uint4* __restrict__ dst,
+                                                            const uint4* __restrict__ src,
+                                                            uint64_t n_vec) {
+    const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+    uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    for (; i + 3 * stride < n_vec; i += 4 * stride) {
+        const uint4 a = src[i], b = src[i + stride], c = src[i + 2 * stride],
+                    d = src[i + 3 * stride];
+        dst[i] = a;
+        dst[i + stride] = b;
+        dst[i + 2 * stride] = c;
+        dst[i + 3 * stride] = d;
+    }
+    for (; i < n_vec; i += stride) dst[i] = src[i];
+}
+
+MoveGeom move_geom(const bkv_pool* p) {
+    return MoveGeom{p->g.n_kv, p->g.hd, p->g.page_cells, p->desc.max_pages_per_seq};
+}
+
+PoolPtrs pool_ptrs(const bkv_pool* p) {
+    PoolPtrs pp;
+    pp.slab = p->slab;
+    pp.layer_stride = p->g.k_pool_bytes + p->g.v_pool_bytes;
+    pp.v_offset = p->g.k_pool_bytes;
+    pp.k_page_bytes = p->g.k_page_bytes;
+    pp.v_page_bytes = p->g.v_page_bytes;
+    pp.n_layers = p->g.n_layers;
+    return pp;
+}
+
+}  // namespace
+
+hipError_t launch_append(const bkv_pool* p, int32_t layer, const AppendBatch& b, int32_t max_tok,
+                         const float* k, const float* v, hipStream_t stream) {
+    const MoveGeom g = move_geom(p);
+    int lanes_per_tok;
+    switch (p->g.layout) {
+        case BKV_LAYOUT_F16: lanes_per_tok = g.n_kv * g.hd / 8; break;
+        case BKV_LAYOUT_Q8V: lanes_per_tok = g.n_kv * g.hd / 32; break;
+        default: lanes_per_tok = g.n_kv * g.hd / 32 * 2; break;
+    }
+    const int64_t lanes = (int64_t)max_tok * lanes_per_tok;
+    dim3 grid((unsigned)((lanes + kBlock - 1) / kBlock), (unsigned)b.n);
+    uint8_t* kp = p->k_layer[(size_t)layer];
+    uint8_t* vp = p->v_layer[(size_t)layer];
+    switch (p->g.layout) {
+        case BKV_LAYOUT_F16:
+            append_f16_kernel<<<grid, kBlock, 0, stream>>>(b, g, (uint16_t*)kp, (uint16_t*)vp,
+                                                          p->table_dev, k, v);
+            break;
+        case BKV_LAYOUT_Q8V:
+            append_q8v_kernel<<<grid, kBlock, 0, stream>>>(b, g, (uint16_t*)kp, (uint32_t*)vp,
+                                                          p->table_dev, k, v);
+            break;
+        default:
+            append_i8h_kernel<<<grid, kBlock, 0, stream>>>(b, g, kp, vp, p->table_dev, k, v);
+            break;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_page_copy(const bkv_pool* p, const bkv_page_pair* pairs_dev, int32_t n_pairs,
+                            hipStream_t stream) {
+    const PoolPtrs pp = pool_ptrs(p);
+    const uint64_t pb = pp.k_page_bytes > pp.v_page_bytes ? pp.k_page_bytes : pp.v_page_bytes;
+    const unsigned chunks = (unsigned)((pb / 16 + 4 * kBlock - 1) / (4 * kBlock));
+    // grid.y is limited to 65535: callers pass at most kMaxPairsPerLaunch pairs.
+    dim3 grid(chunks, (unsigned)n_pairs * (unsigned)pp.n_layers * 2u);
+    page_copy_kernel<<<grid, kBlock, 0, stream>>>(pp, pairs_dev);
+    return hipGetLastError();
+}
+
+hipError_t launch_page_stage(const bkv_pool* p, const int32_t* pages_dev, int32_t n_pages,
+                             uint8_t* stage, int to_stage, hipStream_t stream) {
+    const PoolPtrs pp = pool_ptrs(p);
+    const uint64_t pb = pp.k_page_bytes > pp.v_page_bytes ? pp.k_page_bytes : pp.v_page_bytes;
+    const unsigned chunks = (unsigned)((pb / 16 + 4 * kBlock - 1) / (4 * kBlock));
+    dim3 grid(chunks, (unsigned)n_pages * (unsigned)pp.n_layers * 2u);
+    page_stage_kernel<<<grid, kBlock, 0, stream>>>(pp, pages_dev, stage, to_stage);
+    return hipGetLastError();
+}
+
+hipError_t launch_gather(const bkv_pool* p, int32_t layer, int32_t row, int64_t cell0, int64_t n,
+                         float* k_out, float* v_out, hipStream_t stream) {
+    const MoveGeom g = move_geom(p);
+    const int64_t total = n * g.n_kv * g.hd;
+    if (total == 0) return hipSuccess;
+    const unsigned grid = (unsigned)((total + kBlock - 1) / kBlock);
+    gather_kernel<<<grid, kBlock, 0, stream>>>(
+        g, p->g.layout, p->k_layer[(size_t)layer], p->v_layer[(size_t)layer],
+        p->table_dev + (size_t)row * (size_t)p->desc.max_pages_per_seq, cell0, n, k_out, v_out);
+    return hipGetLastError();
+}
+
+hipError_t launch_table_scatter(int32_t* table, const TableUpdate* upd_dev, int32_t n,
+                                hipStream_t stream) {
+    if (n == 0) return hipSuccess;
+    table_scatter_kernel<<<(n + kBlock - 1) / kBlock, kBlock, 0, stream>>>(table, upd_dev, n);
+    return hipGetLastError();
+}
+
+hipError_t launch_fill(void* dst, uint64_t bytes, uint32_t word, hipStream_t stream) {
+    const uint64_t n_vec = bytes / 16;
+    if (n_vec == 0) return hipSuccess;
+    uint64_t blocks = (n_vec + kBlock - 1) / kBlock;
+    if (blocks > 16384) blocks = 16384;
+    fill_kernel<<<(unsigned)blocks, kBlock, 0, stream>>>((uint4*)dst, n_vec, word);
+    return hipGetLastError();
+}
+
+hipError_t launch_copy_probe(void* dst, const void* src, uint64_t bytes, hipStream_t stream) {
+    const uint64_t n_vec = bytes / 16;
+    if (n_vec == 0) return hipSuccess;
+    uint64_t blocks = (n_vec + 4 * kBlock - 1) / (4 * kBlock);
+    if (blocks > 8192) blocks = 8192;
+    copy_probe_kernel<<<(unsigned)blocks, kBlock, 0, stream>>>((uint4*)dst, (const uint4*)src, n_vec);
+    return hipGetLastError();
+}
+
+}  // namespace bkv

@@ -1,0 +1,352 @@
+"""Thin Python host layer over the C ABI: device buffers, streams, events and the pool.
+
+Everything numerical happens in libbreccia_kv.so; this module only marshals numpy
+arrays and integers into the C calls and turns status codes into exceptions.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from . import lib as L
+from .lib import BkvError, PagePair, PoolDesc, check, lib  # noqa: F401
+
+
+def _i32(a):
+    a = np.ascontiguousarray(a, dtype=np.int32)
+    return a, a.ctypes.data_as(C.POINTER(C.c_int32))
+
+
+def _i64(a):
+    a = np.ascontiguousarray(a, dtype=np.int64)
+    return a, a.ctypes.data_as(C.POINTER(C.c_int64))
+
+
+class Stream:
+    def __init__(self):
+        h = C.c_void_p()
+        check(lib.bkv_stream_create(C.byref(h)))
+        self.handle = h
+
+    def sync(self) -> None:
+        check(lib.bkv_stream_sync(self.handle))
+
+    def close(self) -> None:
+        if self.handle:
+            check(lib.bkv_stream_destroy(self.handle))
+            self.handle = None
+
+
+class Event:
+    def __init__(self):
+        h = C.c_void_p()
+        check(lib.bkv_event_create(C.byref(h)))
+        self.handle = h
+
+    def record(self, stream=None) -> None:
+        check(lib.bkv_event_record(self.handle, _sh(stream)))
+
+    def sync(self) -> None:
+        check(lib.bkv_event_sync(self.handle))
+
+    def elapsed_ms(self, stop: "Event") -> float:
+        ms = C.c_float()
+        check(lib.bkv_event_elapsed_ms(self.handle, stop.handle, C.byref(ms)))
+        return float(ms.value)
+
+    def close(self) -> None:
+        if self.handle:
+            check(lib.bkv_event_destroy(self.handle))
+            self.handle = None
+
+
+def _sh(stream):
+    return stream.handle if isinstance(stream, Stream) else stream
+
+
+def device_sync() -> None:
+    check(lib.bkv_device_sync())
+
+
+def device_info():
+    name = C.create_string_buffer(256)
+    cu = C.c_int32()
+    mem = C.c_uint64()
+    check(lib.bkv_device_info(name, 256, C.byref(cu), C.byref(mem)))
+    return name.value.decode(), int(cu.value), int(mem.value)
+
+
+class DeviceBuffer:
+    """A hipMalloc'd region with numpy upload/download."""
+
+    def __init__(self, nbytes: int):
+        self.nbytes = int(nbytes)
+        p = C.c_void_p()
+        check(lib.bkv_dev_alloc(self.nbytes, C.byref(p)))
+        self.ptr = p
+
+    @classmethod
+    def from_numpy(cls, a: np.ndarray, stream=None) -> "DeviceBuffer":
+        a = np.ascontiguousarray(a)
+        buf = cls(max(a.nbytes, 16))
+        buf.upload(a, stream)
+        return buf
+
+    def upload(self, a: np.ndarray, stream=None, offset: int = 0) -> None:
+        a = np.ascontiguousarray(a)
+        assert offset + a.nbytes <= self.nbytes
+        if a.nbytes == 0:
+            return
+        check(lib.bkv_memcpy_h2d(C.c_void_p(self.ptr.value + offset), a.ctypes.data, a.nbytes,
+                                 _sh(stream)))
+        check(lib.bkv_stream_sync(_sh(stream)))
+
+    def download(self, dtype, count: int | None = None, stream=None, offset: int = 0) -> np.ndarray:
+        dt = np.dtype(dtype)
+        if count is None:
+            count = (self.nbytes - offset) // dt.itemsize
+        out = np.empty(count, dtype=dt)
+        if out.nbytes:
+            assert offset + out.nbytes <= self.nbytes
+            check(lib.bkv_memcpy_d2h(out.ctypes.data, C.c_void_p(self.ptr.value + offset),
+                                     out.nbytes, _sh(stream)))
+            check(lib.bkv_stream_sync(_sh(stream)))
+        return out
+
+    def at(self, offset: int) -> C.c_void_p:
+        return C.c_void_p(self.ptr.value + offset)
+
+    def free(self) -> None:
+        if self.ptr:
+            check(lib.bkv_dev_free(self.ptr))
+            self.ptr = None
+
+
+class Pool:
+    """bkv_pool handle.  Method names follow the C entry points."""
+
+    def __init__(self, n_layers=1, n_pages=512, n_kv_head=2, head_dim=256, page_cells=16,
+                 layout=L.LAYOUT_F16, max_seqs=16, max_pages_per_seq=None, host_only=False):
+        if max_pages_per_seq is None:
+            max_pages_per_seq = n_pages
+        self.desc = PoolDesc(n_layers, n_pages, n_kv_head, head_dim, page_cells, layout, max_seqs,
+                             max_pages_per_seq, L.POOL_HOST_ONLY if host_only else 0)
+        h = C.c_void_p()
+        check(lib.bkv_pool_create(C.byref(self.desc), C.byref(h)))
+        self.handle = h
+
+    # -- lifecycle
+    def destroy(self) -> None:
+        if self.handle:
+            check(lib.bkv_pool_destroy(self.handle))
+            self.handle = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.destroy()
+
+    def reset(self, stream=None) -> None:
+        check(lib.bkv_pool_reset(self.handle, _sh(stream)))
+
+    def fill(self, byte: int, stream=None) -> None:
+        check(lib.bkv_pool_fill(self.handle, byte, _sh(stream)))
+
+    def bytes(self) -> int:
+        return int(lib.bkv_pool_bytes(self.handle))
+
+    def page_bytes(self, which: int) -> int:
+        return int(lib.bkv_page_bytes(self.handle, which))
+
+    def swap_page_bytes(self) -> int:
+        return int(lib.bkv_swap_page_bytes(self.handle))
+
+    def layer_ptr(self, layer: int, which: int):
+        p = C.c_void_p()
+        n = C.c_uint64()
+        check(lib.bkv_pool_layer_ptr(self.handle, layer, which, C.byref(p), C.byref(n)))
+        return p, int(n.value)
+
+    def read_layer(self, layer: int, which: int, stream=None) -> np.ndarray:
+        """Bytes of one layer's K (0) or V (1) pool."""
+        p, n = self.layer_ptr(layer, which)
+        out = np.empty(n, dtype=np.uint8)
+        check(lib.bkv_memcpy_d2h(out.ctypes.data, p, n, _sh(stream)))
+        check(lib.bkv_stream_sync(_sh(stream)))
+        return out
+
+    def write_layer(self, layer: int, which: int, data: np.ndarray, stream=None) -> None:
+        p, n = self.layer_ptr(layer, which)
+        data = np.ascontiguousarray(data).view(np.uint8).reshape(-1)
+        assert data.nbytes == n
+        check(lib.bkv_memcpy_h2d(p, data.ctypes.data, n, _sh(stream)))
+        check(lib.bkv_stream_sync(_sh(stream)))
+
+    # -- allocator
+    def seq_create(self) -> int:
+        s = C.c_int32()
+        check(lib.bkv_seq_create(self.handle, C.byref(s)))
+        return int(s.value)
+
+    def seq_create_identity(self, n_pages: int) -> int:
+        s = C.c_int32()
+        check(lib.bkv_seq_create_identity(self.handle, n_pages, C.byref(s)))
+        return int(s.value)
+
+    def seq_fork(self, parent: int, n_tokens: int) -> int:
+        s = C.c_int32()
+        check(lib.bkv_seq_fork(self.handle, parent, n_tokens, C.byref(s)))
+        return int(s.value)
+
+    def seq_free(self, seq: int) -> None:
+        check(lib.bkv_seq_free(self.handle, seq))
+
+    def seq_reserve(self, seq: int, new_len: int, cow_capacity: int = 4):
+        """Returns the list of (src, dst) copy-on-write pairs the caller must page_copy."""
+        pairs = (PagePair * max(cow_capacity, 1))()
+        n = C.c_int32()
+        check(lib.bkv_seq_reserve(self.handle, seq, new_len, pairs, cow_capacity, C.byref(n)))
+        return [(pairs[i].src, pairs[i].dst) for i in range(n.value)]
+
+    def seq_truncate(self, seq: int, new_len: int) -> None:
+        check(lib.bkv_seq_truncate(self.handle, seq, new_len))
+
+    def seq_len(self, seq: int) -> int:
+        return int(lib.bkv_seq_len(self.handle, seq))
+
+    def seq_capacity(self, seq: int) -> int:
+        return int(lib.bkv_seq_capacity(self.handle, seq))
+
+    def seq_n_pages(self, seq: int) -> int:
+        return int(lib.bkv_seq_n_pages(self.handle, seq))
+
+    def block_table(self, seq: int) -> np.ndarray:
+        n = self.seq_n_pages(seq)
+        if n < 0:
+            raise BkvError(L.ERR_RANGE, "sequence %d is not live" % seq)
+        p = lib.bkv_seq_block_table(self.handle, seq)
+        return np.ctypeslib.as_array(p, shape=(max(n, 1),))[:n].copy()
+
+    def page_refcount(self, page: int) -> int:
+        return int(lib.bkv_page_refcount(self.handle, page))
+
+    def free_pages(self) -> int:
+        return int(lib.bkv_pool_free_pages(self.handle))
+
+    def check(self) -> None:
+        check(lib.bkv_pool_check(self.handle))
+
+    def set_free_order(self, order) -> None:
+        order, po = _i32(order)
+        check(lib.bkv_pool_set_free_order(self.handle, po, order.size))
+
+    # -- per-kernel timing
+    def timing_enable(self, on: bool) -> None:
+        check(lib.bkv_timing_enable(self.handle, 1 if on else 0))
+
+    def timing_reset(self) -> None:
+        check(lib.bkv_timing_reset(self.handle))
+
+    def timing_read(self, stage: int):
+        n = C.c_uint64()
+        ms = C.c_double()
+        check(lib.bkv_timing_read(self.handle, stage, C.byref(n), C.byref(ms)))
+        return int(n.value), float(ms.value)
+
+    # -- hot path
+    def append(self, layer: int, seqs, pos0, n_tokens, k_dev, v_dev, stream=None) -> None:
+        seqs, ps = _i32(seqs)
+        pos0, pp = _i64(pos0)
+        n_tokens, pn = _i32(n_tokens)
+        assert seqs.size == pos0.size == n_tokens.size
+        check(lib.bkv_append(self.handle, layer, seqs.size, ps, pp, pn, _ptr(k_dev), _ptr(v_dev),
+                             _sh(stream)))
+
+    def decode_attn(self, layer: int, seqs, pos, n_q_head: int, q_dev, out_dev, scale: float,
+                    gate_dev=None, gate_seq_stride: int = 0, gate_head_stride: int = 0,
+                    stream=None) -> None:
+        seqs, ps = _i32(seqs)
+        pos, pp = _i64(pos)
+        assert seqs.size == pos.size
+        check(lib.bkv_decode_attn(self.handle, layer, seqs.size, ps, pp, n_q_head, _ptr(q_dev),
+                                  _ptr(gate_dev), gate_seq_stride, gate_head_stride, scale,
+                                  _ptr(out_dev), _sh(stream)))
+
+    def page_copy(self, pairs, stream=None) -> None:
+        pairs = list(pairs)
+        arr = (PagePair * max(len(pairs), 1))()
+        for i, (s, d) in enumerate(pairs):
+            arr[i].src, arr[i].dst = int(s), int(d)
+        check(lib.bkv_page_copy(self.handle, arr, len(pairs), _sh(stream)))
+
+    def gather(self, layer: int, seq: int, cell0: int, n: int, stream=None):
+        """Dequantised K and V rows as float32 arrays [n, n_kv, head_dim]."""
+        shape = (n, self.desc.n_kv_head, self.desc.head_dim)
+        count = int(np.prod(shape))
+        kb = DeviceBuffer(max(count * 4, 16))
+        vb = DeviceBuffer(max(count * 4, 16))
+        try:
+            check(lib.bkv_gather(self.handle, layer, seq, cell0, n, kb.ptr, vb.ptr, _sh(stream)))
+            k = kb.download(np.float32, count, stream).reshape(shape)
+            v = vb.download(np.float32, count, stream).reshape(shape)
+        finally:
+            kb.free()
+            vb.free()
+        return k, v
+
+    # -- swap
+    def host_alloc(self, nbytes: int) -> "PinnedBuffer":
+        return PinnedBuffer(self, nbytes)
+
+    def swap_out(self, pages, host: "PinnedBuffer", stream=None) -> None:
+        pages, pp = _i32(pages)
+        assert pages.size * self.swap_page_bytes() <= host.nbytes
+        check(lib.bkv_swap_out(self.handle, pp, pages.size, host.ptr, _sh(stream)))
+
+    def swap_in(self, pages, host: "PinnedBuffer", stream=None) -> None:
+        pages, pp = _i32(pages)
+        assert pages.size * self.swap_page_bytes() <= host.nbytes
+        check(lib.bkv_swap_in(self.handle, pp, pages.size, host.ptr, _sh(stream)))
+
+    def swap_wait(self) -> None:
+        check(lib.bkv_swap_wait(self.handle))
+
+    def swap_fence(self, stream=None) -> None:
+        check(lib.bkv_swap_fence(self.handle, _sh(stream)))
+
+    def seq_evict(self, seq: int, lp0: int, n: int, host: "PinnedBuffer", stream=None) -> None:
+        assert n * self.swap_page_bytes() <= host.nbytes
+        check(lib.bkv_seq_evict(self.handle, seq, lp0, n, host.ptr, _sh(stream)))
+
+    def seq_restore(self, seq: int, lp0: int, n: int, host: "PinnedBuffer", stream=None) -> None:
+        assert n * self.swap_page_bytes() <= host.nbytes
+        check(lib.bkv_seq_restore(self.handle, seq, lp0, n, host.ptr, _sh(stream)))
+
+
+class PinnedBuffer:
+    """hipHostMalloc'd memory owned through the pool, viewable as a numpy array."""
+
+    def __init__(self, pool: Pool, nbytes: int):
+        self.pool, self.nbytes = pool, int(nbytes)
+        p = C.c_void_p()
+        check(lib.bkv_host_alloc(pool.handle, self.nbytes, C.byref(p)))
+        self.ptr = p
+
+    def view(self) -> np.ndarray:
+        buf = (C.c_uint8 * self.nbytes).from_address(self.ptr.value)
+        return np.frombuffer(buf, dtype=np.uint8)
+
+    def free(self) -> None:
+        if self.ptr:
+            check(lib.bkv_host_free(self.pool.handle, self.ptr))
+            self.ptr = None
+
+
+def _ptr(x):
+    if x is None:
+        return None
+    if isinstance(x, DeviceBuffer):
+        return x.ptr
+    return x

@@ -1,0 +1,124 @@
+"""ctypes binding of libbreccia_kv.so -- one Python function per C entry point.
+
+There is no fallback: if the HIP library has not been built, importing this module
+raises.  Nothing here computes anything on the CPU.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libbreccia_kv.so")
+HEADER_PATH = os.path.join(HERE, "..", "include", "breccia_kv.h")
+
+OK, ERR_INVALID, ERR_RANGE, ERR_NO_PAGES, ERR_STATE, ERR_NO_DEVICE, ERR_HIP, ERR_NOMEM = range(8)
+STATUS_NAMES = ["OK", "INVALID", "RANGE", "NO_PAGES", "STATE", "NO_DEVICE", "HIP", "NOMEM"]
+LAYOUT_F16, LAYOUT_Q8V, LAYOUT_I8H = 0, 1, 2
+POOL_HOST_ONLY = 1
+MAX_BATCH = 64
+STAGE_APPEND, STAGE_ATTN_SPLIT, STAGE_ATTN_MERGE, STAGE_PAGE_COPY = range(4)
+
+
+class BkvError(RuntimeError):
+    def __init__(self, status: int, message: str):
+        super().__init__("BKV_ERR_%s: %s" % (STATUS_NAMES[status], message))
+        self.status = status
+        self.message = message
+
+
+class PoolDesc(C.Structure):
+    _fields_ = [("n_layers", C.c_int32), ("n_pages", C.c_int32), ("n_kv_head", C.c_int32),
+                ("head_dim", C.c_int32), ("page_cells", C.c_int32), ("layout", C.c_int32),
+                ("max_seqs", C.c_int32), ("max_pages_per_seq", C.c_int32), ("flags", C.c_uint32)]
+
+
+class PagePair(C.Structure):
+    _fields_ = [("src", C.c_int32), ("dst", C.c_int32)]
+
+
+def _load() -> C.CDLL:
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            "libbreccia_kv.so is not built (%s). Build it with `python -m breccia_amd.build` "
+            "(needs hipcc); there is no CPU fallback." % LIB_PATH)
+    return C.CDLL(LIB_PATH)
+
+
+lib = _load()
+
+_vp, _i32, _i64, _u64, _f32 = C.c_void_p, C.c_int32, C.c_int64, C.c_uint64, C.c_float
+_pi32, _pi64 = C.POINTER(C.c_int32), C.POINTER(C.c_int64)
+
+_SIGNATURES = {
+    "bkv_last_error": (C.c_char_p, []),
+    "bkv_version": (C.c_char_p, []),
+    "bkv_pool_create": (C.c_int, [C.POINTER(PoolDesc), C.POINTER(_vp)]),
+    "bkv_pool_destroy": (C.c_int, [_vp]),
+    "bkv_pool_reset": (C.c_int, [_vp, _vp]),
+    "bkv_pool_get_desc": (C.c_int, [_vp, C.POINTER(PoolDesc)]),
+    "bkv_pool_bytes": (_u64, [_vp]),
+    "bkv_page_bytes": (_u64, [_vp, C.c_int]),
+    "bkv_pool_fill": (C.c_int, [_vp, C.c_int, _vp]),
+    "bkv_pool_layer_ptr": (C.c_int, [_vp, _i32, C.c_int, C.POINTER(_vp), C.POINTER(_u64)]),
+    "bkv_seq_create": (C.c_int, [_vp, _pi32]),
+    "bkv_seq_create_identity": (C.c_int, [_vp, _i32, _pi32]),
+    "bkv_seq_fork": (C.c_int, [_vp, _i32, _i64, _pi32]),
+    "bkv_seq_free": (C.c_int, [_vp, _i32]),
+    "bkv_seq_reserve": (C.c_int, [_vp, _i32, _i64, C.POINTER(PagePair), _i32, _pi32]),
+    "bkv_seq_truncate": (C.c_int, [_vp, _i32, _i64]),
+    "bkv_seq_len": (_i64, [_vp, _i32]),
+    "bkv_seq_capacity": (_i64, [_vp, _i32]),
+    "bkv_seq_n_pages": (_i32, [_vp, _i32]),
+    "bkv_seq_block_table": (_pi32, [_vp, _i32]),
+    "bkv_page_refcount": (_i32, [_vp, _i32]),
+    "bkv_pool_free_pages": (_i32, [_vp]),
+    "bkv_pool_check": (C.c_int, [_vp]),
+    "bkv_pool_set_free_order": (C.c_int, [_vp, _pi32, _i32]),
+    "bkv_timing_enable": (C.c_int, [_vp, C.c_int]),
+    "bkv_timing_reset": (C.c_int, [_vp]),
+    "bkv_timing_read": (C.c_int, [_vp, C.c_int, C.POINTER(_u64), C.POINTER(C.c_double)]),
+    "bkv_append": (C.c_int, [_vp, _i32, _i32, _pi32, _pi64, _pi32, _vp, _vp, _vp]),
+    "bkv_decode_attn": (C.c_int, [_vp, _i32, _i32, _pi32, _pi64, _i32, _vp, _vp, _i64, _i64, _f32,
+                                  _vp, _vp]),
+    "bkv_page_copy": (C.c_int, [_vp, C.POINTER(PagePair), _i32, _vp]),
+    "bkv_swap_page_bytes": (_u64, [_vp]),
+    "bkv_host_alloc": (C.c_int, [_vp, _u64, C.POINTER(_vp)]),
+    "bkv_host_free": (C.c_int, [_vp, _vp]),
+    "bkv_swap_out": (C.c_int, [_vp, _pi32, _i32, _vp, _vp]),
+    "bkv_swap_in": (C.c_int, [_vp, _pi32, _i32, _vp, _vp]),
+    "bkv_swap_wait": (C.c_int, [_vp]),
+    "bkv_swap_fence": (C.c_int, [_vp, _vp]),
+    "bkv_seq_evict": (C.c_int, [_vp, _i32, _i32, _i32, _vp, _vp]),
+    "bkv_seq_restore": (C.c_int, [_vp, _i32, _i32, _i32, _vp, _vp]),
+    "bkv_gather": (C.c_int, [_vp, _i32, _i32, _i64, _i64, _vp, _vp, _vp]),
+    "bkv_dev_alloc": (C.c_int, [_u64, C.POINTER(_vp)]),
+    "bkv_dev_free": (C.c_int, [_vp]),
+    "bkv_memcpy_h2d": (C.c_int, [_vp, _vp, _u64, _vp]),
+    "bkv_memcpy_d2h": (C.c_int, [_vp, _vp, _u64, _vp]),
+    "bkv_stream_create": (C.c_int, [C.POINTER(_vp)]),
+    "bkv_stream_destroy": (C.c_int, [_vp]),
+    "bkv_stream_sync": (C.c_int, [_vp]),
+    "bkv_device_sync": (C.c_int, []),
+    "bkv_event_create": (C.c_int, [C.POINTER(_vp)]),
+    "bkv_event_destroy": (C.c_int, [_vp]),
+    "bkv_event_record": (C.c_int, [_vp, _vp]),
+    "bkv_event_sync": (C.c_int, [_vp]),
+    "bkv_event_elapsed_ms": (C.c_int, [_vp, _vp, C.POINTER(C.c_float)]),
+    "bkv_device_info": (C.c_int, [C.c_char_p, _i32, _pi32, C.POINTER(_u64)]),
+    "bkv_copy_probe": (C.c_int, [_vp, _vp, _u64, _vp]),
+}
+
+for _name, (_res, _args) in _SIGNATURES.items():
+    _fn = getattr(lib, _name)
+    _fn.restype = _res
+    _fn.argtypes = _args
+
+
+def last_error() -> str:
+    return lib.bkv_last_error().decode("utf-8", "replace")
+
+
+def check(status: int) -> None:
+    if status != OK:
+        raise BkvError(status, last_error())

@@ -1,0 +1,248 @@
+/*
+ * breccia_kv.h -- C ABI of the MI355X paged-KV library (libbreccia_kv.so).
+ *
+ * One GPU, one process.  Every entry point returns a bkv_status; on failure
+ * bkv_last_error() holds a thread-local message naming the failing check.  Every
+ * size / range violation is a host-side error returned BEFORE anything is
+ * launched (the reference's contract: crates/breccia-kernels/src/qsa/mod.rs:
+ * 1108-1116, :405-409, :929-931) -- never a device fault.
+ *
+ * Calls that take a `stream` only enqueue work on it (the HIP analogue of the
+ * reference recording into a device's open batch, crates/breccia-kernels/src/
+ * ops/mod.rs:205-222): results are visible to later work on the same stream.
+ * `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ *
+ * Reference items each group replaces are cited per declaration; paths are
+ * relative to the reference tree, `qsa/` = crates/breccia-kernels/src/qsa/.
+ */
+#ifndef BRECCIA_KV_H
+#define BRECCIA_KV_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum bkv_status {
+    BKV_OK = 0,
+    BKV_ERR_INVALID = 1,    /* bad argument / geometry */
+    BKV_ERR_RANGE = 2,      /* position, page or sequence out of range */
+    BKV_ERR_NO_PAGES = 3,   /* allocator exhausted */
+    BKV_ERR_STATE = 4,      /* refcount / ownership / residency rule violated */
+    BKV_ERR_NO_DEVICE = 5,  /* pool was created host-only, or HIP is unusable */
+    BKV_ERR_HIP = 6,        /* a HIP runtime call failed (message names it) */
+    BKV_ERR_NOMEM = 7       /* host or pinned-host allocation failed */
+} bkv_status;
+
+/* How K and V rows are stored.  qsa/mod.rs:242-254 (VLayout). */
+typedef enum bkv_layout {
+    BKV_LAYOUT_F16 = 0, /* f16 K and V: 2 B / element (reference default)                */
+    BKV_LAYOUT_Q8V = 1, /* f16 K; V as q8_0 blocks [f32 scale][32 x i8] = 36 B / 32 values
+                           (reference BRECCIA_KV_Q8V, shaders/qsa_kv_append.comp:38-44) */
+    BKV_LAYOUT_I8H = 2  /* int8 K and V, row = [head_dim x i8][head_dim/32 x f16 scale],
+                           34 B / 32 values (no reference counterpart)                   */
+} bkv_layout;
+
+enum {
+    BKV_POOL_HOST_ONLY = 1u /* allocator + block tables only; device calls fail with
+                               BKV_ERR_NO_DEVICE (for hosts without a GPU) */
+};
+
+#define BKV_MAX_BATCH 64      /* (sequence, position) entries per append / attention call */
+#define BKV_MAX_HEAD_GROUP 16 /* q heads per kv head */
+
+/* Pool geometry.  One pool = n_layers x (K pool, V pool), each laid out exactly as
+ * the reference's k_pool / v_pool (qsa/mod.rs:20-35):
+ *   row  = (page * n_kv_head + kv_head) * page_cells + cell % page_cells
+ *   f16 element index = row * head_dim + d   (u32 word = index / 2, even = low half)
+ * plus a device-resident int32 block table per sequence (the reference's
+ * `page_table`, one u32 per logical page).  Page ids are shared by all layers. */
+typedef struct bkv_pool_desc {
+    int32_t n_layers;
+    int32_t n_pages;
+    int32_t n_kv_head;
+    int32_t head_dim;           /* multiple of 32, <= 256; kernels are tuned for 256 */
+    int32_t page_cells;         /* 16 */
+    int32_t layout;             /* bkv_layout */
+    int32_t max_seqs;           /* live sequences the block-table arena holds */
+    int32_t max_pages_per_seq;  /* block-table row length */
+    uint32_t flags;             /* BKV_POOL_* */
+} bkv_pool_desc;
+
+typedef struct bkv_pool bkv_pool;
+
+typedef struct bkv_page_pair {
+    int32_t src;
+    int32_t dst;
+} bkv_page_pair;
+
+/* ---- errors / version ------------------------------------------------------ */
+const char *bkv_last_error(void);
+const char *bkv_version(void);
+
+/* ---- pool lifecycle ---------------------------------------------------------
+ * Replaces QsaState::with_layout / reset / bytes / release (qsa/mod.rs:399-535,
+ * :551-570, :572-585, :591-602).  Pools are zeroed at creation and by reset, as in
+ * the reference; reset also frees every sequence. */
+bkv_status bkv_pool_create(const bkv_pool_desc *desc, bkv_pool **out);
+bkv_status bkv_pool_destroy(bkv_pool *pool);
+bkv_status bkv_pool_reset(bkv_pool *pool, void *stream);
+bkv_status bkv_pool_get_desc(const bkv_pool *pool, bkv_pool_desc *out);
+uint64_t bkv_pool_bytes(const bkv_pool *pool);              /* device bytes held */
+uint64_t bkv_page_bytes(const bkv_pool *pool, int which);   /* one layer; 0 = K, 1 = V */
+/* Fill every K/V pool byte with `byte` (the reference's BRECCIA_FAULT_POISON_QSA
+ * knob fills with NaN words, qsa/mod.rs:509-523; 0xff bytes are NaN in f16 and f32). */
+bkv_status bkv_pool_fill(bkv_pool *pool, int byte, void *stream);
+/* Raw device base of one layer's K (which=0) or V (which=1) pool, for callers that
+ * dump or diff pool bytes (the reference's BRECCIA_DUMP_*, graph.rs:2204-2229). */
+bkv_status bkv_pool_layer_ptr(const bkv_pool *pool, int32_t layer, int which, void **dev_ptr,
+                              uint64_t *bytes);
+
+/* ---- page allocator / block tables (host side) -----------------------------
+ * No reference implementation exists (docs/plan/PDF-GAP-ANALYSIS.md:56-60); shaped by
+ * the reference's design notes (docs/reference-engines/02-kv-and-context.md:543-548,
+ * :566-581, :617-620): 16-token pages, {id, refcount, free queue}, only whole pages
+ * move, a page is in exactly one tier.  A sequence handle is a small integer. */
+bkv_status bkv_seq_create(bkv_pool *pool, int32_t *seq_out);
+/* A sequence whose logical page i is physical page i for i < n_pages: the
+ * reference's identity page table (qsa/mod.rs:477-481). */
+bkv_status bkv_seq_create_identity(bkv_pool *pool, int32_t n_pages, int32_t *seq_out);
+/* Child shares every page of the parent's first `n_tokens` cells (refcount + 1). */
+bkv_status bkv_seq_fork(bkv_pool *pool, int32_t parent, int64_t n_tokens, int32_t *child_out);
+bkv_status bkv_seq_free(bkv_pool *pool, int32_t seq);
+/* Make cells [0, new_len) addressable and cells [len, new_len) privately writable:
+ * allocates missing pages; if the page holding cell `len` is shared (refcount > 1)
+ * and partially filled, it is replaced by a fresh page and (old, new) is reported in
+ * cow_pairs -- the caller must bkv_page_copy those pairs before appending.  A shared
+ * page that no other sequence holds any more (refcount back to 1) is written in place.
+ * On BKV_ERR_NO_PAGES nothing is changed. */
+bkv_status bkv_seq_reserve(bkv_pool *pool, int32_t seq, int64_t new_len, bkv_page_pair *cow_pairs,
+                           int32_t cow_capacity, int32_t *n_cow);
+/* Set the sequence's length without touching pages (speculative rollback:
+ * rejected cells are simply overwritten later, docs/specs/qwen4exp-architecture.md:750-759). */
+bkv_status bkv_seq_truncate(bkv_pool *pool, int32_t seq, int64_t new_len);
+int64_t bkv_seq_len(const bkv_pool *pool, int32_t seq);           /* -1 on error */
+int64_t bkv_seq_capacity(const bkv_pool *pool, int32_t seq);      /* cells addressable */
+int32_t bkv_seq_n_pages(const bkv_pool *pool, int32_t seq);
+/* Host view of the block table (valid until the next allocator call); entry -1 =
+ * page swapped out. */
+const int32_t *bkv_seq_block_table(const bkv_pool *pool, int32_t seq);
+int32_t bkv_page_refcount(const bkv_pool *pool, int32_t page);    /* -1 on error */
+int32_t bkv_pool_free_pages(const bkv_pool *pool);
+/* Self-check of the allocator's invariants (sum of refcounts == table entries, free
+ * list disjoint from live pages, ...).  BKV_OK or BKV_ERR_STATE with a message. */
+bkv_status bkv_pool_check(const bkv_pool *pool);
+/* Placement hook: make the free queue hand pages out in `order`, which must be a
+ * permutation of the pages that are free right now (fragmentation studies, tests). */
+bkv_status bkv_pool_set_free_order(bkv_pool *pool, const int32_t *order, int32_t n);
+
+/* ---- hot path ---------------------------------------------------------------
+ * bkv_append replaces Qsa::kv_append + shaders/qsa_kv_append.comp (qsa/mod.rs:
+ * 1105-1156): scatter n_tokens[i] new rows of sequence seqs[i] to cells pos0[i]..
+ * through its block table, f32 -> cache encoding (f16 rule of shaders/
+ * f16_storage.glsl:26-55; q8_0 rule of qsa_kv_append.comp:87-132).
+ * k, v: device f32 [sum n_tokens][n_kv_head][head_dim], sequences concatenated in
+ * call order.  Error if pos0+n_tokens exceeds the cells reserved for the sequence.
+ * Does not change bkv_seq_len; call bkv_seq_reserve first. */
+bkv_status bkv_append(bkv_pool *pool, int32_t layer, int32_t n_seqs, const int32_t *seqs,
+                      const int64_t *pos0, const int32_t *n_tokens, const float *k_dev,
+                      const float *v_dev, void *stream);
+
+/* bkv_decode_attn replaces Qsa::attend + Qsa::apply for decode shapes with the dense
+ * selection (qsa/mod.rs:1382-1462, :1466-1522; shaders qsa_attn_scores_small,
+ * ops_softmax, qsa_attn_apply_split, qsa_attn_apply_reduce; oracle qsa/cpu.rs:197-246):
+ *   out[i][h][:] = sigmoid(gate[i][h][:]) * softmax_c(scale * q[i][h] . K[c]) . V[c],
+ *   c over cells 0..pos[i] of sequence seqs[i], kv head = h * n_kv_head / n_q_head.
+ * q, out: device f32 [n][n_q_head][head_dim].  gate_dev may be NULL (factor omitted);
+ * otherwise gate(i,h,d) = gate_dev[i*gate_seq_stride + h*gate_head_stride + d] (the
+ * reference reads it in place from q_full at h*512+256+d, shaders/qsa_attn_apply.comp).
+ * The same sequence may appear several times with different pos (T > 1 decode).
+ * One split-K online-softmax kernel plus one merge kernel; partials live in a
+ * workspace the pool owns. */
+bkv_status bkv_decode_attn(bkv_pool *pool, int32_t layer, int32_t n, const int32_t *seqs,
+                           const int64_t *pos, int32_t n_q_head, const float *q_dev,
+                           const float *gate_dev, int64_t gate_seq_stride,
+                           int64_t gate_head_stride, float scale, float *out_dev, void *stream);
+
+/* Copy-on-write page copy: for every pair and every layer, K and V bytes of page
+ * `src` -> page `dst`.  No reference implementation (nearest: dispatch_batch.rs:
+ * 1130-1150 record_copy).  Pairs are host memory; dst pages must be distinct. */
+bkv_status bkv_page_copy(bkv_pool *pool, const bkv_page_pair *pairs, int32_t n_pairs,
+                         void *stream);
+
+/* ---- VRAM <-> pinned host swap ------------------------------------------------
+ * No reference implementation (nearest: gemv.rs:1023-1071 staging download/upload).
+ * Host slab of one page = for each layer: [K page bytes][V page bytes]
+ * (bkv_swap_page_bytes).  Device-side gather/scatter runs on `stream`; the PCIe
+ * copy is a hipMemcpyAsync on the pool's side stream, fenced with events both ways.
+ * bkv_swap_wait blocks the host until the side stream is idle; bkv_swap_fence makes
+ * `stream` wait for it without blocking the host. */
+uint64_t bkv_swap_page_bytes(const bkv_pool *pool);
+bkv_status bkv_host_alloc(bkv_pool *pool, uint64_t bytes, void **host_out); /* hipHostMalloc */
+bkv_status bkv_host_free(bkv_pool *pool, void *host);
+/* Raw moves of physical pages (no allocator bookkeeping). */
+bkv_status bkv_swap_out(bkv_pool *pool, const int32_t *pages, int32_t n, void *pinned_host,
+                        void *stream);
+bkv_status bkv_swap_in(bkv_pool *pool, const int32_t *pages, int32_t n, const void *pinned_host,
+                       void *stream);
+bkv_status bkv_swap_wait(bkv_pool *pool);
+bkv_status bkv_swap_fence(bkv_pool *pool, void *stream);
+/* Allocator-aware eviction of logical pages [lp0, lp0+n) of a sequence: each must be
+ * complete and held only by this sequence; bytes go to pinned_host, the physical
+ * pages return to the free list and the table entries become -1.  Restore allocates
+ * fresh pages (ids may differ) and copies the bytes back. */
+bkv_status bkv_seq_evict(bkv_pool *pool, int32_t seq, int32_t lp0, int32_t n, void *pinned_host,
+                         void *stream);
+bkv_status bkv_seq_restore(bkv_pool *pool, int32_t seq, int32_t lp0, int32_t n,
+                           const void *pinned_host, void *stream);
+
+/* ---- parity / debugging -------------------------------------------------------
+ * Dequantised rows of cells [cell0, cell0+n) as f32 [n][n_kv_head][head_dim] in
+ * the flat order the reference's CPU attend consumes (qsa/cpu.rs:219-222). */
+bkv_status bkv_gather(bkv_pool *pool, int32_t layer, int32_t seq, int64_t cell0, int64_t n,
+                      float *k_out_dev, float *v_out_dev, void *stream);
+
+/* ---- per-kernel GPU timing ------------------------------------------------------
+ * The analogue of Qsa::stage_timings / Pipe::run_timed (qsa/mod.rs:1733-1970,
+ * ops/mod.rs:251-274): while enabled, every hot-path call brackets each of its
+ * kernels with events on the call's stream.  bkv_timing_read waits for the recorded
+ * events and returns launches and summed milliseconds of one stage since the last
+ * reset.  Adds event-record gaps between kernels: do not leave it on in production. */
+typedef enum bkv_stage {
+    BKV_STAGE_APPEND = 0,
+    BKV_STAGE_ATTN_SPLIT = 1, /* split-K online-softmax kernel (the dominant one) */
+    BKV_STAGE_ATTN_MERGE = 2,
+    BKV_STAGE_PAGE_COPY = 3,
+    BKV_STAGE_COUNT = 4
+} bkv_stage;
+bkv_status bkv_timing_enable(bkv_pool *pool, int on);
+bkv_status bkv_timing_reset(bkv_pool *pool);
+bkv_status bkv_timing_read(bkv_pool *pool, int stage, uint64_t *launches, double *total_ms);
+
+/* ---- device plumbing for hosts without their own HIP bindings ---------------- */
+bkv_status bkv_dev_alloc(uint64_t bytes, void **dev_out);
+bkv_status bkv_dev_free(void *dev);
+bkv_status bkv_memcpy_h2d(void *dev, const void *host, uint64_t bytes, void *stream);
+bkv_status bkv_memcpy_d2h(void *host, const void *dev, uint64_t bytes, void *stream);
+bkv_status bkv_stream_create(void **stream_out);
+bkv_status bkv_stream_destroy(void *stream);
+bkv_status bkv_stream_sync(void *stream);
+bkv_status bkv_device_sync(void);
+bkv_status bkv_event_create(void **event_out);
+bkv_status bkv_event_destroy(void *event);
+bkv_status bkv_event_record(void *event, void *stream);
+bkv_status bkv_event_sync(void *event);
+bkv_status bkv_event_elapsed_ms(void *start, void *stop, float *ms_out);
+/* name (<= 255 chars), compute units, total device memory */
+bkv_status bkv_device_info(char *name_out, int32_t name_cap, int32_t *cu_out,
+                           uint64_t *mem_bytes_out);
+/* Reference bandwidth probe: a plain 16-byte-vector device copy of `bytes` bytes
+ * (used to scale profiler byte counters and to report the copy ceiling). */
+bkv_status bkv_copy_probe(void *dst_dev, const void *src_dev, uint64_t bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BRECCIA_KV_H */

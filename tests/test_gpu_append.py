@@ -1,0 +1,194 @@
+"""GPU parity of paged K/V append, gather and the pool lifecycle against the CPU oracle.
+Bit-exact: every byte of every pool is compared."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from breccia_amd import lib as L
+from breccia_amd.kv import BkvError, DeviceBuffer, Stream, device_sync
+from gpu_common import Twin
+
+pytestmark = pytest.mark.gpu
+GOLD = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_kats.json")))
+
+
+def test_reference_layout_recipe_on_the_gpu():
+    # crates/breccia-kernels/tests/attn_conformance.rs:1172-1275: identity table, capacity 40,
+    # 33 single-token appends from cell 5; every stored half must be the cache encoding.
+    r = GOLD["layout_recipe"]
+    with Twin(n_pages=3, max_seqs=2) as tw:
+        s = tw.pool.seq_create_identity(3)
+        i = np.arange(512)
+        for t in range(r["n_tokens"]):
+            cell = r["start_cell"] + t
+            k = (np.sin((cell * 97 + i * 13).astype(np.float32) * np.float32(0.017)) * np.float32(3.0)).astype(np.float32)
+            v = (np.cos((cell * 61 + i * 7).astype(np.float32) * np.float32(0.031)) * np.float32(2.0)).astype(np.float32)
+            tw.append(0, [s], [cell], [k], [v])
+        tw.assert_pools_equal()
+        kp = tw.pool.read_layer(0, 0).view(np.uint16).reshape(3, 2, 16, 256)
+        assert kp[0, :, :5].sum() == 0 and kp[2, :, 6:].sum() == 0   # unwritten cells still zero
+        # the reference's capacity error (qsa/mod.rs:1108-1116)
+        z = DeviceBuffer(4096)
+        with pytest.raises(BkvError) as ei:
+            tw.pool.append(0, [s], [47], [2], z, z)
+        assert ei.value.status == L.ERR_RANGE
+        z.free()
+
+
+def test_batched_ragged_append_through_permuted_tables():
+    rng = np.random.Generator(np.random.PCG64(31))
+    with Twin(n_pages=256, max_seqs=8) as tw:
+        perm = rng.permutation(256)
+        seqs = [tw.pool.seq_create() for _ in range(5)]
+        lens = [37, 0, 512, 1000, 16]
+        # scramble physical pages: reserve in interleaved steps so tables are not contiguous
+        for step in range(0, 1100, 48):
+            for s, n in zip(seqs, lens):
+                tgt = min(n, step + 48)
+                if tgt > tw.pool.seq_len(s):
+                    tw.pool.seq_reserve(s, tgt)
+        ks = [rng.standard_normal((n, 2, 256)).astype(np.float32) for n in lens]
+        vs = [rng.standard_normal((n, 2, 256)).astype(np.float32) for n in lens]
+        tw.append(0, seqs, [0] * 5, ks, vs)          # one ragged call, one empty sequence
+        tw.assert_pools_equal()
+        # decode-style step: one token each where there is room, crossing page boundaries
+        for s in seqs:
+            tw.pool.seq_reserve(s, tw.pool.seq_len(s) + 1)
+        k1 = [rng.standard_normal((1, 2, 256)).astype(np.float32) for _ in seqs]
+        v1 = [rng.standard_normal((1, 2, 256)).astype(np.float32) for _ in seqs]
+        tw.append(0, seqs, lens, k1, v1)
+        tw.assert_pools_equal()
+        # gather == the f16 round trip of what went in
+        gk, gv = tw.pool.gather(0, seqs[3], 990, 11)
+        want_k = oracle.to_f16(np.concatenate([ks[3][990:], k1[3]]))
+        assert np.array_equal(gk, want_k)
+        ok, ov = tw.images[0].gather(tw.pool.block_table(seqs[3]), 990, 11)
+        assert np.array_equal(gk, ok) and np.array_equal(gv, ov)
+        tw.pool.check()
+
+
+def test_special_values_follow_the_cache_f16_rule():
+    # crates/breccia-kernels/shaders/f16_storage.glsl:26-55: below 2^-14 -> +-0, NaN -> +-inf,
+    # >= 65520 -> inf, ties to even
+    bits = []
+    for centre in (0x38800000, 0x477FE000, 0x477FF000, 0x00800000, 0x7F800000, 0x33000000):
+        bits.append(np.arange(centre - 512, centre + 512, dtype=np.uint32))
+    exps = np.arange(256, dtype=np.uint32) << np.uint32(23)
+    man = np.array([0, 1, 0xFFF, 0x1000, 0x1001, 0x2FFF, 0x3000, 0x3001, 0x7FEFFF, 0x7FF000, 0x7FFFFF],
+                   dtype=np.uint32)
+    bits.append((exps[:, None] | man[None, :]).reshape(-1))
+    b = np.concatenate(bits)
+    b = np.concatenate([b, b | np.uint32(0x80000000)])
+    rng = np.random.Generator(np.random.PCG64(8))
+    pad = (-b.size) % 512
+    b = np.concatenate([b, rng.integers(0, 2**32, size=pad, dtype=np.uint64).astype(np.uint32)])
+    x = b.view(np.float32).reshape(-1, 2, 256)
+    T = x.shape[0]
+    with Twin(n_pages=(T + 15) // 16 + 1, max_seqs=2) as tw:
+        s = tw.pool.seq_create()
+        tw.pool.seq_reserve(s, T)
+        tw.append(0, [s], [0], [x], [x[::-1].copy()])
+        tw.assert_pools_equal()
+
+
+def test_random_bit_patterns_two_million():
+    rng = np.random.Generator(np.random.PCG64(77))
+    T = 4096
+    x = rng.integers(0, 2**32, size=(T, 2, 256), dtype=np.uint64).astype(np.uint32).view(np.float32)
+    y = rng.integers(0, 2**32, size=(T, 2, 256), dtype=np.uint64).astype(np.uint32).view(np.float32)
+    with Twin(n_pages=T // 16, max_seqs=2) as tw:
+        s = tw.pool.seq_create()
+        tw.pool.seq_reserve(s, T)
+        tw.append(0, [s], [0], [x], [y])
+        tw.assert_pools_equal()
+
+
+def test_prefill_chunks_equal_token_by_token_appends():
+    rng = np.random.Generator(np.random.PCG64(4))
+    k = rng.standard_normal((300, 2, 256)).astype(np.float32)
+    v = rng.standard_normal((300, 2, 256)).astype(np.float32)
+    with Twin(n_pages=64, max_seqs=4) as tw:
+        a, b = tw.pool.seq_create(), tw.pool.seq_create()
+        tw.pool.seq_reserve(a, 303)
+        tw.pool.seq_reserve(b, 303)
+        tw.append(0, [a], [3], [k], [v])
+        kd, vd = DeviceBuffer.from_numpy(k), DeviceBuffer.from_numpy(v)
+        for t in range(300):  # T x append(1) straight through the C ABI, no sync in between
+            tw.pool.append(0, [b], [3 + t], [1], kd.at(t * 2048), vd.at(t * 2048))
+        device_sync()
+        ka, va = tw.pool.gather(0, a, 0, 303)
+        kb, vb = tw.pool.gather(0, b, 0, 303)
+        assert np.array_equal(ka, kb) and np.array_equal(va, vb)
+        kd.free()
+        vd.free()
+
+
+@pytest.mark.parametrize("layout", [L.LAYOUT_Q8V, L.LAYOUT_I8H])
+def test_quantised_append_is_bit_exact(layout):
+    # q8_0 V: crates/breccia-kernels/shaders/qsa_kv_append.comp:87-132, qsa/cpu.rs:65-82
+    rng = np.random.Generator(np.random.PCG64(12 + layout))
+    with Twin(n_pages=96, layout=layout, max_seqs=4) as tw:
+        perm_owner = tw.pool.seq_create()
+        tw.pool.seq_reserve(perm_owner, 16 * 7)     # shift the next sequence's pages
+        s = tw.pool.seq_create()
+        lens = 517
+        tw.pool.seq_reserve(s, lens)
+        k = (rng.standard_normal((lens, 2, 256)) * rng.uniform(0.01, 20, size=(lens, 2, 1))).astype(np.float32)
+        v = (rng.standard_normal((lens, 2, 256)) * rng.uniform(0.01, 20, size=(lens, 2, 1))).astype(np.float32)
+        v[5, 0, 32:64] = 0.0                        # an all-zero block keeps scale 1
+        k[9, 1, :32] *= 1e-5                        # a scale the f16 rule would flush
+        tw.append(0, [s], [0], [k[:500]], [v[:500]])
+        tw.append(0, [s], [500], [k[500:]], [v[500:]])
+        tw.assert_pools_equal()
+        gk, gv = tw.pool.gather(0, s, 0, lens)
+        ok, ov = tw.images[0].gather(tw.pool.block_table(s), 0, lens)
+        assert np.array_equal(gk, ok) and np.array_equal(gv, ov)
+
+
+def test_enqueue_on_a_stream_equals_sync_after_every_call():
+    # the reference's batching contract (crates/breccia-kernels/tests/batching.rs:27-88):
+    # six dependent operations recorded back to back == the same six run one at a time
+    rng = np.random.Generator(np.random.PCG64(6))
+    k = [rng.standard_normal((t, 2, 256)).astype(np.float32) for t in (40, 1, 1, 25, 1, 1)]
+    v = [rng.standard_normal((t, 2, 256)).astype(np.float32) for t in (40, 1, 1, 25, 1, 1)]
+    images = []
+    for sync_each in (False, True):
+        with Twin(n_pages=16, max_seqs=2) as tw:
+            st = Stream()
+            s = tw.pool.seq_create()
+            bufs, pos = [], 0
+            for ki, vi in zip(k, v):
+                tw.pool.seq_reserve(s, pos + ki.shape[0])
+                kd, vd = DeviceBuffer.from_numpy(ki), DeviceBuffer.from_numpy(vi)
+                bufs += [kd, vd]
+                tw.pool.append(0, [s], [pos], [ki.shape[0]], kd, vd, st)
+                if sync_each:
+                    st.sync()
+                pos += ki.shape[0]
+            st.sync()
+            images.append((tw.pool.read_layer(0, 0), tw.pool.read_layer(0, 1)))
+            for b in bufs:
+                b.free()
+            st.close()
+    assert np.array_equal(images[0][0], images[1][0]) and np.array_equal(images[0][1], images[1][1])
+
+
+def test_reset_zeroes_the_pools_and_frees_every_sequence():
+    # crates/breccia-kernels/src/qsa/mod.rs:551-570
+    rng = np.random.Generator(np.random.PCG64(1))
+    with Twin(n_pages=8, max_seqs=2) as tw:
+        s = tw.pool.seq_create()
+        tw.pool.seq_reserve(s, 100)
+        x = rng.standard_normal((100, 2, 256)).astype(np.float32)
+        tw.append(0, [s], [0], [x], [x])
+        assert tw.pool.read_layer(0, 0).any()
+        tw.pool.reset()
+        device_sync()
+        assert not tw.pool.read_layer(0, 0).any() and not tw.pool.read_layer(0, 1).any()
+        assert tw.pool.free_pages() == 8 and tw.pool.seq_len(s) == -1
+        tw.pool.fill(0xFF)
+        device_sync()
+        assert (tw.pool.read_layer(0, 1) == 0xFF).all()

@@ -1,0 +1,140 @@
+"""GPU parity of copy-on-write page copy, prefix sharing and the VRAM <-> pinned-host swap.
+Byte moves: everything is compared bit for bit."""
+import numpy as np
+import pytest
+
+from breccia_amd import lib as L
+from breccia_amd.kv import BkvError, Stream, device_sync
+from gpu_common import Twin, check_attn
+from test_gpu_attn import fill
+
+pytestmark = pytest.mark.gpu
+
+
+def test_page_copy_moves_every_layer_and_leaves_the_rest_alone():
+    rng = np.random.Generator(np.random.PCG64(51))
+    with Twin(n_layers=3, n_pages=40, max_seqs=4) as tw:
+        s = tw.pool.seq_create()
+        tw.pool.seq_reserve(s, 16 * 10)
+        for layer in range(3):
+            x = rng.standard_normal((160, 2, 256)).astype(np.float32)
+            y = rng.standard_normal((160, 2, 256)).astype(np.float32)
+            tw.append(layer, [s], [0], [x], [y])
+        tab = tw.pool.block_table(s)
+        used = set(tab.tolist())
+        free = [p for p in range(40) if p not in used]
+        pairs = [(int(tab[0]), free[0]), (int(tab[7]), free[5]), (int(tab[9]), free[2])]
+        tw.pool.page_copy(pairs)
+        device_sync()
+        for img in tw.images:
+            img.page_copy(pairs)
+        for layer in range(3):
+            tw.assert_pools_equal(layer)
+        tw.pool.page_copy([])  # empty list is a no-op
+
+
+@pytest.mark.parametrize("prefix", [2048, 2040])
+def test_config4_shared_prefix_chunked_prefill_and_cow(prefix):
+    """BASELINE config 4: four sequences share a prefix through shared page ids with refcounts;
+    each appends a distinct 1024-token chunk.  A 2048-token prefix ends on a page boundary (no
+    copy may happen); a 2040-token prefix leaves a shared partial page that each writer but the
+    last must copy before its first append."""
+    rng = np.random.Generator(np.random.PCG64(60 + prefix))
+    with Twin(n_pages=512, max_seqs=8) as tw:
+        root = tw.pool.seq_create()
+        fill(tw, root, prefix, rng, chunk=512)
+        kids = [tw.pool.seq_fork(root, prefix) for _ in range(3)]
+        seqs = [root] + kids
+        shared = tw.pool.block_table(root).copy()
+        assert all(tw.pool.page_refcount(int(p)) == 4 for p in shared)
+        before = [tw.pool.gather(0, s, 0, prefix) for s in seqs]
+        n_copies = 0
+        for s in seqs:
+            pairs = tw.pool.seq_reserve(s, prefix + 1024)
+            n_copies += len(pairs)
+            tw.pool.page_copy(pairs)
+            for img in tw.images:
+                img.page_copy(pairs)
+            k = rng.standard_normal((1024, 2, 256)).astype(np.float32)
+            v = rng.standard_normal((1024, 2, 256)).astype(np.float32)
+            tw.append(0, [s], [prefix], [k], [v])
+        assert n_copies == (0 if prefix % 16 == 0 else 3)
+        tw.assert_pools_equal()
+        tw.pool.check()
+        full = prefix // 16
+        for s, (bk, bv) in zip(seqs, before):
+            tab = tw.pool.block_table(s)
+            assert np.array_equal(tab[:full], shared[:full])       # full prefix pages stay shared
+            gk, gv = tw.pool.gather(0, s, 0, prefix)
+            assert np.array_equal(gk, bk) and np.array_equal(gv, bv)  # nobody's prefix changed
+        tails = [int(tw.pool.block_table(s)[full]) for s in seqs]
+        assert len(set(tails)) == 4                                 # each writer has its own page
+        q = rng.standard_normal((4, 16, 256)).astype(np.float32)
+        pos = [prefix + 1023] * 4
+        out = tw.decode_attn(0, seqs, pos, q, 16)
+        for i, s in enumerate(seqs):
+            check_attn(out[i], tw.oracle_attend(0, s, pos[i], q[i], 16), "shared-prefix seq %d" % i)
+
+
+def test_swap_out_poison_swap_in_is_bit_exact():
+    """Evict a seeded 25 % of cold pages to pinned host memory, overwrite them in VRAM, swap
+    back: every pool byte must return."""
+    rng = np.random.Generator(np.random.PCG64(71))
+    with Twin(n_layers=2, n_pages=96, max_seqs=4) as tw:
+        s = tw.pool.seq_create()
+        tw.pool.seq_reserve(s, 16 * 80)
+        for layer in range(2):
+            x = rng.standard_normal((1280, 2, 256)).astype(np.float32)
+            y = rng.standard_normal((1280, 2, 256)).astype(np.float32)
+            tw.append(layer, [s], [0], [x], [y])
+        tab = tw.pool.block_table(s)
+        cold = rng.choice(tab, size=20, replace=False).astype(np.int32)
+        slab = tw.pool.swap_page_bytes()
+        assert slab == 2 * 32768
+        host = tw.pool.host_alloc(20 * slab)
+        st = Stream()
+        tw.pool.swap_out(cold, host, st)
+        tw.pool.swap_wait()
+        # host slab layout: [page][layer][K page | V page]
+        hv = host.view().reshape(20, 2, 2, 16384)
+        for i, p in enumerate(cold):
+            for layer in range(2):
+                assert np.array_equal(hv[i, layer, 0], tw.images[layer].k.reshape(-1, 16384)[p])
+                assert np.array_equal(hv[i, layer, 1], tw.images[layer].v.reshape(-1, 16384)[p])
+        # poison the evicted pages in VRAM by copying a garbage page over them
+        junk = [p for p in range(96) if p not in set(tab.tolist())][0]
+        tw.pool.page_copy([(junk, int(p)) for p in cold], st)
+        st.sync()
+        assert not np.array_equal(tw.pool.read_layer(0, 0), tw.images[0].k)
+        tw.pool.swap_in(cold, host, st)
+        tw.pool.swap_fence(st)
+        st.sync()
+        for layer in range(2):
+            tw.assert_pools_equal(layer)
+        host.free()
+        st.close()
+
+
+def test_evict_and_restore_through_the_allocator():
+    rng = np.random.Generator(np.random.PCG64(73))
+    with Twin(n_pages=64, max_seqs=4) as tw:
+        s = tw.pool.seq_create()
+        fill(tw, s, 16 * 20 + 5, rng)
+        kb, vb = tw.pool.gather(0, s, 0, 325)
+        host = tw.pool.host_alloc(8 * tw.pool.swap_page_bytes())
+        tw.pool.seq_evict(s, 4, 8, host)
+        tw.pool.swap_wait()
+        assert tw.pool.block_table(s)[4:12].tolist() == [-1] * 8 and tw.pool.free_pages() == 64 - 13
+        q = rng.standard_normal((1, 16, 256)).astype(np.float32)
+        with pytest.raises(BkvError) as ei:
+            tw.decode_attn(0, [s], [324], q, 16)
+        assert ei.value.status == L.ERR_STATE
+        # other sequences reuse the freed pages meanwhile
+        other = tw.pool.seq_create()
+        fill(tw, other, 16 * 30, rng)
+        tw.pool.seq_restore(s, 4, 8, host)
+        device_sync()
+        ka, va = tw.pool.gather(0, s, 0, 325)
+        assert np.array_equal(ka, kb) and np.array_equal(va, vb)
+        tw.pool.check()
+        host.free()

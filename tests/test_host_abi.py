@@ -1,0 +1,256 @@
+"""Host-side checks that need no GPU: the library loads and exports every entry point the
+header declares, every range/size violation is an error return (never a launch), and the
+page allocator keeps its invariants.  Pools here are created host-only."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+from breccia_amd import kv, lib as L
+from breccia_amd.kv import BkvError, Pool
+
+HEADER = os.path.join(os.path.dirname(__file__), "..", "include", "breccia_kv.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(bkv_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = declared_functions()
+    assert len(names) >= 45
+    for name in names:
+        assert hasattr(L.lib, name), "libbreccia_kv.so does not export " + name
+    # and the Python binding covers each of them
+    assert sorted(L._SIGNATURES) == names
+
+
+def test_header_structs_match_the_binding():
+    text = open(HEADER).read()
+    body = re.search(r"typedef struct bkv_pool_desc \{(.*?)\} bkv_pool_desc;", text, re.S).group(1)
+    fields = re.findall(r"(?:int32_t|uint32_t)\s+(\w+);", body)
+    assert fields == [f[0] for f in L.PoolDesc._fields_]
+    assert C.sizeof(L.PagePair) == 8
+    assert int(re.search(r"#define BKV_MAX_BATCH (\d+)", text).group(1)) == L.MAX_BATCH
+
+
+def host_pool(**kw):
+    kw.setdefault("host_only", True)
+    return Pool(**kw)
+
+
+def expect(status, fn, *a, **k):
+    with pytest.raises(BkvError) as ei:
+        fn(*a, **k)
+    assert ei.value.status == status, ei.value
+    assert ei.value.message, "an error must carry a message"
+    return ei.value.message
+
+
+def test_invalid_geometry_is_refused():
+    # crates/breccia-kernels/src/qsa/mod.rs:405-409: a state needs capacity > 0
+    expect(L.ERR_INVALID, host_pool, n_pages=0)
+    expect(L.ERR_INVALID, host_pool, n_layers=0)
+    expect(L.ERR_INVALID, host_pool, head_dim=100)
+    expect(L.ERR_INVALID, host_pool, head_dim=512)
+    expect(L.ERR_INVALID, host_pool, page_cells=4)
+    expect(L.ERR_INVALID, host_pool, layout=7)
+    expect(L.ERR_INVALID, host_pool, max_seqs=0)
+
+
+def test_sizes_follow_the_reference_layouts():
+    # crates/breccia-kernels/src/qsa/mod.rs:237-240, :316-370
+    with host_pool(n_layers=12, n_pages=8) as p:
+        assert p.page_bytes(0) == 16384 and p.page_bytes(1) == 16384
+        assert p.swap_page_bytes() == 12 * 32768
+    with host_pool(n_pages=2048, layout=L.LAYOUT_Q8V) as p:
+        assert p.page_bytes(0) == 16384 and p.page_bytes(1) == 32 * 288
+        assert p.page_bytes(1) / p.page_bytes(0) == 0.5625
+    with host_pool(layout=L.LAYOUT_I8H) as p:
+        assert p.page_bytes(0) == p.page_bytes(1) == 32 * 272
+
+
+def test_device_calls_on_a_host_only_pool_fail_cleanly():
+    with host_pool() as p:
+        s = p.seq_create()
+        p.seq_reserve(s, 20)
+        z = C.c_void_p(0x1000)
+        expect(L.ERR_NO_DEVICE, p.append, 0, [s], [0], [1], z, z)
+        expect(L.ERR_NO_DEVICE, p.decode_attn, 0, [s], [5], 16, z, z, 0.0625)
+        expect(L.ERR_NO_DEVICE, p.page_copy, [(0, 1)])
+        expect(L.ERR_NO_DEVICE, p.fill, 0xFF)
+
+
+def test_append_and_attention_range_checks_come_before_any_launch():
+    # crates/breccia-kernels/src/qsa/mod.rs:1108-1116 (append past capacity is an Err)
+    with host_pool(n_pages=8, max_seqs=4) as p:
+        s = p.seq_create()
+        p.seq_reserve(s, 40)  # 3 pages = 48 addressable cells
+        z = C.c_void_p(0x1000)
+        msg = expect(L.ERR_RANGE, p.append, 0, [s], [47], [2], z, z)
+        assert "47..49" in msg and "48" in msg
+        expect(L.ERR_RANGE, p.append, 0, [s], [-1], [1], z, z)
+        expect(L.ERR_RANGE, p.append, 0, [s], [0], [-1], z, z)
+        expect(L.ERR_RANGE, p.append, 1, [s], [0], [1], z, z)        # layer
+        expect(L.ERR_RANGE, p.append, 0, [3], [0], [1], z, z)        # dead sequence
+        expect(L.ERR_RANGE, p.decode_attn, 0, [s], [48], 16, z, z, 0.0625)
+        expect(L.ERR_RANGE, p.decode_attn, 0, [s], [-1], 16, z, z, 0.0625)
+        expect(L.ERR_INVALID, p.decode_attn, 0, [s], [5], 15, z, z, 0.0625)   # 15 q heads / 2 kv
+        expect(L.ERR_INVALID, p.decode_attn, 0, [s] * 65, [5] * 65, 16, z, z, 0.0625)
+        expect(L.ERR_RANGE, p.page_copy, [(0, 8)])
+        expect(L.ERR_INVALID, p.page_copy, [(0, 1), (2, 1)])
+        expect(L.ERR_RANGE, lambda: kv.check(L.lib.bkv_gather(p.handle, 0, s, 40, 9, z, z, None)))
+
+
+def test_allocator_basic_growth_and_free():
+    with host_pool(n_pages=10, max_seqs=3, max_pages_per_seq=6) as p:
+        a = p.seq_create()
+        assert p.seq_reserve(a, 1) == [] and p.seq_n_pages(a) == 1 and p.seq_len(a) == 1
+        assert p.seq_reserve(a, 16) == [] and p.seq_n_pages(a) == 1
+        assert p.seq_reserve(a, 17) == [] and p.seq_n_pages(a) == 2
+        assert p.free_pages() == 8 and p.seq_capacity(a) == 32
+        p.check()
+        expect(L.ERR_RANGE, p.seq_reserve, a, 16 * 6 + 1)      # longer than a table row
+        expect(L.ERR_RANGE, p.seq_reserve, a, 5)               # shrinking is truncate's job
+        b = p.seq_create()
+        p.seq_reserve(b, 16 * 6)
+        c = p.seq_create()
+        msg = expect(L.ERR_NO_PAGES, p.seq_reserve, c, 16 * 3)  # only 2 pages left
+        assert "2 free" in msg
+        assert p.seq_len(c) == 0 and p.seq_n_pages(c) == 0 and p.free_pages() == 2  # unchanged
+        expect(L.ERR_NO_PAGES, p.seq_create)                    # all 3 slots live
+        p.seq_free(b)
+        assert p.free_pages() == 8
+        expect(L.ERR_STATE, p.seq_free, b)                      # double free
+        p.check()
+        tab = p.block_table(a)
+        assert len(set(tab.tolist())) == 2 and all(p.page_refcount(int(x)) == 1 for x in tab)
+
+
+def test_fork_shares_pages_and_cow_fires_only_on_a_shared_partial_page():
+    with host_pool(n_pages=64, max_seqs=8, max_pages_per_seq=16) as p:
+        root = p.seq_create()
+        p.seq_reserve(root, 40)                 # 2 full pages + 8 cells of a third
+        kids = [p.seq_fork(root, 40) for _ in range(3)]
+        tab = p.block_table(root)
+        assert all(p.page_refcount(int(x)) == 4 for x in tab)
+        for k in kids:
+            assert np.array_equal(p.block_table(k), tab) and p.seq_len(k) == 40
+        p.check()
+        # first writer: copies the shared partial page, leaves the full pages shared
+        pairs = p.seq_reserve(kids[0], 41)
+        assert pairs == [(int(tab[2]), int(p.block_table(kids[0])[2]))]
+        assert pairs[0][1] != pairs[0][0] and p.page_refcount(int(tab[2])) == 3
+        assert np.array_equal(p.block_table(kids[0])[:2], tab[:2])
+        # others likewise; the last holder writes in place (refcount is back to 1)
+        assert len(p.seq_reserve(kids[1], 50)) == 1
+        assert len(p.seq_reserve(kids[2], 41)) == 1
+        assert p.page_refcount(int(tab[2])) == 1
+        assert p.seq_reserve(root, 41) == []
+        assert p.block_table(root)[2] == tab[2]
+        p.check()
+        # a fork at a page boundary never copies: appends start on a fresh page
+        edge = p.seq_fork(root, 32)
+        assert p.seq_reserve(edge, 33) == []
+        assert p.block_table(edge)[2] not in (tab[2],)
+        # the report buffer being too small is an error and changes nothing
+        k4 = p.seq_fork(kids[1], 50)
+        free_before = p.free_pages()
+        expect(L.ERR_INVALID, p.seq_reserve, k4, 51, 0)
+        assert p.free_pages() == free_before and p.seq_len(k4) == 50
+        for s in kids + [root, edge, k4]:
+            p.seq_free(s)
+        assert p.free_pages() == 64
+        p.check()
+
+
+def test_truncate_then_regrow_does_not_write_into_shared_pages():
+    with host_pool(n_pages=32, max_seqs=4, max_pages_per_seq=8) as p:
+        a = p.seq_create()
+        p.seq_reserve(a, 64)
+        b = p.seq_fork(a, 64)
+        p.seq_truncate(b, 20)                       # speculative rollback keeps the pages
+        assert p.seq_n_pages(b) == 4 and p.seq_len(b) == 20
+        pairs = p.seq_reserve(b, 50)                # rewrites cells 20..49: pages 1, 2, 3
+        tb, ta = p.block_table(b), p.block_table(a)
+        assert tb[0] == ta[0]                       # untouched page stays shared
+        assert pairs == [(int(ta[1]), int(tb[1]))]  # partial page is copied
+        assert tb[2] != ta[2] and tb[3] != ta[3]    # fully rewritten pages are fresh, no copy
+        expect(L.ERR_RANGE, p.seq_truncate, b, 51)
+        p.check()
+
+
+def test_identity_sequence_is_the_reference_page_table():
+    # crates/breccia-kernels/src/qsa/mod.rs:477-481
+    with host_pool(n_pages=8, max_seqs=2) as p:
+        s = p.seq_create_identity(3)
+        assert p.block_table(s).tolist() == [0, 1, 2] and p.seq_capacity(s) == 48
+        assert p.free_pages() == 5
+        expect(L.ERR_STATE, p.seq_create_identity, 2)
+        p.check()
+
+
+def test_evict_restore_bookkeeping():
+    with host_pool(n_pages=16, max_seqs=4, max_pages_per_seq=8) as p:
+        a = p.seq_create()
+        p.seq_reserve(a, 70)                        # 4 full pages + 6 cells
+        host = C.c_void_p(0x1000)                   # never dereferenced by a host-only pool
+        expect(L.ERR_STATE, lambda: kv.check(L.lib.bkv_seq_evict(p.handle, a, 3, 2, host, None)))
+        b = p.seq_fork(a, 16)
+        expect(L.ERR_STATE, lambda: kv.check(L.lib.bkv_seq_evict(p.handle, a, 0, 1, host, None)))
+        p.seq_free(b)
+        kv.check(L.lib.bkv_seq_evict(p.handle, a, 1, 2, host, None))
+        assert p.block_table(a).tolist()[1:3] == [-1, -1] and p.free_pages() == 13
+        z = C.c_void_p(0x1000)
+        expect(L.ERR_STATE, p.decode_attn, 0, [a], [69], 16, z, z, 0.0625)
+        expect(L.ERR_STATE, p.append, 0, [a], [20], [1], z, z)
+        expect(L.ERR_STATE, lambda: kv.check(L.lib.bkv_seq_restore(p.handle, a, 0, 1, host, None)))
+        kv.check(L.lib.bkv_seq_restore(p.handle, a, 1, 2, host, None))
+        assert all(x >= 0 for x in p.block_table(a)) and p.free_pages() == 11
+        p.check()
+
+
+def test_randomised_allocator_keeps_its_invariants():
+    rng = np.random.Generator(np.random.PCG64(2))
+    with host_pool(n_pages=48, max_seqs=12, max_pages_per_seq=12) as p:
+        live = {}
+        for step in range(600):
+            op = rng.integers(0, 5)
+            try:
+                if op == 0 or not live:
+                    s = p.seq_create()
+                    live[s] = 0
+                elif op == 1:
+                    s = int(rng.choice(list(live)))
+                    new_len = live[s] + int(rng.integers(1, 40))
+                    p.seq_reserve(s, new_len, cow_capacity=4)
+                    live[s] = new_len
+                elif op == 2:
+                    s = int(rng.choice(list(live)))
+                    n = int(rng.integers(0, live[s] + 1))
+                    c = p.seq_fork(s, n)
+                    live[c] = n
+                elif op == 3:
+                    s = int(rng.choice(list(live)))
+                    p.seq_free(s)
+                    del live[s]
+                else:
+                    s = int(rng.choice(list(live)))
+                    n = int(rng.integers(0, live[s] + 1))
+                    p.seq_truncate(s, n)
+                    live[s] = n
+            except BkvError as e:
+                assert e.status in (L.ERR_NO_PAGES, L.ERR_RANGE), e
+            p.check()
+            for s, n in live.items():
+                assert p.seq_len(s) == n
+        total_refs = sum(p.page_refcount(i) for i in range(48))
+        entries = sum(int((p.block_table(s) >= 0).sum()) for s in live)
+        assert total_refs == entries
+        for s in list(live):
+            p.seq_free(s)
+        assert p.free_pages() == 48
