@@ -102,7 +102,7 @@ bkv_status flush_tables(bkv_pool* p, hipStream_t stream) {
     return BKV_OK;
 }
 
-StageScope::StageScope(bkv_pool* p, int stage, hipStream_t stream) : p_(p), stream_(stream) {
+StageScope::StageScope(bkv_pool* p, int stage, hipStream_t stream) : stream_(stream) {
     StageTimer& t = p->timer;
     if (!t.on) return;
     auto take = [&t]() -> hipEvent_t {

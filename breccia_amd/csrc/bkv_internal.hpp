@@ -114,7 +114,6 @@ public:
     ~StageScope();
 
 private:
-    bkv_pool* p_;
     hipStream_t stream_;
     hipEvent_t stop_ = nullptr;
 };
