@@ -1,0 +1,393 @@
+#!/usr/bin/env python3
+"""Benchmark of the paged-KV hot path on one MI355X.
+
+Headline workload (BASELINE.json configs[2], the one the >=70 %-of-HBM target is quoted
+on): batched decode, 8 concurrent sequences, contexts U{1024..32768} (seeded, each with a
+partially filled last page), f16 K/V, 16 q / 2 kv heads, head_dim 256, 16-token pages on a
+60 %-occupied pool whose pages were shuffled and dealt round-robin across the sequences.
+A step = append one token per sequence + paged decode attention, for one layer; layers
+rotate so that consecutive steps never touch the same pool bytes.
+
+Prints ONE JSON line.  `value` = algorithmic bytes of a step / wall time of a step, inputs
+resident in HBM.  `roofline` prices the split-K attention kernel alone from HIP events on
+its stream.  `cpu_baseline` is the CPU oracle (a restatement of the reference's scalar f64
+CPU path) timed on this host on the same workload.  `extra` carries the batch-1 config and
+the byte-move kernels.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+N_Q, N_KV, HD, PAGE = 16, 2, 256, 16
+ROW_BYTES = N_KV * HD * 2 * 2          # K + V f16 bytes per cell per layer = 2048
+APPEND_BYTES_PER_TOKEN = N_KV * HD * (4 + 2) * 2  # f32 in + f16 out, K and V = 6144
+
+
+def attn_algorithmic_bytes(ctx_after: list[int]) -> int:
+    """K+V rows read once for all heads of a group + block table + q + out."""
+    total = 0
+    for c in ctx_after:
+        total += c * ROW_BYTES + ((c + PAGE - 1) // PAGE) * 4 + 2 * N_Q * HD * 4
+    return total
+
+
+def build_batched(pool_mod, rng, n_seqs: int, lo: int, hi: int, n_layers: int, occupancy: float):
+    from breccia_amd.kv import Pool
+
+    ctx = []
+    for _ in range(n_seqs):
+        c = int(rng.integers(lo, hi + 1))
+        if c % PAGE == 0:
+            c -= 1 + int(rng.integers(0, PAGE - 1))
+        ctx.append(c)
+    live_pages = sum((c + PAGE) // PAGE + 1 for c in ctx)
+    n_pages = int(np.ceil(live_pages / occupancy))
+    pool = Pool(n_layers=n_layers, n_pages=n_pages, n_kv_head=N_KV, head_dim=HD, max_seqs=n_seqs + 1,
+                max_pages_per_seq=max(ctx) // PAGE + 8)
+    pool.set_free_order(rng.permutation(n_pages).astype(np.int32))
+    seqs = [pool.seq_create() for _ in ctx]
+    # deal the shuffled pages round-robin: one page per sequence per turn
+    grown = [0] * n_seqs
+    while any(g < c for g, c in zip(grown, ctx)):
+        for i, s in enumerate(seqs):
+            if grown[i] < ctx[i]:
+                grown[i] = min(ctx[i], grown[i] + PAGE)
+                pool.seq_reserve(s, grown[i])
+    return pool, seqs, ctx
+
+
+def fill_layers(pool, seqs, ctx, n_layers, rng, stream, keep_host_layer0: bool):
+    """N(0,1) f32 K/V through bkv_append, chunked.  Returns layer 0's host K/V per sequence."""
+    from breccia_amd.kv import DeviceBuffer
+
+    host = []
+    chunk = 4096
+    kd = DeviceBuffer(chunk * N_KV * HD * 4)
+    vd = DeviceBuffer(chunk * N_KV * HD * 4)
+    for i, (s, c) in enumerate(zip(seqs, ctx)):
+        k = rng.standard_normal((c, N_KV, HD), dtype=np.float32)
+        v = rng.standard_normal((c, N_KV, HD), dtype=np.float32)
+        for layer in range(n_layers):
+            for at in range(0, c, chunk):
+                n = min(chunk, c - at)
+                kd.upload(k[at:at + n], stream)
+                vd.upload(v[at:at + n], stream)
+                pool.append(layer, [s], [at], [n], kd, vd, stream)
+                stream.sync()
+        host.append((k, v) if keep_host_layer0 else None)
+    kd.free()
+    vd.free()
+    return host
+
+
+def run_steps(pool, seqs, ctx0, n_layers, steps, q_dev, out_dev, newk, newv, stream, first_step=0):
+    """Enqueue `steps` steps (append + attention on layer step % n_layers)."""
+    n = len(seqs)
+    for i in range(first_step, first_step + steps):
+        layer = i % n_layers
+        tok = i // n_layers
+        pos = [c + tok for c in ctx0]
+        if layer == 0:
+            for s, p in zip(seqs, pos):
+                pool.seq_reserve(s, p + 1)
+        off = (i % newk.n_slots) * n * N_KV * HD * 4
+        pool.append(layer, seqs, pos, [1] * n, newk.at(off), newv.at(off), stream)
+        pool.decode_attn(layer, seqs, pos, N_Q, q_dev, out_dev, 1.0 / 16.0, stream=stream)
+
+
+def time_steps(pool, seqs, ctx0, n_layers, steps, warmup, bufs, stream):
+    from breccia_amd.kv import Event, device_sync
+
+    q_dev, out_dev, newk, newv = bufs
+    run_steps(pool, seqs, ctx0, n_layers, warmup, q_dev, out_dev, newk, newv, stream, 0)
+    stream.sync()
+    device_sync()
+    e0, e1 = Event(), Event()
+    t0 = time.perf_counter()
+    e0.record(stream)
+    run_steps(pool, seqs, ctx0, n_layers, steps, q_dev, out_dev, newk, newv, stream, warmup)
+    e1.record(stream)
+    stream.sync()
+    device_sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ev_ms = e0.elapsed_ms(e1)
+    e0.close()
+    e1.close()
+    return wall_ms, ev_ms
+
+
+def make_step_buffers(n_seqs, rng, slots=64):
+    from breccia_amd.kv import DeviceBuffer
+
+    q = rng.standard_normal((n_seqs, N_Q, HD), dtype=np.float32)
+    q_dev = DeviceBuffer.from_numpy(q)
+    out_dev = DeviceBuffer(q.nbytes)
+    newk = DeviceBuffer.from_numpy(rng.standard_normal((slots, n_seqs, N_KV, HD), dtype=np.float32))
+    newv = DeviceBuffer.from_numpy(rng.standard_normal((slots, n_seqs, N_KV, HD), dtype=np.float32))
+    newk.n_slots = newv.n_slots = slots
+    return q, (q_dev, out_dev, newk, newv)
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-extra", action="store_true", help="skip batch-1 / byte-move extras")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the paged-KV path here is single-device "
+              "(--gpus %d is not supported)" % args.gpus, file=sys.stderr)
+        return 2
+
+    from breccia_amd import lib as L
+    from breccia_amd.kv import DeviceBuffer, Stream, device_info, device_sync
+
+    dev_name, n_cu, mem = device_info()
+    stream = Stream()
+    rng = np.random.Generator(np.random.PCG64(20250003))
+    n_layers = 4
+    pool, seqs, ctx = build_batched(None, rng, 8, 1024, 32768, n_layers, 0.6)
+    host_kv = fill_layers(pool, seqs, ctx, n_layers, rng, stream, keep_host_layer0=not args.no_cpu)
+    q_host, bufs = make_step_buffers(len(seqs), rng)
+
+    # ---- headline: K steps, whole path ------------------------------------------------
+    wall_ms, ev_ms = time_steps(pool, seqs, ctx, n_layers, args.steps, args.warmup, bufs, stream)
+    ms_per_step = wall_ms / args.steps
+    tokens_done = (args.warmup + args.steps + n_layers - 1) // n_layers
+    ctx_mid = [c + 1 + (args.warmup + args.steps // 2) // n_layers for c in ctx]
+    attn_bytes = attn_algorithmic_bytes(ctx_mid)
+    step_bytes = attn_bytes + len(seqs) * APPEND_BYTES_PER_TOKEN
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # ---- roofline: the split-K kernel alone, HIP events on its stream -------------------
+    pool.timing_reset()
+    pool.timing_enable(True)
+    first = args.warmup + args.steps
+    run_steps(pool, seqs, ctx, n_layers, args.steps, *bufs, stream, first_step=first)
+    stream.sync()
+    pool.timing_enable(False)
+    n_split, ms_split = pool.timing_read(L.STAGE_ATTN_SPLIT)
+    n_merge, ms_merge = pool.timing_read(L.STAGE_ATTN_MERGE)
+    n_app, ms_app = pool.timing_read(L.STAGE_APPEND)
+    split_us = ms_split / max(n_split, 1) * 1e3
+    achieved = attn_bytes / (split_us * 1e-6) / 1e9
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                "kernel": "decode_attn_f16_kernel<8>", "avg_us": round(split_us, 2),
+                "launches": n_split, "algorithmic_bytes": attn_bytes}
+
+    # ---- sanity: one sequence of the last step against the oracle ----------------------
+    checked = None
+    cpu = None
+    if not args.no_cpu:
+        import oracle
+
+        out = bufs[1].download(np.float32, stream=stream).reshape(len(seqs), N_Q, HD)
+        # shortest sequence, layer of the last step
+        last = first + args.steps - 1
+        layer = last % n_layers
+        i = int(np.argmin(ctx))
+        pos = ctx[i] + last // n_layers
+        k, v = pool.gather(layer, seqs[i], 0, pos + 1, stream)
+        want = oracle.attend(q_host[i], k, v, oracle.dense_cells(pos), pos, N_Q, N_KV, HD, threads=8)
+        checked = float(np.max(np.abs(out[i].astype(np.float64) - want)))
+
+        # ---- CPU baseline: the oracle on the same batch (layer 0 contents), one thread -----
+        kf = [oracle.to_f16(k) for k, _ in host_kv]
+        vf = [oracle.to_f16(v) for _, v in host_kv]
+        cells = [oracle.dense_cells(c - 1) for c in ctx]
+        t0 = time.perf_counter()
+        for j in range(len(seqs)):
+            oracle.attend(q_host[j], kf[j], vf[j], cells[j], ctx[j] - 1, N_Q, N_KV, HD, threads=1)
+        cpu_s = time.perf_counter() - t0
+        cpu_bytes = attn_algorithmic_bytes(ctx)
+        nthr = min(oracle.max_threads(), 16)
+        t0 = time.perf_counter()
+        for j in range(len(seqs)):
+            oracle.attend(q_host[j], kf[j], vf[j], cells[j], ctx[j] - 1, N_Q, N_KV, HD, threads=nthr)
+        cpu_mt_s = time.perf_counter() - t0
+        cpu = {"value": round(cpu_bytes / cpu_s / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+               "sample": "one full batch-8 decode-attention step (all 8 sequences, 16 heads, "
+                         "%d cells) in the scalar f64 oracle: %.2f s" % (sum(ctx), cpu_s),
+               "us_per_layer": round(cpu_s * 1e6, 0),
+               "openmp": {"threads": nthr, "value": round(cpu_bytes / cpu_mt_s / 1e9, 4),
+                          "seconds": round(cpu_mt_s, 3)}}
+        del kf, vf, host_kv
+
+    extra = {"attn_split_us": round(split_us, 2), "attn_merge_us": round(ms_merge / max(n_merge, 1) * 1e3, 2),
+             "append_us": round(ms_app / max(n_app, 1) * 1e3, 2),
+             "step_event_ms": round(ev_ms / args.steps, 4),
+             "contexts": ctx, "pool_pages": pool.desc.n_pages, "device": dev_name, "cus": n_cu,
+             "oracle_check_max_abs": checked}
+    pool.destroy()
+    for b in bufs:
+        b.free()
+
+    if not args.no_extra:
+        extra.update(bench_batch1(stream))
+        extra.update(bench_moves(stream))
+
+    line = {"metric": "paged decode-attn step throughput, batch 8 mixed 1k-32k (append + attention, "
+                      "algorithmic bytes / time)",
+            "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "f16 storage, f32 accumulate",
+            "data": "synthetic N(0,1), seeded",
+            "config": {"workload": "BASELINE configs[2]: batched decode, 8 sequences, ctx U{1k..32k}, "
+                                   "f16 KV, 16q/2kv, d256, page 16, 60% occupied shuffled pool; "
+                                   "step = append 1 token/seq + paged decode attention, 1 layer",
+                       "layers_rotated": n_layers, "us_per_layer": round(ms_per_step * 1e3, 2),
+                       "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4)},
+            "roofline": roofline, "cpu_baseline": cpu, "extra": extra}
+    print(json.dumps(line))
+    return 0
+
+
+def bench_batch1(stream) -> dict:
+    """BASELINE configs[1]: one sequence at 4096 context, pages scattered over a 64k-page pool,
+    12 layers with independent contents; per-layer latency."""
+    from breccia_amd import lib as L
+    from breccia_amd.kv import Pool
+
+    rng = np.random.Generator(np.random.PCG64(20250002))
+    n_layers, ctx = 12, 4096
+    pool = Pool(n_layers=n_layers, n_pages=65536, n_kv_head=N_KV, head_dim=HD, max_seqs=2,
+                max_pages_per_seq=512)
+    pool.set_free_order(rng.permutation(65536).astype(np.int32))
+    s = pool.seq_create()
+    pool.seq_reserve(s, ctx)
+    from breccia_amd.kv import DeviceBuffer
+    kd = DeviceBuffer(ctx * N_KV * HD * 4)
+    vd = DeviceBuffer(ctx * N_KV * HD * 4)
+    for layer in range(n_layers):
+        kd.upload(rng.standard_normal((ctx, N_KV, HD), dtype=np.float32), stream)
+        vd.upload(rng.standard_normal((ctx, N_KV, HD), dtype=np.float32), stream)
+        pool.append(layer, [s], [0], [ctx], kd, vd, stream)
+        stream.sync()
+    kd.free()
+    vd.free()
+    _, bufs = make_step_buffers(1, rng)
+    steps, warm = 600, 60
+    wall_ms, ev_ms = time_steps(pool, [s], [ctx], n_layers, steps, warm, bufs, stream)
+    pool.timing_reset()
+    pool.timing_enable(True)
+    run_steps(pool, [s], [ctx], n_layers, steps, *bufs, stream, first_step=steps + warm)
+    stream.sync()
+    pool.timing_enable(False)
+    n_split, ms_split = pool.timing_read(L.STAGE_ATTN_SPLIT)
+    n_merge, ms_merge = pool.timing_read(L.STAGE_ATTN_MERGE)
+    n_app, ms_app = pool.timing_read(L.STAGE_APPEND)
+    bytes_step = attn_algorithmic_bytes([ctx + 1 + (warm + steps // 2) // n_layers])
+    us = wall_ms / steps * 1e3
+    out = {"batch1": {"workload": "BASELINE configs[1]: 1 sequence, ctx 4096, 64k-page pool, 12 layers",
+                      "us_per_layer": round(us, 2), "GBps": round(bytes_step / (us * 1e-6) / 1e9, 1),
+                      "frac_of_hbm_peak": round(bytes_step / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+                      "attn_split_us": round(ms_split / max(n_split, 1) * 1e3, 2),
+                      "attn_merge_us": round(ms_merge / max(n_merge, 1) * 1e3, 2),
+                      "append_us": round(ms_app / max(n_app, 1) * 1e3, 2),
+                      "ms_per_token_12_layers": round(us * 12 / 1e3, 4)}}
+    pool.destroy()
+    for b in bufs:
+        b.free()
+    return out
+
+
+def bench_moves(stream) -> dict:
+    """Bulk shapes of the byte-move kernels: append (f32 in -> f16 out), copy-on-write page
+    copy, VRAM <-> pinned host swap, and a plain device copy for reference."""
+    from breccia_amd import lib as L
+    from breccia_amd.kv import DeviceBuffer, Event, Pool, check, lib
+
+    rng = np.random.Generator(np.random.PCG64(20250004))
+    n_pages = 40960
+    pool = Pool(n_layers=1, n_pages=n_pages, n_kv_head=N_KV, head_dim=HD, max_seqs=8,
+                max_pages_per_seq=n_pages // 4 + 8)
+    pool.set_free_order(rng.permutation(n_pages).astype(np.int32))
+    res = {}
+
+    def timed(fn, reps):
+        fn()
+        stream.sync()
+        e0, e1 = Event(), Event()
+        e0.record(stream)
+        for _ in range(reps):
+            fn()
+        e1.record(stream)
+        stream.sync()
+        ms = e0.elapsed_ms(e1) / reps
+        e0.close()
+        e1.close()
+        return ms
+
+    # append: 4 sequences x 16384 tokens in one call (BASELINE configs[3] shape, scaled up)
+    T = 16384
+    seqs = [pool.seq_create() for _ in range(4)]
+    for s in seqs:
+        pool.seq_reserve(s, T)
+    kd = DeviceBuffer.from_numpy(rng.standard_normal((4 * T, N_KV, HD), dtype=np.float32))
+    vd = DeviceBuffer.from_numpy(rng.standard_normal((4 * T, N_KV, HD), dtype=np.float32))
+    ms = timed(lambda: pool.append(0, seqs, [0] * 4, [T] * 4, kd, vd, stream), 20)
+    b = 4 * T * APPEND_BYTES_PER_TOKEN
+    res["append_bulk"] = {"tokens": 4 * T, "ms": round(ms, 4), "GBps": round(b / ms / 1e6, 1),
+                          "frac_of_hbm_peak": round(b / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    ms = timed(lambda: pool.append(0, seqs, [7] * 4, [1] * 4, kd, vd, stream), 200)
+    res["append_decode_us"] = round(ms * 1e3, 2)
+    kd.free()
+    vd.free()
+
+    # page copy: 16384 pairs = 512 MiB read + 512 MiB written
+    used = np.concatenate([pool.block_table(s) for s in seqs])
+    free = np.setdiff1d(np.arange(n_pages, dtype=np.int32), used)
+    n_pairs = 16384
+    pairs = list(zip(used[:n_pairs].tolist(), free[:n_pairs].tolist()))
+    ms = timed(lambda: pool.page_copy(pairs, stream), 10)
+    b = 2 * n_pairs * 32768
+    res["page_copy_bulk"] = {"pairs": n_pairs, "ms": round(ms, 4), "GBps": round(b / ms / 1e6, 1),
+                             "frac_of_hbm_peak": round(b / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    ms = timed(lambda: pool.page_copy(pairs[:1], stream), 200)
+    res["page_copy_one_us"] = round(ms * 1e3, 2)
+
+    # plain device copy of the same volume (ceiling of a read+write stream on this box)
+    a = DeviceBuffer(512 << 20)
+    c = DeviceBuffer(512 << 20)
+    ms = timed(lambda: check(lib.bkv_copy_probe(c.ptr, a.ptr, 512 << 20, stream.handle)), 10)
+    res["device_copy_probe"] = {"bytes_moved": 2 * (512 << 20), "ms": round(ms, 4),
+                                "GBps": round(2 * (512 << 20) / ms / 1e6, 1)}
+    a.free()
+    c.free()
+
+    # swap: 25 % of the live pages out to pinned host and back
+    n_swap = 4096
+    host = pool.host_alloc(n_swap * pool.swap_page_bytes())
+    pages = used[:n_swap].astype(np.int32)
+    t0 = time.perf_counter()
+    pool.swap_out(pages, host, stream)
+    pool.swap_wait()
+    t_out = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    pool.swap_in(pages, host, stream)
+    pool.swap_fence(stream)
+    stream.sync()
+    t_in = time.perf_counter() - t0
+    b = n_swap * pool.swap_page_bytes()
+    res["swap"] = {"pages": n_swap, "bytes": b, "out_GBps": round(b / t_out / 1e9, 2),
+                   "in_GBps": round(b / t_in / 1e9, 2)}
+    host.free()
+    pool.destroy()
+    return res
+
+
+if __name__ == "__main__":
+    sys.exit(main())
