@@ -66,10 +66,66 @@ __device__ __forceinline__ float dpp(float v) {
 constexpr int kDppXor1 = 0xB1;  // quad_perm [1,0,3,2]
 constexpr int kDppXor2 = 0x4E;  // quad_perm [2,3,0,1]
 
+constexpr int kDppRor8 = 0x128;  // row_ror:8 == lane ^ 8 inside a row of 16
+
 __device__ __forceinline__ float xor_max(float v, int mask) {
     return fmaxf(v, __shfl_xor(v, mask, 64));
 }
 __device__ __forceinline__ float xor_sum(float v, int mask) { return v + __shfl_xor(v, mask, 64); }
+
+// Lane exchanges across 16 and 32 lanes with the gfx950 permlane swaps, written as inline
+// assembly because this toolchain's builtin returns its first result twice.
+//   v_permlane16_swap a, b : a.row1 <-> b.row0 and a.row3 <-> b.row2 (rows of 16 lanes)
+//   v_permlane32_swap a, b : a.lanes[32..63] <-> b.lanes[0..31]
+// The s_nop covers the wait states a VALU write needs before a permlane reads it.  The asm
+// statements are not `volatile`: a volatile asm counts as a possible memory write and would
+// turn the uniform block-table loads behind it into vector loads.
+__device__ __forceinline__ void permlane16_swap(float& a, float& b) {
+    asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void permlane32_swap(float& a, float& b) {
+    asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+// Swapping a register with a copy of itself puts both partners' values side by side.
+__device__ __forceinline__ void both16(float v, float& a, float& b) {
+    a = v;
+    b = v;
+    permlane16_swap(a, b);
+}
+__device__ __forceinline__ void both32(float v, float& a, float& b) {
+    a = v;
+    b = v;
+    permlane32_swap(a, b);
+}
+// max / sum over the lanes that differ in bits 3, 4 and 5 (the 8 lanes holding one head)
+__device__ __forceinline__ float max_bits345(float v) {
+    float a, b;
+    v = fmaxf(v, dpp<kDppRor8>(v));
+    both16(v, a, b);
+    v = fmaxf(a, b);
+    both32(v, a, b);
+    return fmaxf(a, b);
+}
+__device__ __forceinline__ float sum_bits345(float v) {
+    float a, b;
+    v += dpp<kDppRor8>(v);
+    both16(v, a, b);
+    v = a + b;
+    both32(v, a, b);
+    return a + b;
+}
+
+// f16 -> f32 as a separate conversion.  Folding the conversion into the multiply-add
+// (v_fma_mix_f32) would save the convert, but on gfx950 that packed-encoding instruction
+// issues from one wave at a time, while plain v_fma_f32 from two waves of a SIMD overlap
+// (measured: ~4.8 vs ~2.5 cycles per wave-instruction); with every converted element
+// feeding HG multiply-adds the separate convert is the cheaper form.  The empty asm keeps
+// the compiler from folding it back.
+__device__ __forceinline__ float widen(_Float16 h) {
+    float f = (float)h;
+    asm("" : "+v"(f));
+    return f;
+}
 
 __device__ __forceinline__ half8 load_row8(const uint16_t* base, int idx) {
     return __builtin_bit_cast(half8, reinterpret_cast<const uint4*>(base)[idx]);
@@ -89,22 +145,32 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_f16_kernel(const AttnKe
     __shared__ float wave_l[kWaves][HG];
 
     // ---- which (entry, kv head, head chunk, page range) ---------------------------
-    const int wg = blockIdx.x;
+    // A unit is (entry, page range, kv head); its n_hc head chunks read the same K/V rows.
+    // Work-groups go to the 8 XCDs round-robin by index, so the chunks of a unit are placed 8
+    // indices apart: same XCD (same L2), dispatched together.  `wg` is the unit's slot in
+    // the partial-result workspace, independent of the dispatch order.
+    const int n_units = P.b.wg_base[P.b.n] / P.n_hc;
+    const int blk = blockIdx.x / (8 * P.n_hc);
+    const int rblk = blockIdx.x - blk * (8 * P.n_hc);
+    const int hc = rblk >> 3;
+    const int unit = blk * 8 + (rblk & 7);
+    if (unit >= n_units) return;
     int e = 0;
-    while (e + 1 < P.b.n && wg >= P.b.wg_base[e + 1]) ++e;
-    const int local = wg - P.b.wg_base[e];
+    while (e + 1 < P.b.n && unit * P.n_hc >= P.b.wg_base[e + 1]) ++e;
     const int splits = P.b.splits[e];
-    const int per_hc = splits * P.n_kv;
-    const int hc = local / per_hc;
-    const int rem = local - hc * per_hc;
+    const int rem = unit - P.b.wg_base[e] / P.n_hc;
     const int split = rem / P.n_kv;
     const int kvh = rem - split * P.n_kv;
+    const int wg = P.b.wg_base[e] + hc * splits * P.n_kv + rem;
     const int pos = P.b.pos[e];
     const int n_pages = pos / kPage + 1;
     const int pps = P.b.pps[e];
     const int pg0 = split * pps;
     const int pg1 = min(pg0 + pps, n_pages);
-    const int32_t* __restrict__ bt = P.tables + (size_t)P.b.row[e] * (size_t)P.max_pages_per_seq;
+    // Block-table row through the constant address space: the table is not written while this
+    // kernel runs, and constant-space loads at uniform addresses are always scalar loads.
+    typedef const __attribute__((address_space(4))) int32_t* table_ptr;
+    const table_ptr bt = (table_ptr)(uintptr_t)(P.tables + (size_t)P.b.row[e] * (size_t)P.max_pages_per_seq);
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
@@ -129,6 +195,11 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_f16_kernel(const AttnKe
         }
     }
 
+    // q must have arrived before the first K/V rows are requested: a wait for q placed
+    // inside the page loop would also drain the row loads that are kept in flight there.
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), other counters untouched
+    __builtin_amdgcn_sched_barrier(0);
+
     float o[HG][8];
 #pragma unroll
     for (int h = 0; h < HG; ++h)
@@ -149,25 +220,42 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_f16_kernel(const AttnKe
     const size_t page_elems = (size_t)P.n_kv * kPage * kHd;
     const size_t head_off = (size_t)kvh * kPage * kHd;
 
+    // K and V rows of a page sit in registers (8 x 16 bytes each per lane).  Every register
+    // group is refilled with the next page's row right after its last use, so each load has
+    // a whole page of work in front of it and 16 loads per wave stay in flight.
     int pg = pg0 + wave;
     half8 kk[8], vv[8];
-    int32_t phys = 0;
     if (pg < pg1) {
-        phys = bt[pg];
+        const int32_t phys = bt[pg];
         const uint16_t* kp = P.kpool + (size_t)phys * page_elems + head_off;
+        const uint16_t* vp = P.vpool + (size_t)phys * page_elems + head_off;
 #pragma unroll
         for (int i = 0; i < 8; ++i) kk[i] = load_row8(kp, i * 64 + lane);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) vv[i] = load_row8(vp, i * 64 + lane);
     }
 
+    // Two waves share a SIMD (one from each resident work-group) and the issue arbiter
+    // always prefers the older one, which then finishes a third earlier and leaves the
+    // younger wave alone, with nothing to overlap its latencies, for the rest of the
+    // kernel.  Swapping the two waves' priority on every page shares the SIMD evenly.
+    unsigned slot;
+    asm("s_getreg_b32 %0, hwreg(HW_REG_HW_ID, 0, 4)" : "=s"(slot));  // wave slot within the SIMD
+    unsigned turn = slot;
+
     while (pg < pg1) {
-        {
-            const uint16_t* vp = P.vpool + (size_t)phys * page_elems + head_off;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) vv[i] = load_row8(vp, i * 64 + lane);
-        }
+        if (turn & 1)
+            __builtin_amdgcn_s_setprio(2);
+        else
+            __builtin_amdgcn_s_setprio(0);
+        ++turn;
+        // The next page is fetched unconditionally (the last iteration re-reads its own
+        // page): one straight-line load sequence lets the compiler count outstanding loads
+        // exactly instead of draining them at a control-flow join.
         const int pg_next = pg + kWaves;
-        int32_t phys_next = 0;
-        if (pg_next < pg1) phys_next = bt[pg_next];
+        const int32_t phys_next = bt[min(pg_next, pg1 - 1)];
+        const uint16_t* kp_next = P.kpool + (size_t)phys_next * page_elems + head_off;
+        const uint16_t* vp_next = P.vpool + (size_t)phys_next * page_elems + head_off;
 
         // ---- scores: partial dots -> LDS transpose -> one (row, head) per lane ------
         float sval[NB];
@@ -176,14 +264,20 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_f16_kernel(const AttnKe
 #pragma unroll
             for (int ip = 0; ip < RP; ++ip) {
                 const int i = bch * RP + ip;
+                // element-major order: HG independent accumulators between dependent FMAs
                 float s[HG];
+                {
+                    const float k0 = widen(kk[i][0]);
 #pragma unroll
-                for (int h = 0; h < HG; ++h) {
-                    float acc = 0.0f;
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) acc = fmaf((float)kk[i][j], q[h][j], acc);
-                    s[h] = acc;
+                    for (int h = 0; h < HG; ++h) s[h] = k0 * q[h][0];
                 }
+#pragma unroll
+                for (int j = 1; j < 8; ++j) {
+                    const float kj = widen(kk[i][j]);
+#pragma unroll
+                    for (int h = 0; h < HG; ++h) s[h] = fmaf(kj, q[h][j], s[h]);
+                }
+                kk[i] = load_row8(kp_next, i * 64 + lane);
 #pragma unroll
                 for (int hq = 0; hq < HQ; ++hq) {
                     const int slot = (HG == 8) ? (ip * 2 + hq) : i;
@@ -209,13 +303,6 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_f16_kernel(const AttnKe
             sval[bch] = part == 0 ? r0 : part == 1 ? r1 : part == 2 ? r2 : r3;
         }
 
-        // K registers are free: start the next page's K rows.
-        if (pg_next < pg1) {
-            const uint16_t* kp = P.kpool + (size_t)phys_next * page_elems + head_off;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) kk[i] = load_row8(kp, i * 64 + lane);
-        }
-
         // ---- online softmax for this lane's head -------------------------------------
         float sv[NB];
         int rowv[NB];
@@ -229,9 +316,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_f16_kernel(const AttnKe
             pm = fmaxf(pm, sv[bch]);
         }
         if (HG == 4) pm = xor_max(pm, 4);
-        pm = xor_max(pm, 8);
-        pm = xor_max(pm, 16);
-        pm = xor_max(pm, 32);
+        pm = max_bits345(pm);
         const float m_new = fmaxf(m_run, pm);
         const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
         const bool changed = __builtin_amdgcn_ballot_w64(m_new > m_run) != 0;
@@ -278,37 +363,40 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_f16_kernel(const AttnKe
                             pr[hq * 4 + 3] = t.w;
             }
 #pragma unroll
-            for (int h = 0; h < HG; ++h)
+            for (int j = 0; j < 8; ++j) {
+                const float vj = widen(vv[i][j]);
 #pragma unroll
-                for (int j = 0; j < 8; ++j) o[h][j] = fmaf((float)vv[i][j], pr[h], o[h][j]);
+                for (int h = 0; h < HG; ++h) o[h][j] = fmaf(vj, pr[h], o[h][j]);
+            }
+            vv[i] = load_row8(vp_next, i * 64 + lane);
         }
         wave_lds_sync();
 
         pg = pg_next;
-        phys = phys_next;
     }
 
+    __builtin_amdgcn_s_setprio(0);
     // ---- wave totals ------------------------------------------------------------------
     if (HG == 4) l_run = xor_sum(l_run, 4);
-    l_run = xor_sum(l_run, 8);
-    l_run = xor_sum(l_run, 16);
-    l_run = xor_sum(l_run, 32);
+    l_run = sum_bits345(l_run);
     if ((lane >> 3) == 0 && (HG == 8 || (lane & 4) == 0)) {
         wave_m[wave][my_head] = m_run;
         wave_l[wave][my_head] = l_run;
     }
     float* ow = reinterpret_cast<float*>(&xs[wave][0]);  // [HG][256] floats = 8 KiB at HG 8
+    // The two half-waves hold partial sums over different rows of the same 8 elements.
+    // Swapping the upper half of o[h][j] with the lower half of o[h][j+4] leaves, after one
+    // add, element j's total in lanes 0-31 and element j+4's total in lanes 32-63.
 #pragma unroll
     for (int h = 0; h < HG; ++h) {
+        f4 t;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) o[h][j] += __shfl_xor(o[h][j], 32, 64);
-        if (hw == 0) {
-            f4 a, c;
-            a.x = o[h][0], a.y = o[h][1], a.z = o[h][2], a.w = o[h][3];
-            c.x = o[h][4], c.y = o[h][5], c.z = o[h][6], c.w = o[h][7];
-            reinterpret_cast<f4*>(ow + h * kHd + dl * 8)[0] = a;
-            reinterpret_cast<f4*>(ow + h * kHd + dl * 8)[1] = c;
+        for (int j = 0; j < 4; ++j) {
+            float a = o[h][j], c = o[h][j + 4];
+            permlane32_swap(a, c);
+            t[j] = a + c;
         }
+        *reinterpret_cast<f4*>(ow + h * kHd + dl * 8 + hw * 4) = t;
     }
     __syncthreads();
 
@@ -345,8 +433,16 @@ struct MergeParams {
     int32_t n_kv, n_q, group, hg;
 };
 
-// One work-group per (entry, q head); thread = head-dim element.
-__global__ __launch_bounds__(kHd) void decode_attn_merge_kernel(const MergeParams P) {
+constexpr int kMergeGroups = 4;  // split ranges summed side by side, then folded in LDS
+
+// One work-group per (entry, q head): kMergeGroups x 256 threads.  Thread (g, d) adds the
+// partial outputs of splits g, g + 4, ... for head-dim element d with four loads in flight;
+// the per-split (m, l) pairs are staged in LDS once.
+__global__ __launch_bounds__(kHd * kMergeGroups) void decode_attn_merge_kernel(const MergeParams P) {
+    constexpr int kMaxStaged = 1024;
+    __shared__ float sm[kMaxStaged];
+    __shared__ float sl[kMaxStaged];
+    __shared__ float red[kMergeGroups][kHd];
     const int e = blockIdx.x / P.n_q;
     const int h = blockIdx.x % P.n_q;
     const int kvh = h / P.group;
@@ -355,29 +451,71 @@ __global__ __launch_bounds__(kHd) void decode_attn_merge_kernel(const MergeParam
     const int hh = hl % P.hg;
     const int splits = P.b.splits[e];
     const int wg0 = P.b.wg_base[e] + hc * splits * P.n_kv + kvh;
-    const int d = threadIdx.x;
+    const int d = threadIdx.x & (kHd - 1);
+    const int g = threadIdx.x >> 8;
+    const int staged = min(splits, kMaxStaged);
+    for (int s = threadIdx.x; s < staged; s += kHd * kMergeGroups) {
+        const size_t wg = (size_t)(wg0 + s * P.n_kv);
+        sm[s] = P.part_ml[(wg * P.hg + hh) * 2];
+        sl[s] = P.part_ml[(wg * P.hg + hh) * 2 + 1];
+    }
+    __syncthreads();
     float mx = -INFINITY;
     for (int s = 0; s < splits; ++s) {
-        const size_t wg = (size_t)(wg0 + s * P.n_kv);
-        mx = fmaxf(mx, P.part_ml[(wg * P.hg + hh) * 2]);
+        const float ms = s < kMaxStaged ? sm[s]
+                                        : P.part_ml[((size_t)(wg0 + s * P.n_kv) * P.hg + hh) * 2];
+        mx = fmaxf(mx, ms);
     }
     float acc = 0.0f, lsum = 0.0f;
-    for (int s = 0; s < splits; ++s) {
-        const size_t wg = (size_t)(wg0 + s * P.n_kv);
-        const float ms = P.part_ml[(wg * P.hg + hh) * 2];
+    const size_t ostride = (size_t)P.n_kv * P.hg * kHd;  // floats between consecutive splits
+    const float* po = P.part_o + ((size_t)wg0 * P.hg + hh) * kHd + d;
+    int s = g;
+    for (; s + 3 * kMergeGroups < splits; s += 4 * kMergeGroups) {
+        float v[4], f[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = po[(size_t)(s + u * kMergeGroups) * ostride];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int su = s + u * kMergeGroups;
+            const float ms = su < kMaxStaged
+                                 ? sm[su]
+                                 : P.part_ml[((size_t)(wg0 + su * P.n_kv) * P.hg + hh) * 2];
+            const float ls = su < kMaxStaged
+                                 ? sl[su]
+                                 : P.part_ml[((size_t)(wg0 + su * P.n_kv) * P.hg + hh) * 2 + 1];
+            f[u] = ms == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(ms - mx);
+            lsum = fmaf(f[u], ls, lsum);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) acc = fmaf(f[u], v[u], acc);
+    }
+    for (; s < splits; s += kMergeGroups) {
+        const float ms =
+            s < kMaxStaged ? sm[s] : P.part_ml[((size_t)(wg0 + s * P.n_kv) * P.hg + hh) * 2];
+        const float ls =
+            s < kMaxStaged ? sl[s] : P.part_ml[((size_t)(wg0 + s * P.n_kv) * P.hg + hh) * 2 + 1];
         const float f = ms == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(ms - mx);
-        acc = fmaf(f, P.part_o[(wg * P.hg + hh) * kHd + d], acc);
-        lsum = fmaf(f, P.part_ml[(wg * P.hg + hh) * 2 + 1], lsum);
+        acc = fmaf(f, po[(size_t)s * ostride], acc);
+        lsum = fmaf(f, ls, lsum);
+    }
+    red[g][d] = acc;
+    if (d == 0) sm[g] = lsum;  // sm is free again: every thread has its own copy of mx
+    __syncthreads();
+    if (g != 0) return;
+#pragma unroll
+    for (int k = 1; k < kMergeGroups; ++k) {
+        acc += red[k][d];
+        lsum += sm[k];
     }
     float r = lsum > 0.0f ? acc / lsum : 0.0f;
     if (P.gate) {
-        const float g = P.gate[(size_t)e * P.gate_seq_stride + (size_t)h * P.gate_head_stride + d];
+        const float gt = P.gate[(size_t)e * P.gate_seq_stride + (size_t)h * P.gate_head_stride + d];
         // sigmoid in the overflow-free form of the reference (qsa/cpu.rs:84-91)
         float sg;
-        if (g >= 0.0f) {
-            sg = 1.0f / (1.0f + expf(-g));
+        if (gt >= 0.0f) {
+            sg = 1.0f / (1.0f + expf(-gt));
         } else {
-            const float t = expf(g);
+            const float t = expf(gt);
             sg = t / (1.0f + t);
         }
         r *= sg;
@@ -442,16 +580,17 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
     kp.n_hc = (group + hg - 1) / hg;
     kp.scale_log2e = a.scale * kLog2e;
     const int32_t total = b.wg_base[b.n];
+    const int32_t n_units = total / kp.n_hc;
+    const int32_t grid = (n_units + 7) / 8 * 8 * kp.n_hc;
     {
         StageScope timed(p, BKV_STAGE_ATTN_SPLIT, stream);
         if (hg == 8)
-            decode_attn_f16_kernel<8><<<total, kBlock, 0, stream>>>(kp);
+            decode_attn_f16_kernel<8><<<grid, kBlock, 0, stream>>>(kp);
         else
-            decode_attn_f16_kernel<4><<<total, kBlock, 0, stream>>>(kp);
+            decode_attn_f16_kernel<4><<<grid, kBlock, 0, stream>>>(kp);
     }
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) return err;
-
     MergeParams mp;
     mp.b = b;
     mp.part_o = p->part_o;
@@ -466,7 +605,7 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
     mp.hg = hg;
     {
         StageScope timed(p, BKV_STAGE_ATTN_MERGE, stream);
-        decode_attn_merge_kernel<<<b.n * a.n_q_head, kHd, 0, stream>>>(mp);
+        decode_attn_merge_kernel<<<b.n * a.n_q_head, kHd * kMergeGroups, 0, stream>>>(mp);
     }
     return hipGetLastError();
 }
