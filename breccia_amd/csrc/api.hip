@@ -207,6 +207,9 @@ bkv_status bkv_pool_create(const bkv_pool_desc* d, bkv_pool** out) {
                                           d->page_cells));
     if (d->layout < BKV_LAYOUT_F16 || d->layout > BKV_LAYOUT_I8H)
         return fail(BKV_ERR_INVALID, sfmt("pool_create: unknown layout %lld", d->layout));
+    if (d->layout == BKV_LAYOUT_I8H && d->head_dim != 256)
+        return fail(BKV_ERR_INVALID, "pool_create: the int8 + f16-scale layout is built for "
+                                     "head_dim 256 (272-byte rows keep 16-byte alignment)");
     if ((int64_t)d->n_pages * d->page_cells >= (int64_t)1 << 31)
         return fail(BKV_ERR_INVALID, "pool_create: n_pages * page_cells must stay below 2^31");
 
@@ -577,9 +580,7 @@ bkv_status bkv_page_copy(bkv_pool* p, const bkv_page_pair* pairs, int32_t n_pair
         return fail(BKV_ERR_INVALID, "page_copy: a destination page appears twice");
     bkv_status st = need_device(p);
     if (st != BKV_OK) return st;
-    const int32_t per_launch = std::min<int32_t>(
-        (int32_t)(ParamRing::kSlotBytes / sizeof(bkv_page_pair)), 65535 / (p->g.n_layers * 2));
-    if (per_launch <= 0) return fail(BKV_ERR_INVALID, "page_copy: too many layers for one launch");
+    const int32_t per_launch = (int32_t)(ParamRing::kSlotBytes / sizeof(bkv_page_pair));
     for (int32_t at = 0; at < n_pairs; at += per_launch) {
         const int32_t n = std::min(per_launch, n_pairs - at);
         void* dev;

@@ -11,6 +11,17 @@ namespace {
 
 constexpr int kBlock = 256;
 
+// 16-byte vector the nontemporal builtins accept.  Streaming copies that will not be re-read
+// by this kernel go around the caches' replacement policy (measured on MI355X: 6.2 vs 5.8
+// TB/s for a page-granular device copy).
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ v4u ld_stream(const void* p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const v4u*>(p));
+}
+__device__ __forceinline__ void st_stream(void* p, v4u v) {
+    __builtin_nontemporal_store(v, reinterpret_cast<v4u*>(p));
+}
+
 // f32 -> binary16 code under the cache's storage rule
 // (crates/breccia-kernels/shaders/f16_storage.glsl:26-55, qsa/cpu.rs:23-53):
 // round-to-nearest-even like the hardware convert, except that every |x| < 2^-14
@@ -71,21 +82,20 @@ __global__ __launch_bounds__(kBlock) void append_f16_kernel(AppendBatch b, MoveG
     const size_t dst = row * (size_t)g.hd + d0;
     const size_t src = ((size_t)b.src0[s] + (size_t)t) * (size_t)(g.n_kv * g.hd) + (size_t)r * 8;
 
-    const float4 k0 = *reinterpret_cast<const float4*>(k + src);
-    const float4 k1 = *reinterpret_cast<const float4*>(k + src + 4);
-    const float4 v0 = *reinterpret_cast<const float4*>(v + src);
-    const float4 v1 = *reinterpret_cast<const float4*>(v + src + 4);
-    uint4 ko, vo;
-    ko.x = pack2(k0.x, k0.y);
-    ko.y = pack2(k0.z, k0.w);
-    ko.z = pack2(k1.x, k1.y);
-    ko.w = pack2(k1.z, k1.w);
-    vo.x = pack2(v0.x, v0.y);
-    vo.y = pack2(v0.z, v0.w);
-    vo.z = pack2(v1.x, v1.y);
-    vo.w = pack2(v1.z, v1.w);
-    *reinterpret_cast<uint4*>(kpool + dst) = ko;
-    *reinterpret_cast<uint4*>(vpool + dst) = vo;
+    const v4u k0 = ld_stream(k + src), k1 = ld_stream(k + src + 4);
+    const v4u v0 = ld_stream(v + src), v1 = ld_stream(v + src + 4);
+    const auto f = [](unsigned bits) { return __uint_as_float(bits); };
+    v4u ko, vo;
+    ko.x = pack2(f(k0.x), f(k0.y));
+    ko.y = pack2(f(k0.z), f(k0.w));
+    ko.z = pack2(f(k1.x), f(k1.y));
+    ko.w = pack2(f(k1.z), f(k1.w));
+    vo.x = pack2(f(v0.x), f(v0.y));
+    vo.y = pack2(f(v0.z), f(v0.w));
+    vo.z = pack2(f(v1.x), f(v1.y));
+    vo.w = pack2(f(v1.z), f(v1.w));
+    st_stream(kpool + dst, ko);
+    st_stream(vpool + dst, vo);
 }
 
 // q8_0 codes of 32 values (shaders/qsa_kv_append.comp:113-132, qsa/cpu.rs:65-82):
@@ -242,16 +252,16 @@ __global__ __launch_bounds__(kBlock) void append_i8h_kernel(AppendBatch b, MoveG
 // to 16 KiB, which is one f16 K or V page.
 __device__ __forceinline__ void move_bytes16(const uint4* __restrict__ src, uint4* __restrict__ dst,
                                              uint32_t n_vec, uint32_t base) {
-    uint4 r[4];
+    v4u r[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const uint32_t idx = base + (uint32_t)i * kBlock + threadIdx.x;
-        if (idx < n_vec) r[i] = src[idx];
+        if (idx < n_vec) r[i] = ld_stream(src + idx);
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const uint32_t idx = base + (uint32_t)i * kBlock + threadIdx.x;
-        if (idx < n_vec) dst[idx] = r[i];
+        if (idx < n_vec) st_stream(dst + idx, r[i]);
     }
 }
 
@@ -263,21 +273,57 @@ struct PoolPtrs {
     int32_t n_layers;
 };
 
-// grid.y = pair * n_layers * 2 + layer * 2 + which; grid.x = 16 KiB chunk of the page.
-__global__ __launch_bounds__(kBlock) void page_copy_kernel(PoolPtrs pp,
-                                                           const bkv_page_pair* __restrict__ pairs) {
-    const uint32_t u = blockIdx.y;
-    const uint32_t which = u & 1u;
-    const uint32_t layer = (u >> 1) % (uint32_t)pp.n_layers;
-    const uint32_t pair = (u >> 1) / (uint32_t)pp.n_layers;
+// A unit is one 16 KiB chunk of one (pair, layer, K|V) page image.  A work-group copies
+// whole chunks (each wave 4 x 1 KiB contiguous), walking the unit list with a grid stride;
+// the (src, dst) pair of the next unit is fetched while the current chunk is in flight.
+struct CopyUnit {
+    const uint8_t* src;
+    uint8_t* dst;
+    uint32_t n_vec;  // 16-byte vectors left in the page image from this chunk's start
+};
+
+__device__ __forceinline__ CopyUnit copy_unit(const PoolPtrs& pp, const bkv_page_pair pr,
+                                              uint32_t pl, uint32_t chunk, uint32_t chunks_k) {
+    const uint32_t which = chunk >= chunks_k ? 1u : 0u;
+    if (which) chunk -= chunks_k;
+    const uint32_t layer = pl % (uint32_t)pp.n_layers;
     const uint64_t pb = which ? pp.v_page_bytes : pp.k_page_bytes;
-    const uint32_t n_vec = (uint32_t)(pb / 16);
-    const uint32_t base = blockIdx.x * (4u * kBlock);
-    if (base >= n_vec) return;
     uint8_t* pool = pp.slab + (uint64_t)layer * pp.layer_stride + (which ? pp.v_offset : 0);
-    const bkv_page_pair pr = pairs[pair];
-    move_bytes16(reinterpret_cast<const uint4*>(pool + (uint64_t)pr.src * pb),
-                 reinterpret_cast<uint4*>(pool + (uint64_t)pr.dst * pb), n_vec, base);
+    const uint64_t off = (uint64_t)chunk * (4u * kBlock * 16u);
+    CopyUnit u;
+    u.src = pool + (uint64_t)pr.src * pb + off;
+    u.dst = pool + (uint64_t)pr.dst * pb + off;
+    u.n_vec = (uint32_t)((pb - off) / 16);
+    return u;
+}
+
+__global__ __launch_bounds__(kBlock) void page_copy_kernel(PoolPtrs pp,
+                                                           const bkv_page_pair* __restrict__ pairs,
+                                                           uint32_t n_pairs, uint32_t chunks_k,
+                                                           uint32_t chunks_v) {
+    const uint32_t per_pl = chunks_k + chunks_v;
+    const uint32_t total = n_pairs * (uint32_t)pp.n_layers * per_pl;
+    uint32_t c = blockIdx.x;
+    if (c >= total) return;
+    bkv_page_pair pr = pairs[(c / per_pl) / (uint32_t)pp.n_layers];
+    while (c < total) {
+        const uint32_t pl = c / per_pl;
+        const CopyUnit u = copy_unit(pp, pr, pl, c - pl * per_pl, chunks_k);
+        const uint32_t c_next = c + gridDim.x;
+        if (c_next < total) pr = pairs[(c_next / per_pl) / (uint32_t)pp.n_layers];
+        v4u r[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t idx = (uint32_t)i * kBlock + threadIdx.x;
+            if (idx < u.n_vec) r[i] = ld_stream(u.src + (size_t)idx * 16);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t idx = (uint32_t)i * kBlock + threadIdx.x;
+            if (idx < u.n_vec) st_stream(u.dst + (size_t)idx * 16, r[i]);
+        }
+        c = c_next;
+    }
 }
 
 // Staging layout: [page i][layer][K page bytes | V page bytes].
@@ -429,11 +475,14 @@ hipError_t launch_append(const bkv_pool* p, int32_t layer, const AppendBatch& b,
 hipError_t launch_page_copy(const bkv_pool* p, const bkv_page_pair* pairs_dev, int32_t n_pairs,
                             hipStream_t stream) {
     const PoolPtrs pp = pool_ptrs(p);
-    const uint64_t pb = pp.k_page_bytes > pp.v_page_bytes ? pp.k_page_bytes : pp.v_page_bytes;
-    const unsigned chunks = (unsigned)((pb / 16 + 4 * kBlock - 1) / (4 * kBlock));
-    // grid.y is limited to 65535: callers pass at most kMaxPairsPerLaunch pairs.
-    dim3 grid(chunks, (unsigned)n_pairs * (unsigned)pp.n_layers * 2u);
-    page_copy_kernel<<<grid, kBlock, 0, stream>>>(pp, pairs_dev);
+    const uint32_t chunks_k = (uint32_t)((pp.k_page_bytes / 16 + 4 * kBlock - 1) / (4 * kBlock));
+    const uint32_t chunks_v = (uint32_t)((pp.v_page_bytes / 16 + 4 * kBlock - 1) / (4 * kBlock));
+    const uint64_t total = (uint64_t)n_pairs * (uint64_t)pp.n_layers * (chunks_k + chunks_v);
+    uint64_t grid = total;
+    const uint64_t cap = (uint64_t)(p->n_cu > 0 ? p->n_cu : 256) * 32;
+    if (grid > cap) grid = cap;
+    page_copy_kernel<<<(unsigned)grid, kBlock, 0, stream>>>(pp, pairs_dev, (uint32_t)n_pairs, chunks_k,
+                                                         chunks_v);
     return hipGetLastError();
 }
 

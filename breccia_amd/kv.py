@@ -275,11 +275,11 @@ class Pool:
                                   _ptr(out_dev), _sh(stream)))
 
     def page_copy(self, pairs, stream=None) -> None:
-        pairs = list(pairs)
-        arr = (PagePair * max(len(pairs), 1))()
-        for i, (s, d) in enumerate(pairs):
-            arr[i].src, arr[i].dst = int(s), int(d)
-        check(lib.bkv_page_copy(self.handle, arr, len(pairs), _sh(stream)))
+        """pairs: iterable of (src, dst), or an int32 array of shape [n, 2]."""
+        arr = np.ascontiguousarray(np.asarray(list(pairs) if not isinstance(pairs, np.ndarray)
+                                              else pairs, dtype=np.int32).reshape(-1, 2))
+        ptr = arr.ctypes.data_as(C.POINTER(PagePair))
+        check(lib.bkv_page_copy(self.handle, ptr, arr.shape[0], _sh(stream)))
 
     def gather(self, layer: int, seq: int, cell0: int, n: int, stream=None):
         """Dequantised K and V rows as float32 arrays [n, n_kv, head_dim]."""
