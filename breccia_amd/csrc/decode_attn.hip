@@ -127,13 +127,23 @@ __device__ __forceinline__ float widen(_Float16 h) {
     return f;
 }
 
+// K/V rows are read exactly once per kernel: nontemporal loads keep them from displacing
+// the block tables, q and the split partials in the caches.
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ half8 load_row8(const uint16_t* base, int idx) {
-    return __builtin_bit_cast(half8, reinterpret_cast<const uint4*>(base)[idx]);
+    return __builtin_bit_cast(half8,
+                              __builtin_nontemporal_load(reinterpret_cast<const v4u*>(base) + idx));
 }
 
-// HG = q heads carried by one wave (8 or 4).
-template <int HG>
-__global__ __launch_bounds__(kBlock, 2) void decode_attn_f16_kernel(const AttnKernelParams P) {
+// HG = q heads carried by one wave (8 or 4).  CH = head chunks inside the work-group: with
+// CH = 2, waves 2s and 2s+1 walk the same pages (page stream s) for different halves of the
+// head group, so the second wave's row loads hit the CU's L1; each wave then needs half the
+// q / accumulator registers, which lifts occupancy from 2 to 3 waves per SIMD.
+template <int HG, int CH>
+__global__ __launch_bounds__(kBlock, (HG * CH > 4 && CH == 1) ? 2 : 3) void decode_attn_f16_kernel(
+    const AttnKernelParams P) {
+    constexpr int kStreams = kWaves / CH;  // page streams per work-group
+    constexpr int HW = HG * CH;            // heads per work-group
     constexpr int HQ = HG / 4;           // float4 groups of heads
     constexpr int NB = HG / 4;           // score batches per page (8 float4 slots each)
     constexpr int RP = 8 / NB;           // row pairs per batch
@@ -173,6 +183,8 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_f16_kernel(const AttnKe
     const table_ptr bt = (table_ptr)(uintptr_t)(P.tables + (size_t)P.b.row[e] * (size_t)P.max_pages_per_seq);
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int chunk = wave % CH;    // head chunk inside the work-group
+    const int stream = wave / CH;   // page stream
     const int lane = threadIdx.x & 63;
     const int hw = lane >> 5;   // row parity this lane loads
     const int dl = lane & 31;   // 8-element slice of the head dim
@@ -181,7 +193,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_f16_kernel(const AttnKe
     float q[HG][8];
 #pragma unroll
     for (int h = 0; h < HG; ++h) {
-        const int hl = hc * HG + h;
+        const int hl = (hc * CH + chunk) * HG + h;
         if (hl < P.group) {
             const float* qp =
                 P.q + ((size_t)e * P.n_q + (size_t)kvh * P.group + hl) * kHd + dl * 8;
@@ -223,7 +235,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_f16_kernel(const AttnKe
     // K and V rows of a page sit in registers (8 x 16 bytes each per lane).  Every register
     // group is refilled with the next page's row right after its last use, so each load has
     // a whole page of work in front of it and 16 loads per wave stay in flight.
-    int pg = pg0 + wave;
+    int pg = pg0 + stream;
     half8 kk[8], vv[8];
     if (pg < pg1) {
         const int32_t phys = bt[pg];
@@ -252,7 +264,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_f16_kernel(const AttnKe
         // The next page is fetched unconditionally (the last iteration re-reads its own
         // page): one straight-line load sequence lets the compiler count outstanding loads
         // exactly instead of draining them at a control-flow join.
-        const int pg_next = pg + kWaves;
+        const int pg_next = pg + kStreams;
         const int32_t phys_next = bt[min(pg_next, pg1 - 1)];
         const uint16_t* kp_next = P.kpool + (size_t)phys_next * page_elems + head_off;
         const uint16_t* vp_next = P.vpool + (size_t)phys_next * page_elems + head_off;
@@ -403,22 +415,25 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_f16_kernel(const AttnKe
     // ---- merge the four waves; thread = head-dim element ----------------------------
     const int d = threadIdx.x;
 #pragma unroll
-    for (int h = 0; h < HG; ++h) {
-        float mx = wave_m[0][h];
+    for (int hw_ = 0; hw_ < HW; ++hw_) {
+        const int c = hw_ / HG;  // chunk that carried this head
+        const int h = hw_ % HG;
+        float mx = wave_m[c][h];
 #pragma unroll
-        for (int w = 1; w < kWaves; ++w) mx = fmaxf(mx, wave_m[w][h]);
+        for (int s = 1; s < kStreams; ++s) mx = fmaxf(mx, wave_m[s * CH + c][h]);
         float acc = 0.0f, lsum = 0.0f;
 #pragma unroll
-        for (int w = 0; w < kWaves; ++w) {
+        for (int s = 0; s < kStreams; ++s) {
+            const int w = s * CH + c;
             const float mw = wave_m[w][h];
             const float f = mw == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(mw - mx);
             acc = fmaf(f, reinterpret_cast<const float*>(&xs[w][0])[h * kHd + d], acc);
             lsum = fmaf(f, wave_l[w][h], lsum);
         }
-        P.part_o[((size_t)wg * HG + h) * kHd + d] = acc;
+        P.part_o[((size_t)wg * HW + hw_) * kHd + d] = acc;
         if (d == 0) {
-            P.part_ml[((size_t)wg * HG + h) * 2 + 0] = mx;
-            P.part_ml[((size_t)wg * HG + h) * 2 + 1] = lsum;
+            P.part_ml[((size_t)wg * HW + hw_) * 2 + 0] = mx;
+            P.part_ml[((size_t)wg * HW + hw_) * 2 + 1] = lsum;
         }
     }
 }
@@ -525,7 +540,10 @@ __global__ __launch_bounds__(kHd * kMergeGroups) void decode_attn_merge_kernel(c
 
 }  // namespace
 
+// Heads one work-group carries for a given q-heads-per-kv-head group.
 int32_t attn_heads_per_wave(int32_t group) { return group % 8 == 0 ? 8 : 4; }
+// Whole groups of 8 heads are carried as two in-work-group chunks of 4 (see the kernel).
+constexpr bool kSplitEightInWorkgroup = false;
 
 int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b) {
     const int32_t n_kv = p->g.n_kv;
@@ -535,8 +553,13 @@ int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b) {
     const int64_t per_page = (int64_t)n_kv * n_hc;
     int64_t total_pages = 0;
     for (int i = 0; i < b.n; ++i) total_pages += b.pos[i] / kPage + 1;
-    // Two work-groups stay resident per CU (register budget); aim at one generation.
-    const int64_t target = (int64_t)(p->n_cu > 0 ? p->n_cu : 256) * 2;
+    // All work-groups should be resident at once (one generation): a handful of left-over
+    // work-groups would run alone after the rest and double the kernel's time.  `resident`
+    // follows from the register budget of the kernel variant that will run.
+    const bool split8 = hg == 8 && kSplitEightInWorkgroup;
+    const int64_t resident = split8 ? 3 : 2;
+    int64_t target = (int64_t)(p->n_cu > 0 ? p->n_cu : 256) * resident;
+    if (target > p->max_wgs) target = p->max_wgs;
     int64_t pps = (total_pages * per_page + target - 1) / target;
     pps = ((pps + kWaves - 1) / kWaves) * kWaves;
     if (pps < kWaves) pps = kWaves;
@@ -544,19 +567,18 @@ int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b) {
         int64_t total = 0;
         for (int i = 0; i < b.n; ++i) {
             const int64_t pages = b.pos[i] / kPage + 1;
-            int64_t splits = (pages + pps - 1) / pps;
+            const int64_t splits = (pages + pps - 1) / pps;
             // even the ranges out inside the entry, keeping whole groups of kWaves pages
             int64_t each = (pages + splits - 1) / splits;
             each = ((each + kWaves - 1) / kWaves) * kWaves;
-            splits = (pages + each - 1) / each;
-            b.splits[i] = (int32_t)splits;
+            b.splits[i] = (int32_t)((pages + each - 1) / each);
             b.pps[i] = (int32_t)each;
             b.wg_base[i] = (int32_t)total;
-            total += splits * per_page;
+            total += (int64_t)b.splits[i] * per_page;
         }
         b.wg_base[b.n] = (int32_t)total;
-        if (total <= p->max_wgs) return (int32_t)total;
-        pps *= 2;
+        if (total <= target) return (int32_t)total;
+        pps += kWaves;
     }
 }
 
@@ -584,10 +606,12 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
     const int32_t grid = (n_units + 7) / 8 * 8 * kp.n_hc;
     {
         StageScope timed(p, BKV_STAGE_ATTN_SPLIT, stream);
-        if (hg == 8)
-            decode_attn_f16_kernel<8><<<grid, kBlock, 0, stream>>>(kp);
+        if (hg == 8 && kSplitEightInWorkgroup)
+            decode_attn_f16_kernel<4, 2><<<grid, kBlock, 0, stream>>>(kp);
+        else if (hg == 8)
+            decode_attn_f16_kernel<8, 1><<<grid, kBlock, 0, stream>>>(kp);
         else
-            decode_attn_f16_kernel<4><<<grid, kBlock, 0, stream>>>(kp);
+            decode_attn_f16_kernel<4, 1><<<grid, kBlock, 0, stream>>>(kp);
     }
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) return err;
