@@ -59,5 +59,20 @@ def build(verbose: bool = False) -> str:
     return LIB
 
 
+def build_cpp_mirror_test(verbose: bool = False) -> str:
+    """The C++ test program of the host mirror (tests/cpp); links the library and the oracle."""
+    root = os.path.abspath(os.path.join(HERE, ".."))
+    src = os.path.join(root, "tests", "cpp", "qsa_mirror_test.cpp")
+    out = os.path.join(root, "tests", "cpp", "qsa_mirror_test")
+    cmd = ["g++", "-std=c++17", "-O2", "-Wall", src, "-o", out,
+           "-L" + HERE, "-lbreccia_kv", "-L" + os.path.join(root, "oracle"), "-lbkv_oracle",
+           "-Wl,-rpath,$ORIGIN/../../breccia_amd", "-Wl,-rpath,$ORIGIN/../../oracle",
+           "-Wl,-rpath,/opt/rocm/lib"]
+    if verbose:
+        print(" ".join(cmd))
+    _run(cmd)
+    return out
+
+
 if __name__ == "__main__":
     print(build(verbose=True))

@@ -1,0 +1,189 @@
+// Drives the C++ host mirror of the reference interface (breccia_amd/csrc/qsa.hpp) the way
+// the reference's own conformance tests drive Qsa (crates/breccia-kernels/tests/
+// attn_conformance.rs:1172-1275 for the layout recipe), checking the GPU against the CPU
+// oracle.  Built by __graft_entry__.build(); run on the GPU box by tests/test_gpu_cpp_mirror.py.
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <vector>
+
+#include "../../breccia_amd/csrc/qsa.hpp"
+
+// CPU oracle (test infrastructure), oracle/bkv_oracle.c
+extern "C" {
+typedef struct {
+    int32_t n_kv, head_dim, page_cells;
+} bkvo_geom;
+int bkvo_append_f16(const bkvo_geom*, uint16_t*, uint16_t*, const int32_t*, int64_t, int64_t, int64_t,
+                    const float*, const float*);
+int bkvo_gather(const bkvo_geom*, int, const void*, const void*, const int32_t*, int64_t, int64_t, float*,
+                float*);
+int bkvo_attend(const float*, const float*, const float*, const uint32_t*, size_t, int64_t, int32_t,
+                int32_t, int32_t, const float*, float*, int);
+void bkvo_normalish(uint64_t, size_t, float*);
+}
+
+using namespace breccia::qsa;
+
+static int failures = 0;
+#define EXPECT(cond, ...)                                  \
+    do {                                                   \
+        if (!(cond)) {                                     \
+            std::printf("FAIL %s:%d: ", __FILE__, __LINE__); \
+            std::printf(__VA_ARGS__);                      \
+            std::printf("\n");                             \
+            ++failures;                                    \
+        }                                                  \
+    } while (0)
+
+static void upload(float* dev, const std::vector<float>& h) {
+    check(bkv_memcpy_h2d(dev, h.data(), h.size() * 4, nullptr));
+    check(bkv_stream_sync(nullptr));
+}
+
+template <typename T>
+static std::vector<T> download(const void* dev, size_t count) {
+    std::vector<T> h(count);
+    check(bkv_memcpy_d2h(h.data(), dev, count * sizeof(T), nullptr));
+    check(bkv_stream_sync(nullptr));
+    return h;
+}
+
+static void test_errors() {
+    bool threw = false;
+    try {
+        QsaState::create(0, 64);
+    } catch (const Error& e) {
+        threw = e.status == BKV_ERR_INVALID;
+    }
+    EXPECT(threw, "capacity 0 must be refused");
+    Qsa qsa;
+    threw = false;
+    try {
+        qsa.workspace(0, 1);
+    } catch (const Error& e) {
+        threw = e.status == BKV_ERR_INVALID;
+    }
+    EXPECT(threw, "a workspace of 0 tokens must be refused");
+}
+
+static void test_layout_recipe() {
+    // capacity 40 cells = 3 pages, 33 single-token appends from cell 5
+    QsaState state = QsaState::create(40, 64);
+    EXPECT(state.capacity_cells == 48, "capacity rounds up to pages, got %zu", state.capacity_cells);
+    Qsa qsa;
+    QsaWorkspace ws = qsa.workspace(1, 38);
+    const bkvo_geom g{2, 256, 16};
+    const int32_t table[3] = {0, 1, 2};
+    std::vector<uint16_t> want_k(3 * 2 * 16 * 256, 0), want_v(want_k.size(), 0);
+    for (int t = 0; t < 33; ++t) {
+        const int cell = 5 + t;
+        std::vector<float> k(512), v(512);
+        for (int i = 0; i < 512; ++i) {
+            k[i] = std::sin((float)(cell * 97 + i * 13) * 0.017f) * 3.0f;
+            v[i] = std::cos((float)(cell * 61 + i * 7) * 0.031f) * 2.0f;
+        }
+        upload(ws.k_cur, k);
+        upload(ws.v_cur, v);
+        qsa.kv_append(state, ws, (size_t)cell);
+        bkvo_append_f16(&g, want_k.data(), want_v.data(), table, 48, cell, 1, k.data(), v.data());
+    }
+    uint64_t nbytes = 0;
+    void* kp = state.pool_ptr(0, &nbytes);
+    EXPECT(nbytes == want_k.size() * 2, "k_pool is %llu bytes", (unsigned long long)nbytes);
+    const auto got_k = download<uint16_t>(kp, want_k.size());
+    const auto got_v = download<uint16_t>(state.pool_ptr(1), want_v.size());
+    size_t bad = 0;
+    for (size_t i = 0; i < want_k.size(); ++i) bad += (got_k[i] != want_k[i]) + (got_v[i] != want_v[i]);
+    EXPECT(bad == 0, "%zu of %zu stored halves differ from the cache encoding", bad, 2 * want_k.size());
+    std::printf("qsa kv layout+f16   %d K/V elements, %zu differ (33 cells, 3 pages)\n", 33 * 512, bad);
+
+    // append past the capacity is an Err, not a launch (qsa/mod.rs:1108-1116)
+    bool threw = false;
+    try {
+        qsa.kv_append(state, ws, 48);
+    } catch (const Error& e) {
+        threw = e.status == BKV_ERR_RANGE;
+    }
+    EXPECT(threw, "append at cell 48 of a 48-cell cache must be refused");
+
+    state.reset();
+    const auto zero = download<uint16_t>(state.pool_ptr(0), want_k.size());
+    bad = 0;
+    for (uint16_t h : zero) bad += h != 0;
+    EXPECT(bad == 0, "reset must zero the pool");
+    qsa.release(ws);
+    state.release();
+}
+
+static void test_attention() {
+    // 24 heads, gate read in place from q_full, T = 3 decode tokens after a 61-cell prefill
+    const int cells = 64, T = 3, H = MODEL_N_HEAD, hd = MODEL_HEAD_DIM;
+    QsaState state = QsaState::create(cells, 64);
+    Qsa qsa;
+    const bkvo_geom g{2, 256, 16};
+    const int32_t table[4] = {0, 1, 2, 3};
+    std::vector<float> k_all(cells * 512), v_all(cells * 512), q(T * H * hd), q_full(T * H * 2 * hd);
+    bkvo_normalish(0xF1, k_all.size(), k_all.data());
+    bkvo_normalish(0xF2, v_all.size(), v_all.data());
+    bkvo_normalish(0xF3, q.size(), q.data());
+    bkvo_normalish(0xF4, q_full.size(), q_full.data());
+    QsaWorkspace fill = qsa.workspace(cells, cells);
+    upload(fill.k_cur, k_all);
+    upload(fill.v_cur, v_all);
+    qsa.kv_append(state, fill, 0);
+    QsaWorkspace ws = qsa.workspace(T, cells);
+    upload(ws.q, q);
+    upload(ws.q_full, q_full);
+    const size_t pos0 = 61;
+    qsa.attend(state, ws, pos0);
+    qsa.apply(state, ws, pos0);
+    check(bkv_device_sync());
+    const auto out = download<float>(ws.attn_out, (size_t)T * H * hd);
+
+    std::vector<uint16_t> pk(4 * 2 * 16 * 256, 0), pv(pk.size(), 0);
+    bkvo_append_f16(&g, pk.data(), pv.data(), table, cells, 0, cells, k_all.data(), v_all.data());
+    std::vector<float> kf(cells * 512), vf(cells * 512);
+    bkvo_gather(&g, 0, pk.data(), pv.data(), table, 0, cells, kf.data(), vf.data());
+    std::vector<uint32_t> cell_list(cells);
+    for (int c = 0; c < cells; ++c) cell_list[c] = (uint32_t)c;
+    double worst = 0.0;
+    for (int t = 0; t < T; ++t) {
+        std::vector<float> gate(H * hd), want(H * hd);
+        for (int h = 0; h < H; ++h)
+            std::memcpy(&gate[h * hd], &q_full[((size_t)t * H + h) * 2 * hd + hd], hd * 4);
+        bkvo_attend(&q[(size_t)t * H * hd], kf.data(), vf.data(), cell_list.data(), cell_list.size(),
+                    (int64_t)(pos0 + t), H, 2, hd, gate.data(), want.data(), 1);
+        for (int i = 0; i < H * hd; ++i) {
+            const double w = want[i], e = std::fabs((double)out[(size_t)t * H * hd + i] - w);
+            worst = std::fmax(worst, e / std::fmax(std::fabs(w), 1.0));
+        }
+    }
+    // the reference's bar: max |g-w| / max(|w|,1) <= 1e-5 (attn_conformance.rs:102-108, :1148-1151)
+    EXPECT(worst <= 1e-5, "attention max_rel %.3e exceeds 1e-5", worst);
+    std::printf("qsa attend+apply    T=%d, %d heads, gated: max_rel %.3e\n", T, H, worst);
+
+    bool threw = false;
+    try {
+        qsa.apply(state, ws, 62);  // 62 + 3 tokens > 64 cells
+    } catch (const Error& e) {
+        threw = e.status == BKV_ERR_RANGE;
+    }
+    EXPECT(threw, "attention past the capacity must be refused");
+    qsa.release(ws);
+    qsa.release(fill);
+    state.release();
+}
+
+int main() {
+    try {
+        test_errors();
+        test_layout_recipe();
+        test_attention();
+    } catch (const Error& e) {
+        std::printf("FAIL: unexpected error %d: %s\n", (int)e.status, e.what());
+        return 2;
+    }
+    std::printf(failures ? "%d check(s) failed\n" : "all checks passed\n", failures);
+    return failures ? 1 : 0;
+}
