@@ -519,8 +519,6 @@ bkv_status bkv_decode_attn(bkv_pool* p, int32_t layer, int32_t n, const int32_t*
     if (p->g.hd != 256)
         return fail(BKV_ERR_INVALID, sfmt("decode_attn is built for head_dim 256, pool has %lld",
                                           p->g.hd));
-    if (p->g.layout != BKV_LAYOUT_F16)
-        return fail(BKV_ERR_INVALID, "decode_attn: only the f16 K/V layout is built");
     if (n > 0 && (!seqs || !pos)) return fail(BKV_ERR_INVALID, "decode_attn: NULL seqs / pos");
     AttnBatch b{};
     for (int i = 0; i < n; ++i) {

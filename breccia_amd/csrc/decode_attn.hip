@@ -39,8 +39,8 @@ typedef float f4 __attribute__((ext_vector_type(4)));
 
 struct AttnKernelParams {
     AttnBatch b;
-    const uint16_t* kpool;
-    const uint16_t* vpool;
+    const uint8_t* kpool;
+    const uint8_t* vpool;
     const int32_t* tables;
     const float* q;
     float* part_o;
@@ -127,23 +127,99 @@ __device__ __forceinline__ float widen(_Float16 h) {
     return f;
 }
 
+// ---- row buffers -------------------------------------------------------------------
+// A lane owns 8 consecutive head-dim elements (dl = lane % 32) of the rows with parity
+// hw = lane / 32, i.e. rows 2i + hw, i = 0..7, of a 16-cell page.  A RowBuf holds that
+// lane's share of the 8 rows in registers for one of the three row encodings:
+//   kRowF16   256 f16                          one 16-byte load per row
+//   kRowQ8    8 x [f32 scale][32 x i8]         (reference q8_0 V, shaders/qsa_kv_append.comp:
+//             38-44; value = i8 * scale, qsa_attn_apply.comp:70-77): 8 code bytes + scale
+//   kRowI8H   [256 x i8][8 x f16 scale]        8 code bytes + the block's f16 scale
 // K/V rows are read exactly once per kernel: nontemporal loads keep them from displacing
 // the block tables, q and the split partials in the caches.
+constexpr int kRowF16 = 0, kRowQ8 = 1, kRowI8H = 2;
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ half8 load_row8(const uint16_t* base, int idx) {
-    return __builtin_bit_cast(half8,
-                              __builtin_nontemporal_load(reinterpret_cast<const v4u*>(base) + idx));
+typedef unsigned v2u __attribute__((ext_vector_type(2)));
+
+__host__ __device__ constexpr int row_bytes_of(int enc) {
+    return enc == kRowF16 ? kHd * 2 : enc == kRowQ8 ? (kHd / 32) * 36 : kHd + (kHd / 32) * 2;
 }
 
-// HG = q heads carried by one wave (8 or 4).  CH = head chunks inside the work-group: with
-// CH = 2, waves 2s and 2s+1 walk the same pages (page stream s) for different halves of the
-// head group, so the second wave's row loads hit the CU's L1; each wave then needs half the
-// q / accumulator registers, which lifts occupancy from 2 to 3 waves per SIMD.
-template <int HG, int CH>
-__global__ __launch_bounds__(kBlock, (HG * CH > 4 && CH == 1) ? 2 : 3) void decode_attn_f16_kernel(
-    const AttnKernelParams P) {
-    constexpr int kStreams = kWaves / CH;  // page streams per work-group
-    constexpr int HW = HG * CH;            // heads per work-group
+template <int ENC>
+struct RowBuf;
+
+template <>
+struct RowBuf<kRowF16> {
+    half8 r[8];
+    // page = first byte of this (page, kv head)'s 16 rows
+    __device__ __forceinline__ void load(const uint8_t* page, int i, int lane) {
+        r[i] = __builtin_bit_cast(
+            half8, __builtin_nontemporal_load(reinterpret_cast<const v4u*>(page) + i * 64 + lane));
+    }
+    __device__ __forceinline__ float elem(int i, int j) const { return widen(r[i][j]); }
+    static constexpr bool kScaled = false;
+    __device__ __forceinline__ float scale(int) const { return 1.0f; }
+    __device__ __forceinline__ void zero(int i) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) r[i][j] = (_Float16)0.0f;
+    }
+};
+
+__device__ __forceinline__ float code_to_float(v2u w, int j) {
+    // sign-extending byte convert (one SDWA instruction per element)
+    const int sh = (j & 3) * 8;
+    return (float)(int)(int8_t)((j < 4 ? w.x : w.y) >> sh);
+}
+
+template <>
+struct RowBuf<kRowQ8> {
+    v2u code[8];
+    float sc[8];
+    __device__ __forceinline__ void load(const uint8_t* page, int i, int lane) {
+        const int row = 2 * i + (lane >> 5), dl = lane & 31;
+        const uint8_t* blk = page + row * row_bytes_of(kRowQ8) + (dl >> 2) * 36;
+        sc[i] = __builtin_nontemporal_load(reinterpret_cast<const float*>(blk));
+        const unsigned* c = reinterpret_cast<const unsigned*>(blk + 4 + (dl & 3) * 8);
+        code[i].x = __builtin_nontemporal_load(c);
+        code[i].y = __builtin_nontemporal_load(c + 1);
+    }
+    __device__ __forceinline__ float elem(int i, int j) const { return code_to_float(code[i], j); }
+    static constexpr bool kScaled = true;
+    __device__ __forceinline__ float scale(int i) const { return sc[i]; }
+    __device__ __forceinline__ void zero(int i) {
+        code[i].x = code[i].y = 0u;
+        sc[i] = 0.0f;
+    }
+};
+
+template <>
+struct RowBuf<kRowI8H> {
+    v2u code[8];
+    unsigned short sc[8];
+    __device__ __forceinline__ void load(const uint8_t* page, int i, int lane) {
+        const int row = 2 * i + (lane >> 5), dl = lane & 31;
+        const uint8_t* rp = page + row * row_bytes_of(kRowI8H);
+        code[i] = __builtin_nontemporal_load(reinterpret_cast<const v2u*>(rp + dl * 8));
+        sc[i] = __builtin_nontemporal_load(
+            reinterpret_cast<const unsigned short*>(rp + kHd + (dl >> 2) * 2));
+    }
+    __device__ __forceinline__ float elem(int i, int j) const { return code_to_float(code[i], j); }
+    static constexpr bool kScaled = true;
+    // f16 scale under the cache's load rule (exponent field 0 reads as zero)
+    __device__ __forceinline__ float scale(int i) const {
+        const unsigned h = sc[i];
+        const float f = (float)__builtin_bit_cast(_Float16, sc[i]);
+        return (h & 0x7c00u) == 0 ? 0.0f : f;
+    }
+    __device__ __forceinline__ void zero(int i) {
+        code[i].x = code[i].y = 0u;
+        sc[i] = 0;
+    }
+};
+
+// HG = q heads carried by one wave (8 or 4); KENC / VENC = row encodings of the K and V pools.
+template <int HG, int KENC, int VENC>
+__global__ __launch_bounds__(kBlock, HG == 8 ? 2 : 3) void decode_attn_kernel(const AttnKernelParams P) {
     constexpr int HQ = HG / 4;           // float4 groups of heads
     constexpr int NB = HG / 4;           // score batches per page (8 float4 slots each)
     constexpr int RP = 8 / NB;           // row pairs per batch
@@ -183,8 +259,6 @@ __global__ __launch_bounds__(kBlock, (HG * CH > 4 && CH == 1) ? 2 : 3) void deco
     const table_ptr bt = (table_ptr)(uintptr_t)(P.tables + (size_t)P.b.row[e] * (size_t)P.max_pages_per_seq);
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int chunk = wave % CH;    // head chunk inside the work-group
-    const int stream = wave / CH;   // page stream
     const int lane = threadIdx.x & 63;
     const int hw = lane >> 5;   // row parity this lane loads
     const int dl = lane & 31;   // 8-element slice of the head dim
@@ -193,7 +267,7 @@ __global__ __launch_bounds__(kBlock, (HG * CH > 4 && CH == 1) ? 2 : 3) void deco
     float q[HG][8];
 #pragma unroll
     for (int h = 0; h < HG; ++h) {
-        const int hl = (hc * CH + chunk) * HG + h;
+        const int hl = hc * HG + h;
         if (hl < P.group) {
             const float* qp =
                 P.q + ((size_t)e * P.n_q + (size_t)kvh * P.group + hl) * kHd + dl * 8;
@@ -229,22 +303,25 @@ __global__ __launch_bounds__(kBlock, (HG * CH > 4 && CH == 1) ? 2 : 3) void deco
     float m_run = -INFINITY;  // running max of this lane's head (base-2 logits)
     float l_run = 0.0f;       // this lane's share of the denominator
 
-    const size_t page_elems = (size_t)P.n_kv * kPage * kHd;
-    const size_t head_off = (size_t)kvh * kPage * kHd;
+    constexpr size_t kKHead = (size_t)kPage * row_bytes_of(KENC);  // bytes of one kv head's rows
+    constexpr size_t kVHead = (size_t)kPage * row_bytes_of(VENC);
+    const size_t k_page = (size_t)P.n_kv * kKHead, v_page = (size_t)P.n_kv * kVHead;
+    const size_t k_head_off = (size_t)kvh * kKHead, v_head_off = (size_t)kvh * kVHead;
 
-    // K and V rows of a page sit in registers (8 x 16 bytes each per lane).  Every register
-    // group is refilled with the next page's row right after its last use, so each load has
-    // a whole page of work in front of it and 16 loads per wave stay in flight.
-    int pg = pg0 + stream;
-    half8 kk[8], vv[8];
+    // K and V rows of a page sit in registers.  Every register group is refilled with the
+    // next page's row right after its last use, so each load has a whole page of work in
+    // front of it and 16 row loads per wave stay in flight.
+    int pg = pg0 + wave;
+    RowBuf<KENC> kk;
+    RowBuf<VENC> vv;
     if (pg < pg1) {
         const int32_t phys = bt[pg];
-        const uint16_t* kp = P.kpool + (size_t)phys * page_elems + head_off;
-        const uint16_t* vp = P.vpool + (size_t)phys * page_elems + head_off;
+        const uint8_t* kp = P.kpool + (size_t)phys * k_page + k_head_off;
+        const uint8_t* vp = P.vpool + (size_t)phys * v_page + v_head_off;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) kk[i] = load_row8(kp, i * 64 + lane);
+        for (int i = 0; i < 8; ++i) kk.load(kp, i, lane);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) vv[i] = load_row8(vp, i * 64 + lane);
+        for (int i = 0; i < 8; ++i) vv.load(vp, i, lane);
     }
 
     // Two waves share a SIMD (one from each resident work-group) and the issue arbiter
@@ -264,10 +341,10 @@ __global__ __launch_bounds__(kBlock, (HG * CH > 4 && CH == 1) ? 2 : 3) void deco
         // The next page is fetched unconditionally (the last iteration re-reads its own
         // page): one straight-line load sequence lets the compiler count outstanding loads
         // exactly instead of draining them at a control-flow join.
-        const int pg_next = pg + kStreams;
+        const int pg_next = pg + kWaves;
         const int32_t phys_next = bt[min(pg_next, pg1 - 1)];
-        const uint16_t* kp_next = P.kpool + (size_t)phys_next * page_elems + head_off;
-        const uint16_t* vp_next = P.vpool + (size_t)phys_next * page_elems + head_off;
+        const uint8_t* kp_next = P.kpool + (size_t)phys_next * k_page + k_head_off;
+        const uint8_t* vp_next = P.vpool + (size_t)phys_next * v_page + v_head_off;
 
         // ---- scores: partial dots -> LDS transpose -> one (row, head) per lane ------
         float sval[NB];
@@ -279,17 +356,23 @@ __global__ __launch_bounds__(kBlock, (HG * CH > 4 && CH == 1) ? 2 : 3) void deco
                 // element-major order: HG independent accumulators between dependent FMAs
                 float s[HG];
                 {
-                    const float k0 = widen(kk[i][0]);
+                    const float k0 = kk.elem(i, 0);
 #pragma unroll
                     for (int h = 0; h < HG; ++h) s[h] = k0 * q[h][0];
                 }
 #pragma unroll
                 for (int j = 1; j < 8; ++j) {
-                    const float kj = widen(kk[i][j]);
+                    const float kj = kk.elem(i, j);
 #pragma unroll
                     for (int h = 0; h < HG; ++h) s[h] = fmaf(kj, q[h][j], s[h]);
                 }
-                kk[i] = load_row8(kp_next, i * 64 + lane);
+                if (RowBuf<KENC>::kScaled) {
+                    // the lane's 8 elements lie inside one 32-element block: one scale per row
+                    const float ks = kk.scale(i);
+#pragma unroll
+                    for (int h = 0; h < HG; ++h) s[h] *= ks;
+                }
+                kk.load(kp_next, i, lane);
 #pragma unroll
                 for (int hq = 0; hq < HQ; ++hq) {
                     const int slot = (HG == 8) ? (ip * 2 + hq) : i;
@@ -357,12 +440,8 @@ __global__ __launch_bounds__(kBlock, (HG * CH > 4 && CH == 1) ? 2 : 3) void deco
         if (pg == n_pages - 1) {
             // Rows past `pos` may hold anything (even NaN): make them exact zeros.
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                if (pg * kPage + 2 * i + hw > pos) {
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) vv[i][j] = (_Float16)0.0f;
-                }
-            }
+            for (int i = 0; i < 8; ++i)
+                if (pg * kPage + 2 * i + hw > pos) vv.zero(i);
         }
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -374,13 +453,19 @@ __global__ __launch_bounds__(kBlock, (HG * CH > 4 && CH == 1) ? 2 : 3) void deco
                 pr[hq * 4 + 0] = t.x, pr[hq * 4 + 1] = t.y, pr[hq * 4 + 2] = t.z,
                             pr[hq * 4 + 3] = t.w;
             }
+            if (RowBuf<VENC>::kScaled) {
+                // dequantisation folded into the probabilities: p * scale, then * code
+                const float vs = vv.scale(i);
+#pragma unroll
+                for (int h = 0; h < HG; ++h) pr[h] *= vs;
+            }
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                const float vj = widen(vv[i][j]);
+                const float vj = vv.elem(i, j);
 #pragma unroll
                 for (int h = 0; h < HG; ++h) o[h][j] = fmaf(vj, pr[h], o[h][j]);
             }
-            vv[i] = load_row8(vp_next, i * 64 + lane);
+            vv.load(vp_next, i, lane);
         }
         wave_lds_sync();
 
@@ -415,25 +500,22 @@ __global__ __launch_bounds__(kBlock, (HG * CH > 4 && CH == 1) ? 2 : 3) void deco
     // ---- merge the four waves; thread = head-dim element ----------------------------
     const int d = threadIdx.x;
 #pragma unroll
-    for (int hw_ = 0; hw_ < HW; ++hw_) {
-        const int c = hw_ / HG;  // chunk that carried this head
-        const int h = hw_ % HG;
-        float mx = wave_m[c][h];
+    for (int h = 0; h < HG; ++h) {
+        float mx = wave_m[0][h];
 #pragma unroll
-        for (int s = 1; s < kStreams; ++s) mx = fmaxf(mx, wave_m[s * CH + c][h]);
+        for (int w = 1; w < kWaves; ++w) mx = fmaxf(mx, wave_m[w][h]);
         float acc = 0.0f, lsum = 0.0f;
 #pragma unroll
-        for (int s = 0; s < kStreams; ++s) {
-            const int w = s * CH + c;
+        for (int w = 0; w < kWaves; ++w) {
             const float mw = wave_m[w][h];
             const float f = mw == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(mw - mx);
             acc = fmaf(f, reinterpret_cast<const float*>(&xs[w][0])[h * kHd + d], acc);
             lsum = fmaf(f, wave_l[w][h], lsum);
         }
-        P.part_o[((size_t)wg * HW + hw_) * kHd + d] = acc;
+        P.part_o[((size_t)wg * HG + h) * kHd + d] = acc;
         if (d == 0) {
-            P.part_ml[((size_t)wg * HW + hw_) * 2 + 0] = mx;
-            P.part_ml[((size_t)wg * HW + hw_) * 2 + 1] = lsum;
+            P.part_ml[((size_t)wg * HG + h) * 2 + 0] = mx;
+            P.part_ml[((size_t)wg * HG + h) * 2 + 1] = lsum;
         }
     }
 }
@@ -542,8 +624,6 @@ __global__ __launch_bounds__(kHd * kMergeGroups) void decode_attn_merge_kernel(c
 
 // Heads one work-group carries for a given q-heads-per-kv-head group.
 int32_t attn_heads_per_wave(int32_t group) { return group % 8 == 0 ? 8 : 4; }
-// Whole groups of 8 heads are carried as two in-work-group chunks of 4 (see the kernel).
-constexpr bool kSplitEightInWorkgroup = false;
 
 int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b) {
     const int32_t n_kv = p->g.n_kv;
@@ -556,8 +636,7 @@ int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b) {
     // All work-groups should be resident at once (one generation): a handful of left-over
     // work-groups would run alone after the rest and double the kernel's time.  `resident`
     // follows from the register budget of the kernel variant that will run.
-    const bool split8 = hg == 8 && kSplitEightInWorkgroup;
-    const int64_t resident = split8 ? 3 : 2;
+    const int64_t resident = hg == 8 ? 2 : 3;
     int64_t target = (int64_t)(p->n_cu > 0 ? p->n_cu : 256) * resident;
     if (target > p->max_wgs) target = p->max_wgs;
     int64_t pps = (total_pages * per_page + target - 1) / target;
@@ -589,8 +668,8 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
     const int32_t hg = attn_heads_per_wave(group);
     AttnKernelParams kp;
     kp.b = b;
-    kp.kpool = reinterpret_cast<const uint16_t*>(p->k_layer[(size_t)layer]);
-    kp.vpool = reinterpret_cast<const uint16_t*>(p->v_layer[(size_t)layer]);
+    kp.kpool = p->k_layer[(size_t)layer];
+    kp.vpool = p->v_layer[(size_t)layer];
     kp.tables = p->table_dev;
     kp.q = a.q;
     kp.part_o = p->part_o;
@@ -606,12 +685,16 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
     const int32_t grid = (n_units + 7) / 8 * 8 * kp.n_hc;
     {
         StageScope timed(p, BKV_STAGE_ATTN_SPLIT, stream);
-        if (hg == 8 && kSplitEightInWorkgroup)
-            decode_attn_f16_kernel<4, 2><<<grid, kBlock, 0, stream>>>(kp);
-        else if (hg == 8)
-            decode_attn_f16_kernel<8, 1><<<grid, kBlock, 0, stream>>>(kp);
-        else
-            decode_attn_f16_kernel<4, 1><<<grid, kBlock, 0, stream>>>(kp);
+        const int layout = p->g.layout;
+#define BKV_LAUNCH(HGV, KE, VE) decode_attn_kernel<HGV, KE, VE><<<grid, kBlock, 0, stream>>>(kp)
+        if (layout == BKV_LAYOUT_F16) {
+            if (hg == 8) BKV_LAUNCH(8, kRowF16, kRowF16); else BKV_LAUNCH(4, kRowF16, kRowF16);
+        } else if (layout == BKV_LAYOUT_Q8V) {
+            if (hg == 8) BKV_LAUNCH(8, kRowF16, kRowQ8); else BKV_LAUNCH(4, kRowF16, kRowQ8);
+        } else {
+            if (hg == 8) BKV_LAUNCH(8, kRowI8H, kRowI8H); else BKV_LAUNCH(4, kRowI8H, kRowI8H);
+        }
+#undef BKV_LAUNCH
     }
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) return err;
