@@ -263,46 +263,6 @@ __global__ __launch_bounds__(kBlock, HG == 8 ? 2 : 3) void decode_attn_kernel(co
     const int hw = lane >> 5;   // row parity this lane loads
     const int dl = lane & 31;   // 8-element slice of the head dim
 
-    // ---- q slice (dead heads of a padded chunk stay zero) ---------------------------
-    float q[HG][8];
-#pragma unroll
-    for (int h = 0; h < HG; ++h) {
-        const int hl = hc * HG + h;
-        if (hl < P.group) {
-            const float* qp =
-                P.q + ((size_t)e * P.n_q + (size_t)kvh * P.group + hl) * kHd + dl * 8;
-            const float4 a = *reinterpret_cast<const float4*>(qp);
-            const float4 c = *reinterpret_cast<const float4*>(qp + 4);
-            q[h][0] = a.x, q[h][1] = a.y, q[h][2] = a.z, q[h][3] = a.w;
-            q[h][4] = c.x, q[h][5] = c.y, q[h][6] = c.z, q[h][7] = c.w;
-        } else {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) q[h][j] = 0.0f;
-        }
-    }
-
-    // q must have arrived before the first K/V rows are requested: a wait for q placed
-    // inside the page loop would also drain the row loads that are kept in flight there.
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), other counters untouched
-    __builtin_amdgcn_sched_barrier(0);
-
-    float o[HG][8];
-#pragma unroll
-    for (int h = 0; h < HG; ++h)
-#pragma unroll
-        for (int j = 0; j < 8; ++j) o[h][j] = 0.0f;
-
-    // ---- this lane's role when it finishes score sums ------------------------------
-    // part: which quarter of the 32 slices it adds; slot/rhw: which float4 slot and row
-    // parity; after the quad combine it keeps component `part`, i.e. one head.
-    const int part = lane & 3;
-    const int rslot = ((lane >> 4) << 1) | ((lane >> 2) & 1);
-    const int rhw = (lane >> 3) & 1;
-    const int my_head = (HG == 8) ? (lane & 7) : (lane & 3);
-    const int rbase = rslot * 64 + rhw * 32 + part * 8;
-    float m_run = -INFINITY;  // running max of this lane's head (base-2 logits)
-    float l_run = 0.0f;       // this lane's share of the denominator
-
     constexpr size_t kKHead = (size_t)kPage * row_bytes_of(KENC);  // bytes of one kv head's rows
     constexpr size_t kVHead = (size_t)kPage * row_bytes_of(VENC);
     const size_t k_page = (size_t)P.n_kv * kKHead, v_page = (size_t)P.n_kv * kVHead;
@@ -324,20 +284,66 @@ __global__ __launch_bounds__(kBlock, HG == 8 ? 2 : 3) void decode_attn_kernel(co
         for (int i = 0; i < 8; ++i) vv.load(vp, i, lane);
     }
 
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- q slice (dead heads of a padded chunk stay zero) ---------------------------
+    float q[HG][8];
+#pragma unroll
+    for (int h = 0; h < HG; ++h) {
+        const int hl = hc * HG + h;
+        if (hl < P.group) {
+            const float* qp =
+                P.q + ((size_t)e * P.n_q + (size_t)kvh * P.group + hl) * kHd + dl * 8;
+            const float4 a = *reinterpret_cast<const float4*>(qp);
+            const float4 c = *reinterpret_cast<const float4*>(qp + 4);
+            q[h][0] = a.x, q[h][1] = a.y, q[h][2] = a.z, q[h][3] = a.w;
+            q[h][4] = c.x, q[h][5] = c.y, q[h][6] = c.z, q[h][7] = c.w;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) q[h][j] = 0.0f;
+        }
+    }
+
+    // The first page's rows (requested above) and q travel together; both must have arrived
+    // before the page loop starts: a wait for q placed inside the loop would also drain the
+    // row loads that are kept in flight there on every iteration.
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), other counters untouched
+    __builtin_amdgcn_sched_barrier(0);
+
+    float o[HG][8];
+#pragma unroll
+    for (int h = 0; h < HG; ++h)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o[h][j] = 0.0f;
+
+    // ---- this lane's role when it finishes score sums ------------------------------
+    // part: which quarter of the 32 slices it adds; slot/rhw: which float4 slot and row
+    // parity; after the quad combine it keeps component `part`, i.e. one head.
+    const int part = lane & 3;
+    const int rslot = ((lane >> 4) << 1) | ((lane >> 2) & 1);
+    const int rhw = (lane >> 3) & 1;
+    const int my_head = (HG == 8) ? (lane & 7) : (lane & 3);
+    const int rbase = rslot * 64 + rhw * 32 + part * 8;
+    float m_run = -INFINITY;  // running max of this lane's head (base-2 logits)
+    float l_run = 0.0f;       // this lane's share of the denominator
+
     // Two waves share a SIMD (one from each resident work-group) and the issue arbiter
-    // always prefers the older one, which then finishes a third earlier and leaves the
-    // younger wave alone, with nothing to overlap its latencies, for the rest of the
-    // kernel.  Swapping the two waves' priority on every page shares the SIMD evenly.
+    // prefers the older one whenever priorities are equal; it then finishes a third earlier
+    // and leaves the younger wave alone, with nothing to overlap its latencies, for the rest
+    // of the kernel (measured: 47 vs 64 us loop times on every CU).  The younger wave (odd
+    // wave slot) therefore raises its priority on two of every three pages; the older one
+    // never does.  Measured loop times with this duty cycle: 52.8 vs 51.3 us.
     unsigned slot;
     asm("s_getreg_b32 %0, hwreg(HW_REG_HW_ID, 0, 4)" : "=s"(slot));  // wave slot within the SIMD
-    unsigned turn = slot;
+    const bool younger = (slot & 1u) != 0;
+    unsigned turn = 0;
 
     while (pg < pg1) {
-        if (turn & 1)
+        if (younger && turn != 0)
             __builtin_amdgcn_s_setprio(2);
         else
             __builtin_amdgcn_s_setprio(0);
-        ++turn;
+        turn = turn == 2 ? 0 : turn + 1;
         // The next page is fetched unconditionally (the last iteration re-reads its own
         // page): one straight-line load sequence lets the compiler count outstanding loads
         // exactly instead of draining them at a control-flow join.
@@ -530,16 +536,19 @@ struct MergeParams {
     int32_t n_kv, n_q, group, hg;
 };
 
-constexpr int kMergeGroups = 4;  // split ranges summed side by side, then folded in LDS
+constexpr int kMergeGroups = 4;   // split ranges summed side by side, then folded in LDS
+constexpr int kMergeInFlight = 8; // partial rows a thread requests before it needs the factors
 
-// One work-group per (entry, q head): kMergeGroups x 256 threads.  Thread (g, d) adds the
-// partial outputs of splits g, g + 4, ... for head-dim element d with four loads in flight;
-// the per-split (m, l) pairs are staged in LDS once.
+// One work-group per (entry, q head): kMergeGroups x 256 threads.  Thread (g, d) owns head-dim
+// element d of splits g, g + 4, ...; it requests its first 8 partial values straight away, and
+// only then are the per-split (m, l) pairs staged in LDS and the maximum agreed, so the two
+// round trips to memory overlap.
 __global__ __launch_bounds__(kHd * kMergeGroups) void decode_attn_merge_kernel(const MergeParams P) {
     constexpr int kMaxStaged = 1024;
     __shared__ float sm[kMaxStaged];
     __shared__ float sl[kMaxStaged];
     __shared__ float red[kMergeGroups][kHd];
+    __shared__ float red_l[kMergeGroups];
     const int e = blockIdx.x / P.n_q;
     const int h = blockIdx.x % P.n_q;
     const int kvh = h / P.group;
@@ -550,59 +559,52 @@ __global__ __launch_bounds__(kHd * kMergeGroups) void decode_attn_merge_kernel(c
     const int wg0 = P.b.wg_base[e] + hc * splits * P.n_kv + kvh;
     const int d = threadIdx.x & (kHd - 1);
     const int g = threadIdx.x >> 8;
-    const int staged = min(splits, kMaxStaged);
-    for (int s = threadIdx.x; s < staged; s += kHd * kMergeGroups) {
-        const size_t wg = (size_t)(wg0 + s * P.n_kv);
-        sm[s] = P.part_ml[(wg * P.hg + hh) * 2];
-        sl[s] = P.part_ml[(wg * P.hg + hh) * 2 + 1];
-    }
-    __syncthreads();
-    float mx = -INFINITY;
-    for (int s = 0; s < splits; ++s) {
-        const float ms = s < kMaxStaged ? sm[s]
-                                        : P.part_ml[((size_t)(wg0 + s * P.n_kv) * P.hg + hh) * 2];
-        mx = fmaxf(mx, ms);
-    }
-    float acc = 0.0f, lsum = 0.0f;
     const size_t ostride = (size_t)P.n_kv * P.hg * kHd;  // floats between consecutive splits
     const float* po = P.part_o + ((size_t)wg0 * P.hg + hh) * kHd + d;
-    int s = g;
-    for (; s + 3 * kMergeGroups < splits; s += 4 * kMergeGroups) {
-        float v[4], f[4];
+    const float* pml = P.part_ml + ((size_t)wg0 * P.hg + hh) * 2;
+    const size_t mlstride = (size_t)P.n_kv * P.hg * 2;
+
+    float v[kMergeInFlight];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) v[u] = po[(size_t)(s + u * kMergeGroups) * ostride];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int su = s + u * kMergeGroups;
-            const float ms = su < kMaxStaged
-                                 ? sm[su]
-                                 : P.part_ml[((size_t)(wg0 + su * P.n_kv) * P.hg + hh) * 2];
-            const float ls = su < kMaxStaged
-                                 ? sl[su]
-                                 : P.part_ml[((size_t)(wg0 + su * P.n_kv) * P.hg + hh) * 2 + 1];
-            f[u] = ms == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(ms - mx);
-            lsum = fmaf(f[u], ls, lsum);
-        }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) acc = fmaf(f[u], v[u], acc);
+    for (int u = 0; u < kMergeInFlight; ++u) {
+        const int s = g + u * kMergeGroups;
+        v[u] = s < splits ? po[(size_t)s * ostride] : 0.0f;
     }
-    for (; s < splits; s += kMergeGroups) {
-        const float ms =
-            s < kMaxStaged ? sm[s] : P.part_ml[((size_t)(wg0 + s * P.n_kv) * P.hg + hh) * 2];
-        const float ls =
-            s < kMaxStaged ? sl[s] : P.part_ml[((size_t)(wg0 + s * P.n_kv) * P.hg + hh) * 2 + 1];
+    const int staged = min(splits, kMaxStaged);
+    for (int s = threadIdx.x; s < staged; s += kHd * kMergeGroups) {
+        sm[s] = pml[(size_t)s * mlstride];
+        sl[s] = pml[(size_t)s * mlstride + 1];
+    }
+    __syncthreads();
+    const auto m_of = [&](int s) { return s < kMaxStaged ? sm[s] : pml[(size_t)s * mlstride]; };
+    const auto l_of = [&](int s) { return s < kMaxStaged ? sl[s] : pml[(size_t)s * mlstride + 1]; };
+    float mx = -INFINITY;
+    for (int s = 0; s < splits; ++s) mx = fmaxf(mx, m_of(s));
+    float acc = 0.0f, lsum = 0.0f;
+#pragma unroll
+    for (int u = 0; u < kMergeInFlight; ++u) {
+        const int s = g + u * kMergeGroups;
+        if (s < splits) {
+            const float ms = m_of(s);
+            const float f = ms == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(ms - mx);
+            acc = fmaf(f, v[u], acc);
+            lsum = fmaf(f, l_of(s), lsum);
+        }
+    }
+    for (int s = g + kMergeInFlight * kMergeGroups; s < splits; s += kMergeGroups) {
+        const float ms = m_of(s);
         const float f = ms == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(ms - mx);
         acc = fmaf(f, po[(size_t)s * ostride], acc);
-        lsum = fmaf(f, ls, lsum);
+        lsum = fmaf(f, l_of(s), lsum);
     }
     red[g][d] = acc;
-    if (d == 0) sm[g] = lsum;  // sm is free again: every thread has its own copy of mx
+    if (d == 0) red_l[g] = lsum;
     __syncthreads();
     if (g != 0) return;
 #pragma unroll
     for (int k = 1; k < kMergeGroups; ++k) {
         acc += red[k][d];
-        lsum += sm[k];
+        lsum += red_l[k];
     }
     float r = lsum > 0.0f ? acc / lsum : 0.0f;
     if (P.gate) {
