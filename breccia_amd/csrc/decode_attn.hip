@@ -549,6 +549,7 @@ __global__ __launch_bounds__(kHd * kMergeGroups) void decode_attn_merge_kernel(c
     __shared__ float sl[kMaxStaged];
     __shared__ float red[kMergeGroups][kHd];
     __shared__ float red_l[kMergeGroups];
+    __shared__ float wave_max[kHd * kMergeGroups / 64];
     const int e = blockIdx.x / P.n_q;
     const int h = blockIdx.x % P.n_q;
     const int kvh = h / P.group;
@@ -570,16 +571,28 @@ __global__ __launch_bounds__(kHd * kMergeGroups) void decode_attn_merge_kernel(c
         const int s = g + u * kMergeGroups;
         v[u] = s < splits ? po[(size_t)s * ostride] : 0.0f;
     }
-    const int staged = min(splits, kMaxStaged);
-    for (int s = threadIdx.x; s < staged; s += kHd * kMergeGroups) {
-        sm[s] = pml[(size_t)s * mlstride];
-        sl[s] = pml[(size_t)s * mlstride + 1];
+    // stage (m, l) and agree on the maximum: per-thread max over its splits, wave reduction,
+    // then one LDS slot per wave (a serial scan over the splits would cost a dependent LDS
+    // round trip per split)
+    constexpr int kThreads = kHd * kMergeGroups;
+    float my_m = -INFINITY;
+    for (int s = threadIdx.x; s < splits; s += kThreads) {
+        const float ms = pml[(size_t)s * mlstride];
+        if (s < kMaxStaged) {
+            sm[s] = ms;
+            sl[s] = pml[(size_t)s * mlstride + 1];
+        }
+        my_m = fmaxf(my_m, ms);
     }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) my_m = fmaxf(my_m, __shfl_xor(my_m, off, 64));
+    if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = my_m;
     __syncthreads();
     const auto m_of = [&](int s) { return s < kMaxStaged ? sm[s] : pml[(size_t)s * mlstride]; };
     const auto l_of = [&](int s) { return s < kMaxStaged ? sl[s] : pml[(size_t)s * mlstride + 1]; };
-    float mx = -INFINITY;
-    for (int s = 0; s < splits; ++s) mx = fmaxf(mx, m_of(s));
+    float mx = wave_max[0];
+#pragma unroll
+    for (int w = 1; w < kThreads / 64; ++w) mx = fmaxf(mx, wave_max[w]);
     float acc = 0.0f, lsum = 0.0f;
 #pragma unroll
     for (int u = 0; u < kMergeInFlight; ++u) {
