@@ -604,11 +604,24 @@ __global__ __launch_bounds__(kHd * kMergeGroups) void decode_attn_merge_kernel(c
             lsum = fmaf(f, l_of(s), lsum);
         }
     }
-    for (int s = g + kMergeInFlight * kMergeGroups; s < splits; s += kMergeGroups) {
-        const float ms = m_of(s);
-        const float f = ms == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(ms - mx);
-        acc = fmaf(f, po[(size_t)s * ostride], acc);
-        lsum = fmaf(f, l_of(s), lsum);
+    // further rounds of kMergeInFlight requests for long split lists
+    for (int s0 = g + kMergeInFlight * kMergeGroups; s0 < splits;
+         s0 += kMergeInFlight * kMergeGroups) {
+#pragma unroll
+        for (int u = 0; u < kMergeInFlight; ++u) {
+            const int s = s0 + u * kMergeGroups;
+            v[u] = s < splits ? po[(size_t)s * ostride] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < kMergeInFlight; ++u) {
+            const int s = s0 + u * kMergeGroups;
+            if (s < splits) {
+                const float ms = m_of(s);
+                const float f = ms == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(ms - mx);
+                acc = fmaf(f, v[u], acc);
+                lsum = fmaf(f, l_of(s), lsum);
+            }
+        }
     }
     red[g][d] = acc;
     if (d == 0) red_l[g] = lsum;
