@@ -30,18 +30,27 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0
 N_Q, N_KV, HD, PAGE = 16, 2, 256, 16
 ROW_BYTES = N_KV * HD * 2 * 2          # K + V f16 bytes per cell per layer = 2048
+# bytes per cell per layer of the quantised pools: f16 K + q8_0 V (36 B per 32 values), and
+# int8 K and V with one f16 scale per 32 values (34 B per 32 values)
+ROW_BYTES_Q8V = N_KV * (HD * 2 + HD // 32 * 36)   # 1600
+ROW_BYTES_I8H = N_KV * 2 * (HD // 32 * 34)        # 1088
+# HBM traffic of one launch of the split-K kernel on the default seeded workload, from
+# rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this file, each scaled by what the same counter
+# reads for the plain copy probe (profiles/decode_attn_batch8_hbm_traffic.md)
+MEASURED_TRAFFIC = {"seed": 20250003, "fetch_bytes": 336.6e6, "write_bytes": 4.16e6}
 APPEND_BYTES_PER_TOKEN = N_KV * HD * (4 + 2) * 2  # f32 in + f16 out, K and V = 6144
 
 
-def attn_algorithmic_bytes(ctx_after: list[int]) -> int:
+def attn_algorithmic_bytes(ctx_after: list[int], row_bytes: int = ROW_BYTES) -> int:
     """K+V rows read once for all heads of a group + block table + q + out."""
     total = 0
     for c in ctx_after:
-        total += c * ROW_BYTES + ((c + PAGE - 1) // PAGE) * 4 + 2 * N_Q * HD * 4
+        total += c * row_bytes + ((c + PAGE - 1) // PAGE) * 4 + 2 * N_Q * HD * 4
     return total
 
 
-def build_batched(pool_mod, rng, n_seqs: int, lo: int, hi: int, n_layers: int, occupancy: float):
+def build_batched(pool_mod, rng, n_seqs: int, lo: int, hi: int, n_layers: int, occupancy: float,
+                  layout: int = 0):
     from breccia_amd.kv import Pool
 
     ctx = []
@@ -53,7 +62,7 @@ def build_batched(pool_mod, rng, n_seqs: int, lo: int, hi: int, n_layers: int, o
     live_pages = sum((c + PAGE) // PAGE + 1 for c in ctx)
     n_pages = int(np.ceil(live_pages / occupancy))
     pool = Pool(n_layers=n_layers, n_pages=n_pages, n_kv_head=N_KV, head_dim=HD, max_seqs=n_seqs + 1,
-                max_pages_per_seq=max(ctx) // PAGE + 8)
+                max_pages_per_seq=max(ctx) // PAGE + 8, layout=layout)
     pool.set_free_order(rng.permutation(n_pages).astype(np.int32))
     seqs = [pool.seq_create() for _ in ctx]
     # deal the shuffled pages round-robin: one page per sequence per turn
@@ -184,8 +193,10 @@ def main() -> int:
     split_us = ms_split / max(n_split, 1) * 1e3
     achieved = attn_bytes / (split_us * 1e-6) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-                "kernel": "decode_attn_f16_kernel<8>", "avg_us": round(split_us, 2),
+                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                "traffic": MEASURED_TRAFFIC["fetch_bytes"] + MEASURED_TRAFFIC["write_bytes"],
+                "kernel": "decode_attn_kernel<8, 0, 0> (f16 K, f16 V, 8 q heads per kv head)",
+                "avg_us": round(split_us, 2),
                 "launches": n_split, "algorithmic_bytes": attn_bytes}
 
     # ---- sanity: one sequence of the last step against the oracle ----------------------
@@ -237,6 +248,7 @@ def main() -> int:
 
     if not args.no_extra:
         extra.update(bench_batch1(stream))
+        extra.update(bench_quantised(stream))
         extra.update(bench_moves(stream))
 
     line = {"metric": "paged decode-attn step throughput, batch 8 mixed 1k-32k (append + attention, "
@@ -302,6 +314,55 @@ def bench_batch1(stream) -> dict:
     for b in bufs:
         b.free()
     return out
+
+
+def bench_quantised(stream) -> dict:
+    """Decode attention over the quantised pools: the headline batch on f16 K + q8_0 V, and
+    BASELINE configs[4] (16 sequences, ctx U{8192..131072}, int8 K/V with f16 block scales)."""
+    from breccia_amd import lib as L
+    from breccia_amd.kv import DeviceBuffer
+
+    res = {}
+    cases = [("attn_q8v_batch8", L.LAYOUT_Q8V, ROW_BYTES_Q8V, 8, 1024, 32768, 4, 20250003,
+              "headline batch on f16 K + q8_0 V"),
+             ("attn_int8_batch16", L.LAYOUT_I8H, ROW_BYTES_I8H, 16, 8192, 131072, 2, 20250005,
+              "BASELINE configs[4]: 16 sequences, ctx U{8k..128k}, int8 K/V + f16 scales")]
+    for name, layout, row_bytes, n_seqs, lo, hi, n_layers, seed, what in cases:
+        rng = np.random.Generator(np.random.PCG64(seed))
+        pool, seqs, ctx = build_batched(None, rng, n_seqs, lo, hi, n_layers, 0.6, layout)
+        # contents: one resident block of N(0,1) rows appended at every chunk of every sequence
+        chunk = 8192
+        kd = DeviceBuffer.from_numpy(rng.standard_normal((chunk, N_KV, HD), dtype=np.float32))
+        vd = DeviceBuffer.from_numpy(rng.standard_normal((chunk, N_KV, HD), dtype=np.float32))
+        for layer in range(n_layers):
+            for s, c in zip(seqs, ctx):
+                for at in range(0, c, chunk):
+                    pool.append(layer, [s], [at], [min(chunk, c - at)], kd, vd, stream)
+            stream.sync()
+        kd.free()
+        vd.free()
+        _, bufs = make_step_buffers(n_seqs, rng, slots=16)
+        steps, warm = 40, 8
+        wall_ms, _ = time_steps(pool, seqs, ctx, n_layers, steps, warm, bufs, stream)
+        pool.timing_reset()
+        pool.timing_enable(True)
+        run_steps(pool, seqs, ctx, n_layers, steps, *bufs, stream, first_step=steps + warm)
+        stream.sync()
+        pool.timing_enable(False)
+        n_split, ms_split = pool.timing_read(L.STAGE_ATTN_SPLIT)
+        n_merge, ms_merge = pool.timing_read(L.STAGE_ATTN_MERGE)
+        b = attn_algorithmic_bytes([c + 1 + (steps + warm) // n_layers for c in ctx], row_bytes)
+        split_us = ms_split / max(n_split, 1) * 1e3
+        res[name] = {"workload": what, "cells": sum(ctx), "algorithmic_bytes": b,
+                     "us_per_layer": round(wall_ms / steps * 1e3, 2),
+                     "attn_split_us": round(split_us, 2),
+                     "attn_merge_us": round(ms_merge / max(n_merge, 1) * 1e3, 2),
+                     "split_GBps": round(b / split_us / 1e3, 1),
+                     "split_frac_of_hbm_peak": round(b / split_us / 1e3 / HBM_PEAK_GBPS, 4)}
+        pool.destroy()
+        for x in bufs:
+            x.free()
+    return res
 
 
 def bench_moves(stream) -> dict:
