@@ -406,6 +406,11 @@ def bench_moves(stream) -> dict:
                           "frac_of_hbm_peak": round(b / ms / 1e6 / HBM_PEAK_GBPS, 4)}
     ms = timed(lambda: pool.append(0, seqs, [7] * 4, [1] * 4, kd, vd, stream), 200)
     res["append_decode_us"] = round(ms * 1e3, 2)
+    # the same rows handed over as raw f16 (bkv_append_f16): 2048 B in + 2048 B out per token
+    ms = timed(lambda: pool.append(0, seqs, [0] * 4, [T] * 4, kd, vd, stream, f16_rows=True), 20)
+    b = 4 * T * N_KV * HD * (2 + 2) * 2
+    res["append_bulk_f16_rows"] = {"tokens": 4 * T, "ms": round(ms, 4), "GBps": round(b / ms / 1e6, 1),
+                                   "frac_of_hbm_peak": round(b / ms / 1e6 / HBM_PEAK_GBPS, 4)}
     kd.free()
     vd.free()
 

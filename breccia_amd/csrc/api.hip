@@ -439,9 +439,9 @@ bkv_status bkv_pool_check(const bkv_pool* p) {
 }
 
 // ---- append ------------------------------------------------------------------------
-bkv_status bkv_append(bkv_pool* p, int32_t layer, int32_t n_seqs, const int32_t* seqs,
-                      const int64_t* pos0, const int32_t* n_tokens, const float* k_dev,
-                      const float* v_dev, void* stream) {
+static bkv_status append_rows(bkv_pool* p, int32_t layer, int32_t n_seqs, const int32_t* seqs,
+                              const int64_t* pos0, const int32_t* n_tokens, const void* k_dev,
+                              const void* v_dev, bool src_is_f16, void* stream) {
     if (!p) return fail(BKV_ERR_INVALID, "append: NULL pool");
     if (layer < 0 || layer >= p->g.n_layers)
         return fail(BKV_ERR_RANGE, sfmt("append: layer %lld is outside 0..%lld", layer,
@@ -494,10 +494,22 @@ bkv_status bkv_append(bkv_pool* p, int32_t layer, int32_t n_seqs, const int32_t*
     if (st != BKV_OK) return st;
     {
         StageScope timed(p, BKV_STAGE_APPEND, S(stream));
-        BKV_HIP(launch_append(p, layer, b, max_tok, k_dev, v_dev, S(stream)));
+        BKV_HIP(launch_append(p, layer, b, max_tok, k_dev, v_dev, src_is_f16, S(stream)));
     }
     if (p->timer.open.size() > 8192) return timer_collect(p);
     return BKV_OK;
+}
+
+bkv_status bkv_append(bkv_pool* p, int32_t layer, int32_t n_seqs, const int32_t* seqs,
+                      const int64_t* pos0, const int32_t* n_tokens, const float* k_dev,
+                      const float* v_dev, void* stream) {
+    return append_rows(p, layer, n_seqs, seqs, pos0, n_tokens, k_dev, v_dev, false, stream);
+}
+
+bkv_status bkv_append_f16(bkv_pool* p, int32_t layer, int32_t n_seqs, const int32_t* seqs,
+                          const int64_t* pos0, const int32_t* n_tokens, const uint16_t* k_dev,
+                          const uint16_t* v_dev, void* stream) {
+    return append_rows(p, layer, n_seqs, seqs, pos0, n_tokens, k_dev, v_dev, true, stream);
 }
 
 // ---- decode attention ----------------------------------------------------------------

@@ -128,7 +128,7 @@ struct AppendBatch {
     int32_t src0[BKV_MAX_BATCH];     // first source row in k/v
 };
 hipError_t launch_append(const bkv_pool* p, int32_t layer, const AppendBatch& b, int32_t max_tok,
-                         const float* k, const float* v, hipStream_t stream);
+                         const void* k, const void* v, bool src_is_f16, hipStream_t stream);
 
 struct AttnBatch {
     int32_t n;

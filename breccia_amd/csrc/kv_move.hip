@@ -57,15 +57,40 @@ struct MoveGeom {
     int32_t n_kv, hd, page_cells, max_pages_per_seq;
 };
 
+// Eight consecutive source values as f32.  Sources are f32 rows, or raw binary16 rows that
+// are widened under the cache's load rule (so an f16 source appends exactly what the f32
+// row of its widened values would).
+__device__ __forceinline__ void load8(const float* p, float (&x)[8]) {
+    const v4u a = ld_stream(p), b = ld_stream(p + 4);
+    x[0] = __uint_as_float(a.x);
+    x[1] = __uint_as_float(a.y);
+    x[2] = __uint_as_float(a.z);
+    x[3] = __uint_as_float(a.w);
+    x[4] = __uint_as_float(b.x);
+    x[5] = __uint_as_float(b.y);
+    x[6] = __uint_as_float(b.z);
+    x[7] = __uint_as_float(b.w);
+}
+__device__ __forceinline__ void load8(const uint16_t* p, float (&x)[8]) {
+    const v4u a = ld_stream(p);
+    const unsigned w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        x[2 * i] = f16_load(w[i] & 0xffffu);
+        x[2 * i + 1] = f16_load(w[i] >> 16);
+    }
+}
+
 // ---- append, f16 rows ---------------------------------------------------------
 // One lane converts 8 consecutive elements of one (token, kv head) row of K and of V:
 // two 16-byte loads and one 16-byte store per pool.  grid.y = sequence of the call.
+template <typename SrcT>
 __global__ __launch_bounds__(kBlock) void append_f16_kernel(AppendBatch b, MoveGeom g,
                                                             uint16_t* __restrict__ kpool,
                                                             uint16_t* __restrict__ vpool,
                                                             const int32_t* __restrict__ tables,
-                                                            const float* __restrict__ k,
-                                                            const float* __restrict__ v) {
+                                                            const SrcT* __restrict__ k,
+                                                            const SrcT* __restrict__ v) {
     const int s = blockIdx.y;
     const int lanes_per_tok = g.n_kv * g.hd / 8;
     const int64_t unit = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -82,18 +107,18 @@ __global__ __launch_bounds__(kBlock) void append_f16_kernel(AppendBatch b, MoveG
     const size_t dst = row * (size_t)g.hd + d0;
     const size_t src = ((size_t)b.src0[s] + (size_t)t) * (size_t)(g.n_kv * g.hd) + (size_t)r * 8;
 
-    const v4u k0 = ld_stream(k + src), k1 = ld_stream(k + src + 4);
-    const v4u v0 = ld_stream(v + src), v1 = ld_stream(v + src + 4);
-    const auto f = [](unsigned bits) { return __uint_as_float(bits); };
+    float kx[8], vx[8];
+    load8(k + src, kx);
+    load8(v + src, vx);
     v4u ko, vo;
-    ko.x = pack2(f(k0.x), f(k0.y));
-    ko.y = pack2(f(k0.z), f(k0.w));
-    ko.z = pack2(f(k1.x), f(k1.y));
-    ko.w = pack2(f(k1.z), f(k1.w));
-    vo.x = pack2(f(v0.x), f(v0.y));
-    vo.y = pack2(f(v0.z), f(v0.w));
-    vo.z = pack2(f(v1.x), f(v1.y));
-    vo.w = pack2(f(v1.z), f(v1.w));
+    ko.x = pack2(kx[0], kx[1]);
+    ko.y = pack2(kx[2], kx[3]);
+    ko.z = pack2(kx[4], kx[5]);
+    ko.w = pack2(kx[6], kx[7]);
+    vo.x = pack2(vx[0], vx[1]);
+    vo.y = pack2(vx[2], vx[3]);
+    vo.z = pack2(vx[4], vx[5]);
+    vo.w = pack2(vx[6], vx[7]);
     st_stream(kpool + dst, ko);
     st_stream(vpool + dst, vo);
 }
@@ -126,25 +151,26 @@ __device__ __forceinline__ float amax32(const float (&x)[32]) {
     return amax;
 }
 
-__device__ __forceinline__ void load32(const float* p, float (&x)[32]) {
+template <typename SrcT>
+__device__ __forceinline__ void load32(const SrcT* p, float (&x)[32]) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const float4 f = reinterpret_cast<const float4*>(p)[i];
-        x[i * 4 + 0] = f.x;
-        x[i * 4 + 1] = f.y;
-        x[i * 4 + 2] = f.z;
-        x[i * 4 + 3] = f.w;
+    for (int i = 0; i < 4; ++i) {
+        float y[8];
+        load8(p + i * 8, y);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) x[i * 8 + j] = y[j];
     }
 }
 
 // ---- append, reference q8_0-V rows: K f16, V [f32 scale][32 x i8] per 32 values ---
 // One lane per (token, kv head, 32-element block), as the reference shader does.
+template <typename SrcT>
 __global__ __launch_bounds__(kBlock) void append_q8v_kernel(AppendBatch b, MoveGeom g,
                                                             uint16_t* __restrict__ kpool,
                                                             uint32_t* __restrict__ vpool,
                                                             const int32_t* __restrict__ tables,
-                                                            const float* __restrict__ k,
-                                                            const float* __restrict__ v) {
+                                                            const SrcT* __restrict__ k,
+                                                            const SrcT* __restrict__ v) {
     const int s = blockIdx.y;
     const int blocks = g.hd / 32;
     const int lanes_per_tok = g.n_kv * blocks;
@@ -187,7 +213,8 @@ __global__ __launch_bounds__(kBlock) void append_q8v_kernel(AppendBatch b, MoveG
 // ---- append, int8 K and V with f16 scales: row = [hd x i8][hd/32 x f16] -----------
 // The q8_0 rule with the scale stored through the cache's f16 encoding; a scale the
 // f16 rule would flush is raised to 2^-14.  (No reference counterpart.)
-__device__ __forceinline__ void i8h_block(const float* src, uint8_t* row_base, int hd, int blk) {
+template <typename SrcT>
+__device__ __forceinline__ void i8h_block(const SrcT* src, uint8_t* row_base, int hd, int blk) {
     float x[32];
     load32(src, x);
     const float amax = amax32(x);
@@ -219,12 +246,13 @@ __device__ __forceinline__ void i8h_block(const float* src, uint8_t* row_base, i
     *reinterpret_cast<uint16_t*>(row_base + hd + blk * 2) = (uint16_t)hb;
 }
 
+template <typename SrcT>
 __global__ __launch_bounds__(kBlock) void append_i8h_kernel(AppendBatch b, MoveGeom g,
                                                             uint8_t* __restrict__ kpool,
                                                             uint8_t* __restrict__ vpool,
                                                             const int32_t* __restrict__ tables,
-                                                            const float* __restrict__ k,
-                                                            const float* __restrict__ v) {
+                                                            const SrcT* __restrict__ k,
+                                                            const SrcT* __restrict__ v) {
     const int s = blockIdx.y;
     const int blocks = g.hd / 32;
     const int lanes_per_tok = g.n_kv * blocks * 2;  // K and V blocks
@@ -443,8 +471,10 @@ PoolPtrs pool_ptrs(const bkv_pool* p) {
 
 }  // namespace
 
-hipError_t launch_append(const bkv_pool* p, int32_t layer, const AppendBatch& b, int32_t max_tok,
-                         const float* k, const float* v, hipStream_t stream) {
+template <typename SrcT>
+static hipError_t launch_append_from(const bkv_pool* p, int32_t layer, const AppendBatch& b,
+                                     int32_t max_tok, const SrcT* k, const SrcT* v,
+                                     hipStream_t stream) {
     const MoveGeom g = move_geom(p);
     int lanes_per_tok;
     switch (p->g.layout) {
@@ -458,18 +488,25 @@ hipError_t launch_append(const bkv_pool* p, int32_t layer, const AppendBatch& b,
     uint8_t* vp = p->v_layer[(size_t)layer];
     switch (p->g.layout) {
         case BKV_LAYOUT_F16:
-            append_f16_kernel<<<grid, kBlock, 0, stream>>>(b, g, (uint16_t*)kp, (uint16_t*)vp,
-                                                          p->table_dev, k, v);
+            append_f16_kernel<SrcT><<<grid, kBlock, 0, stream>>>(b, g, (uint16_t*)kp, (uint16_t*)vp,
+                                                                p->table_dev, k, v);
             break;
         case BKV_LAYOUT_Q8V:
-            append_q8v_kernel<<<grid, kBlock, 0, stream>>>(b, g, (uint16_t*)kp, (uint32_t*)vp,
-                                                          p->table_dev, k, v);
+            append_q8v_kernel<SrcT><<<grid, kBlock, 0, stream>>>(b, g, (uint16_t*)kp, (uint32_t*)vp,
+                                                                p->table_dev, k, v);
             break;
         default:
-            append_i8h_kernel<<<grid, kBlock, 0, stream>>>(b, g, kp, vp, p->table_dev, k, v);
+            append_i8h_kernel<SrcT><<<grid, kBlock, 0, stream>>>(b, g, kp, vp, p->table_dev, k, v);
             break;
     }
     return hipGetLastError();
+}
+
+hipError_t launch_append(const bkv_pool* p, int32_t layer, const AppendBatch& b, int32_t max_tok,
+                         const void* k, const void* v, bool src_is_f16, hipStream_t stream) {
+    if (src_is_f16)
+        return launch_append_from(p, layer, b, max_tok, (const uint16_t*)k, (const uint16_t*)v, stream);
+    return launch_append_from(p, layer, b, max_tok, (const float*)k, (const float*)v, stream);
 }
 
 hipError_t launch_page_copy(const bkv_pool* p, const bkv_page_pair* pairs_dev, int32_t n_pairs,

@@ -256,13 +256,15 @@ class Pool:
         return int(n.value), float(ms.value)
 
     # -- hot path
-    def append(self, layer: int, seqs, pos0, n_tokens, k_dev, v_dev, stream=None) -> None:
+    def append(self, layer: int, seqs, pos0, n_tokens, k_dev, v_dev, stream=None,
+               f16_rows: bool = False) -> None:
+        """k_dev / v_dev hold f32 rows, or raw binary16 rows when f16_rows is set."""
         seqs, ps = _i32(seqs)
         pos0, pp = _i64(pos0)
         n_tokens, pn = _i32(n_tokens)
         assert seqs.size == pos0.size == n_tokens.size
-        check(lib.bkv_append(self.handle, layer, seqs.size, ps, pp, pn, _ptr(k_dev), _ptr(v_dev),
-                             _sh(stream)))
+        fn = lib.bkv_append_f16 if f16_rows else lib.bkv_append
+        check(fn(self.handle, layer, seqs.size, ps, pp, pn, _ptr(k_dev), _ptr(v_dev), _sh(stream)))
 
     def decode_attn(self, layer: int, seqs, pos, n_q_head: int, q_dev, out_dev, scale: float,
                     gate_dev=None, gate_seq_stride: int = 0, gate_head_stride: int = 0,

@@ -149,6 +149,15 @@ bkv_status bkv_pool_set_free_order(bkv_pool *pool, const int32_t *order, int32_t
 bkv_status bkv_append(bkv_pool *pool, int32_t layer, int32_t n_seqs, const int32_t *seqs,
                       const int64_t *pos0, const int32_t *n_tokens, const float *k_dev,
                       const float *v_dev, void *stream);
+/* The same append from rows that are already binary16 (raw codes, same shape): what a
+ * producer that keeps K/V in f16 hands over, half the bytes read.  The codes are widened
+ * under the cache's load rule (shaders/f16_storage.glsl:58-69: exponent field 0 reads as a
+ * signed zero) and then take the path of bkv_append, so the pool holds exactly what
+ * bkv_append of the widened rows would have stored (f16 pools: the codes themselves, with
+ * subnormals flushed to zero and NaN stored as infinity). */
+bkv_status bkv_append_f16(bkv_pool *pool, int32_t layer, int32_t n_seqs, const int32_t *seqs,
+                          const int64_t *pos0, const int32_t *n_tokens, const uint16_t *k_dev,
+                          const uint16_t *v_dev, void *stream);
 
 /* bkv_decode_attn replaces Qsa::attend + Qsa::apply for decode shapes with the dense
  * selection (qsa/mod.rs:1382-1462, :1466-1522; shaders qsa_attn_scores_small,

@@ -36,18 +36,21 @@ class Twin:
     def __exit__(self, *exc):
         self.close()
 
-    def append(self, layer, seqs, pos0, k_list, v_list, stream=None):
-        """k_list[i], v_list[i]: float32 [T_i, n_kv, hd].  Appends on the device (one call) and
-        in the oracle image."""
+    def append(self, layer, seqs, pos0, k_list, v_list, stream=None, f16_rows=False):
+        """k_list[i], v_list[i]: float32 [T_i, n_kv, hd] -- or raw binary16 codes (uint16) of the
+        same shape when f16_rows is set, which go through bkv_append_f16 on the device and,
+        widened under the cache's load rule, through the same oracle append.  Appends on the
+        device (one call) and in the oracle image."""
+        dt = np.uint16 if f16_rows else np.float32
         n_tok = [int(np.asarray(k).reshape(-1, self.g.n_kv, self.g.head_dim).shape[0]) for k in k_list]
         if sum(n_tok):
-            kcat = np.concatenate([np.asarray(k, dtype=np.float32).reshape(-1) for k in k_list])
-            vcat = np.concatenate([np.asarray(v, dtype=np.float32).reshape(-1) for v in v_list])
+            kcat = np.concatenate([np.asarray(k, dtype=dt).reshape(-1) for k in k_list])
+            vcat = np.concatenate([np.asarray(v, dtype=dt).reshape(-1) for v in v_list])
         else:
-            kcat = vcat = np.zeros(4, dtype=np.float32)
+            kcat = vcat = np.zeros(8, dtype=dt)
         kd, vd = DeviceBuffer.from_numpy(kcat), DeviceBuffer.from_numpy(vcat)
         try:
-            self.pool.append(layer, seqs, pos0, n_tok, kd, vd, stream)
+            self.pool.append(layer, seqs, pos0, n_tok, kd, vd, stream, f16_rows=f16_rows)
             if stream is not None:
                 stream.sync()
             else:
@@ -58,6 +61,9 @@ class Twin:
             vd.free()
         for s, p0, k, v, t in zip(seqs, pos0, k_list, v_list, n_tok):
             if t:
+                if f16_rows:
+                    k = oracle.f16_bits_to_f32(np.asarray(k, dtype=np.uint16).reshape(-1))
+                    v = oracle.f16_bits_to_f32(np.asarray(v, dtype=np.uint16).reshape(-1))
                 rc = self.images[layer].append(self.pool.block_table(s), p0, k, v,
                                                capacity_cells=self.pool.seq_capacity(s))
                 assert rc == 0

@@ -148,6 +148,50 @@ def test_quantised_append_is_bit_exact(layout):
         assert np.array_equal(gk, ok) and np.array_equal(gv, ov)
 
 
+@pytest.mark.parametrize("layout", [L.LAYOUT_F16, L.LAYOUT_Q8V, L.LAYOUT_I8H])
+def test_f16_rows_append_like_their_widened_f32_rows(layout):
+    # bkv_append_f16: raw binary16 rows, read under the cache's load rule
+    # (crates/breccia-kernels/shaders/f16_storage.glsl:58-69), then the path of bkv_append.
+    rng = np.random.Generator(np.random.PCG64(90 + layout))
+    T = 259
+    k = rng.standard_normal((T, 2, 256)).astype(np.float16).view(np.uint16)
+    v = rng.standard_normal((T, 2, 256)).astype(np.float16).view(np.uint16)
+    # every one of the 65536 codes appears at least once: subnormals, infinities, NaN payloads
+    codes = np.arange(65536, dtype=np.uint16).reshape(128, 2, 256)
+    k = np.concatenate([k, codes[:64], v[:5]])
+    v = np.concatenate([v, codes[64:], k[:5]])
+    n = k.shape[0]
+    with Twin(n_pages=64, layout=layout, max_seqs=4) as tw:
+        other = tw.pool.seq_create()
+        tw.pool.seq_reserve(other, 40)
+        s = tw.pool.seq_create()
+        tw.pool.seq_reserve(s, n + 3)
+        tw.append(0, [s], [3], [k], [v], f16_rows=True)
+        tw.assert_pools_equal()
+        if layout == L.LAYOUT_F16:
+            # finite normal codes are stored verbatim; subnormal codes as signed zeros; NaN as inf
+            got = tw.pool.gather(0, s, 3, n)[0].reshape(-1)
+            src = k.reshape(-1)
+            normal = ((src >> 10) & 0x1F != 0) & ((src >> 10) & 0x1F != 31)
+            assert np.array_equal(oracle.f32_to_f16_bits(got[normal]), src[normal])
+        # the f32 append of the widened rows lands on the same bytes
+        t2 = tw.pool.seq_create()
+        tw.pool.seq_reserve(t2, n + 3)
+        wk = oracle.f16_bits_to_f32(k.reshape(-1)).reshape(k.shape)
+        wv = oracle.f16_bits_to_f32(v.reshape(-1)).reshape(v.shape)
+        tw.append(0, [t2], [3], [wk], [wv])
+        a = tw.pool.gather(0, s, 3, n)
+        b = tw.pool.gather(0, t2, 3, n)
+        assert np.array_equal(a[0].view(np.uint32), b[0].view(np.uint32))
+        assert np.array_equal(a[1].view(np.uint32), b[1].view(np.uint32))
+        # errors are the same as bkv_append's
+        z = DeviceBuffer(4096)
+        with pytest.raises(BkvError) as ei:
+            tw.pool.append(0, [s], [tw.pool.seq_capacity(s)], [1], z, z, f16_rows=True)
+        assert ei.value.status == L.ERR_RANGE
+        z.free()
+
+
 def test_enqueue_on_a_stream_equals_sync_after_every_call():
     # the reference's batching contract (crates/breccia-kernels/tests/batching.rs:27-88):
     # six dependent operations recorded back to back == the same six run one at a time
