@@ -411,6 +411,20 @@ def bench_moves(stream) -> dict:
     b = 4 * T * N_KV * HD * (2 + 2) * 2
     res["append_bulk_f16_rows"] = {"tokens": 4 * T, "ms": round(ms, 4), "GBps": round(b / ms / 1e6, 1),
                                    "frac_of_hbm_peak": round(b / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    # K preparation fused into the append (RMSNorm * gamma -> rotary -> store): same bytes
+    from breccia_amd.kv import rope_table
+    gd = DeviceBuffer.from_numpy(np.ones(HD, dtype=np.float32))
+    td = DeviceBuffer.from_numpy(rope_table(1e7, 64, T))
+    ms = timed(lambda: pool.append_kprep(0, seqs, [0] * 4, [T] * 4, kd, vd, gd, 1e-6, td, 64, T,
+                                         stream=stream), 20)
+    b = 4 * T * APPEND_BYTES_PER_TOKEN
+    res["append_kprep_bulk"] = {"tokens": 4 * T, "ms": round(ms, 4), "GBps": round(b / ms / 1e6, 1),
+                                "frac_of_hbm_peak": round(b / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    ms = timed(lambda: pool.append_kprep(0, seqs, [7] * 4, [1] * 4, kd, vd, gd, 1e-6, td, 64, T,
+                                         stream=stream), 200)
+    res["append_kprep_decode_us"] = round(ms * 1e3, 2)
+    gd.free()
+    td.free()
     kd.free()
     vd.free()
 

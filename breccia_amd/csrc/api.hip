@@ -8,6 +8,8 @@
 #include <new>
 #include <unordered_map>
 
+#include <cmath>
+
 #include "bkv_internal.hpp"
 
 namespace bkv {
@@ -439,9 +441,11 @@ bkv_status bkv_pool_check(const bkv_pool* p) {
 }
 
 // ---- append ------------------------------------------------------------------------
-static bkv_status append_rows(bkv_pool* p, int32_t layer, int32_t n_seqs, const int32_t* seqs,
-                              const int64_t* pos0, const int32_t* n_tokens, const void* k_dev,
-                              const void* v_dev, bool src_is_f16, void* stream) {
+// Range checks shared by the append entry points (qsa/mod.rs:1108-1116: a write past the
+// cache is an error before anything is launched) and the per-sequence launch arguments.
+static bkv_status build_append_batch(bkv_pool* p, int32_t layer, int32_t n_seqs, const int32_t* seqs,
+                                     const int64_t* pos0, const int32_t* n_tokens, AppendBatch& b,
+                                     int64_t& total, int32_t& max_tok) {
     if (!p) return fail(BKV_ERR_INVALID, "append: NULL pool");
     if (layer < 0 || layer >= p->g.n_layers)
         return fail(BKV_ERR_RANGE, sfmt("append: layer %lld is outside 0..%lld", layer,
@@ -451,9 +455,9 @@ static bkv_status append_rows(bkv_pool* p, int32_t layer, int32_t n_seqs, const 
                                           n_seqs, BKV_MAX_BATCH));
     if (n_seqs > 0 && (!seqs || !pos0 || !n_tokens))
         return fail(BKV_ERR_INVALID, "append: NULL sequence / position / token-count array");
-    AppendBatch b{};
-    int64_t src = 0;
-    int32_t max_tok = 0;
+    b = AppendBatch{};
+    total = 0;
+    max_tok = 0;
     for (int i = 0; i < n_seqs; ++i) {
         if (!p->alloc->seq_valid(seqs[i]))
             return fail(BKV_ERR_RANGE, sfmt("append: sequence %lld is not live", seqs[i]));
@@ -477,16 +481,25 @@ static bkv_status append_rows(bkv_pool* p, int32_t layer, int32_t n_seqs, const 
         b.row[i] = seqs[i];
         b.pos0[i] = (int32_t)pos0[i];
         b.n_tok[i] = n_tokens[i];
-        b.src0[i] = (int32_t)src;
-        src += n_tokens[i];
+        b.src0[i] = (int32_t)total;
+        total += n_tokens[i];
         max_tok = std::max(max_tok, n_tokens[i]);
     }
     b.n = n_seqs;
-    if (src > ((int64_t)1 << 30))
+    if (total > ((int64_t)1 << 30))
         return fail(BKV_ERR_INVALID, "append: more than 2^30 tokens in one call");
-    bkv_status st = need_device(p);
+    return need_device(p);
+}
+
+static bkv_status append_rows(bkv_pool* p, int32_t layer, int32_t n_seqs, const int32_t* seqs,
+                              const int64_t* pos0, const int32_t* n_tokens, const void* k_dev,
+                              const void* v_dev, bool src_is_f16, void* stream) {
+    AppendBatch b;
+    int64_t total;
+    int32_t max_tok;
+    bkv_status st = build_append_batch(p, layer, n_seqs, seqs, pos0, n_tokens, b, total, max_tok);
     if (st != BKV_OK) return st;
-    if (src == 0) return flush_tables(p, S(stream));
+    if (total == 0) return flush_tables(p, S(stream));
     if (!k_dev || !v_dev || !aligned16(k_dev) || !aligned16(v_dev))
         return fail(BKV_ERR_INVALID, "append: k/v device pointers must be non-NULL and 16-byte "
                                      "aligned");
@@ -510,6 +523,56 @@ bkv_status bkv_append_f16(bkv_pool* p, int32_t layer, int32_t n_seqs, const int3
                           const int64_t* pos0, const int32_t* n_tokens, const uint16_t* k_dev,
                           const uint16_t* v_dev, void* stream) {
     return append_rows(p, layer, n_seqs, seqs, pos0, n_tokens, k_dev, v_dev, true, stream);
+}
+
+bkv_status bkv_append_kprep(bkv_pool* p, int32_t layer, int32_t n_seqs, const int32_t* seqs,
+                            const int64_t* pos0, const int32_t* n_tokens, const float* k_dev,
+                            const float* v_dev, const float* k_gamma_dev, float eps,
+                            const float* rope_table_dev, int32_t n_rot, int32_t max_pos,
+                            const int32_t* positions_dev, void* stream) {
+    AppendBatch b;
+    int64_t total;
+    int32_t max_tok;
+    bkv_status st = build_append_batch(p, layer, n_seqs, seqs, pos0, n_tokens, b, total, max_tok);
+    if (st != BKV_OK) return st;
+    if (n_rot <= 0 || n_rot % 2 != 0 || n_rot > p->g.hd)
+        return fail(BKV_ERR_INVALID, sfmt("append_kprep: n_rot %lld must be even and within 2..%lld",
+                                          n_rot, p->g.hd));
+    if (max_pos <= 0)
+        return fail(BKV_ERR_INVALID, sfmt("append_kprep: a rotary table of %lld positions", max_pos));
+    if (!(eps >= 0.0f)) return fail(BKV_ERR_INVALID, "append_kprep: eps must be >= 0");
+    if (total == 0) return flush_tables(p, S(stream));
+    if (!k_dev || !v_dev || !aligned16(k_dev) || !aligned16(v_dev))
+        return fail(BKV_ERR_INVALID, "append_kprep: k/v device pointers must be non-NULL and "
+                                     "16-byte aligned");
+    if (!k_gamma_dev || !rope_table_dev || ((uintptr_t)rope_table_dev & 7u))
+        return fail(BKV_ERR_INVALID, "append_kprep: gamma and the rotary table must be non-NULL "
+                                     "device pointers (table 8-byte aligned)");
+    st = flush_tables(p, S(stream));
+    if (st != BKV_OK) return st;
+    {
+        StageScope timed(p, BKV_STAGE_APPEND, S(stream));
+        BKV_HIP(launch_append_kprep(p, layer, b, max_tok, k_dev, v_dev, k_gamma_dev, eps,
+                                    rope_table_dev, n_rot, max_pos, positions_dev, S(stream)));
+    }
+    if (p->timer.open.size() > 8192) return timer_collect(p);
+    return BKV_OK;
+}
+
+bkv_status bkv_rope_table(double freq_base, int32_t n_rot, int32_t max_pos, float* host_out) {
+    if (n_rot <= 0 || n_rot % 2 != 0)
+        return fail(BKV_ERR_INVALID, sfmt("rope_table: n_rot %lld must be even and positive", n_rot));
+    if (max_pos <= 0) return fail(BKV_ERR_INVALID, "rope_table: an empty table");
+    if (!host_out) return fail(BKV_ERR_INVALID, "rope_table: NULL output");
+    const int half = n_rot / 2;
+    for (int64_t pos = 0; pos < max_pos; ++pos)
+        for (int i = 0; i < half; ++i) {
+            const double inv = std::pow(freq_base, -2.0 * (double)i / (double)n_rot);
+            const double ang = (double)pos * inv;
+            host_out[(pos * half + i) * 2] = (float)std::cos(ang);
+            host_out[(pos * half + i) * 2 + 1] = (float)std::sin(ang);
+        }
+    return BKV_OK;
 }
 
 // ---- decode attention ----------------------------------------------------------------

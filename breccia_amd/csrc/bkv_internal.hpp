@@ -130,6 +130,11 @@ struct AppendBatch {
 hipError_t launch_append(const bkv_pool* p, int32_t layer, const AppendBatch& b, int32_t max_tok,
                          const void* k, const void* v, bool src_is_f16, hipStream_t stream);
 
+hipError_t launch_append_kprep(const bkv_pool* p, int32_t layer, const AppendBatch& b, int32_t max_tok,
+                               const float* k, const float* v, const float* gamma, float eps,
+                               const float* table, int32_t n_rot, int32_t max_pos,
+                               const int32_t* positions, hipStream_t stream);
+
 struct AttnBatch {
     int32_t n;
     int32_t row[BKV_MAX_BATCH];       // block-table row

@@ -162,6 +162,17 @@ __device__ __forceinline__ void load32(const SrcT* p, float (&x)[32]) {
     }
 }
 
+// One q8_0 block as the V pool holds it: [f32 scale][32 x i8] = 9 words.
+__device__ __forceinline__ void q8v_encode(const float (&x)[32], uint32_t* vd) {
+    const float amax = amax32(x);
+    const float scale = amax > 0.0f ? amax / 127.0f : 1.0f;
+    uint32_t w[8];
+    q8_block(x, scale, w);
+    vd[0] = __float_as_uint(scale);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) vd[1 + j] = w[j];
+}
+
 // ---- append, reference q8_0-V rows: K f16, V [f32 scale][32 x i8] per 32 values ---
 // One lane per (token, kv head, 32-element block), as the reference shader does.
 template <typename SrcT>
@@ -200,23 +211,13 @@ __global__ __launch_bounds__(kBlock) void append_q8v_kernel(AppendBatch b, MoveG
         kd[i] = o;
     }
     load32(v + src, x);
-    const float amax = amax32(x);
-    const float scale = amax > 0.0f ? amax / 127.0f : 1.0f;
-    uint32_t w[8];
-    q8_block(x, scale, w);
-    uint32_t* vd = vpool + (row * (size_t)blocks + (size_t)blk) * 9u;
-    vd[0] = __float_as_uint(scale);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) vd[1 + j] = w[j];
+    q8v_encode(x, vpool + (row * (size_t)blocks + (size_t)blk) * 9u);
 }
 
 // ---- append, int8 K and V with f16 scales: row = [hd x i8][hd/32 x f16] -----------
 // The q8_0 rule with the scale stored through the cache's f16 encoding; a scale the
 // f16 rule would flush is raised to 2^-14.  (No reference counterpart.)
-template <typename SrcT>
-__device__ __forceinline__ void i8h_block(const SrcT* src, uint8_t* row_base, int hd, int blk) {
-    float x[32];
-    load32(src, x);
+__device__ __forceinline__ void i8h_encode(const float (&x)[32], uint8_t* row_base, int hd, int blk) {
     const float amax = amax32(x);
     uint32_t hb;
     if (amax > 0.0f) {
@@ -247,6 +248,13 @@ __device__ __forceinline__ void i8h_block(const SrcT* src, uint8_t* row_base, in
 }
 
 template <typename SrcT>
+__device__ __forceinline__ void i8h_block(const SrcT* src, uint8_t* row_base, int hd, int blk) {
+    float x[32];
+    load32(src, x);
+    i8h_encode(x, row_base, hd, blk);
+}
+
+template <typename SrcT>
 __global__ __launch_bounds__(kBlock) void append_i8h_kernel(AppendBatch b, MoveGeom g,
                                                             uint8_t* __restrict__ kpool,
                                                             uint8_t* __restrict__ vpool,
@@ -273,6 +281,160 @@ __global__ __launch_bounds__(kBlock) void append_i8h_kernel(AppendBatch b, MoveG
                        (size_t)kvh * g.hd + (size_t)blk * 32;
     const size_t row_bytes = (size_t)g.hd + (size_t)blocks * 2;
     i8h_block((which ? v : k) + src, (which ? vpool : kpool) + row * row_bytes, g.hd, blk);
+}
+
+// ---- K preparation fused into the append ------------------------------------------
+// RMSNorm with gamma per (token, kv head) row, partial NEOX rotary at the token's
+// position, then the append; V rows are appended as they are.  Replaces the chain
+// Qsa::k_norm -> Qsa::rope_k -> Qsa::kv_append (qsa/mod.rs:1051-1058, :1079-1089,
+// :1105-1156; shaders ops_rmsnorm.comp, ops_rope.comp, qsa_kv_append.comp) and its two
+// f32 round trips through memory.  The arithmetic is the CPU reference's, operation for
+// operation (ops/cpu.rs:52-88, :124-154): f64 sum of squares in element order,
+// inv = 1/sqrt(ss/cols + eps), y = (f32)(x * inv * gamma), rotary products and sums in
+// f64 without fusing, one f32 rounding per stage -- so the stored codes are bit-identical
+// to that path followed by the cache's f16 rule.
+struct KPrepParams {
+    const float* gamma;        // [hd]
+    const float* table;        // [max_pos][n_rot/2] of (cos, sin)
+    const int32_t* positions;  // optional: rotary position of cell c; null = c itself
+    float eps;
+    int32_t n_rot, max_pos;
+};
+
+constexpr int kPrepRows = 16;  // (token, kv head) rows per work-group
+
+__device__ __forceinline__ double row_sum_squares(const float* row, int n) {
+#pragma clang fp contract(off)
+    double ss = 0.0;
+    for (int i = 0; i < n; ++i) {
+        const double v = (double)row[i];
+        ss += v * v;
+    }
+    return ss;
+}
+
+__device__ __forceinline__ void rotate_pair(float& lo, float& hi, float c32, float s32) {
+#pragma clang fp contract(off)
+    const double a = (double)lo, b = (double)hi, c = (double)c32, sn = (double)s32;
+    const double ac = a * c, bs = b * sn, as = a * sn, bc = b * c;
+    lo = (float)(ac - bs);
+    hi = (float)(as + bc);
+}
+
+template <int LAYOUT>
+__global__ __launch_bounds__(kBlock) void append_kprep_kernel(AppendBatch b, MoveGeom g,
+                                                              KPrepParams kp,
+                                                              uint8_t* __restrict__ kpool,
+                                                              uint8_t* __restrict__ vpool,
+                                                              const int32_t* __restrict__ tables,
+                                                              const float* __restrict__ k,
+                                                              const float* __restrict__ v) {
+    extern __shared__ float prep_lds[];  // [kPrepRows][hd + 1] floats, then kPrepRows doubles
+    const int s = blockIdx.y;
+    const int hd = g.hd;
+    const int stride = hd + 1;  // odd stride: the per-row serial sums do not collide on banks
+    const int rows_total = b.n_tok[s] * g.n_kv;
+    const int r0 = (int)blockIdx.x * kPrepRows;
+    if (r0 >= rows_total) return;
+    const int nrows = min(kPrepRows, rows_total - r0);
+    double* inv_s = reinterpret_cast<double*>(prep_lds + ((kPrepRows * stride + 1) & ~1));
+    const size_t src_base = ((size_t)b.src0[s] * g.n_kv + (size_t)r0) * (size_t)hd;
+    const int tid = threadIdx.x;
+
+    // rows of one sequence are contiguous in the source: one coalesced sweep
+    for (int idx = tid; idx < nrows * hd / 4; idx += kBlock) {
+        const v4u w = ld_stream(k + src_base + (size_t)idx * 4);
+        const int row = (idx * 4) / hd, col = (idx * 4) % hd;
+        float* d = prep_lds + row * stride + col;
+        d[0] = __uint_as_float(w.x);
+        d[1] = __uint_as_float(w.y);
+        d[2] = __uint_as_float(w.z);
+        d[3] = __uint_as_float(w.w);
+    }
+    __syncthreads();
+    if (tid < nrows) {
+        const double ss = row_sum_squares(prep_lds + tid * stride, hd);
+        inv_s[tid] = 1.0 / sqrt(ss / (double)hd + (double)kp.eps);
+    }
+    __syncthreads();
+    for (int idx = tid; idx < nrows * hd; idx += kBlock) {
+        const int row = idx / hd, col = idx % hd;
+        float* d = prep_lds + row * stride + col;
+        *d = (float)((double)*d * inv_s[row] * (double)kp.gamma[col]);
+    }
+    __syncthreads();
+    const int half = kp.n_rot / 2;
+    for (int idx = tid; idx < nrows * half; idx += kBlock) {
+        const int row = idx / half, j = idx % half;
+        const int64_t cell = (int64_t)b.pos0[s] + (r0 + row) / g.n_kv;
+        int64_t pos = kp.positions ? (int64_t)kp.positions[cell] : cell;
+        pos = pos < 0 ? 0 : (pos > kp.max_pos - 1 ? kp.max_pos - 1 : pos);
+        const float2 cs = reinterpret_cast<const float2*>(kp.table)[(size_t)pos * half + j];
+        float* d = prep_lds + row * stride;
+        rotate_pair(d[j], d[j + half], cs.x, cs.y);
+    }
+    __syncthreads();
+
+    // pool row of (sequence row r) = (token, kv head)
+    const auto pool_row = [&](int row) -> size_t {
+        const int r = r0 + row;
+        const int64_t cell = (int64_t)b.pos0[s] + r / g.n_kv;
+        const int kvh = r % g.n_kv;
+        const int32_t phys = tables[(size_t)b.row[s] * (size_t)g.max_pages_per_seq +
+                                    (size_t)(cell / g.page_cells)];
+        return ((size_t)phys * g.n_kv + kvh) * g.page_cells + (size_t)(cell % g.page_cells);
+    };
+    const int blocks = hd / 32;
+
+    // K from LDS
+    if (LAYOUT == BKV_LAYOUT_I8H) {
+        const size_t row_bytes = (size_t)hd + (size_t)blocks * 2;
+        for (int idx = tid; idx < nrows * blocks; idx += kBlock) {
+            const int row = idx / blocks, blk = idx % blocks;
+            float x[32];
+#pragma unroll
+            for (int i = 0; i < 32; ++i) x[i] = prep_lds[row * stride + blk * 32 + i];
+            i8h_encode(x, kpool + pool_row(row) * row_bytes, hd, blk);
+        }
+    } else {
+        for (int idx = tid; idx < nrows * hd / 8; idx += kBlock) {
+            const int row = (idx * 8) / hd, col = (idx * 8) % hd;
+            const float* x = prep_lds + row * stride + col;
+            v4u o;
+            o.x = pack2(x[0], x[1]);
+            o.y = pack2(x[2], x[3]);
+            o.z = pack2(x[4], x[5]);
+            o.w = pack2(x[6], x[7]);
+            st_stream(reinterpret_cast<uint16_t*>(kpool) + pool_row(row) * (size_t)hd + col, o);
+        }
+    }
+
+    // V straight from the source rows
+    if (LAYOUT == BKV_LAYOUT_F16) {
+        for (int idx = tid; idx < nrows * hd / 8; idx += kBlock) {
+            const int row = (idx * 8) / hd, col = (idx * 8) % hd;
+            float x[8];
+            load8(v + src_base + (size_t)idx * 8, x);
+            v4u o;
+            o.x = pack2(x[0], x[1]);
+            o.y = pack2(x[2], x[3]);
+            o.z = pack2(x[4], x[5]);
+            o.w = pack2(x[6], x[7]);
+            st_stream(reinterpret_cast<uint16_t*>(vpool) + pool_row(row) * (size_t)hd + col, o);
+        }
+    } else {
+        const size_t row_bytes = (size_t)hd + (size_t)blocks * 2;
+        for (int idx = tid; idx < nrows * blocks; idx += kBlock) {
+            const int row = idx / blocks, blk = idx % blocks;
+            float x[32];
+            load32(v + src_base + (size_t)idx * 32, x);
+            if (LAYOUT == BKV_LAYOUT_Q8V)
+                q8v_encode(x, reinterpret_cast<uint32_t*>(vpool) +
+                                  (pool_row(row) * (size_t)blocks + (size_t)blk) * 9u);
+            else
+                i8h_encode(x, vpool + pool_row(row) * row_bytes, hd, blk);
+        }
+    }
 }
 
 // ---- whole-page moves -----------------------------------------------------------
@@ -507,6 +669,35 @@ hipError_t launch_append(const bkv_pool* p, int32_t layer, const AppendBatch& b,
     if (src_is_f16)
         return launch_append_from(p, layer, b, max_tok, (const uint16_t*)k, (const uint16_t*)v, stream);
     return launch_append_from(p, layer, b, max_tok, (const float*)k, (const float*)v, stream);
+}
+
+hipError_t launch_append_kprep(const bkv_pool* p, int32_t layer, const AppendBatch& b, int32_t max_tok,
+                               const float* k, const float* v, const float* gamma, float eps,
+                               const float* table, int32_t n_rot, int32_t max_pos,
+                               const int32_t* positions, hipStream_t stream) {
+    const MoveGeom g = move_geom(p);
+    const KPrepParams kp{gamma, table, positions, eps, n_rot, max_pos};
+    const int rows = max_tok * g.n_kv;
+    dim3 grid((unsigned)((rows + kPrepRows - 1) / kPrepRows), (unsigned)b.n);
+    const size_t lds = (size_t)((kPrepRows * (g.hd + 1) + 1) & ~1) * sizeof(float) +
+                       kPrepRows * sizeof(double);
+    uint8_t* kpl = p->k_layer[(size_t)layer];
+    uint8_t* vpl = p->v_layer[(size_t)layer];
+    switch (p->g.layout) {
+        case BKV_LAYOUT_F16:
+            append_kprep_kernel<BKV_LAYOUT_F16><<<grid, kBlock, lds, stream>>>(b, g, kp, kpl, vpl,
+                                                                              p->table_dev, k, v);
+            break;
+        case BKV_LAYOUT_Q8V:
+            append_kprep_kernel<BKV_LAYOUT_Q8V><<<grid, kBlock, lds, stream>>>(b, g, kp, kpl, vpl,
+                                                                              p->table_dev, k, v);
+            break;
+        default:
+            append_kprep_kernel<BKV_LAYOUT_I8H><<<grid, kBlock, lds, stream>>>(b, g, kp, kpl, vpl,
+                                                                              p->table_dev, k, v);
+            break;
+    }
+    return hipGetLastError();
 }
 
 hipError_t launch_page_copy(const bkv_pool* p, const bkv_page_pair* pairs_dev, int32_t n_pairs,

@@ -33,6 +33,8 @@ constexpr int MODEL_N_HEAD = 24;      // qsa/mod.rs:69
 constexpr int MODEL_N_KV_HEAD = 2;    // qsa/mod.rs:71
 constexpr int MODEL_HEAD_DIM = 256;   // qsa/mod.rs:73
 constexpr int PAGE_CELLS = 16;        // qsa/mod.rs:116
+constexpr int MODEL_N_ROT = 64;       // ops/mod.rs:454
+constexpr float MODEL_RMS_EPS = 1e-6f;  // ops/mod.rs:316
 
 enum class VLayout { F16, Q8_0 };  // qsa/mod.rs:242-254
 
@@ -151,6 +153,24 @@ public:
                                       nullptr));
         }
         check(bkv_append(state.pool, 0, 1, &state.seq, &p0, &n, ws.k_cur, ws.v_cur, stream_));
+    }
+
+    // Qsa::k_norm + Qsa::rope_k + Qsa::kv_append in one launch (qsa/mod.rs:1051-1058,
+    // :1079-1089, :1105-1131): ws.k_cur is normalised with k_norm_gamma[head_dim], rotated
+    // over the first MODEL_N_ROT dims at positions pos0.. (identity positions, as the
+    // reference's state.positions holds), and stored; ws.k_cur itself is left unchanged.
+    void k_prep_append(const QsaState& state, const QsaWorkspace& ws, const float* k_norm_gamma,
+                       const float* rope_table, int32_t rope_max_pos, size_t pos0) const {
+        const int64_t p0 = (int64_t)pos0;
+        const int32_t n = (int32_t)ws.tokens;
+        if (pos0 + ws.tokens <= state.capacity_cells) {
+            const int64_t len = bkv_seq_len(state.pool, state.seq);
+            if ((int64_t)(pos0 + ws.tokens) > len)
+                check(bkv_seq_reserve(state.pool, state.seq, (int64_t)(pos0 + ws.tokens), nullptr, 0,
+                                      nullptr));
+        }
+        check(bkv_append_kprep(state.pool, 0, 1, &state.seq, &p0, &n, ws.k_cur, ws.v_cur, k_norm_gamma,
+                               MODEL_RMS_EPS, rope_table, MODEL_N_ROT, rope_max_pos, nullptr, stream_));
     }
 
     // Range checks of the attention call; nothing is launched (no score matrix exists).

@@ -65,6 +65,13 @@ def _sh(stream):
     return stream.handle if isinstance(stream, Stream) else stream
 
 
+def rope_table(freq_base: float, n_rot: int, max_pos: int) -> np.ndarray:
+    """float32 [max_pos, n_rot/2, 2] of (cos, sin), built by the library on the host."""
+    out = np.empty((max_pos, max(n_rot // 2, 1), 2), dtype=np.float32)
+    check(lib.bkv_rope_table(freq_base, n_rot, max_pos, out.ctypes.data))
+    return out
+
+
 def device_sync() -> None:
     check(lib.bkv_device_sync())
 
@@ -265,6 +272,18 @@ class Pool:
         assert seqs.size == pos0.size == n_tokens.size
         fn = lib.bkv_append_f16 if f16_rows else lib.bkv_append
         check(fn(self.handle, layer, seqs.size, ps, pp, pn, _ptr(k_dev), _ptr(v_dev), _sh(stream)))
+
+    def append_kprep(self, layer: int, seqs, pos0, n_tokens, k_dev, v_dev, gamma_dev, eps: float,
+                     table_dev, n_rot: int, max_pos: int, positions_dev=None, stream=None) -> None:
+        """RMSNorm(k) * gamma -> rotary at the token's position -> append, in one launch."""
+        seqs, ps = _i32(seqs)
+        pos0, pp = _i64(pos0)
+        n_tokens, pn = _i32(n_tokens)
+        assert seqs.size == pos0.size == n_tokens.size
+        check(lib.bkv_append_kprep(self.handle, layer, seqs.size, ps, pp, pn, _ptr(k_dev), _ptr(v_dev),
+                                   _ptr(gamma_dev), eps, _ptr(table_dev), n_rot, max_pos,
+                                   _ptr(positions_dev) if positions_dev is not None else None,
+                                   _sh(stream)))
 
     def decode_attn(self, layer: int, seqs, pos, n_q_head: int, q_dev, out_dev, scale: float,
                     gate_dev=None, gate_seq_stride: int = 0, gate_head_stride: int = 0,

@@ -80,6 +80,9 @@ _SIGNATURES = {
     "bkv_timing_read": (C.c_int, [_vp, C.c_int, C.POINTER(_u64), C.POINTER(C.c_double)]),
     "bkv_append": (C.c_int, [_vp, _i32, _i32, _pi32, _pi64, _pi32, _vp, _vp, _vp]),
     "bkv_append_f16": (C.c_int, [_vp, _i32, _i32, _pi32, _pi64, _pi32, _vp, _vp, _vp]),
+    "bkv_append_kprep": (C.c_int, [_vp, _i32, _i32, _pi32, _pi64, _pi32, _vp, _vp, _vp, _f32, _vp, _i32,
+                                   _i32, _vp, _vp]),
+    "bkv_rope_table": (C.c_int, [C.c_double, _i32, _i32, _vp]),
     "bkv_decode_attn": (C.c_int, [_vp, _i32, _i32, _pi32, _pi64, _i32, _vp, _vp, _i64, _i64, _f32,
                                   _vp, _vp]),
     "bkv_page_copy": (C.c_int, [_vp, C.POINTER(PagePair), _i32, _vp]),

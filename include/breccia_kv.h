@@ -159,6 +159,31 @@ bkv_status bkv_append_f16(bkv_pool *pool, int32_t layer, int32_t n_seqs, const i
                           const int64_t *pos0, const int32_t *n_tokens, const uint16_t *k_dev,
                           const uint16_t *v_dev, void *stream);
 
+/* K preparation fused into the append: per (token, kv head) row RMSNorm with gamma
+ * (Qsa::k_norm, qsa/mod.rs:1051-1058; ops/mod.rs:317-420), the partial NEOX-paired rotary
+ * at the token's position (Qsa::rope_k, qsa/mod.rs:1079-1089; ops/mod.rs:634-654), then
+ * bkv_append's store; V rows are appended untouched (qsa/cpu.rs:383-397).  One launch
+ * instead of three and no f32 round trip of K.  Arithmetic follows the reference CPU path
+ * operation for operation (ops/cpu.rs:52-88, :124-154: f64, one f32 rounding per stage).
+ *   k_gamma_dev     device f32 [head_dim]
+ *   eps             RMSNorm epsilon (the model's is 1e-6, ops/mod.rs:316)
+ *   rope_table_dev  device f32 [max_pos][n_rot/2][2] of (cos, sin), see bkv_rope_table
+ *   positions_dev   optional device int32 indexed by cell (the reference's positions
+ *                   buffer, read at pos0 + token); NULL = the cell index itself.  When
+ *                   given it must cover every cell written.  Positions outside the table
+ *                   are clamped to its first / last row (shaders/ops_rope.comp).
+ * Shapes, errors and ordering are those of bkv_append. */
+bkv_status bkv_append_kprep(bkv_pool *pool, int32_t layer, int32_t n_seqs, const int32_t *seqs,
+                            const int64_t *pos0, const int32_t *n_tokens, const float *k_dev,
+                            const float *v_dev, const float *k_gamma_dev, float eps,
+                            const float *rope_table_dev, int32_t n_rot, int32_t max_pos,
+                            const int32_t *positions_dev, void *stream);
+/* Host-side rotary table, the reference's formula (ops/cpu.rs:103-119, RopeTable::build
+ * ops/mod.rs:475-487): table[p][i] = (cos, sin)(p * freq_base^(-2i/n_rot)) evaluated in
+ * double and rounded to float.  host_out: max_pos * n_rot floats.  The model's table is
+ * freq_base 1e7, n_rot 64. */
+bkv_status bkv_rope_table(double freq_base, int32_t n_rot, int32_t max_pos, float *host_out);
+
 /* bkv_decode_attn replaces Qsa::attend + Qsa::apply for decode shapes with the dense
  * selection (qsa/mod.rs:1382-1462, :1466-1522; shaders qsa_attn_scores_small,
  * ops_softmax, qsa_attn_apply_split, qsa_attn_apply_reduce; oracle qsa/cpu.rs:197-246):

@@ -96,6 +96,11 @@ _lib.bkvo_swap_out.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C
                                C.c_size_t, C.c_size_t]
 _lib.bkvo_swap_in.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p,
                               C.c_size_t, C.c_size_t]
+_lib.bkvo_rmsnorm.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p, C.c_float,
+                              C.c_void_p]
+_lib.bkvo_rope_table.argtypes = [C.c_double, C.c_size_t, C.c_size_t, C.c_void_p]
+_lib.bkvo_rope_apply.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p,
+                                 C.c_size_t, C.c_void_p, C.c_void_p]
 _lib.bkvo_normalish.argtypes = [C.c_uint64, C.c_size_t, C.c_void_p]
 _lib.bkvo_q8_fixture.argtypes = [C.c_void_p, C.c_size_t]
 _lib.bkvo_max_threads.restype = C.c_int
@@ -275,6 +280,56 @@ def dense_cells(pos: int) -> np.ndarray:
 
 
 # -------------------------------------------------------------- test generators
+# ------------------------------------------------------------------ K preparation
+def rmsnorm(x, cols: int, gamma=None, wgroups: int | None = None, eps: float = 1e-6) -> np.ndarray:
+    """Row-wise RMSNorm of x viewed as [rows, cols]; gamma is [wgroups, cols] or None."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    rows = x.size // cols
+    assert rows * cols == x.size
+    if gamma is None:
+        wg, gp = 0, None
+    else:
+        gamma = np.ascontiguousarray(gamma, dtype=np.float32)
+        wg = gamma.size // cols if wgroups is None else wgroups
+        assert gamma.size >= wg * cols and wg > 0
+        gp = gamma.ctypes.data
+    out = np.empty_like(x)
+    _lib.bkvo_rmsnorm(x.ctypes.data, rows, cols, wg, gp, C.c_float(eps), out.ctypes.data)
+    return out
+
+
+def rope_table(freq_base: float, n_rot: int, max_pos: int) -> np.ndarray:
+    """float32 [max_pos, n_rot/2, 2] of (cos, sin)."""
+    assert n_rot % 2 == 0
+    out = np.empty((max_pos, n_rot // 2, 2), dtype=np.float32)
+    _lib.bkvo_rope_table(float(freq_base), n_rot, max_pos, out.ctypes.data)
+    return out
+
+
+def rope_apply(x, head_dim: int, n_rot: int, table, positions) -> np.ndarray:
+    """x viewed as [rows, head_dim]; positions int32 [rows]."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    rows = x.size // head_dim
+    table = np.ascontiguousarray(table, dtype=np.float32)
+    positions = np.ascontiguousarray(positions, dtype=np.int32)
+    assert positions.size >= rows and n_rot <= head_dim and n_rot % 2 == 0
+    max_pos = table.size // n_rot
+    out = np.empty_like(x)
+    _lib.bkvo_rope_apply(x.ctypes.data, rows, head_dim, n_rot, table.ctypes.data, max_pos,
+                         positions.ctypes.data, out.ctypes.data)
+    return out
+
+
+def k_prep(k, n_kv: int, hd: int, gamma, eps: float, table, n_rot: int, token_pos) -> np.ndarray:
+    """What reaches the cache as K: per-(token, kv head) RMSNorm with gamma[hd], then the
+    rotary at the token's position (crates/breccia-kernels/src/qsa/cpu.rs:383-397).
+    k: [T, n_kv, hd]; token_pos: int [T]."""
+    k = np.ascontiguousarray(k, dtype=np.float32).reshape(-1, n_kv, hd)
+    normed = rmsnorm(k, hd, gamma, wgroups=1, eps=eps)
+    pos = np.repeat(np.asarray(token_pos, dtype=np.int32), n_kv)
+    return rope_apply(normed, hd, n_rot, table, pos).reshape(k.shape)
+
+
 def normalish(seed: int, n: int) -> np.ndarray:
     out = np.empty(n, dtype=np.float32)
     _lib.bkvo_normalish(seed, n, out.ctypes.data)

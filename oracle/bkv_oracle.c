@@ -22,6 +22,10 @@
  *                                        x 512 elements) + permutation round trips
  *   bkvo_attend                          pinned: torch float64 SDPA, independent
  *                                        numpy softmax, closed forms
+ *   bkvo_rmsnorm / bkvo_rope_table /     pinned: reference KATs (ops/cpu.rs:373-421: constant row,
+ *   bkvo_rope_apply                      identity at position 0, NEOX pairing one-hot),
+ *                                        independent numpy float64 statements, rotation
+ *                                        invariants (pair norms kept, angles add)
  *   bkvo_to_i8h / append_i8 / gather_i8  NOT IN THE REFERENCE (int8 K+V with an f16
  *                                        scale): parity unpinned against the
  *                                        reference; pinned only by closed-form
@@ -482,6 +486,64 @@ size_t bkvo_dense_ids(int64_t pos, int64_t n_kv_after, uint32_t idx_block, uint3
     for (int64_t b = 0; b < lim; ++b) out[n++] = (uint32_t)b;
     if (own >= n_blocks) out[n++] = (uint32_t)own;
     return n;
+}
+
+/* ---- K preparation ahead of the append (Qsa::k_norm + Qsa::rope_k) ---------------
+ * crates/breccia-kernels/src/ops/cpu.rs:52-88: row-wise RMSNorm, f64 throughout,
+ * sequential sum, y = (f32)(x * inv * w) with inv = 1/sqrt(ss/cols + eps); row r uses
+ * gamma slice r % wgroups; wgroups == 0 means no gamma. */
+void bkvo_rmsnorm(const float *x, size_t rows, size_t cols, size_t wgroups, const float *gamma,
+                  float eps, float *out) {
+    for (size_t r = 0; r < rows; ++r) {
+        const float *xr = x + r * cols;
+        double ss = 0.0;
+        for (size_t i = 0; i < cols; ++i) {
+            const double v = (double)xr[i];
+            ss += v * v;
+        }
+        const double inv = 1.0 / sqrt(ss / (double)cols + (double)eps);
+        const float *g = wgroups ? gamma + (r % wgroups) * cols : NULL;
+        for (size_t i = 0; i < cols; ++i) {
+            const double w = g ? (double)g[i] : 1.0;
+            out[r * cols + i] = (float)((double)xr[i] * inv * w);
+        }
+    }
+}
+
+/* ops/cpu.rs:103-119: table[p][i] = (cos, sin)(p * freq_base^(-2i/n_rot)), f64 then f32. */
+void bkvo_rope_table(double freq_base, size_t n_rot, size_t max_pos, float *out) {
+    const size_t half = n_rot / 2;
+    for (size_t p = 0; p < max_pos; ++p)
+        for (size_t i = 0; i < half; ++i) {
+            const double inv = pow(freq_base, -2.0 * (double)i / (double)n_rot);
+            const double ang = (double)p * inv;
+            out[(p * half + i) * 2] = (float)cos(ang);
+            out[(p * half + i) * 2 + 1] = (float)sin(ang);
+        }
+}
+
+/* ops/cpu.rs:121-154 (rope_apply at :124): partial NEOX-paired rotary.  out[j] = x[j]*c - x[j+half]*s,
+ * out[j+half] = x[j]*s + x[j+half]*c for j < half = n_rot/2, f64 products and sums, cast
+ * to f32; dims [n_rot, head_dim) copied; the position is clamped into the table. */
+void bkvo_rope_apply(const float *x, size_t rows, size_t head_dim, size_t n_rot, const float *table,
+                     size_t max_pos, const int32_t *positions, float *out) {
+    const size_t half = n_rot / 2;
+    for (size_t r = 0; r < rows; ++r) {
+        const float *xr = x + r * head_dim;
+        float *o = out + r * head_dim;
+        int64_t pc = positions[r];
+        if (pc < 0) pc = 0;
+        if (pc > (int64_t)max_pos - 1) pc = (int64_t)max_pos - 1;
+        const size_t p = (size_t)pc;
+        for (size_t j = 0; j < half; ++j) {
+            const double a = (double)xr[j], b = (double)xr[j + half];
+            const double c = (double)table[(p * half + j) * 2];
+            const double sn = (double)table[(p * half + j) * 2 + 1];
+            o[j] = (float)(a * c - b * sn);
+            o[j + half] = (float)(a * sn + b * c);
+        }
+        for (size_t j = n_rot; j < head_dim; ++j) o[j] = xr[j];
+    }
 }
 
 /* ---------------------------------------------------------------------------

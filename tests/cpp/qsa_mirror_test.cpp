@@ -21,6 +21,9 @@ int bkvo_gather(const bkvo_geom*, int, const void*, const void*, const int32_t*,
 int bkvo_attend(const float*, const float*, const float*, const uint32_t*, size_t, int64_t, int32_t,
                 int32_t, int32_t, const float*, float*, int);
 void bkvo_normalish(uint64_t, size_t, float*);
+void bkvo_rmsnorm(const float*, size_t, size_t, size_t, const float*, float, float*);
+void bkvo_rope_table(double, size_t, size_t, float*);
+void bkvo_rope_apply(const float*, size_t, size_t, size_t, const float*, size_t, const int32_t*, float*);
 }
 
 using namespace breccia::qsa;
@@ -175,11 +178,59 @@ static void test_attention() {
     state.release();
 }
 
+static void test_k_prep_append() {
+    // k_norm -> rope_k -> kv_append in one call: 19 tokens at cells 9..27, the model's table
+    const int T = 19, hd = MODEL_HEAD_DIM, max_pos = 64;
+    const size_t pos0 = 9;
+    QsaState state = QsaState::create(48, max_pos);
+    Qsa qsa;
+    QsaWorkspace ws = qsa.workspace(T, 28);
+    std::vector<float> k(T * 512), v(T * 512), gamma(hd), table((size_t)max_pos * MODEL_N_ROT);
+    bkvo_normalish(0xA1, k.size(), k.data());
+    bkvo_normalish(0xA2, v.size(), v.data());
+    bkvo_normalish(0xFEED, gamma.size(), gamma.data());
+    check(bkv_rope_table(1e7, MODEL_N_ROT, max_pos, table.data()));
+    std::vector<float> want_table(table.size());
+    bkvo_rope_table(1e7, MODEL_N_ROT, max_pos, want_table.data());
+    EXPECT(std::memcmp(table.data(), want_table.data(), table.size() * 4) == 0, "rotary table differs");
+    float *gamma_dev = nullptr, *table_dev = nullptr;
+    check(bkv_dev_alloc(gamma.size() * 4, (void**)&gamma_dev));
+    check(bkv_dev_alloc(table.size() * 4, (void**)&table_dev));
+    upload(gamma_dev, gamma);
+    upload(table_dev, table);
+    upload(ws.k_cur, k);
+    upload(ws.v_cur, v);
+    qsa.k_prep_append(state, ws, gamma_dev, table_dev, max_pos, pos0);
+    check(bkv_device_sync());
+
+    std::vector<float> normed(k.size()), rotated(k.size());
+    bkvo_rmsnorm(k.data(), (size_t)T * 2, hd, 1, gamma.data(), MODEL_RMS_EPS, normed.data());
+    std::vector<int32_t> positions(T * 2);
+    for (int r = 0; r < T * 2; ++r) positions[r] = (int32_t)(pos0 + r / 2);
+    bkvo_rope_apply(normed.data(), (size_t)T * 2, hd, MODEL_N_ROT, table.data(), max_pos, positions.data(),
+                    rotated.data());
+    const bkvo_geom g{2, 256, 16};
+    const int32_t pages[3] = {0, 1, 2};
+    std::vector<uint16_t> want_k(3 * 2 * 16 * 256, 0), want_v(want_k.size(), 0);
+    bkvo_append_f16(&g, want_k.data(), want_v.data(), pages, 48, (int64_t)pos0, T, rotated.data(), v.data());
+    const auto got_k = download<uint16_t>(state.pool_ptr(0), want_k.size());
+    const auto got_v = download<uint16_t>(state.pool_ptr(1), want_v.size());
+    size_t bad = 0;
+    for (size_t i = 0; i < want_k.size(); ++i) bad += (got_k[i] != want_k[i]) + (got_v[i] != want_v[i]);
+    EXPECT(bad == 0, "k_prep_append: %zu halves differ from norm -> rotary -> append on the CPU", bad);
+    std::printf("qsa k_prep_append   T=%d at cell %zu: %zu differing halves\n", T, pos0, bad);
+    check(bkv_dev_free(gamma_dev));
+    check(bkv_dev_free(table_dev));
+    qsa.release(ws);
+    state.release();
+}
+
 int main() {
     try {
         test_errors();
         test_layout_recipe();
         test_attention();
+        test_k_prep_append();
     } catch (const Error& e) {
         std::printf("FAIL: unexpected error %d: %s\n", (int)e.status, e.what());
         return 2;

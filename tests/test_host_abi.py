@@ -254,3 +254,18 @@ def test_randomised_allocator_keeps_its_invariants():
         for s in list(live):
             p.seq_free(s)
         assert p.free_pages() == 48
+
+
+def test_rope_table_is_the_reference_formula():
+    # crates/breccia-kernels/src/ops/mod.rs:2504-2522 (bit for bit against the formula) and
+    # the errors of RopeTable::build (odd n_rot, empty table)
+    import oracle
+    from breccia_amd.kv import rope_table
+
+    for base, n_rot, max_pos in [(1e7, 64, 8), (1e7, 64, 300), (1e4, 128, 17), (5e5, 2, 3)]:
+        got = rope_table(base, n_rot, max_pos)
+        assert np.array_equal(got.view(np.uint32), oracle.rope_table(base, n_rot, max_pos).view(np.uint32))
+    for bad in [(1e7, 63, 8), (1e7, 64, 0), (1e7, 0, 8)]:
+        with pytest.raises(BkvError) as ei:
+            rope_table(*bad)
+        assert ei.value.status == L.ERR_INVALID
