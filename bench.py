@@ -249,6 +249,7 @@ def main() -> int:
     if not args.no_extra:
         extra.update(bench_batch1(stream))
         extra.update(bench_quantised(stream))
+        extra.update(bench_select(stream))
         extra.update(bench_moves(stream))
 
     line = {"metric": "paged decode-attn step throughput, batch 8 mixed 1k-32k (append + attention, "
@@ -362,6 +363,74 @@ def bench_quantised(stream) -> dict:
         pool.destroy()
         for x in bufs:
             x.free()
+    return res
+
+
+def bench_select(stream) -> dict:
+    """Attention over selection lists, the reference's long-context regime: 8 sequences of
+    U{8k..32k} cells, each query attends 512 selected 4-cell blocks + its own block (2052 cells:
+    the reference's top-k budget), f16 pool."""
+    from breccia_amd import lib as L
+    from breccia_amd.kv import DeviceBuffer
+
+    rng = np.random.Generator(np.random.PCG64(20250006))
+    n_layers, n_seqs, max_ids = 4, 8, 513
+    pool, seqs, ctx = build_batched(None, rng, n_seqs, 8192, 32768, n_layers, 0.6)
+    chunk = 8192
+    kd = DeviceBuffer.from_numpy(rng.standard_normal((chunk, N_KV, HD), dtype=np.float32))
+    vd = DeviceBuffer.from_numpy(rng.standard_normal((chunk, N_KV, HD), dtype=np.float32))
+    for layer in range(n_layers):
+        for s, c in zip(seqs, ctx):
+            for at in range(0, c, chunk):
+                pool.append(layer, [s], [at], [min(chunk, c - at)], kd, vd, stream)
+        stream.sync()
+    kd.free()
+    vd.free()
+    ids = np.zeros((n_seqs, max_ids), dtype=np.uint32)
+    for i, c in enumerate(ctx):
+        own = (c - 1) // 4
+        ids[i, :512] = rng.choice(own, size=512, replace=False)
+        ids[i, 512] = own
+    idd = DeviceBuffer.from_numpy(ids)
+    cd = DeviceBuffer.from_numpy(np.full(n_seqs, max_ids, dtype=np.uint32))
+    q = DeviceBuffer.from_numpy(rng.standard_normal((n_seqs, N_Q, HD), dtype=np.float32))
+    out = DeviceBuffer(n_seqs * N_Q * HD * 4)
+    pos = [c - 1 for c in ctx]
+
+    def run(n):
+        for i in range(n):
+            pool.decode_attn_select(i % n_layers, seqs, pos, N_Q, q, out, 1.0 / 16.0, idd, max_ids, cd,
+                                    max_ids, stream=stream)
+
+    from breccia_amd.kv import Event
+    run(20)
+    stream.sync()
+    e0, e1 = Event(), Event()
+    e0.record(stream)
+    run(200)
+    e1.record(stream)
+    stream.sync()
+    us = e0.elapsed_ms(e1) / 200 * 1e3
+    e0.close()
+    e1.close()
+    pool.timing_reset()
+    pool.timing_enable(True)
+    run(100)
+    stream.sync()
+    pool.timing_enable(False)
+    n_split, ms_split = pool.timing_read(L.STAGE_ATTN_SPLIT)
+    n_merge, ms_merge = pool.timing_read(L.STAGE_ATTN_MERGE)
+    cells = n_seqs * (max_ids * 4 - 0)
+    b = cells * ROW_BYTES + n_seqs * (max_ids * 4 + 2 * N_Q * HD * 4)
+    split_us = ms_split / max(n_split, 1) * 1e3
+    res = {"attn_select_batch8": {
+        "workload": "8 sequences U{8k..32k}, 513 selected blocks (2052 cells) each, f16",
+        "algorithmic_bytes": b, "us_per_layer": round(us, 2), "attn_split_us": round(split_us, 2),
+        "attn_merge_us": round(ms_merge / max(n_merge, 1) * 1e3, 2),
+        "GBps": round(b / us / 1e3, 1), "split_GBps": round(b / split_us / 1e3, 1)}}
+    for x in (idd, cd, q, out):
+        x.free()
+    pool.destroy()
     return res
 
 

@@ -576,10 +576,13 @@ bkv_status bkv_rope_table(double freq_base, int32_t n_rot, int32_t max_pos, floa
 }
 
 // ---- decode attention ----------------------------------------------------------------
-bkv_status bkv_decode_attn(bkv_pool* p, int32_t layer, int32_t n, const int32_t* seqs,
-                           const int64_t* pos, int32_t n_q_head, const float* q_dev,
-                           const float* gate_dev, int64_t gate_seq_stride,
-                           int64_t gate_head_stride, float scale, float* out_dev, void* stream) {
+// Shared by the dense and the selection-list entry points.
+static bkv_status decode_attn_common(bkv_pool* p, int32_t layer, int32_t n, const int32_t* seqs,
+                                     const int64_t* pos, int32_t n_q_head, const float* q_dev,
+                                     const float* gate_dev, int64_t gate_seq_stride,
+                                     int64_t gate_head_stride, float scale, const uint32_t* ids_dev,
+                                     int64_t id_stride, const uint32_t* counts_dev, int32_t max_ids,
+                                     bool select, float* out_dev, void* stream) {
     if (!p) return fail(BKV_ERR_INVALID, "decode_attn: NULL pool");
     if (layer < 0 || layer >= p->g.n_layers)
         return fail(BKV_ERR_RANGE, sfmt("decode_attn: layer %lld is outside 0..%lld", layer,
@@ -594,6 +597,17 @@ bkv_status bkv_decode_attn(bkv_pool* p, int32_t layer, int32_t n, const int32_t*
     if (p->g.hd != 256)
         return fail(BKV_ERR_INVALID, sfmt("decode_attn is built for head_dim 256, pool has %lld",
                                           p->g.hd));
+    if (select) {
+        if (p->g.page_cells % 4 != 0)
+            return fail(BKV_ERR_INVALID, "decode_attn_select: 4-cell blocks need a page size that "
+                                         "is a multiple of 4");
+        if (max_ids <= 0 || max_ids > (1 << 24))
+            return fail(BKV_ERR_INVALID, sfmt("decode_attn_select: max_ids %lld is outside "
+                                              "1..2^24", max_ids));
+        if (id_stride < max_ids)
+            return fail(BKV_ERR_INVALID, sfmt("decode_attn_select: id_stride %lld is smaller than "
+                                              "max_ids %lld", id_stride, max_ids));
+    }
     if (n > 0 && (!seqs || !pos)) return fail(BKV_ERR_INVALID, "decode_attn: NULL seqs / pos");
     AttnBatch b{};
     for (int i = 0; i < n; ++i) {
@@ -617,9 +631,12 @@ bkv_status bkv_decode_attn(bkv_pool* p, int32_t layer, int32_t n, const int32_t*
     if (!q_dev || !out_dev || !aligned16(q_dev) || !aligned16(out_dev))
         return fail(BKV_ERR_INVALID, "decode_attn: q/out device pointers must be non-NULL and "
                                      "16-byte aligned");
+    if (select && (!ids_dev || !counts_dev || ((uintptr_t)ids_dev & 3u) || ((uintptr_t)counts_dev & 3u)))
+        return fail(BKV_ERR_INVALID, "decode_attn_select: ids/counts device pointers must be "
+                                     "non-NULL and 4-byte aligned");
     st = flush_tables(p, S(stream));
     if (st != BKV_OK) return st;
-    plan_attn(p, n_q_head, b);
+    plan_attn(p, n_q_head, b, select ? (max_ids + 3) / 4 : 0);
     AttnArgs a;
     a.n_q_head = n_q_head;
     a.q = q_dev;
@@ -628,9 +645,34 @@ bkv_status bkv_decode_attn(bkv_pool* p, int32_t layer, int32_t n, const int32_t*
     a.gate_head_stride = gate_head_stride;
     a.scale = scale;
     a.out = out_dev;
+    if (select) {
+        a.ids = ids_dev;
+        a.counts = counts_dev;
+        a.id_stride = id_stride;
+        a.max_ids = max_ids;
+    }
     BKV_HIP(launch_decode_attn(p, layer, b, a, S(stream)));
     if (p->timer.open.size() > 8192) return timer_collect(p);
     return BKV_OK;
+}
+
+bkv_status bkv_decode_attn(bkv_pool* p, int32_t layer, int32_t n, const int32_t* seqs,
+                           const int64_t* pos, int32_t n_q_head, const float* q_dev,
+                           const float* gate_dev, int64_t gate_seq_stride,
+                           int64_t gate_head_stride, float scale, float* out_dev, void* stream) {
+    return decode_attn_common(p, layer, n, seqs, pos, n_q_head, q_dev, gate_dev, gate_seq_stride,
+                              gate_head_stride, scale, nullptr, 0, nullptr, 0, false, out_dev, stream);
+}
+
+bkv_status bkv_decode_attn_select(bkv_pool* p, int32_t layer, int32_t n, const int32_t* seqs,
+                                  const int64_t* pos, int32_t n_q_head, const float* q_dev,
+                                  const float* gate_dev, int64_t gate_seq_stride,
+                                  int64_t gate_head_stride, float scale, const uint32_t* ids_dev,
+                                  int64_t id_stride, const uint32_t* counts_dev, int32_t max_ids,
+                                  float* out_dev, void* stream) {
+    return decode_attn_common(p, layer, n, seqs, pos, n_q_head, q_dev, gate_dev, gate_seq_stride,
+                              gate_head_stride, scale, ids_dev, id_stride, counts_dev, max_ids, true,
+                              out_dev, stream);
 }
 
 // ---- page copy -------------------------------------------------------------------------

@@ -150,9 +150,15 @@ struct AttnArgs {
     int64_t gate_seq_stride, gate_head_stride;
     float scale;
     float* out;
+    // selection lists; ids == nullptr means the dense selection (every cell 0..=pos)
+    const uint32_t* ids = nullptr;
+    const uint32_t* counts = nullptr;
+    int64_t id_stride = 0;
+    int32_t max_ids = 0;
 };
-// Fills wg_base/splits/pps from row/pos; returns the total work-group count.
-int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b);
+// Fills wg_base/splits/pps from row/pos; returns the total work-group count.  sel_groups > 0:
+// every entry is planned for that many groups of four selected blocks instead of its pages.
+int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b, int32_t sel_groups = 0);
 hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, const AttnArgs& a,
                               hipStream_t stream);
 // heads one wave carries for a given q-heads-per-kv-head group

@@ -48,6 +48,12 @@ struct AttnKernelParams {
     int32_t max_pages_per_seq;
     int32_t n_kv, n_q, group, n_hc;
     float scale_log2e;
+    // selection lists (decode_attn_kernel<..., true> only): entry e attends the 4-cell blocks
+    // ids[e * id_stride + 0 .. min(counts[e], max_ids))
+    const uint32_t* ids;
+    const uint32_t* counts;
+    int64_t id_stride;
+    int32_t max_ids;
 };
 
 __device__ __forceinline__ void wave_lds_sync() {
@@ -151,10 +157,11 @@ struct RowBuf;
 template <>
 struct RowBuf<kRowF16> {
     half8 r[8];
-    // page = first byte of this (page, kv head)'s 16 rows
-    __device__ __forceinline__ void load(const uint8_t* page, int i, int lane) {
+    // base = first byte of a run of rows of one kv head; the lane's row of pair `ia` in that
+    // run goes to register group i
+    __device__ __forceinline__ void load(const uint8_t* base, int ia, int i, int lane) {
         r[i] = __builtin_bit_cast(
-            half8, __builtin_nontemporal_load(reinterpret_cast<const v4u*>(page) + i * 64 + lane));
+            half8, __builtin_nontemporal_load(reinterpret_cast<const v4u*>(base) + ia * 64 + lane));
     }
     __device__ __forceinline__ float elem(int i, int j) const { return widen(r[i][j]); }
     static constexpr bool kScaled = false;
@@ -175,9 +182,9 @@ template <>
 struct RowBuf<kRowQ8> {
     v2u code[8];
     float sc[8];
-    __device__ __forceinline__ void load(const uint8_t* page, int i, int lane) {
-        const int row = 2 * i + (lane >> 5), dl = lane & 31;
-        const uint8_t* blk = page + row * row_bytes_of(kRowQ8) + (dl >> 2) * 36;
+    __device__ __forceinline__ void load(const uint8_t* base, int ia, int i, int lane) {
+        const int row = 2 * ia + (lane >> 5), dl = lane & 31;
+        const uint8_t* blk = base + row * row_bytes_of(kRowQ8) + (dl >> 2) * 36;
         sc[i] = __builtin_nontemporal_load(reinterpret_cast<const float*>(blk));
         const unsigned* c = reinterpret_cast<const unsigned*>(blk + 4 + (dl & 3) * 8);
         code[i].x = __builtin_nontemporal_load(c);
@@ -196,9 +203,9 @@ template <>
 struct RowBuf<kRowI8H> {
     v2u code[8];
     unsigned short sc[8];
-    __device__ __forceinline__ void load(const uint8_t* page, int i, int lane) {
-        const int row = 2 * i + (lane >> 5), dl = lane & 31;
-        const uint8_t* rp = page + row * row_bytes_of(kRowI8H);
+    __device__ __forceinline__ void load(const uint8_t* base, int ia, int i, int lane) {
+        const int row = 2 * ia + (lane >> 5), dl = lane & 31;
+        const uint8_t* rp = base + row * row_bytes_of(kRowI8H);
         code[i] = __builtin_nontemporal_load(reinterpret_cast<const v2u*>(rp + dl * 8));
         sc[i] = __builtin_nontemporal_load(
             reinterpret_cast<const unsigned short*>(rp + kHd + (dl >> 2) * 2));
@@ -217,8 +224,26 @@ struct RowBuf<kRowI8H> {
     }
 };
 
-// HG = q heads carried by one wave (8 or 4); KENC / VENC = row encodings of the K and V pools.
-template <int HG, int KENC, int VENC>
+// Where the 16 rows of one loop iteration live.  Dense: one page (one run of 16 rows).
+// Selection: four selected blocks of four cells (crates/breccia-kernels/src/qsa/cpu.rs:
+// 248-257: block b covers cells 4b..4b+3), each a run of 4 rows inside some page; `id` keeps
+// the block ids for the causal test, 0xffffffff for a slot past the end of the list.
+template <bool SEL>
+struct RowRuns {
+    const uint8_t* k[SEL ? 4 : 1];
+    const uint8_t* v[SEL ? 4 : 1];
+    uint32_t id[SEL ? 4 : 1];
+};
+
+// cell 4*id + r of a selected block is attended iff it is not past the query's position
+// (shaders/qsa_attn_scores_small.comp: `cell > pos` is a dead slot)
+__device__ __forceinline__ bool block_cell_live(uint32_t id, int r, int pos) {
+    return id < 0x40000000u && id * 4u + (uint32_t)r <= (uint32_t)pos;
+}
+
+// HG = q heads carried by one wave (8 or 4); KENC / VENC = row encodings of the K and V pools;
+// SEL = attend the cells of a per-entry list of selected blocks instead of every cell 0..=pos.
+template <int HG, int KENC, int VENC, bool SEL>
 __global__ __launch_bounds__(kBlock, HG == 8 ? 2 : 3) void decode_attn_kernel(const AttnKernelParams P) {
     constexpr int HQ = HG / 4;           // float4 groups of heads
     constexpr int NB = HG / 4;           // score batches per page (8 float4 slots each)
@@ -249,14 +274,23 @@ __global__ __launch_bounds__(kBlock, HG == 8 ? 2 : 3) void decode_attn_kernel(co
     const int kvh = rem - split * P.n_kv;
     const int wg = P.b.wg_base[e] + hc * splits * P.n_kv + rem;
     const int pos = P.b.pos[e];
-    const int n_pages = pos / kPage + 1;
+    // Block-table row (and selection list) through the constant address space: neither is
+    // written while this kernel runs, and constant-space loads at uniform addresses are always
+    // scalar loads.
+    typedef const __attribute__((address_space(4))) int32_t* table_ptr;
+    typedef const __attribute__((address_space(4))) uint32_t* list_ptr;
+    const table_ptr bt = (table_ptr)(uintptr_t)(P.tables + (size_t)P.b.row[e] * (size_t)P.max_pages_per_seq);
+    uint32_t n_sel = 0;
+    list_ptr sel = nullptr;
+    if constexpr (SEL) {
+        n_sel = min(((list_ptr)(uintptr_t)P.counts)[e], (uint32_t)P.max_ids);
+        sel = (list_ptr)(uintptr_t)(P.ids + (size_t)e * (size_t)P.id_stride);
+    }
+    // loop iterations of this entry: pages, or groups of four selected blocks
+    const int n_pages = SEL ? (int)((n_sel + 3u) >> 2) : pos / kPage + 1;
     const int pps = P.b.pps[e];
     const int pg0 = split * pps;
     const int pg1 = min(pg0 + pps, n_pages);
-    // Block-table row through the constant address space: the table is not written while this
-    // kernel runs, and constant-space loads at uniform addresses are always scalar loads.
-    typedef const __attribute__((address_space(4))) int32_t* table_ptr;
-    const table_ptr bt = (table_ptr)(uintptr_t)(P.tables + (size_t)P.b.row[e] * (size_t)P.max_pages_per_seq);
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
@@ -271,17 +305,47 @@ __global__ __launch_bounds__(kBlock, HG == 8 ? 2 : 3) void decode_attn_kernel(co
     // K and V rows of a page sit in registers.  Every register group is refilled with the
     // next page's row right after its last use, so each load has a whole page of work in
     // front of it and 16 row loads per wave stay in flight.
+    // Row runs of iteration g.  A selected block id is clamped to the blocks at or below `pos`
+    // for addressing (so that no list content can reach outside the sequence's pages); its
+    // cells past `pos`, and slots past the end of the list, are masked where they are used.
+    const auto locate = [&](int g, RowRuns<SEL>& rr) {
+        if constexpr (SEL) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t at = (uint32_t)g * 4u + (uint32_t)j;
+                const uint32_t id = sel[min(at, n_sel - 1u)];
+                rr.id[j] = at < n_sel ? id : 0xffffffffu;
+                const uint32_t idc = min(id, (uint32_t)pos >> 2);
+                const int32_t phys = bt[idc >> 2];
+                const size_t in_page = (size_t)(idc & 3u) * 4u;
+                rr.k[j] = P.kpool + (size_t)phys * k_page + k_head_off + in_page * row_bytes_of(KENC);
+                rr.v[j] = P.vpool + (size_t)phys * v_page + v_head_off + in_page * row_bytes_of(VENC);
+            }
+        } else {
+            const int32_t phys = bt[g];
+            rr.k[0] = P.kpool + (size_t)phys * k_page + k_head_off;
+            rr.v[0] = P.vpool + (size_t)phys * v_page + v_head_off;
+            rr.id[0] = 0;
+        }
+    };
+    // row pair i of an iteration: run i/2, pair i%2 of that run (selection), or pair i of the page
+    const auto load_k = [&](RowBuf<KENC>& buf, const RowRuns<SEL>& rr, int i) {
+        if constexpr (SEL) buf.load(rr.k[i >> 1], i & 1, i, lane); else buf.load(rr.k[0], i, i, lane);
+    };
+    const auto load_v = [&](RowBuf<VENC>& buf, const RowRuns<SEL>& rr, int i) {
+        if constexpr (SEL) buf.load(rr.v[i >> 1], i & 1, i, lane); else buf.load(rr.v[0], i, i, lane);
+    };
+
     int pg = pg0 + wave;
     RowBuf<KENC> kk;
     RowBuf<VENC> vv;
+    RowRuns<SEL> cur{};
     if (pg < pg1) {
-        const int32_t phys = bt[pg];
-        const uint8_t* kp = P.kpool + (size_t)phys * k_page + k_head_off;
-        const uint8_t* vp = P.vpool + (size_t)phys * v_page + v_head_off;
+        locate(pg, cur);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) kk.load(kp, i, lane);
+        for (int i = 0; i < 8; ++i) load_k(kk, cur, i);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) vv.load(vp, i, lane);
+        for (int i = 0; i < 8; ++i) load_v(vv, cur, i);
     }
 
     __builtin_amdgcn_sched_barrier(0);
@@ -348,9 +412,8 @@ __global__ __launch_bounds__(kBlock, HG == 8 ? 2 : 3) void decode_attn_kernel(co
         // page): one straight-line load sequence lets the compiler count outstanding loads
         // exactly instead of draining them at a control-flow join.
         const int pg_next = pg + kWaves;
-        const int32_t phys_next = bt[min(pg_next, pg1 - 1)];
-        const uint8_t* kp_next = P.kpool + (size_t)phys_next * k_page + k_head_off;
-        const uint8_t* vp_next = P.vpool + (size_t)phys_next * v_page + v_head_off;
+        RowRuns<SEL> nxt;
+        locate(min(pg_next, pg1 - 1), nxt);
 
         // ---- scores: partial dots -> LDS transpose -> one (row, head) per lane ------
         float sval[NB];
@@ -378,7 +441,7 @@ __global__ __launch_bounds__(kBlock, HG == 8 ? 2 : 3) void decode_attn_kernel(co
 #pragma unroll
                     for (int h = 0; h < HG; ++h) s[h] *= ks;
                 }
-                kk.load(kp_next, i, lane);
+                load_k(kk, nxt, i);
 #pragma unroll
                 for (int hq = 0; hq < HQ; ++hq) {
                     const int slot = (HG == 8) ? (ip * 2 + hq) : i;
@@ -412,7 +475,14 @@ __global__ __launch_bounds__(kBlock, HG == 8 ? 2 : 3) void decode_attn_kernel(co
         for (int bch = 0; bch < NB; ++bch) {
             const int i = (HG == 8) ? (bch * RP + (lane >> 4)) : rslot;
             rowv[bch] = 2 * i + rhw;
-            const bool live = pg * kPage + rowv[bch] <= pos;
+            bool live;
+            if constexpr (SEL) {
+                const int j = rowv[bch] >> 2;
+                const uint32_t id = j == 0 ? cur.id[0] : j == 1 ? cur.id[1] : j == 2 ? cur.id[2] : cur.id[3];
+                live = block_cell_live(id, rowv[bch] & 3, pos);
+            } else {
+                live = pg * kPage + rowv[bch] <= pos;
+            }
             sv[bch] = live ? sval[bch] * P.scale_log2e : -INFINITY;
             pm = fmaxf(pm, sv[bch]);
         }
@@ -443,8 +513,17 @@ __global__ __launch_bounds__(kBlock, HG == 8 ? 2 : 3) void decode_attn_kernel(co
                 for (int j = 0; j < 8; ++j) o[h][j] *= a;
             }
         }
-        if (pg == n_pages - 1) {
-            // Rows past `pos` may hold anything (even NaN): make them exact zeros.
+        // Rows that are not attended may hold anything (even NaN): make them exact zeros.
+        if constexpr (SEL) {
+            bool all_live = true;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) all_live = all_live && block_cell_live(cur.id[j], 3, pos);
+            if (!all_live) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    if (!block_cell_live(cur.id[i >> 1], 2 * (i & 1) + hw, pos)) vv.zero(i);
+            }
+        } else if (pg == n_pages - 1) {
 #pragma unroll
             for (int i = 0; i < 8; ++i)
                 if (pg * kPage + 2 * i + hw > pos) vv.zero(i);
@@ -471,11 +550,12 @@ __global__ __launch_bounds__(kBlock, HG == 8 ? 2 : 3) void decode_attn_kernel(co
 #pragma unroll
                 for (int h = 0; h < HG; ++h) o[h][j] = fmaf(vj, pr[h], o[h][j]);
             }
-            vv.load(vp_next, i, lane);
+            load_v(vv, nxt, i);
         }
         wave_lds_sync();
 
         pg = pg_next;
+        cur = nxt;
     }
 
     __builtin_amdgcn_s_setprio(0);
@@ -653,14 +733,17 @@ __global__ __launch_bounds__(kHd * kMergeGroups) void decode_attn_merge_kernel(c
 // Heads one work-group carries for a given q-heads-per-kv-head group.
 int32_t attn_heads_per_wave(int32_t group) { return group % 8 == 0 ? 8 : 4; }
 
-int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b) {
+int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b, int32_t sel_groups) {
     const int32_t n_kv = p->g.n_kv;
     const int32_t group = n_q_head / n_kv;
     const int32_t hg = attn_heads_per_wave(group);
     const int32_t n_hc = (group + hg - 1) / hg;
     const int64_t per_page = (int64_t)n_kv * n_hc;
     int64_t total_pages = 0;
-    for (int i = 0; i < b.n; ++i) total_pages += b.pos[i] / kPage + 1;
+    // loop iterations of an entry: its pages, or (selection lists, whose true lengths only the
+    // device knows) the most groups of four blocks a list can hold
+    const auto iters = [&](int i) -> int64_t { return sel_groups > 0 ? sel_groups : b.pos[i] / kPage + 1; };
+    for (int i = 0; i < b.n; ++i) total_pages += iters(i);
     // All work-groups should be resident at once (one generation): a handful of left-over
     // work-groups would run alone after the rest and double the kernel's time.  `resident`
     // follows from the register budget of the kernel variant that will run.
@@ -673,7 +756,7 @@ int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b) {
     for (;;) {
         int64_t total = 0;
         for (int i = 0; i < b.n; ++i) {
-            const int64_t pages = b.pos[i] / kPage + 1;
+            const int64_t pages = iters(i);
             const int64_t splits = (pages + pps - 1) / pps;
             // even the ranges out inside the entry, keeping whole groups of kWaves pages
             int64_t each = (pages + splits - 1) / splits;
@@ -708,13 +791,24 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
     kp.group = group;
     kp.n_hc = (group + hg - 1) / hg;
     kp.scale_log2e = a.scale * kLog2e;
+    kp.ids = a.ids;
+    kp.counts = a.counts;
+    kp.id_stride = a.id_stride;
+    kp.max_ids = a.max_ids;
+    const bool sel = a.ids != nullptr;
     const int32_t total = b.wg_base[b.n];
     const int32_t n_units = total / kp.n_hc;
     const int32_t grid = (n_units + 7) / 8 * 8 * kp.n_hc;
     {
         StageScope timed(p, BKV_STAGE_ATTN_SPLIT, stream);
         const int layout = p->g.layout;
-#define BKV_LAUNCH(HGV, KE, VE) decode_attn_kernel<HGV, KE, VE><<<grid, kBlock, 0, stream>>>(kp)
+#define BKV_LAUNCH(HGV, KE, VE)                                                  \
+    do {                                                                        \
+        if (sel)                                                                \
+            decode_attn_kernel<HGV, KE, VE, true><<<grid, kBlock, 0, stream>>>(kp);  \
+        else                                                                    \
+            decode_attn_kernel<HGV, KE, VE, false><<<grid, kBlock, 0, stream>>>(kp); \
+    } while (0)
         if (layout == BKV_LAYOUT_F16) {
             if (hg == 8) BKV_LAUNCH(8, kRowF16, kRowF16); else BKV_LAUNCH(4, kRowF16, kRowF16);
         } else if (layout == BKV_LAYOUT_Q8V) {

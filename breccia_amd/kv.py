@@ -295,6 +295,18 @@ class Pool:
                                   _ptr(gate_dev), gate_seq_stride, gate_head_stride, scale,
                                   _ptr(out_dev), _sh(stream)))
 
+    def decode_attn_select(self, layer: int, seqs, pos, n_q_head: int, q_dev, out_dev, scale: float,
+                           ids_dev, id_stride: int, counts_dev, max_ids: int, gate_dev=None,
+                           gate_seq_stride: int = 0, gate_head_stride: int = 0, stream=None) -> None:
+        """Attention over per-entry lists of selected 4-cell blocks (device u32 ids / counts)."""
+        seqs, ps = _i32(seqs)
+        pos, pp = _i64(pos)
+        assert seqs.size == pos.size
+        check(lib.bkv_decode_attn_select(self.handle, layer, seqs.size, ps, pp, n_q_head, _ptr(q_dev),
+                                         _ptr(gate_dev), gate_seq_stride, gate_head_stride, scale,
+                                         _ptr(ids_dev), id_stride, _ptr(counts_dev), max_ids,
+                                         _ptr(out_dev), _sh(stream)))
+
     def page_copy(self, pairs, stream=None) -> None:
         """pairs: iterable of (src, dst), or an int32 array of shape [n, 2]."""
         arr = np.ascontiguousarray(np.asarray(list(pairs) if not isinstance(pairs, np.ndarray)

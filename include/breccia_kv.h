@@ -200,6 +200,24 @@ bkv_status bkv_decode_attn(bkv_pool *pool, int32_t layer, int32_t n, const int32
                            const float *gate_dev, int64_t gate_seq_stride,
                            int64_t gate_head_stride, float scale, float *out_dev, void *stream);
 
+/* The same attention over a selection list instead of every cell: the reference's real
+ * long-context form (Qsa::attend / Qsa::apply read ws.ids [T, max_ids] and ws.counts [T],
+ * qsa/mod.rs:1382-1462; shaders/qsa_attn_scores_small.comp; oracle qsa/cpu.rs:197-257).
+ * Entry i attends the cells 4*b .. 4*b+3 of every block id b in
+ *   ids_dev[i*id_stride + 0 .. min(counts_dev[i], max_ids)),
+ * keeping only cells <= pos[i]; a block listed twice counts twice (as in the oracle); an
+ * empty list gives a zero output row.  ids and counts are device u32 buffers (what a
+ * top-k kernel leaves behind): their contents are never trusted for addressing -- a block
+ * id is clamped to the sequence's blocks at or below pos[i] before any address is formed,
+ * and its cells are masked by the causal test -- so no list content can fault.
+ * Work is planned for max_ids blocks per entry, the bound the host knows. */
+bkv_status bkv_decode_attn_select(bkv_pool *pool, int32_t layer, int32_t n, const int32_t *seqs,
+                                  const int64_t *pos, int32_t n_q_head, const float *q_dev,
+                                  const float *gate_dev, int64_t gate_seq_stride,
+                                  int64_t gate_head_stride, float scale, const uint32_t *ids_dev,
+                                  int64_t id_stride, const uint32_t *counts_dev, int32_t max_ids,
+                                  float *out_dev, void *stream);
+
 /* Copy-on-write page copy: for every pair and every layer, K and V bytes of page
  * `src` -> page `dst`.  No reference implementation (nearest: dispatch_batch.rs:
  * 1130-1150 record_copy).  Pairs are host memory; dst pages must be distinct. */
