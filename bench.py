@@ -428,7 +428,27 @@ def bench_select(stream) -> dict:
         "algorithmic_bytes": b, "us_per_layer": round(us, 2), "attn_split_us": round(split_us, 2),
         "attn_merge_us": round(ms_merge / max(n_merge, 1) * 1e3, 2),
         "GBps": round(b / us / 1e3, 1), "split_GBps": round(b / split_us / 1e3, 1)}}
-    for x in (idd, cd, q, out):
+    # the selection itself: indexer score of every pooled block (4 heads x 128) + exact top-512
+    n_blocks = [c // 4 for c in ctx]
+    pooled = [DeviceBuffer.from_numpy(rng.standard_normal((nb, 128), dtype=np.float32)) for nb in n_blocks]
+    iq = DeviceBuffer.from_numpy(rng.standard_normal((n_seqs, 4, 128), dtype=np.float32))
+
+    def run_sel(n):
+        for _ in range(n):
+            pool.select_blocks(pos, iq, pooled, n_blocks, 4, 128, 512, idd, max_ids, cd, max_ids, stream=stream)
+
+    run_sel(5)
+    stream.sync()
+    e0, e1 = Event(), Event()
+    e0.record(stream)
+    run_sel(50)
+    e1.record(stream)
+    stream.sync()
+    res["select_blocks_batch8"] = {"blocks_scored": sum(n_blocks), "kept_per_list": 512,
+                                   "us": round(e0.elapsed_ms(e1) / 50 * 1e3, 2)}
+    e0.close()
+    e1.close()
+    for x in [idd, cd, q, out, iq] + pooled:
         x.free()
     pool.destroy()
     return res

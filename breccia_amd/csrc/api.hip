@@ -166,6 +166,7 @@ static void destroy_device_side(bkv_pool* p) {
     if (p->table_dev) (void)hipFree(p->table_dev);
     if (p->part_o) (void)hipFree(p->part_o);
     if (p->part_ml) (void)hipFree(p->part_ml);
+    if (p->sel_scores) (void)hipFree(p->sel_scores);
     if (p->ring.host) (void)hipHostFree(p->ring.host);
     if (p->ring.dev) (void)hipFree(p->ring.dev);
     for (int i = 0; i < ParamRing::kSlots; ++i)
@@ -673,6 +674,103 @@ bkv_status bkv_decode_attn_select(bkv_pool* p, int32_t layer, int32_t n, const i
     return decode_attn_common(p, layer, n, seqs, pos, n_q_head, q_dev, gate_dev, gate_seq_stride,
                               gate_head_stride, scale, ids_dev, id_stride, counts_dev, max_ids, true,
                               out_dev, stream);
+}
+
+// ---- block selection ---------------------------------------------------------------------
+static bkv_status select_common_checks(bkv_pool* p, const char* what, int32_t n, const int64_t* pos,
+                                       int32_t topk_blocks, const uint32_t* ids_dev, int64_t id_stride,
+                                       const uint32_t* counts_dev, int32_t max_ids) {
+    if (!p) return fail(BKV_ERR_INVALID, std::string(what) + ": NULL pool");
+    if (n < 0 || n > BKV_MAX_BATCH)
+        return fail(BKV_ERR_INVALID, std::string(what) + sfmt(": %lld lists in one call; the limit is "
+                                                              "%lld", n, BKV_MAX_BATCH));
+    if (n > 0 && !pos) return fail(BKV_ERR_INVALID, std::string(what) + ": NULL pos");
+    if (topk_blocks <= 0 || topk_blocks > select_max_topk())
+        return fail(BKV_ERR_INVALID, std::string(what) + sfmt(": topk_blocks %lld is outside 1..%lld",
+                                                              topk_blocks, select_max_topk()));
+    if (max_ids <= 0 || id_stride < max_ids)
+        return fail(BKV_ERR_INVALID, std::string(what) + sfmt(": max_ids %lld / id_stride %lld (need "
+                                                              "0 < max_ids <= id_stride)", max_ids,
+                                                              id_stride));
+    for (int i = 0; i < n; ++i)
+        if (pos[i] < 0 || pos[i] > 0x7fffffff)
+            return fail(BKV_ERR_RANGE, std::string(what) + sfmt(": position %lld of list %lld", pos[i], i));
+    bkv_status st = need_device(p);
+    if (st != BKV_OK) return st;
+    if (n > 0 && (!ids_dev || !counts_dev || ((uintptr_t)ids_dev & 3u) || ((uintptr_t)counts_dev & 3u)))
+        return fail(BKV_ERR_INVALID, std::string(what) + ": ids/counts device pointers must be "
+                                                         "non-NULL and 4-byte aligned");
+    return BKV_OK;
+}
+
+bkv_status bkv_topk_blocks(bkv_pool* p, int32_t n, const int64_t* pos, const float* scores_dev,
+                           int32_t n_blocks, int32_t topk_blocks, int32_t dense, uint32_t* ids_dev,
+                           int64_t id_stride, uint32_t* counts_dev, int32_t max_ids, void* stream) {
+    bkv_status st = select_common_checks(p, "topk_blocks", n, pos, topk_blocks, ids_dev, id_stride,
+                                         counts_dev, max_ids);
+    if (st != BKV_OK) return st;
+    if (n_blocks < 0) return fail(BKV_ERR_INVALID, sfmt("topk_blocks: n_blocks %lld", n_blocks));
+    if (n == 0) return BKV_OK;
+    if (!dense && n_blocks > 0 && (!scores_dev || ((uintptr_t)scores_dev & 3u)))
+        return fail(BKV_ERR_INVALID, "topk_blocks: scores device pointer must be non-NULL and "
+                                     "4-byte aligned");
+    SelectBatch b{};
+    b.n = n;
+    for (int i = 0; i < n; ++i) {
+        b.pos[i] = (int32_t)pos[i];
+        b.n_blocks[i] = n_blocks;
+    }
+    BKV_HIP(launch_topk_blocks(b, scores_dev, false, n_blocks, topk_blocks, 4, dense != 0, ids_dev,
+                               id_stride, counts_dev, max_ids, S(stream)));
+    return BKV_OK;
+}
+
+bkv_status bkv_select_blocks(bkv_pool* p, int32_t n, const int64_t* pos, const float* idx_q_dev,
+                             const float* const* pooled_dev, const int32_t* n_blocks,
+                             int32_t idx_n_head, int32_t idx_dim, int32_t topk_blocks,
+                             uint32_t* ids_dev, int64_t id_stride, uint32_t* counts_dev,
+                             int32_t max_ids, void* stream) {
+    bkv_status st = select_common_checks(p, "select_blocks", n, pos, topk_blocks, ids_dev, id_stride,
+                                         counts_dev, max_ids);
+    if (st != BKV_OK) return st;
+    if (idx_n_head <= 0 || idx_n_head > select_max_idx_head() || idx_dim <= 0 ||
+        idx_dim > select_max_idx_dim())
+        return fail(BKV_ERR_INVALID, sfmt("select_blocks: %lld indexer heads of %lld values (limits "
+                                          "%lld, %lld)", idx_n_head, idx_dim, select_max_idx_head(),
+                                          select_max_idx_dim()));
+    if (n == 0) return BKV_OK;
+    if (!n_blocks || !pooled_dev || !idx_q_dev || ((uintptr_t)idx_q_dev & 3u))
+        return fail(BKV_ERR_INVALID, "select_blocks: NULL n_blocks / pooled / idx_q");
+    SelectBatch b{};
+    b.n = n;
+    int32_t max_blocks = 0;
+    for (int i = 0; i < n; ++i) {
+        if (n_blocks[i] < 0 || (n_blocks[i] > 0 && (!pooled_dev[i] || ((uintptr_t)pooled_dev[i] & 3u))))
+            return fail(BKV_ERR_INVALID, sfmt("select_blocks: list %lld has %lld blocks and a NULL or "
+                                              "misaligned pooled pointer", i, n_blocks[i]));
+        b.pos[i] = (int32_t)pos[i];
+        b.n_blocks[i] = n_blocks[i];
+        b.pooled[i] = pooled_dev[i];
+        max_blocks = std::max(max_blocks, n_blocks[i]);
+    }
+    const uint64_t stride = ((uint64_t)std::max(max_blocks, 1) + 63u) & ~(uint64_t)63u;
+    const uint64_t need = stride * (uint64_t)n;
+    if (need > p->sel_scores_cap) {
+        // grow the score workspace; earlier launches may still read the old one
+        BKV_HIP(hipDeviceSynchronize());
+        if (p->sel_scores) BKV_HIP(hipFree(p->sel_scores));
+        p->sel_scores = nullptr;
+        p->sel_scores_cap = 0;
+        const uint64_t cap = std::max<uint64_t>(need, (uint64_t)BKV_MAX_BATCH * 8192u);
+        BKV_HIP(hipMalloc(reinterpret_cast<void**>(&p->sel_scores), cap * sizeof(double)));
+        p->sel_scores_cap = cap;
+    }
+    if (max_blocks > 0)
+        BKV_HIP(launch_idx_score(b, idx_q_dev, idx_n_head, idx_dim, 4, p->sel_scores, (int64_t)stride,
+                                 max_blocks, S(stream)));
+    BKV_HIP(launch_topk_blocks(b, p->sel_scores, true, (int64_t)stride, topk_blocks, 4, false, ids_dev,
+                               id_stride, counts_dev, max_ids, S(stream)));
+    return BKV_OK;
 }
 
 // ---- page copy -------------------------------------------------------------------------

@@ -86,6 +86,9 @@ struct bkv_pool {
     float* part_o = nullptr;
     float* part_ml = nullptr;
     int32_t max_wgs = 0;
+    // block selection: f64 indexer scores [entry][block], grown on demand
+    double* sel_scores = nullptr;
+    uint64_t sel_scores_cap = 0;  // doubles
 
     bkv::ParamRing ring;
     bkv::StageTimer timer;
@@ -134,6 +137,24 @@ hipError_t launch_append_kprep(const bkv_pool* p, int32_t layer, const AppendBat
                                const float* k, const float* v, const float* gamma, float eps,
                                const float* table, int32_t n_rot, int32_t max_pos,
                                const int32_t* positions, hipStream_t stream);
+
+// Block selection (select.hip): one entry per (token) list.
+struct SelectBatch {
+    int32_t n;
+    int32_t pos[BKV_MAX_BATCH];       // query position
+    int32_t n_blocks[BKV_MAX_BATCH];  // pooled / scored blocks of the entry
+    const float* pooled[BKV_MAX_BATCH];  // [n_blocks][idx_dim] (score kernel only)
+};
+hipError_t launch_idx_score(const SelectBatch& b, const float* q, int32_t idx_n_head, int32_t idx_dim,
+                            int32_t idx_block, double* scores, int64_t score_stride, int32_t max_blocks,
+                            hipStream_t stream);
+hipError_t launch_topk_blocks(const SelectBatch& b, const void* scores, bool scores_f64,
+                              int64_t score_stride, int32_t topk_blocks, int32_t idx_block, bool dense,
+                              uint32_t* ids, int64_t id_stride, uint32_t* counts, int32_t max_ids,
+                              hipStream_t stream);
+int32_t select_max_topk();
+int32_t select_max_idx_head();
+int32_t select_max_idx_dim();
 
 struct AttnBatch {
     int32_t n;

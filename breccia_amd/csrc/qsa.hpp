@@ -15,7 +15,8 @@
 // fused kernel: the score matrix is never materialised, so attend() only validates and
 // apply() launches the split-K kernel plus the merge (which applies sigmoid(gate) read in
 // place from q_full at h*2*head_dim + head_dim + d, as shaders/qsa_attn_apply.comp does);
-// selection is the dense one (every cell 0..=pos), ids/counts are not consulted.
+// apply() attends the lists in ws.ids / ws.counts once select() or topk_dense() has filled
+// them, and every cell 0..=pos otherwise.
 #pragma once
 
 #include <cstddef>
@@ -33,6 +34,10 @@ constexpr int MODEL_N_HEAD = 24;      // qsa/mod.rs:69
 constexpr int MODEL_N_KV_HEAD = 2;    // qsa/mod.rs:71
 constexpr int MODEL_HEAD_DIM = 256;   // qsa/mod.rs:73
 constexpr int PAGE_CELLS = 16;        // qsa/mod.rs:116
+constexpr int IDX_N_HEAD = 4;         // qsa/mod.rs:77
+constexpr int IDX_DIM = 128;          // qsa/mod.rs:79
+constexpr int IDX_BLOCK = 4;          // qsa/mod.rs:81
+constexpr int IDX_TOPK_BLOCKS = 512;  // qsa/mod.rs:85 (IDX_TOP_K 2048 cells / IDX_BLOCK)
 constexpr int MODEL_N_ROT = 64;       // ops/mod.rs:454
 constexpr float MODEL_RMS_EPS = 1e-6f;  // ops/mod.rs:316
 
@@ -114,6 +119,14 @@ struct QsaWorkspace {
     float* k_cur = nullptr;     // [T, n_kv_head, head_dim]
     float* v_cur = nullptr;     // [T, n_kv_head, head_dim]
     float* attn_out = nullptr;  // [T, n_head, head_dim]
+    // block selection (qsa/mod.rs:604-660): indexer queries in, id lists out
+    float* idx_q = nullptr;     // [T, IDX_N_HEAD, IDX_DIM]
+    uint32_t* ids = nullptr;    // [T, max_ids] selected block ids
+    uint32_t* counts = nullptr; // [T]
+    size_t n_blocks = 0;        // completed (pooled) blocks the selection ranges over
+    size_t max_ids = 0;         // topk_blocks + 1
+    size_t topk_blocks = 0;
+    bool selected = false;      // a selection call has filled ids / counts
 };
 
 class Qsa {
@@ -121,10 +134,18 @@ public:
     explicit Qsa(int n_head = MODEL_N_HEAD, void* stream = nullptr) : n_head_(n_head), stream_(stream) {}
 
     // tokens == 0 is an error (qsa/mod.rs:929-931).
-    QsaWorkspace workspace(size_t tokens, size_t /*n_kv_after*/) const {
+    // n_kv_after = cells the cache holds once this call's tokens are appended; it sizes the
+    // selection (n_blocks = completed 4-cell blocks, qsa/mod.rs:928-1048).
+    QsaWorkspace workspace(size_t tokens, size_t n_kv_after) const {
         if (tokens == 0) throw Error(BKV_ERR_INVALID, "a qsa workspace needs tokens > 0");
         QsaWorkspace ws;
         ws.tokens = tokens;
+        ws.n_blocks = n_kv_after / IDX_BLOCK;
+        ws.topk_blocks = IDX_TOPK_BLOCKS;
+        ws.max_ids = ws.topk_blocks + 1;
+        check(bkv_dev_alloc(tokens * IDX_N_HEAD * IDX_DIM * 4, (void**)&ws.idx_q));
+        check(bkv_dev_alloc(tokens * ws.max_ids * 4, (void**)&ws.ids));
+        check(bkv_dev_alloc(tokens * 4, (void**)&ws.counts));
         const size_t hd = MODEL_HEAD_DIM;
         check(bkv_dev_alloc(tokens * n_head_ * 2 * hd * 4, (void**)&ws.q_full));
         check(bkv_dev_alloc(tokens * n_head_ * hd * 4, (void**)&ws.q));
@@ -134,10 +155,13 @@ public:
         return ws;
     }
     void release(QsaWorkspace& ws) const {
-        for (float** p : {&ws.q_full, &ws.q, &ws.k_cur, &ws.v_cur, &ws.attn_out}) {
+        for (float** p : {&ws.q_full, &ws.q, &ws.k_cur, &ws.v_cur, &ws.attn_out, &ws.idx_q}) {
             if (*p) check(bkv_dev_free(*p));
             *p = nullptr;
         }
+        if (ws.ids) check(bkv_dev_free(ws.ids));
+        if (ws.counts) check(bkv_dev_free(ws.counts));
+        ws.ids = ws.counts = nullptr;
     }
 
     // Append ws.tokens rows of ws.k_cur / ws.v_cur at cells pos0.. (qsa/mod.rs:1107-1131).
@@ -173,6 +197,31 @@ public:
                                MODEL_RMS_EPS, rope_table, MODEL_N_ROT, rope_max_pos, nullptr, stream_));
     }
 
+    // Qsa::idx_score + Qsa::topk (qsa/mod.rs:1234-1376): score ws.n_blocks pooled indexer keys
+    // (idx_pooled: device f32 [n_blocks, IDX_DIM], the sequence's QsaState::idx_pooled) against
+    // every token's ws.idx_q and leave the selected block ids in ws.ids / ws.counts.
+    void select(QsaWorkspace& ws, const float* idx_pooled, size_t pos0) const {
+        std::vector<int64_t> pos(ws.tokens);
+        std::vector<const float*> pooled(ws.tokens, idx_pooled);
+        std::vector<int32_t> nb(ws.tokens, (int32_t)ws.n_blocks);
+        for (size_t t = 0; t < ws.tokens; ++t) pos[t] = (int64_t)(pos0 + t);
+        check(bkv_select_blocks(pool_of_last_state_, (int32_t)ws.tokens, pos.data(), ws.idx_q, pooled.data(),
+                                nb.data(), IDX_N_HEAD, IDX_DIM, (int32_t)ws.topk_blocks, ws.ids,
+                                (int64_t)ws.max_ids, ws.counts, (int32_t)ws.max_ids, stream_));
+        ws.selected = true;
+    }
+    // Qsa::topk_dense (qsa/mod.rs:1363-1376): every visible block, ascending, no scores read.
+    void topk_dense(QsaWorkspace& ws, size_t pos0) const {
+        std::vector<int64_t> pos(ws.tokens);
+        for (size_t t = 0; t < ws.tokens; ++t) pos[t] = (int64_t)(pos0 + t);
+        check(bkv_topk_blocks(pool_of_last_state_, (int32_t)ws.tokens, pos.data(), nullptr,
+                              (int32_t)ws.n_blocks, (int32_t)ws.topk_blocks, 1, ws.ids, (int64_t)ws.max_ids,
+                              ws.counts, (int32_t)ws.max_ids, stream_));
+        ws.selected = true;
+    }
+    // The selection calls run on the library context of a cache: name it once.
+    void bind(const QsaState& state) { pool_of_last_state_ = state.pool; }
+
     // Range checks of the attention call; nothing is launched (no score matrix exists).
     void attend(const QsaState& state, const QsaWorkspace& ws, size_t pos0) const {
         if (pos0 + ws.tokens > state.capacity_cells)
@@ -191,6 +240,14 @@ public:
         std::vector<int64_t> pos(ws.tokens);
         for (size_t t = 0; t < ws.tokens; ++t) pos[t] = (int64_t)(pos0 + t);
         const int64_t hd = MODEL_HEAD_DIM;
+        if (ws.selected) {
+            // over the lists a selection call left in ws.ids / ws.counts, as the reference does
+            check(bkv_decode_attn_select(state.pool, 0, (int32_t)ws.tokens, seqs.data(), pos.data(), n_head_,
+                                         ws.q, ws.q_full + hd, (int64_t)n_head_ * 2 * hd, 2 * hd, 0.0625f,
+                                         ws.ids, (int64_t)ws.max_ids, ws.counts, (int32_t)ws.max_ids,
+                                         ws.attn_out, stream_));
+            return;
+        }
         check(bkv_decode_attn(state.pool, 0, (int32_t)ws.tokens, seqs.data(), pos.data(), n_head_, ws.q,
                               ws.q_full + hd, (int64_t)n_head_ * 2 * hd, 2 * hd, 0.0625f, ws.attn_out,
                               stream_));
@@ -199,6 +256,7 @@ public:
 private:
     int n_head_;
     void* stream_;
+    bkv_pool* pool_of_last_state_ = nullptr;
 };
 
 }  // namespace qsa

@@ -1,0 +1,429 @@
+// Block selection for the sparse attention path on gfx950: the indexer score of every
+// pooled block against a token's indexer queries, and the top-k over those scores that
+// leaves the id list attention consumes.  Replaces the reference's qsa_idx_score.comp and
+// its qsa_topk*.comp family (crates/breccia-kernels/src/qsa/mod.rs:1234-1376) and must
+// emit exactly the list of the CPU path (qsa/cpu.rs:93-152): descending score, ties to
+// the lower block, dead blocks never, the query's own block appended when missed.
+//
+// The list is only reproducible if the scores are: two blocks whose scores differ in the
+// last bits must come out in the CPU's order.  The score kernel therefore computes what
+// the CPU computes, operation for operation -- f64 products and sums in index order -- and
+// the selection works on those f64 scores.  The work is tiny next to attention (a 32k
+// context has 8192 blocks of 128 values).
+//
+// Top-k = one work-group per list: an 8-bit radix select finds the key of the k-th largest
+// score, the survivors (at most k) are compacted in index order, sorted by a bitonic network
+// in LDS and written out.  Everything is deterministic: no atomic decides an
+// order (the histogram counts are order-independent).
+#include <algorithm>
+
+#include "bkv_internal.hpp"
+
+namespace bkv {
+
+namespace {
+
+constexpr int kScoreTile = 64;    // blocks per work-group of the score kernel
+constexpr int kScoreThreads = 256;
+constexpr int kMaxIdxHead = 8;    // as shaders/qsa_idx_score.comp
+constexpr int kMaxIdxDim = 128;
+
+constexpr int kTopkThreads = 1024;
+constexpr int kMaxTopk = 2048;    // candidates the sort network holds in LDS
+
+struct ScoreParams {
+    SelectBatch b;
+    const float* q;      // [n][idx_n_head][idx_dim]
+    double* scores;      // [n][score_stride]
+    int64_t score_stride;
+    int32_t idx_n_head, idx_dim, idx_block;
+};
+
+// score[b] = (1/sqrt(idx_dim)) * sum_h relu(q_h . pooled_b), -inf for a block that starts
+// after the query's position (qsa/cpu.rs:93-123).
+__global__ __launch_bounds__(kScoreThreads) void idx_score_kernel(const ScoreParams P) {
+    __shared__ float pooled_s[kScoreTile * (kMaxIdxDim + 1)];
+    __shared__ float q_s[kMaxIdxHead * kMaxIdxDim];
+    __shared__ double part_s[kMaxIdxHead][kScoreTile];
+    const int e = blockIdx.y;
+    const int n_blocks = P.b.n_blocks[e];
+    const int b0 = (int)blockIdx.x * kScoreTile;
+    if (b0 >= n_blocks) return;
+    const int nb = min(kScoreTile, n_blocks - b0);
+    const int D = P.idx_dim, H = P.idx_n_head;
+    const int stride = D + 1;  // odd: lanes walking one column of 64 rows hit 64 banks
+    const int tid = threadIdx.x;
+    const float* pooled = P.b.pooled[e] + (size_t)b0 * D;
+    for (int i = tid; i < nb * D; i += kScoreThreads) pooled_s[(i / D) * stride + i % D] = pooled[i];
+    for (int i = tid; i < H * D; i += kScoreThreads) q_s[i] = P.q[(size_t)e * H * D + i];
+    __syncthreads();
+
+    const int b = tid % kScoreTile;
+    if (b < nb) {
+#pragma clang fp contract(off)
+        const double scale = 1.0 / sqrt((double)D);
+        for (int h = tid / kScoreTile; h < H; h += kScoreThreads / kScoreTile) {
+            double dot = 0.0;
+            for (int d = 0; d < D; ++d) dot += (double)q_s[h * D + d] * (double)pooled_s[b * stride + d];
+            part_s[h][b] = (dot > 0.0 ? dot : 0.0) * scale;
+        }
+    }
+    __syncthreads();
+    if (tid < nb) {
+#pragma clang fp contract(off)
+        double acc = 0.0;
+        for (int h = 0; h < H; ++h) acc += part_s[h][tid];
+        const int64_t first_cell = (int64_t)(b0 + tid) * P.idx_block;
+        P.scores[(size_t)e * P.score_stride + b0 + tid] =
+            first_cell > (int64_t)P.b.pos[e] ? -INFINITY : acc;
+    }
+}
+
+// ---- top-k ---------------------------------------------------------------------------
+// Keys: unsigned integers that order like the scores.  A score is dead (never selected)
+// unless it is greater than -1e29: that covers -inf, NaN and the reference shaders' own
+// dead marker -1e30 (shaders/qsa_topk.comp stops at the first best <= -1e29).  -0 is keyed
+// as +0 so that equal scores stay equal.  Live keys are never 0.
+__device__ __forceinline__ uint64_t score_key(double s) {
+    if (!(s > -1.0e29)) return 0;
+    if (s == 0.0) s = 0.0;
+    const uint64_t u = (uint64_t)__double_as_longlong(s);
+    return (u >> 63) ? ~u : (u | 0x8000000000000000ull);
+}
+__device__ __forceinline__ uint64_t score_key(float s) {
+    if (!(s > -1.0e29f)) return 0;
+    if (s == 0.0f) s = 0.0f;
+    const uint32_t u = __float_as_uint(s);
+    const uint32_t k = (u >> 31) ? ~u : (u | 0x80000000u);
+    return (uint64_t)k << 32;
+}
+template <typename T>
+struct KeyBits;
+template <>
+struct KeyBits<double> {
+    static constexpr int kLowShift = 0;
+};
+template <>
+struct KeyBits<float> {
+    static constexpr int kLowShift = 32;  // the low half of a float's key is zero
+};
+
+// Exclusive prefix sum of one int per thread over the work-group, in thread order.
+__device__ __forceinline__ int block_exclusive_scan(int v, int* wave_sums, int* total) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int inc = v;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const int t = __shfl_up(inc, off, 64);
+        if (lane >= off) inc += t;
+    }
+    __syncthreads();  // wave_sums may still be read from the previous scan
+    if (lane == 63) wave_sums[wave] = inc;
+    __syncthreads();
+    int before = 0, all = 0;
+    for (int w = 0; w < kTopkThreads / 64; ++w) {
+        const int s = wave_sums[w];
+        if (w < wave) before += s;
+        all += s;
+    }
+    *total = all;
+    return before + inc - v;
+}
+
+struct TopkParams {
+    SelectBatch b;
+    const void* scores;   // [n][score_stride] of T
+    int64_t score_stride;
+    uint32_t* ids;        // [n][id_stride]
+    int64_t id_stride;
+    uint32_t* counts;     // [n]
+    int32_t topk_blocks, max_ids, idx_block, dense;
+};
+
+// kRegKeys = keys a thread keeps in registers: 8 serves lists of up to 8192 blocks (a 32k
+// context), 32 up to 32768 (128k); longer lists re-read their scores on every pass.
+template <typename T, int kRegKeys>
+__global__ __launch_bounds__(kTopkThreads) void topk_blocks_kernel(const TopkParams P) {
+    __shared__ int hist[256];
+    __shared__ int wave_sums[kTopkThreads / 64];
+    __shared__ uint64_t cand_key[kMaxTopk];
+    __shared__ uint32_t cand_idx[kMaxTopk];
+    __shared__ uint64_t wave_min[kTopkThreads / 64], wave_max[kTopkThreads / 64];
+    __shared__ uint64_t sh_prefix;
+    __shared__ int sh_rem, sh_done;
+    __shared__ int sh_present;
+
+    const int e = blockIdx.x;
+    const int tid = threadIdx.x;
+    const int N = P.b.n_blocks[e];
+    const uint32_t own = (uint32_t)(P.b.pos[e] / P.idx_block);
+    uint32_t* ids = P.ids + (size_t)e * P.id_stride;
+
+    if (P.dense) {
+        // every visible block in ascending order, unscored (shaders/qsa_topk.comp dense branch,
+        // Qsa::topk_dense qsa/mod.rs:1363-1376)
+        uint32_t n = min(min((uint32_t)N, own + 1u), (uint32_t)P.max_ids);
+        for (uint32_t i = tid; i < n; i += kTopkThreads) ids[i] = i;
+        if (tid == 0) {
+            if (own >= (uint32_t)N && n < (uint32_t)P.max_ids) ids[n++] = own;
+            P.counts[e] = n;
+        }
+        return;
+    }
+
+    const T* sc = reinterpret_cast<const T*>(P.scores) + (size_t)e * P.score_stride;
+    // thread t owns the contiguous index range [lo, hi): compaction keeps index order
+    const int per = (N + kTopkThreads - 1) / kTopkThreads;
+    const int lo = min(tid * per, N), hi = min(lo + per, N);
+    const bool in_regs = per <= kRegKeys;
+    uint64_t rk[kRegKeys];
+#pragma unroll
+    for (int u = 0; u < kRegKeys; ++u) rk[u] = in_regs && lo + u < hi ? score_key(sc[lo + u]) : 0;
+    // f(index, key) for every element of this thread, in index order
+    const auto for_keys = [&](auto f) {
+        if (in_regs) {
+#pragma unroll
+            for (int u = 0; u < kRegKeys; ++u)
+                if (lo + u < hi) f(lo + u, rk[u]);
+        } else {
+            for (int i = lo; i < hi; ++i) f(i, score_key(sc[i]));
+        }
+    };
+
+    int live = 0;
+    for_keys([&](int, uint64_t k) { live += k != 0; });
+    int n_live;
+    block_exclusive_scan(live, wave_sums, &n_live);
+    const int want = min(min(min(N, P.topk_blocks), n_live), P.max_ids);
+
+    if (want > 0) {
+        // ---- radix select: a threshold that exactly `want` live keys pass ------------------
+        // All live keys agree on the bits above the highest bit in which the smallest and the
+        // largest differ (for scores of similar magnitude that is sign, exponent and more), so
+        // the digits start there: the first histogram is already well spread, and the LDS
+        // atomics do not pile up on one bin.
+        uint64_t kmin = ~0ull, kmax = 0;
+        for_keys([&](int, uint64_t k) {
+            if (k != 0) {
+                kmin = min(kmin, k);
+                kmax = max(kmax, k);
+            }
+        });
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            kmin = min(kmin, (uint64_t)__shfl_xor((unsigned long long)kmin, off, 64));
+            kmax = max(kmax, (uint64_t)__shfl_xor((unsigned long long)kmax, off, 64));
+        }
+        if ((tid & 63) == 0) {
+            wave_min[tid >> 6] = kmin;
+            wave_max[tid >> 6] = kmax;
+        }
+        if (tid == 0) sh_done = 0;
+        __syncthreads();
+        for (int w = 0; w < kTopkThreads / 64; ++w) {
+            kmin = min(kmin, wave_min[w]);
+            kmax = max(kmax, wave_max[w]);
+        }
+        uint64_t kth = kmax;    // keys greater than kth are selected ...
+        int ties_wanted = want; // ... and the first ties_wanted (by index) of those equal to it
+        if (kmin != kmax) {
+            int hi_bit = 63 - __builtin_clzll(kmin ^ kmax);
+            if (tid == 0) {
+                sh_prefix = hi_bit == 63 ? 0 : (kmax >> (hi_bit + 1)) << (hi_bit + 1);
+                sh_rem = want;
+            }
+            bool resolved = false;  // became exact: every bit of the threshold key is known
+            while (!resolved) {
+                const int width = min(8, hi_bit - KeyBits<T>::kLowShift + 1);
+                const int shift = hi_bit - width + 1;
+                if (tid < 256) hist[tid] = 0;
+                __syncthreads();
+                const uint64_t prefix = sh_prefix;
+                const int rem = sh_rem;
+                for_keys([&](int, uint64_t k) {
+                    const bool match = hi_bit == 63 || ((k ^ prefix) >> (hi_bit + 1)) == 0;
+                    if (k != 0 && match)
+                        atomicAdd(&hist[(int)((k >> shift) & ((1u << width) - 1u))], 1);
+                });
+                __syncthreads();
+                // The digit of the rem-th largest matching key: wave 0 walks the bins from the top,
+                // lane l holding bins 255-4l .. 252-4l; the inclusive running count first reaches
+                // rem in exactly one bin.
+                if (tid < 64) {
+                    int c[4], mine = 0;
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        c[u] = hist[255 - 4 * tid - u];
+                        mine += c[u];
+                    }
+                    int inc = mine;
+#pragma unroll
+                    for (int off = 1; off < 64; off <<= 1) {
+                        const int t = __shfl_up(inc, off, 64);
+                        if (tid >= off) inc += t;
+                    }
+                    int above = inc - mine;
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        if (above < rem && above + c[u] >= rem) {
+                            sh_rem = rem - above;
+                            sh_prefix = prefix | ((uint64_t)(255 - 4 * tid - u) << shift);
+                            sh_done = above + c[u] == rem;  // the whole bin is wanted
+                        }
+                        above += c[u];
+                    }
+                }
+                __syncthreads();
+                hi_bit = shift - 1;
+                resolved = hi_bit < KeyBits<T>::kLowShift;
+                if (sh_done) break;
+            }
+            if (resolved && !sh_done) {
+                kth = sh_prefix;
+                ties_wanted = sh_rem;
+            } else {
+                // every key at or above the chosen bin's lowest value is selected
+                const uint64_t floor_key = sh_prefix;
+                kth = floor_key == 0 ? 0 : floor_key - 1;
+                ties_wanted = 0;
+            }
+        }
+
+        // ---- compaction in index order ---------------------------------------------------
+        int ties = 0, greater = 0;
+        for_keys([&](int, uint64_t k) {
+            ties += k == kth;
+            greater += k > kth;
+        });
+        int total;
+        const int ties_before = block_exclusive_scan(ties, wave_sums, &total);
+        const int take = max(0, min(ties, ties_wanted - ties_before));
+        int at = block_exclusive_scan(greater + take, wave_sums, &total);
+        int tie_rank = ties_before;
+        for_keys([&](int i, uint64_t k) {
+            bool keep = k > kth;
+            if (k == kth) keep = tie_rank++ < ties_wanted;
+            if (keep) {
+                cand_key[at] = k;
+                cand_idx[at] = (uint32_t)i;
+                ++at;
+            }
+        });
+        __syncthreads();
+
+        // ---- order: descending key, ascending index among equal keys -------------------------
+        // Bitonic network over the candidates padded to a power of two.  A wave owns a chunk of
+        // 128 elements: every stage whose partner distance stays inside a chunk needs no
+        // work-group barrier (a wave's LDS operations execute in order), so a 512-entry list
+        // costs 3 barriers for its 45 stages.
+        int padded = 1;
+        while (padded < want) padded <<= 1;
+        for (int i = want + tid; i < padded; i += kTopkThreads) {
+            cand_key[i] = 0;
+            cand_idx[i] = 0xffffffffu;
+        }
+        __syncthreads();
+        const auto exchange = [&](int a, int b, bool reversed_run) {
+            const uint64_t ka = cand_key[a], kb = cand_key[b];
+            const uint32_t ia = cand_idx[a], ib = cand_idx[b];
+            const bool a_first = ka > kb || (ka == kb && ia < ib);
+            if (a_first == reversed_run) {
+                cand_key[a] = kb, cand_key[b] = ka;
+                cand_idx[a] = ib, cand_idx[b] = ia;
+            }
+        };
+        const int wave = tid >> 6, lane = tid & 63;
+        for (int k2 = 2; k2 <= padded; k2 <<= 1) {
+            for (int j2 = k2 >> 1; j2 > 0; j2 >>= 1) {
+                if (j2 >= 128) {
+                    __syncthreads();
+                    for (int t = tid; t < padded / 2; t += kTopkThreads) {
+                        const int a = (t / j2) * 2 * j2 + t % j2;
+                        exchange(a, a + j2, (a & k2) != 0);
+                    }
+                    __syncthreads();
+                } else {
+                    const int a = wave * 128 + (lane / j2) * 2 * j2 + lane % j2;
+                    if (a + j2 < padded) exchange(a, a + j2, (a & k2) != 0);
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                    __builtin_amdgcn_wave_barrier();
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                }
+            }
+        }
+        __syncthreads();
+    }
+
+    // ---- emit, then the query's own block when the selection missed it ---------------------
+    if (tid == 0) sh_present = 0;
+    __syncthreads();
+    bool mine = false;
+    for (int i = tid; i < want; i += kTopkThreads) {
+        const uint32_t id = cand_idx[i];
+        ids[i] = id;
+        mine = mine || id == own;
+    }
+    if (mine) sh_present = 1;
+    __syncthreads();
+    if (tid == 0) {
+        uint32_t count = (uint32_t)want;
+        if (!sh_present && count < (uint32_t)P.max_ids) ids[count++] = own;
+        P.counts[e] = count;
+    }
+}
+
+}  // namespace
+
+hipError_t launch_idx_score(const SelectBatch& b, const float* q, int32_t idx_n_head, int32_t idx_dim,
+                            int32_t idx_block, double* scores, int64_t score_stride, int32_t max_blocks,
+                            hipStream_t stream) {
+    ScoreParams sp;
+    sp.b = b;
+    sp.q = q;
+    sp.scores = scores;
+    sp.score_stride = score_stride;
+    sp.idx_n_head = idx_n_head;
+    sp.idx_dim = idx_dim;
+    sp.idx_block = idx_block;
+    dim3 grid((unsigned)((max_blocks + kScoreTile - 1) / kScoreTile), (unsigned)b.n);
+    idx_score_kernel<<<grid, kScoreThreads, 0, stream>>>(sp);
+    return hipGetLastError();
+}
+
+hipError_t launch_topk_blocks(const SelectBatch& b, const void* scores, bool scores_f64,
+                              int64_t score_stride, int32_t topk_blocks, int32_t idx_block, bool dense,
+                              uint32_t* ids, int64_t id_stride, uint32_t* counts, int32_t max_ids,
+                              hipStream_t stream) {
+    TopkParams tp;
+    tp.b = b;
+    tp.scores = scores;
+    tp.score_stride = score_stride;
+    tp.ids = ids;
+    tp.id_stride = id_stride;
+    tp.counts = counts;
+    tp.topk_blocks = topk_blocks;
+    tp.max_ids = max_ids;
+    tp.idx_block = idx_block;
+    tp.dense = dense ? 1 : 0;
+    int32_t longest = 0;
+    for (int i = 0; i < b.n; ++i) longest = std::max(longest, b.n_blocks[i]);
+    const bool few = longest <= 8 * kTopkThreads;
+    if (scores_f64) {
+        if (few)
+            topk_blocks_kernel<double, 8><<<b.n, kTopkThreads, 0, stream>>>(tp);
+        else
+            topk_blocks_kernel<double, 32><<<b.n, kTopkThreads, 0, stream>>>(tp);
+    } else {
+        if (few)
+            topk_blocks_kernel<float, 8><<<b.n, kTopkThreads, 0, stream>>>(tp);
+        else
+            topk_blocks_kernel<float, 32><<<b.n, kTopkThreads, 0, stream>>>(tp);
+    }
+    return hipGetLastError();
+}
+
+int32_t select_max_topk() { return kMaxTopk; }
+int32_t select_max_idx_head() { return kMaxIdxHead; }
+int32_t select_max_idx_dim() { return kMaxIdxDim; }
+
+}  // namespace bkv

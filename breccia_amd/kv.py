@@ -307,6 +307,25 @@ class Pool:
                                          _ptr(ids_dev), id_stride, _ptr(counts_dev), max_ids,
                                          _ptr(out_dev), _sh(stream)))
 
+    def select_blocks(self, pos, idx_q_dev, pooled_devs, n_blocks, idx_n_head: int, idx_dim: int,
+                      topk_blocks: int, ids_dev, id_stride: int, counts_dev, max_ids: int,
+                      stream=None) -> None:
+        """Indexer score + top-k: leaves ids / counts on the device for decode_attn_select."""
+        pos, pp = _i64(pos)
+        n_blocks, pn = _i32(n_blocks)
+        assert pos.size == n_blocks.size == len(pooled_devs)
+        ptrs = (C.c_void_p * max(len(pooled_devs), 1))(*[_ptr(x) for x in pooled_devs])
+        check(lib.bkv_select_blocks(self.handle, pos.size, pp, _ptr(idx_q_dev), ptrs, pn, idx_n_head,
+                                    idx_dim, topk_blocks, _ptr(ids_dev), id_stride, _ptr(counts_dev),
+                                    max_ids, _sh(stream)))
+
+    def topk_blocks(self, pos, scores_dev, n_blocks: int, topk_blocks: int, ids_dev, id_stride: int,
+                    counts_dev, max_ids: int, dense: bool = False, stream=None) -> None:
+        pos, pp = _i64(pos)
+        check(lib.bkv_topk_blocks(self.handle, pos.size, pp, _ptr(scores_dev), n_blocks, topk_blocks,
+                                  1 if dense else 0, _ptr(ids_dev), id_stride, _ptr(counts_dev), max_ids,
+                                  _sh(stream)))
+
     def page_copy(self, pairs, stream=None) -> None:
         """pairs: iterable of (src, dst), or an int32 array of shape [n, 2]."""
         arr = np.ascontiguousarray(np.asarray(list(pairs) if not isinstance(pairs, np.ndarray)

@@ -218,6 +218,36 @@ bkv_status bkv_decode_attn_select(bkv_pool *pool, int32_t layer, int32_t n, cons
                                   int64_t id_stride, const uint32_t *counts_dev, int32_t max_ids,
                                   float *out_dev, void *stream);
 
+/* Block selection, the step that produces those lists (Qsa::idx_score + Qsa::topk,
+ * qsa/mod.rs:1234-1376; shaders qsa_idx_score.comp, qsa_topk*.comp; oracle qsa/cpu.rs:93-152).
+ * A block is 4 cells.  For list i (a query at pos[i]):
+ *   score[b] = (1/sqrt(idx_dim)) * sum_h relu(idx_q[i][h] . pooled_i[b]),  b < n_blocks[i],
+ *              dead when block b starts after pos[i];
+ *   ids      = the topk_blocks best live blocks by descending score, ties to the lower block,
+ *              then block pos[i]/4 (the query's own) when the selection missed it;
+ *   counts[i] = length of the list (<= max_ids; the own block is dropped when there is no room).
+ * Scores are computed as the CPU reference computes them (f64, sums in index order) and are
+ * kept in a workspace the pool owns, so the emitted list is the reference CPU list exactly,
+ * not merely a list of equal quality.
+ *   idx_q_dev   device f32 [n][idx_n_head][idx_dim]  (the model: 4 x 128)
+ *   pooled_dev  host array of n device pointers, f32 [n_blocks[i]][idx_dim] each (the
+ *               sequence's pooled indexer keys, QsaState::idx_pooled)
+ *   n_blocks    host array; pos host array.  topk_blocks <= 2048 (the model: 512). */
+bkv_status bkv_select_blocks(bkv_pool *pool, int32_t n, const int64_t *pos, const float *idx_q_dev,
+                             const float *const *pooled_dev, const int32_t *n_blocks,
+                             int32_t idx_n_head, int32_t idx_dim, int32_t topk_blocks,
+                             uint32_t *ids_dev, int64_t id_stride, uint32_t *counts_dev,
+                             int32_t max_ids, void *stream);
+/* The top-k alone over f32 scores the caller already holds: Qsa::topk / Qsa::topk_dense on
+ * ws.idx_scores [n][n_blocks] (qsa/mod.rs:1264-1376).  A score is live iff it is greater than
+ * -1e29 (the shaders' dead marker is -1e30; -inf and NaN are dead too).  The scores are not
+ * modified (the reference's serial kernel destroys them).  dense != 0: no scores read, every
+ * visible block 0..min(n_blocks, own+1) in ascending order, then the own block if it lies
+ * beyond n_blocks. */
+bkv_status bkv_topk_blocks(bkv_pool *pool, int32_t n, const int64_t *pos, const float *scores_dev,
+                           int32_t n_blocks, int32_t topk_blocks, int32_t dense, uint32_t *ids_dev,
+                           int64_t id_stride, uint32_t *counts_dev, int32_t max_ids, void *stream);
+
 /* Copy-on-write page copy: for every pair and every layer, K and V bytes of page
  * `src` -> page `dst`.  No reference implementation (nearest: dispatch_batch.rs:
  * 1130-1150 record_copy).  Pairs are host memory; dst pages must be distinct. */

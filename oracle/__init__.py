@@ -96,6 +96,10 @@ _lib.bkvo_swap_out.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C
                                C.c_size_t, C.c_size_t]
 _lib.bkvo_swap_in.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p,
                               C.c_size_t, C.c_size_t]
+_lib.bkvo_indexer_score.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int64, C.c_size_t,
+                                    C.c_size_t, C.c_size_t, C.c_void_p]
+_lib.bkvo_topk_blocks.restype = C.c_size_t
+_lib.bkvo_topk_blocks.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_int64, C.c_void_p]
 _lib.bkvo_rmsnorm.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p, C.c_float,
                               C.c_void_p]
 _lib.bkvo_rope_table.argtypes = [C.c_double, C.c_size_t, C.c_size_t, C.c_void_p]
@@ -280,6 +284,28 @@ def dense_cells(pos: int) -> np.ndarray:
 
 
 # -------------------------------------------------------------- test generators
+# ------------------------------------------------------------------ block selection
+def indexer_score(q, pooled, n_blocks: int, pos: int, idx_n_head: int = 4, idx_dim: int = 128,
+                  idx_block: int = 4) -> np.ndarray:
+    """float64 [n_blocks]; q: [idx_n_head, idx_dim], pooled: [>= n_blocks, idx_dim]."""
+    q = np.ascontiguousarray(q, dtype=np.float32)
+    pooled = np.ascontiguousarray(pooled, dtype=np.float32)
+    assert q.size == idx_n_head * idx_dim and pooled.size >= n_blocks * idx_dim
+    out = np.empty(n_blocks, dtype=np.float64)
+    _lib.bkvo_indexer_score(q.ctypes.data, pooled.ctypes.data, n_blocks, pos, idx_n_head, idx_dim,
+                            idx_block, out.ctypes.data)
+    return out
+
+
+def topk_blocks(scores, k: int, own_block: int | None) -> np.ndarray:
+    """uint32 ids: descending score, ties to the lower block, own block appended when missed."""
+    scores = np.ascontiguousarray(scores, dtype=np.float64)
+    out = np.empty(k + 1, dtype=np.uint32)
+    n = _lib.bkvo_topk_blocks(scores.ctypes.data, scores.size, k, -1 if own_block is None else own_block,
+                              out.ctypes.data)
+    return out[:n].copy()
+
+
 # ------------------------------------------------------------------ K preparation
 def rmsnorm(x, cols: int, gamma=None, wgroups: int | None = None, eps: float = 1e-6) -> np.ndarray:
     """Row-wise RMSNorm of x viewed as [rows, cols]; gamma is [wgroups, cols] or None."""

@@ -26,6 +26,11 @@
  *   bkvo_rope_apply                      identity at position 0, NEOX pairing one-hot),
  *                                        independent numpy float64 statements, rotation
  *                                        invariants (pair norms kept, angles add)
+ *   bkvo_indexer_score / bkvo_topk_blocks pinned: reference KATs (qsa/cpu.rs:517-536: ties to the
+ *                                        lower block, own block appended once, dead blocks
+ *                                        never selected), the reference's LCG score recipes
+ *                                        (tests/qsa_topk.rs:87-122) against numpy lexsort,
+ *                                        numpy float64 statement of the score
  *   bkvo_to_i8h / append_i8 / gather_i8  NOT IN THE REFERENCE (int8 K+V with an f16
  *                                        scale): parity unpinned against the
  *                                        reference; pinned only by closed-form
@@ -486,6 +491,59 @@ size_t bkvo_dense_ids(int64_t pos, int64_t n_kv_after, uint32_t idx_block, uint3
     for (int64_t b = 0; b < lim; ++b) out[n++] = (uint32_t)b;
     if (own >= n_blocks) out[n++] = (uint32_t)own;
     return n;
+}
+
+/* ---- block selection (the indexer's score and the top-k over it) -------------------
+ * qsa/cpu.rs:93-123: score[b] = (1/sqrt(idx_dim)) * sum_h relu(q_h . pooled_b), f64,
+ * sums in index order; -inf for a block that starts after the query's position. */
+void bkvo_indexer_score(const float *q, const float *pooled, size_t n_blocks, int64_t pos,
+                        size_t idx_n_head, size_t idx_dim, size_t idx_block, double *out) {
+    const double scale = 1.0 / sqrt((double)idx_dim);
+    for (size_t b = 0; b < n_blocks; ++b) {
+        if ((int64_t)(b * idx_block) > pos) {
+            out[b] = -INFINITY;
+            continue;
+        }
+        double acc = 0.0;
+        for (size_t h = 0; h < idx_n_head; ++h) {
+            double dot = 0.0;
+            for (size_t d = 0; d < idx_dim; ++d)
+                dot += (double)q[h * idx_dim + d] * (double)pooled[b * idx_dim + d];
+            acc += (dot > 0.0 ? dot : 0.0) * scale;
+        }
+        out[b] = acc;
+    }
+}
+
+static const double *topk_scores_for_sort;
+static int topk_order(const void *pa, const void *pb) {
+    const uint32_t a = *(const uint32_t *)pa, b = *(const uint32_t *)pb;
+    const double sa = topk_scores_for_sort[a], sb = topk_scores_for_sort[b];
+    if (sa > sb) return -1;
+    if (sa < sb) return 1;
+    return a < b ? -1 : (a > b ? 1 : 0);
+}
+
+/* qsa/cpu.rs:125-152: blocks by descending score, ties to the lower index, non-finite
+ * scores dropped, the first k kept, then the query's own block when the selection missed
+ * it (own < 0: no own block).  Returns the list length; out holds up to k + 1 ids.
+ * Not re-entrant (qsort has no context argument). */
+size_t bkvo_topk_blocks(const double *scores, size_t n, size_t k, int64_t own, uint32_t *out) {
+    uint32_t *order = (uint32_t *)malloc((n ? n : 1) * sizeof(uint32_t));
+    size_t live = 0;
+    for (size_t i = 0; i < n; ++i)
+        if (isfinite(scores[i])) order[live++] = (uint32_t)i;
+    topk_scores_for_sort = scores;
+    qsort(order, live, sizeof(uint32_t), topk_order);
+    size_t count = live < k ? live : k;
+    memcpy(out, order, count * sizeof(uint32_t));
+    free(order);
+    if (own >= 0) {
+        int present = 0;
+        for (size_t i = 0; i < count; ++i) present |= out[i] == (uint32_t)own;
+        if (!present) out[count++] = (uint32_t)own;
+    }
+    return count;
 }
 
 /* ---- K preparation ahead of the append (Qsa::k_norm + Qsa::rope_k) ---------------

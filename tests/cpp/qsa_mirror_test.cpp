@@ -21,6 +21,9 @@ int bkvo_gather(const bkvo_geom*, int, const void*, const void*, const int32_t*,
 int bkvo_attend(const float*, const float*, const float*, const uint32_t*, size_t, int64_t, int32_t,
                 int32_t, int32_t, const float*, float*, int);
 void bkvo_normalish(uint64_t, size_t, float*);
+void bkvo_indexer_score(const float*, const float*, size_t, int64_t, size_t, size_t, size_t, double*);
+size_t bkvo_topk_blocks(const double*, size_t, size_t, int64_t, uint32_t*);
+size_t bkvo_cells_of(const uint32_t*, size_t, uint32_t, uint32_t*);
 void bkvo_rmsnorm(const float*, size_t, size_t, size_t, const float*, float, float*);
 void bkvo_rope_table(double, size_t, size_t, float*);
 void bkvo_rope_apply(const float*, size_t, size_t, size_t, const float*, size_t, const int32_t*, float*);
@@ -225,12 +228,85 @@ static void test_k_prep_append() {
     state.release();
 }
 
+static void test_selection_then_attention() {
+    // crates/breccia-kernels/tests/attn_conformance.rs:897-1004 through the mirror: 2062 cells,
+    // select 512 of 515 blocks + the tail block, then attend exactly that list
+    const int cells = 2062, n_blocks = 515, H = MODEL_N_HEAD, hd = MODEL_HEAD_DIM;
+    const size_t pos0 = cells - 1;
+    QsaState state = QsaState::create(cells, 4096);
+    Qsa qsa;
+    qsa.bind(state);
+    std::vector<float> idx_q(IDX_N_HEAD * IDX_DIM), pooled((n_blocks + 1) * IDX_DIM), k_all((size_t)cells * 512),
+        v_all((size_t)cells * 512), q(H * hd), q_full(H * 2 * hd);
+    bkvo_normalish(0xE1, idx_q.size(), idx_q.data());
+    bkvo_normalish(0xE2, pooled.size(), pooled.data());
+    bkvo_normalish(0xE3, k_all.size(), k_all.data());
+    bkvo_normalish(0xE4, v_all.size(), v_all.data());
+    bkvo_normalish(0xE5, q.size(), q.data());
+    bkvo_normalish(0xE6, q_full.size(), q_full.data());
+    QsaWorkspace fill = qsa.workspace(cells, cells);
+    upload(fill.k_cur, k_all);
+    upload(fill.v_cur, v_all);
+    qsa.kv_append(state, fill, 0);
+    QsaWorkspace ws = qsa.workspace(1, cells);
+    EXPECT(ws.n_blocks == (size_t)n_blocks && ws.max_ids == 513, "workspace sizes %zu %zu", ws.n_blocks, ws.max_ids);
+    float* pooled_dev = nullptr;
+    check(bkv_dev_alloc(pooled.size() * 4, (void**)&pooled_dev));
+    upload(pooled_dev, pooled);
+    upload(ws.idx_q, idx_q);
+    upload(ws.q, q);
+    upload(ws.q_full, q_full);
+    qsa.select(ws, pooled_dev, pos0);
+    qsa.attend(state, ws, pos0);
+    qsa.apply(state, ws, pos0);
+    check(bkv_device_sync());
+    const auto got_ids = download<uint32_t>(ws.ids, ws.max_ids);
+    const auto got_count = download<uint32_t>(ws.counts, 1);
+    const auto out = download<float>(ws.attn_out, (size_t)H * hd);
+
+    std::vector<double> scores(n_blocks);
+    bkvo_indexer_score(idx_q.data(), pooled.data(), n_blocks, (int64_t)pos0, IDX_N_HEAD, IDX_DIM, IDX_BLOCK,
+                       scores.data());
+    std::vector<uint32_t> want_ids(IDX_TOPK_BLOCKS + 1);
+    const size_t want_n = bkvo_topk_blocks(scores.data(), n_blocks, IDX_TOPK_BLOCKS, (int64_t)(pos0 / IDX_BLOCK),
+                                           want_ids.data());
+    EXPECT(got_count[0] == want_n, "selection length %u vs %zu", got_count[0], want_n);
+    EXPECT(std::memcmp(got_ids.data(), want_ids.data(), want_n * 4) == 0, "selection order/set differs");
+
+    const bkvo_geom g{2, 256, 16};
+    const int pages = (cells + 15) / 16;
+    std::vector<int32_t> table(pages);
+    for (int i = 0; i < pages; ++i) table[i] = i;
+    std::vector<uint16_t> pk((size_t)pages * 2 * 16 * 256, 0), pv(pk.size(), 0);
+    bkvo_append_f16(&g, pk.data(), pv.data(), table.data(), (int64_t)pages * 16, 0, cells, k_all.data(), v_all.data());
+    std::vector<float> kf((size_t)cells * 512), vf((size_t)cells * 512);
+    bkvo_gather(&g, 0, pk.data(), pv.data(), table.data(), 0, cells, kf.data(), vf.data());
+    std::vector<uint32_t> cell_list(want_n * IDX_BLOCK);
+    const size_t n_cells = bkvo_cells_of(want_ids.data(), want_n, IDX_BLOCK, cell_list.data());
+    std::vector<float> gate(H * hd), want(H * hd);
+    for (int h = 0; h < H; ++h) std::memcpy(&gate[h * hd], &q_full[(size_t)h * 2 * hd + hd], hd * 4);
+    bkvo_attend(q.data(), kf.data(), vf.data(), cell_list.data(), n_cells, (int64_t)pos0, H, 2, hd, gate.data(),
+                want.data(), 4);
+    double worst = 0.0;
+    for (int i = 0; i < H * hd; ++i) {
+        const double w = want[i], e = std::fabs((double)out[i] - w);
+        worst = std::fmax(worst, e / std::fmax(std::fabs(w), 1.0));
+    }
+    EXPECT(worst <= 1e-5, "sparse attention max_rel %.3e exceeds 1e-5", worst);
+    std::printf("qsa select+attend   blocks=%d selected=%u: ids exact, max_rel %.3e\n", n_blocks, got_count[0], worst);
+    check(bkv_dev_free(pooled_dev));
+    qsa.release(ws);
+    qsa.release(fill);
+    state.release();
+}
+
 int main() {
     try {
         test_errors();
         test_layout_recipe();
         test_attention();
         test_k_prep_append();
+        test_selection_then_attention();
     } catch (const Error& e) {
         std::printf("FAIL: unexpected error %d: %s\n", (int)e.status, e.what());
         return 2;

@@ -1,0 +1,195 @@
+"""GPU parity of block selection (indexer score + top-k) against the CPU oracle: the emitted
+id lists must be identical, element for element (crates/breccia-kernels/src/qsa/cpu.rs:93-152;
+recipes of tests/qsa_topk.rs and tests/attn_conformance.rs:897-1004)."""
+import numpy as np
+import pytest
+
+import oracle
+from breccia_amd import lib as L
+from breccia_amd.kv import BkvError, DeviceBuffer, Pool, device_sync
+from gpu_common import REF_BAR_MAX_REL, Twin, check_attn
+from test_gpu_attn import fill
+from test_oracle_select import DEAD, lcg_scores
+
+pytestmark = pytest.mark.gpu
+
+
+def gpu_topk(pool, scores, pos, topk, max_ids, dense=False, id_stride=None):
+    """scores: float32 [n, n_blocks] -> list of uint32 id arrays."""
+    scores = np.ascontiguousarray(scores, dtype=np.float32)
+    n, nb = scores.shape
+    id_stride = id_stride or max_ids
+    sd = DeviceBuffer.from_numpy(scores if scores.size else np.zeros(4, np.float32))
+    idd = DeviceBuffer.from_numpy(np.full((n, id_stride), 0xFFFFFFFF, dtype=np.uint32))
+    cd = DeviceBuffer.from_numpy(np.full(n, 0xFFFFFFFF, dtype=np.uint32))
+    try:
+        pool.topk_blocks(pos, sd, nb, topk, idd, id_stride, cd, max_ids, dense=dense)
+        device_sync()
+        ids = idd.download(np.uint32, n * id_stride).reshape(n, id_stride)
+        cnt = cd.download(np.uint32, n)
+        after = sd.download(np.float32, max(scores.size, 4))[:scores.size].reshape(n, nb)
+        assert np.array_equal(after.view(np.uint32), scores.view(np.uint32))    # scores untouched
+        for i in range(n):
+            assert np.all(ids[i, cnt[i]:] == 0xFFFFFFFF)                          # nothing past count
+        return [ids[i, :cnt[i]].copy() for i in range(n)]
+    finally:
+        for b in (sd, idd, cd):
+            b.free()
+
+
+def oracle_topk_f32(scores_row, topk, own, max_ids):
+    # the shaders' dead rule: a score <= -1e29 is never selected (shaders/qsa_topk.comp)
+    s = np.asarray(scores_row, dtype=np.float64).copy()
+    s[~(s > -1.0e29)] = -np.inf
+    ids = oracle.topk_blocks(s, min(topk, max_ids), None)
+    if own not in ids and ids.size < max_ids:
+        ids = np.append(ids, np.uint32(own))
+    return ids
+
+
+@pytest.mark.parametrize("cells", [65536, 65521])
+def test_reference_topk_recipes_are_exact(cells):
+    # crates/breccia-kernels/tests/qsa_topk.rs:87-122, 16384 / 16380 blocks, 512 kept
+    n, k, max_ids = cells // 4, 512, 513
+    distinct = lcg_scores(n)
+    tied = np.zeros(n, dtype=np.float32)
+    tied[:100] = 1.0
+    dead = distinct.copy()
+    dead[::3] = DEAD
+    rows = [distinct, tied, dead, np.full(n, 0.5, dtype=np.float32), distinct]
+    pos = [0, 0, 0, 0, 4 * (n - 3)]
+    with Pool(n_pages=4, max_seqs=2) as pool:
+        got = gpu_topk(pool, np.stack(rows), pos, k, max_ids)
+    for i, (row, p) in enumerate(zip(rows, pos)):
+        want = oracle_topk_f32(row, k, p // 4, max_ids)
+        assert np.array_equal(got[i], want), "recipe %d: first difference at %s" % (
+            i, np.nonzero(got[i][:min(got[i].size, want.size)] != want[:min(got[i].size, want.size)])[0][:3])
+
+
+def test_topk_edge_cases():
+    rng = np.random.Generator(np.random.PCG64(700))
+    with Pool(n_pages=4, max_seqs=2) as pool:
+        # reference known answers (qsa/cpu.rs:517-536) on f32 scores
+        s = np.array([[1.0, 3.0, 3.0, 2.0]], dtype=np.float32)
+        assert list(gpu_topk(pool, s, [4 * 9], 2, 8)[0]) == [1, 2, 9]
+        assert list(gpu_topk(pool, s, [4 * 9], 4, 8)[0]) == [1, 2, 3, 0, 9]
+        assert list(gpu_topk(pool, s, [4 * 3 + 1], 3, 8)[0]) == [1, 2, 3]
+        s = np.array([[-np.inf, -np.inf, 1.0]], dtype=np.float32)
+        assert list(gpu_topk(pool, s, [8], 3, 8)[0]) == [2]
+        # fewer live than k; NaN and the shaders' -1e30 marker are dead; -0 ties with +0 by index
+        s = np.array([[0.25, -1e30, 0.75, np.nan, 0.5, -0.0, 0.0, -3.0]], dtype=np.float32)
+        assert list(gpu_topk(pool, s, [4], 512, 16)[0]) == [2, 4, 0, 5, 6, 7, 1]
+        # no room for the own block; max_ids caps the list
+        assert list(gpu_topk(pool, s, [4 * 40], 3, 3)[0]) == [2, 4, 0]
+        assert list(gpu_topk(pool, s, [4 * 40], 512, 2, id_stride=5)[0]) == [2, 4]
+        # zero blocks: only the own block
+        assert list(gpu_topk(pool, np.zeros((1, 0), np.float32), [21], 512, 4)[0]) == [5]
+        # several lists of one call, random scores with many exact ties, k not a power of two
+        sc = rng.integers(0, 50, size=(7, 3000)).astype(np.float32) / 8 - 2
+        pos = [int(p) for p in rng.integers(0, 4 * 3000, size=7)]
+        got = gpu_topk(pool, sc, pos, 300, 301)
+        for i in range(7):
+            assert np.array_equal(got[i], oracle_topk_f32(sc[i], 300, pos[i] // 4, 301)), i
+        # negative scores order correctly (key transform of negative floats)
+        sc = -np.abs(rng.standard_normal((2, 1000))).astype(np.float32) * 1e3
+        got = gpu_topk(pool, sc, [0, 3999], 2048, 2049)
+        for i, p in enumerate([0, 3999]):
+            assert np.array_equal(got[i], oracle_topk_f32(sc[i], 2048, p // 4, 2049)), i
+        # dense: every visible block ascending, own appended when it lies beyond n_blocks
+        d = gpu_topk(pool, np.zeros((3, 515), np.float32), [2061, 100, 2059], 512, 600, dense=True)
+        assert list(d[0]) == list(range(515)) + [515]
+        assert list(d[1]) == list(range(26))
+        assert list(d[2]) == list(range(515))
+
+
+def gpu_select(pool, pos, idx_q, pooled_list, topk, max_ids):
+    n = len(pos)
+    qd = DeviceBuffer.from_numpy(np.ascontiguousarray(idx_q, dtype=np.float32))
+    pds = [DeviceBuffer.from_numpy(np.ascontiguousarray(p, dtype=np.float32)) for p in pooled_list]
+    idd = DeviceBuffer.from_numpy(np.full((n, max_ids), 0xFFFFFFFF, dtype=np.uint32))
+    cd = DeviceBuffer.from_numpy(np.zeros(n, dtype=np.uint32))
+    pool.select_blocks(pos, qd, pds, [p.shape[0] for p in pooled_list], idx_q.shape[1], idx_q.shape[2], topk,
+                       idd, max_ids, cd, max_ids)
+    device_sync()
+    ids = idd.download(np.uint32, n * max_ids).reshape(n, max_ids)
+    cnt = cd.download(np.uint32, n)
+    for b in [qd, cd] + pds:
+        b.free()
+    return idd, ids, cnt
+
+
+def test_reference_selection_and_attention_at_2062_cells():
+    # crates/breccia-kernels/tests/attn_conformance.rs:897-1004: 515 whole blocks + 2 tail cells,
+    # indexer queries 0xE1, pooled keys 0xE2, K/V 0xE3/0xE4 appended in 256-cell chunks, q 0xE5,
+    # gate in place from q_full 0xE6, 24 heads; selection list, then attention over exactly it
+    cells, n_blocks, pos = 2062, 515, 2061
+    idx_q = oracle.normalish(0xE1, 4 * 128).reshape(1, 4, 128)
+    pooled = oracle.normalish(0xE2, (n_blocks + 1) * 128).reshape(n_blocks + 1, 128)
+    k_all = oracle.normalish(0xE3, cells * 512).reshape(cells, 2, 256)
+    v_all = oracle.normalish(0xE4, cells * 512).reshape(cells, 2, 256)
+    q = oracle.normalish(0xE5, 24 * 256).reshape(1, 24, 256)
+    q_full = oracle.normalish(0xE6, 24 * 512)
+    with Twin(n_pages=129, max_seqs=2) as tw:
+        s = tw.pool.seq_create_identity(129)
+        tw.pool.seq_reserve(s, cells)
+        for at in range(0, cells, 256):
+            tw.append(0, [s], [at], [k_all[at:at + 256]], [v_all[at:at + 256]])
+        idd, ids, cnt = gpu_select(tw.pool, [pos], idx_q, [pooled[:n_blocks]], 512, 513)
+        want_ids = oracle.topk_blocks(oracle.indexer_score(idx_q[0], pooled, n_blocks, pos), 512, pos // 4)
+        assert cnt[0] == want_ids.size == 513
+        assert np.array_equal(ids[0, :cnt[0]], want_ids)      # order and set, tail block last
+        # attention over exactly those cells, lists left on the device
+        cd = DeviceBuffer.from_numpy(cnt)
+        qd = DeviceBuffer.from_numpy(q)
+        gd = DeviceBuffer.from_numpy(q_full)
+        od = DeviceBuffer(q.nbytes)
+        tw.pool.decode_attn_select(0, [s], [pos], 24, qd, od, 0.0625, idd, 513, cd, 513, gate_dev=gd.at(256 * 4),
+                                   gate_seq_stride=24 * 512, gate_head_stride=512)
+        out = od.download(np.float32, q.size).reshape(24, 256)
+        kk, vv = tw.images[0].gather(tw.pool.block_table(s), 0, cells)
+        gate = np.ascontiguousarray(q_full.reshape(24, 512)[:, 256:])
+        want = oracle.attend(q[0], kk, vv, oracle.cells_of(want_ids), pos, 24, 2, 256, gate=gate, threads=4)
+        _, rel = check_attn(out, want, "2062-cell sparse")
+        assert rel <= REF_BAR_MAX_REL, rel
+        for b in (idd, cd, qd, gd, od):
+            b.free()
+
+
+def test_score_and_select_batched_lists_are_exact():
+    # several sequences of different lengths in one call; scores are dense in value (many near
+    # ties), which is where an f32 score would reorder the list
+    rng = np.random.Generator(np.random.PCG64(710))
+    n_blocks = [8192, 515, 3, 0, 12001, 64]
+    pos = [4 * 8192 + 2, 2061, 9, 1, 48007, 130]       # entry 5: only blocks 0..32 are visible
+    idx_q = rng.standard_normal((6, 4, 128)).astype(np.float32)
+    pooled = [rng.standard_normal((nb, 128)).astype(np.float32) * 0.05 for nb in n_blocks]
+    with Pool(n_pages=4, max_seqs=2) as pool:
+        idd, ids, cnt = gpu_select(pool, pos, idx_q, pooled, 512, 513)
+        idd.free()
+    for i in range(6):
+        sc = oracle.indexer_score(idx_q[i], pooled[i], n_blocks[i], pos[i]) if n_blocks[i] else np.zeros(0)
+        want = oracle.topk_blocks(sc, 512, pos[i] // 4)
+        assert cnt[i] == want.size, (i, cnt[i], want.size)
+        assert np.array_equal(ids[i, :cnt[i]], want), i
+    assert cnt[5] == 33 and 32 in ids[5, :33]
+
+
+def test_select_errors_come_before_any_launch():
+    with Pool(n_pages=4, max_seqs=2) as pool:
+        z = DeviceBuffer(1 << 16)
+        for kw, status in [(dict(topk_blocks=0), L.ERR_INVALID), (dict(topk_blocks=4096), L.ERR_INVALID),
+                           (dict(max_ids=0), L.ERR_INVALID), (dict(id_stride=4), L.ERR_INVALID),
+                           (dict(ids_dev=None), L.ERR_INVALID), (dict(pos=[-1]), L.ERR_RANGE)]:
+            a = dict(pos=[5], scores_dev=z, n_blocks=16, topk_blocks=8, ids_dev=z, id_stride=16, counts_dev=z,
+                     max_ids=9)
+            a.update(kw)
+            with pytest.raises(BkvError) as ei:
+                pool.topk_blocks(**a)
+            assert ei.value.status == status, kw
+        with pytest.raises(BkvError) as ei:
+            pool.select_blocks([5], z, [z], [16], 9, 128, 8, z, 16, z, 9)       # too many indexer heads
+        assert ei.value.status == L.ERR_INVALID
+        with pytest.raises(BkvError) as ei:
+            pool.select_blocks([5], z, [None], [16], 4, 128, 8, z, 16, z, 9)    # NULL pooled keys
+        assert ei.value.status == L.ERR_INVALID
+        z.free()
