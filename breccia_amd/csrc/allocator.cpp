@@ -21,6 +21,7 @@ PageAllocator::PageAllocator(int32_t n_pages, int32_t page_cells, int32_t max_se
       max_seqs_(max_seqs),
       max_pages_per_seq_(max_pages_per_seq),
       refcount_((size_t)n_pages, 0),
+      external_((size_t)n_pages, 0),
       seqs_((size_t)max_seqs),
       table_((size_t)max_seqs * (size_t)max_pages_per_seq, -1) {
     for (int32_t p = 0; p < n_pages; ++p) free_.push_back(p);
@@ -28,6 +29,7 @@ PageAllocator::PageAllocator(int32_t n_pages, int32_t page_cells, int32_t max_se
 
 void PageAllocator::reset() {
     std::fill(refcount_.begin(), refcount_.end(), 0);
+    std::fill(external_.begin(), external_.end(), 0);
     free_.clear();
     for (int32_t p = 0; p < n_pages_; ++p) free_.push_back(p);
     for (int32_t s = 0; s < max_seqs_; ++s) {
@@ -110,6 +112,52 @@ AllocErr PageAllocator::seq_create_identity(int32_t n, int32_t* seq_out, std::st
     }
     seqs_[(size_t)s].n_pages = n;
     *seq_out = s;
+    return AllocErr::Ok;
+}
+
+AllocErr PageAllocator::seq_create_shared(const int32_t* pages, int32_t n, int32_t* seq_out,
+                                          std::string& err) {
+    if (n < 0 || n > max_pages_per_seq_ || (n > 0 && !pages)) {
+        err = fmt("shared sequence of %lld pages does not fit a block-table row of %lld", n,
+                  max_pages_per_seq_);
+        return AllocErr::Invalid;
+    }
+    for (int32_t c = 0; c < n; ++c) {
+        if (pages[c] < 0 || pages[c] >= n_pages_ || refcount_[(size_t)pages[c]] <= 0) {
+            err = fmt("shared sequence: entry %lld (page %lld) is not a live page", c, pages[c]);
+            return AllocErr::State;
+        }
+    }
+    int32_t s;
+    const AllocErr e = seq_create(&s, err);
+    if (e != AllocErr::Ok) return e;
+    for (int32_t c = 0; c < n; ++c) {
+        ++refcount_[(size_t)pages[c]];
+        set_entry(s, c, pages[c]);
+    }
+    seqs_[(size_t)s].n_pages = n;
+    seqs_[(size_t)s].len = (int64_t)n * page_cells_;
+    *seq_out = s;
+    return AllocErr::Ok;
+}
+
+AllocErr PageAllocator::retain_page(int32_t page, std::string& err) {
+    if (page < 0 || page >= n_pages_ || refcount_[(size_t)page] <= 0) {
+        err = fmt("retain: page %lld is not live", page);
+        return AllocErr::State;
+    }
+    ++refcount_[(size_t)page];
+    ++external_[(size_t)page];
+    return AllocErr::Ok;
+}
+
+AllocErr PageAllocator::release_page(int32_t page, std::string& err) {
+    if (page < 0 || page >= n_pages_ || external_[(size_t)page] <= 0) {
+        err = fmt("release: page %lld holds no external reference", page);
+        return AllocErr::State;
+    }
+    --external_[(size_t)page];
+    drop_page(page);
     return AllocErr::Ok;
 }
 
@@ -362,9 +410,9 @@ bool PageAllocator::check(std::string& err) const {
         is_free[(size_t)p] = 1;
     }
     for (int32_t p = 0; p < n_pages_; ++p) {
-        if (seen[(size_t)p] != refcount_[(size_t)p]) {
-            err = fmt("page %lld: refcount %lld but %lld table entries", p, refcount_[(size_t)p],
-                      seen[(size_t)p]);
+        if (seen[(size_t)p] + external_[(size_t)p] != refcount_[(size_t)p]) {
+            err = fmt("page %lld: refcount %lld but %lld table entries and external references", p,
+                      refcount_[(size_t)p], seen[(size_t)p] + external_[(size_t)p]);
             return false;
         }
         if ((refcount_[(size_t)p] == 0) != (is_free[(size_t)p] != 0)) {

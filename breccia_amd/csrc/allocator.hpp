@@ -47,6 +47,13 @@ public:
     // Restore bookkeeping: entries [lp0, lp0+n) must be -1; fresh pages are attached.
     AllocErr seq_attach_pages(int32_t seq, int32_t lp0, int32_t n, std::vector<int32_t>& phys_out,
                               std::string& err);
+    // A new sequence whose first n logical pages are the given live physical pages (one more
+    // reference each) and whose length is n whole pages: how a request adopts a cached prefix.
+    AllocErr seq_create_shared(const int32_t* pages, int32_t n, int32_t* seq_out, std::string& err);
+    // References held by an owner that is not a sequence (the prefix tree).
+    AllocErr retain_page(int32_t page, std::string& err);
+    AllocErr release_page(int32_t page, std::string& err);
+    int32_t external_refs(int32_t page) const { return external_[(size_t)page]; }
     AllocErr set_free_order(const int32_t* order, int32_t n, std::string& err);
     void reset();
 
@@ -88,6 +95,7 @@ private:
 
     int32_t n_pages_, page_cells_, max_seqs_, max_pages_per_seq_;
     std::vector<int32_t> refcount_;
+    std::vector<int32_t> external_;  // part of refcount_ held by non-sequence owners
     std::deque<int32_t> free_;  // FIFO: the longest-free page is reused first
     std::vector<Seq> seqs_;
     std::vector<int32_t> table_;  // [max_seqs][max_pages_per_seq], -1 = none

@@ -237,6 +237,7 @@ bkv_status bkv_pool_create(const bkv_pool_desc* d, bkv_pool** out) {
     try {
         p->alloc.reset(new PageAllocator(d->n_pages, d->page_cells, d->max_seqs,
                                          d->max_pages_per_seq));
+        p->prefix.reset(new PrefixTree(p->alloc.get(), d->page_cells));
     } catch (const std::bad_alloc&) {
         delete p;
         return fail(BKV_ERR_NOMEM, "pool_create: out of host memory for the block tables");
@@ -317,6 +318,7 @@ bkv_status bkv_pool_destroy(bkv_pool* p) {
 
 bkv_status bkv_pool_reset(bkv_pool* p, void* stream) {
     if (!p) return fail(BKV_ERR_INVALID, "pool_reset: NULL pool");
+    p->prefix->clear();
     p->alloc->reset();
     if (p->host_only) {
         p->alloc->pending().clear();
@@ -395,9 +397,100 @@ bkv_status bkv_seq_reserve(bkv_pool* p, int32_t seq, int64_t new_len, bkv_page_p
     if (!p) return fail(BKV_ERR_INVALID, "seq_reserve: NULL pool");
     std::string err;
     static_assert(sizeof(PagePair) == sizeof(bkv_page_pair), "pair layouts must agree");
-    return from_alloc(p->alloc->seq_reserve(seq, new_len, reinterpret_cast<PagePair*>(cow), cow_cap,
-                                            n_cow, err),
-                      err);
+    AllocErr e = p->alloc->seq_reserve(seq, new_len, reinterpret_cast<PagePair*>(cow), cow_cap, n_cow, err);
+    if (e == AllocErr::NoPages && p->prefix->nodes() > 0) {
+        // Out of free pages: cached prefixes that nobody uses are the first thing to go
+        // (least recently used first), then the request is tried once more.
+        const int64_t grow = (new_len - p->alloc->seq_len(seq) + p->g.page_cells - 1) / p->g.page_cells + 1;
+        const int64_t missing = grow - p->alloc->free_pages();
+        if (missing > 0 && p->prefix->evict((int32_t)missing) > 0) {
+            err.clear();
+            e = p->alloc->seq_reserve(seq, new_len, reinterpret_cast<PagePair*>(cow), cow_cap, n_cow, err);
+        }
+    }
+    return from_alloc(e, err);
+}
+
+// ---- prefix tree ----------------------------------------------------------------------------
+static bkv_status prefix_args(const bkv_pool* p, const char* what, const int32_t* tokens, int64_t n) {
+    if (!p) return fail(BKV_ERR_INVALID, std::string(what) + ": NULL pool");
+    if (n < 0 || (n > 0 && !tokens))
+        return fail(BKV_ERR_INVALID, std::string(what) + sfmt(": %lld tokens and a NULL pointer", n));
+    return BKV_OK;
+}
+
+bkv_status bkv_prefix_match(bkv_pool* p, const int32_t* tokens, int64_t n_tokens,
+                            int64_t* matched_tokens) {
+    bkv_status st = prefix_args(p, "prefix_match", tokens, n_tokens);
+    if (st != BKV_OK) return st;
+    std::vector<int32_t> pages;
+    p->prefix->match(tokens, n_tokens, false, pages);
+    if (matched_tokens) *matched_tokens = (int64_t)pages.size() * p->g.page_cells;
+    return BKV_OK;
+}
+
+bkv_status bkv_seq_create_from_prefix(bkv_pool* p, const int32_t* tokens, int64_t n_tokens,
+                                      int32_t* seq_out, int64_t* matched_tokens) {
+    bkv_status st = prefix_args(p, "seq_create_from_prefix", tokens, n_tokens);
+    if (st != BKV_OK) return st;
+    if (!seq_out) return fail(BKV_ERR_INVALID, "seq_create_from_prefix: NULL output");
+    std::vector<int32_t> pages;
+    p->prefix->match(tokens, n_tokens, true, pages);
+    if ((int64_t)pages.size() > p->alloc->max_pages_per_seq()) pages.resize((size_t)p->alloc->max_pages_per_seq());
+    std::string err;
+    st = from_alloc(p->alloc->seq_create_shared(pages.data(), (int32_t)pages.size(), seq_out, err), err);
+    if (st != BKV_OK) return st;
+    if (matched_tokens) *matched_tokens = (int64_t)pages.size() * p->g.page_cells;
+    return BKV_OK;
+}
+
+bkv_status bkv_prefix_insert(bkv_pool* p, int32_t seq, const int32_t* tokens, int64_t n_tokens,
+                             int32_t* new_pages) {
+    bkv_status st = prefix_args(p, "prefix_insert", tokens, n_tokens);
+    if (st != BKV_OK) return st;
+    if (!p->alloc->seq_valid(seq))
+        return fail(BKV_ERR_RANGE, sfmt("prefix_insert: sequence %lld is not live", seq));
+    if (n_tokens > p->alloc->seq_len(seq))
+        return fail(BKV_ERR_RANGE, sfmt("prefix_insert: %lld tokens listed but sequence %lld holds %lld",
+                                        n_tokens, seq, p->alloc->seq_len(seq)));
+    std::string err;
+    const int32_t added = p->prefix->insert(tokens, n_tokens, p->alloc->seq_table(seq),
+                                            p->alloc->seq_n_pages(seq), err);
+    if (added < 0) return fail(BKV_ERR_STATE, err);
+    if (new_pages) *new_pages = added;
+    return BKV_OK;
+}
+
+bkv_status bkv_prefix_evict(bkv_pool* p, int32_t want_pages, int32_t* freed) {
+    if (!p) return fail(BKV_ERR_INVALID, "prefix_evict: NULL pool");
+    if (want_pages < 0) return fail(BKV_ERR_INVALID, sfmt("prefix_evict: %lld pages wanted", want_pages));
+    const int32_t n = p->prefix->evict(want_pages);
+    if (freed) *freed = n;
+    return BKV_OK;
+}
+
+bkv_status bkv_prefix_pin(bkv_pool* p, const int32_t* tokens, int64_t n_tokens, int32_t pin,
+                          int64_t* affected_tokens) {
+    bkv_status st = prefix_args(p, "prefix_pin", tokens, n_tokens);
+    if (st != BKV_OK) return st;
+    const int32_t n = p->prefix->pin(tokens, n_tokens, pin ? +1 : -1);
+    if (affected_tokens) *affected_tokens = (int64_t)n * p->g.page_cells;
+    return BKV_OK;
+}
+
+bkv_status bkv_prefix_stats(const bkv_pool* p, int32_t* nodes, int32_t* evictable_pages,
+                            int32_t* pinned_nodes) {
+    if (!p) return fail(BKV_ERR_INVALID, "prefix_stats: NULL pool");
+    if (nodes) *nodes = p->prefix->nodes();
+    if (evictable_pages) *evictable_pages = p->prefix->evictable_pages();
+    if (pinned_nodes) *pinned_nodes = p->prefix->pinned_nodes();
+    return BKV_OK;
+}
+
+bkv_status bkv_prefix_clear(bkv_pool* p) {
+    if (!p) return fail(BKV_ERR_INVALID, "prefix_clear: NULL pool");
+    p->prefix->clear();
+    return BKV_OK;
 }
 
 bkv_status bkv_seq_truncate(bkv_pool* p, int32_t seq, int64_t new_len) {

@@ -10,6 +10,7 @@
 
 #include "../../include/breccia_kv.h"
 #include "allocator.hpp"
+#include "prefix_tree.hpp"
 
 namespace bkv {
 
@@ -74,6 +75,7 @@ struct bkv_pool {
     bkv_pool_desc desc{};
     bkv::Geom g{};
     std::unique_ptr<bkv::PageAllocator> alloc;
+    std::unique_ptr<bkv::PrefixTree> prefix;  // declared after alloc: destroyed first
     bool host_only = false;
     int device = 0;
     int n_cu = 0;

@@ -262,6 +262,46 @@ class Pool:
         check(lib.bkv_timing_read(self.handle, stage, C.byref(n), C.byref(ms)))
         return int(n.value), float(ms.value)
 
+    # -- prefix tree
+    def prefix_insert(self, seq: int, tokens) -> int:
+        tokens, pt = _i32(tokens)
+        n = C.c_int32()
+        check(lib.bkv_prefix_insert(self.handle, seq, pt, tokens.size, C.byref(n)))
+        return int(n.value)
+
+    def prefix_match(self, tokens) -> int:
+        tokens, pt = _i32(tokens)
+        m = C.c_int64()
+        check(lib.bkv_prefix_match(self.handle, pt, tokens.size, C.byref(m)))
+        return int(m.value)
+
+    def seq_create_from_prefix(self, tokens):
+        """-> (seq, matched_tokens)"""
+        tokens, pt = _i32(tokens)
+        s, m = C.c_int32(), C.c_int64()
+        check(lib.bkv_seq_create_from_prefix(self.handle, pt, tokens.size, C.byref(s), C.byref(m)))
+        return int(s.value), int(m.value)
+
+    def prefix_evict(self, want_pages: int) -> int:
+        n = C.c_int32()
+        check(lib.bkv_prefix_evict(self.handle, want_pages, C.byref(n)))
+        return int(n.value)
+
+    def prefix_pin(self, tokens, pin: bool = True) -> int:
+        tokens, pt = _i32(tokens)
+        m = C.c_int64()
+        check(lib.bkv_prefix_pin(self.handle, pt, tokens.size, 1 if pin else 0, C.byref(m)))
+        return int(m.value)
+
+    def prefix_stats(self):
+        """-> (nodes, evictable_pages, pinned_nodes)"""
+        a, b, c = C.c_int32(), C.c_int32(), C.c_int32()
+        check(lib.bkv_prefix_stats(self.handle, C.byref(a), C.byref(b), C.byref(c)))
+        return int(a.value), int(b.value), int(c.value)
+
+    def prefix_clear(self) -> None:
+        check(lib.bkv_prefix_clear(self.handle))
+
     # -- hot path
     def append(self, layer: int, seqs, pos0, n_tokens, k_dev, v_dev, stream=None,
                f16_rows: bool = False) -> None:

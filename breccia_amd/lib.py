@@ -75,6 +75,13 @@ _SIGNATURES = {
     "bkv_pool_free_pages": (_i32, [_vp]),
     "bkv_pool_check": (C.c_int, [_vp]),
     "bkv_pool_set_free_order": (C.c_int, [_vp, _pi32, _i32]),
+    "bkv_prefix_insert": (C.c_int, [_vp, _i32, _pi32, _i64, _pi32]),
+    "bkv_prefix_match": (C.c_int, [_vp, _pi32, _i64, _pi64]),
+    "bkv_seq_create_from_prefix": (C.c_int, [_vp, _pi32, _i64, _pi32, _pi64]),
+    "bkv_prefix_evict": (C.c_int, [_vp, _i32, _pi32]),
+    "bkv_prefix_pin": (C.c_int, [_vp, _pi32, _i64, _i32, _pi64]),
+    "bkv_prefix_stats": (C.c_int, [_vp, _pi32, _pi32, _pi32]),
+    "bkv_prefix_clear": (C.c_int, [_vp]),
     "bkv_timing_enable": (C.c_int, [_vp, C.c_int]),
     "bkv_timing_reset": (C.c_int, [_vp]),
     "bkv_timing_read": (C.c_int, [_vp, C.c_int, C.POINTER(_u64), C.POINTER(C.c_double)]),

@@ -138,6 +138,41 @@ bkv_status bkv_pool_check(const bkv_pool *pool);
  * permutation of the pages that are free right now (fragmentation studies, tests). */
 bkv_status bkv_pool_set_free_order(bkv_pool *pool, const int32_t *order, int32_t n);
 
+/* ---- prefix tree: reuse of cached prefixes ------------------------------------
+ * No reference implementation; the shape follows its design notes (docs/reference-engines/
+ * 02-kv-and-context.md:543-548 page-aligned 16-token hash granularity, :566-581 tier
+ * movement rules, :600-603 radix tree with refcount / last_access, eviction as a strategy,
+ * pinned read-only subtree).  One tree per pool, one node per COMPLETE page, keyed by that
+ * page's token ids; the tree holds one reference on every page it lists, so a listed prefix
+ * outlives the sequence that computed it.  Host-side only; nothing is launched.
+ *
+ * bkv_prefix_insert: list the complete pages of the first n_tokens tokens of `seq` (whose K/V
+ *   the caller has appended).  Prefixes already listed keep their pages (first publisher
+ *   wins); *new_pages = nodes added.
+ * bkv_prefix_match: how many leading tokens of `tokens` are covered by listed pages
+ *   (a multiple of the page size); does not count as a use.
+ * bkv_seq_create_from_prefix: a new sequence that shares those pages (refcount + 1 each),
+ *   length = *matched_tokens; the caller appends the rest, starting on a fresh page -- a
+ *   page-aligned share never needs a copy-on-write copy.
+ * bkv_prefix_evict: drop least-recently-used unpinned leaves that nobody else holds until
+ *   want_pages went back to the free queue.  bkv_seq_reserve does this by itself when it
+ *   runs out of free pages, before it reports BKV_ERR_NO_PAGES.
+ * bkv_prefix_pin: pin != 0 pins, 0 unpins the listed chain of `tokens` (injected read-only
+ *   context: never evicted while pinned).
+ * bkv_pool_reset clears the tree. */
+bkv_status bkv_prefix_insert(bkv_pool *pool, int32_t seq, const int32_t *tokens, int64_t n_tokens,
+                             int32_t *new_pages);
+bkv_status bkv_prefix_match(bkv_pool *pool, const int32_t *tokens, int64_t n_tokens,
+                            int64_t *matched_tokens);
+bkv_status bkv_seq_create_from_prefix(bkv_pool *pool, const int32_t *tokens, int64_t n_tokens,
+                                      int32_t *seq_out, int64_t *matched_tokens);
+bkv_status bkv_prefix_evict(bkv_pool *pool, int32_t want_pages, int32_t *freed);
+bkv_status bkv_prefix_pin(bkv_pool *pool, const int32_t *tokens, int64_t n_tokens, int32_t pin,
+                          int64_t *affected_tokens);
+bkv_status bkv_prefix_stats(const bkv_pool *pool, int32_t *nodes, int32_t *evictable_pages,
+                            int32_t *pinned_nodes);
+bkv_status bkv_prefix_clear(bkv_pool *pool);
+
 /* ---- hot path ---------------------------------------------------------------
  * bkv_append replaces Qsa::kv_append + shaders/qsa_kv_append.comp (qsa/mod.rs:
  * 1105-1156): scatter n_tokens[i] new rows of sequence seqs[i] to cells pos0[i]..
