@@ -676,8 +676,13 @@ static bkv_status decode_attn_common(bkv_pool* p, int32_t layer, int32_t n, cons
                                      const float* gate_dev, int64_t gate_seq_stride,
                                      int64_t gate_head_stride, float scale, const uint32_t* ids_dev,
                                      int64_t id_stride, const uint32_t* counts_dev, int32_t max_ids,
-                                     bool select, float* out_dev, void* stream) {
+                                     bool select, float* out_dev, void* stream,
+                                     const float* new_k_dev = nullptr, const float* new_v_dev = nullptr,
+                                     bool step = false) {
     if (!p) return fail(BKV_ERR_INVALID, "decode_attn: NULL pool");
+    if (step && p->g.layout != BKV_LAYOUT_F16)
+        return fail(BKV_ERR_INVALID, "decode_step is built for f16 pools; append and attend in two "
+                                     "calls on a quantised pool");
     if (layer < 0 || layer >= p->g.n_layers)
         return fail(BKV_ERR_RANGE, sfmt("decode_attn: layer %lld is outside 0..%lld", layer,
                                         p->g.n_layers));
@@ -715,6 +720,11 @@ static bkv_status decode_attn_common(bkv_pool* p, int32_t layer, int32_t n, cons
         if (!p->alloc->seq_resident(seqs[i], pos[i] + 1))
             return fail(BKV_ERR_STATE, sfmt("decode_attn: sequence %lld has swapped-out pages "
                                             "below position %lld", seqs[i], pos[i]));
+        if (step)
+            for (int j = 0; j < i; ++j)
+                if (seqs[j] == seqs[i])
+                    return fail(BKV_ERR_INVALID, sfmt("decode_step: sequence %lld appears twice; one "
+                                                      "new token per sequence and call", seqs[i]));
         b.row[i] = seqs[i];
         b.pos[i] = (int32_t)pos[i];
     }
@@ -725,6 +735,9 @@ static bkv_status decode_attn_common(bkv_pool* p, int32_t layer, int32_t n, cons
     if (!q_dev || !out_dev || !aligned16(q_dev) || !aligned16(out_dev))
         return fail(BKV_ERR_INVALID, "decode_attn: q/out device pointers must be non-NULL and "
                                      "16-byte aligned");
+    if (step && (!new_k_dev || !new_v_dev || !aligned16(new_k_dev) || !aligned16(new_v_dev)))
+        return fail(BKV_ERR_INVALID, "decode_step: k/v device pointers must be non-NULL and 16-byte "
+                                     "aligned");
     if (select && (!ids_dev || !counts_dev || ((uintptr_t)ids_dev & 3u) || ((uintptr_t)counts_dev & 3u)))
         return fail(BKV_ERR_INVALID, "decode_attn_select: ids/counts device pointers must be "
                                      "non-NULL and 4-byte aligned");
@@ -745,6 +758,10 @@ static bkv_status decode_attn_common(bkv_pool* p, int32_t layer, int32_t n, cons
         a.id_stride = id_stride;
         a.max_ids = max_ids;
     }
+    if (step) {
+        a.new_k = new_k_dev;
+        a.new_v = new_v_dev;
+    }
     BKV_HIP(launch_decode_attn(p, layer, b, a, S(stream)));
     if (p->timer.open.size() > 8192) return timer_collect(p);
     return BKV_OK;
@@ -756,6 +773,15 @@ bkv_status bkv_decode_attn(bkv_pool* p, int32_t layer, int32_t n, const int32_t*
                            int64_t gate_head_stride, float scale, float* out_dev, void* stream) {
     return decode_attn_common(p, layer, n, seqs, pos, n_q_head, q_dev, gate_dev, gate_seq_stride,
                               gate_head_stride, scale, nullptr, 0, nullptr, 0, false, out_dev, stream);
+}
+
+bkv_status bkv_decode_step(bkv_pool* p, int32_t layer, int32_t n, const int32_t* seqs, const int64_t* pos,
+                           const float* k_new_dev, const float* v_new_dev, int32_t n_q_head,
+                           const float* q_dev, const float* gate_dev, int64_t gate_seq_stride,
+                           int64_t gate_head_stride, float scale, float* out_dev, void* stream) {
+    return decode_attn_common(p, layer, n, seqs, pos, n_q_head, q_dev, gate_dev, gate_seq_stride,
+                              gate_head_stride, scale, nullptr, 0, nullptr, 0, false, out_dev, stream,
+                              k_new_dev, v_new_dev, true);
 }
 
 bkv_status bkv_decode_attn_select(bkv_pool* p, int32_t layer, int32_t n, const int32_t* seqs,

@@ -178,6 +178,9 @@ struct AttnArgs {
     const uint32_t* counts = nullptr;
     int64_t id_stride = 0;
     int32_t max_ids = 0;
+    // fused decode step: new rows [n][n_kv][head_dim] f32; nullptr = plain attention
+    const float* new_k = nullptr;
+    const float* new_v = nullptr;
 };
 // Fills wg_base/splits/pps from row/pos; returns the total work-group count.  sel_groups > 0:
 // every entry is planned for that many groups of four selected blocks instead of its pages.

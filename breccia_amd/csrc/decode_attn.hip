@@ -23,6 +23,7 @@
 // Partial (m, l, O) of the four waves are merged in LDS and written per work-group;
 // the merge kernel combines the splits and applies sigmoid(gate).
 #include "bkv_internal.hpp"
+#include "f16_rule.hpp"
 
 namespace bkv {
 
@@ -54,6 +55,12 @@ struct AttnKernelParams {
     const uint32_t* counts;
     int64_t id_stride;
     int32_t max_ids;
+    // fused decode step (decode_attn_kernel<..., STEP = true> only): the K/V row of cell pos of
+    // entry e comes from new_k / new_v [n][n_kv][head_dim] f32 and is stored into the pool on the way
+    const float* new_k;
+    const float* new_v;
+    uint8_t* kpool_w;
+    uint8_t* vpool_w;
 };
 
 __device__ __forceinline__ void wave_lds_sync() {
@@ -243,7 +250,10 @@ __device__ __forceinline__ bool block_cell_live(uint32_t id, int r, int pos) {
 
 // HG = q heads carried by one wave (8 or 4); KENC / VENC = row encodings of the K and V pools;
 // SEL = attend the cells of a per-entry list of selected blocks instead of every cell 0..=pos.
-template <int HG, int KENC, int VENC, bool SEL>
+// STEP = the decode step in one launch: the row of cell pos is taken from the caller's f32 K/V
+// (stored under the cache's f16 rule, exactly what the append kernel stores) and written to
+// the pool by the wave that owns the last page, so no append launch precedes the attention.
+template <int HG, int KENC, int VENC, bool SEL, bool STEP = false>
 __global__ __launch_bounds__(kBlock, HG == 8 ? 2 : 3) void decode_attn_kernel(const AttnKernelParams P) {
     constexpr int HQ = HG / 4;           // float4 groups of heads
     constexpr int NB = HG / 4;           // score batches per page (8 float4 slots each)
@@ -403,6 +413,39 @@ __global__ __launch_bounds__(kBlock, HG == 8 ? 2 : 3) void decode_attn_kernel(co
     unsigned turn = 0;
 
     while (pg < pg1) {
+        if constexpr (STEP) {
+            static_assert(!STEP || (KENC == kRowF16 && VENC == kRowF16 && !SEL),
+                          "the fused step is built for f16 pools and the dense selection");
+            if (pg == n_pages - 1) {
+                // This wave holds the page of cell pos.  Its pool row is stale (the token has
+                // not been appended): replace the lane's share of it with the new row, and let
+                // the lanes of that row's parity store it.
+                const int r = pos & (kPage - 1);
+                const size_t src = ((size_t)e * P.n_kv + (size_t)kvh) * kHd + (size_t)dl * 8;
+                const float4 ka = *reinterpret_cast<const float4*>(P.new_k + src);
+                const float4 kb = *reinterpret_cast<const float4*>(P.new_k + src + 4);
+                const float4 va = *reinterpret_cast<const float4*>(P.new_v + src);
+                const float4 vb = *reinterpret_cast<const float4*>(P.new_v + src + 4);
+                v4u kw, vw;
+                kw.x = f16_store_pair(ka.x, ka.y), kw.y = f16_store_pair(ka.z, ka.w);
+                kw.z = f16_store_pair(kb.x, kb.y), kw.w = f16_store_pair(kb.z, kb.w);
+                vw.x = f16_store_pair(va.x, va.y), vw.y = f16_store_pair(va.z, va.w);
+                vw.z = f16_store_pair(vb.x, vb.y), vw.w = f16_store_pair(vb.z, vb.w);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    if (2 * i + hw == r) {
+                        kk.r[i] = __builtin_bit_cast(half8, kw);
+                        vv.r[i] = __builtin_bit_cast(half8, vw);
+                    }
+                }
+                if (hw == (r & 1) && hc == 0) {
+                    const size_t off = (size_t)(cur.k[0] - P.kpool) + (size_t)r * (kHd * 2) + (size_t)dl * 16;
+                    *reinterpret_cast<v4u*>(P.kpool_w + off) = kw;
+                    const size_t voff = (size_t)(cur.v[0] - P.vpool) + (size_t)r * (kHd * 2) + (size_t)dl * 16;
+                    *reinterpret_cast<v4u*>(P.vpool_w + voff) = vw;
+                }
+            }
+        }
         if (younger && turn != 0)
             __builtin_amdgcn_s_setprio(2);
         else
@@ -795,7 +838,12 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
     kp.counts = a.counts;
     kp.id_stride = a.id_stride;
     kp.max_ids = a.max_ids;
+    kp.new_k = a.new_k;
+    kp.new_v = a.new_v;
+    kp.kpool_w = p->k_layer[(size_t)layer];
+    kp.vpool_w = p->v_layer[(size_t)layer];
     const bool sel = a.ids != nullptr;
+    const bool step = a.new_k != nullptr;
     const int32_t total = b.wg_base[b.n];
     const int32_t n_units = total / kp.n_hc;
     const int32_t grid = (n_units + 7) / 8 * 8 * kp.n_hc;
@@ -809,7 +857,13 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
         else                                                                    \
             decode_attn_kernel<HGV, KE, VE, false><<<grid, kBlock, 0, stream>>>(kp); \
     } while (0)
-        if (layout == BKV_LAYOUT_F16) {
+        if (step) {
+            // f16 pools, dense selection (checked by the caller)
+            if (hg == 8)
+                decode_attn_kernel<8, kRowF16, kRowF16, false, true><<<grid, kBlock, 0, stream>>>(kp);
+            else
+                decode_attn_kernel<4, kRowF16, kRowF16, false, true><<<grid, kBlock, 0, stream>>>(kp);
+        } else if (layout == BKV_LAYOUT_F16) {
             if (hg == 8) BKV_LAUNCH(8, kRowF16, kRowF16); else BKV_LAUNCH(4, kRowF16, kRowF16);
         } else if (layout == BKV_LAYOUT_Q8V) {
             if (hg == 8) BKV_LAUNCH(8, kRowF16, kRowQ8); else BKV_LAUNCH(4, kRowF16, kRowQ8);

@@ -4,6 +4,7 @@
 // All of it is HBM-bound; the rules that matter are 16-byte accesses, whole-line
 // coalescing and several independent loads in flight per lane.
 #include "bkv_internal.hpp"
+#include "f16_rule.hpp"
 
 namespace bkv {
 
@@ -22,25 +23,7 @@ __device__ __forceinline__ void st_stream(void* p, v4u v) {
     __builtin_nontemporal_store(v, reinterpret_cast<v4u*>(p));
 }
 
-// f32 -> binary16 code under the cache's storage rule
-// (crates/breccia-kernels/shaders/f16_storage.glsl:26-55, qsa/cpu.rs:23-53):
-// round-to-nearest-even like the hardware convert, except that every |x| < 2^-14
-// becomes a signed zero (no subnormals, even where rounding would reach 2^-14) and
-// NaN becomes a signed infinity.
-__device__ __forceinline__ uint32_t f16_store_bits(float x) {
-    const uint32_t b = __float_as_uint(x);
-    const uint32_t sign = (b >> 16) & 0x8000u;
-    const uint32_t mag = b & 0x7fffffffu;
-    const _Float16 h = static_cast<_Float16>(x);  // v_cvt_f16_f32, RNE, overflow -> inf
-    uint32_t code = static_cast<uint32_t>(__builtin_bit_cast(uint16_t, h));
-    if (mag < 0x38800000u) code = sign;
-    if (mag > 0x7f800000u) code = sign | 0x7c00u;
-    return code;
-}
-
-__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-    return f16_store_bits(lo) | (f16_store_bits(hi) << 16);
-}
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) { return f16_store_pair(lo, hi); }
 
 // binary16 code -> f32 under the cache's load rule (f16_storage.glsl:58-69):
 // exponent field 0 reads as a signed zero.

@@ -335,6 +335,17 @@ class Pool:
                                   _ptr(gate_dev), gate_seq_stride, gate_head_stride, scale,
                                   _ptr(out_dev), _sh(stream)))
 
+    def decode_step(self, layer: int, seqs, pos, k_new_dev, v_new_dev, n_q_head: int, q_dev, out_dev,
+                    scale: float, gate_dev=None, gate_seq_stride: int = 0, gate_head_stride: int = 0,
+                    stream=None) -> None:
+        """Append one token per sequence at pos and attend 0..pos, in one call (f16 pools)."""
+        seqs, ps = _i32(seqs)
+        pos, pp = _i64(pos)
+        assert seqs.size == pos.size
+        check(lib.bkv_decode_step(self.handle, layer, seqs.size, ps, pp, _ptr(k_new_dev), _ptr(v_new_dev),
+                                  n_q_head, _ptr(q_dev), _ptr(gate_dev), gate_seq_stride, gate_head_stride,
+                                  scale, _ptr(out_dev), _sh(stream)))
+
     def decode_attn_select(self, layer: int, seqs, pos, n_q_head: int, q_dev, out_dev, scale: float,
                            ids_dev, id_stride: int, counts_dev, max_ids: int, gate_dev=None,
                            gate_seq_stride: int = 0, gate_head_stride: int = 0, stream=None) -> None:

@@ -235,6 +235,21 @@ bkv_status bkv_decode_attn(bkv_pool *pool, int32_t layer, int32_t n, const int32
                            const float *gate_dev, int64_t gate_seq_stride,
                            int64_t gate_head_stride, float scale, float *out_dev, void *stream);
 
+/* One decode step in one call: append the new token's K/V row of every listed sequence at cell
+ * pos[i] and attend cells 0..pos[i] -- bkv_append of one token per sequence followed by
+ * bkv_decode_attn, without the append launch (Qsa::kv_append + Qsa::attend + Qsa::apply of
+ * a T = 1 call, qsa/mod.rs:1617-1639).  The work-group that owns the last page of a sequence
+ * takes the row from k_new_dev / v_new_dev (f32 [n][n_kv_head][head_dim]), stores it under
+ * the cache's f16 rule -- the pool afterwards holds exactly what bkv_append would have
+ * written -- and uses it in place of the stale pool row; the output is bit-identical to the
+ * two-call sequence.  f16 pools only; every sequence at most once per call; the cell must
+ * have been reserved (bkv_seq_reserve) like for bkv_append. */
+bkv_status bkv_decode_step(bkv_pool *pool, int32_t layer, int32_t n, const int32_t *seqs,
+                           const int64_t *pos, const float *k_new_dev, const float *v_new_dev,
+                           int32_t n_q_head, const float *q_dev, const float *gate_dev,
+                           int64_t gate_seq_stride, int64_t gate_head_stride, float scale,
+                           float *out_dev, void *stream);
+
 /* The same attention over a selection list instead of every cell: the reference's real
  * long-context form (Qsa::attend / Qsa::apply read ws.ids [T, max_ids] and ws.counts [T],
  * qsa/mod.rs:1382-1462; shaders/qsa_attn_scores_small.comp; oracle qsa/cpu.rs:197-257).
