@@ -822,6 +822,35 @@ static bkv_status select_common_checks(bkv_pool* p, const char* what, int32_t n,
     return BKV_OK;
 }
 
+bkv_status bkv_idx_pool(bkv_pool* p, float* pooled_dev, int32_t max_blocks, float* tail_dev,
+                        const float* idx_k_dev, int64_t pos0, int32_t tokens, const float* gamma_dev,
+                        float eps, const float* rope_table_dev, int32_t n_rot, int32_t max_pos,
+                        int32_t idx_dim, void* stream) {
+    if (!p) return fail(BKV_ERR_INVALID, "idx_pool: NULL pool");
+    if (idx_dim <= 0 || idx_dim > select_max_idx_dim() || idx_dim % 2 != 0)
+        return fail(BKV_ERR_INVALID, sfmt("idx_pool: idx_dim %lld is outside 2..%lld", idx_dim,
+                                          select_max_idx_dim()));
+    if (n_rot <= 0 || n_rot % 2 != 0 || n_rot > idx_dim)
+        return fail(BKV_ERR_INVALID, sfmt("idx_pool: n_rot %lld must be even and within 2..%lld", n_rot,
+                                          idx_dim));
+    if (max_pos <= 0) return fail(BKV_ERR_INVALID, "idx_pool: an empty rotary table");
+    if (tokens < 0 || pos0 < 0 || pos0 + tokens > 0x7fffffff)
+        return fail(BKV_ERR_RANGE, sfmt("idx_pool: %lld tokens at position %lld", tokens, pos0));
+    if (!(eps >= 0.0f)) return fail(BKV_ERR_INVALID, "idx_pool: eps must be >= 0");
+    const int64_t blocks_after = (pos0 + tokens) / 4;
+    if (blocks_after > max_blocks)
+        return fail(BKV_ERR_RANGE, sfmt("idx_pool would write pooled rows up to %lld but the buffer "
+                                        "holds %lld", blocks_after, max_blocks));
+    bkv_status st = need_device(p);
+    if (st != BKV_OK) return st;
+    if (tokens == 0) return BKV_OK;
+    if (!pooled_dev || !tail_dev || !idx_k_dev || !gamma_dev || !rope_table_dev)
+        return fail(BKV_ERR_INVALID, "idx_pool: NULL device pointer");
+    BKV_HIP(launch_idx_pool(idx_k_dev, tail_dev, gamma_dev, rope_table_dev, pooled_dev, (int32_t)pos0, tokens,
+                            idx_dim, 4, n_rot, max_pos, eps, S(stream)));
+    return BKV_OK;
+}
+
 bkv_status bkv_topk_blocks(bkv_pool* p, int32_t n, const int64_t* pos, const float* scores_dev,
                            int32_t n_blocks, int32_t topk_blocks, int32_t dense, uint32_t* ids_dev,
                            int64_t id_stride, uint32_t* counts_dev, int32_t max_ids, void* stream) {

@@ -154,6 +154,9 @@ hipError_t launch_topk_blocks(const SelectBatch& b, const void* scores, bool sco
                               int64_t score_stride, int32_t topk_blocks, int32_t idx_block, bool dense,
                               uint32_t* ids, int64_t id_stride, uint32_t* counts, int32_t max_ids,
                               hipStream_t stream);
+hipError_t launch_idx_pool(const float* raw, float* tail, const float* gamma, const float* table,
+                           float* pooled, int32_t pos0, int32_t tokens, int32_t idx_dim, int32_t idx_block,
+                           int32_t n_rot, int32_t max_pos, float eps, hipStream_t stream);
 int32_t select_max_topk();
 int32_t select_max_idx_head();
 int32_t select_max_idx_dim();

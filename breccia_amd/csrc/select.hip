@@ -79,6 +79,86 @@ __global__ __launch_bounds__(kScoreThreads) void idx_score_kernel(const ScorePar
     }
 }
 
+// ---- pooled indexer keys ---------------------------------------------------------------
+// pooled[b] = rotary(rmsnorm(mean(raw[4b .. 4b+3])), position 4b) for every block the call
+// completes (Qsa::idx_pool, qsa/mod.rs:1167-1207, shaders/qsa_idx_pool.comp; CPU path
+// qsa/cpu.rs:154-185): rows of the block come from this call's raw keys or, for cells before
+// pos0, from the rolling tail of the previous call.  Arithmetic as on the CPU: the mean adds
+// raw/idx_block in f32 in cell order, the norm sums squares in f64 in element order, the
+// rotary multiplies and adds in f64 without fusing -- so the pooled rows, and through them
+// the selection, are the CPU's bit for bit.
+struct PoolKeysParams {
+    const float* raw;    // [tokens][idx_dim]
+    const float* tail;   // [idx_block - 1][idx_dim]
+    const float* gamma;  // [idx_dim]
+    const float* table;  // [max_pos][n_rot / 2][2]
+    float* pooled;       // [blocks][idx_dim]
+    int32_t b0, n_new, pos0, tokens, idx_block, idx_dim, n_rot, max_pos;
+    float eps;
+};
+
+__global__ __launch_bounds__(kMaxIdxDim) void idx_pool_kernel(const PoolKeysParams P) {
+    __shared__ float val[kMaxIdxDim];
+    __shared__ double inv_s;
+    const int block = P.b0 + (int)blockIdx.x;
+    const int d = threadIdx.x;
+    if (d < P.idx_dim) {
+        float mean = 0.0f;
+        for (int k = 0; k < P.idx_block; ++k) {
+            const int cell = block * P.idx_block + k;
+            const int slot = cell - P.pos0;
+            float v = 0.0f;
+            if (slot >= 0 && slot < P.tokens)
+                v = P.raw[(size_t)slot * P.idx_dim + d];
+            else if (cell % P.idx_block + 1 < P.idx_block)
+                v = P.tail[(size_t)(cell % P.idx_block) * P.idx_dim + d];
+            mean += v / (float)P.idx_block;
+        }
+        val[d] = mean;
+    }
+    __syncthreads();
+    if (d == 0) {
+#pragma clang fp contract(off)
+        double ss = 0.0;
+        for (int i = 0; i < P.idx_dim; ++i) {
+            const double x = (double)val[i];
+            ss += x * x;
+        }
+        inv_s = 1.0 / sqrt(ss / (double)P.idx_dim + (double)P.eps);
+    }
+    __syncthreads();
+    if (d < P.idx_dim) val[d] = (float)((double)val[d] * inv_s * (double)P.gamma[d]);
+    __syncthreads();
+    const int half = P.n_rot / 2;
+    float out = d < P.idx_dim ? val[d] : 0.0f;
+    if (d < P.n_rot) {
+#pragma clang fp contract(off)
+        const int j = d < half ? d : d - half;
+        int64_t pos = (int64_t)block * P.idx_block;
+        pos = pos > P.max_pos - 1 ? P.max_pos - 1 : pos;
+        const double c = (double)P.table[((size_t)pos * half + j) * 2];
+        const double sn = (double)P.table[((size_t)pos * half + j) * 2 + 1];
+        const double a = (double)val[j], b = (double)val[j + half];
+        const double ac = a * c, bs = b * sn, as = a * sn, bc = b * c;
+        out = d < half ? (float)(ac - bs) : (float)(as + bc);
+    }
+    if (d < P.idx_dim) P.pooled[(size_t)block * P.idx_dim + d] = out;
+}
+
+// The rows of the last, incomplete block go to the rolling tail (Qsa::idx_tail,
+// shaders/qsa_idx_tail.comp): slot = cell % idx_block, the last slot is never needed.
+__global__ __launch_bounds__(256) void idx_tail_kernel(const float* __restrict__ raw, float* __restrict__ tail,
+                                                       int32_t tokens, int32_t pos0, int32_t idx_dim,
+                                                       int32_t idx_block) {
+    const int i = (int)blockIdx.x * 256 + (int)threadIdx.x;
+    if (i >= tokens * idx_dim) return;
+    const int d = i % idx_dim, t = i / idx_dim;
+    const int cell = pos0 + t, last_cell = pos0 + tokens - 1;
+    const int slot = cell % idx_block;
+    if (cell / idx_block == last_cell / idx_block && slot + 1 < idx_block)
+        tail[(size_t)slot * idx_dim + d] = raw[i];
+}
+
 // ---- top-k ---------------------------------------------------------------------------
 // Keys: unsigned integers that order like the scores.  A score is dead (never selected)
 // unless it is greater than -1e29: that covers -inf, NaN and the reference shaders' own
@@ -419,6 +499,35 @@ hipError_t launch_topk_blocks(const SelectBatch& b, const void* scores, bool sco
         else
             topk_blocks_kernel<float, 32><<<b.n, kTopkThreads, 0, stream>>>(tp);
     }
+    return hipGetLastError();
+}
+
+hipError_t launch_idx_pool(const float* raw, float* tail, const float* gamma, const float* table,
+                           float* pooled, int32_t pos0, int32_t tokens, int32_t idx_dim, int32_t idx_block,
+                           int32_t n_rot, int32_t max_pos, float eps, hipStream_t stream) {
+    PoolKeysParams pp;
+    pp.raw = raw;
+    pp.tail = tail;
+    pp.gamma = gamma;
+    pp.table = table;
+    pp.pooled = pooled;
+    pp.b0 = pos0 / idx_block;
+    pp.n_new = (pos0 + tokens) / idx_block - pp.b0;
+    pp.pos0 = pos0;
+    pp.tokens = tokens;
+    pp.idx_block = idx_block;
+    pp.idx_dim = idx_dim;
+    pp.n_rot = n_rot;
+    pp.max_pos = max_pos;
+    pp.eps = eps;
+    if (pp.n_new > 0) {
+        idx_pool_kernel<<<pp.n_new, kMaxIdxDim, 0, stream>>>(pp);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    // the tail is read by the pooling above and rewritten here: stream order keeps them apart
+    const int total = tokens * idx_dim;
+    idx_tail_kernel<<<(total + 255) / 256, 256, 0, stream>>>(raw, tail, tokens, pos0, idx_dim, idx_block);
     return hipGetLastError();
 }
 

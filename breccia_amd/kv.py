@@ -370,6 +370,13 @@ class Pool:
                                     idx_dim, topk_blocks, _ptr(ids_dev), id_stride, _ptr(counts_dev),
                                     max_ids, _sh(stream)))
 
+    def idx_pool(self, pooled_dev, max_blocks: int, tail_dev, idx_k_dev, pos0: int, tokens: int, gamma_dev,
+                 eps: float, table_dev, n_rot: int, max_pos: int, idx_dim: int = 128, stream=None) -> None:
+        """Pool the indexer keys of every block this call completes; keep the incomplete tail."""
+        check(lib.bkv_idx_pool(self.handle, _ptr(pooled_dev), max_blocks, _ptr(tail_dev), _ptr(idx_k_dev), pos0,
+                               tokens, _ptr(gamma_dev), eps, _ptr(table_dev), n_rot, max_pos, idx_dim,
+                               _sh(stream)))
+
     def topk_blocks(self, pos, scores_dev, n_blocks: int, topk_blocks: int, ids_dev, id_stride: int,
                     counts_dev, max_ids: int, dense: bool = False, stream=None) -> None:
         pos, pp = _i64(pos)

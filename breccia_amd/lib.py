@@ -98,6 +98,7 @@ _SIGNATURES = {
                                          _vp, _i64, _vp, _i32, _vp, _vp]),
     "bkv_select_blocks": (C.c_int, [_vp, _i32, _pi64, _vp, C.POINTER(_vp), _pi32, _i32, _i32, _i32, _vp,
                                     _i64, _vp, _i32, _vp]),
+    "bkv_idx_pool": (C.c_int, [_vp, _vp, _i32, _vp, _vp, _i64, _i32, _vp, _f32, _vp, _i32, _i32, _i32, _vp]),
     "bkv_topk_blocks": (C.c_int, [_vp, _i32, _pi64, _vp, _i32, _i32, _i32, _vp, _i64, _vp, _i32, _vp]),
     "bkv_page_copy": (C.c_int, [_vp, C.POINTER(PagePair), _i32, _vp]),
     "bkv_swap_page_bytes": (_u64, [_vp]),

@@ -288,6 +288,21 @@ bkv_status bkv_select_blocks(bkv_pool *pool, int32_t n, const int64_t *pos, cons
                              int32_t idx_n_head, int32_t idx_dim, int32_t topk_blocks,
                              uint32_t *ids_dev, int64_t id_stride, uint32_t *counts_dev,
                              int32_t max_ids, void *stream);
+/* The pooled indexer keys bkv_select_blocks scores against: Qsa::idx_pool + Qsa::idx_tail
+ * (qsa/mod.rs:1167-1232; shaders qsa_idx_pool.comp, qsa_idx_tail.comp; oracle qsa/cpu.rs:154-185).
+ * For every 4-cell block b completed by the tokens at pos0 .. pos0+tokens-1:
+ *   pooled[b] = rotary(rmsnorm(mean(raw rows 4b..4b+3)) * gamma, position 4b),
+ * rows before pos0 taken from the rolling tail (3 rows, slot = cell % 4) that the previous
+ * call left; afterwards the tail holds the rows of the last, incomplete block.  Arithmetic as
+ * on the CPU path (f32 mean in cell order, f64 norm and rotary), bit for bit.
+ *   pooled_dev  device f32 [max_blocks][idx_dim];  tail_dev device f32 [3][idx_dim]
+ *   idx_k_dev   device f32 [tokens][idx_dim] raw indexer keys of this call
+ *   gamma_dev   device f32 [idx_dim];  rope_table_dev as for bkv_append_kprep (the model
+ *               shares one table: n_rot 64 of idx_dim 128) */
+bkv_status bkv_idx_pool(bkv_pool *pool, float *pooled_dev, int32_t max_blocks, float *tail_dev,
+                        const float *idx_k_dev, int64_t pos0, int32_t tokens, const float *gamma_dev,
+                        float eps, const float *rope_table_dev, int32_t n_rot, int32_t max_pos,
+                        int32_t idx_dim, void *stream);
 /* The top-k alone over f32 scores the caller already holds: Qsa::topk / Qsa::topk_dense on
  * ws.idx_scores [n][n_blocks] (qsa/mod.rs:1264-1376).  A score is live iff it is greater than
  * -1e29 (the shaders' dead marker is -1e30; -inf and NaN are dead too).  The scores are not

@@ -105,6 +105,8 @@ _lib.bkvo_rmsnorm.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.
 _lib.bkvo_rope_table.argtypes = [C.c_double, C.c_size_t, C.c_size_t, C.c_void_p]
 _lib.bkvo_rope_apply.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p,
                                  C.c_size_t, C.c_void_p, C.c_void_p]
+_lib.bkvo_pool_keys.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t,
+                                C.c_size_t, C.c_size_t, C.c_float, C.c_void_p]
 _lib.bkvo_normalish.argtypes = [C.c_uint64, C.c_size_t, C.c_void_p]
 _lib.bkvo_q8_fixture.argtypes = [C.c_void_p, C.c_size_t]
 _lib.bkvo_max_threads.restype = C.c_int
@@ -354,6 +356,18 @@ def k_prep(k, n_kv: int, hd: int, gamma, eps: float, table, n_rot: int, token_po
     normed = rmsnorm(k, hd, gamma, wgroups=1, eps=eps)
     pos = np.repeat(np.asarray(token_pos, dtype=np.int32), n_kv)
     return rope_apply(normed, hd, n_rot, table, pos).reshape(k.shape)
+
+
+def pool_keys(raw, gamma, table, idx_dim: int = 128, idx_block: int = 4, n_rot: int = 64,
+              eps: float = 1e-6) -> np.ndarray:
+    """raw: [cells, idx_dim] raw indexer keys -> pooled [cells // idx_block, idx_dim]."""
+    raw = np.ascontiguousarray(raw, dtype=np.float32).reshape(-1, idx_dim)
+    gamma = np.ascontiguousarray(gamma, dtype=np.float32)
+    table = np.ascontiguousarray(table, dtype=np.float32)
+    out = np.empty((raw.shape[0] // idx_block, idx_dim), dtype=np.float32)
+    _lib.bkvo_pool_keys(raw.ctypes.data, raw.shape[0], gamma.ctypes.data, table.ctypes.data,
+                        table.size // n_rot, idx_dim, idx_block, n_rot, C.c_float(eps), out.ctypes.data)
+    return out
 
 
 def normalish(seed: int, n: int) -> np.ndarray:

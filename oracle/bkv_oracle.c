@@ -22,6 +22,9 @@
  *                                        x 512 elements) + permutation round trips
  *   bkvo_attend                          pinned: torch float64 SDPA, independent
  *                                        numpy softmax, closed forms
+ *   bkvo_pool_keys                       pinned: composition of the pinned norm and rotary with
+ *                                        a mean that closed forms fix (constant blocks, one
+ *                                        non-zero row) and a numpy float32 statement
  *   bkvo_rmsnorm / bkvo_rope_table /     pinned: reference KATs (ops/cpu.rs:373-421: constant row,
  *   bkvo_rope_apply                      identity at position 0, NEOX pairing one-hot),
  *                                        independent numpy float64 statements, rotation
@@ -602,6 +605,28 @@ void bkvo_rope_apply(const float *x, size_t rows, size_t head_dim, size_t n_rot,
         }
         for (size_t j = n_rot; j < head_dim; ++j) o[j] = xr[j];
     }
+}
+
+/* qsa/cpu.rs:154-185: pooled indexer keys.  pooled[b] = rope(rmsnorm(mean(raw[4b..4b+3])),
+ * position 4b): the mean accumulates raw/idx_block in f32 in cell order, the norm uses one
+ * gamma of idx_dim values, the rotary reads the table row of the block's first cell. */
+void bkvo_pool_keys(const float *raw, size_t cells, const float *gamma, const float *table,
+                    size_t max_pos, size_t idx_dim, size_t idx_block, size_t n_rot, float eps,
+                    float *out) {
+    const size_t n_blocks = cells / idx_block;
+    float *mean = (float *)malloc(idx_dim * sizeof(float));
+    float *normed = (float *)malloc(idx_dim * sizeof(float));
+    for (size_t b = 0; b < n_blocks; ++b) {
+        for (size_t d = 0; d < idx_dim; ++d) mean[d] = 0.0f;
+        for (size_t k = 0; k < idx_block; ++k)
+            for (size_t d = 0; d < idx_dim; ++d)
+                mean[d] += raw[(b * idx_block + k) * idx_dim + d] / (float)idx_block;
+        bkvo_rmsnorm(mean, 1, idx_dim, 1, gamma, eps, normed);
+        const int32_t pos = (int32_t)(b * idx_block);
+        bkvo_rope_apply(normed, 1, idx_dim, n_rot, table, max_pos, &pos, out + b * idx_dim);
+    }
+    free(mean);
+    free(normed);
 }
 
 /* ---------------------------------------------------------------------------

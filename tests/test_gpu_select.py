@@ -193,3 +193,49 @@ def test_select_errors_come_before_any_launch():
             pool.select_blocks([5], z, [None], [16], 4, 128, 8, z, 16, z, 9)    # NULL pooled keys
         assert ei.value.status == L.ERR_INVALID
         z.free()
+
+
+def test_pooled_indexer_keys_in_ragged_chunks_are_bit_exact():
+    # Qsa::idx_pool + Qsa::idx_tail over a sequence fed in chunks of every residue mod 4: the pooled
+    # rows must equal the oracle's pool_keys over the whole sequence, and feed the same selection
+    from breccia_amd.kv import rope_table
+    rng = np.random.Generator(np.random.PCG64(720))
+    cells, max_blocks = 1203, 320
+    raw = (rng.standard_normal((cells, 128)) * rng.uniform(0.1, 4.0, size=(cells, 1))).astype(np.float32)
+    gamma = (1.0 + 0.2 * rng.standard_normal(128)).astype(np.float32)
+    table = rope_table(1e7, 64, 2048)
+    want = oracle.pool_keys(raw, gamma, table)
+    with Pool(n_pages=4, max_seqs=2) as pool:
+        pooled = DeviceBuffer.from_numpy(np.full((max_blocks, 128), np.nan, dtype=np.float32))
+        tail = DeviceBuffer.from_numpy(np.full((3, 128), np.nan, dtype=np.float32))
+        gd, td = DeviceBuffer.from_numpy(gamma), DeviceBuffer.from_numpy(table)
+        at = 0
+        chunks = [1, 1, 1, 1, 2, 3, 5, 7, 4, 8, 1, 2, 300, 6, 1, 1, 3, 512]
+        while at < cells:
+            n = min(chunks.pop(0) if chunks else 97, cells - at)
+            kd = DeviceBuffer.from_numpy(raw[at:at + n])
+            pool.idx_pool(pooled, max_blocks, tail, kd, at, n, gd, 1e-6, td, 64, 2048)
+            device_sync()
+            kd.free()
+            at += n
+        got = pooled.download(np.float32, max_blocks * 128).reshape(max_blocks, 128)
+        assert np.array_equal(got[:cells // 4].view(np.uint32), want.view(np.uint32))
+        assert np.all(np.isnan(got[cells // 4:]))                       # nothing past the completed blocks
+        t = tail.download(np.float32, 3 * 128).reshape(3, 128)
+        assert np.array_equal(t[:3], raw[1200:1203])                    # the incomplete block's rows
+        # selection over the device-pooled keys == selection over the oracle's
+        idx_q = rng.standard_normal((1, 4, 128)).astype(np.float32)
+        qd = DeviceBuffer.from_numpy(idx_q)
+        idd = DeviceBuffer.from_numpy(np.zeros((1, 129), dtype=np.uint32))
+        cd = DeviceBuffer.from_numpy(np.zeros(1, dtype=np.uint32))
+        pool.select_blocks([cells - 1], qd, [pooled], [cells // 4], 4, 128, 128, idd, 129, cd, 129)
+        device_sync()
+        n = int(cd.download(np.uint32, 1)[0])
+        ids = idd.download(np.uint32, 129)[:n]
+        ref = oracle.topk_blocks(oracle.indexer_score(idx_q[0], want, cells // 4, cells - 1), 128, (cells - 1) // 4)
+        assert np.array_equal(ids, ref)
+        with pytest.raises(BkvError) as ei:
+            pool.idx_pool(pooled, 10, tail, gd, 36, 8, gd, 1e-6, td, 64, 2048)     # would write block 10
+        assert ei.value.status == L.ERR_RANGE
+        for b in (pooled, tail, gd, td, qd, idd, cd):
+            b.free()

@@ -155,3 +155,31 @@ def test_k_prep_composes_norm_then_rotary_per_kv_head():
             n = oracle.rmsnorm(k[t, h], hd, g, eps=1e-6)
             r = oracle.rope_apply(n, hd, 64, table, [pos[t]])
             assert np.array_equal(got[t, h], r.reshape(-1))
+
+
+def test_pool_keys_mean_then_norm_then_rotary_at_the_first_cell():
+    # crates/breccia-kernels/src/qsa/cpu.rs:154-185
+    rng = np.random.Generator(np.random.PCG64(33))
+    raw = rng.standard_normal((23, 128)).astype(np.float32)          # 5 whole blocks + 3 cells
+    gamma = rng.standard_normal(128).astype(np.float32)
+    table = oracle.rope_table(1e7, 64, 64)
+    got = oracle.pool_keys(raw, gamma, table)
+    assert got.shape == (5, 128)
+    for b in range(5):
+        mean = np.zeros(128, dtype=np.float32)
+        for k in range(4):
+            mean = (mean + raw[4 * b + k] / np.float32(4)).astype(np.float32)    # f32, cell order
+        want = oracle.rope_apply(oracle.rmsnorm(mean, 128, gamma, eps=1e-6), 128, 64, table, [4 * b])
+        assert np.array_equal(got[b], want.reshape(-1))
+    # closed forms: four equal rows pool to that row's normalised rotation; block 0 is not rotated
+    same = np.tile(raw[:1], (4, 1))
+    one = oracle.pool_keys(same, gamma, table)[0]
+    assert np.array_equal(one, oracle.rmsnorm(raw[0], 128, gamma, eps=1e-6).reshape(-1))
+    # a block with one non-zero row equals that row / 4 before the norm, and the norm undoes the 4
+    lone = np.zeros((8, 128), dtype=np.float32)
+    lone[5] = raw[5]
+    got2 = oracle.pool_keys(lone, np.ones(128, dtype=np.float32), table, eps=0.0)
+    ref2 = oracle.rope_apply(oracle.rmsnorm(raw[5], 128, None, eps=0.0), 128, 64, table, [4])
+    assert np.max(np.abs(got2[1] - ref2.reshape(-1))) < 1e-6
+    # (block 0 is all zeros: with eps = 0 its norm is 0/0, as the formula says)
+    assert np.all(oracle.pool_keys(lone, np.ones(128, dtype=np.float32), table, eps=1e-6)[0] == 0.0)
