@@ -795,6 +795,76 @@ bkv_status bkv_decode_attn_select(bkv_pool* p, int32_t layer, int32_t n, const i
                               out_dev, stream);
 }
 
+// ---- prefill attention ---------------------------------------------------------------------
+bkv_status bkv_prefill_attn(bkv_pool* p, int32_t layer, int32_t n_seqs, const int32_t* seqs,
+                            const int64_t* pos0, const int32_t* n_tokens, int32_t n_q_head,
+                            const float* q_dev, const float* gate_dev, int64_t gate_tok_stride,
+                            int64_t gate_head_stride, float scale, float* out_dev, void* stream) {
+    if (!p) return fail(BKV_ERR_INVALID, "prefill_attn: NULL pool");
+    if (layer < 0 || layer >= p->g.n_layers)
+        return fail(BKV_ERR_RANGE, sfmt("prefill_attn: layer %lld is outside 0..%lld", layer, p->g.n_layers));
+    if (n_seqs < 0 || n_seqs > BKV_MAX_BATCH)
+        return fail(BKV_ERR_INVALID, sfmt("prefill_attn: %lld chunks in one call; the limit is %lld", n_seqs,
+                                          BKV_MAX_BATCH));
+    if (n_q_head <= 0 || n_q_head % p->g.n_kv != 0)
+        return fail(BKV_ERR_INVALID, sfmt("prefill_attn: %lld q heads over %lld kv heads (need a whole "
+                                          "group)", n_q_head, p->g.n_kv));
+    if (p->g.layout != BKV_LAYOUT_F16 || p->g.hd != 256 || p->g.page_cells != 16)
+        return fail(BKV_ERR_INVALID, "prefill_attn is built for f16 pools with head_dim 256 and 16-cell "
+                                     "pages");
+    if (n_seqs > 0 && (!seqs || !pos0 || !n_tokens))
+        return fail(BKV_ERR_INVALID, "prefill_attn: NULL sequence / position / token-count array");
+    PrefillBatch b{};
+    const int64_t group = n_q_head / p->g.n_kv;
+    int64_t total = 0, wgs = 0;
+    for (int i = 0; i < n_seqs; ++i) {
+        if (!p->alloc->seq_valid(seqs[i]))
+            return fail(BKV_ERR_RANGE, sfmt("prefill_attn: sequence %lld is not live", seqs[i]));
+        if (n_tokens[i] < 0 || pos0[i] < 0)
+            return fail(BKV_ERR_RANGE, sfmt("prefill_attn: chunk %lld has pos0 %lld, n_tokens %lld", i, pos0[i],
+                                            n_tokens[i]));
+        const int64_t end = pos0[i] + n_tokens[i];
+        if (end > p->alloc->seq_capacity(seqs[i]))
+            return fail(BKV_ERR_RANGE, sfmt("prefill_attn: positions up to %lld of sequence %lld are outside "
+                                            "its %lld addressable cells", end - 1, seqs[i],
+                                            p->alloc->seq_capacity(seqs[i])));
+        if (n_tokens[i] > 0 && !p->alloc->seq_resident(seqs[i], end))
+            return fail(BKV_ERR_STATE, sfmt("prefill_attn: sequence %lld has swapped-out pages below "
+                                            "position %lld", seqs[i], end - 1));
+        b.row[i] = seqs[i];
+        b.pos0[i] = (int32_t)pos0[i];
+        b.n_tok[i] = n_tokens[i];
+        b.src0[i] = (int32_t)total;
+        b.wg_base[i] = (int32_t)wgs;
+        total += n_tokens[i];
+        const int64_t rows = (int64_t)n_tokens[i] * group;
+        wgs += (rows + prefill_rows_per_wg() - 1) / prefill_rows_per_wg() * p->g.n_kv;
+        if (total > ((int64_t)1 << 24) || wgs > ((int64_t)1 << 30))
+            return fail(BKV_ERR_INVALID, "prefill_attn: more than 2^24 tokens in one call");
+    }
+    b.n = n_seqs;
+    b.wg_base[n_seqs] = (int32_t)wgs;
+    bkv_status st = need_device(p);
+    if (st != BKV_OK) return st;
+    if (total == 0) return BKV_OK;
+    if (!q_dev || !out_dev || !aligned16(q_dev) || !aligned16(out_dev))
+        return fail(BKV_ERR_INVALID, "prefill_attn: q/out device pointers must be non-NULL and 16-byte "
+                                     "aligned");
+    st = flush_tables(p, S(stream));
+    if (st != BKV_OK) return st;
+    AttnArgs a;
+    a.n_q_head = n_q_head;
+    a.q = q_dev;
+    a.gate = gate_dev;
+    a.gate_seq_stride = gate_tok_stride;
+    a.gate_head_stride = gate_head_stride;
+    a.scale = scale;
+    a.out = out_dev;
+    BKV_HIP(launch_prefill_attn(p, layer, b, a, S(stream)));
+    if (p->timer.open.size() > 8192) return timer_collect(p);
+    return BKV_OK;
+}
+
 // ---- block selection ---------------------------------------------------------------------
 static bkv_status select_common_checks(bkv_pool* p, const char* what, int32_t n, const int64_t* pos,
                                        int32_t topk_blocks, const uint32_t* ids_dev, int64_t id_stride,

@@ -190,6 +190,18 @@ struct AttnArgs {
 int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b, int32_t sel_groups = 0);
 hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, const AttnArgs& a,
                               hipStream_t stream);
+// Prefill attention (prefill_attn.hip): one entry per sequence chunk.
+struct PrefillBatch {
+    int32_t n;
+    int32_t row[BKV_MAX_BATCH];     // block-table row
+    int32_t pos0[BKV_MAX_BATCH];    // position of the chunk's first token
+    int32_t n_tok[BKV_MAX_BATCH];   // tokens of the chunk
+    int32_t src0[BKV_MAX_BATCH];    // first token row in q / out
+    int32_t wg_base[BKV_MAX_BATCH + 1];
+};
+int32_t prefill_rows_per_wg();
+hipError_t launch_prefill_attn(bkv_pool* p, int32_t layer, const PrefillBatch& b, const AttnArgs& a,
+                               hipStream_t stream);
 // heads one wave carries for a given q-heads-per-kv-head group
 int32_t attn_heads_per_wave(int32_t group);
 

@@ -1,0 +1,284 @@
+// Paged causal attention for chunks of many query tokens (prefill) on gfx950 matrix cores.
+// The reference's counterpart is its GQA pair for T >= 16 (crates/breccia-kernels/shaders/
+// qsa_attn_scores_gqa.comp, qsa_attn_apply_gqa.comp; qsa/mod.rs:116-150); the contract is the
+// CPU attend (qsa/cpu.rs:197-246) with the dense selection: query token t of a chunk that
+// starts at pos0 attends cells 0..pos0+t.
+//
+// With hundreds of query rows per kv head the work is a real matrix product (each K/V row is
+// used by every query row behind it), so it goes to MFMA -- unlike the decode kernel, which
+// is a GEMV per sequence.  One wave owns 16 query rows ((token, head) pairs of one kv head)
+// and walks the pages 0..page(pos); per page of 16 cells:
+//   S^T[cell][query] = K[cell][:] . Q[query][:]        v_mfma_f32_16x16x16_f16, A = K, B = Q
+//   online softmax per query (base 2), P^T in the layout S^T came out in
+//   O^T[d][query]   += V^T[d][cell] . P^T[cell][query]  A = V gathered per lane, B = P^T
+// Both products keep the per-lane query (lane % 16) fixed, so the softmax statistics never
+// move between lanes, and P^T feeds the second product straight from registers.  K and V are
+// exact f16; q and p are f32 values split into a high and a low f16 part (two MFMAs each), so
+// the products carry ~22 significant bits and the result stays at f32-accumulate accuracy.
+// The V operand needs four cells of one head-dim column per lane: each lane loads 16 bytes
+// (8 columns) of four rows and regroups them in registers; the 8 MFMAs that use them produce
+// columns 8i + t of the output, i = the MFMA row, t = 0..7.
+#include "bkv_internal.hpp"
+
+namespace bkv {
+
+namespace {
+
+constexpr int kHd = 256;
+constexpr int kPage = 16;
+constexpr int kRowsPerWave = 16;
+constexpr int kWavesPerWg = 4;
+constexpr int kRowsPerWg = kRowsPerWave * kWavesPerWg;
+constexpr float kLog2e = 1.4426950408889634f;
+
+typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+
+struct PrefillKernelParams {
+    PrefillBatch b;
+    const uint8_t* kpool;
+    const uint8_t* vpool;
+    const int32_t* tables;
+    const float* q;     // [sum n_tok][n_q][256]
+    const float* gate;  // optional
+    float* out;         // [sum n_tok][n_q][256]
+    int64_t gate_tok_stride, gate_head_stride;
+    int32_t max_pages_per_seq, n_kv, n_q, group;
+    float scale_log2e;
+};
+
+__device__ __forceinline__ f4 mfma16(h4 a, h4 b, f4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ void split_f16(float x, _Float16& hi, _Float16& lo) {
+    hi = (_Float16)x;
+    lo = (_Float16)(x - (float)hi);
+}
+
+__global__ __launch_bounds__(64 * kWavesPerWg, 2) void prefill_attn_kernel(const PrefillKernelParams P) {
+    // ---- which (entry, kv head, block of 64 query rows) ---------------------------------
+    int e = 0;
+    while (e + 1 < P.b.n && (int)blockIdx.x >= P.b.wg_base[e + 1]) ++e;
+    const int rem = (int)blockIdx.x - P.b.wg_base[e];
+    const int kvh = rem % P.n_kv;
+    const int n_rows = P.b.n_tok[e] * P.group;  // query rows of this kv head
+    const int n_blocks = (n_rows + kRowsPerWg - 1) / kRowsPerWg;
+    // later rows attend more cells: the heaviest blocks are dispatched first
+    const int rb = n_blocks - 1 - rem / P.n_kv;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int c = lane & 15;  // query row of the tile / cell of the page / output column group
+    const int g = lane >> 4;  // which quarter of the contraction index this lane feeds
+    const int row0 = rb * kRowsPerWg + wave * kRowsPerWave;
+    if (row0 >= n_rows) return;
+
+    // this lane's query row
+    const int row = row0 + c;
+    const bool row_live = row < n_rows;
+    const int tok = row_live ? row / P.group : 0;
+    const int head = kvh * P.group + (row_live ? row % P.group : 0);
+    const int pos_q = row_live ? P.b.pos0[e] + tok : -1;
+    // the last token any row of this wave belongs to bounds the page walk
+    const int last_row = min(row0 + kRowsPerWave, n_rows) - 1;
+    const int pos_max = P.b.pos0[e] + last_row / P.group;
+    const int n_pages = pos_max / kPage + 1;
+
+    typedef const __attribute__((address_space(4))) int32_t* table_ptr;
+    const table_ptr bt = (table_ptr)(uintptr_t)(P.tables + (size_t)P.b.row[e] * (size_t)P.max_pages_per_seq);
+    const size_t page_bytes = (size_t)P.n_kv * kPage * kHd * 2;
+    const size_t head_off = (size_t)kvh * kPage * kHd * 2;
+
+    // ---- q fragments: lane (c, g) holds q[row][32 m + 8 g + 0..7], m = 0..7, as hi + lo f16 ----
+    h4 qhi[8][2], qlo[8][2];
+    {
+        const float* qp = P.q + ((size_t)(P.b.src0[e] + tok) * P.n_q + head) * kHd + g * 8;
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+            float x[8];
+            if (row_live) {
+                const float4 a = *reinterpret_cast<const float4*>(qp + m * 32);
+                const float4 b = *reinterpret_cast<const float4*>(qp + m * 32 + 4);
+                x[0] = a.x, x[1] = a.y, x[2] = a.z, x[3] = a.w;
+                x[4] = b.x, x[5] = b.y, x[6] = b.z, x[7] = b.w;
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) x[j] = 0.0f;
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                _Float16 hi, lo;
+                split_f16(x[j], hi, lo);
+                qhi[m][j >> 2][j & 3] = hi;
+                qlo[m][j >> 2][j & 3] = lo;
+            }
+        }
+    }
+
+    // O^T accumulators: o[half][t][r] = out[row][128 half + 8 (4 g + r) + t]
+    f4 o[2][8];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int t = 0; t < 8; ++t) o[h][t] = f4{0.0f, 0.0f, 0.0f, 0.0f};
+    float m_run = -INFINITY;  // running max of this lane's query (base-2 logits), same in all 4 g lanes
+    float l_run = 0.0f;       // this lane's share (its 4 cells per page) of the denominator
+
+    for (int pg = 0; pg < n_pages; ++pg) {
+        const int32_t phys = bt[pg];
+        const uint8_t* kp = P.kpool + (size_t)phys * page_bytes + head_off;
+        const uint8_t* vp = P.vpool + (size_t)phys * page_bytes + head_off;
+        // K: row c, 16 bytes at element 32 m + 8 g (the same split of the head dim as q)
+        v4u kf[8];
+#pragma unroll
+        for (int m = 0; m < 8; ++m)
+            kf[m] = *reinterpret_cast<const v4u*>(kp + (size_t)c * (kHd * 2) + (size_t)(m * 32 + g * 8) * 2);
+        // V: rows 4 g + r, 16 bytes at element 128 half + 8 c
+        v4u vf[2][4];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                vf[h][r] = *reinterpret_cast<const v4u*>(vp + (size_t)(4 * g + r) * (kHd * 2) +
+                                                         (size_t)(h * 128 + c * 8) * 2);
+
+        // ---- S^T = K . Q^T ------------------------------------------------------------------
+        f4 s = f4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+            const h8 k8 = __builtin_bit_cast(h8, kf[m]);
+            const h4 ka = h4{k8[0], k8[1], k8[2], k8[3]};
+            const h4 kb = h4{k8[4], k8[5], k8[6], k8[7]};
+            s = mfma16(ka, qhi[m][0], s);
+            s = mfma16(ka, qlo[m][0], s);
+            s = mfma16(kb, qhi[m][1], s);
+            s = mfma16(kb, qlo[m][1], s);
+        }
+        // s[r] = q[row c] . k[cell 4 g + r]
+
+        // ---- online softmax for this lane's query ------------------------------------------------
+        float t4[4];
+        float pm = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int cell = pg * kPage + 4 * g + r;
+            t4[r] = cell <= pos_q ? s[r] * P.scale_log2e : -INFINITY;
+            pm = fmaxf(pm, t4[r]);
+        }
+        pm = fmaxf(pm, __shfl_xor(pm, 16, 64));
+        pm = fmaxf(pm, __shfl_xor(pm, 32, 64));
+        const float m_new = fmaxf(m_run, pm);
+        // a query with no live cell yet keeps m = -inf: exp2(-inf - -inf) would be NaN
+        const float alpha = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
+        h4 phi, plo;
+        float psum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float p = m_new == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(t4[r] - m_new);
+            psum += p;
+            _Float16 hi, lo;
+            split_f16(p, hi, lo);
+            phi[r] = hi;
+            plo[r] = lo;
+        }
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int t = 0; t < 8; ++t) o[h][t] *= alpha;
+        }
+
+        // Rows past the last position of this wave were never written for these queries and may
+        // hold anything (even NaN): make them exact zeros before they meet a zero probability.
+        if (pg == n_pages - 1) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (pg * kPage + 4 * g + r > pos_max) {
+                    vf[0][r] = v4u{0u, 0u, 0u, 0u};
+                    vf[1][r] = v4u{0u, 0u, 0u, 0u};
+                }
+        }
+
+        // ---- O^T += V^T . P^T ---------------------------------------------------------------------
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const h8 v0 = __builtin_bit_cast(h8, vf[h][0]), v1 = __builtin_bit_cast(h8, vf[h][1]);
+            const h8 v2 = __builtin_bit_cast(h8, vf[h][2]), v3 = __builtin_bit_cast(h8, vf[h][3]);
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const h4 va = h4{v0[t], v1[t], v2[t], v3[t]};  // column 128 h + 8 c + t of cells 4 g ..
+                o[h][t] = mfma16(va, phi, o[h][t]);
+                o[h][t] = mfma16(va, plo, o[h][t]);
+            }
+        }
+    }
+
+    // ---- normalise, gate, store ---------------------------------------------------------------------
+    l_run += __shfl_xor(l_run, 16, 64);
+    l_run += __shfl_xor(l_run, 32, 64);
+    if (!row_live) return;
+    const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
+    float* op = P.out + ((size_t)(P.b.src0[e] + tok) * P.n_q + head) * kHd;
+    const float* gp = P.gate ? P.gate + (size_t)(P.b.src0[e] + tok) * P.gate_tok_stride +
+                                   (size_t)head * P.gate_head_stride
+                             : nullptr;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int d0 = h * 128 + 8 * (4 * g + r);
+            float y[8];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                y[t] = o[h][t][r] * inv;
+                if (gp) {
+                    // sigmoid in the overflow-free form of the reference (qsa/cpu.rs:84-91)
+                    const float gt = gp[d0 + t];
+                    float sg;
+                    if (gt >= 0.0f) {
+                        sg = 1.0f / (1.0f + expf(-gt));
+                    } else {
+                        const float ex = expf(gt);
+                        sg = ex / (1.0f + ex);
+                    }
+                    y[t] *= sg;
+                }
+            }
+            *reinterpret_cast<float4*>(op + d0) = make_float4(y[0], y[1], y[2], y[3]);
+            *reinterpret_cast<float4*>(op + d0 + 4) = make_float4(y[4], y[5], y[6], y[7]);
+        }
+}
+
+}  // namespace
+
+int32_t prefill_rows_per_wg() { return kRowsPerWg; }
+
+hipError_t launch_prefill_attn(bkv_pool* p, int32_t layer, const PrefillBatch& b, const AttnArgs& a,
+                               hipStream_t stream) {
+    PrefillKernelParams kp;
+    kp.b = b;
+    kp.kpool = p->k_layer[(size_t)layer];
+    kp.vpool = p->v_layer[(size_t)layer];
+    kp.tables = p->table_dev;
+    kp.q = a.q;
+    kp.gate = a.gate;
+    kp.out = a.out;
+    kp.gate_tok_stride = a.gate_seq_stride;
+    kp.gate_head_stride = a.gate_head_stride;
+    kp.max_pages_per_seq = p->desc.max_pages_per_seq;
+    kp.n_kv = p->g.n_kv;
+    kp.n_q = a.n_q_head;
+    kp.group = a.n_q_head / p->g.n_kv;
+    kp.scale_log2e = a.scale * kLog2e;
+    const int32_t grid = b.wg_base[b.n];
+    if (grid == 0) return hipSuccess;
+    StageScope timed(p, BKV_STAGE_ATTN_SPLIT, stream);
+    prefill_attn_kernel<<<grid, 64 * kWavesPerWg, 0, stream>>>(kp);
+    return hipGetLastError();
+}
+
+}  // namespace bkv

@@ -335,6 +335,17 @@ class Pool:
                                   _ptr(gate_dev), gate_seq_stride, gate_head_stride, scale,
                                   _ptr(out_dev), _sh(stream)))
 
+    def prefill_attn(self, layer: int, seqs, pos0, n_tokens, n_q_head: int, q_dev, out_dev, scale: float,
+                     gate_dev=None, gate_tok_stride: int = 0, gate_head_stride: int = 0, stream=None) -> None:
+        """Causal attention of whole chunks (token t of chunk i sees cells 0..pos0[i]+t), on MFMA."""
+        seqs, ps = _i32(seqs)
+        pos0, pp = _i64(pos0)
+        n_tokens, pn = _i32(n_tokens)
+        assert seqs.size == pos0.size == n_tokens.size
+        check(lib.bkv_prefill_attn(self.handle, layer, seqs.size, ps, pp, pn, n_q_head, _ptr(q_dev),
+                                   _ptr(gate_dev), gate_tok_stride, gate_head_stride, scale, _ptr(out_dev),
+                                   _sh(stream)))
+
     def decode_step(self, layer: int, seqs, pos, k_new_dev, v_new_dev, n_q_head: int, q_dev, out_dev,
                     scale: float, gate_dev=None, gate_seq_stride: int = 0, gate_head_stride: int = 0,
                     stream=None) -> None:

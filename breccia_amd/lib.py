@@ -92,6 +92,8 @@ _SIGNATURES = {
     "bkv_rope_table": (C.c_int, [C.c_double, _i32, _i32, _vp]),
     "bkv_decode_attn": (C.c_int, [_vp, _i32, _i32, _pi32, _pi64, _i32, _vp, _vp, _i64, _i64, _f32,
                                   _vp, _vp]),
+    "bkv_prefill_attn": (C.c_int, [_vp, _i32, _i32, _pi32, _pi64, _pi32, _i32, _vp, _vp, _i64, _i64, _f32,
+                                   _vp, _vp]),
     "bkv_decode_step": (C.c_int, [_vp, _i32, _i32, _pi32, _pi64, _vp, _vp, _i32, _vp, _vp, _i64, _i64, _f32,
                                   _vp, _vp]),
     "bkv_decode_attn_select": (C.c_int, [_vp, _i32, _i32, _pi32, _pi64, _i32, _vp, _vp, _i64, _i64, _f32,

@@ -235,6 +235,21 @@ bkv_status bkv_decode_attn(bkv_pool *pool, int32_t layer, int32_t n, const int32
                            const float *gate_dev, int64_t gate_seq_stride,
                            int64_t gate_head_stride, float scale, float *out_dev, void *stream);
 
+/* Causal attention for chunks of many query tokens (prefill), on the matrix cores: the
+ * reference's GQA pair for T >= 16 (shaders/qsa_attn_scores_gqa.comp, qsa_attn_apply_gqa.comp;
+ * qsa/mod.rs:116-150), same contract as bkv_decode_attn (oracle qsa/cpu.rs:197-246, dense
+ * selection): token t of chunk i, at position pos0[i] + t, attends cells 0..pos0[i]+t of
+ * sequence seqs[i].  The chunk's own K/V must have been appended first.  q, out: device f32
+ * [sum n_tokens][n_q_head][head_dim], chunks concatenated in call order; gate(token, h, d) =
+ * gate_dev[token*gate_tok_stride + h*gate_head_stride + d] or NULL.  K and V enter the MFMAs
+ * as the exact f16 the cache holds; q and the probabilities are f32 split into two f16 parts,
+ * so accuracy is that of f32 accumulation.  f16 pools, head_dim 256, 16-cell pages.  Written
+ * for chunks of tens to thousands of tokens; a handful of tokens is bkv_decode_attn's case. */
+bkv_status bkv_prefill_attn(bkv_pool *pool, int32_t layer, int32_t n_seqs, const int32_t *seqs,
+                            const int64_t *pos0, const int32_t *n_tokens, int32_t n_q_head,
+                            const float *q_dev, const float *gate_dev, int64_t gate_tok_stride,
+                            int64_t gate_head_stride, float scale, float *out_dev, void *stream);
+
 /* One decode step in one call: append the new token's K/V row of every listed sequence at cell
  * pos[i] and attend cells 0..pos[i] -- bkv_append of one token per sequence followed by
  * bkv_decode_attn, without the append launch (Qsa::kv_append + Qsa::attend + Qsa::apply of

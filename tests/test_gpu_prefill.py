@@ -1,0 +1,119 @@
+"""GPU parity of the MFMA prefill attention (causal attention of whole chunks over the paged
+cache) against the CPU oracle, token by token, and against the decode kernel.  Tolerances as in
+test_gpu_attn.py, including the reference's own 1e-5 bar."""
+import numpy as np
+import pytest
+
+from breccia_amd import lib as L
+from breccia_amd.kv import BkvError, DeviceBuffer
+from gpu_common import REF_BAR_MAX_REL, Twin, check_attn
+from helpers import max_abs
+from test_gpu_attn import fill
+
+pytestmark = pytest.mark.gpu
+
+
+def prefill(tw, layer, seqs, pos0, q_list, n_head, gate_list=None):
+    """q_list[i]: [T_i, n_head, 256] -> list of outputs of the same shapes (one call)."""
+    n_tok = [q.shape[0] for q in q_list]
+    qcat = np.ascontiguousarray(np.concatenate([q.reshape(-1) for q in q_list] + [np.zeros(4, np.float32)]),
+                                dtype=np.float32)
+    qd, od = DeviceBuffer.from_numpy(qcat), DeviceBuffer(qcat.nbytes)
+    gd = None
+    if gate_list is not None:
+        gd = DeviceBuffer.from_numpy(np.concatenate([g.reshape(-1) for g in gate_list] + [np.zeros(4, np.float32)]))
+    try:
+        tw.pool.prefill_attn(layer, seqs, pos0, n_tok, n_head, qd, od, 1.0 / 16.0, gate_dev=gd,
+                             gate_tok_stride=n_head * 256 if gd else 0, gate_head_stride=256 if gd else 0)
+        flat = od.download(np.float32, qcat.size)
+    finally:
+        for b in (qd, od, gd):
+            if b is not None:
+                b.free()
+    outs, at = [], 0
+    for t in n_tok:
+        outs.append(flat[at:at + t * n_head * 256].reshape(t, n_head, 256))
+        at += t * n_head * 256
+    return outs
+
+
+@pytest.mark.parametrize("n_q", [16, 24])
+def test_chunks_match_the_oracle_token_by_token(n_q):
+    rng = np.random.Generator(np.random.PCG64(1000 + n_q))
+    # (cells before the chunk, chunk length): from scratch, on a prefix, single token, page edges
+    cases = [(0, 100), (517, 300), (64, 1), (15, 17), (2048, 130)]
+    with Twin(n_pages=400, max_seqs=8) as tw:
+        tw.pool.set_free_order(rng.permutation(400).astype(np.int32))
+        seqs = [tw.pool.seq_create() for _ in cases]
+        for s, (before, t) in zip(seqs, cases):
+            fill(tw, s, before + t, rng, chunk=1024)            # the chunk's own K/V are in the cache
+        qs = [rng.standard_normal((t, n_q, 256)).astype(np.float32) for _, t in cases]
+        gates = [rng.standard_normal((t, n_q, 256)).astype(np.float32) for _, t in cases]
+        outs = prefill(tw, 0, seqs, [b for b, _ in cases], qs, n_q, gates)
+        worst = 0.0
+        for s, (before, t), q, g, out in zip(seqs, cases, qs, gates, outs):
+            picks = sorted(set([0, t - 1, t // 2] + [int(x) for x in rng.integers(0, t, size=6)] +
+                               [i for i in range(t) if (before + i) % 16 in (0, 15)][:6]))
+            for i in picks:
+                want = tw.oracle_attend(0, s, before + i, q[i], n_q, gate=g[i])
+                _, rel = check_attn(out[i], want, "chunk at %d, token %d" % (before, i))
+                worst = max(worst, rel)
+        assert worst <= REF_BAR_MAX_REL, worst
+        # the decode kernel on the same positions agrees to f32 noise
+        s, (before, t) = seqs[1], cases[1]
+        pos = list(range(before + t - 40, before + t))
+        dec = tw.decode_attn(0, [s] * 40, pos, qs[1][-40:], n_q, scale=1.0 / 16.0, gate=gates[1][-40:])
+        assert max_abs(dec, outs[1][-40:]) < 5e-6
+
+
+def test_prefill_ignores_poisoned_cells_and_future_tokens():
+    rng = np.random.Generator(np.random.PCG64(1010))
+    with Twin(n_pages=64, max_seqs=4) as tw:
+        s = tw.pool.seq_create()
+        fill(tw, s, 200, rng, chunk=200)
+        # attend a chunk that ends before the cache does (tokens 100..149): cells 150..199 are real
+        # but in the future; cells 200..207 of the last page hold NaN patterns
+        kp = tw.pool.read_layer(0, 0).view(np.uint16).copy()
+        vp = tw.pool.read_layer(0, 1).view(np.uint16).copy()
+        t = tw.pool.block_table(s)
+        for c in range(200, 208):
+            for h in range(2):
+                row = ((int(t[c // 16]) * 2 + h) * 16 + c % 16) * 256
+                kp[row:row + 256] = 0x7E00
+                vp[row:row + 256] = 0xFE01
+        tw.pool.write_layer(0, 0, kp.view(np.uint8))
+        tw.pool.write_layer(0, 1, vp.view(np.uint8))
+        q = rng.standard_normal((50, 16, 256)).astype(np.float32)
+        out = prefill(tw, 0, [s], [100], [q], 16)[0]
+        assert np.all(np.isfinite(out))
+        for i in (0, 11, 27, 49):
+            check_attn(out[i], tw.oracle_attend(0, s, 100 + i, q[i], 16), "token %d" % i)
+        # a chunk that ends exactly at the poisoned page's last live cell
+        q2 = rng.standard_normal((9, 16, 256)).astype(np.float32)
+        out2 = prefill(tw, 0, [s], [191], [q2], 16)[0]
+        assert np.all(np.isfinite(out2))
+        check_attn(out2[8], tw.oracle_attend(0, s, 199, q2[8], 16), "last cell")
+
+
+def test_prefill_errors_come_before_any_launch():
+    with Twin(n_pages=8, max_seqs=2) as tw:
+        s = tw.pool.seq_create()
+        tw.pool.seq_reserve(s, 40)
+        z = DeviceBuffer(1 << 20)
+        for kw, status in [(dict(pos0=[30], n_tokens=[19]), L.ERR_RANGE), (dict(n_q_head=15), L.ERR_INVALID),
+                           (dict(q_dev=None), L.ERR_INVALID), (dict(layer=2), L.ERR_RANGE),
+                           (dict(seqs=[1]), L.ERR_RANGE)]:
+            a = dict(layer=0, seqs=[s], pos0=[0], n_tokens=[40], n_q_head=16, q_dev=z, out_dev=z, scale=0.0625)
+            a.update(kw)
+            with pytest.raises(BkvError) as ei:
+                tw.pool.prefill_attn(**a)
+            assert ei.value.status == status, kw
+        z.free()
+    with Twin(n_pages=8, max_seqs=2, layout=L.LAYOUT_Q8V) as tw:
+        s = tw.pool.seq_create()
+        tw.pool.seq_reserve(s, 40)
+        z = DeviceBuffer(1 << 20)
+        with pytest.raises(BkvError) as ei:
+            tw.pool.prefill_attn(0, [s], [0], [40], 16, z, z, 0.0625)
+        assert ei.value.status == L.ERR_INVALID
+        z.free()
