@@ -6,8 +6,12 @@
 //
 // With hundreds of query rows per kv head the work is a real matrix product (each K/V row is
 // used by every query row behind it), so it goes to MFMA -- unlike the decode kernel, which
-// is a GEMV per sequence.  One wave owns 16 query rows ((token, head) pairs of one kv head)
-// and walks the pages 0..page(pos); per page of 16 cells:
+// is a GEMV per sequence.  A work-group of four waves owns 64 consecutive query rows ((token,
+// head) pairs of one kv head), 16 per wave, and walks the pages 0..page(pos) together: each
+// page's K and V rows are fetched from memory once per work-group into LDS (double-buffered,
+// the next page in flight while the current one is multiplied; fetching them per wave ran into
+// the L2's bandwidth), and every wave takes its operand fragments from there.  Per page of 16
+// cells and per wave:
 //   S^T[cell][query] = K[cell][:] . Q[query][:]        v_mfma_f32_16x16x16_f16, A = K, B = Q
 //   online softmax per query (base 2), P^T in the layout S^T came out in
 //   O^T[d][query]   += V^T[d][cell] . P^T[cell][query]  A = V gathered per lane, B = P^T
@@ -30,6 +34,7 @@ constexpr int kRowsPerWave = 16;
 constexpr int kWavesPerWg = 4;
 constexpr int kRowsPerWg = kRowsPerWave * kWavesPerWg;
 constexpr float kLog2e = 1.4426950408889634f;
+constexpr int kLdsRow = kHd + 8;  // halves per row of a page image in LDS (528 bytes)
 
 typedef _Float16 h4 __attribute__((ext_vector_type(4)));
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
@@ -73,18 +78,22 @@ __global__ __launch_bounds__(64 * kWavesPerWg, 2) void prefill_attn_kernel(const
     const int c = lane & 15;  // query row of the tile / cell of the page / output column group
     const int g = lane >> 4;  // which quarter of the contraction index this lane feeds
     const int row0 = rb * kRowsPerWg + wave * kRowsPerWave;
-    if (row0 >= n_rows) return;
+    // a wave whose rows lie past the end still helps to fetch pages and joins the barriers
+    const bool wave_live = row0 < n_rows;
 
     // this lane's query row
     const int row = row0 + c;
-    const bool row_live = row < n_rows;
+    const bool row_live = wave_live && row < n_rows;
     const int tok = row_live ? row / P.group : 0;
     const int head = kvh * P.group + (row_live ? row % P.group : 0);
     const int pos_q = row_live ? P.b.pos0[e] + tok : -1;
     // the last token any row of this wave belongs to bounds the page walk
     const int last_row = min(row0 + kRowsPerWave, n_rows) - 1;
-    const int pos_max = P.b.pos0[e] + last_row / P.group;
-    const int n_pages = pos_max / kPage + 1;
+    const int pos_max = wave_live ? P.b.pos0[e] + last_row / P.group : -1;
+    const int n_pages = wave_live ? pos_max / kPage + 1 : 0;
+    // pages the work-group walks: those of its last row
+    const int wg_last_row = min(rb * kRowsPerWg + kRowsPerWg, n_rows) - 1;
+    const int wg_pages = (P.b.pos0[e] + wg_last_row / P.group) / kPage + 1;
 
     typedef const __attribute__((address_space(4))) int32_t* table_ptr;
     const table_ptr bt = (table_ptr)(uintptr_t)(P.tables + (size_t)P.b.row[e] * (size_t)P.max_pages_per_seq);
@@ -126,36 +135,50 @@ __global__ __launch_bounds__(64 * kWavesPerWg, 2) void prefill_attn_kernel(const
     float m_run = -INFINITY;  // running max of this lane's query (base-2 logits), same in all 4 g lanes
     float l_run = 0.0f;       // this lane's share (its 4 cells per page) of the denominator
 
-    for (int pg = 0; pg < n_pages; ++pg) {
+    // ---- pages through LDS: [buffer][K | V][16 rows][264 halves] -------------------------------
+    // Rows are padded to 528 bytes so that the 16-byte fragment reads of the 64 lanes spread
+    // evenly over the banks.  A page image is 2 x 512 chunks of 16 bytes: thread t moves chunks
+    // t and t + 256 of K and of V.
+    __shared__ __attribute__((aligned(16))) _Float16 lds[2][2][kPage][kLdsRow];
+    const int tid = threadIdx.x;
+    v4u stage[4];
+    const auto fetch = [&](int pg) {
         const int32_t phys = bt[pg];
         const uint8_t* kp = P.kpool + (size_t)phys * page_bytes + head_off;
         const uint8_t* vp = P.vpool + (size_t)phys * page_bytes + head_off;
-        // K: row c, 16 bytes at element 32 m + 8 g (the same split of the head dim as q)
-        v4u kf[8];
-#pragma unroll
-        for (int m = 0; m < 8; ++m)
-            kf[m] = *reinterpret_cast<const v4u*>(kp + (size_t)c * (kHd * 2) + (size_t)(m * 32 + g * 8) * 2);
-        // V: rows 4 g + r, 16 bytes at element 128 half + 8 c
-        v4u vf[2][4];
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-                vf[h][r] = *reinterpret_cast<const v4u*>(vp + (size_t)(4 * g + r) * (kHd * 2) +
-                                                         (size_t)(h * 128 + c * 8) * 2);
+        stage[0] = *reinterpret_cast<const v4u*>(kp + (size_t)tid * 16);
+        stage[1] = *reinterpret_cast<const v4u*>(kp + (size_t)(tid + 256) * 16);
+        stage[2] = *reinterpret_cast<const v4u*>(vp + (size_t)tid * 16);
+        stage[3] = *reinterpret_cast<const v4u*>(vp + (size_t)(tid + 256) * 16);
+    };
+    const auto deposit = [&](int buf) {
+        // chunk q of a page image: row q / 32, halves (q % 32) * 8 ..
+        *reinterpret_cast<v4u*>(&lds[buf][0][tid >> 5][(tid & 31) * 8]) = stage[0];
+        *reinterpret_cast<v4u*>(&lds[buf][0][(tid >> 5) + 8][(tid & 31) * 8]) = stage[1];
+        *reinterpret_cast<v4u*>(&lds[buf][1][tid >> 5][(tid & 31) * 8]) = stage[2];
+        *reinterpret_cast<v4u*>(&lds[buf][1][(tid >> 5) + 8][(tid & 31) * 8]) = stage[3];
+    };
 
+    // one page of this wave: scores -> softmax -> accumulate, operands from LDS buffer `buf`
+    const auto process = [&](int pg, int buf) {
+        const _Float16* ks = &lds[buf][0][0][0];
+        const _Float16* vs = &lds[buf][1][0][0];
         // ---- S^T = K . Q^T ------------------------------------------------------------------
-        f4 s = f4{0.0f, 0.0f, 0.0f, 0.0f};
+        // four independent accumulation chains: an MFMA that waits for the previous one's result
+        // costs its full latency
+        f4 s0 = f4{0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0, s2 = s0, s3 = s0;
 #pragma unroll
         for (int m = 0; m < 8; ++m) {
-            const h8 k8 = __builtin_bit_cast(h8, kf[m]);
+            // K: row c, 16 bytes at element 32 m + 8 g (the same split of the head dim as q)
+            const h8 k8 = *reinterpret_cast<const h8*>(ks + c * kLdsRow + m * 32 + g * 8);
             const h4 ka = h4{k8[0], k8[1], k8[2], k8[3]};
             const h4 kb = h4{k8[4], k8[5], k8[6], k8[7]};
-            s = mfma16(ka, qhi[m][0], s);
-            s = mfma16(ka, qlo[m][0], s);
-            s = mfma16(kb, qhi[m][1], s);
-            s = mfma16(kb, qlo[m][1], s);
+            s0 = mfma16(ka, qhi[m][0], s0);
+            s1 = mfma16(ka, qlo[m][0], s1);
+            s2 = mfma16(kb, qhi[m][1], s2);
+            s3 = mfma16(kb, qlo[m][1], s3);
         }
+        const f4 s = (s0 + s1) + (s2 + s3);
         // s[r] = q[row c] . k[cell 4 g + r]
 
         // ---- online softmax for this lane's query ------------------------------------------------
@@ -194,6 +217,13 @@ __global__ __launch_bounds__(64 * kWavesPerWg, 2) void prefill_attn_kernel(const
 
         // Rows past the last position of this wave were never written for these queries and may
         // hold anything (even NaN): make them exact zeros before they meet a zero probability.
+        // V: rows 4 g + r, 16 bytes at element 128 half + 8 c
+        v4u vf[2][4];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                vf[h][r] = *reinterpret_cast<const v4u*>(vs + (4 * g + r) * kLdsRow + h * 128 + c * 8);
         if (pg == n_pages - 1) {
 #pragma unroll
             for (int r = 0; r < 4; ++r)
@@ -215,6 +245,18 @@ __global__ __launch_bounds__(64 * kWavesPerWg, 2) void prefill_attn_kernel(const
                 o[h][t] = mfma16(va, plo, o[h][t]);
             }
         }
+    };
+
+    fetch(0);
+    deposit(0);
+    __syncthreads();
+    for (int pg = 0; pg < wg_pages; ++pg) {
+        // the next page travels while this one is multiplied (past the end: the last page again)
+        fetch(min(pg + 1, wg_pages - 1));
+        if (pg < n_pages) process(pg, pg & 1);
+        deposit((pg + 1) & 1);
+        // after the barrier the other buffer is complete, and nobody reads this one any more
+        __syncthreads();
     }
 
     // ---- normalise, gate, store ---------------------------------------------------------------------
