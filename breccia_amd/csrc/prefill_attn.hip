@@ -12,9 +12,10 @@
 // the next page in flight while the current one is multiplied; fetching them per wave ran into
 // the L2's bandwidth), and every wave takes its operand fragments from there.  Per page of 16
 // cells and per wave:
-//   S^T[cell][query] = K[cell][:] . Q[query][:]        v_mfma_f32_16x16x16_f16, A = K, B = Q
+//   S^T[cell][query] = K[cell][:] . Q[query][:]        v_mfma_f32_16x16x32_f16, A = K, B = Q
 //   online softmax per query (base 2), P^T in the layout S^T came out in
-//   O^T[d][query]   += V^T[d][cell] . P^T[cell][query]  A = V gathered per lane, B = P^T
+//   O^T[d][query]   += V^T[d][cell] . P^T[cell][query]  v_mfma_f32_16x16x16_f16 (a page is 16
+//                                                       cells), A = V gathered per lane, B = P^T
 // Both products keep the per-lane query (lane % 16) fixed, so the softmax statistics never
 // move between lanes, and P^T feeds the second product straight from registers.  K and V are
 // exact f16; q and p are f32 values split into a high and a low f16 part (two MFMAs each), so
@@ -56,6 +57,10 @@ struct PrefillKernelParams {
 
 __device__ __forceinline__ f4 mfma16(h4 a, h4 b, f4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x16f16(a, b, c, 0, 0, 0);
+}
+// gfx950's double-depth form: 32 contraction steps, 8 halves per lane (k = 8 (lane / 16) + 0..7)
+__device__ __forceinline__ f4 mfma32(h8 a, h8 b, f4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
 }
 
 __device__ __forceinline__ void split_f16(float x, _Float16& hi, _Float16& lo) {
@@ -101,7 +106,7 @@ __global__ __launch_bounds__(64 * kWavesPerWg, 2) void prefill_attn_kernel(const
     const size_t head_off = (size_t)kvh * kPage * kHd * 2;
 
     // ---- q fragments: lane (c, g) holds q[row][32 m + 8 g + 0..7], m = 0..7, as hi + lo f16 ----
-    h4 qhi[8][2], qlo[8][2];
+    h8 qhi[8], qlo[8];
     {
         const float* qp = P.q + ((size_t)(P.b.src0[e] + tok) * P.n_q + head) * kHd + g * 8;
 #pragma unroll
@@ -120,8 +125,8 @@ __global__ __launch_bounds__(64 * kWavesPerWg, 2) void prefill_attn_kernel(const
             for (int j = 0; j < 8; ++j) {
                 _Float16 hi, lo;
                 split_f16(x[j], hi, lo);
-                qhi[m][j >> 2][j & 3] = hi;
-                qlo[m][j >> 2][j & 3] = lo;
+                qhi[m][j] = hi;
+                qlo[m][j] = lo;
             }
         }
     }
@@ -141,8 +146,7 @@ __global__ __launch_bounds__(64 * kWavesPerWg, 2) void prefill_attn_kernel(const
     // t and t + 256 of K and of V.
     __shared__ __attribute__((aligned(16))) _Float16 lds[2][2][kPage][kLdsRow];
     const int tid = threadIdx.x;
-    v4u stage[4];
-    const auto fetch = [&](int pg) {
+    const auto fetch = [&](int pg, v4u (&stage)[4]) {
         const int32_t phys = bt[pg];
         const uint8_t* kp = P.kpool + (size_t)phys * page_bytes + head_off;
         const uint8_t* vp = P.vpool + (size_t)phys * page_bytes + head_off;
@@ -151,7 +155,7 @@ __global__ __launch_bounds__(64 * kWavesPerWg, 2) void prefill_attn_kernel(const
         stage[2] = *reinterpret_cast<const v4u*>(vp + (size_t)tid * 16);
         stage[3] = *reinterpret_cast<const v4u*>(vp + (size_t)(tid + 256) * 16);
     };
-    const auto deposit = [&](int buf) {
+    const auto deposit = [&](int buf, const v4u (&stage)[4]) {
         // chunk q of a page image: row q / 32, halves (q % 32) * 8 ..
         *reinterpret_cast<v4u*>(&lds[buf][0][tid >> 5][(tid & 31) * 8]) = stage[0];
         *reinterpret_cast<v4u*>(&lds[buf][0][(tid >> 5) + 8][(tid & 31) * 8]) = stage[1];
@@ -168,15 +172,15 @@ __global__ __launch_bounds__(64 * kWavesPerWg, 2) void prefill_attn_kernel(const
         // costs its full latency
         f4 s0 = f4{0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0, s2 = s0, s3 = s0;
 #pragma unroll
-        for (int m = 0; m < 8; ++m) {
-            // K: row c, 16 bytes at element 32 m + 8 g (the same split of the head dim as q)
-            const h8 k8 = *reinterpret_cast<const h8*>(ks + c * kLdsRow + m * 32 + g * 8);
-            const h4 ka = h4{k8[0], k8[1], k8[2], k8[3]};
-            const h4 kb = h4{k8[4], k8[5], k8[6], k8[7]};
-            s0 = mfma16(ka, qhi[m][0], s0);
-            s1 = mfma16(ka, qlo[m][0], s1);
-            s2 = mfma16(kb, qhi[m][1], s2);
-            s3 = mfma16(kb, qlo[m][1], s3);
+        for (int m = 0; m < 8; m += 2) {
+            // K: row c, 16 bytes at element 32 m + 8 g (the same split of the head dim as q): the
+            // 8 halves of a lane are the 8 contraction steps it feeds to the 32-deep MFMA
+            const h8 ka = *reinterpret_cast<const h8*>(ks + c * kLdsRow + m * 32 + g * 8);
+            const h8 kb = *reinterpret_cast<const h8*>(ks + c * kLdsRow + (m + 1) * 32 + g * 8);
+            s0 = mfma32(ka, qhi[m], s0);
+            s1 = mfma32(ka, qlo[m], s1);
+            s2 = mfma32(kb, qhi[m + 1], s2);
+            s3 = mfma32(kb, qlo[m + 1], s3);
         }
         const f4 s = (s0 + s1) + (s2 + s3);
         // s[r] = q[row c] . k[cell 4 g + r]
@@ -247,15 +251,24 @@ __global__ __launch_bounds__(64 * kWavesPerWg, 2) void prefill_attn_kernel(const
         }
     };
 
-    fetch(0);
-    deposit(0);
+    // Two pages are in flight behind the one being multiplied: staging set A carries the even
+    // pages, B the odd ones (past the end they carry the last page again).
+    v4u stage_a[4], stage_b[4];
+    const int last_pg = wg_pages - 1;
+    fetch(0, stage_a);
+    fetch(min(1, last_pg), stage_b);
+    deposit(0, stage_a);
+    fetch(min(2, last_pg), stage_a);
     __syncthreads();
-    for (int pg = 0; pg < wg_pages; ++pg) {
-        // the next page travels while this one is multiplied (past the end: the last page again)
-        fetch(min(pg + 1, wg_pages - 1));
-        if (pg < n_pages) process(pg, pg & 1);
-        deposit((pg + 1) & 1);
+    for (int pg = 0; pg < wg_pages; pg += 2) {
+        if (pg < n_pages) process(pg, 0);
+        deposit(1, stage_b);                      // page pg + 1
+        fetch(min(pg + 3, last_pg), stage_b);
         // after the barrier the other buffer is complete, and nobody reads this one any more
+        __syncthreads();
+        if (pg + 1 < n_pages) process(pg + 1, 1);
+        deposit(0, stage_a);                      // page pg + 2
+        fetch(min(pg + 4, last_pg), stage_a);
         __syncthreads();
     }
 
