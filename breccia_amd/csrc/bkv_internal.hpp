@@ -184,10 +184,13 @@ struct AttnArgs {
     // fused decode step: new rows [n][n_kv][head_dim] f32; nullptr = plain attention
     const float* new_k = nullptr;
     const float* new_v = nullptr;
+    bool mfma = false;  // dense f16 call routed to the MFMA kernel (all heads of a group at once)
 };
 // Fills wg_base/splits/pps from row/pos; returns the total work-group count.  sel_groups > 0:
 // every entry is planned for that many groups of four selected blocks instead of its pages.
-int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b, int32_t sel_groups = 0);
+int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b, int32_t sel_groups = 0,
+                  bool mfma = false);
+bool attn_on_mfma(const bkv_pool* p, int32_t group);
 hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, const AttnArgs& a,
                               hipStream_t stream);
 // Prefill attention (prefill_attn.hip): one entry per sequence chunk.

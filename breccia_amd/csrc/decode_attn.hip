@@ -649,6 +649,300 @@ __global__ __launch_bounds__(kBlock, HG == 8 ? 2 : 3) void decode_attn_kernel(co
     }
 }
 
+// ---- decode attention on the matrix cores -----------------------------------------------------
+// The same split-K decomposition and the same partial-result layout as decode_attn_kernel, for
+// f16 pools and head groups the 8- or 4-head VALU kernel would have to walk in several chunks
+// (the reference's own 24 q / 2 kv heads = 12 per group; 32 / 2 = 16): a 16-column MFMA tile
+// holds up to 16 heads of a kv head at once, every K/V row is still read once, and the VALU
+// only does the softmax.  Lane (c = lane % 16, g = lane / 16) of a wave owns head c; per page:
+//   S^T[cell][head] = K[cell][:] . q[head][:]          v_mfma_f32_16x16x32_f16, A = K, B = q
+//   O^T[d][head]   += V^T[d][cell] . P^T[cell][head]   v_mfma_f32_16x16x16_f16, A = V regrouped
+// with q and p split into a high and a low f16 part (K and V are exact f16), as in the prefill
+// kernel.  K fragment m of a lane is the 16 bytes at element 32 m + 8 g of row c; V fragments
+// are the 16 bytes at element 128 h + 8 c of rows 4 g + r.  Every fragment register is
+// refilled with the next page's data right after its last use.
+typedef _Float16 h4m __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void split_hi_lo(float x, _Float16& hi, _Float16& lo) {
+    hi = (_Float16)x;
+    lo = (_Float16)(x - (float)hi);
+}
+
+constexpr int kOwStride = kHd + 4;  // floats per head in the wave-merge staging
+
+// STEP: the row of cell pos comes from the caller's f32 K/V (stored under the f16 rule into the
+// pool on the way), as in decode_attn_kernel<..., STEP = true>.
+template <bool STEP>
+__global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnKernelParams P) {
+    __shared__ __attribute__((aligned(16))) float ow[2][16][kOwStride];
+    __shared__ float wave_m[kWaves][16];
+    __shared__ float wave_l[kWaves][16];
+
+    // ---- which (entry, kv head, page range); one work-group per unit (no head chunks) --------
+    const int unit = blockIdx.x;
+    int e = 0;
+    while (e + 1 < P.b.n && unit >= P.b.wg_base[e + 1]) ++e;
+    const int rem = unit - P.b.wg_base[e];
+    const int split = rem / P.n_kv;
+    const int kvh = rem - split * P.n_kv;
+    const int wg = unit;
+    const int pos = P.b.pos[e];
+    const int n_pages = pos / kPage + 1;
+    const int pps = P.b.pps[e];
+    const int pg0 = split * pps;
+    const int pg1 = min(pg0 + pps, n_pages);
+    typedef const __attribute__((address_space(4))) int32_t* table_ptr;
+    const table_ptr bt = (table_ptr)(uintptr_t)(P.tables + (size_t)P.b.row[e] * (size_t)P.max_pages_per_seq);
+
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int c = lane & 15;
+    const int g = lane >> 4;
+    const size_t page_bytes = (size_t)P.n_kv * kPage * kHd * 2;
+    const size_t head_off = (size_t)kvh * kPage * kHd * 2;
+
+    const auto k_addr = [&](const uint8_t* page, int m) {
+        return reinterpret_cast<const v4u*>(page + (size_t)c * (kHd * 2) + (size_t)(m * 32 + g * 8) * 2);
+    };
+    const auto v_addr = [&](const uint8_t* page, int h, int r) {
+        return reinterpret_cast<const v4u*>(page + (size_t)(4 * g + r) * (kHd * 2) + (size_t)(h * 128 + c * 8) * 2);
+    };
+
+    int pg = pg0 + wave;
+    v4u kf[8], vf[2][4];
+    if (pg < pg1) {
+        const int32_t phys = bt[pg];
+        const uint8_t* kp = P.kpool + (size_t)phys * page_bytes + head_off;
+        const uint8_t* vp = P.vpool + (size_t)phys * page_bytes + head_off;
+#pragma unroll
+        for (int m = 0; m < 8; ++m) kf[m] = __builtin_nontemporal_load(k_addr(kp, m));
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) vf[h][r] = __builtin_nontemporal_load(v_addr(vp, h, r));
+    }
+
+    // ---- q fragments of head c (heads past the group stay zero) ----------------------------------
+    half8 qhi[8], qlo[8];
+    {
+        const bool head_live = c < P.group;
+        const float* qp = P.q + ((size_t)e * P.n_q + (size_t)kvh * P.group + (head_live ? c : 0)) * kHd + g * 8;
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+            float x[8];
+            const float4 a = *reinterpret_cast<const float4*>(qp + m * 32);
+            const float4 b = *reinterpret_cast<const float4*>(qp + m * 32 + 4);
+            x[0] = a.x, x[1] = a.y, x[2] = a.z, x[3] = a.w;
+            x[4] = b.x, x[5] = b.y, x[6] = b.z, x[7] = b.w;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                _Float16 hi, lo;
+                split_hi_lo(head_live ? x[j] : 0.0f, hi, lo);
+                qhi[m][j] = hi;
+                qlo[m][j] = lo;
+            }
+        }
+    }
+
+    // O^T accumulators: o[h][t][r] = out[head c][128 h + 8 (4 g + r) + t]
+    f4 o[2][8];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int t = 0; t < 8; ++t) o[h][t] = f4{0.0f, 0.0f, 0.0f, 0.0f};
+    float m_run = -INFINITY;  // running max of head c (base-2 logits), equal in the 4 g lanes
+    float l_run = 0.0f;       // this lane's share (its 4 cells per page) of the denominator
+
+    while (pg < pg1) {
+        // the next page is fetched unconditionally (the last iteration re-reads its own page)
+        const int pg_next = pg + kWaves;
+        const int32_t phys_next = bt[min(pg_next, pg1 - 1)];
+        const uint8_t* kp_next = P.kpool + (size_t)phys_next * page_bytes + head_off;
+        const uint8_t* vp_next = P.vpool + (size_t)phys_next * page_bytes + head_off;
+
+        if constexpr (STEP) {
+            if (pg == n_pages - 1) {
+                // This wave holds the page of cell pos; its pool row is stale.  Every lane converts
+                // its slices of the new row; the lanes whose fragments are that row keep and store them.
+                const int r = pos & (kPage - 1);
+                const size_t here = (size_t)bt[pg] * page_bytes + head_off + (size_t)r * (kHd * 2);
+                const float* nk = P.new_k + ((size_t)e * P.n_kv + (size_t)kvh) * kHd;
+                const float* nv = P.new_v + ((size_t)e * P.n_kv + (size_t)kvh) * kHd;
+                const auto row_slice = [](const float* src) {
+                    const float4 a = *reinterpret_cast<const float4*>(src);
+                    const float4 b = *reinterpret_cast<const float4*>(src + 4);
+                    v4u w;
+                    w.x = f16_store_pair(a.x, a.y), w.y = f16_store_pair(a.z, a.w);
+                    w.z = f16_store_pair(b.x, b.y), w.w = f16_store_pair(b.z, b.w);
+                    return w;
+                };
+#pragma unroll
+                for (int m = 0; m < 8; ++m) {
+                    const v4u w = row_slice(nk + m * 32 + g * 8);
+                    if (c == r) {
+                        kf[m] = w;
+                        *reinterpret_cast<v4u*>(P.kpool_w + here + (size_t)(m * 32 + g * 8) * 2) = w;
+                    }
+                }
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const v4u w = row_slice(nv + h * 128 + c * 8);
+                    if (g == (r >> 2)) {
+#pragma unroll
+                        for (int rr = 0; rr < 4; ++rr)
+                            if (rr == (r & 3)) vf[h][rr] = w;
+                        *reinterpret_cast<v4u*>(P.vpool_w + here + (size_t)(h * 128 + c * 8) * 2) = w;
+                    }
+                }
+            }
+        }
+
+        // ---- S^T = K . q^T: four independent accumulation chains ------------------------------
+        f4 s0 = f4{0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0, s2 = s0, s3 = s0;
+#pragma unroll
+        for (int m = 0; m < 8; m += 2) {
+            const half8 ka = __builtin_bit_cast(half8, kf[m]);
+            const half8 kb = __builtin_bit_cast(half8, kf[m + 1]);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qhi[m], s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qlo[m], s1, 0, 0, 0);
+            s2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kb, qhi[m + 1], s2, 0, 0, 0);
+            s3 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kb, qlo[m + 1], s3, 0, 0, 0);
+            kf[m] = __builtin_nontemporal_load(k_addr(kp_next, m));
+            kf[m + 1] = __builtin_nontemporal_load(k_addr(kp_next, m + 1));
+        }
+        const f4 s = (s0 + s1) + (s2 + s3);  // s[r] = q[head c] . k[cell 4 g + r]
+
+        // ---- online softmax of head c ---------------------------------------------------------------
+        float t4[4];
+        float pm = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const bool live = pg * kPage + 4 * g + r <= pos;
+            t4[r] = live ? s[r] * P.scale_log2e : -INFINITY;
+            pm = fmaxf(pm, t4[r]);
+        }
+        pm = fmaxf(pm, __shfl_xor(pm, 16, 64));
+        pm = fmaxf(pm, __shfl_xor(pm, 32, 64));
+        const float m_new = fmaxf(m_run, pm);  // finite: every page of a range holds a live cell
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        h4m phi, plo;
+        float psum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float p = __builtin_amdgcn_exp2f(t4[r] - m_new);
+            psum += p;
+            _Float16 hi, lo;
+            split_hi_lo(p, hi, lo);
+            phi[r] = hi;
+            plo[r] = lo;
+        }
+        l_run = l_run * alpha + psum;
+        if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int t = 0; t < 8; ++t) o[h][t] *= alpha;
+        }
+        m_run = m_new;
+
+        if (pg == n_pages - 1) {
+            // Rows past `pos` may hold anything (even NaN): make them exact zeros.
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (pg * kPage + 4 * g + r > pos) {
+                    vf[0][r] = v4u{0u, 0u, 0u, 0u};
+                    vf[1][r] = v4u{0u, 0u, 0u, 0u};
+                }
+        }
+
+        // ---- O^T += V^T . P^T ------------------------------------------------------------------------
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const half8 v0 = __builtin_bit_cast(half8, vf[h][0]), v1 = __builtin_bit_cast(half8, vf[h][1]);
+            const half8 v2 = __builtin_bit_cast(half8, vf[h][2]), v3 = __builtin_bit_cast(half8, vf[h][3]);
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const h4m va = h4m{v0[t], v1[t], v2[t], v3[t]};
+                o[h][t] = __builtin_amdgcn_mfma_f32_16x16x16f16(va, phi, o[h][t], 0, 0, 0);
+                o[h][t] = __builtin_amdgcn_mfma_f32_16x16x16f16(va, plo, o[h][t], 0, 0, 0);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) vf[h][r] = __builtin_nontemporal_load(v_addr(vp_next, h, r));
+        }
+        pg = pg_next;
+    }
+
+    // ---- wave totals, then the four waves are folded pairwise through LDS -------------------------
+    l_run += __shfl_xor(l_run, 16, 64);
+    l_run += __shfl_xor(l_run, 32, 64);
+    if (g == 0) {
+        wave_m[wave][c] = m_run;
+        wave_l[wave][c] = l_run;
+    }
+    __syncthreads();
+    float mx = wave_m[0][c];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) mx = fmaxf(mx, wave_m[w][c]);
+    float lsum = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+        const float mw = wave_m[w][c];
+        lsum = fmaf(mw == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(mw - mx), wave_l[w][c], lsum);
+    }
+    {
+        const float f = m_run == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m_run - mx);
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int t = 0; t < 8; ++t) o[h][t] *= f;
+    }
+    // element (h, r, t) of a lane is out[head c][128 h + 8 (4 g + r) + t]: 8 consecutive floats per (h, r)
+    const auto put = [&](float* base) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float* d = base + (size_t)c * kOwStride + 128 * h + 8 * (4 * g + r);
+                *reinterpret_cast<f4*>(d) = f4{o[h][0][r], o[h][1][r], o[h][2][r], o[h][3][r]};
+                *reinterpret_cast<f4*>(d + 4) = f4{o[h][4][r], o[h][5][r], o[h][6][r], o[h][7][r]};
+            }
+    };
+    const auto add = [&](const float* base) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float* d = base + (size_t)c * kOwStride + 128 * h + 8 * (4 * g + r);
+                const f4 a = *reinterpret_cast<const f4*>(d), b = *reinterpret_cast<const f4*>(d + 4);
+                o[h][0][r] += a.x, o[h][1][r] += a.y, o[h][2][r] += a.z, o[h][3][r] += a.w;
+                o[h][4][r] += b.x, o[h][5][r] += b.y, o[h][6][r] += b.z, o[h][7][r] += b.w;
+            }
+    };
+    if (wave & 1) put(&ow[wave >> 1][0][0]);   // waves 1 and 3 hand over ...
+    __syncthreads();
+    if (!(wave & 1)) add(&ow[wave >> 1][0][0]);  // ... to waves 0 and 2
+    __syncthreads();
+    if (wave == 2) put(&ow[0][0][0]);
+    __syncthreads();
+    if (wave != 0) return;
+    add(&ow[0][0][0]);
+    if (c >= P.group) return;
+    const int hg = P.group;
+    float* po = P.part_o + ((size_t)wg * hg + c) * kHd;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float* d = po + 128 * h + 8 * (4 * g + r);
+            *reinterpret_cast<f4*>(d) = f4{o[h][0][r], o[h][1][r], o[h][2][r], o[h][3][r]};
+            *reinterpret_cast<f4*>(d + 4) = f4{o[h][4][r], o[h][5][r], o[h][6][r], o[h][7][r]};
+        }
+    if (g == 0) {
+        P.part_ml[((size_t)wg * hg + c) * 2 + 0] = mx;
+        P.part_ml[((size_t)wg * hg + c) * 2 + 1] = lsum;
+    }
+}
+
 struct MergeParams {
     AttnBatch b;
     const float* part_o;
@@ -776,10 +1070,16 @@ __global__ __launch_bounds__(kHd * kMergeGroups) void decode_attn_merge_kernel(c
 // Heads one work-group carries for a given q-heads-per-kv-head group.
 int32_t attn_heads_per_wave(int32_t group) { return group % 8 == 0 ? 8 : 4; }
 
-int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b, int32_t sel_groups) {
+// Whether a dense call on this pool goes to the MFMA kernel: f16 rows, unless the pool was
+// created with BKV_POOL_ATTN_VALU (the VALU formulation, kept for comparison).
+bool attn_on_mfma(const bkv_pool* p, int32_t group) {
+    return p->g.layout == BKV_LAYOUT_F16 && group <= 16 && (p->desc.flags & BKV_POOL_ATTN_VALU) == 0;
+}
+
+int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b, int32_t sel_groups, bool mfma) {
     const int32_t n_kv = p->g.n_kv;
     const int32_t group = n_q_head / n_kv;
-    const int32_t hg = attn_heads_per_wave(group);
+    const int32_t hg = mfma ? group : attn_heads_per_wave(group);
     const int32_t n_hc = (group + hg - 1) / hg;
     const int64_t per_page = (int64_t)n_kv * n_hc;
     int64_t total_pages = 0;
@@ -790,7 +1090,7 @@ int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b, int32_t sel
     // All work-groups should be resident at once (one generation): a handful of left-over
     // work-groups would run alone after the rest and double the kernel's time.  `resident`
     // follows from the register budget of the kernel variant that will run.
-    const int64_t resident = hg == 8 ? 2 : 3;
+    const int64_t resident = (mfma || hg == 8) ? 2 : 3;
     int64_t target = (int64_t)(p->n_cu > 0 ? p->n_cu : 256) * resident;
     if (target > p->max_wgs) target = p->max_wgs;
     int64_t pps = (total_pages * per_page + target - 1) / target;
@@ -819,7 +1119,7 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
                               hipStream_t stream) {
     const int32_t n_kv = p->g.n_kv;
     const int32_t group = a.n_q_head / n_kv;
-    const int32_t hg = attn_heads_per_wave(group);
+    const int32_t hg = a.mfma ? group : attn_heads_per_wave(group);
     AttnKernelParams kp;
     kp.b = b;
     kp.kpool = p->k_layer[(size_t)layer];
@@ -857,7 +1157,13 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
         else                                                                    \
             decode_attn_kernel<HGV, KE, VE, false><<<grid, kBlock, 0, stream>>>(kp); \
     } while (0)
-        if (step) {
+        if (a.mfma) {
+            // f16 pools, dense selection, one work-group per unit (checked by the caller)
+            if (step)
+                decode_attn_mfma_kernel<true><<<total, kBlock, 0, stream>>>(kp);
+            else
+                decode_attn_mfma_kernel<false><<<total, kBlock, 0, stream>>>(kp);
+        } else if (step) {
             // f16 pools, dense selection (checked by the caller)
             if (hg == 8)
                 decode_attn_kernel<8, kRowF16, kRowF16, false, true><<<grid, kBlock, 0, stream>>>(kp);

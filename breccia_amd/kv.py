@@ -134,11 +134,13 @@ class Pool:
     """bkv_pool handle.  Method names follow the C entry points."""
 
     def __init__(self, n_layers=1, n_pages=512, n_kv_head=2, head_dim=256, page_cells=16,
-                 layout=L.LAYOUT_F16, max_seqs=16, max_pages_per_seq=None, host_only=False):
+                 layout=L.LAYOUT_F16, max_seqs=16, max_pages_per_seq=None, host_only=False,
+                 attn_valu=False):
         if max_pages_per_seq is None:
             max_pages_per_seq = n_pages
+        flags = (L.POOL_HOST_ONLY if host_only else 0) | (L.POOL_ATTN_VALU if attn_valu else 0)
         self.desc = PoolDesc(n_layers, n_pages, n_kv_head, head_dim, page_cells, layout, max_seqs,
-                             max_pages_per_seq, L.POOL_HOST_ONLY if host_only else 0)
+                             max_pages_per_seq, flags)
         h = C.c_void_p()
         check(lib.bkv_pool_create(C.byref(self.desc), C.byref(h)))
         self.handle = h

@@ -16,6 +16,7 @@ OK, ERR_INVALID, ERR_RANGE, ERR_NO_PAGES, ERR_STATE, ERR_NO_DEVICE, ERR_HIP, ERR
 STATUS_NAMES = ["OK", "INVALID", "RANGE", "NO_PAGES", "STATE", "NO_DEVICE", "HIP", "NOMEM"]
 LAYOUT_F16, LAYOUT_Q8V, LAYOUT_I8H = 0, 1, 2
 POOL_HOST_ONLY = 1
+POOL_ATTN_VALU = 2
 MAX_BATCH = 64
 STAGE_APPEND, STAGE_ATTN_SPLIT, STAGE_ATTN_MERGE, STAGE_PAGE_COPY = range(4)
 

@@ -15,6 +15,17 @@ from gpu_common import REF_BAR_MAX_REL, Twin, check_attn
 from helpers import max_abs
 
 pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True, params=["mfma", "valu"])
+def attn_formulation(request):
+    """Every case runs in both formulations of f16 decode attention (matrix cores / VALU)."""
+    import gpu_common
+    gpu_common.DEFAULT_ATTN_VALU = request.param == "valu"
+    yield
+    gpu_common.DEFAULT_ATTN_VALU = False
+
+
 GOLD = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_kats.json")))
 
 

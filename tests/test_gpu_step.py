@@ -12,6 +12,15 @@ from test_gpu_attn import fill
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True, params=["mfma", "valu"])
+def attn_formulation(request):
+    """Every case runs in both formulations of f16 decode attention (matrix cores / VALU)."""
+    import gpu_common
+    gpu_common.DEFAULT_ATTN_VALU = request.param == "valu"
+    yield
+    gpu_common.DEFAULT_ATTN_VALU = False
+
+
 def step(tw, layer, seqs, pos, k_new, v_new, q, n_head, gate=None):
     n = len(seqs)
     kd, vd = DeviceBuffer.from_numpy(k_new), DeviceBuffer.from_numpy(v_new)
