@@ -672,8 +672,12 @@ constexpr int kOwStride = kHd + 4;  // floats per head in the wave-merge staging
 
 // STEP: the row of cell pos comes from the caller's f32 K/V (stored under the f16 rule into the
 // pool on the way), as in decode_attn_kernel<..., STEP = true>.
-template <bool STEP>
+// SEL: the 16 rows of an iteration are four listed 4-cell blocks instead of a page, as in
+// decode_attn_kernel<..., SEL = true> (block g supplies the V rows of lane group g, block c / 4
+// the K row of lane c).
+template <bool STEP, bool SEL = false>
 __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnKernelParams P) {
+    static_assert(!(STEP && SEL), "the fused step attends the dense selection");
     __shared__ __attribute__((aligned(16))) float ow[2][16][kOwStride];
     __shared__ float wave_m[kWaves][16];
     __shared__ float wave_l[kWaves][16];
@@ -687,12 +691,20 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
     const int kvh = rem - split * P.n_kv;
     const int wg = unit;
     const int pos = P.b.pos[e];
-    const int n_pages = pos / kPage + 1;
+    typedef const __attribute__((address_space(4))) int32_t* table_ptr;
+    typedef const __attribute__((address_space(4))) uint32_t* list_ptr;
+    const table_ptr bt = (table_ptr)(uintptr_t)(P.tables + (size_t)P.b.row[e] * (size_t)P.max_pages_per_seq);
+    uint32_t n_sel = 0;
+    list_ptr sel = nullptr;
+    if constexpr (SEL) {
+        n_sel = min(((list_ptr)(uintptr_t)P.counts)[e], (uint32_t)P.max_ids);
+        sel = (list_ptr)(uintptr_t)(P.ids + (size_t)e * (size_t)P.id_stride);
+    }
+    // loop iterations of this entry: pages, or groups of four selected blocks
+    const int n_pages = SEL ? (int)((n_sel + 3u) >> 2) : pos / kPage + 1;
     const int pps = P.b.pps[e];
     const int pg0 = split * pps;
     const int pg1 = min(pg0 + pps, n_pages);
-    typedef const __attribute__((address_space(4))) int32_t* table_ptr;
-    const table_ptr bt = (table_ptr)(uintptr_t)(P.tables + (size_t)P.b.row[e] * (size_t)P.max_pages_per_seq);
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
@@ -701,19 +713,51 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
     const size_t page_bytes = (size_t)P.n_kv * kPage * kHd * 2;
     const size_t head_off = (size_t)kvh * kPage * kHd * 2;
 
-    const auto k_addr = [&](const uint8_t* page, int m) {
-        return reinterpret_cast<const v4u*>(page + (size_t)c * (kHd * 2) + (size_t)(m * 32 + g * 8) * 2);
+    // Row runs of iteration i (see decode_attn_kernel): a page, or four listed blocks whose ids
+    // are clamped to the blocks at or below `pos` before any address is formed.
+    const auto locate = [&](int i, RowRuns<SEL>& rr) {
+        if constexpr (SEL) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t at = (uint32_t)i * 4u + (uint32_t)j;
+                const uint32_t id = sel[min(at, n_sel - 1u)];
+                rr.id[j] = at < n_sel ? id : 0xffffffffu;
+                const uint32_t idc = min(id, (uint32_t)pos >> 2);
+                const size_t off = (size_t)bt[idc >> 2] * page_bytes + head_off + (size_t)(idc & 3u) * 4u * (kHd * 2);
+                rr.k[j] = P.kpool + off;
+                rr.v[j] = P.vpool + off;
+            }
+        } else {
+            const size_t off = (size_t)bt[i] * page_bytes + head_off;
+            rr.k[0] = P.kpool + off;
+            rr.v[0] = P.vpool + off;
+            rr.id[0] = 0;
+        }
     };
-    const auto v_addr = [&](const uint8_t* page, int h, int r) {
-        return reinterpret_cast<const v4u*>(page + (size_t)(4 * g + r) * (kHd * 2) + (size_t)(h * 128 + c * 8) * 2);
+    const auto pick = [](const auto (&a)[SEL ? 4 : 1], int j) {
+        if constexpr (SEL) return j == 0 ? a[0] : j == 1 ? a[1] : j == 2 ? a[2] : a[3]; else return a[0];
+    };
+    // this lane's K row (row c of the iteration) and the first of its four V rows (row 4 g)
+    const auto k_row = [&](const RowRuns<SEL>& rr) {
+        return SEL ? pick(rr.k, c >> 2) + (size_t)(c & 3) * (kHd * 2) : rr.k[0] + (size_t)c * (kHd * 2);
+    };
+    const auto v_rows = [&](const RowRuns<SEL>& rr) {
+        return SEL ? pick(rr.v, g) : rr.v[0] + (size_t)(4 * g) * (kHd * 2);
+    };
+    const auto k_addr = [&](const uint8_t* row, int m) {
+        return reinterpret_cast<const v4u*>(row + (size_t)(m * 32 + g * 8) * 2);
+    };
+    const auto v_addr = [&](const uint8_t* rows, int h, int r) {
+        return reinterpret_cast<const v4u*>(rows + (size_t)r * (kHd * 2) + (size_t)(h * 128 + c * 8) * 2);
     };
 
     int pg = pg0 + wave;
     v4u kf[8], vf[2][4];
+    RowRuns<SEL> cur{};
     if (pg < pg1) {
-        const int32_t phys = bt[pg];
-        const uint8_t* kp = P.kpool + (size_t)phys * page_bytes + head_off;
-        const uint8_t* vp = P.vpool + (size_t)phys * page_bytes + head_off;
+        locate(pg, cur);
+        const uint8_t* kp = k_row(cur);
+        const uint8_t* vp = v_rows(cur);
 #pragma unroll
         for (int m = 0; m < 8; ++m) kf[m] = __builtin_nontemporal_load(k_addr(kp, m));
 #pragma unroll
@@ -756,16 +800,17 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
     while (pg < pg1) {
         // the next page is fetched unconditionally (the last iteration re-reads its own page)
         const int pg_next = pg + kWaves;
-        const int32_t phys_next = bt[min(pg_next, pg1 - 1)];
-        const uint8_t* kp_next = P.kpool + (size_t)phys_next * page_bytes + head_off;
-        const uint8_t* vp_next = P.vpool + (size_t)phys_next * page_bytes + head_off;
+        RowRuns<SEL> nxt;
+        locate(min(pg_next, pg1 - 1), nxt);
+        const uint8_t* kp_next = k_row(nxt);
+        const uint8_t* vp_next = v_rows(nxt);
 
         if constexpr (STEP) {
             if (pg == n_pages - 1) {
                 // This wave holds the page of cell pos; its pool row is stale.  Every lane converts
                 // its slices of the new row; the lanes whose fragments are that row keep and store them.
                 const int r = pos & (kPage - 1);
-                const size_t here = (size_t)bt[pg] * page_bytes + head_off + (size_t)r * (kHd * 2);
+                const size_t here = (size_t)(cur.k[0] - P.kpool) + (size_t)r * (kHd * 2);
                 const float* nk = P.new_k + ((size_t)e * P.n_kv + (size_t)kvh) * kHd;
                 const float* nv = P.new_v + ((size_t)e * P.n_kv + (size_t)kvh) * kHd;
                 const auto row_slice = [](const float* src) {
@@ -817,19 +862,26 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
         float pm = -INFINITY;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const bool live = pg * kPage + 4 * g + r <= pos;
+            bool live;
+            if constexpr (SEL)
+                live = block_cell_live(pick(cur.id, g), r, pos);
+            else
+                live = pg * kPage + 4 * g + r <= pos;
             t4[r] = live ? s[r] * P.scale_log2e : -INFINITY;
             pm = fmaxf(pm, t4[r]);
         }
         pm = fmaxf(pm, __shfl_xor(pm, 16, 64));
         pm = fmaxf(pm, __shfl_xor(pm, 32, 64));
-        const float m_new = fmaxf(m_run, pm);  // finite: every page of a range holds a live cell
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        // dense: finite, every page of a range holds a live cell; a group of listed blocks may be
+        // dead as a whole, and exp2(-inf - -inf) would be NaN
+        const float m_new = fmaxf(m_run, pm);
+        const bool none_yet = SEL && m_new == -INFINITY;
+        const float alpha = none_yet ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
         h4m phi, plo;
         float psum = 0.0f;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const float p = __builtin_amdgcn_exp2f(t4[r] - m_new);
+            const float p = none_yet ? 0.0f : __builtin_amdgcn_exp2f(t4[r] - m_new);
             psum += p;
             _Float16 hi, lo;
             split_hi_lo(p, hi, lo);
@@ -845,8 +897,15 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
         }
         m_run = m_new;
 
-        if (pg == n_pages - 1) {
-            // Rows past `pos` may hold anything (even NaN): make them exact zeros.
+        // Rows that are not attended may hold anything (even NaN): make them exact zeros.
+        if constexpr (SEL) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (!block_cell_live(pick(cur.id, g), r, pos)) {
+                    vf[0][r] = v4u{0u, 0u, 0u, 0u};
+                    vf[1][r] = v4u{0u, 0u, 0u, 0u};
+                }
+        } else if (pg == n_pages - 1) {
 #pragma unroll
             for (int r = 0; r < 4; ++r)
                 if (pg * kPage + 4 * g + r > pos) {
@@ -870,6 +929,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
             for (int r = 0; r < 4; ++r) vf[h][r] = __builtin_nontemporal_load(v_addr(vp_next, h, r));
         }
         pg = pg_next;
+        cur = nxt;
     }
 
     // ---- wave totals, then the four waves are folded pairwise through LDS -------------------------
@@ -1070,7 +1130,7 @@ __global__ __launch_bounds__(kHd * kMergeGroups) void decode_attn_merge_kernel(c
 // Heads one work-group carries for a given q-heads-per-kv-head group.
 int32_t attn_heads_per_wave(int32_t group) { return group % 8 == 0 ? 8 : 4; }
 
-// Whether a dense call on this pool goes to the MFMA kernel: f16 rows, unless the pool was
+// Whether a call on this pool goes to the MFMA kernel: f16 rows, unless the pool was
 // created with BKV_POOL_ATTN_VALU (the VALU formulation, kept for comparison).
 bool attn_on_mfma(const bkv_pool* p, int32_t group) {
     return p->g.layout == BKV_LAYOUT_F16 && group <= 16 && (p->desc.flags & BKV_POOL_ATTN_VALU) == 0;
@@ -1161,6 +1221,8 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
             // f16 pools, dense selection, one work-group per unit (checked by the caller)
             if (step)
                 decode_attn_mfma_kernel<true><<<total, kBlock, 0, stream>>>(kp);
+            else if (sel)
+                decode_attn_mfma_kernel<false, true><<<total, kBlock, 0, stream>>>(kp);
             else
                 decode_attn_mfma_kernel<false><<<total, kBlock, 0, stream>>>(kp);
         } else if (step) {

@@ -234,8 +234,8 @@ bkv_status bkv_rope_table(double freq_base, int32_t n_rot, int32_t max_pos, floa
  * One split-K online-softmax kernel plus one merge kernel; partials live in a
  * workspace the pool owns.  On f16 pools the split-K kernel multiplies on the matrix cores
  * (all heads of a kv head, up to 16, in one pass over the K/V rows; q and the probabilities
- * as high + low f16 parts, so accuracy is that of f32 accumulation); quantised pools and
- * selection lists use the VALU kernel (heads in chunks of 8 or 4). */
+ * as high + low f16 parts, so accuracy is that of f32 accumulation), also for selection
+ * lists and the fused step; quantised pools use the VALU kernel (heads in chunks of 8 or 4). */
 bkv_status bkv_decode_attn(bkv_pool *pool, int32_t layer, int32_t n, const int32_t *seqs,
                            const int64_t *pos, int32_t n_q_head, const float *q_dev,
                            const float *gate_dev, int64_t gate_seq_stride,
