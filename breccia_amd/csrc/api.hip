@@ -743,7 +743,7 @@ static bkv_status decode_attn_common(bkv_pool* p, int32_t layer, int32_t n, cons
                                      "non-NULL and 4-byte aligned");
     st = flush_tables(p, S(stream));
     if (st != BKV_OK) return st;
-    const bool mfma = attn_on_mfma(p, n_q_head / p->g.n_kv);
+    const bool mfma = attn_on_mfma(p, n_q_head / p->g.n_kv, !select && !step);
     plan_attn(p, n_q_head, b, select ? (max_ids + 3) / 4 : 0, mfma);
     AttnArgs a;
     a.mfma = mfma;

@@ -190,7 +190,7 @@ struct AttnArgs {
 // every entry is planned for that many groups of four selected blocks instead of its pages.
 int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b, int32_t sel_groups = 0,
                   bool mfma = false);
-bool attn_on_mfma(const bkv_pool* p, int32_t group);
+bool attn_on_mfma(const bkv_pool* p, int32_t group, bool dense);
 hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, const AttnArgs& a,
                               hipStream_t stream);
 // Prefill attention (prefill_attn.hip): one entry per sequence chunk.

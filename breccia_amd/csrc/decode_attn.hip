@@ -663,12 +663,108 @@ __global__ __launch_bounds__(kBlock, HG == 8 ? 2 : 3) void decode_attn_kernel(co
 // refilled with the next page's data right after its last use.
 typedef _Float16 h4m __attribute__((ext_vector_type(4)));
 
+// max over the four lanes {c, c + 16, c + 32, c + 48} in every one of them, on the VALU
+// (v_permlane32_swap / v_permlane16_swap exchange half-waves / odd and even rows of two registers)
+typedef unsigned v2u_pair __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float max_over_lane_groups(float x) {
+    const unsigned b = __builtin_bit_cast(unsigned, x);
+    const v2u_pair a = __builtin_amdgcn_permlane32_swap(b, b, false, false);
+    const float m = fmaxf(__builtin_bit_cast(float, a[0]), __builtin_bit_cast(float, a[1]));
+    const unsigned mb = __builtin_bit_cast(unsigned, m);
+    const v2u_pair d = __builtin_amdgcn_permlane16_swap(mb, mb, false, false);
+    return fmaxf(__builtin_bit_cast(float, d[0]), __builtin_bit_cast(float, d[1]));
+}
+
 __device__ __forceinline__ void split_hi_lo(float x, _Float16& hi, _Float16& lo) {
     hi = (_Float16)x;
     lo = (_Float16)(x - (float)hi);
 }
 
 constexpr int kOwStride = kHd + 4;  // floats per head in the wave-merge staging
+
+// Shared tail of the MFMA decode kernels: wave totals, then the four waves are folded pairwise
+// through LDS and wave 0 writes the work-group's partial (m, l, O) in the layout the merge
+// kernel reads.  o[h][t][r] of lane (c, g) is out[head c][128 h + 8 (4 g + r) + t].
+struct MfmaFoldLds {
+    float ow[2][16][kOwStride];
+    float wave_m[kWaves][16];
+    float wave_l[kWaves][16];
+};
+
+__device__ __forceinline__ void mfma_fold_and_store(const AttnKernelParams& P, MfmaFoldLds& L, int wg, int wave,
+                                                    int c, int g, f4 (&o)[2][8], float m_run, float l_run) {
+    auto& ow = L.ow;
+    auto& wave_m = L.wave_m;
+    auto& wave_l = L.wave_l;
+    l_run += __shfl_xor(l_run, 16, 64);
+    l_run += __shfl_xor(l_run, 32, 64);
+    if (g == 0) {
+        wave_m[wave][c] = m_run;
+        wave_l[wave][c] = l_run;
+    }
+    __syncthreads();
+    float mx = wave_m[0][c];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) mx = fmaxf(mx, wave_m[w][c]);
+    float lsum = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+        const float mw = wave_m[w][c];
+        lsum = fmaf(mw == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(mw - mx), wave_l[w][c], lsum);
+    }
+    {
+        const float f = m_run == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m_run - mx);
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int t = 0; t < 8; ++t) o[h][t] *= f;
+    }
+    // element (h, r, t) of a lane is out[head c][128 h + 8 (4 g + r) + t]: 8 consecutive floats per (h, r)
+    const auto put = [&](float* base) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float* d = base + (size_t)c * kOwStride + 128 * h + 8 * (4 * g + r);
+                *reinterpret_cast<f4*>(d) = f4{o[h][0][r], o[h][1][r], o[h][2][r], o[h][3][r]};
+                *reinterpret_cast<f4*>(d + 4) = f4{o[h][4][r], o[h][5][r], o[h][6][r], o[h][7][r]};
+            }
+    };
+    const auto add = [&](const float* base) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float* d = base + (size_t)c * kOwStride + 128 * h + 8 * (4 * g + r);
+                const f4 a = *reinterpret_cast<const f4*>(d), b = *reinterpret_cast<const f4*>(d + 4);
+                o[h][0][r] += a.x, o[h][1][r] += a.y, o[h][2][r] += a.z, o[h][3][r] += a.w;
+                o[h][4][r] += b.x, o[h][5][r] += b.y, o[h][6][r] += b.z, o[h][7][r] += b.w;
+            }
+    };
+    if (wave & 1) put(&ow[wave >> 1][0][0]);   // waves 1 and 3 hand over ...
+    __syncthreads();
+    if (!(wave & 1)) add(&ow[wave >> 1][0][0]);  // ... to waves 0 and 2
+    __syncthreads();
+    if (wave == 2) put(&ow[0][0][0]);
+    __syncthreads();
+    if (wave != 0) return;
+    add(&ow[0][0][0]);
+    if (c >= P.group) return;
+    const int hg = P.group;
+    float* po = P.part_o + ((size_t)wg * hg + c) * kHd;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float* d = po + 128 * h + 8 * (4 * g + r);
+            *reinterpret_cast<f4*>(d) = f4{o[h][0][r], o[h][1][r], o[h][2][r], o[h][3][r]};
+            *reinterpret_cast<f4*>(d + 4) = f4{o[h][4][r], o[h][5][r], o[h][6][r], o[h][7][r]};
+        }
+    if (g == 0) {
+        P.part_ml[((size_t)wg * hg + c) * 2 + 0] = mx;
+        P.part_ml[((size_t)wg * hg + c) * 2 + 1] = lsum;
+    }
+}
 
 // STEP: the row of cell pos comes from the caller's f32 K/V (stored under the f16 rule into the
 // pool on the way), as in decode_attn_kernel<..., STEP = true>.
@@ -678,9 +774,7 @@ constexpr int kOwStride = kHd + 4;  // floats per head in the wave-merge staging
 template <bool STEP, bool SEL = false>
 __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnKernelParams P) {
     static_assert(!(STEP && SEL), "the fused step attends the dense selection");
-    __shared__ __attribute__((aligned(16))) float ow[2][16][kOwStride];
-    __shared__ float wave_m[kWaves][16];
-    __shared__ float wave_l[kWaves][16];
+    __shared__ __attribute__((aligned(16))) MfmaFoldLds lds;
 
     // ---- which (entry, kv head, page range); one work-group per unit (no head chunks) --------
     const int unit = blockIdx.x;
@@ -932,75 +1026,305 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
         cur = nxt;
     }
 
-    // ---- wave totals, then the four waves are folded pairwise through LDS -------------------------
-    l_run += __shfl_xor(l_run, 16, 64);
-    l_run += __shfl_xor(l_run, 32, 64);
-    if (g == 0) {
-        wave_m[wave][c] = m_run;
-        wave_l[wave][c] = l_run;
-    }
-    __syncthreads();
-    float mx = wave_m[0][c];
+    mfma_fold_and_store(P, lds, wg, wave, c, g, o, m_run, l_run);
+}
+
+// ---- decode attention on the matrix cores, int8 rows with f16 block scales ---------------------
+// The I8H layout ([256 x i8][8 x f16 scale] per row) through the same MFMA decomposition as
+// decode_attn_mfma_kernel.  An int8 code is exactly representable in f16, so codes enter the
+// MFMAs as they are and the block scales are applied where a block's sum is complete:
+//   scores: one 32-deep MFMA pair per 32-value block m (the block is the contraction), then
+//           s[cell] += scale_k[cell][m] * partial[cell]           (4 FMAs per block and lane)
+//   P.V   : the dequantised value code * scale (7 + 11 significant bits) is split exactly into
+//           two f16 terms, hi = f16(code * scale) and lo = fma(code, scale, -hi) (the remainder
+//           has at most 7 significant bits and its lowest bit is 2^(e - 10) >= 2^-24 for a normal
+//           scale 2^e * f, so it is a representable f16 number, subnormal at worst); the three
+//           products (hi + lo).(p_hi + p_lo) then carry the result to f32 accuracy.  A lane's 8 columns lie in one block (4 h + c / 4), so it
+//           needs one scale per V row and half.
+// The VALU formulation of this layout is bound by instruction issue (conversions and FMAs, 40 %
+// of the HBM roofline on long contexts); here the VALU only converts and scales.
+typedef _Float16 h2m __attribute__((ext_vector_type(2)));
+
+// four int8 codes (one dword) -> four exact f16 values: 0x6400 | (code ^ 0x80) is 1024 + (code + 128)
+__device__ __forceinline__ void codes_to_f16(unsigned w, h2m& lo, h2m& hi) {
+    const unsigned u = w ^ 0x80808080u;
+    const h2m bias = h2m{(_Float16)1152.0f, (_Float16)1152.0f};
+    lo = __builtin_bit_cast(h2m, __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u)) - bias;
+    hi = __builtin_bit_cast(h2m, __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - bias;
+}
+// the same for codes that already carry the ^ 0x80 bias
+__device__ __forceinline__ void biased_to_f16(unsigned u, h2m& lo, h2m& hi) {
+    const h2m bias = h2m{(_Float16)1152.0f, (_Float16)1152.0f};
+    lo = __builtin_bit_cast(h2m, __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u)) - bias;
+    hi = __builtin_bit_cast(h2m, __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - bias;
+}
+// 4 x 4 byte transpose: t[j] = { w[0].byte j, w[1].byte j, w[2].byte j, w[3].byte j }
+__device__ __forceinline__ void transpose4x4_bytes(const unsigned (&w)[4], unsigned (&t)[4]) {
+    const unsigned a_lo = __builtin_amdgcn_perm(w[1], w[0], 0x05010400u);  // w0.0 w1.0 w0.1 w1.1
+    const unsigned a_hi = __builtin_amdgcn_perm(w[1], w[0], 0x07030602u);  // w0.2 w1.2 w0.3 w1.3
+    const unsigned b_lo = __builtin_amdgcn_perm(w[3], w[2], 0x05010400u);
+    const unsigned b_hi = __builtin_amdgcn_perm(w[3], w[2], 0x07030602u);
+    t[0] = __builtin_amdgcn_perm(b_lo, a_lo, 0x05040100u);
+    t[1] = __builtin_amdgcn_perm(b_lo, a_lo, 0x07060302u);
+    t[2] = __builtin_amdgcn_perm(b_hi, a_hi, 0x05040100u);
+    t[3] = __builtin_amdgcn_perm(b_hi, a_hi, 0x07060302u);
+}
+// whether either f16 of a dword has exponent field 0 (the values the cache reads as zero)
+__device__ __forceinline__ bool has_zero_exponent(unsigned two_halves) {
+    const unsigned t = two_halves & 0x7c007c00u;
+    return (t & 0xffffu) == 0 || (t >> 16) == 0;
+}
+__device__ __forceinline__ half8 codes8_to_f16(v2u w) {
+    h2m a, b, c2, d;
+    codes_to_f16(w.x, a, b);
+    codes_to_f16(w.y, c2, d);
+    return half8{a[0], a[1], b[0], b[1], c2[0], c2[1], d[0], d[1]};
+}
+// f16 scale under the cache's load rule (exponent field 0 reads as zero)
+__device__ __forceinline__ float scale_of(_Float16 h) {
+    const unsigned short bits = __builtin_bit_cast(unsigned short, h);
+    return (bits & 0x7c00u) == 0 ? 0.0f : (float)h;
+}
+
+// Data path: rows reach the matrix cores through LDS, not through registers.  Every wave owns two
+// slots of 2 x 4352 bytes (the K unit and the V unit of one page and kv head, scales included)
+// and fills them with 16-byte global->LDS loads, 64 lanes x 16 contiguous bytes per instruction
+// (whole cache lines, nothing fetched twice), two pages ahead of the page it computes: the K half
+// of a slot is refilled right after the scores that read it, the V half right after P.V.  A
+// wave has 20 such loads in flight in a fixed order (K, V of the next page, K, V of the one
+// after), so "the oldest five have landed" is s_waitcnt vmcnt(15) at both points of use.
+constexpr int kI8hUnit = kPage * row_bytes_of(kRowI8H);  // 4352
+constexpr int kI8hSlot = 2 * kI8hUnit;                    // K unit, then V unit
+
+// 4352 bytes = 4 x 1024 + 256: four full instructions and one of 16 lanes
+__device__ __forceinline__ void i8h_unit_to_lds(const uint8_t* src, uint8_t* dst, int lane) {
+    typedef const __attribute__((address_space(1))) void* gptr;
+    typedef __attribute__((address_space(3))) void* lptr;
 #pragma unroll
-    for (int w = 1; w < kWaves; ++w) mx = fmaxf(mx, wave_m[w][c]);
-    float lsum = 0.0f;
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w) {
-        const float mw = wave_m[w][c];
-        lsum = fmaf(mw == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(mw - mx), wave_l[w][c], lsum);
+    for (int n = 0; n < 4; ++n)
+        __builtin_amdgcn_global_load_lds((gptr)(src + n * 1024 + lane * 16), (lptr)(dst + n * 1024), 16, 0, 0);
+    if (lane < 16) __builtin_amdgcn_global_load_lds((gptr)(src + 4096 + lane * 16), (lptr)(dst + 4096), 16, 0, 0);
+}
+
+__global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const AttnKernelParams P) {
+    // slot 0 and slot 1 of the four waves; the fold staging of the epilogue reuses slot 0's memory
+    __shared__ __attribute__((aligned(16))) uint8_t ring0[kWaves * kI8hSlot];
+    __shared__ __attribute__((aligned(16))) uint8_t ring1[kWaves * kI8hSlot];
+    static_assert(sizeof(MfmaFoldLds) <= sizeof(ring0), "fold staging must fit the first slot array");
+    constexpr int kRow = row_bytes_of(kRowI8H);  // 272
+
+    const int unit = blockIdx.x;
+    int e = 0;
+    while (e + 1 < P.b.n && unit >= P.b.wg_base[e + 1]) ++e;
+    const int rem = unit - P.b.wg_base[e];
+    const int split = rem / P.n_kv;
+    const int kvh = rem - split * P.n_kv;
+    const int wg = unit;
+    const int pos = P.b.pos[e];
+    const int n_pages = pos / kPage + 1;
+    const int pps = P.b.pps[e];
+    const int pg0 = split * pps;
+    const int pg1 = min(pg0 + pps, n_pages);
+    typedef const __attribute__((address_space(4))) int32_t* table_ptr;
+    const table_ptr bt = (table_ptr)(uintptr_t)(P.tables + (size_t)P.b.row[e] * (size_t)P.max_pages_per_seq);
+
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int c = lane & 15;
+    const int g = lane >> 4;
+    const int my_block = c >> 2;  // which of the 4 blocks of a half this lane's 8 columns lie in
+    const size_t page_bytes = (size_t)P.n_kv * kI8hUnit;
+    const size_t head_off = (size_t)kvh * kI8hUnit;
+    uint8_t* const slot0 = ring0 + wave * kI8hSlot;
+    uint8_t* const slot1 = ring1 + wave * kI8hSlot;
+
+    // page of pipeline step i of this wave; past the range the last page is fetched again (and
+    // never used) so that the number of loads in flight stays what the waits assume
+    const auto unit_off = [&](int i) -> size_t {
+        return (size_t)bt[min(pg0 + wave + kWaves * i, pg1 - 1)] * page_bytes + head_off;
+    };
+    if (pg0 < pg1) {  // always: a range holds at least one page
+        i8h_unit_to_lds(P.kpool + unit_off(0), slot0, lane);
+        i8h_unit_to_lds(P.vpool + unit_off(0), slot0 + kI8hUnit, lane);
+        i8h_unit_to_lds(P.kpool + unit_off(1), slot1, lane);
+        i8h_unit_to_lds(P.vpool + unit_off(1), slot1 + kI8hUnit, lane);
     }
+
+    // ---- q fragments of head c (heads past the group stay zero) ----------------------------------
+    half8 qhi[8], qlo[8];
     {
-        const float f = m_run == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m_run - mx);
+        const bool head_live = c < P.group;
+        const float* qp = P.q + ((size_t)e * P.n_q + (size_t)kvh * P.group + (head_live ? c : 0)) * kHd + g * 8;
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
+        for (int m = 0; m < 8; ++m) {
+            float x[8];
+            const float4 a = *reinterpret_cast<const float4*>(qp + m * 32);
+            const float4 b = *reinterpret_cast<const float4*>(qp + m * 32 + 4);
+            x[0] = a.x, x[1] = a.y, x[2] = a.z, x[3] = a.w;
+            x[4] = b.x, x[5] = b.y, x[6] = b.z, x[7] = b.w;
 #pragma unroll
-            for (int t = 0; t < 8; ++t) o[h][t] *= f;
+            for (int j = 0; j < 8; ++j) {
+                _Float16 hi, lo;
+                split_hi_lo(head_live ? x[j] : 0.0f, hi, lo);
+                qhi[m][j] = hi;
+                qlo[m][j] = lo;
+            }
+        }
     }
-    // element (h, r, t) of a lane is out[head c][128 h + 8 (4 g + r) + t]: 8 consecutive floats per (h, r)
-    const auto put = [&](float* base) {
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                float* d = base + (size_t)c * kOwStride + 128 * h + 8 * (4 * g + r);
-                *reinterpret_cast<f4*>(d) = f4{o[h][0][r], o[h][1][r], o[h][2][r], o[h][3][r]};
-                *reinterpret_cast<f4*>(d + 4) = f4{o[h][4][r], o[h][5][r], o[h][6][r], o[h][7][r]};
-            }
-    };
-    const auto add = [&](const float* base) {
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const float* d = base + (size_t)c * kOwStride + 128 * h + 8 * (4 * g + r);
-                const f4 a = *reinterpret_cast<const f4*>(d), b = *reinterpret_cast<const f4*>(d + 4);
-                o[h][0][r] += a.x, o[h][1][r] += a.y, o[h][2][r] += a.z, o[h][3][r] += a.w;
-                o[h][4][r] += b.x, o[h][5][r] += b.y, o[h][6][r] += b.z, o[h][7][r] += b.w;
-            }
-    };
-    if (wave & 1) put(&ow[wave >> 1][0][0]);   // waves 1 and 3 hand over ...
-    __syncthreads();
-    if (!(wave & 1)) add(&ow[wave >> 1][0][0]);  // ... to waves 0 and 2
-    __syncthreads();
-    if (wave == 2) put(&ow[0][0][0]);
-    __syncthreads();
-    if (wave != 0) return;
-    add(&ow[0][0][0]);
-    if (c >= P.group) return;
-    const int hg = P.group;
-    float* po = P.part_o + ((size_t)wg * hg + c) * kHd;
+
+    f4 o[2][8];
 #pragma unroll
     for (int h = 0; h < 2; ++h)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            float* d = po + 128 * h + 8 * (4 * g + r);
-            *reinterpret_cast<f4*>(d) = f4{o[h][0][r], o[h][1][r], o[h][2][r], o[h][3][r]};
-            *reinterpret_cast<f4*>(d + 4) = f4{o[h][4][r], o[h][5][r], o[h][6][r], o[h][7][r]};
+        for (int t = 0; t < 8; ++t) o[h][t] = f4{0.0f, 0.0f, 0.0f, 0.0f};
+    float m_run = -INFINITY;
+    float l_run = 0.0f;
+
+    // One page: step i of the wave, resident in `slot`; the slot is refilled with step i + 2.
+    const auto one_page = [&](uint8_t* slot, int i) {
+        const int pg = pg0 + wave + kWaves * i;
+        const uint8_t* ks = slot;
+        const uint8_t* vs = slot + kI8hUnit;
+        const size_t off_next = unit_off(i + 2);
+
+        // ---- scores: per block, codes . q on the matrix core, then the block's scale ----------------
+        __builtin_amdgcn_s_waitcnt(0x0F7F);  // vmcnt(15): this page's K unit has landed
+        f4 s = f4{0.0f, 0.0f, 0.0f, 0.0f};
+        // all fragments of the unit are requested from LDS in one batch, ahead of the first use
+        half8 ksc[4];
+        v2u kc[8];
+#pragma unroll
+        for (int m = 0; m < 8; ++m) kc[m] = *reinterpret_cast<const v2u*>(ks + c * kRow + m * 32 + g * 8);
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            ksc[r] = __builtin_bit_cast(half8, *reinterpret_cast<const v4u*>(ks + (4 * g + r) * kRow + kHd));
+        const unsigned k_screen = *reinterpret_cast<const unsigned*>(ks + (lane >> 2) * kRow + kHd + 4 * (lane & 3));
+        __builtin_amdgcn_sched_barrier(0);
+        // A scale with exponent field 0 reads as zero.  The store rule never writes one, so the
+        // unit's 64 scale dwords are screened one per lane, and only a unit that holds such a scale
+        // (foreign data, rows never written) pays for the per-value rule.
+        if (__builtin_amdgcn_ballot_w64(has_zero_exponent(k_screen)) != 0) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int m = 0; m < 8; ++m)
+                    if ((__builtin_bit_cast(unsigned short, ksc[r][m]) & 0x7c00u) == 0) ksc[r][m] = (_Float16)0.0f;
         }
-    if (g == 0) {
-        P.part_ml[((size_t)wg * hg + c) * 2 + 0] = mx;
-        P.part_ml[((size_t)wg * hg + c) * 2 + 1] = lsum;
-    }
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+            const half8 ka = codes8_to_f16(kc[m]);
+            f4 part = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qhi[m], f4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+            part = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qlo[m], part, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) s[r] = fmaf((float)ksc[r][m], part[r], s[r]);
+        }
+        i8h_unit_to_lds(P.kpool + off_next, slot, lane);
+
+        // ---- online softmax of head c ---------------------------------------------------------------
+        float t4[4];
+        float pm = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const bool live = pg * kPage + 4 * g + r <= pos;
+            t4[r] = live ? s[r] * P.scale_log2e : -INFINITY;
+            pm = fmaxf(pm, t4[r]);
+        }
+        pm = max_over_lane_groups(pm);
+        const float m_new = fmaxf(m_run, pm);  // finite: every page of a range holds a live cell
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        float p[4];
+        float psum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            p[r] = __builtin_amdgcn_exp2f(t4[r] - m_new);
+            psum += p[r];
+        }
+        l_run = l_run * alpha + psum;
+        if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int t = 0; t < 8; ++t) o[h][t] *= alpha;
+        }
+        m_run = m_new;
+        h4m phi, plo;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            _Float16 hi, lo;
+            split_hi_lo(p[r], hi, lo);
+            phi[r] = hi;
+            plo[r] = lo;
+        }
+        const half8 phh = half8{phi[0], phi[1], phi[2], phi[3], phi[0], phi[1], phi[2], phi[3]};
+        const half8 pll = half8{plo[0], plo[1], plo[2], plo[3], plo[0], plo[1], plo[2], plo[3]};
+        // ---- P.V: dequantise into the exact (hi, lo) pair, two 32-deep MFMAs per 16 columns ---------------
+        __builtin_amdgcn_s_waitcnt(0x0F7F);  // vmcnt(15): this page's V unit has landed
+        // Scales of the lane's rows 4 g + r for its block of either half.  Rows past `pos` may hold
+        // anything: their probabilities are exact zeros already, and their scales are made zeros
+        // too, so that 0 * (garbage scale) cannot produce a NaN (any int8 code is a finite number).
+        unsigned vsb[2][4];
+        v2u vc[2][4];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                vc[h][r] = *reinterpret_cast<const v2u*>(vs + (4 * g + r) * kRow + h * 128 + c * 8);
+                vsb[h][r] = *reinterpret_cast<const unsigned short*>(vs + (4 * g + r) * kRow + kHd + 2 * (4 * h + my_block));
+            }
+        const unsigned v_screen = *reinterpret_cast<const unsigned*>(vs + (lane >> 2) * kRow + kHd + 4 * (lane & 3));
+        __builtin_amdgcn_sched_barrier(0);
+        const bool last_page = pg == n_pages - 1;
+        if (last_page || __builtin_amdgcn_ballot_w64(has_zero_exponent(v_screen)) != 0) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if ((vsb[h][r] & 0x7c00u) == 0 || pg * kPage + 4 * g + r > pos) vsb[h][r] = 0;
+        }
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const h2m s01 = __builtin_bit_cast(h2m, vsb[h][0] | (vsb[h][1] << 16));
+            const h2m s23 = __builtin_bit_cast(h2m, vsb[h][2] | (vsb[h][3] << 16));
+            // the lane's 4 rows x 8 codes, transposed as bytes so that a dword holds one column's
+            // four rows: converted, it is the A fragment of that column's MFMA
+            unsigned wx[4], wy[4], col[8];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                wx[r] = vc[h][r].x ^ 0x80808080u;
+                wy[r] = vc[h][r].y ^ 0x80808080u;
+            }
+            {
+                unsigned t0[4], t1[4];
+                transpose4x4_bytes(wx, t0);
+                transpose4x4_bytes(wy, t1);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) col[t] = t0[t], col[4 + t] = t1[t];
+            }
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                h2m c01, c23;
+                biased_to_f16(col[t], c01, c23);
+                const h2m hi01 = c01 * s01, hi23 = c23 * s23;
+                const h2m lo01 = __builtin_elementwise_fma(c01, s01, -hi01);
+                const h2m lo23 = __builtin_elementwise_fma(c23, s23, -hi23);
+                // (hi + lo) . p_hi and (hi + lo) . p_lo as two 32-deep MFMAs: the contraction runs
+                // over the 16 cells twice, a lane's eight slots being its four cells' hi parts and then
+                // their lo parts
+                const half8 ahl = half8{hi01[0], hi01[1], hi23[0], hi23[1], lo01[0], lo01[1], lo23[0], lo23[1]};
+                o[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahl, phh, o[h][t], 0, 0, 0);
+                o[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahl, pll, o[h][t], 0, 0, 0);
+            }
+        }
+        i8h_unit_to_lds(P.vpool + off_next, slot + kI8hUnit, lane);
+    };
+
+    const int n_steps = pg0 + wave < pg1 ? (pg1 - pg0 - wave + kWaves - 1) / kWaves : 0;
+    for (int i = 0; i < n_steps; ++i) one_page((i & 1) ? slot1 : slot0, i);
+
+    // no load may still be on its way into the slots when the fold staging takes their place
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0)
+    __syncthreads();
+    mfma_fold_and_store(P, *reinterpret_cast<MfmaFoldLds*>(ring0), wg, wave, c, g, o, m_run, l_run);
 }
 
 struct MergeParams {
@@ -1132,8 +1456,10 @@ int32_t attn_heads_per_wave(int32_t group) { return group % 8 == 0 ? 8 : 4; }
 
 // Whether a call on this pool goes to the MFMA kernel: f16 rows, unless the pool was
 // created with BKV_POOL_ATTN_VALU (the VALU formulation, kept for comparison).
-bool attn_on_mfma(const bkv_pool* p, int32_t group) {
-    return p->g.layout == BKV_LAYOUT_F16 && group <= 16 && (p->desc.flags & BKV_POOL_ATTN_VALU) == 0;
+bool attn_on_mfma(const bkv_pool* p, int32_t group, bool dense) {
+    if (group > 16 || (p->desc.flags & BKV_POOL_ATTN_VALU) != 0) return false;
+    // f16 rows: every call; int8 rows with f16 scales: the dense selection
+    return p->g.layout == BKV_LAYOUT_F16 || (p->g.layout == BKV_LAYOUT_I8H && dense);
 }
 
 int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b, int32_t sel_groups, bool mfma) {
@@ -1219,7 +1545,9 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
     } while (0)
         if (a.mfma) {
             // f16 pools, dense selection, one work-group per unit (checked by the caller)
-            if (step)
+            if (layout == BKV_LAYOUT_I8H)
+                decode_attn_mfma_i8h_kernel<<<total, kBlock, 0, stream>>>(kp);
+            else if (step)
                 decode_attn_mfma_kernel<true><<<total, kBlock, 0, stream>>>(kp);
             else if (sel)
                 decode_attn_mfma_kernel<false, true><<<total, kBlock, 0, stream>>>(kp);

@@ -64,6 +64,34 @@ def test_quantised_pools_ragged_batch(layout, n_q):
 
 
 @pytest.mark.parametrize("layout", [L.LAYOUT_Q8V, L.LAYOUT_I8H])
+@pytest.mark.parametrize("v_mag", [1.2e-2, 3e-3, 1.0, 900.0])
+def test_quantised_values_across_the_scale_range(layout, v_mag):
+    # block scales from just above 2^-14 (dequantised values and their low-order parts in the f16
+    # subnormal range) up to 7: the result must stay at the same-quantised-reference bar, relative
+    # to the largest output.  v_mag 3e-3 puts some blocks' scales below 2^-14: those are stored,
+    # and read, as zero by pool and oracle alike.
+    rng = np.random.Generator(np.random.PCG64(97 + layout))
+    with Twin(n_pages=80, max_seqs=2, layout=layout) as tw:
+        s = tw.pool.seq_create()
+        n = 1203
+        tw.pool.seq_reserve(s, n)
+        k = rng.standard_normal((n, 2, 256)).astype(np.float32)
+        v = (rng.standard_normal((n, 2, 256)) * v_mag).astype(np.float32)
+        v[:, :, 64:96] *= 0.37      # blocks of one row differ in scale
+        v[5::7] *= 0.11
+        tw.append(0, [s], [0], [k], [v])
+        tw.assert_pools_equal()
+        q = rng.standard_normal((2, 16, 256)).astype(np.float32)
+        pos = [n - 1, 700]
+        out = tw.decode_attn(0, [s, s], pos, q, 16)
+        for i in range(2):
+            want = tw.oracle_attend(0, s, pos[i], q[i], 16)
+            assert np.max(np.abs(want)) > 0.0
+            rel = max_abs(out[i], want) / float(np.max(np.abs(want)))
+            assert rel <= REF_BAR_MAX_REL, (i, rel)
+
+
+@pytest.mark.parametrize("layout", [L.LAYOUT_Q8V, L.LAYOUT_I8H])
 def test_quantised_pools_ignore_poisoned_cells(layout):
     # a NaN scale in an unwritten row must not reach the output through 0 * NaN
     rng = np.random.Generator(np.random.PCG64(95 + layout))
