@@ -663,16 +663,35 @@ __global__ __launch_bounds__(kBlock, HG == 8 ? 2 : 3) void decode_attn_kernel(co
 // refilled with the next page's data right after its last use.
 typedef _Float16 h4m __attribute__((ext_vector_type(4)));
 
-// max over the four lanes {c, c + 16, c + 32, c + 48} in every one of them, on the VALU
-// (v_permlane32_swap / v_permlane16_swap exchange half-waves / odd and even rows of two registers)
-typedef unsigned v2u_pair __attribute__((ext_vector_type(2)));
+// Reductions over the four lanes {c, c + 16, c + 32, c + 48}, result in every one of them, on the
+// VALU: v_permlane32_swap exchanges the upper half of its first register with the lower half of
+// its second, v_permlane16_swap the odd rows of the first with the even rows of the second, so
+// with two copies of x the two registers then hold x[l] and x[l ^ 32] (x[l ^ 16]) side by side.
+// Written as asm with both registers as in/out operands: the compiler's two-result builtin for
+// these instructions hands back its first result twice.  The s_nop covers the wait states the
+// swap needs after a VALU write of its operands.
+struct LanePair {
+    float a, b;
+};
+__device__ __forceinline__ LanePair swap_halves(float x) {
+    LanePair p{x, x};
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(p.a), "+v"(p.b));
+    return p;
+}
+__device__ __forceinline__ LanePair swap_rows(float x) {
+    LanePair p{x, x};
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(p.a), "+v"(p.b));
+    return p;
+}
 __device__ __forceinline__ float max_over_lane_groups(float x) {
-    const unsigned b = __builtin_bit_cast(unsigned, x);
-    const v2u_pair a = __builtin_amdgcn_permlane32_swap(b, b, false, false);
-    const float m = fmaxf(__builtin_bit_cast(float, a[0]), __builtin_bit_cast(float, a[1]));
-    const unsigned mb = __builtin_bit_cast(unsigned, m);
-    const v2u_pair d = __builtin_amdgcn_permlane16_swap(mb, mb, false, false);
-    return fmaxf(__builtin_bit_cast(float, d[0]), __builtin_bit_cast(float, d[1]));
+    const LanePair p = swap_halves(x);
+    const LanePair q = swap_rows(fmaxf(p.a, p.b));
+    return fmaxf(q.a, q.b);
+}
+__device__ __forceinline__ float sum_over_lane_groups(float x) {
+    const LanePair p = swap_halves(x);
+    const LanePair q = swap_rows(p.a + p.b);
+    return q.a + q.b;
 }
 
 __device__ __forceinline__ void split_hi_lo(float x, _Float16& hi, _Float16& lo) {
@@ -682,11 +701,12 @@ __device__ __forceinline__ void split_hi_lo(float x, _Float16& hi, _Float16& lo)
 
 constexpr int kOwStride = kHd + 4;  // floats per head in the wave-merge staging
 
-// Shared tail of the MFMA decode kernels: wave totals, then the four waves are folded pairwise
-// through LDS and wave 0 writes the work-group's partial (m, l, O) in the layout the merge
-// kernel reads.  o[h][t][r] of lane (c, g) is out[head c][128 h + 8 (4 g + r) + t].
+// Shared tail of the MFMA decode kernels: wave totals, then every wave stages its scaled O in
+// LDS and each wave sums one quarter of the columns over the four stagings and writes it as the
+// work-group's partial (m, l, O) in the layout the merge kernel reads.
+// o[h][t][r] of lane (c, g) is out[head c][128 h + 8 (4 g + r) + t].
 struct MfmaFoldLds {
-    float ow[2][16][kOwStride];
+    float ow[kWaves][16][kOwStride];
     float wave_m[kWaves][16];
     float wave_l[kWaves][16];
 };
@@ -696,8 +716,7 @@ __device__ __forceinline__ void mfma_fold_and_store(const AttnKernelParams& P, M
     auto& ow = L.ow;
     auto& wave_m = L.wave_m;
     auto& wave_l = L.wave_l;
-    l_run += __shfl_xor(l_run, 16, 64);
-    l_run += __shfl_xor(l_run, 32, 64);
+    l_run = sum_over_lane_groups(l_run);
     if (g == 0) {
         wave_m[wave][c] = m_run;
         wave_l[wave][c] = l_run;
@@ -714,53 +733,32 @@ __device__ __forceinline__ void mfma_fold_and_store(const AttnKernelParams& P, M
     }
     {
         const float f = m_run == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m_run - mx);
+        // element (h, r, t) of a lane is out[head c][128 h + 8 (4 g + r) + t]: 8 consecutive floats per (h, r)
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
-            for (int t = 0; t < 8; ++t) o[h][t] *= f;
+            for (int r = 0; r < 4; ++r) {
+                float* d = &ow[wave][c][128 * h + 8 * (4 * g + r)];
+                *reinterpret_cast<f4*>(d) = f4{o[h][0][r] * f, o[h][1][r] * f, o[h][2][r] * f, o[h][3][r] * f};
+                *reinterpret_cast<f4*>(d + 4) = f4{o[h][4][r] * f, o[h][5][r] * f, o[h][6][r] * f, o[h][7][r] * f};
+            }
     }
-    // element (h, r, t) of a lane is out[head c][128 h + 8 (4 g + r) + t]: 8 consecutive floats per (h, r)
-    const auto put = [&](float* base) {
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                float* d = base + (size_t)c * kOwStride + 128 * h + 8 * (4 * g + r);
-                *reinterpret_cast<f4*>(d) = f4{o[h][0][r], o[h][1][r], o[h][2][r], o[h][3][r]};
-                *reinterpret_cast<f4*>(d + 4) = f4{o[h][4][r], o[h][5][r], o[h][6][r], o[h][7][r]};
-            }
-    };
-    const auto add = [&](const float* base) {
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const float* d = base + (size_t)c * kOwStride + 128 * h + 8 * (4 * g + r);
-                const f4 a = *reinterpret_cast<const f4*>(d), b = *reinterpret_cast<const f4*>(d + 4);
-                o[h][0][r] += a.x, o[h][1][r] += a.y, o[h][2][r] += a.z, o[h][3][r] += a.w;
-                o[h][4][r] += b.x, o[h][5][r] += b.y, o[h][6][r] += b.z, o[h][7][r] += b.w;
-            }
-    };
-    if (wave & 1) put(&ow[wave >> 1][0][0]);   // waves 1 and 3 hand over ...
     __syncthreads();
-    if (!(wave & 1)) add(&ow[wave >> 1][0][0]);  // ... to waves 0 and 2
-    __syncthreads();
-    if (wave == 2) put(&ow[0][0][0]);
-    __syncthreads();
-    if (wave != 0) return;
-    add(&ow[0][0][0]);
-    if (c >= P.group) return;
+    // wave w sums columns [64 w, 64 w + 64): lane (c, g) takes 4 columns at 4 c of heads g, g + 4, ...
     const int hg = P.group;
-    float* po = P.part_o + ((size_t)wg * hg + c) * kHd;
 #pragma unroll
-    for (int h = 0; h < 2; ++h)
+    for (int hp = 0; hp < 16; hp += 4) {
+        const int head = hp + g;
+        if (hp >= hg) break;
+        if (head < hg) {
+            const int col = 64 * wave + 4 * c;
+            f4 acc = *reinterpret_cast<const f4*>(&ow[0][head][col]);
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            float* d = po + 128 * h + 8 * (4 * g + r);
-            *reinterpret_cast<f4*>(d) = f4{o[h][0][r], o[h][1][r], o[h][2][r], o[h][3][r]};
-            *reinterpret_cast<f4*>(d + 4) = f4{o[h][4][r], o[h][5][r], o[h][6][r], o[h][7][r]};
+            for (int w = 1; w < kWaves; ++w) acc += *reinterpret_cast<const f4*>(&ow[w][head][col]);
+            *reinterpret_cast<f4*>(P.part_o + ((size_t)wg * hg + head) * kHd + col) = acc;
         }
-    if (g == 0) {
+    }
+    if (wave == 0 && g == 0 && c < hg) {
         P.part_ml[((size_t)wg * hg + c) * 2 + 0] = mx;
         P.part_ml[((size_t)wg * hg + c) * 2 + 1] = lsum;
     }
@@ -892,12 +890,18 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
     float l_run = 0.0f;       // this lane's share (its 4 cells per page) of the denominator
 
     while (pg < pg1) {
-        // the next page is fetched unconditionally (the last iteration re-reads its own page)
+        // the rows of this wave's next iteration, if it has one, are requested into the fragment
+        // registers as these are used up (the last iteration requests nothing)
         const int pg_next = pg + kWaves;
-        RowRuns<SEL> nxt;
-        locate(min(pg_next, pg1 - 1), nxt);
-        const uint8_t* kp_next = k_row(nxt);
-        const uint8_t* vp_next = v_rows(nxt);
+        const bool more = pg_next < pg1;
+        RowRuns<SEL> nxt{};
+        const uint8_t* kp_next = nullptr;
+        const uint8_t* vp_next = nullptr;
+        if (more) {
+            locate(pg_next, nxt);
+            kp_next = k_row(nxt);
+            vp_next = v_rows(nxt);
+        }
 
         if constexpr (STEP) {
             if (pg == n_pages - 1) {
@@ -946,8 +950,10 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
             s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qlo[m], s1, 0, 0, 0);
             s2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kb, qhi[m + 1], s2, 0, 0, 0);
             s3 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kb, qlo[m + 1], s3, 0, 0, 0);
-            kf[m] = __builtin_nontemporal_load(k_addr(kp_next, m));
-            kf[m + 1] = __builtin_nontemporal_load(k_addr(kp_next, m + 1));
+            if (more) {
+                kf[m] = __builtin_nontemporal_load(k_addr(kp_next, m));
+                kf[m + 1] = __builtin_nontemporal_load(k_addr(kp_next, m + 1));
+            }
         }
         const f4 s = (s0 + s1) + (s2 + s3);  // s[r] = q[head c] . k[cell 4 g + r]
 
@@ -964,8 +970,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
             t4[r] = live ? s[r] * P.scale_log2e : -INFINITY;
             pm = fmaxf(pm, t4[r]);
         }
-        pm = fmaxf(pm, __shfl_xor(pm, 16, 64));
-        pm = fmaxf(pm, __shfl_xor(pm, 32, 64));
+        pm = max_over_lane_groups(pm);
         // dense: finite, every page of a range holds a live cell; a group of listed blocks may be
         // dead as a whole, and exp2(-inf - -inf) would be NaN
         const float m_new = fmaxf(m_run, pm);
@@ -1019,8 +1024,10 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
                 o[h][t] = __builtin_amdgcn_mfma_f32_16x16x16f16(va, phi, o[h][t], 0, 0, 0);
                 o[h][t] = __builtin_amdgcn_mfma_f32_16x16x16f16(va, plo, o[h][t], 0, 0, 0);
             }
+            if (more) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) vf[h][r] = __builtin_nontemporal_load(v_addr(vp_next, h, r));
+                for (int r = 0; r < 4; ++r) vf[h][r] = __builtin_nontemporal_load(v_addr(vp_next, h, r));
+            }
         }
         pg = pg_next;
         cur = nxt;
@@ -1107,10 +1114,11 @@ __device__ __forceinline__ void i8h_unit_to_lds(const uint8_t* src, uint8_t* dst
 }
 
 __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const AttnKernelParams P) {
-    // slot 0 and slot 1 of the four waves; the fold staging of the epilogue reuses slot 0's memory
-    __shared__ __attribute__((aligned(16))) uint8_t ring0[kWaves * kI8hSlot];
-    __shared__ __attribute__((aligned(16))) uint8_t ring1[kWaves * kI8hSlot];
-    static_assert(sizeof(MfmaFoldLds) <= sizeof(ring0), "fold staging must fit the first slot array");
+    // slot 0 and slot 1 of the four waves; the fold staging of the epilogue reuses their memory
+    __shared__ __attribute__((aligned(16))) uint8_t ring[2 * kWaves * kI8hSlot];
+    static_assert(sizeof(MfmaFoldLds) <= sizeof(ring), "fold staging must fit the slots");
+    uint8_t* const ring0 = ring;
+    uint8_t* const ring1 = ring + kWaves * kI8hSlot;
     constexpr int kRow = row_bytes_of(kRowI8H);  // 272
 
     const int unit = blockIdx.x;
@@ -1181,7 +1189,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
     float l_run = 0.0f;
 
     // One page: step i of the wave, resident in `slot`; the slot is refilled with step i + 2.
-    const auto one_page = [&](uint8_t* slot, int i) {
+    const auto one_page = [&](uint8_t* slot, int i) __attribute__((always_inline)) {
         const int pg = pg0 + wave + kWaves * i;
         const uint8_t* ks = slot;
         const uint8_t* vs = slot + kI8hUnit;
@@ -1324,7 +1332,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
     // no load may still be on its way into the slots when the fold staging takes their place
     __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0)
     __syncthreads();
-    mfma_fold_and_store(P, *reinterpret_cast<MfmaFoldLds*>(ring0), wg, wave, c, g, o, m_run, l_run);
+    mfma_fold_and_store(P, *reinterpret_cast<MfmaFoldLds*>(ring), wg, wave, c, g, o, m_run, l_run);
 }
 
 struct MergeParams {
