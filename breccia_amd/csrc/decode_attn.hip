@@ -1335,6 +1335,277 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
     mfma_fold_and_store(P, *reinterpret_cast<MfmaFoldLds*>(ring), wg, wave, c, g, o, m_run, l_run);
 }
 
+// ---- decode attention on the matrix cores, f16 K and q8_0 V -----------------------------------
+// The MFMA decomposition of decode_attn_mfma_kernel with both operands staged through LDS like the
+// int8 kernel's units (every load of the loop is then a global->LDS load, which keeps the count of
+// loads in flight, and with it every wait, exact): the f16 K unit of the next page is requested
+// when the scores have used this page's, the V units ([f32 scale][32 x i8] blocks, 288 bytes a
+// row) two pages ahead.  A q8_0 value is code * scale with an f32 scale, so it takes a per-cell
+// power of two out first to stay inside f16:
+//   E[cell]  = exponent of the largest of the cell's 8 block scales (clamped to +-120),
+//   a[cell][d] = code * (scale * 2^-E[cell])       |a| < 256; split into hi + lo f16 as below,
+//   weight   = exp2(logit + E[cell] - M)            M the running maximum of logit + E,
+// so that weight * a is the term softmax-weight * value up to the common factor 2^-M, the largest
+// terms have weights near 1 whatever the magnitudes of their values, and what falls off the f16
+// range is small against the largest term.  The denominator sums exp2(logit - M) in f32.
+// scale' = scale * 2^-E is split into two f16 (s_hi + s_lo, 22 bits); code * s_hi is split exactly
+// into hi = f16(.) and its remainder (at most 7 significant bits, a representable f16 number),
+// and lo = remainder + code * s_lo; (hi + lo) . (w_hi + w_lo) on two 32-deep MFMAs as in the int8
+// kernel.
+constexpr int kQ8vRow = row_bytes_of(kRowQ8);  // 288
+constexpr int kQ8vUnit = kPage * kQ8vRow;      // 4608
+
+// K unit in LDS: 8 instructions of 1024 bytes (two rows each), 32 bytes apart so that the rows a
+// fragment read touches spread over the banks.
+constexpr int kQ8vKStep = 1024 + 32;
+constexpr int kQ8vKSlot = 8 * kQ8vKStep;  // 8448
+__device__ __forceinline__ void q8v_k_unit_to_lds(const uint8_t* src, bool real, uint8_t* dst, int lane) {
+    typedef const __attribute__((address_space(1))) void* gptr;
+    typedef __attribute__((address_space(3))) void* lptr;
+    const uint8_t* lane_src = src + (real ? lane * 16 : 0);
+    const int step = real ? 1024 : 0;
+#pragma unroll
+    for (int n = 0; n < 8; ++n)
+        __builtin_amdgcn_global_load_lds((gptr)(lane_src + n * step), (lptr)(dst + n * kQ8vKStep), 16, 0, 0);
+}
+
+// 4608 bytes = 4 x 1024 + 512: four full instructions and one of 32 lanes.  `real` false issues the
+// same five instructions on one 16-byte location (the data is never used): the number of loads
+// in flight, which the waits count, then does not depend on where in its range a wave is.
+__device__ __forceinline__ void q8v_unit_to_lds(const uint8_t* src, bool real, uint8_t* dst, int lane) {
+    typedef const __attribute__((address_space(1))) void* gptr;
+    typedef __attribute__((address_space(3))) void* lptr;
+    const uint8_t* lane_src = src + (real ? lane * 16 : 0);
+    const int step = real ? 1024 : 0;
+#pragma unroll
+    for (int n = 0; n < 4; ++n)
+        __builtin_amdgcn_global_load_lds((gptr)(lane_src + n * step), (lptr)(dst + n * 1024), 16, 0, 0);
+    if (lane < 32) __builtin_amdgcn_global_load_lds((gptr)(lane_src + 4 * step), (lptr)(dst + 4096), 16, 0, 0);
+}
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
+}
+
+__global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const AttnKernelParams P) {
+    // per wave one K slot and two V slots during the loop, the fold staging after it
+    constexpr int kWaveLds = kQ8vKSlot + 2 * kQ8vUnit;
+    constexpr int kLds = kWaves * kWaveLds > (int)sizeof(MfmaFoldLds) ? kWaves * kWaveLds : (int)sizeof(MfmaFoldLds);
+    __shared__ __attribute__((aligned(16))) uint8_t smem[kLds];
+
+    const int unit = blockIdx.x;
+    int e = 0;
+    while (e + 1 < P.b.n && unit >= P.b.wg_base[e + 1]) ++e;
+    const int rem = unit - P.b.wg_base[e];
+    const int split = rem / P.n_kv;
+    const int kvh = rem - split * P.n_kv;
+    const int wg = unit;
+    const int pos = P.b.pos[e];
+    const int n_pages = pos / kPage + 1;
+    const int pps = P.b.pps[e];
+    const int pg0 = split * pps;
+    const int pg1 = min(pg0 + pps, n_pages);
+    typedef const __attribute__((address_space(4))) int32_t* table_ptr;
+    const table_ptr bt = (table_ptr)(uintptr_t)(P.tables + (size_t)P.b.row[e] * (size_t)P.max_pages_per_seq);
+
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int c = lane & 15;
+    const int g = lane >> 4;
+    const size_t k_page_bytes = (size_t)P.n_kv * kPage * kHd * 2;
+    const size_t k_head_off = (size_t)kvh * kPage * kHd * 2;
+    const size_t v_page_bytes = (size_t)P.n_kv * kQ8vUnit;
+    const size_t v_head_off = (size_t)kvh * kQ8vUnit;
+    uint8_t* const kslot = smem + wave * kWaveLds;
+    uint8_t* const slots = kslot + kQ8vKSlot;
+
+    // pipeline steps of this wave: pages pg0 + wave, + kWaves, ...
+    const int n_steps = pg0 + wave < pg1 ? (pg1 - pg0 - wave + kWaves - 1) / kWaves : 0;
+    // physical page of step i; past the wave's last step the answer is not used for its data
+    const auto phys = [&](int i) -> size_t { return (size_t)bt[min(pg0 + wave + kWaves * i, pg1 - 1)]; };
+
+    // Loads complete in order.  Issue order per step: K(i+1) when the scores of step i are done,
+    // V(i+2) at its end; the prologue keeps that order (V0, K0, V1).  Behind K(i) at the top of step
+    // i there is V(i+1) = 5 loads; behind V(i) where step i needs it there are K(i), V(i+1), K(i+1)
+    // = 8 + 5 + 8.  Steps that do not exist are requested all the same, as loads of one location,
+    // so that these counts hold everywhere.
+    const auto k_unit = [&](int i) { return P.kpool + phys(i) * k_page_bytes + k_head_off; };
+    const auto v_unit = [&](int i) { return P.vpool + phys(i) * v_page_bytes + v_head_off; };
+    q8v_unit_to_lds(v_unit(0), n_steps > 0, slots, lane);
+    q8v_k_unit_to_lds(k_unit(0), n_steps > 0, kslot, lane);
+    q8v_unit_to_lds(v_unit(1), n_steps > 1, slots + kQ8vUnit, lane);
+
+    // ---- q fragments of head c (heads past the group stay zero) ----------------------------------
+    half8 qhi[8], qlo[8];
+    {
+        const bool head_live = c < P.group;
+        const float* qp = P.q + ((size_t)e * P.n_q + (size_t)kvh * P.group + (head_live ? c : 0)) * kHd + g * 8;
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+            float x[8];
+            const float4 a = *reinterpret_cast<const float4*>(qp + m * 32);
+            const float4 b = *reinterpret_cast<const float4*>(qp + m * 32 + 4);
+            x[0] = a.x, x[1] = a.y, x[2] = a.z, x[3] = a.w;
+            x[4] = b.x, x[5] = b.y, x[6] = b.z, x[7] = b.w;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                _Float16 hi, lo;
+                split_hi_lo(head_live ? x[j] : 0.0f, hi, lo);
+                qhi[m][j] = hi;
+                qlo[m][j] = lo;
+            }
+        }
+    }
+
+    f4 o[2][8];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int t = 0; t < 8; ++t) o[h][t] = f4{0.0f, 0.0f, 0.0f, 0.0f};
+    float m_run = -INFINITY;  // running maximum of logit + E (base 2)
+    float l_run = 0.0f;       // this lane's share of sum exp2(logit - m_run)
+    const int my_block = c >> 2;  // which of the 4 blocks of a half this lane's 8 columns lie in
+
+    for (int i = 0; i < n_steps; ++i) {
+        const int pg = pg0 + wave + kWaves * i;
+        const uint8_t* vs = slots + (i & 1) * kQ8vUnit;
+        const int behind = n_steps - 1 - i;  // steps after this one
+
+        // ---- S^T = K . q^T: four independent accumulation chains ------------------------------
+        __builtin_amdgcn_s_waitcnt(0x0F75);  // vmcnt(5): this page's K unit has landed
+        v4u kf[8];
+        {
+            // row c: two rows per 1056-byte step; fragment m of lane group g at 64 m + 16 g
+            const uint8_t* kr = kslot + (c >> 1) * kQ8vKStep + (c & 1) * 512 + g * 16;
+#pragma unroll
+            for (int m = 0; m < 8; ++m) kf[m] = *reinterpret_cast<const v4u*>(kr + m * 64);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        f4 s0 = f4{0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0, s2 = s0, s3 = s0;
+#pragma unroll
+        for (int m = 0; m < 8; m += 2) {
+            const half8 ka = __builtin_bit_cast(half8, kf[m]);
+            const half8 kb = __builtin_bit_cast(half8, kf[m + 1]);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qhi[m], s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qlo[m], s1, 0, 0, 0);
+            s2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kb, qhi[m + 1], s2, 0, 0, 0);
+            s3 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kb, qlo[m + 1], s3, 0, 0, 0);
+        }
+        const f4 s = (s0 + s1) + (s2 + s3);  // s[r] = q[head c] . k[cell 4 g + r]
+        q8v_k_unit_to_lds(k_unit(i + 1), behind >= 1, kslot, lane);
+
+        // ---- this page's V unit: scales first -------------------------------------------------
+        __builtin_amdgcn_s_waitcnt(0x4F75);  // vmcnt(21): K(i), V(i+1), K(i+1) behind V(i)
+        // lane (c, g): scale of blocks 2 (c / 4), + 1 of row 4 g + c % 4, the row's maximum over the
+        // lanes c, c ^ 4, c ^ 8, c ^ 12, then the four rows' maxima from the lanes of the quad
+        const bool last_page = pg == n_pages - 1;
+        float smax;
+        {
+            const uint8_t* rp = vs + (4 * g + (c & 3)) * kQ8vRow + (c >> 2) * 72;
+            const float a = *reinterpret_cast<const float*>(rp);
+            const float b = *reinterpret_cast<const float*>(rp + 36);
+            smax = fmaxf(a, b);
+            // rows past `pos` may hold anything: they count as scale 1 here and as zeros below
+            if (last_page && pg * kPage + 4 * g + (c & 3) > pos) smax = 1.0f;
+            smax = fmaxf(smax, dpp_mov<0x124>(smax));  // row_ror:4
+            smax = fmaxf(smax, dpp_mov<0x128>(smax));  // row_ror:8
+        }
+        int ex[4];
+        float down[4];  // 2^-E
+        {
+            const float m0 = dpp_mov<0x00>(smax), m1 = dpp_mov<0x55>(smax);
+            const float m2 = dpp_mov<0xAA>(smax), m3 = dpp_mov<0xFF>(smax);
+            const float mr[4] = {m0, m1, m2, m3};
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                int ee = (int)((__builtin_bit_cast(unsigned, mr[r]) >> 23) & 0xffu) - 127;
+                ee = min(max(ee, -120), 120);
+                ex[r] = ee;
+                down[r] = __builtin_bit_cast(float, (unsigned)(127 - ee) << 23);
+            }
+        }
+
+        // ---- online softmax of head c over logit + E ------------------------------------------------
+        float t4[4], tw[4];
+        float pm = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const bool live = pg * kPage + 4 * g + r <= pos;
+            t4[r] = live ? s[r] * P.scale_log2e : -INFINITY;
+            tw[r] = t4[r] + (float)ex[r];
+            pm = fmaxf(pm, tw[r]);
+        }
+        pm = max_over_lane_groups(pm);
+        const float m_new = fmaxf(m_run, pm);  // finite: every page of a range holds a live cell
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        h4m whi, wlo;
+        float psum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float w = __builtin_amdgcn_exp2f(tw[r] - m_new);
+            psum += __builtin_amdgcn_exp2f(t4[r] - m_new);
+            _Float16 hi, lo;
+            split_hi_lo(w, hi, lo);
+            whi[r] = hi;
+            wlo[r] = lo;
+        }
+        l_run = l_run * alpha + psum;
+        if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int t = 0; t < 8; ++t) o[h][t] *= alpha;
+        }
+        m_run = m_new;
+        const half8 whh = half8{whi[0], whi[1], whi[2], whi[3], whi[0], whi[1], whi[2], whi[3]};
+        const half8 wll = half8{wlo[0], wlo[1], wlo[2], wlo[3], wlo[0], wlo[1], wlo[2], wlo[3]};
+
+        // ---- P.V ----------------------------------------------------------------------------------
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            unsigned wx[4], wy[4], col[8];
+            _Float16 shi[4], slo[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const uint8_t* blk = vs + (4 * g + r) * kQ8vRow + (4 * h + my_block) * 36;
+                float sc = *reinterpret_cast<const float*>(blk) * down[r];
+                if (last_page && pg * kPage + 4 * g + r > pos) sc = 0.0f;
+                split_hi_lo(sc, shi[r], slo[r]);
+                const unsigned* cw = reinterpret_cast<const unsigned*>(blk + 4 + (c & 3) * 8);
+                wx[r] = cw[0] ^ 0x80808080u;
+                wy[r] = cw[1] ^ 0x80808080u;
+            }
+            const h2m s01 = h2m{shi[0], shi[1]}, s23 = h2m{shi[2], shi[3]};
+            const h2m l01 = h2m{slo[0], slo[1]}, l23 = h2m{slo[2], slo[3]};
+            {
+                unsigned t0[4], t1[4];
+                transpose4x4_bytes(wx, t0);
+                transpose4x4_bytes(wy, t1);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) col[t] = t0[t], col[4 + t] = t1[t];
+            }
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                h2m c01, c23;
+                biased_to_f16(col[t], c01, c23);
+                const h2m hi01 = c01 * s01, hi23 = c23 * s23;
+                const h2m lo01 = __builtin_elementwise_fma(c01, l01, __builtin_elementwise_fma(c01, s01, -hi01));
+                const h2m lo23 = __builtin_elementwise_fma(c23, l23, __builtin_elementwise_fma(c23, s23, -hi23));
+                const half8 ahl = half8{hi01[0], hi01[1], hi23[0], hi23[1], lo01[0], lo01[1], lo23[0], lo23[1]};
+                o[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahl, whh, o[h][t], 0, 0, 0);
+                o[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahl, wll, o[h][t], 0, 0, 0);
+            }
+        }
+        q8v_unit_to_lds(v_unit(i + 2), behind >= 2, slots + (i & 1) * kQ8vUnit, lane);
+    }
+
+    // no load may still be on its way into the slots when the fold staging takes their place
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0)
+    __syncthreads();
+    mfma_fold_and_store(P, *reinterpret_cast<MfmaFoldLds*>(smem), wg, wave, c, g, o, m_run, l_run);
+}
+
 struct MergeParams {
     AttnBatch b;
     const float* part_o;
@@ -1466,8 +1737,8 @@ int32_t attn_heads_per_wave(int32_t group) { return group % 8 == 0 ? 8 : 4; }
 // created with BKV_POOL_ATTN_VALU (the VALU formulation, kept for comparison).
 bool attn_on_mfma(const bkv_pool* p, int32_t group, bool dense) {
     if (group > 16 || (p->desc.flags & BKV_POOL_ATTN_VALU) != 0) return false;
-    // f16 rows: every call; int8 rows with f16 scales: the dense selection
-    return p->g.layout == BKV_LAYOUT_F16 || (p->g.layout == BKV_LAYOUT_I8H && dense);
+    // f16 rows: every call; the quantised layouts: the dense selection
+    return p->g.layout == BKV_LAYOUT_F16 || dense;
 }
 
 int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b, int32_t sel_groups, bool mfma) {
@@ -1555,6 +1826,8 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
             // f16 pools, dense selection, one work-group per unit (checked by the caller)
             if (layout == BKV_LAYOUT_I8H)
                 decode_attn_mfma_i8h_kernel<<<total, kBlock, 0, stream>>>(kp);
+            else if (layout == BKV_LAYOUT_Q8V)
+                decode_attn_mfma_q8v_kernel<<<total, kBlock, 0, stream>>>(kp);
             else if (step)
                 decode_attn_mfma_kernel<true><<<total, kBlock, 0, stream>>>(kp);
             else if (sel)

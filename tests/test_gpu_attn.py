@@ -161,14 +161,13 @@ def test_closed_forms_on_the_gpu():
         assert max_abs(out_s[0], want) < 1e-5
 
 
-@pytest.mark.parametrize("loud_rows", [(0, 4), (4, 16), (9, 10), (12, 16)])
-def test_score_spread_across_the_rows_of_a_page(loud_rows):
+def score_spread_case(loud_rows, layout=0):
     # The running maximum of a head must be the maximum over all 16 rows of a page, whichever
     # lanes hold them: cells at page rows [lo, hi) carry scores some 40 (base-2: 58) above the
     # rest, so a maximum taken over part of the rows only would overflow the probabilities.
     rng = np.random.Generator(np.random.PCG64(640 + loud_rows[0]))
     n = 16 * 23 + 7
-    with Twin(n_pages=40, max_seqs=2) as tw:
+    with Twin(n_pages=40, max_seqs=2, layout=layout) as tw:
         s = tw.pool.seq_create()
         tw.pool.seq_reserve(s, n)
         q = rng.standard_normal((1, 16, 256)).astype(np.float32)
@@ -185,6 +184,11 @@ def test_score_spread_across_the_rows_of_a_page(loud_rows):
         out = tw.decode_attn(0, [s], [n - 1], q, 16)
         want = tw.oracle_attend(0, s, n - 1, q[0], 16)
         check_attn(out[0], want, "loud rows %d..%d" % loud_rows)
+
+
+@pytest.mark.parametrize("loud_rows", [(0, 4), (4, 16), (9, 10), (12, 16)])
+def test_score_spread_across_the_rows_of_a_page(loud_rows):
+    score_spread_case(loud_rows)
 
 
 def test_unwritten_and_poisoned_cells_are_never_read_as_values():

@@ -10,7 +10,7 @@ import oracle
 from breccia_amd import lib as L
 from gpu_common import REF_BAR_MAX_REL, Twin, check_attn
 from helpers import max_abs, max_rel
-from test_gpu_attn import fill
+from test_gpu_attn import fill, score_spread_case
 
 pytestmark = pytest.mark.gpu
 
@@ -89,6 +89,12 @@ def test_quantised_values_across_the_scale_range(layout, v_mag):
             assert np.max(np.abs(want)) > 0.0
             rel = max_abs(out[i], want) / float(np.max(np.abs(want)))
             assert rel <= REF_BAR_MAX_REL, (i, rel)
+
+
+@pytest.mark.parametrize("layout", [L.LAYOUT_Q8V, L.LAYOUT_I8H])
+@pytest.mark.parametrize("loud_rows", [(4, 16), (9, 10)])
+def test_quantised_score_spread_across_the_rows_of_a_page(layout, loud_rows):
+    score_spread_case(loud_rows, layout)
 
 
 @pytest.mark.parametrize("layout", [L.LAYOUT_Q8V, L.LAYOUT_I8H])
