@@ -341,10 +341,11 @@ def bench_quantised(stream) -> dict:
 
     res = {}
     cases = [("attn_q8v_batch8", L.LAYOUT_Q8V, ROW_BYTES_Q8V, 8, 1024, 32768, 4, 20250003,
-              "headline batch on f16 K + q8_0 V"),
+              "headline batch on f16 K + q8_0 V", "decode_attn_mfma_q8v_kernel"),
              ("attn_int8_batch16", L.LAYOUT_I8H, ROW_BYTES_I8H, 16, 8192, 131072, 2, 20250005,
-              "BASELINE configs[4]: 16 sequences, ctx U{8k..128k}, int8 K/V + f16 scales")]
-    for name, layout, row_bytes, n_seqs, lo, hi, n_layers, seed, what in cases:
+              "BASELINE configs[4]: 16 sequences, ctx U{8k..128k}, int8 K/V + f16 scales",
+              "decode_attn_mfma_i8h_kernel")]
+    for name, layout, row_bytes, n_seqs, lo, hi, n_layers, seed, what, kernel in cases:
         rng = np.random.Generator(np.random.PCG64(seed))
         pool, seqs, ctx = build_batched(None, rng, n_seqs, lo, hi, n_layers, 0.6, layout)
         # contents: one resident block of N(0,1) rows appended at every chunk of every sequence
@@ -370,7 +371,7 @@ def bench_quantised(stream) -> dict:
         n_merge, ms_merge = pool.timing_read(L.STAGE_ATTN_MERGE)
         b = attn_algorithmic_bytes([c + 1 + (steps + warm) // n_layers for c in ctx], row_bytes)
         split_us = ms_split / max(n_split, 1) * 1e3
-        res[name] = {"workload": what, "cells": sum(ctx), "algorithmic_bytes": b,
+        res[name] = {"workload": what, "kernel": kernel, "cells": sum(ctx), "algorithmic_bytes": b,
                      "us_per_layer": round(wall_ms / steps * 1e3, 2),
                      "attn_split_us": round(split_us, 2),
                      "attn_merge_us": round(ms_merge / max(n_merge, 1) * 1e3, 2),

@@ -1103,14 +1103,18 @@ __device__ __forceinline__ float scale_of(_Float16 h) {
 constexpr int kI8hUnit = kPage * row_bytes_of(kRowI8H);  // 4352
 constexpr int kI8hSlot = 2 * kI8hUnit;                    // K unit, then V unit
 
-// 4352 bytes = 4 x 1024 + 256: four full instructions and one of 16 lanes
-__device__ __forceinline__ void i8h_unit_to_lds(const uint8_t* src, uint8_t* dst, int lane) {
+// 4352 bytes = 4 x 1024 + 256: four full instructions and one of 16 lanes.  `real` false issues the
+// same five instructions on one 16-byte location (the data is never used): the number of loads
+// in flight, which the waits count, then does not depend on where in its range a wave is.
+__device__ __forceinline__ void i8h_unit_to_lds(const uint8_t* src, bool real, uint8_t* dst, int lane) {
     typedef const __attribute__((address_space(1))) void* gptr;
     typedef __attribute__((address_space(3))) void* lptr;
+    const uint8_t* lane_src = src + (real ? lane * 16 : 0);
+    const int step = real ? 1024 : 0;
 #pragma unroll
     for (int n = 0; n < 4; ++n)
-        __builtin_amdgcn_global_load_lds((gptr)(src + n * 1024 + lane * 16), (lptr)(dst + n * 1024), 16, 0, 0);
-    if (lane < 16) __builtin_amdgcn_global_load_lds((gptr)(src + 4096 + lane * 16), (lptr)(dst + 4096), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gptr)(lane_src + n * step), (lptr)(dst + n * 1024), 16, 0, 0);
+    if (lane < 16) __builtin_amdgcn_global_load_lds((gptr)(lane_src + 4 * step), (lptr)(dst + 4096), 16, 0, 0);
 }
 
 __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const AttnKernelParams P) {
@@ -1146,17 +1150,16 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
     uint8_t* const slot0 = ring0 + wave * kI8hSlot;
     uint8_t* const slot1 = ring1 + wave * kI8hSlot;
 
-    // page of pipeline step i of this wave; past the range the last page is fetched again (and
-    // never used) so that the number of loads in flight stays what the waits assume
+    // unit of pipeline step i of this wave; steps past the wave's last are requested all the same,
+    // as loads of one location, so that the number of loads in flight stays what the waits assume
+    const int n_steps = pg0 + wave < pg1 ? (pg1 - pg0 - wave + kWaves - 1) / kWaves : 0;
     const auto unit_off = [&](int i) -> size_t {
         return (size_t)bt[min(pg0 + wave + kWaves * i, pg1 - 1)] * page_bytes + head_off;
     };
-    if (pg0 < pg1) {  // always: a range holds at least one page
-        i8h_unit_to_lds(P.kpool + unit_off(0), slot0, lane);
-        i8h_unit_to_lds(P.vpool + unit_off(0), slot0 + kI8hUnit, lane);
-        i8h_unit_to_lds(P.kpool + unit_off(1), slot1, lane);
-        i8h_unit_to_lds(P.vpool + unit_off(1), slot1 + kI8hUnit, lane);
-    }
+    i8h_unit_to_lds(P.kpool + unit_off(0), n_steps > 0, slot0, lane);
+    i8h_unit_to_lds(P.vpool + unit_off(0), n_steps > 0, slot0 + kI8hUnit, lane);
+    i8h_unit_to_lds(P.kpool + unit_off(1), n_steps > 1, slot1, lane);
+    i8h_unit_to_lds(P.vpool + unit_off(1), n_steps > 1, slot1 + kI8hUnit, lane);
 
     // ---- q fragments of head c (heads past the group stay zero) ----------------------------------
     half8 qhi[8], qlo[8];
@@ -1226,7 +1229,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
 #pragma unroll
             for (int r = 0; r < 4; ++r) s[r] = fmaf((float)ksc[r][m], part[r], s[r]);
         }
-        i8h_unit_to_lds(P.kpool + off_next, slot, lane);
+        i8h_unit_to_lds(P.kpool + off_next, i + 2 < n_steps, slot, lane);
 
         // ---- online softmax of head c ---------------------------------------------------------------
         float t4[4];
@@ -1323,10 +1326,9 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
                 o[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahl, pll, o[h][t], 0, 0, 0);
             }
         }
-        i8h_unit_to_lds(P.vpool + off_next, slot + kI8hUnit, lane);
+        i8h_unit_to_lds(P.vpool + off_next, i + 2 < n_steps, slot + kI8hUnit, lane);
     };
 
-    const int n_steps = pg0 + wave < pg1 ? (pg1 - pg0 - wave + kWaves - 1) / kWaves : 0;
     for (int i = 0; i < n_steps; ++i) one_page((i & 1) ? slot1 : slot0, i);
 
     // no load may still be on its way into the slots when the fold staging takes their place

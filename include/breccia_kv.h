@@ -48,9 +48,9 @@ typedef enum bkv_layout {
 enum {
     BKV_POOL_HOST_ONLY = 1u, /* allocator + block tables only; device calls fail with
                                 BKV_ERR_NO_DEVICE (for hosts without a GPU) */
-    BKV_POOL_ATTN_VALU = 2u  /* f16 pools: dense decode attention in the VALU formulation (chunks
-                                of 8 or 4 heads, no MFMA) instead of the MFMA one; same results,
-                                kept for comparison */
+    BKV_POOL_ATTN_VALU = 2u  /* decode attention in the VALU formulation (chunks of 8 or 4 heads,
+                                no MFMA) instead of the MFMA one; same results, kept for
+                                comparison */
 };
 
 #define BKV_MAX_BATCH 64      /* (sequence, position) entries per append / attention call */
@@ -232,10 +232,12 @@ bkv_status bkv_rope_table(double freq_base, int32_t n_rot, int32_t max_pos, floa
  * reference reads it in place from q_full at h*512+256+d, shaders/qsa_attn_apply.comp).
  * The same sequence may appear several times with different pos (T > 1 decode).
  * One split-K online-softmax kernel plus one merge kernel; partials live in a
- * workspace the pool owns.  On f16 pools the split-K kernel multiplies on the matrix cores
- * (all heads of a kv head, up to 16, in one pass over the K/V rows; q and the probabilities
- * as high + low f16 parts, so accuracy is that of f32 accumulation), also for selection
- * lists and the fused step; quantised pools use the VALU kernel (heads in chunks of 8 or 4). */
+ * workspace the pool owns.  The split-K kernel multiplies on the matrix cores (all heads of a
+ * kv head, up to 16, in one pass over the K/V rows; q and the probabilities as high + low f16
+ * parts, quantised values as exact high + low f16 parts, so accuracy is that of f32
+ * accumulation): on f16 pools always, also for selection lists and the fused step; on the
+ * quantised pools for this call, while their selection lists use the VALU kernel (heads in
+ * chunks of 8 or 4). */
 bkv_status bkv_decode_attn(bkv_pool *pool, int32_t layer, int32_t n, const int32_t *seqs,
                            const int64_t *pos, int32_t n_q_head, const float *q_dev,
                            const float *gate_dev, int64_t gate_seq_stride,
