@@ -24,6 +24,7 @@
 // the merge kernel combines the splits and applies sigmoid(gate).
 #include "bkv_internal.hpp"
 #include "f16_rule.hpp"
+#include "lane_groups.hpp"
 
 namespace bkv {
 
@@ -656,43 +657,13 @@ __global__ __launch_bounds__(kBlock, HG == 8 ? 2 : 3) void decode_attn_kernel(co
 // holds up to 16 heads of a kv head at once, every K/V row is still read once, and the VALU
 // only does the softmax.  Lane (c = lane % 16, g = lane / 16) of a wave owns head c; per page:
 //   S^T[cell][head] = K[cell][:] . q[head][:]          v_mfma_f32_16x16x32_f16, A = K, B = q
-//   O^T[d][head]   += V^T[d][cell] . P^T[cell][head]   v_mfma_f32_16x16x16_f16, A = V regrouped
+//   O^T[d][head]   += V^T[d][cell] . P^T[cell][head]   v_mfma_f32_16x16x32_f16, A = V regrouped
 // with q and p split into a high and a low f16 part (K and V are exact f16), as in the prefill
-// kernel.  K fragment m of a lane is the 16 bytes at element 32 m + 8 g of row c; V fragments
+// kernel: two MFMAs per K fragment, and for P.V one MFMA whose 32-deep contraction runs over the
+// page's 16 cells twice, against p's high parts and against its low parts.  K fragment m of a lane is the 16 bytes at element 32 m + 8 g of row c; V fragments
 // are the 16 bytes at element 128 h + 8 c of rows 4 g + r.  Every fragment register is
 // refilled with the next page's data right after its last use.
 typedef _Float16 h4m __attribute__((ext_vector_type(4)));
-
-// Reductions over the four lanes {c, c + 16, c + 32, c + 48}, result in every one of them, on the
-// VALU: v_permlane32_swap exchanges the upper half of its first register with the lower half of
-// its second, v_permlane16_swap the odd rows of the first with the even rows of the second, so
-// with two copies of x the two registers then hold x[l] and x[l ^ 32] (x[l ^ 16]) side by side.
-// Written as asm with both registers as in/out operands: the compiler's two-result builtin for
-// these instructions hands back its first result twice.  The s_nop covers the wait states the
-// swap needs after a VALU write of its operands.
-struct LanePair {
-    float a, b;
-};
-__device__ __forceinline__ LanePair swap_halves(float x) {
-    LanePair p{x, x};
-    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(p.a), "+v"(p.b));
-    return p;
-}
-__device__ __forceinline__ LanePair swap_rows(float x) {
-    LanePair p{x, x};
-    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(p.a), "+v"(p.b));
-    return p;
-}
-__device__ __forceinline__ float max_over_lane_groups(float x) {
-    const LanePair p = swap_halves(x);
-    const LanePair q = swap_rows(fmaxf(p.a, p.b));
-    return fmaxf(q.a, q.b);
-}
-__device__ __forceinline__ float sum_over_lane_groups(float x) {
-    const LanePair p = swap_halves(x);
-    const LanePair q = swap_rows(p.a + p.b);
-    return q.a + q.b;
-}
 
 __device__ __forceinline__ void split_hi_lo(float x, _Float16& hi, _Float16& lo) {
     hi = (_Float16)x;
@@ -987,6 +958,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
             phi[r] = hi;
             plo[r] = lo;
         }
+        const half8 phl = half8{phi[0], phi[1], phi[2], phi[3], plo[0], plo[1], plo[2], plo[3]};
         l_run = l_run * alpha + psum;
         if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
 #pragma unroll
@@ -1020,9 +992,10 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
             const half8 v2 = __builtin_bit_cast(half8, vf[h][2]), v3 = __builtin_bit_cast(half8, vf[h][3]);
 #pragma unroll
             for (int t = 0; t < 8; ++t) {
-                const h4m va = h4m{v0[t], v1[t], v2[t], v3[t]};
-                o[h][t] = __builtin_amdgcn_mfma_f32_16x16x16f16(va, phi, o[h][t], 0, 0, 0);
-                o[h][t] = __builtin_amdgcn_mfma_f32_16x16x16f16(va, plo, o[h][t], 0, 0, 0);
+                // the 32-deep MFMA runs over the page's 16 cells twice: against the high parts of p
+                // and against the low parts
+                const half8 vv = half8{v0[t], v1[t], v2[t], v3[t], v0[t], v1[t], v2[t], v3[t]};
+                o[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vv, phl, o[h][t], 0, 0, 0);
             }
             if (more) {
 #pragma unroll

@@ -14,16 +14,20 @@
 // cells and per wave:
 //   S^T[cell][query] = K[cell][:] . Q[query][:]        v_mfma_f32_16x16x32_f16, A = K, B = Q
 //   online softmax per query (base 2), P^T in the layout S^T came out in
-//   O^T[d][query]   += V^T[d][cell] . P^T[cell][query]  v_mfma_f32_16x16x16_f16 (a page is 16
-//                                                       cells), A = V gathered per lane, B = P^T
+//   O^T[d][query]   += V^T[d][cell] . P^T[cell][query]  v_mfma_f32_16x16x32_f16 over the page's 16
+//                                                       cells twice, A = V gathered per lane (the
+//                                                       same four cells in both halves of a lane's
+//                                                       slots), B = P^T high parts, then low parts
 // Both products keep the per-lane query (lane % 16) fixed, so the softmax statistics never
 // move between lanes, and P^T feeds the second product straight from registers.  K and V are
-// exact f16; q and p are f32 values split into a high and a low f16 part (two MFMAs each), so
-// the products carry ~22 significant bits and the result stays at f32-accumulate accuracy.
+// exact f16; q and p are f32 values split into a high and a low f16 part (two MFMAs for the
+// scores, the two halves of one for P.V), so the products carry ~22 significant bits and the
+// result stays at f32-accumulate accuracy.
 // The V operand needs four cells of one head-dim column per lane: each lane loads 16 bytes
 // (8 columns) of four rows and regroups them in registers; the 8 MFMAs that use them produce
 // columns 8i + t of the output, i = the MFMA row, t = 0..7.
 #include "bkv_internal.hpp"
+#include "lane_groups.hpp"
 
 namespace bkv {
 
@@ -33,6 +37,8 @@ constexpr int kHd = 256;
 constexpr int kPage = 16;
 constexpr int kRowsPerWave = 16;
 constexpr int kWavesPerWg = 4;
+constexpr int kThreads = 64 * kWavesPerWg;
+constexpr int kChunks = kPage * kHd * 2 / 16 / kThreads;  // 16-byte chunks of a K (or V) page image per thread
 constexpr int kRowsPerWg = kRowsPerWave * kWavesPerWg;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kLdsRow = kHd + 8;  // halves per row of a page image in LDS (528 bytes)
@@ -55,9 +61,6 @@ struct PrefillKernelParams {
     float scale_log2e;
 };
 
-__device__ __forceinline__ f4 mfma16(h4 a, h4 b, f4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x16f16(a, b, c, 0, 0, 0);
-}
 // gfx950's double-depth form: 32 contraction steps, 8 halves per lane (k = 8 (lane / 16) + 0..7)
 __device__ __forceinline__ f4 mfma32(h8 a, h8 b, f4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
@@ -68,7 +71,7 @@ __device__ __forceinline__ void split_f16(float x, _Float16& hi, _Float16& lo) {
     lo = (_Float16)(x - (float)hi);
 }
 
-__global__ __launch_bounds__(64 * kWavesPerWg, 2) void prefill_attn_kernel(const PrefillKernelParams P) {
+__global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const PrefillKernelParams P) {
     // ---- which (entry, kv head, block of 64 query rows) ---------------------------------
     int e = 0;
     while (e + 1 < P.b.n && (int)blockIdx.x >= P.b.wg_base[e + 1]) ++e;
@@ -142,25 +145,28 @@ __global__ __launch_bounds__(64 * kWavesPerWg, 2) void prefill_attn_kernel(const
 
     // ---- pages through LDS: [buffer][K | V][16 rows][264 halves] -------------------------------
     // Rows are padded to 528 bytes so that the 16-byte fragment reads of the 64 lanes spread
-    // evenly over the banks.  A page image is 2 x 512 chunks of 16 bytes: thread t moves chunks
-    // t and t + 256 of K and of V.
+    // evenly over the banks.  A page image is 2 x 512 chunks of 16 bytes: thread t moves chunk
+    // t (+ kThreads, ...) of K and of V.
     __shared__ __attribute__((aligned(16))) _Float16 lds[2][2][kPage][kLdsRow];
     const int tid = threadIdx.x;
-    const auto fetch = [&](int pg, v4u (&stage)[4]) {
+    const auto fetch = [&](int pg, v4u (&stage)[2 * kChunks]) {
         const int32_t phys = bt[pg];
         const uint8_t* kp = P.kpool + (size_t)phys * page_bytes + head_off;
         const uint8_t* vp = P.vpool + (size_t)phys * page_bytes + head_off;
-        stage[0] = *reinterpret_cast<const v4u*>(kp + (size_t)tid * 16);
-        stage[1] = *reinterpret_cast<const v4u*>(kp + (size_t)(tid + 256) * 16);
-        stage[2] = *reinterpret_cast<const v4u*>(vp + (size_t)tid * 16);
-        stage[3] = *reinterpret_cast<const v4u*>(vp + (size_t)(tid + 256) * 16);
+#pragma unroll
+        for (int j = 0; j < kChunks; ++j) {
+            stage[j] = *reinterpret_cast<const v4u*>(kp + (size_t)(tid + j * kThreads) * 16);
+            stage[kChunks + j] = *reinterpret_cast<const v4u*>(vp + (size_t)(tid + j * kThreads) * 16);
+        }
     };
-    const auto deposit = [&](int buf, const v4u (&stage)[4]) {
+    const auto deposit = [&](int buf, const v4u (&stage)[2 * kChunks]) {
         // chunk q of a page image: row q / 32, halves (q % 32) * 8 ..
-        *reinterpret_cast<v4u*>(&lds[buf][0][tid >> 5][(tid & 31) * 8]) = stage[0];
-        *reinterpret_cast<v4u*>(&lds[buf][0][(tid >> 5) + 8][(tid & 31) * 8]) = stage[1];
-        *reinterpret_cast<v4u*>(&lds[buf][1][tid >> 5][(tid & 31) * 8]) = stage[2];
-        *reinterpret_cast<v4u*>(&lds[buf][1][(tid >> 5) + 8][(tid & 31) * 8]) = stage[3];
+#pragma unroll
+        for (int j = 0; j < kChunks; ++j) {
+            const int q = tid + j * kThreads;
+            *reinterpret_cast<v4u*>(&lds[buf][0][q >> 5][(q & 31) * 8]) = stage[j];
+            *reinterpret_cast<v4u*>(&lds[buf][1][q >> 5][(q & 31) * 8]) = stage[kChunks + j];
+        }
     };
 
     // one page of this wave: scores -> softmax -> accumulate, operands from LDS buffer `buf`
@@ -170,17 +176,27 @@ __global__ __launch_bounds__(64 * kWavesPerWg, 2) void prefill_attn_kernel(const
         // ---- S^T = K . Q^T ------------------------------------------------------------------
         // four independent accumulation chains: an MFMA that waits for the previous one's result
         // costs its full latency
+        // K: row c, 16 bytes at element 32 m + 8 g (the same split of the head dim as q): the 8
+        // halves of a lane are the 8 contraction steps it feeds to the 32-deep MFMA.  All fragments
+        // of the page are requested from LDS in one batch; V's follow while the scores are formed.
+        h8 kf[8];
+#pragma unroll
+        for (int m = 0; m < 8; ++m) kf[m] = *reinterpret_cast<const h8*>(ks + c * kLdsRow + m * 32 + g * 8);
+        __builtin_amdgcn_sched_barrier(0);
+        // V: rows 4 g + r, 16 bytes at element 128 half + 8 c
+        v4u vf[2][4];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                vf[h][r] = *reinterpret_cast<const v4u*>(vs + (4 * g + r) * kLdsRow + h * 128 + c * 8);
         f4 s0 = f4{0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0, s2 = s0, s3 = s0;
 #pragma unroll
         for (int m = 0; m < 8; m += 2) {
-            // K: row c, 16 bytes at element 32 m + 8 g (the same split of the head dim as q): the
-            // 8 halves of a lane are the 8 contraction steps it feeds to the 32-deep MFMA
-            const h8 ka = *reinterpret_cast<const h8*>(ks + c * kLdsRow + m * 32 + g * 8);
-            const h8 kb = *reinterpret_cast<const h8*>(ks + c * kLdsRow + (m + 1) * 32 + g * 8);
-            s0 = mfma32(ka, qhi[m], s0);
-            s1 = mfma32(ka, qlo[m], s1);
-            s2 = mfma32(kb, qhi[m + 1], s2);
-            s3 = mfma32(kb, qlo[m + 1], s3);
+            s0 = mfma32(kf[m], qhi[m], s0);
+            s1 = mfma32(kf[m], qlo[m], s1);
+            s2 = mfma32(kf[m + 1], qhi[m + 1], s2);
+            s3 = mfma32(kf[m + 1], qlo[m + 1], s3);
         }
         const f4 s = (s0 + s1) + (s2 + s3);
         // s[r] = q[row c] . k[cell 4 g + r]
@@ -194,8 +210,7 @@ __global__ __launch_bounds__(64 * kWavesPerWg, 2) void prefill_attn_kernel(const
             t4[r] = cell <= pos_q ? s[r] * P.scale_log2e : -INFINITY;
             pm = fmaxf(pm, t4[r]);
         }
-        pm = fmaxf(pm, __shfl_xor(pm, 16, 64));
-        pm = fmaxf(pm, __shfl_xor(pm, 32, 64));
+        pm = max_over_lane_groups(pm);
         const float m_new = fmaxf(m_run, pm);
         // a query with no live cell yet keeps m = -inf: exp2(-inf - -inf) would be NaN
         const float alpha = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
@@ -210,6 +225,7 @@ __global__ __launch_bounds__(64 * kWavesPerWg, 2) void prefill_attn_kernel(const
             phi[r] = hi;
             plo[r] = lo;
         }
+        const h8 phl = h8{phi[0], phi[1], phi[2], phi[3], plo[0], plo[1], plo[2], plo[3]};
         l_run = l_run * alpha + psum;
         m_run = m_new;
         if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
@@ -221,13 +237,6 @@ __global__ __launch_bounds__(64 * kWavesPerWg, 2) void prefill_attn_kernel(const
 
         // Rows past the last position of this wave were never written for these queries and may
         // hold anything (even NaN): make them exact zeros before they meet a zero probability.
-        // V: rows 4 g + r, 16 bytes at element 128 half + 8 c
-        v4u vf[2][4];
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-                vf[h][r] = *reinterpret_cast<const v4u*>(vs + (4 * g + r) * kLdsRow + h * 128 + c * 8);
         if (pg == n_pages - 1) {
 #pragma unroll
             for (int r = 0; r < 4; ++r)
@@ -244,16 +253,17 @@ __global__ __launch_bounds__(64 * kWavesPerWg, 2) void prefill_attn_kernel(const
             const h8 v2 = __builtin_bit_cast(h8, vf[h][2]), v3 = __builtin_bit_cast(h8, vf[h][3]);
 #pragma unroll
             for (int t = 0; t < 8; ++t) {
-                const h4 va = h4{v0[t], v1[t], v2[t], v3[t]};  // column 128 h + 8 c + t of cells 4 g ..
-                o[h][t] = mfma16(va, phi, o[h][t]);
-                o[h][t] = mfma16(va, plo, o[h][t]);
+                // column 128 h + 8 c + t of cells 4 g ..: the 32-deep MFMA runs over the 16 cells twice,
+                // against the high parts of p and then the low parts
+                const h8 vv = h8{v0[t], v1[t], v2[t], v3[t], v0[t], v1[t], v2[t], v3[t]};
+                o[h][t] = mfma32(vv, phl, o[h][t]);
             }
         }
     };
 
     // Two pages are in flight behind the one being multiplied: staging set A carries the even
     // pages, B the odd ones (past the end they carry the last page again).
-    v4u stage_a[4], stage_b[4];
+    v4u stage_a[2 * kChunks], stage_b[2 * kChunks];
     const int last_pg = wg_pages - 1;
     fetch(0, stage_a);
     fetch(min(1, last_pg), stage_b);
@@ -273,8 +283,7 @@ __global__ __launch_bounds__(64 * kWavesPerWg, 2) void prefill_attn_kernel(const
     }
 
     // ---- normalise, gate, store ---------------------------------------------------------------------
-    l_run += __shfl_xor(l_run, 16, 64);
-    l_run += __shfl_xor(l_run, 32, 64);
+    l_run = sum_over_lane_groups(l_run);
     if (!row_live) return;
     const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
     float* op = P.out + ((size_t)(P.b.src0[e] + tok) * P.n_q + head) * kHd;
@@ -332,7 +341,7 @@ hipError_t launch_prefill_attn(bkv_pool* p, int32_t layer, const PrefillBatch& b
     const int32_t grid = b.wg_base[b.n];
     if (grid == 0) return hipSuccess;
     StageScope timed(p, BKV_STAGE_ATTN_SPLIT, stream);
-    prefill_attn_kernel<<<grid, 64 * kWavesPerWg, 0, stream>>>(kp);
+    prefill_attn_kernel<<<grid, kThreads, 0, stream>>>(kp);
     return hipGetLastError();
 }
 
