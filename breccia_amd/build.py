@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libbreccia_kv.so")
 
-SOURCES = ["allocator.cpp", "prefix_tree.cpp", "api.hip", "kv_move.hip", "decode_attn.hip", "prefill_attn.hip", "select.hip"]
+SOURCES = ["allocator.cpp", "prefix_tree.cpp", "api.hip", "kv_move.hip", "decode_attn.hip", "decode_attn_mfma.hip", "prefill_attn.hip", "select.hip"]
 ARCH = "gfx950"
 # Packed-FP32 VALU forms are switched off for every kernel in this library.
 HIP_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",

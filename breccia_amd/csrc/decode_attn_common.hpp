@@ -1,0 +1,79 @@
+// Shared by the decode attention translation units: the kernel parameter block, the geometry the
+// kernels are built for, the row encodings of the pools and where the rows of one loop iteration
+// live.
+#pragma once
+
+#include "bkv_internal.hpp"
+
+namespace bkv {
+
+constexpr int kHd = 256;      // head_dim the kernel is built for
+constexpr int kPage = 16;     // cells per page
+constexpr int kWaves = 4;
+constexpr int kBlock = 64 * kWaves;
+constexpr float kLog2e = 1.4426950408889634f;
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+
+struct AttnKernelParams {
+    AttnBatch b;
+    const uint8_t* kpool;
+    const uint8_t* vpool;
+    const int32_t* tables;
+    const float* q;
+    float* part_o;
+    float* part_ml;
+    int32_t max_pages_per_seq;
+    int32_t n_kv, n_q, group, n_hc;
+    float scale_log2e;
+    // selection lists (decode_attn_kernel<..., true> only): entry e attends the 4-cell blocks
+    // ids[e * id_stride + 0 .. min(counts[e], max_ids))
+    const uint32_t* ids;
+    const uint32_t* counts;
+    int64_t id_stride;
+    int32_t max_ids;
+    // fused decode step (decode_attn_kernel<..., STEP = true> only): the K/V row of cell pos of
+    // entry e comes from new_k / new_v [n][n_kv][head_dim] f32 and is stored into the pool on the way
+    const float* new_k;
+    const float* new_v;
+    uint8_t* kpool_w;
+    uint8_t* vpool_w;
+};
+
+// Row encodings of the K and V pools:
+//   kRowF16   256 f16
+//   kRowQ8    8 x [f32 scale][32 x i8]         (reference q8_0 V, shaders/qsa_kv_append.comp:
+//             38-44; value = i8 * scale, qsa_attn_apply.comp:70-77)
+//   kRowI8H   [256 x i8][8 x f16 scale]
+constexpr int kRowF16 = 0, kRowQ8 = 1, kRowI8H = 2;
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+typedef unsigned v2u __attribute__((ext_vector_type(2)));
+
+__host__ __device__ constexpr int row_bytes_of(int enc) {
+    return enc == kRowF16 ? kHd * 2 : enc == kRowQ8 ? (kHd / 32) * 36 : kHd + (kHd / 32) * 2;
+}
+
+// Where the 16 rows of one loop iteration live.  Dense: one page (one run of 16 rows).
+// Selection: four selected blocks of four cells (crates/breccia-kernels/src/qsa/cpu.rs:
+// 248-257: block b covers cells 4b..4b+3), each a run of 4 rows inside some page; `id` keeps
+// the block ids for the causal test, 0xffffffff for a slot past the end of the list.
+template <bool SEL>
+struct RowRuns {
+    const uint8_t* k[SEL ? 4 : 1];
+    const uint8_t* v[SEL ? 4 : 1];
+    uint32_t id[SEL ? 4 : 1];
+};
+
+// cell 4*id + r of a selected block is attended iff it is not past the query's position
+// (shaders/qsa_attn_scores_small.comp: `cell > pos` is a dead slot)
+__device__ __forceinline__ bool block_cell_live(uint32_t id, int r, int pos) {
+    return id < 0x40000000u && id * 4u + (uint32_t)r <= (uint32_t)pos;
+}
+
+// The split-K kernels on the matrix cores (decode_attn_mfma.hip); `total` work-groups, one per
+// (entry, kv head, page range).
+hipError_t launch_decode_attn_mfma(const AttnKernelParams& kp, int layout, bool step, bool sel, int32_t total,
+                                   hipStream_t stream);
+
+}  // namespace bkv

@@ -1,0 +1,961 @@
+// Paged decode attention for gfx950 on the matrix cores: the split-K kernels for f16 pools, for
+// int8 K/V with f16 block scales and for f16 K + q8_0 V.  Same work decomposition, partial layout
+// and merge kernel as the VALU formulation in decode_attn.hip; must agree with the reference's
+// f64 CPU attend (crates/breccia-kernels/src/qsa/cpu.rs:197-246).
+#include "decode_attn_common.hpp"
+#include "f16_rule.hpp"
+#include "lane_groups.hpp"
+
+namespace bkv {
+
+namespace {
+
+// ---- decode attention on the matrix cores -----------------------------------------------------
+// The same split-K decomposition and the same partial-result layout as decode_attn_kernel, for
+// f16 pools and head groups the 8- or 4-head VALU kernel would have to walk in several chunks
+// (the reference's own 24 q / 2 kv heads = 12 per group; 32 / 2 = 16): a 16-column MFMA tile
+// holds up to 16 heads of a kv head at once, every K/V row is still read once, and the VALU
+// only does the softmax.  Lane (c = lane % 16, g = lane / 16) of a wave owns head c; per page:
+//   S^T[cell][head] = K[cell][:] . q[head][:]          v_mfma_f32_16x16x32_f16, A = K, B = q
+//   O^T[d][head]   += V^T[d][cell] . P^T[cell][head]   v_mfma_f32_16x16x32_f16, A = V regrouped
+// with q and p split into a high and a low f16 part (K and V are exact f16), as in the prefill
+// kernel: two MFMAs per K fragment, and for P.V one MFMA whose 32-deep contraction runs over the
+// page's 16 cells twice, against p's high parts and against its low parts.  K fragment m of a lane is the 16 bytes at element 32 m + 8 g of row c; V fragments
+// are the 16 bytes at element 128 h + 8 c of rows 4 g + r.  Every fragment register is
+// refilled with the next page's data right after its last use.
+typedef _Float16 h4m __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void split_hi_lo(float x, _Float16& hi, _Float16& lo) {
+    hi = (_Float16)x;
+    lo = (_Float16)(x - (float)hi);
+}
+
+constexpr int kOwStride = kHd + 4;  // floats per head in the wave-merge staging
+
+// Shared tail of the MFMA decode kernels: wave totals, then every wave stages its scaled O in
+// LDS and each wave sums one quarter of the columns over the four stagings and writes it as the
+// work-group's partial (m, l, O) in the layout the merge kernel reads.
+// o[h][t][r] of lane (c, g) is out[head c][128 h + 8 (4 g + r) + t].
+struct MfmaFoldLds {
+    float ow[kWaves][16][kOwStride];
+    float wave_m[kWaves][16];
+    float wave_l[kWaves][16];
+};
+
+__device__ __forceinline__ void mfma_fold_and_store(const AttnKernelParams& P, MfmaFoldLds& L, int wg, int wave,
+                                                    int c, int g, f4 (&o)[2][8], float m_run, float l_run) {
+    auto& ow = L.ow;
+    auto& wave_m = L.wave_m;
+    auto& wave_l = L.wave_l;
+    l_run = sum_over_lane_groups(l_run);
+    if (g == 0) {
+        wave_m[wave][c] = m_run;
+        wave_l[wave][c] = l_run;
+    }
+    __syncthreads();
+    float mx = wave_m[0][c];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) mx = fmaxf(mx, wave_m[w][c]);
+    float lsum = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+        const float mw = wave_m[w][c];
+        lsum = fmaf(mw == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(mw - mx), wave_l[w][c], lsum);
+    }
+    {
+        const float f = m_run == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m_run - mx);
+        // element (h, r, t) of a lane is out[head c][128 h + 8 (4 g + r) + t]: 8 consecutive floats per (h, r)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float* d = &ow[wave][c][128 * h + 8 * (4 * g + r)];
+                *reinterpret_cast<f4*>(d) = f4{o[h][0][r] * f, o[h][1][r] * f, o[h][2][r] * f, o[h][3][r] * f};
+                *reinterpret_cast<f4*>(d + 4) = f4{o[h][4][r] * f, o[h][5][r] * f, o[h][6][r] * f, o[h][7][r] * f};
+            }
+    }
+    __syncthreads();
+    // wave w sums columns [64 w, 64 w + 64): lane (c, g) takes 4 columns at 4 c of heads g, g + 4, ...
+    const int hg = P.group;
+#pragma unroll
+    for (int hp = 0; hp < 16; hp += 4) {
+        const int head = hp + g;
+        if (hp >= hg) break;
+        if (head < hg) {
+            const int col = 64 * wave + 4 * c;
+            f4 acc = *reinterpret_cast<const f4*>(&ow[0][head][col]);
+#pragma unroll
+            for (int w = 1; w < kWaves; ++w) acc += *reinterpret_cast<const f4*>(&ow[w][head][col]);
+            *reinterpret_cast<f4*>(P.part_o + ((size_t)wg * hg + head) * kHd + col) = acc;
+        }
+    }
+    if (wave == 0 && g == 0 && c < hg) {
+        P.part_ml[((size_t)wg * hg + c) * 2 + 0] = mx;
+        P.part_ml[((size_t)wg * hg + c) * 2 + 1] = lsum;
+    }
+}
+
+// STEP: the row of cell pos comes from the caller's f32 K/V (stored under the f16 rule into the
+// pool on the way), as in decode_attn_kernel<..., STEP = true>.
+// SEL: the 16 rows of an iteration are four listed 4-cell blocks instead of a page, as in
+// decode_attn_kernel<..., SEL = true> (block g supplies the V rows of lane group g, block c / 4
+// the K row of lane c).
+template <bool STEP, bool SEL = false>
+__global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnKernelParams P) {
+    static_assert(!(STEP && SEL), "the fused step attends the dense selection");
+    __shared__ __attribute__((aligned(16))) MfmaFoldLds lds;
+
+    // ---- which (entry, kv head, page range); one work-group per unit (no head chunks) --------
+    const int unit = blockIdx.x;
+    int e = 0;
+    while (e + 1 < P.b.n && unit >= P.b.wg_base[e + 1]) ++e;
+    const int rem = unit - P.b.wg_base[e];
+    const int split = rem / P.n_kv;
+    const int kvh = rem - split * P.n_kv;
+    const int wg = unit;
+    const int pos = P.b.pos[e];
+    typedef const __attribute__((address_space(4))) int32_t* table_ptr;
+    typedef const __attribute__((address_space(4))) uint32_t* list_ptr;
+    const table_ptr bt = (table_ptr)(uintptr_t)(P.tables + (size_t)P.b.row[e] * (size_t)P.max_pages_per_seq);
+    uint32_t n_sel = 0;
+    list_ptr sel = nullptr;
+    if constexpr (SEL) {
+        n_sel = min(((list_ptr)(uintptr_t)P.counts)[e], (uint32_t)P.max_ids);
+        sel = (list_ptr)(uintptr_t)(P.ids + (size_t)e * (size_t)P.id_stride);
+    }
+    // loop iterations of this entry: pages, or groups of four selected blocks
+    const int n_pages = SEL ? (int)((n_sel + 3u) >> 2) : pos / kPage + 1;
+    const int pps = P.b.pps[e];
+    const int pg0 = split * pps;
+    const int pg1 = min(pg0 + pps, n_pages);
+
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int c = lane & 15;
+    const int g = lane >> 4;
+    const size_t page_bytes = (size_t)P.n_kv * kPage * kHd * 2;
+    const size_t head_off = (size_t)kvh * kPage * kHd * 2;
+
+    // Row runs of iteration i (see decode_attn_kernel): a page, or four listed blocks whose ids
+    // are clamped to the blocks at or below `pos` before any address is formed.
+    const auto locate = [&](int i, RowRuns<SEL>& rr) {
+        if constexpr (SEL) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t at = (uint32_t)i * 4u + (uint32_t)j;
+                const uint32_t id = sel[min(at, n_sel - 1u)];
+                rr.id[j] = at < n_sel ? id : 0xffffffffu;
+                const uint32_t idc = min(id, (uint32_t)pos >> 2);
+                const size_t off = (size_t)bt[idc >> 2] * page_bytes + head_off + (size_t)(idc & 3u) * 4u * (kHd * 2);
+                rr.k[j] = P.kpool + off;
+                rr.v[j] = P.vpool + off;
+            }
+        } else {
+            const size_t off = (size_t)bt[i] * page_bytes + head_off;
+            rr.k[0] = P.kpool + off;
+            rr.v[0] = P.vpool + off;
+            rr.id[0] = 0;
+        }
+    };
+    const auto pick = [](const auto (&a)[SEL ? 4 : 1], int j) {
+        if constexpr (SEL) return j == 0 ? a[0] : j == 1 ? a[1] : j == 2 ? a[2] : a[3]; else return a[0];
+    };
+    // this lane's K row (row c of the iteration) and the first of its four V rows (row 4 g)
+    const auto k_row = [&](const RowRuns<SEL>& rr) {
+        return SEL ? pick(rr.k, c >> 2) + (size_t)(c & 3) * (kHd * 2) : rr.k[0] + (size_t)c * (kHd * 2);
+    };
+    const auto v_rows = [&](const RowRuns<SEL>& rr) {
+        return SEL ? pick(rr.v, g) : rr.v[0] + (size_t)(4 * g) * (kHd * 2);
+    };
+    const auto k_addr = [&](const uint8_t* row, int m) {
+        return reinterpret_cast<const v4u*>(row + (size_t)(m * 32 + g * 8) * 2);
+    };
+    const auto v_addr = [&](const uint8_t* rows, int h, int r) {
+        return reinterpret_cast<const v4u*>(rows + (size_t)r * (kHd * 2) + (size_t)(h * 128 + c * 8) * 2);
+    };
+
+    int pg = pg0 + wave;
+    v4u kf[8], vf[2][4];
+    RowRuns<SEL> cur{};
+    if (pg < pg1) {
+        locate(pg, cur);
+        const uint8_t* kp = k_row(cur);
+        const uint8_t* vp = v_rows(cur);
+#pragma unroll
+        for (int m = 0; m < 8; ++m) kf[m] = __builtin_nontemporal_load(k_addr(kp, m));
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) vf[h][r] = __builtin_nontemporal_load(v_addr(vp, h, r));
+    }
+
+    // ---- q fragments of head c (heads past the group stay zero) ----------------------------------
+    half8 qhi[8], qlo[8];
+    {
+        const bool head_live = c < P.group;
+        const float* qp = P.q + ((size_t)e * P.n_q + (size_t)kvh * P.group + (head_live ? c : 0)) * kHd + g * 8;
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+            float x[8];
+            const float4 a = *reinterpret_cast<const float4*>(qp + m * 32);
+            const float4 b = *reinterpret_cast<const float4*>(qp + m * 32 + 4);
+            x[0] = a.x, x[1] = a.y, x[2] = a.z, x[3] = a.w;
+            x[4] = b.x, x[5] = b.y, x[6] = b.z, x[7] = b.w;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                _Float16 hi, lo;
+                split_hi_lo(head_live ? x[j] : 0.0f, hi, lo);
+                qhi[m][j] = hi;
+                qlo[m][j] = lo;
+            }
+        }
+    }
+
+    // O^T accumulators: o[h][t][r] = out[head c][128 h + 8 (4 g + r) + t]
+    f4 o[2][8];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int t = 0; t < 8; ++t) o[h][t] = f4{0.0f, 0.0f, 0.0f, 0.0f};
+    float m_run = -INFINITY;  // running max of head c (base-2 logits), equal in the 4 g lanes
+    float l_run = 0.0f;       // this lane's share (its 4 cells per page) of the denominator
+
+    while (pg < pg1) {
+        // the rows of this wave's next iteration, if it has one, are requested into the fragment
+        // registers as these are used up (the last iteration requests nothing)
+        const int pg_next = pg + kWaves;
+        const bool more = pg_next < pg1;
+        RowRuns<SEL> nxt{};
+        const uint8_t* kp_next = nullptr;
+        const uint8_t* vp_next = nullptr;
+        if (more) {
+            locate(pg_next, nxt);
+            kp_next = k_row(nxt);
+            vp_next = v_rows(nxt);
+        }
+
+        if constexpr (STEP) {
+            if (pg == n_pages - 1) {
+                // This wave holds the page of cell pos; its pool row is stale.  Every lane converts
+                // its slices of the new row; the lanes whose fragments are that row keep and store them.
+                const int r = pos & (kPage - 1);
+                const size_t here = (size_t)(cur.k[0] - P.kpool) + (size_t)r * (kHd * 2);
+                const float* nk = P.new_k + ((size_t)e * P.n_kv + (size_t)kvh) * kHd;
+                const float* nv = P.new_v + ((size_t)e * P.n_kv + (size_t)kvh) * kHd;
+                const auto row_slice = [](const float* src) {
+                    const float4 a = *reinterpret_cast<const float4*>(src);
+                    const float4 b = *reinterpret_cast<const float4*>(src + 4);
+                    v4u w;
+                    w.x = f16_store_pair(a.x, a.y), w.y = f16_store_pair(a.z, a.w);
+                    w.z = f16_store_pair(b.x, b.y), w.w = f16_store_pair(b.z, b.w);
+                    return w;
+                };
+#pragma unroll
+                for (int m = 0; m < 8; ++m) {
+                    const v4u w = row_slice(nk + m * 32 + g * 8);
+                    if (c == r) {
+                        kf[m] = w;
+                        *reinterpret_cast<v4u*>(P.kpool_w + here + (size_t)(m * 32 + g * 8) * 2) = w;
+                    }
+                }
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const v4u w = row_slice(nv + h * 128 + c * 8);
+                    if (g == (r >> 2)) {
+#pragma unroll
+                        for (int rr = 0; rr < 4; ++rr)
+                            if (rr == (r & 3)) vf[h][rr] = w;
+                        *reinterpret_cast<v4u*>(P.vpool_w + here + (size_t)(h * 128 + c * 8) * 2) = w;
+                    }
+                }
+            }
+        }
+
+        // ---- S^T = K . q^T: four independent accumulation chains ------------------------------
+        f4 s0 = f4{0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0, s2 = s0, s3 = s0;
+#pragma unroll
+        for (int m = 0; m < 8; m += 2) {
+            const half8 ka = __builtin_bit_cast(half8, kf[m]);
+            const half8 kb = __builtin_bit_cast(half8, kf[m + 1]);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qhi[m], s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qlo[m], s1, 0, 0, 0);
+            s2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kb, qhi[m + 1], s2, 0, 0, 0);
+            s3 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kb, qlo[m + 1], s3, 0, 0, 0);
+            if (more) {
+                kf[m] = __builtin_nontemporal_load(k_addr(kp_next, m));
+                kf[m + 1] = __builtin_nontemporal_load(k_addr(kp_next, m + 1));
+            }
+        }
+        const f4 s = (s0 + s1) + (s2 + s3);  // s[r] = q[head c] . k[cell 4 g + r]
+
+        // ---- online softmax of head c ---------------------------------------------------------------
+        float t4[4];
+        float pm = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            bool live;
+            if constexpr (SEL)
+                live = block_cell_live(pick(cur.id, g), r, pos);
+            else
+                live = pg * kPage + 4 * g + r <= pos;
+            t4[r] = live ? s[r] * P.scale_log2e : -INFINITY;
+            pm = fmaxf(pm, t4[r]);
+        }
+        pm = max_over_lane_groups(pm);
+        // dense: finite, every page of a range holds a live cell; a group of listed blocks may be
+        // dead as a whole, and exp2(-inf - -inf) would be NaN
+        const float m_new = fmaxf(m_run, pm);
+        const bool none_yet = SEL && m_new == -INFINITY;
+        const float alpha = none_yet ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
+        h4m phi, plo;
+        float psum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float p = none_yet ? 0.0f : __builtin_amdgcn_exp2f(t4[r] - m_new);
+            psum += p;
+            _Float16 hi, lo;
+            split_hi_lo(p, hi, lo);
+            phi[r] = hi;
+            plo[r] = lo;
+        }
+        const half8 phl = half8{phi[0], phi[1], phi[2], phi[3], plo[0], plo[1], plo[2], plo[3]};
+        l_run = l_run * alpha + psum;
+        if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int t = 0; t < 8; ++t) o[h][t] *= alpha;
+        }
+        m_run = m_new;
+
+        // Rows that are not attended may hold anything (even NaN): make them exact zeros.
+        if constexpr (SEL) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (!block_cell_live(pick(cur.id, g), r, pos)) {
+                    vf[0][r] = v4u{0u, 0u, 0u, 0u};
+                    vf[1][r] = v4u{0u, 0u, 0u, 0u};
+                }
+        } else if (pg == n_pages - 1) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (pg * kPage + 4 * g + r > pos) {
+                    vf[0][r] = v4u{0u, 0u, 0u, 0u};
+                    vf[1][r] = v4u{0u, 0u, 0u, 0u};
+                }
+        }
+
+        // ---- O^T += V^T . P^T ------------------------------------------------------------------------
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const half8 v0 = __builtin_bit_cast(half8, vf[h][0]), v1 = __builtin_bit_cast(half8, vf[h][1]);
+            const half8 v2 = __builtin_bit_cast(half8, vf[h][2]), v3 = __builtin_bit_cast(half8, vf[h][3]);
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                // the 32-deep MFMA runs over the page's 16 cells twice: against the high parts of p
+                // and against the low parts
+                const half8 vv = half8{v0[t], v1[t], v2[t], v3[t], v0[t], v1[t], v2[t], v3[t]};
+                o[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vv, phl, o[h][t], 0, 0, 0);
+            }
+            if (more) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) vf[h][r] = __builtin_nontemporal_load(v_addr(vp_next, h, r));
+            }
+        }
+        pg = pg_next;
+        cur = nxt;
+    }
+
+    mfma_fold_and_store(P, lds, wg, wave, c, g, o, m_run, l_run);
+}
+
+// ---- decode attention on the matrix cores, int8 rows with f16 block scales ---------------------
+// The I8H layout ([256 x i8][8 x f16 scale] per row) through the same MFMA decomposition as
+// decode_attn_mfma_kernel.  An int8 code is exactly representable in f16, so codes enter the
+// MFMAs as they are and the block scales are applied where a block's sum is complete:
+//   scores: one 32-deep MFMA pair per 32-value block m (the block is the contraction), then
+//           s[cell] += scale_k[cell][m] * partial[cell]           (4 FMAs per block and lane)
+//   P.V   : the dequantised value code * scale (7 + 11 significant bits) is split exactly into
+//           two f16 terms, hi = f16(code * scale) and lo = fma(code, scale, -hi) (the remainder
+//           has at most 7 significant bits and its lowest bit is 2^(e - 10) >= 2^-24 for a normal
+//           scale 2^e * f, so it is a representable f16 number, subnormal at worst); the three
+//           products (hi + lo).(p_hi + p_lo) then carry the result to f32 accuracy.  A lane's 8 columns lie in one block (4 h + c / 4), so it
+//           needs one scale per V row and half.
+// The VALU formulation of this layout is bound by instruction issue (conversions and FMAs, 40 %
+// of the HBM roofline on long contexts); here the VALU only converts and scales.
+typedef _Float16 h2m __attribute__((ext_vector_type(2)));
+
+// four int8 codes (one dword) -> four exact f16 values: 0x6400 | (code ^ 0x80) is 1024 + (code + 128)
+__device__ __forceinline__ void codes_to_f16(unsigned w, h2m& lo, h2m& hi) {
+    const unsigned u = w ^ 0x80808080u;
+    const h2m bias = h2m{(_Float16)1152.0f, (_Float16)1152.0f};
+    lo = __builtin_bit_cast(h2m, __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u)) - bias;
+    hi = __builtin_bit_cast(h2m, __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - bias;
+}
+// the same for codes that already carry the ^ 0x80 bias
+__device__ __forceinline__ void biased_to_f16(unsigned u, h2m& lo, h2m& hi) {
+    const h2m bias = h2m{(_Float16)1152.0f, (_Float16)1152.0f};
+    lo = __builtin_bit_cast(h2m, __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u)) - bias;
+    hi = __builtin_bit_cast(h2m, __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - bias;
+}
+// 4 x 4 byte transpose: t[j] = { w[0].byte j, w[1].byte j, w[2].byte j, w[3].byte j }
+__device__ __forceinline__ void transpose4x4_bytes(const unsigned (&w)[4], unsigned (&t)[4]) {
+    const unsigned a_lo = __builtin_amdgcn_perm(w[1], w[0], 0x05010400u);  // w0.0 w1.0 w0.1 w1.1
+    const unsigned a_hi = __builtin_amdgcn_perm(w[1], w[0], 0x07030602u);  // w0.2 w1.2 w0.3 w1.3
+    const unsigned b_lo = __builtin_amdgcn_perm(w[3], w[2], 0x05010400u);
+    const unsigned b_hi = __builtin_amdgcn_perm(w[3], w[2], 0x07030602u);
+    t[0] = __builtin_amdgcn_perm(b_lo, a_lo, 0x05040100u);
+    t[1] = __builtin_amdgcn_perm(b_lo, a_lo, 0x07060302u);
+    t[2] = __builtin_amdgcn_perm(b_hi, a_hi, 0x05040100u);
+    t[3] = __builtin_amdgcn_perm(b_hi, a_hi, 0x07060302u);
+}
+// whether either f16 of a dword has exponent field 0 (the values the cache reads as zero)
+__device__ __forceinline__ bool has_zero_exponent(unsigned two_halves) {
+    const unsigned t = two_halves & 0x7c007c00u;
+    return (t & 0xffffu) == 0 || (t >> 16) == 0;
+}
+__device__ __forceinline__ half8 codes8_to_f16(v2u w) {
+    h2m a, b, c2, d;
+    codes_to_f16(w.x, a, b);
+    codes_to_f16(w.y, c2, d);
+    return half8{a[0], a[1], b[0], b[1], c2[0], c2[1], d[0], d[1]};
+}
+// f16 scale under the cache's load rule (exponent field 0 reads as zero)
+__device__ __forceinline__ float scale_of(_Float16 h) {
+    const unsigned short bits = __builtin_bit_cast(unsigned short, h);
+    return (bits & 0x7c00u) == 0 ? 0.0f : (float)h;
+}
+
+// Data path: rows reach the matrix cores through LDS, not through registers.  Every wave owns two
+// slots of 2 x 4352 bytes (the K unit and the V unit of one page and kv head, scales included)
+// and fills them with 16-byte global->LDS loads, 64 lanes x 16 contiguous bytes per instruction
+// (whole cache lines, nothing fetched twice), two pages ahead of the page it computes: the K half
+// of a slot is refilled right after the scores that read it, the V half right after P.V.  A
+// wave has 20 such loads in flight in a fixed order (K, V of the next page, K, V of the one
+// after), so "the oldest five have landed" is s_waitcnt vmcnt(15) at both points of use.
+constexpr int kI8hUnit = kPage * row_bytes_of(kRowI8H);  // 4352
+constexpr int kI8hSlot = 2 * kI8hUnit;                    // K unit, then V unit
+
+// 4352 bytes = 4 x 1024 + 256: four full instructions and one of 16 lanes.  `real` false issues the
+// same five instructions on one 16-byte location (the data is never used): the number of loads
+// in flight, which the waits count, then does not depend on where in its range a wave is.
+__device__ __forceinline__ void i8h_unit_to_lds(const uint8_t* src, bool real, uint8_t* dst, int lane) {
+    typedef const __attribute__((address_space(1))) void* gptr;
+    typedef __attribute__((address_space(3))) void* lptr;
+    const uint8_t* lane_src = src + (real ? lane * 16 : 0);
+    const int step = real ? 1024 : 0;
+#pragma unroll
+    for (int n = 0; n < 4; ++n)
+        __builtin_amdgcn_global_load_lds((gptr)(lane_src + n * step), (lptr)(dst + n * 1024), 16, 0, 0);
+    if (lane < 16) __builtin_amdgcn_global_load_lds((gptr)(lane_src + 4 * step), (lptr)(dst + 4096), 16, 0, 0);
+}
+
+__global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const AttnKernelParams P) {
+    // slot 0 and slot 1 of the four waves; the fold staging of the epilogue reuses their memory
+    __shared__ __attribute__((aligned(16))) uint8_t ring[2 * kWaves * kI8hSlot];
+    static_assert(sizeof(MfmaFoldLds) <= sizeof(ring), "fold staging must fit the slots");
+    uint8_t* const ring0 = ring;
+    uint8_t* const ring1 = ring + kWaves * kI8hSlot;
+    constexpr int kRow = row_bytes_of(kRowI8H);  // 272
+
+    const int unit = blockIdx.x;
+    int e = 0;
+    while (e + 1 < P.b.n && unit >= P.b.wg_base[e + 1]) ++e;
+    const int rem = unit - P.b.wg_base[e];
+    const int split = rem / P.n_kv;
+    const int kvh = rem - split * P.n_kv;
+    const int wg = unit;
+    const int pos = P.b.pos[e];
+    const int n_pages = pos / kPage + 1;
+    const int pps = P.b.pps[e];
+    const int pg0 = split * pps;
+    const int pg1 = min(pg0 + pps, n_pages);
+    typedef const __attribute__((address_space(4))) int32_t* table_ptr;
+    const table_ptr bt = (table_ptr)(uintptr_t)(P.tables + (size_t)P.b.row[e] * (size_t)P.max_pages_per_seq);
+
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int c = lane & 15;
+    const int g = lane >> 4;
+    const int my_block = c >> 2;  // which of the 4 blocks of a half this lane's 8 columns lie in
+    const size_t page_bytes = (size_t)P.n_kv * kI8hUnit;
+    const size_t head_off = (size_t)kvh * kI8hUnit;
+    uint8_t* const slot0 = ring0 + wave * kI8hSlot;
+    uint8_t* const slot1 = ring1 + wave * kI8hSlot;
+
+    // unit of pipeline step i of this wave; steps past the wave's last are requested all the same,
+    // as loads of one location, so that the number of loads in flight stays what the waits assume
+    const int n_steps = pg0 + wave < pg1 ? (pg1 - pg0 - wave + kWaves - 1) / kWaves : 0;
+    const auto unit_off = [&](int i) -> size_t {
+        return (size_t)bt[min(pg0 + wave + kWaves * i, pg1 - 1)] * page_bytes + head_off;
+    };
+    i8h_unit_to_lds(P.kpool + unit_off(0), n_steps > 0, slot0, lane);
+    i8h_unit_to_lds(P.vpool + unit_off(0), n_steps > 0, slot0 + kI8hUnit, lane);
+    i8h_unit_to_lds(P.kpool + unit_off(1), n_steps > 1, slot1, lane);
+    i8h_unit_to_lds(P.vpool + unit_off(1), n_steps > 1, slot1 + kI8hUnit, lane);
+
+    // ---- q fragments of head c (heads past the group stay zero) ----------------------------------
+    half8 qhi[8], qlo[8];
+    {
+        const bool head_live = c < P.group;
+        const float* qp = P.q + ((size_t)e * P.n_q + (size_t)kvh * P.group + (head_live ? c : 0)) * kHd + g * 8;
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+            float x[8];
+            const float4 a = *reinterpret_cast<const float4*>(qp + m * 32);
+            const float4 b = *reinterpret_cast<const float4*>(qp + m * 32 + 4);
+            x[0] = a.x, x[1] = a.y, x[2] = a.z, x[3] = a.w;
+            x[4] = b.x, x[5] = b.y, x[6] = b.z, x[7] = b.w;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                _Float16 hi, lo;
+                split_hi_lo(head_live ? x[j] : 0.0f, hi, lo);
+                qhi[m][j] = hi;
+                qlo[m][j] = lo;
+            }
+        }
+    }
+
+    f4 o[2][8];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int t = 0; t < 8; ++t) o[h][t] = f4{0.0f, 0.0f, 0.0f, 0.0f};
+    float m_run = -INFINITY;
+    float l_run = 0.0f;
+
+    // One page: step i of the wave, resident in `slot`; the slot is refilled with step i + 2.
+    const auto one_page = [&](uint8_t* slot, int i) __attribute__((always_inline)) {
+        const int pg = pg0 + wave + kWaves * i;
+        const uint8_t* ks = slot;
+        const uint8_t* vs = slot + kI8hUnit;
+        const size_t off_next = unit_off(i + 2);
+
+        // ---- scores: per block, codes . q on the matrix core, then the block's scale ----------------
+        __builtin_amdgcn_s_waitcnt(0x0F7F);  // vmcnt(15): this page's K unit has landed
+        f4 s = f4{0.0f, 0.0f, 0.0f, 0.0f};
+        // all fragments of the unit are requested from LDS in one batch, ahead of the first use
+        half8 ksc[4];
+        v2u kc[8];
+#pragma unroll
+        for (int m = 0; m < 8; ++m) kc[m] = *reinterpret_cast<const v2u*>(ks + c * kRow + m * 32 + g * 8);
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            ksc[r] = __builtin_bit_cast(half8, *reinterpret_cast<const v4u*>(ks + (4 * g + r) * kRow + kHd));
+        const unsigned k_screen = *reinterpret_cast<const unsigned*>(ks + (lane >> 2) * kRow + kHd + 4 * (lane & 3));
+        __builtin_amdgcn_sched_barrier(0);
+        // A scale with exponent field 0 reads as zero.  The store rule never writes one, so the
+        // unit's 64 scale dwords are screened one per lane, and only a unit that holds such a scale
+        // (foreign data, rows never written) pays for the per-value rule.
+        if (__builtin_amdgcn_ballot_w64(has_zero_exponent(k_screen)) != 0) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int m = 0; m < 8; ++m)
+                    if ((__builtin_bit_cast(unsigned short, ksc[r][m]) & 0x7c00u) == 0) ksc[r][m] = (_Float16)0.0f;
+        }
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+            const half8 ka = codes8_to_f16(kc[m]);
+            f4 part = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qhi[m], f4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+            part = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qlo[m], part, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) s[r] = fmaf((float)ksc[r][m], part[r], s[r]);
+        }
+        i8h_unit_to_lds(P.kpool + off_next, i + 2 < n_steps, slot, lane);
+
+        // ---- online softmax of head c ---------------------------------------------------------------
+        float t4[4];
+        float pm = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const bool live = pg * kPage + 4 * g + r <= pos;
+            t4[r] = live ? s[r] * P.scale_log2e : -INFINITY;
+            pm = fmaxf(pm, t4[r]);
+        }
+        pm = max_over_lane_groups(pm);
+        const float m_new = fmaxf(m_run, pm);  // finite: every page of a range holds a live cell
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        float p[4];
+        float psum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            p[r] = __builtin_amdgcn_exp2f(t4[r] - m_new);
+            psum += p[r];
+        }
+        l_run = l_run * alpha + psum;
+        if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int t = 0; t < 8; ++t) o[h][t] *= alpha;
+        }
+        m_run = m_new;
+        h4m phi, plo;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            _Float16 hi, lo;
+            split_hi_lo(p[r], hi, lo);
+            phi[r] = hi;
+            plo[r] = lo;
+        }
+        const half8 phh = half8{phi[0], phi[1], phi[2], phi[3], phi[0], phi[1], phi[2], phi[3]};
+        const half8 pll = half8{plo[0], plo[1], plo[2], plo[3], plo[0], plo[1], plo[2], plo[3]};
+        // ---- P.V: dequantise into the exact (hi, lo) pair, two 32-deep MFMAs per 16 columns ---------------
+        __builtin_amdgcn_s_waitcnt(0x0F7F);  // vmcnt(15): this page's V unit has landed
+        // Scales of the lane's rows 4 g + r for its block of either half.  Rows past `pos` may hold
+        // anything: their probabilities are exact zeros already, and their scales are made zeros
+        // too, so that 0 * (garbage scale) cannot produce a NaN (any int8 code is a finite number).
+        unsigned vsb[2][4];
+        v2u vc[2][4];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                vc[h][r] = *reinterpret_cast<const v2u*>(vs + (4 * g + r) * kRow + h * 128 + c * 8);
+                vsb[h][r] = *reinterpret_cast<const unsigned short*>(vs + (4 * g + r) * kRow + kHd + 2 * (4 * h + my_block));
+            }
+        const unsigned v_screen = *reinterpret_cast<const unsigned*>(vs + (lane >> 2) * kRow + kHd + 4 * (lane & 3));
+        __builtin_amdgcn_sched_barrier(0);
+        const bool last_page = pg == n_pages - 1;
+        if (last_page || __builtin_amdgcn_ballot_w64(has_zero_exponent(v_screen)) != 0) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if ((vsb[h][r] & 0x7c00u) == 0 || pg * kPage + 4 * g + r > pos) vsb[h][r] = 0;
+        }
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const h2m s01 = __builtin_bit_cast(h2m, vsb[h][0] | (vsb[h][1] << 16));
+            const h2m s23 = __builtin_bit_cast(h2m, vsb[h][2] | (vsb[h][3] << 16));
+            // the lane's 4 rows x 8 codes, transposed as bytes so that a dword holds one column's
+            // four rows: converted, it is the A fragment of that column's MFMA
+            unsigned wx[4], wy[4], col[8];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                wx[r] = vc[h][r].x ^ 0x80808080u;
+                wy[r] = vc[h][r].y ^ 0x80808080u;
+            }
+            {
+                unsigned t0[4], t1[4];
+                transpose4x4_bytes(wx, t0);
+                transpose4x4_bytes(wy, t1);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) col[t] = t0[t], col[4 + t] = t1[t];
+            }
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                h2m c01, c23;
+                biased_to_f16(col[t], c01, c23);
+                const h2m hi01 = c01 * s01, hi23 = c23 * s23;
+                const h2m lo01 = __builtin_elementwise_fma(c01, s01, -hi01);
+                const h2m lo23 = __builtin_elementwise_fma(c23, s23, -hi23);
+                // (hi + lo) . p_hi and (hi + lo) . p_lo as two 32-deep MFMAs: the contraction runs
+                // over the 16 cells twice, a lane's eight slots being its four cells' hi parts and then
+                // their lo parts
+                const half8 ahl = half8{hi01[0], hi01[1], hi23[0], hi23[1], lo01[0], lo01[1], lo23[0], lo23[1]};
+                o[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahl, phh, o[h][t], 0, 0, 0);
+                o[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahl, pll, o[h][t], 0, 0, 0);
+            }
+        }
+        i8h_unit_to_lds(P.vpool + off_next, i + 2 < n_steps, slot + kI8hUnit, lane);
+    };
+
+    for (int i = 0; i < n_steps; ++i) one_page((i & 1) ? slot1 : slot0, i);
+
+    // no load may still be on its way into the slots when the fold staging takes their place
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0)
+    __syncthreads();
+    mfma_fold_and_store(P, *reinterpret_cast<MfmaFoldLds*>(ring), wg, wave, c, g, o, m_run, l_run);
+}
+
+// ---- decode attention on the matrix cores, f16 K and q8_0 V -----------------------------------
+// The MFMA decomposition of decode_attn_mfma_kernel with both operands staged through LDS like the
+// int8 kernel's units (every load of the loop is then a global->LDS load, which keeps the count of
+// loads in flight, and with it every wait, exact): the f16 K unit of the next page is requested
+// when the scores have used this page's, the V units ([f32 scale][32 x i8] blocks, 288 bytes a
+// row) two pages ahead.  A q8_0 value is code * scale with an f32 scale, so it takes a per-cell
+// power of two out first to stay inside f16:
+//   E[cell]  = exponent of the largest of the cell's 8 block scales (clamped to +-120),
+//   a[cell][d] = code * (scale * 2^-E[cell])       |a| < 256; split into hi + lo f16 as below,
+//   weight   = exp2(logit + E[cell] - M)            M the running maximum of logit + E,
+// so that weight * a is the term softmax-weight * value up to the common factor 2^-M, the largest
+// terms have weights near 1 whatever the magnitudes of their values, and what falls off the f16
+// range is small against the largest term.  The denominator sums exp2(logit - M) in f32.
+// scale' = scale * 2^-E is split into two f16 (s_hi + s_lo, 22 bits); code * s_hi is split exactly
+// into hi = f16(.) and its remainder (at most 7 significant bits, a representable f16 number),
+// and lo = remainder + code * s_lo; (hi + lo) . (w_hi + w_lo) on two 32-deep MFMAs as in the int8
+// kernel.
+constexpr int kQ8vRow = row_bytes_of(kRowQ8);  // 288
+constexpr int kQ8vUnit = kPage * kQ8vRow;      // 4608
+
+// K unit in LDS: 8 instructions of 1024 bytes (two rows each), 32 bytes apart so that the rows a
+// fragment read touches spread over the banks.
+constexpr int kQ8vKStep = 1024 + 32;
+constexpr int kQ8vKSlot = 8 * kQ8vKStep;  // 8448
+__device__ __forceinline__ void q8v_k_unit_to_lds(const uint8_t* src, bool real, uint8_t* dst, int lane) {
+    typedef const __attribute__((address_space(1))) void* gptr;
+    typedef __attribute__((address_space(3))) void* lptr;
+    const uint8_t* lane_src = src + (real ? lane * 16 : 0);
+    const int step = real ? 1024 : 0;
+#pragma unroll
+    for (int n = 0; n < 8; ++n)
+        __builtin_amdgcn_global_load_lds((gptr)(lane_src + n * step), (lptr)(dst + n * kQ8vKStep), 16, 0, 0);
+}
+
+// 4608 bytes = 4 x 1024 + 512: four full instructions and one of 32 lanes.  `real` false issues the
+// same five instructions on one 16-byte location (the data is never used): the number of loads
+// in flight, which the waits count, then does not depend on where in its range a wave is.
+__device__ __forceinline__ void q8v_unit_to_lds(const uint8_t* src, bool real, uint8_t* dst, int lane) {
+    typedef const __attribute__((address_space(1))) void* gptr;
+    typedef __attribute__((address_space(3))) void* lptr;
+    const uint8_t* lane_src = src + (real ? lane * 16 : 0);
+    const int step = real ? 1024 : 0;
+#pragma unroll
+    for (int n = 0; n < 4; ++n)
+        __builtin_amdgcn_global_load_lds((gptr)(lane_src + n * step), (lptr)(dst + n * 1024), 16, 0, 0);
+    if (lane < 32) __builtin_amdgcn_global_load_lds((gptr)(lane_src + 4 * step), (lptr)(dst + 4096), 16, 0, 0);
+}
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
+}
+
+__global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const AttnKernelParams P) {
+    // per wave one K slot and two V slots during the loop, the fold staging after it
+    constexpr int kWaveLds = kQ8vKSlot + 2 * kQ8vUnit;
+    constexpr int kLds = kWaves * kWaveLds > (int)sizeof(MfmaFoldLds) ? kWaves * kWaveLds : (int)sizeof(MfmaFoldLds);
+    __shared__ __attribute__((aligned(16))) uint8_t smem[kLds];
+
+    const int unit = blockIdx.x;
+    int e = 0;
+    while (e + 1 < P.b.n && unit >= P.b.wg_base[e + 1]) ++e;
+    const int rem = unit - P.b.wg_base[e];
+    const int split = rem / P.n_kv;
+    const int kvh = rem - split * P.n_kv;
+    const int wg = unit;
+    const int pos = P.b.pos[e];
+    const int n_pages = pos / kPage + 1;
+    const int pps = P.b.pps[e];
+    const int pg0 = split * pps;
+    const int pg1 = min(pg0 + pps, n_pages);
+    typedef const __attribute__((address_space(4))) int32_t* table_ptr;
+    const table_ptr bt = (table_ptr)(uintptr_t)(P.tables + (size_t)P.b.row[e] * (size_t)P.max_pages_per_seq);
+
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int c = lane & 15;
+    const int g = lane >> 4;
+    const size_t k_page_bytes = (size_t)P.n_kv * kPage * kHd * 2;
+    const size_t k_head_off = (size_t)kvh * kPage * kHd * 2;
+    const size_t v_page_bytes = (size_t)P.n_kv * kQ8vUnit;
+    const size_t v_head_off = (size_t)kvh * kQ8vUnit;
+    uint8_t* const kslot = smem + wave * kWaveLds;
+    uint8_t* const slots = kslot + kQ8vKSlot;
+
+    // pipeline steps of this wave: pages pg0 + wave, + kWaves, ...
+    const int n_steps = pg0 + wave < pg1 ? (pg1 - pg0 - wave + kWaves - 1) / kWaves : 0;
+    // physical page of step i; past the wave's last step the answer is not used for its data
+    const auto phys = [&](int i) -> size_t { return (size_t)bt[min(pg0 + wave + kWaves * i, pg1 - 1)]; };
+
+    // Loads complete in order.  Issue order per step: K(i+1) when the scores of step i are done,
+    // V(i+2) at its end; the prologue keeps that order (V0, K0, V1).  Behind K(i) at the top of step
+    // i there is V(i+1) = 5 loads; behind V(i) where step i needs it there are K(i), V(i+1), K(i+1)
+    // = 8 + 5 + 8.  Steps that do not exist are requested all the same, as loads of one location,
+    // so that these counts hold everywhere.
+    const auto k_unit = [&](int i) { return P.kpool + phys(i) * k_page_bytes + k_head_off; };
+    const auto v_unit = [&](int i) { return P.vpool + phys(i) * v_page_bytes + v_head_off; };
+    q8v_unit_to_lds(v_unit(0), n_steps > 0, slots, lane);
+    q8v_k_unit_to_lds(k_unit(0), n_steps > 0, kslot, lane);
+    q8v_unit_to_lds(v_unit(1), n_steps > 1, slots + kQ8vUnit, lane);
+
+    // ---- q fragments of head c (heads past the group stay zero) ----------------------------------
+    half8 qhi[8], qlo[8];
+    {
+        const bool head_live = c < P.group;
+        const float* qp = P.q + ((size_t)e * P.n_q + (size_t)kvh * P.group + (head_live ? c : 0)) * kHd + g * 8;
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+            float x[8];
+            const float4 a = *reinterpret_cast<const float4*>(qp + m * 32);
+            const float4 b = *reinterpret_cast<const float4*>(qp + m * 32 + 4);
+            x[0] = a.x, x[1] = a.y, x[2] = a.z, x[3] = a.w;
+            x[4] = b.x, x[5] = b.y, x[6] = b.z, x[7] = b.w;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                _Float16 hi, lo;
+                split_hi_lo(head_live ? x[j] : 0.0f, hi, lo);
+                qhi[m][j] = hi;
+                qlo[m][j] = lo;
+            }
+        }
+    }
+
+    f4 o[2][8];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int t = 0; t < 8; ++t) o[h][t] = f4{0.0f, 0.0f, 0.0f, 0.0f};
+    float m_run = -INFINITY;  // running maximum of logit + E (base 2)
+    float l_run = 0.0f;       // this lane's share of sum exp2(logit - m_run)
+    const int my_block = c >> 2;  // which of the 4 blocks of a half this lane's 8 columns lie in
+
+    for (int i = 0; i < n_steps; ++i) {
+        const int pg = pg0 + wave + kWaves * i;
+        const uint8_t* vs = slots + (i & 1) * kQ8vUnit;
+        const int behind = n_steps - 1 - i;  // steps after this one
+
+        // ---- S^T = K . q^T: four independent accumulation chains ------------------------------
+        __builtin_amdgcn_s_waitcnt(0x0F75);  // vmcnt(5): this page's K unit has landed
+        v4u kf[8];
+        {
+            // row c: two rows per 1056-byte step; fragment m of lane group g at 64 m + 16 g
+            const uint8_t* kr = kslot + (c >> 1) * kQ8vKStep + (c & 1) * 512 + g * 16;
+#pragma unroll
+            for (int m = 0; m < 8; ++m) kf[m] = *reinterpret_cast<const v4u*>(kr + m * 64);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        f4 s0 = f4{0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0, s2 = s0, s3 = s0;
+#pragma unroll
+        for (int m = 0; m < 8; m += 2) {
+            const half8 ka = __builtin_bit_cast(half8, kf[m]);
+            const half8 kb = __builtin_bit_cast(half8, kf[m + 1]);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qhi[m], s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qlo[m], s1, 0, 0, 0);
+            s2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kb, qhi[m + 1], s2, 0, 0, 0);
+            s3 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kb, qlo[m + 1], s3, 0, 0, 0);
+        }
+        const f4 s = (s0 + s1) + (s2 + s3);  // s[r] = q[head c] . k[cell 4 g + r]
+        q8v_k_unit_to_lds(k_unit(i + 1), behind >= 1, kslot, lane);
+
+        // ---- this page's V unit: scales first -------------------------------------------------
+        __builtin_amdgcn_s_waitcnt(0x4F75);  // vmcnt(21): K(i), V(i+1), K(i+1) behind V(i)
+        // lane (c, g): scale of blocks 2 (c / 4), + 1 of row 4 g + c % 4, the row's maximum over the
+        // lanes c, c ^ 4, c ^ 8, c ^ 12, then the four rows' maxima from the lanes of the quad
+        const bool last_page = pg == n_pages - 1;
+        float smax;
+        {
+            const uint8_t* rp = vs + (4 * g + (c & 3)) * kQ8vRow + (c >> 2) * 72;
+            const float a = *reinterpret_cast<const float*>(rp);
+            const float b = *reinterpret_cast<const float*>(rp + 36);
+            smax = fmaxf(a, b);
+            // rows past `pos` may hold anything: they count as scale 1 here and as zeros below
+            if (last_page && pg * kPage + 4 * g + (c & 3) > pos) smax = 1.0f;
+            smax = fmaxf(smax, dpp_mov<0x124>(smax));  // row_ror:4
+            smax = fmaxf(smax, dpp_mov<0x128>(smax));  // row_ror:8
+        }
+        int ex[4];
+        float down[4];  // 2^-E
+        {
+            const float m0 = dpp_mov<0x00>(smax), m1 = dpp_mov<0x55>(smax);
+            const float m2 = dpp_mov<0xAA>(smax), m3 = dpp_mov<0xFF>(smax);
+            const float mr[4] = {m0, m1, m2, m3};
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                int ee = (int)((__builtin_bit_cast(unsigned, mr[r]) >> 23) & 0xffu) - 127;
+                ee = min(max(ee, -120), 120);
+                ex[r] = ee;
+                down[r] = __builtin_bit_cast(float, (unsigned)(127 - ee) << 23);
+            }
+        }
+
+        // ---- online softmax of head c over logit + E ------------------------------------------------
+        float t4[4], tw[4];
+        float pm = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const bool live = pg * kPage + 4 * g + r <= pos;
+            t4[r] = live ? s[r] * P.scale_log2e : -INFINITY;
+            tw[r] = t4[r] + (float)ex[r];
+            pm = fmaxf(pm, tw[r]);
+        }
+        pm = max_over_lane_groups(pm);
+        const float m_new = fmaxf(m_run, pm);  // finite: every page of a range holds a live cell
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        h4m whi, wlo;
+        float psum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float w = __builtin_amdgcn_exp2f(tw[r] - m_new);
+            psum += __builtin_amdgcn_exp2f(t4[r] - m_new);
+            _Float16 hi, lo;
+            split_hi_lo(w, hi, lo);
+            whi[r] = hi;
+            wlo[r] = lo;
+        }
+        l_run = l_run * alpha + psum;
+        if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int t = 0; t < 8; ++t) o[h][t] *= alpha;
+        }
+        m_run = m_new;
+        const half8 whh = half8{whi[0], whi[1], whi[2], whi[3], whi[0], whi[1], whi[2], whi[3]};
+        const half8 wll = half8{wlo[0], wlo[1], wlo[2], wlo[3], wlo[0], wlo[1], wlo[2], wlo[3]};
+
+        // ---- P.V ----------------------------------------------------------------------------------
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            unsigned wx[4], wy[4], col[8];
+            _Float16 shi[4], slo[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const uint8_t* blk = vs + (4 * g + r) * kQ8vRow + (4 * h + my_block) * 36;
+                float sc = *reinterpret_cast<const float*>(blk) * down[r];
+                if (last_page && pg * kPage + 4 * g + r > pos) sc = 0.0f;
+                split_hi_lo(sc, shi[r], slo[r]);
+                const unsigned* cw = reinterpret_cast<const unsigned*>(blk + 4 + (c & 3) * 8);
+                wx[r] = cw[0] ^ 0x80808080u;
+                wy[r] = cw[1] ^ 0x80808080u;
+            }
+            const h2m s01 = h2m{shi[0], shi[1]}, s23 = h2m{shi[2], shi[3]};
+            const h2m l01 = h2m{slo[0], slo[1]}, l23 = h2m{slo[2], slo[3]};
+            {
+                unsigned t0[4], t1[4];
+                transpose4x4_bytes(wx, t0);
+                transpose4x4_bytes(wy, t1);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) col[t] = t0[t], col[4 + t] = t1[t];
+            }
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                h2m c01, c23;
+                biased_to_f16(col[t], c01, c23);
+                const h2m hi01 = c01 * s01, hi23 = c23 * s23;
+                const h2m lo01 = __builtin_elementwise_fma(c01, l01, __builtin_elementwise_fma(c01, s01, -hi01));
+                const h2m lo23 = __builtin_elementwise_fma(c23, l23, __builtin_elementwise_fma(c23, s23, -hi23));
+                const half8 ahl = half8{hi01[0], hi01[1], hi23[0], hi23[1], lo01[0], lo01[1], lo23[0], lo23[1]};
+                o[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahl, whh, o[h][t], 0, 0, 0);
+                o[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahl, wll, o[h][t], 0, 0, 0);
+            }
+        }
+        q8v_unit_to_lds(v_unit(i + 2), behind >= 2, slots + (i & 1) * kQ8vUnit, lane);
+    }
+
+    // no load may still be on its way into the slots when the fold staging takes their place
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0)
+    __syncthreads();
+    mfma_fold_and_store(P, *reinterpret_cast<MfmaFoldLds*>(smem), wg, wave, c, g, o, m_run, l_run);
+}
+
+}  // namespace
+
+hipError_t launch_decode_attn_mfma(const AttnKernelParams& kp, int layout, bool step, bool sel, int32_t total,
+                                   hipStream_t stream) {
+    if (layout == BKV_LAYOUT_I8H)
+        decode_attn_mfma_i8h_kernel<<<total, kBlock, 0, stream>>>(kp);
+    else if (layout == BKV_LAYOUT_Q8V)
+        decode_attn_mfma_q8v_kernel<<<total, kBlock, 0, stream>>>(kp);
+    else if (step)
+        decode_attn_mfma_kernel<true><<<total, kBlock, 0, stream>>>(kp);
+    else if (sel)
+        decode_attn_mfma_kernel<false, true><<<total, kBlock, 0, stream>>>(kp);
+    else
+        decode_attn_mfma_kernel<false><<<total, kBlock, 0, stream>>>(kp);
+    return hipGetLastError();
+}
+
+}  // namespace bkv
