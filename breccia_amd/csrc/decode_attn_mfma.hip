@@ -30,6 +30,29 @@ __device__ __forceinline__ void split_hi_lo(float x, _Float16& hi, _Float16& lo)
     lo = (_Float16)(x - (float)hi);
 }
 
+// q fragments of head c of the kv head (heads past the group stay zero): lane (c, g) holds
+// q[head][32 m + 8 g + 0..7], m = 0..7, as a high and a low f16 part
+__device__ __forceinline__ void load_q_fragments(const AttnKernelParams& P, int e, int kvh, int c, int g,
+                                                 half8 (&qhi)[8], half8 (&qlo)[8]) {
+    const bool head_live = c < P.group;
+    const float* qp = P.q + ((size_t)e * P.n_q + (size_t)kvh * P.group + (head_live ? c : 0)) * kHd + g * 8;
+#pragma unroll
+    for (int m = 0; m < 8; ++m) {
+        float x[8];
+        const float4 a = *reinterpret_cast<const float4*>(qp + m * 32);
+        const float4 b = *reinterpret_cast<const float4*>(qp + m * 32 + 4);
+        x[0] = a.x, x[1] = a.y, x[2] = a.z, x[3] = a.w;
+        x[4] = b.x, x[5] = b.y, x[6] = b.z, x[7] = b.w;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            _Float16 hi, lo;
+            split_hi_lo(head_live ? x[j] : 0.0f, hi, lo);
+            qhi[m][j] = hi;
+            qlo[m][j] = lo;
+        }
+    }
+}
+
 constexpr int kOwStride = kHd + 4;  // floats per head in the wave-merge staging
 
 // Shared tail of the MFMA decode kernels: wave totals, then every wave stages its scaled O in
@@ -189,27 +212,8 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
             for (int r = 0; r < 4; ++r) vf[h][r] = __builtin_nontemporal_load(v_addr(vp, h, r));
     }
 
-    // ---- q fragments of head c (heads past the group stay zero) ----------------------------------
     half8 qhi[8], qlo[8];
-    {
-        const bool head_live = c < P.group;
-        const float* qp = P.q + ((size_t)e * P.n_q + (size_t)kvh * P.group + (head_live ? c : 0)) * kHd + g * 8;
-#pragma unroll
-        for (int m = 0; m < 8; ++m) {
-            float x[8];
-            const float4 a = *reinterpret_cast<const float4*>(qp + m * 32);
-            const float4 b = *reinterpret_cast<const float4*>(qp + m * 32 + 4);
-            x[0] = a.x, x[1] = a.y, x[2] = a.z, x[3] = a.w;
-            x[4] = b.x, x[5] = b.y, x[6] = b.z, x[7] = b.w;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                _Float16 hi, lo;
-                split_hi_lo(head_live ? x[j] : 0.0f, hi, lo);
-                qhi[m][j] = hi;
-                qlo[m][j] = lo;
-            }
-        }
-    }
+    load_q_fragments(P, e, kvh, c, g, qhi, qlo);
 
     // O^T accumulators: o[h][t][r] = out[head c][128 h + 8 (4 g + r) + t]
     f4 o[2][8];
@@ -494,27 +498,8 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
     i8h_unit_to_lds(P.kpool + unit_off(1), n_steps > 1, slot1, lane);
     i8h_unit_to_lds(P.vpool + unit_off(1), n_steps > 1, slot1 + kI8hUnit, lane);
 
-    // ---- q fragments of head c (heads past the group stay zero) ----------------------------------
     half8 qhi[8], qlo[8];
-    {
-        const bool head_live = c < P.group;
-        const float* qp = P.q + ((size_t)e * P.n_q + (size_t)kvh * P.group + (head_live ? c : 0)) * kHd + g * 8;
-#pragma unroll
-        for (int m = 0; m < 8; ++m) {
-            float x[8];
-            const float4 a = *reinterpret_cast<const float4*>(qp + m * 32);
-            const float4 b = *reinterpret_cast<const float4*>(qp + m * 32 + 4);
-            x[0] = a.x, x[1] = a.y, x[2] = a.z, x[3] = a.w;
-            x[4] = b.x, x[5] = b.y, x[6] = b.z, x[7] = b.w;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                _Float16 hi, lo;
-                split_hi_lo(head_live ? x[j] : 0.0f, hi, lo);
-                qhi[m][j] = hi;
-                qlo[m][j] = lo;
-            }
-        }
-    }
+    load_q_fragments(P, e, kvh, c, g, qhi, qlo);
 
     f4 o[2][8];
 #pragma unroll
@@ -771,27 +756,8 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
     q8v_k_unit_to_lds(k_unit(0), n_steps > 0, kslot, lane);
     q8v_unit_to_lds(v_unit(1), n_steps > 1, slots + kQ8vUnit, lane);
 
-    // ---- q fragments of head c (heads past the group stay zero) ----------------------------------
     half8 qhi[8], qlo[8];
-    {
-        const bool head_live = c < P.group;
-        const float* qp = P.q + ((size_t)e * P.n_q + (size_t)kvh * P.group + (head_live ? c : 0)) * kHd + g * 8;
-#pragma unroll
-        for (int m = 0; m < 8; ++m) {
-            float x[8];
-            const float4 a = *reinterpret_cast<const float4*>(qp + m * 32);
-            const float4 b = *reinterpret_cast<const float4*>(qp + m * 32 + 4);
-            x[0] = a.x, x[1] = a.y, x[2] = a.z, x[3] = a.w;
-            x[4] = b.x, x[5] = b.y, x[6] = b.z, x[7] = b.w;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                _Float16 hi, lo;
-                split_hi_lo(head_live ? x[j] : 0.0f, hi, lo);
-                qhi[m][j] = hi;
-                qlo[m][j] = lo;
-            }
-        }
-    }
+    load_q_fragments(P, e, kvh, c, g, qhi, qlo);
 
     f4 o[2][8];
 #pragma unroll
