@@ -227,8 +227,11 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
         }
         const h8 phl = h8{phi[0], phi[1], phi[2], phi[3], plo[0], plo[1], plo[2], plo[3]};
         l_run = l_run * alpha + psum;
+        // rescale only on pages where some query's maximum moved (the test is on the maxima, not on
+        // alpha != 1: with the latter the compiler multiplies unconditionally, 64 instructions a page)
+        const bool moved = m_new > m_run;
         m_run = m_new;
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+        if (__builtin_amdgcn_ballot_w64(moved) != 0) {
 #pragma unroll
             for (int h = 0; h < 2; ++h)
 #pragma unroll
