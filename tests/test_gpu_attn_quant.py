@@ -8,6 +8,7 @@ import pytest
 
 import oracle
 from breccia_amd import lib as L
+from breccia_amd.kv import BkvError, DeviceBuffer
 from gpu_common import REF_BAR_MAX_REL, Twin, check_attn
 from helpers import max_abs, max_rel
 from test_gpu_attn import fill, score_spread_case
@@ -104,6 +105,38 @@ def test_quantised_values_across_the_scale_range(layout, v_mag):
 @pytest.mark.parametrize("loud_rows", [(4, 16), (9, 10)])
 def test_quantised_score_spread_across_the_rows_of_a_page(layout, loud_rows):
     score_spread_case(loud_rows, layout)
+
+
+@pytest.mark.parametrize("layout", [L.LAYOUT_F16, L.LAYOUT_Q8V, L.LAYOUT_I8H])
+def test_largest_batch_of_entries_and_the_empty_call(layout):
+    # 64 entries (the limit of one call): 16 sequences, 4 positions each (T = 4 decode), lengths
+    # from 1 cell to several pages; then 65 entries and 0 entries
+    rng = np.random.Generator(np.random.PCG64(98 + layout))
+    lens = [1, 2, 15, 16, 17, 31, 33, 64, 65, 100, 129, 200, 255, 256, 257, 300]
+    with Twin(n_pages=200, max_seqs=20, layout=layout) as tw:
+        tw.pool.set_free_order(rng.permutation(200).astype(np.int32))
+        seqs = [tw.pool.seq_create() for _ in lens]
+        for s, n in zip(seqs, lens):
+            fill(tw, s, n, rng, chunk=128)
+        ent_seq, pos = [], []
+        for s, n in zip(seqs, lens):
+            for back in range(4):
+                ent_seq.append(s)
+                pos.append(max(n - 1 - back, 0))
+        assert len(ent_seq) == L.MAX_BATCH
+        q = rng.standard_normal((64, 16, 256)).astype(np.float32)
+        out = tw.decode_attn(0, ent_seq, pos, q, 16)
+        for i in range(64):
+            want = tw.oracle_attend(0, ent_seq[i], pos[i], q[i], 16)
+            _, rel = check_attn(out[i], want, "layout %d entry %d" % (layout, i))
+            assert rel <= REF_BAR_MAX_REL, (i, rel)
+        with pytest.raises(BkvError) as ei:
+            tw.decode_attn(0, ent_seq + [seqs[0]], pos + [0], np.concatenate([q, q[:1]]), 16)
+        assert ei.value.status == L.ERR_INVALID
+        # an empty call is a no-op that succeeds
+        z = DeviceBuffer(64)
+        tw.pool.decode_attn(0, [], [], 16, z, z, 0.0625)
+        z.free()
 
 
 @pytest.mark.parametrize("layout", [L.LAYOUT_Q8V, L.LAYOUT_I8H])
