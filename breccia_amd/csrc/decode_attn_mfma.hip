@@ -549,6 +549,23 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
         }
         i8h_unit_to_lds(P.kpool + off_next, i + 2 < n_steps, slot, lane);
 
+        // ---- this page's V fragments are requested before the softmax, whose chain of dependent
+        // instructions then has the dequantisation to overlap with -----------------------------------
+        __builtin_amdgcn_s_waitcnt(0x0F7F);  // vmcnt(15): this page's V unit has landed
+        // Scales of the lane's rows 4 g + r for its block of either half.  Rows past `pos` may hold
+        // anything: their probabilities are exact zeros already, and their scales are made zeros
+        // too, so that 0 * (garbage scale) cannot produce a NaN (any int8 code is a finite number).
+        unsigned vsb[2][4];
+        v2u vc[2][4];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                vc[h][r] = *reinterpret_cast<const v2u*>(vs + (4 * g + r) * kRow + h * 128 + c * 8);
+                vsb[h][r] = *reinterpret_cast<const unsigned short*>(vs + (4 * g + r) * kRow + kHd + 2 * (4 * h + my_block));
+            }
+        const unsigned v_screen = *reinterpret_cast<const unsigned*>(vs + (lane >> 2) * kRow + kHd + 4 * (lane & 3));
+
         // ---- online softmax of head c ---------------------------------------------------------------
         float t4[4];
         float pm = -INFINITY;
@@ -587,21 +604,6 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
         const half8 phh = half8{phi[0], phi[1], phi[2], phi[3], phi[0], phi[1], phi[2], phi[3]};
         const half8 pll = half8{plo[0], plo[1], plo[2], plo[3], plo[0], plo[1], plo[2], plo[3]};
         // ---- P.V: dequantise into the exact (hi, lo) pair, two 32-deep MFMAs per 16 columns ---------------
-        __builtin_amdgcn_s_waitcnt(0x0F7F);  // vmcnt(15): this page's V unit has landed
-        // Scales of the lane's rows 4 g + r for its block of either half.  Rows past `pos` may hold
-        // anything: their probabilities are exact zeros already, and their scales are made zeros
-        // too, so that 0 * (garbage scale) cannot produce a NaN (any int8 code is a finite number).
-        unsigned vsb[2][4];
-        v2u vc[2][4];
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                vc[h][r] = *reinterpret_cast<const v2u*>(vs + (4 * g + r) * kRow + h * 128 + c * 8);
-                vsb[h][r] = *reinterpret_cast<const unsigned short*>(vs + (4 * g + r) * kRow + kHd + 2 * (4 * h + my_block));
-            }
-        const unsigned v_screen = *reinterpret_cast<const unsigned*>(vs + (lane >> 2) * kRow + kHd + 4 * (lane & 3));
-        __builtin_amdgcn_sched_barrier(0);
         const bool last_page = pg == n_pages - 1;
         if (last_page || __builtin_amdgcn_ballot_w64(has_zero_exponent(v_screen)) != 0) {
 #pragma unroll
