@@ -601,7 +601,7 @@ struct MergeParams {
 };
 
 constexpr int kMergeGroups = 4;   // split ranges summed side by side, then folded in LDS
-constexpr int kMergeInFlight = 16; // partial rows a thread requests before it needs the factors
+constexpr int kMergeInFlight = 20; // partial rows a thread requests before it needs the factors
 
 // One work-group per (entry, q head): kMergeGroups x 256 threads.  Thread (g, d) owns head-dim
 // element d of splits g, g + 4, ...; it requests its first 8 partial values straight away, and
