@@ -600,20 +600,21 @@ struct MergeParams {
     int32_t n_kv, n_q, group, hg;
 };
 
-constexpr int kMergeGroups = 4;   // split ranges summed side by side, then folded in LDS
-constexpr int kMergeInFlight = 20; // partial rows a thread requests before it needs the factors
+constexpr int kMergeGroups = 16;   // waves of a work-group; wave g sums splits g, g + 16, ...
+constexpr int kMergeInFlight = 8;  // partial rows (16 bytes a lane) a wave requests per round
 
-// One work-group per (entry, q head): kMergeGroups x 256 threads.  Thread (g, d) owns head-dim
-// element d of splits g, g + 4, ...; it requests its first 8 partial values straight away, and
-// only then are the per-split (m, l) pairs staged in LDS and the maximum agreed, so the two
-// round trips to memory overlap.
-__global__ __launch_bounds__(kHd * kMergeGroups) void decode_attn_merge_kernel(const MergeParams P) {
+// One work-group per (entry, q head): 16 waves.  Lane d4 of wave g owns head-dim elements
+// 4 d4 .. 4 d4 + 3 of splits g, g + 16, ...; it requests its first 8 partial rows straight away,
+// and only then are the per-split (m, l) pairs staged in LDS and the maximum agreed, so the two
+// round trips to memory overlap.  One round covers 128 splits.
+__global__ __launch_bounds__(64 * kMergeGroups) void decode_attn_merge_kernel(const MergeParams P) {
     constexpr int kMaxStaged = 1024;
+    constexpr int kThreads = 64 * kMergeGroups;
     __shared__ float sm[kMaxStaged];
     __shared__ float sl[kMaxStaged];
-    __shared__ float red[kMergeGroups][kHd];
+    __shared__ __attribute__((aligned(16))) float red[kMergeGroups][kHd];
     __shared__ float red_l[kMergeGroups];
-    __shared__ float wave_max[kHd * kMergeGroups / 64];
+    __shared__ float wave_max[kMergeGroups];
     const int e = blockIdx.x / P.n_q;
     const int h = blockIdx.x % P.n_q;
     const int kvh = h / P.group;
@@ -622,23 +623,22 @@ __global__ __launch_bounds__(kHd * kMergeGroups) void decode_attn_merge_kernel(c
     const int hh = hl % P.hg;
     const int splits = P.b.splits[e];
     const int wg0 = P.b.wg_base[e] + hc * splits * P.n_kv + kvh;
-    const int d = threadIdx.x & (kHd - 1);
-    const int g = threadIdx.x >> 8;
+    const int d4 = threadIdx.x & 63;
+    const int g = threadIdx.x >> 6;
     const size_t ostride = (size_t)P.n_kv * P.hg * kHd;  // floats between consecutive splits
-    const float* po = P.part_o + ((size_t)wg0 * P.hg + hh) * kHd + d;
+    const float* po = P.part_o + ((size_t)wg0 * P.hg + hh) * kHd + 4 * d4;
     const float* pml = P.part_ml + ((size_t)wg0 * P.hg + hh) * 2;
     const size_t mlstride = (size_t)P.n_kv * P.hg * 2;
 
-    float v[kMergeInFlight];
+    f4 v[kMergeInFlight];
 #pragma unroll
     for (int u = 0; u < kMergeInFlight; ++u) {
         const int s = g + u * kMergeGroups;
-        v[u] = s < splits ? po[(size_t)s * ostride] : 0.0f;
+        v[u] = s < splits ? *reinterpret_cast<const f4*>(po + (size_t)s * ostride) : f4{0.0f, 0.0f, 0.0f, 0.0f};
     }
     // stage (m, l) and agree on the maximum: per-thread max over its splits, wave reduction,
     // then one LDS slot per wave (a serial scan over the splits would cost a dependent LDS
     // round trip per split)
-    constexpr int kThreads = kHd * kMergeGroups;
     float my_m = -INFINITY;
     for (int s = threadIdx.x; s < splits; s += kThreads) {
         const float ms = pml[(size_t)s * mlstride];
@@ -650,31 +650,31 @@ __global__ __launch_bounds__(kHd * kMergeGroups) void decode_attn_merge_kernel(c
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) my_m = fmaxf(my_m, __shfl_xor(my_m, off, 64));
-    if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = my_m;
+    if ((threadIdx.x & 63) == 0) wave_max[g] = my_m;
     __syncthreads();
     const auto m_of = [&](int s) { return s < kMaxStaged ? sm[s] : pml[(size_t)s * mlstride]; };
     const auto l_of = [&](int s) { return s < kMaxStaged ? sl[s] : pml[(size_t)s * mlstride + 1]; };
     float mx = wave_max[0];
 #pragma unroll
-    for (int w = 1; w < kThreads / 64; ++w) mx = fmaxf(mx, wave_max[w]);
-    float acc = 0.0f, lsum = 0.0f;
+    for (int w = 1; w < kMergeGroups; ++w) mx = fmaxf(mx, wave_max[w]);
+    f4 acc = f4{0.0f, 0.0f, 0.0f, 0.0f};
+    float lsum = 0.0f;
 #pragma unroll
     for (int u = 0; u < kMergeInFlight; ++u) {
         const int s = g + u * kMergeGroups;
         if (s < splits) {
             const float ms = m_of(s);
             const float f = ms == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(ms - mx);
-            acc = fmaf(f, v[u], acc);
+            acc += v[u] * f;
             lsum = fmaf(f, l_of(s), lsum);
         }
     }
-    // further rounds of kMergeInFlight requests for long split lists
-    for (int s0 = g + kMergeInFlight * kMergeGroups; s0 < splits;
-         s0 += kMergeInFlight * kMergeGroups) {
+    // further rounds for split lists beyond 128
+    for (int s0 = g + kMergeInFlight * kMergeGroups; s0 < splits; s0 += kMergeInFlight * kMergeGroups) {
 #pragma unroll
         for (int u = 0; u < kMergeInFlight; ++u) {
             const int s = s0 + u * kMergeGroups;
-            v[u] = s < splits ? po[(size_t)s * ostride] : 0.0f;
+            v[u] = s < splits ? *reinterpret_cast<const f4*>(po + (size_t)s * ostride) : f4{0.0f, 0.0f, 0.0f, 0.0f};
         }
 #pragma unroll
         for (int u = 0; u < kMergeInFlight; ++u) {
@@ -682,21 +682,24 @@ __global__ __launch_bounds__(kHd * kMergeGroups) void decode_attn_merge_kernel(c
             if (s < splits) {
                 const float ms = m_of(s);
                 const float f = ms == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(ms - mx);
-                acc = fmaf(f, v[u], acc);
+                acc += v[u] * f;
                 lsum = fmaf(f, l_of(s), lsum);
             }
         }
     }
-    red[g][d] = acc;
-    if (d == 0) red_l[g] = lsum;
+    *reinterpret_cast<f4*>(&red[g][4 * d4]) = acc;
+    if (d4 == 0) red_l[g] = lsum;
     __syncthreads();
-    if (g != 0) return;
+    // the first four waves fold the 16 rows: thread d sums element d
+    if (threadIdx.x >= kHd) return;
+    const int d = threadIdx.x;
+    float r = 0.0f, lt = 0.0f;
 #pragma unroll
-    for (int k = 1; k < kMergeGroups; ++k) {
-        acc += red[k][d];
-        lsum += red_l[k];
+    for (int k = 0; k < kMergeGroups; ++k) {
+        r += red[k][d];
+        lt += red_l[k];
     }
-    float r = lsum > 0.0f ? acc / lsum : 0.0f;
+    r = lt > 0.0f ? r / lt : 0.0f;
     if (P.gate) {
         const float gt = P.gate[(size_t)e * P.gate_seq_stride + (size_t)h * P.gate_head_stride + d];
         // sigmoid in the overflow-free form of the reference (qsa/cpu.rs:84-91)
@@ -841,7 +844,7 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
     mp.hg = hg;
     {
         StageScope timed(p, BKV_STAGE_ATTN_MERGE, stream);
-        decode_attn_merge_kernel<<<b.n * a.n_q_head, kHd * kMergeGroups, 0, stream>>>(mp);
+        decode_attn_merge_kernel<<<b.n * a.n_q_head, 64 * kMergeGroups, 0, stream>>>(mp);
     }
     return hipGetLastError();
 }
