@@ -341,10 +341,10 @@ def bench_quantised(stream) -> dict:
 
     res = {}
     cases = [("attn_q8v_batch8", L.LAYOUT_Q8V, ROW_BYTES_Q8V, 8, 1024, 32768, 4, 20250003,
-              "headline batch on f16 K + q8_0 V", "decode_attn_mfma_q8v_kernel"),
+              "headline batch on f16 K + q8_0 V", "decode_attn_mfma_q8v_kernel<true>"),
              ("attn_int8_batch16", L.LAYOUT_I8H, ROW_BYTES_I8H, 16, 8192, 131072, 2, 20250005,
               "BASELINE configs[4]: 16 sequences, ctx U{8k..128k}, int8 K/V + f16 scales",
-              "decode_attn_mfma_i8h_kernel")]
+              "decode_attn_mfma_i8h_kernel<true>")]
     for name, layout, row_bytes, n_seqs, lo, hi, n_layers, seed, what, kernel in cases:
         rng = np.random.Generator(np.random.PCG64(seed))
         pool, seqs, ctx = build_batched(None, rng, n_seqs, lo, hi, n_layers, 0.6, layout)
@@ -361,10 +361,10 @@ def bench_quantised(stream) -> dict:
         vd.free()
         _, bufs = make_step_buffers(n_seqs, rng, slots=16)
         steps, warm = 40, 8
-        wall_ms, _ = time_steps(pool, seqs, ctx, n_layers, steps, warm, bufs, stream, fused=False)
+        wall_ms, _ = time_steps(pool, seqs, ctx, n_layers, steps, warm, bufs, stream, fused=True)
         pool.timing_reset()
         pool.timing_enable(True)
-        run_steps(pool, seqs, ctx, n_layers, steps, *bufs, stream, first_step=steps + warm, fused=False)
+        run_steps(pool, seqs, ctx, n_layers, steps, *bufs, stream, first_step=steps + warm, fused=True)
         stream.sync()
         pool.timing_enable(False)
         n_split, ms_split = pool.timing_read(L.STAGE_ATTN_SPLIT)

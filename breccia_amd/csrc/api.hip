@@ -680,9 +680,6 @@ static bkv_status decode_attn_common(bkv_pool* p, int32_t layer, int32_t n, cons
                                      const float* new_k_dev = nullptr, const float* new_v_dev = nullptr,
                                      bool step = false) {
     if (!p) return fail(BKV_ERR_INVALID, "decode_attn: NULL pool");
-    if (step && p->g.layout != BKV_LAYOUT_F16)
-        return fail(BKV_ERR_INVALID, "decode_step is built for f16 pools; append and attend in two "
-                                     "calls on a quantised pool");
     if (layer < 0 || layer >= p->g.n_layers)
         return fail(BKV_ERR_RANGE, sfmt("decode_attn: layer %lld is outside 0..%lld", layer,
                                         p->g.n_layers));
@@ -741,9 +738,13 @@ static bkv_status decode_attn_common(bkv_pool* p, int32_t layer, int32_t n, cons
     if (select && (!ids_dev || !counts_dev || ((uintptr_t)ids_dev & 3u) || ((uintptr_t)counts_dev & 3u)))
         return fail(BKV_ERR_INVALID, "decode_attn_select: ids/counts device pointers must be "
                                      "non-NULL and 4-byte aligned");
+    const bool mfma = attn_on_mfma(p, n_q_head / p->g.n_kv, !select);
+    if (step && !mfma && p->g.layout != BKV_LAYOUT_F16)
+        return fail(BKV_ERR_INVALID, "decode_step on a quantised pool is served by the matrix-core kernels "
+                                     "only (at most 16 q heads per kv head, pool without "
+                                     "BKV_POOL_ATTN_VALU); append and attend in two calls instead");
     st = flush_tables(p, S(stream));
     if (st != BKV_OK) return st;
-    const bool mfma = attn_on_mfma(p, n_q_head / p->g.n_kv, !select && !step);
     plan_attn(p, n_q_head, b, select ? (max_ids + 3) / 4 : 0, mfma);
     AttnArgs a;
     a.mfma = mfma;

@@ -5,6 +5,7 @@
 #include "decode_attn_common.hpp"
 #include "f16_rule.hpp"
 #include "lane_groups.hpp"
+#include "quant_encode.hpp"
 
 namespace bkv {
 
@@ -454,6 +455,7 @@ __device__ __forceinline__ void i8h_unit_to_lds(const uint8_t* src, bool real, u
     if (lane < 16) __builtin_amdgcn_global_load_lds((gptr)(lane_src + 4 * step), (lptr)(dst + 4096), 16, 0, 0);
 }
 
+template <bool STEP>
 __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const AttnKernelParams P) {
     // slot 0 and slot 1 of the four waves; the fold staging of the epilogue reuses their memory
     __shared__ __attribute__((aligned(16))) uint8_t ring[2 * kWaves * kI8hSlot];
@@ -509,6 +511,36 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
     float m_run = -INFINITY;
     float l_run = 0.0f;
 
+    // STEP: the wave that holds the page of cell pos (always in its last step) encodes the new row
+    // with the append kernel's encoder, one lane per 32-value block, into the LDS unit that has
+    // just landed and into the pool.
+    const auto take_new_row = [&](const float* new_rows, uint8_t* lds_unit, uint8_t* pool_unit) {
+        if (lane < 8) {
+            float x[32];
+            const float* src = new_rows + ((size_t)e * P.n_kv + (size_t)kvh) * kHd + lane * 32;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float4 a = *reinterpret_cast<const float4*>(src + 4 * j);
+                x[4 * j] = a.x, x[4 * j + 1] = a.y, x[4 * j + 2] = a.z, x[4 * j + 3] = a.w;
+            }
+            uint32_t w[8], hb;
+            i8h_block_words(x, w, hb);
+            const int r = pos & (kPage - 1);
+            uint8_t* const rows[2] = {lds_unit + r * kRow, pool_unit + (size_t)r * kRow};
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                *reinterpret_cast<v4u*>(rows[t] + lane * 32) = v4u{w[0], w[1], w[2], w[3]};
+                *reinterpret_cast<v4u*>(rows[t] + lane * 32 + 16) = v4u{w[4], w[5], w[6], w[7]};
+                *reinterpret_cast<unsigned short*>(rows[t] + kHd + 2 * lane) = (unsigned short)hb;
+            }
+        }
+        // the wave's own LDS writes are in order with its later reads; keep the compiler from
+        // moving those reads up
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+
     // One page: step i of the wave, resident in `slot`; the slot is refilled with step i + 2.
     const auto one_page = [&](uint8_t* slot, int i) __attribute__((always_inline)) {
         const int pg = pg0 + wave + kWaves * i;
@@ -518,6 +550,9 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
 
         // ---- scores: per block, codes . q on the matrix core, then the block's scale ----------------
         __builtin_amdgcn_s_waitcnt(0x0F7F);  // vmcnt(15): this page's K unit has landed
+        if constexpr (STEP) {
+            if (pg == n_pages - 1) take_new_row(P.new_k, slot, P.kpool_w + unit_off(i));
+        }
         f4 s = f4{0.0f, 0.0f, 0.0f, 0.0f};
         // all fragments of the unit are requested from LDS in one batch, ahead of the first use
         half8 ksc[4];
@@ -552,6 +587,9 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
         // ---- this page's V fragments are requested before the softmax, whose chain of dependent
         // instructions then has the dequantisation to overlap with -----------------------------------
         __builtin_amdgcn_s_waitcnt(0x0F7F);  // vmcnt(15): this page's V unit has landed
+        if constexpr (STEP) {
+            if (pg == n_pages - 1) take_new_row(P.new_v, slot + kI8hUnit, P.vpool_w + unit_off(i));
+        }
         // Scales of the lane's rows 4 g + r for its block of either half.  Rows past `pos` may hold
         // anything: their probabilities are exact zeros already, and their scales are made zeros
         // too, so that 0 * (garbage scale) cannot produce a NaN (any int8 code is a finite number).
@@ -710,6 +748,7 @@ __device__ __forceinline__ float dpp_mov(float x) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
 }
 
+template <bool STEP>
 __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const AttnKernelParams P) {
     // per wave one K slot and two V slots during the loop, the fold staging after it
     constexpr int kWaveLds = kQ8vKSlot + 2 * kQ8vUnit;
@@ -770,6 +809,52 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
     float l_run = 0.0f;       // this lane's share of sum exp2(logit - m_run)
     const int my_block = c >> 2;  // which of the 4 blocks of a half this lane's 8 columns lie in
 
+    // STEP: the wave that holds the page of cell pos (always in its last step) stores the new row
+    // as the append kernel does -- K under the f16 rule, 8 values a lane; V as q8_0 blocks, one lane
+    // per block -- into the LDS units that have just landed and into the pool.
+    const auto wave_lds_fence = [&]() {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+    const auto take_new_k = [&](int i) {
+        const int r = pos & (kPage - 1);
+        if (lane < 32) {
+            const float* src = P.new_k + ((size_t)e * P.n_kv + (size_t)kvh) * kHd + lane * 8;
+            const float4 a = *reinterpret_cast<const float4*>(src);
+            const float4 b = *reinterpret_cast<const float4*>(src + 4);
+            v4u w;
+            w.x = f16_store_pair(a.x, a.y), w.y = f16_store_pair(a.z, a.w);
+            w.z = f16_store_pair(b.x, b.y), w.w = f16_store_pair(b.z, b.w);
+            *reinterpret_cast<v4u*>(kslot + (r >> 1) * kQ8vKStep + (r & 1) * 512 + lane * 16) = w;
+            *reinterpret_cast<v4u*>(P.kpool_w + phys(i) * k_page_bytes + k_head_off + (size_t)r * 512 + lane * 16) = w;
+        }
+        wave_lds_fence();
+    };
+    const auto take_new_v = [&](int i, uint8_t* lds_unit) {
+        const int r = pos & (kPage - 1);
+        if (lane < 8) {
+            float x[32];
+            const float* src = P.new_v + ((size_t)e * P.n_kv + (size_t)kvh) * kHd + lane * 32;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float4 a = *reinterpret_cast<const float4*>(src + 4 * j);
+                x[4 * j] = a.x, x[4 * j + 1] = a.y, x[4 * j + 2] = a.z, x[4 * j + 3] = a.w;
+            }
+            uint32_t w[9];
+            q8v_block_words(x, w);
+            uint32_t* const ld = reinterpret_cast<uint32_t*>(lds_unit + r * kQ8vRow + lane * 36);
+            uint32_t* const gd = reinterpret_cast<uint32_t*>(P.vpool_w + phys(i) * v_page_bytes + v_head_off +
+                                                              (size_t)r * kQ8vRow + lane * 36);
+#pragma unroll
+            for (int j = 0; j < 9; ++j) {
+                ld[j] = w[j];
+                gd[j] = w[j];
+            }
+        }
+        wave_lds_fence();
+    };
+
     for (int i = 0; i < n_steps; ++i) {
         const int pg = pg0 + wave + kWaves * i;
         const uint8_t* vs = slots + (i & 1) * kQ8vUnit;
@@ -777,6 +862,9 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
 
         // ---- S^T = K . q^T: four independent accumulation chains ------------------------------
         __builtin_amdgcn_s_waitcnt(0x0F75);  // vmcnt(5): this page's K unit has landed
+        if constexpr (STEP) {
+            if (pg == n_pages - 1) take_new_k(i);
+        }
         v4u kf[8];
         {
             // row c: two rows per 1056-byte step; fragment m of lane group g at 64 m + 16 g
@@ -800,6 +888,9 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
 
         // ---- this page's V unit: scales first -------------------------------------------------
         __builtin_amdgcn_s_waitcnt(0x4F75);  // vmcnt(21): K(i), V(i+1), K(i+1) behind V(i)
+        if constexpr (STEP) {
+            if (pg == n_pages - 1) take_new_v(i, slots + (i & 1) * kQ8vUnit);
+        }
         // lane (c, g): scale of blocks 2 (c / 4), + 1 of row 4 g + c % 4, the row's maximum over the
         // lanes c, c ^ 4, c ^ 8, c ^ 12, then the four rows' maxima from the lanes of the quad
         const bool last_page = pg == n_pages - 1;
@@ -913,11 +1004,17 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
 
 hipError_t launch_decode_attn_mfma(const AttnKernelParams& kp, int layout, bool step, bool sel, int32_t total,
                                    hipStream_t stream) {
-    if (layout == BKV_LAYOUT_I8H)
-        decode_attn_mfma_i8h_kernel<<<total, kBlock, 0, stream>>>(kp);
-    else if (layout == BKV_LAYOUT_Q8V)
-        decode_attn_mfma_q8v_kernel<<<total, kBlock, 0, stream>>>(kp);
-    else if (step)
+    if (layout == BKV_LAYOUT_I8H) {
+        if (step)
+            decode_attn_mfma_i8h_kernel<true><<<total, kBlock, 0, stream>>>(kp);
+        else
+            decode_attn_mfma_i8h_kernel<false><<<total, kBlock, 0, stream>>>(kp);
+    } else if (layout == BKV_LAYOUT_Q8V) {
+        if (step)
+            decode_attn_mfma_q8v_kernel<true><<<total, kBlock, 0, stream>>>(kp);
+        else
+            decode_attn_mfma_q8v_kernel<false><<<total, kBlock, 0, stream>>>(kp);
+    } else if (step)
         decode_attn_mfma_kernel<true><<<total, kBlock, 0, stream>>>(kp);
     else if (sel)
         decode_attn_mfma_kernel<false, true><<<total, kBlock, 0, stream>>>(kp);

@@ -5,6 +5,7 @@
 // coalescing and several independent loads in flight per lane.
 #include "bkv_internal.hpp"
 #include "f16_rule.hpp"
+#include "quant_encode.hpp"
 
 namespace bkv {
 
@@ -24,17 +25,6 @@ __device__ __forceinline__ void st_stream(void* p, v4u v) {
 }
 
 __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return f16_store_pair(lo, hi); }
-
-// binary16 code -> f32 under the cache's load rule (f16_storage.glsl:58-69):
-// exponent field 0 reads as a signed zero.
-__device__ __forceinline__ float f16_load(uint32_t h) {
-    const uint32_t sign = (h & 0x8000u) << 16;
-    const uint32_t e = (h >> 10) & 0x1fu;
-    const uint32_t m = h & 0x3ffu;
-    if (e == 0) return __uint_as_float(sign);
-    if (e == 31) return __uint_as_float(sign | 0x7f800000u | (m << 13));
-    return __uint_as_float(sign | ((e + 112u) << 23) | (m << 13));
-}
 
 struct MoveGeom {
     int32_t n_kv, hd, page_cells, max_pages_per_seq;
@@ -106,34 +96,6 @@ __global__ __launch_bounds__(kBlock) void append_f16_kernel(AppendBatch b, MoveG
     st_stream(vpool + dst, vo);
 }
 
-// q8_0 codes of 32 values (shaders/qsa_kv_append.comp:113-132, qsa/cpu.rs:65-82):
-// scale = amax/127 (1 if amax == 0), q = round-half-away(clamp(x/scale, +-127)).
-__device__ __forceinline__ void q8_block(const float (&x)[32], float scale, uint32_t (&w)[8]) {
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        uint32_t packed = 0;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            float t = x[j * 4 + i] / scale;
-            t = t < -127.0f ? -127.0f : t;
-            t = t > 127.0f ? 127.0f : t;
-            const int q = (int)roundf(t);
-            packed |= ((uint32_t)q & 0xffu) << (8 * i);
-        }
-        w[j] = packed;
-    }
-}
-
-__device__ __forceinline__ float amax32(const float (&x)[32]) {
-    float amax = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 32; ++i) {
-        const float a = fabsf(x[i]);
-        amax = a > amax ? a : amax;
-    }
-    return amax;
-}
-
 template <typename SrcT>
 __device__ __forceinline__ void load32(const SrcT* p, float (&x)[32]) {
 #pragma unroll
@@ -147,13 +109,10 @@ __device__ __forceinline__ void load32(const SrcT* p, float (&x)[32]) {
 
 // One q8_0 block as the V pool holds it: [f32 scale][32 x i8] = 9 words.
 __device__ __forceinline__ void q8v_encode(const float (&x)[32], uint32_t* vd) {
-    const float amax = amax32(x);
-    const float scale = amax > 0.0f ? amax / 127.0f : 1.0f;
-    uint32_t w[8];
-    q8_block(x, scale, w);
-    vd[0] = __float_as_uint(scale);
+    uint32_t w[9];
+    q8v_block_words(x, w);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) vd[1 + j] = w[j];
+    for (int j = 0; j < 9; ++j) vd[j] = w[j];
 }
 
 // ---- append, reference q8_0-V rows: K f16, V [f32 scale][32 x i8] per 32 values ---
@@ -201,29 +160,8 @@ __global__ __launch_bounds__(kBlock) void append_q8v_kernel(AppendBatch b, MoveG
 // The q8_0 rule with the scale stored through the cache's f16 encoding; a scale the
 // f16 rule would flush is raised to 2^-14.  (No reference counterpart.)
 __device__ __forceinline__ void i8h_encode(const float (&x)[32], uint8_t* row_base, int hd, int blk) {
-    const float amax = amax32(x);
-    uint32_t hb;
-    if (amax > 0.0f) {
-        hb = f16_store_bits(amax / 127.0f);
-        if ((hb & 0x7fffu) == 0) hb = 0x0400u;
-    } else {
-        hb = 0x3c00u;
-    }
-    const float sh = f16_load(hb);
-    uint32_t w[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        uint32_t packed = 0;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            float t = x[j * 4 + i] / sh;
-            t = !(t >= -127.0f) ? -127.0f : t;
-            t = t > 127.0f ? 127.0f : t;
-            const int q = (int)roundf(t);
-            packed |= ((uint32_t)q & 0xffu) << (8 * i);
-        }
-        w[j] = packed;
-    }
+    uint32_t w[8], hb;
+    i8h_block_words(x, w, hb);
     uint4* qd = reinterpret_cast<uint4*>(row_base + (size_t)blk * 32);
     qd[0] = make_uint4(w[0], w[1], w[2], w[3]);
     qd[1] = make_uint4(w[4], w[5], w[6], w[7]);

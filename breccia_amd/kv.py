@@ -351,7 +351,7 @@ class Pool:
     def decode_step(self, layer: int, seqs, pos, k_new_dev, v_new_dev, n_q_head: int, q_dev, out_dev,
                     scale: float, gate_dev=None, gate_seq_stride: int = 0, gate_head_stride: int = 0,
                     stream=None) -> None:
-        """Append one token per sequence at pos and attend 0..pos, in one call (f16 pools)."""
+        """Append one token per sequence at pos and attend 0..pos, in one call."""
         seqs, ps = _i32(seqs)
         pos, pp = _i64(pos)
         assert seqs.size == pos.size

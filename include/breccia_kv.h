@@ -262,11 +262,13 @@ bkv_status bkv_prefill_attn(bkv_pool *pool, int32_t layer, int32_t n_seqs, const
  * pos[i] and attend cells 0..pos[i] -- bkv_append of one token per sequence followed by
  * bkv_decode_attn, without the append launch (Qsa::kv_append + Qsa::attend + Qsa::apply of
  * a T = 1 call, qsa/mod.rs:1617-1639).  The work-group that owns the last page of a sequence
- * takes the row from k_new_dev / v_new_dev (f32 [n][n_kv_head][head_dim]), stores it under
- * the cache's f16 rule -- the pool afterwards holds exactly what bkv_append would have
- * written -- and uses it in place of the stale pool row; the output is bit-identical to the
- * two-call sequence.  f16 pools only; every sequence at most once per call; the cell must
- * have been reserved (bkv_seq_reserve) like for bkv_append. */
+ * takes the row from k_new_dev / v_new_dev (f32 [n][n_kv_head][head_dim]), stores it in the
+ * pool's layout with the append kernels' own encoders (f16 rule, q8_0 blocks, int8 blocks) --
+ * the pool afterwards holds exactly what bkv_append would have written -- and uses it in
+ * place of the stale pool row; the output is bit-identical to the two-call sequence.  Every
+ * sequence at most once per call; the cell must have been reserved (bkv_seq_reserve) like for
+ * bkv_append.  On quantised pools the step is served by the matrix-core kernels only (at most
+ * 16 q heads per kv head, pool without BKV_POOL_ATTN_VALU; BKV_ERR_INVALID otherwise). */
 bkv_status bkv_decode_step(bkv_pool *pool, int32_t layer, int32_t n, const int32_t *seqs,
                            const int64_t *pos, const float *k_new_dev, const float *v_new_dev,
                            int32_t n_q_head, const float *q_dev, const float *gate_dev,

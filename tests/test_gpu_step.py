@@ -36,11 +36,24 @@ def step(tw, layer, seqs, pos, k_new, v_new, q, n_head, gate=None):
                 b.free()
 
 
+@pytest.mark.parametrize("layout", [L.LAYOUT_F16, L.LAYOUT_Q8V, L.LAYOUT_I8H])
 @pytest.mark.parametrize("n_q", [16, 24])
-def test_fused_step_equals_append_then_attend(n_q):
-    rng = np.random.Generator(np.random.PCG64(800 + n_q))
+def test_fused_step_equals_append_then_attend(n_q, layout):
+    import gpu_common
+    rng = np.random.Generator(np.random.PCG64(800 + n_q + 7 * layout))
     lens = [37, 512, 1000, 2048, 15, 16, 1, 0, 4099]      # page edges, an empty sequence, long
-    with Twin(n_pages=700, max_seqs=24) as tw:
+    if layout != L.LAYOUT_F16 and gpu_common.DEFAULT_ATTN_VALU:
+        # on quantised pools the step exists on the matrix-core path only: refused, pool untouched
+        with Twin(n_pages=16, max_seqs=4, layout=layout) as tw:
+            s = tw.pool.seq_create()
+            tw.pool.seq_reserve(s, 20)
+            z = DeviceBuffer(1 << 16)
+            with pytest.raises(BkvError) as ei:
+                tw.pool.decode_step(0, [s], [19], z, z, n_q, z, z, 0.0625)
+            assert ei.value.status == L.ERR_INVALID
+            z.free()
+        return
+    with Twin(n_pages=700, max_seqs=24, layout=layout) as tw:
         tw.pool.set_free_order(rng.permutation(700).astype(np.int32))
         fused = [tw.pool.seq_create() for _ in lens]
         for s, n in zip(fused, lens):
@@ -52,6 +65,8 @@ def test_fused_step_equals_append_then_attend(n_q):
             k_new = rng.standard_normal((len(lens), 2, 256)).astype(np.float32)
             v_new = rng.standard_normal((len(lens), 2, 256)).astype(np.float32)
             k_new[0, 0, :4] = [1e-6, -1e-9, np.nan, 7e4]     # the store rule's special cases
+            v_new[1, 1, 32:64] = 0.0                           # an all-zero block (scale 1 by rule)
+            v_new[2, 0, 64:96] *= 1e-7                         # a block whose f16 scale would flush
             q = rng.standard_normal((len(lens), n_q, 256)).astype(np.float32)
             gate = rng.standard_normal((len(lens), n_q, 256)).astype(np.float32)
             # two calls on the forks (copy-on-write where a shared partial page is written)
@@ -103,10 +118,11 @@ def test_step_errors_come_before_any_launch():
         assert np.array_equal(before, tw.pool.read_layer(0, 0))
         z.free()
     with Twin(n_pages=16, max_seqs=4, layout=L.LAYOUT_I8H) as tw:
+        # 24 q heads per kv head are beyond what the kernels take
         s = tw.pool.seq_create()
         tw.pool.seq_reserve(s, 20)
-        z = DeviceBuffer(1 << 16)
+        z = DeviceBuffer(1 << 18)
         with pytest.raises(BkvError) as ei:
-            tw.pool.decode_step(0, [s], [19], z, z, 16, z, z, 0.0625)
+            tw.pool.decode_step(0, [s], [19], z, z, 48, z, z, 0.0625)
         assert ei.value.status == L.ERR_INVALID
         z.free()
