@@ -14,15 +14,15 @@
 // cells and per wave:
 //   S^T[cell][query] = K[cell][:] . Q[query][:]        v_mfma_f32_16x16x32_f16, A = K, B = Q
 //   online softmax per query (base 2), P^T in the layout S^T came out in
-//   O^T[d][query]   += V^T[d][cell] . P^T[cell][query]  v_mfma_f32_16x16x32_f16 over the page's 16
-//                                                       cells twice, A = V gathered per lane (the
-//                                                       same four cells in both halves of a lane's
-//                                                       slots), B = P^T high parts, then low parts
+//   O^T[d][query]   += V^T[d][cell] . P^T[cell][query]  v_mfma_f32_16x16x32_f16 over the 32 cells of
+//                                                       two pages, A = V gathered per lane (four
+//                                                       cells of either page), B = P^T, high parts
+//                                                       and low parts in one MFMA each
 // Both products keep the per-lane query (lane % 16) fixed, so the softmax statistics never
 // move between lanes, and P^T feeds the second product straight from registers.  K and V are
-// exact f16; q and p are f32 values split into a high and a low f16 part (two MFMAs for the
-// scores, the two halves of one for P.V), so the products carry ~22 significant bits and the
-// result stays at f32-accumulate accuracy.
+// exact f16; q and p are f32 values split into a high and a low f16 part (two MFMAs each), so the
+// products carry ~22 significant bits and the result stays at f32-accumulate accuracy.  Pages are
+// walked two at a time: one softmax update and one barrier per pair.
 // The V operand needs four cells of one head-dim column per lane: each lane loads 16 bytes
 // (8 columns) of four rows and regroups them in registers; the 8 MFMAs that use them produce
 // columns 8i + t of the output, i = the MFMA row, t = 0..7.
@@ -146,8 +146,10 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
     // ---- pages through LDS: [buffer][K | V][16 rows][264 halves] -------------------------------
     // Rows are padded to 528 bytes so that the 16-byte fragment reads of the 64 lanes spread
     // evenly over the banks.  A page image is 2 x 512 chunks of 16 bytes: thread t moves chunk
-    // t (+ kThreads, ...) of K and of V.
-    __shared__ __attribute__((aligned(16))) _Float16 lds[2][2][kPage][kLdsRow];
+    // t (+ kThreads, ...) of K and of V.  Pages are taken two at a time (one softmax update, one
+    // barrier and P.V MFMAs that contract over the 32 cells of the pair): four buffers, the pair
+    // being multiplied and the pair being filled.
+    __shared__ __attribute__((aligned(16))) _Float16 lds[4][2][kPage][kLdsRow];
     const int tid = threadIdx.x;
     const auto fetch = [&](int pg, v4u (&stage)[2 * kChunks]) {
         const int32_t phys = bt[pg];
@@ -169,27 +171,16 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
         }
     };
 
-    // one page of this wave: scores -> softmax -> accumulate, operands from LDS buffer `buf`
-    const auto process = [&](int pg, int buf) {
+    // scores of one page: s[r] = q[row c] . k[cell 4 g + r], masked and in base 2
+    const auto scores = [&](int pg, int buf, float (&t4)[4]) {
         const _Float16* ks = &lds[buf][0][0][0];
-        const _Float16* vs = &lds[buf][1][0][0];
-        // ---- S^T = K . Q^T ------------------------------------------------------------------
-        // four independent accumulation chains: an MFMA that waits for the previous one's result
-        // costs its full latency
         // K: row c, 16 bytes at element 32 m + 8 g (the same split of the head dim as q): the 8
-        // halves of a lane are the 8 contraction steps it feeds to the 32-deep MFMA.  All fragments
-        // of the page are requested from LDS in one batch; V's follow while the scores are formed.
+        // halves of a lane are the 8 contraction steps it feeds to the 32-deep MFMA
         h8 kf[8];
 #pragma unroll
         for (int m = 0; m < 8; ++m) kf[m] = *reinterpret_cast<const h8*>(ks + c * kLdsRow + m * 32 + g * 8);
-        __builtin_amdgcn_sched_barrier(0);
-        // V: rows 4 g + r, 16 bytes at element 128 half + 8 c
-        v4u vf[2][4];
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-                vf[h][r] = *reinterpret_cast<const v4u*>(vs + (4 * g + r) * kLdsRow + h * 128 + c * 8);
+        // four independent accumulation chains: an MFMA that waits for the previous one's result
+        // costs its full latency
         f4 s0 = f4{0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0, s2 = s0, s3 = s0;
 #pragma unroll
         for (int m = 0; m < 8; m += 2) {
@@ -199,36 +190,49 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
             s3 = mfma32(kf[m + 1], qlo[m + 1], s3);
         }
         const f4 s = (s0 + s1) + (s2 + s3);
-        // s[r] = q[row c] . k[cell 4 g + r]
-
-        // ---- online softmax for this lane's query ------------------------------------------------
-        float t4[4];
-        float pm = -INFINITY;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int cell = pg * kPage + 4 * g + r;
             t4[r] = cell <= pos_q ? s[r] * P.scale_log2e : -INFINITY;
-            pm = fmaxf(pm, t4[r]);
         }
+    };
+
+    // pages pg and pg + 1 of this wave: scores -> softmax -> accumulate, operands from the LDS
+    // buffers buf and buf + 1.  The second page may lie past the wave's last one: it then counts
+    // as all dead (its buffer holds some finite page of the work-group, or nothing yet).
+    const auto process_pair = [&](int pg, int buf) {
+        const bool second = pg + 1 < n_pages;
+        float ta[4], tb[4];
+        scores(pg, buf, ta);
+        if (second) {
+            scores(pg + 1, buf + 1, tb);
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) tb[r] = -INFINITY;
+        }
+
+        // ---- online softmax for this lane's query, over the pair's 32 cells ---------------------------
+        float pm = fmaxf(fmaxf(fmaxf(ta[0], ta[1]), fmaxf(ta[2], ta[3])), fmaxf(fmaxf(tb[0], tb[1]), fmaxf(tb[2], tb[3])));
         pm = max_over_lane_groups(pm);
         const float m_new = fmaxf(m_run, pm);
         // a query with no live cell yet keeps m = -inf: exp2(-inf - -inf) would be NaN
-        const float alpha = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
-        h4 phi, plo;
+        const bool none_yet = m_new == -INFINITY;
+        const float alpha = none_yet ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
+        h8 ph, pl;  // slots 0..3: the first page's cells 4 g + r, slots 4..7: the second page's
         float psum = 0.0f;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const float p = m_new == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(t4[r] - m_new);
+        for (int r = 0; r < 8; ++r) {
+            const float tt = r < 4 ? ta[r & 3] : tb[r & 3];
+            const float p = none_yet ? 0.0f : __builtin_amdgcn_exp2f(tt - m_new);
             psum += p;
             _Float16 hi, lo;
             split_f16(p, hi, lo);
-            phi[r] = hi;
-            plo[r] = lo;
+            ph[r] = hi;
+            pl[r] = lo;
         }
-        const h8 phl = h8{phi[0], phi[1], phi[2], phi[3], plo[0], plo[1], plo[2], plo[3]};
         l_run = l_run * alpha + psum;
-        // rescale only on pages where some query's maximum moved (the test is on the maxima, not on
-        // alpha != 1: with the latter the compiler multiplies unconditionally, 64 instructions a page)
+        // rescale only where some query's maximum moved (the test is on the maxima, not on
+        // alpha != 1: with the latter the compiler multiplies unconditionally, 64 instructions)
         const bool moved = m_new > m_run;
         m_run = m_new;
         if (__builtin_amdgcn_ballot_w64(moved) != 0) {
@@ -238,50 +242,61 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
                 for (int t = 0; t < 8; ++t) o[h][t] *= alpha;
         }
 
-        // Rows past the last position of this wave were never written for these queries and may
-        // hold anything (even NaN): make them exact zeros before they meet a zero probability.
-        if (pg == n_pages - 1) {
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-                if (pg * kPage + 4 * g + r > pos_max) {
-                    vf[0][r] = v4u{0u, 0u, 0u, 0u};
-                    vf[1][r] = v4u{0u, 0u, 0u, 0u};
-                }
-        }
-
-        // ---- O^T += V^T . P^T ---------------------------------------------------------------------
+        // ---- O^T += V^T . P^T over the 32 cells of the pair ----------------------------------------
+        // V: rows 4 g + r of either page, 16 bytes at element 128 half + 8 c.  Rows past the last
+        // position of this wave were never written for these queries and may hold anything (even
+        // NaN): they are made exact zeros before they meet a zero probability.
+        const _Float16* va_s = &lds[buf][1][0][0];
+        const _Float16* vb_s = &lds[buf + 1][1][0][0];
+        const bool a_last = pg == n_pages - 1, b_last = pg + 1 == n_pages - 1;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            const h8 v0 = __builtin_bit_cast(h8, vf[h][0]), v1 = __builtin_bit_cast(h8, vf[h][1]);
-            const h8 v2 = __builtin_bit_cast(h8, vf[h][2]), v3 = __builtin_bit_cast(h8, vf[h][3]);
+            v4u fa[4], fb[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                fa[r] = *reinterpret_cast<const v4u*>(va_s + (4 * g + r) * kLdsRow + h * 128 + c * 8);
+                fb[r] = *reinterpret_cast<const v4u*>(vb_s + (4 * g + r) * kLdsRow + h * 128 + c * 8);
+            }
+            if (a_last || b_last || !second) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if (a_last && pg * kPage + 4 * g + r > pos_max) fa[r] = v4u{0u, 0u, 0u, 0u};
+                    if (!second || (b_last && (pg + 1) * kPage + 4 * g + r > pos_max)) fb[r] = v4u{0u, 0u, 0u, 0u};
+                }
+            }
+            const h8 a0 = __builtin_bit_cast(h8, fa[0]), a1 = __builtin_bit_cast(h8, fa[1]);
+            const h8 a2 = __builtin_bit_cast(h8, fa[2]), a3 = __builtin_bit_cast(h8, fa[3]);
+            const h8 b0 = __builtin_bit_cast(h8, fb[0]), b1 = __builtin_bit_cast(h8, fb[1]);
+            const h8 b2 = __builtin_bit_cast(h8, fb[2]), b3 = __builtin_bit_cast(h8, fb[3]);
 #pragma unroll
             for (int t = 0; t < 8; ++t) {
-                // column 128 h + 8 c + t of cells 4 g ..: the 32-deep MFMA runs over the 16 cells twice,
-                // against the high parts of p and then the low parts
-                const h8 vv = h8{v0[t], v1[t], v2[t], v3[t], v0[t], v1[t], v2[t], v3[t]};
-                o[h][t] = mfma32(vv, phl, o[h][t]);
+                // column 128 h + 8 c + t of the pair's cells 4 g .. of either page
+                const h8 vv = h8{a0[t], a1[t], a2[t], a3[t], b0[t], b1[t], b2[t], b3[t]};
+                o[h][t] = mfma32(vv, ph, o[h][t]);
+                o[h][t] = mfma32(vv, pl, o[h][t]);
             }
         }
     };
 
-    // Two pages are in flight behind the one being multiplied: staging set A carries the even
-    // pages, B the odd ones (past the end they carry the last page again).
+    // Two pairs are in flight behind the one being multiplied: one in the other two LDS buffers,
+    // one in the staging registers (past the end they carry the last page again).
     v4u stage_a[2 * kChunks], stage_b[2 * kChunks];
     const int last_pg = wg_pages - 1;
     fetch(0, stage_a);
     fetch(min(1, last_pg), stage_b);
     deposit(0, stage_a);
+    deposit(1, stage_b);
     fetch(min(2, last_pg), stage_a);
+    fetch(min(3, last_pg), stage_b);
     __syncthreads();
     for (int pg = 0; pg < wg_pages; pg += 2) {
-        if (pg < n_pages) process(pg, 0);
-        deposit(1, stage_b);                      // page pg + 1
-        fetch(min(pg + 3, last_pg), stage_b);
-        // after the barrier the other buffer is complete, and nobody reads this one any more
-        __syncthreads();
-        if (pg + 1 < n_pages) process(pg + 1, 1);
-        deposit(0, stage_a);                      // page pg + 2
+        const int buf = pg & 2;  // 0 or 2
+        if (pg < n_pages) process_pair(pg, buf);
+        deposit(buf ^ 2, stage_a);  // pages pg + 2, pg + 3
+        deposit((buf ^ 2) + 1, stage_b);
         fetch(min(pg + 4, last_pg), stage_a);
+        fetch(min(pg + 5, last_pg), stage_b);
+        // after the barrier the other pair of buffers is complete, and nobody reads this one any more
         __syncthreads();
     }
 
