@@ -425,12 +425,6 @@ __device__ __forceinline__ half8 codes8_to_f16(v2u w) {
     codes_to_f16(w.y, c2, d);
     return half8{a[0], a[1], b[0], b[1], c2[0], c2[1], d[0], d[1]};
 }
-// f16 scale under the cache's load rule (exponent field 0 reads as zero)
-__device__ __forceinline__ float scale_of(_Float16 h) {
-    const unsigned short bits = __builtin_bit_cast(unsigned short, h);
-    return (bits & 0x7c00u) == 0 ? 0.0f : (float)h;
-}
-
 // Data path: rows reach the matrix cores through LDS, not through registers.  Every wave owns two
 // slots of 2 x 4352 bytes (the K unit and the V unit of one page and kv head, scales included)
 // and fills them with 16-byte global->LDS loads, 64 lanes x 16 contiguous bytes per instruction
