@@ -425,11 +425,13 @@ __device__ __forceinline__ half8 codes8_to_f16(v2u w) {
     codes_to_f16(w.y, c2, d);
     return half8{a[0], a[1], b[0], b[1], c2[0], c2[1], d[0], d[1]};
 }
+
 // Data path: rows reach the matrix cores through LDS, not through registers.  Every wave owns two
 // slots of 2 x 4352 bytes (the K unit and the V unit of one page and kv head, scales included)
 // and fills them with 16-byte global->LDS loads, 64 lanes x 16 contiguous bytes per instruction
 // (whole cache lines, nothing fetched twice), two pages ahead of the page it computes: the K half
-// of a slot is refilled right after the scores that read it, the V half right after P.V.  A
+// of a slot is refilled right after the scores that read it, the V half right after P.V (whose
+// fragments are requested before the softmax, so that their dequantisation overlaps it).  A
 // wave has 20 such loads in flight in a fixed order (K, V of the next page, K, V of the one
 // after), so "the oldest five have landed" is s_waitcnt vmcnt(15) at both points of use.
 constexpr int kI8hUnit = kPage * row_bytes_of(kRowI8H);  // 4352
