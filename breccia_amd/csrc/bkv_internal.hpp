@@ -202,7 +202,7 @@ struct PrefillBatch {
     int32_t src0[BKV_MAX_BATCH];    // first token row in q / out
     int32_t wg_base[BKV_MAX_BATCH + 1];
 };
-int32_t prefill_rows_per_wg();
+int32_t prefill_rows_per_wg(int32_t layout);  // query rows one work-group owns
 hipError_t launch_prefill_attn(bkv_pool* p, int32_t layer, const PrefillBatch& b, const AttnArgs& a,
                                hipStream_t stream);
 // heads one wave carries for a given q-heads-per-kv-head group

@@ -5,6 +5,7 @@
 #include "decode_attn_common.hpp"
 #include "f16_rule.hpp"
 #include "lane_groups.hpp"
+#include "quant_decode.hpp"
 #include "quant_encode.hpp"
 
 namespace bkv {
@@ -388,32 +389,6 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
 //           needs one scale per V row and half.
 // The VALU formulation of this layout is bound by instruction issue (conversions and FMAs, 40 %
 // of the HBM roofline on long contexts); here the VALU only converts and scales.
-typedef _Float16 h2m __attribute__((ext_vector_type(2)));
-
-// four int8 codes (one dword) -> four exact f16 values: 0x6400 | (code ^ 0x80) is 1024 + (code + 128)
-__device__ __forceinline__ void codes_to_f16(unsigned w, h2m& lo, h2m& hi) {
-    const unsigned u = w ^ 0x80808080u;
-    const h2m bias = h2m{(_Float16)1152.0f, (_Float16)1152.0f};
-    lo = __builtin_bit_cast(h2m, __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u)) - bias;
-    hi = __builtin_bit_cast(h2m, __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - bias;
-}
-// the same for codes that already carry the ^ 0x80 bias
-__device__ __forceinline__ void biased_to_f16(unsigned u, h2m& lo, h2m& hi) {
-    const h2m bias = h2m{(_Float16)1152.0f, (_Float16)1152.0f};
-    lo = __builtin_bit_cast(h2m, __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u)) - bias;
-    hi = __builtin_bit_cast(h2m, __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - bias;
-}
-// 4 x 4 byte transpose: t[j] = { w[0].byte j, w[1].byte j, w[2].byte j, w[3].byte j }
-__device__ __forceinline__ void transpose4x4_bytes(const unsigned (&w)[4], unsigned (&t)[4]) {
-    const unsigned a_lo = __builtin_amdgcn_perm(w[1], w[0], 0x05010400u);  // w0.0 w1.0 w0.1 w1.1
-    const unsigned a_hi = __builtin_amdgcn_perm(w[1], w[0], 0x07030602u);  // w0.2 w1.2 w0.3 w1.3
-    const unsigned b_lo = __builtin_amdgcn_perm(w[3], w[2], 0x05010400u);
-    const unsigned b_hi = __builtin_amdgcn_perm(w[3], w[2], 0x07030602u);
-    t[0] = __builtin_amdgcn_perm(b_lo, a_lo, 0x05040100u);
-    t[1] = __builtin_amdgcn_perm(b_lo, a_lo, 0x07060302u);
-    t[2] = __builtin_amdgcn_perm(b_hi, a_hi, 0x05040100u);
-    t[3] = __builtin_amdgcn_perm(b_hi, a_hi, 0x07060302u);
-}
 // whether either f16 of a dword has exponent field 0 (the values the cache reads as zero)
 __device__ __forceinline__ bool has_zero_exponent(unsigned two_halves) {
     const unsigned t = two_halves & 0x7c007c00u;
@@ -737,11 +712,6 @@ __device__ __forceinline__ void q8v_unit_to_lds(const uint8_t* src, bool real, u
     for (int n = 0; n < 4; ++n)
         __builtin_amdgcn_global_load_lds((gptr)(lane_src + n * step), (lptr)(dst + n * 1024), 16, 0, 0);
     if (lane < 32) __builtin_amdgcn_global_load_lds((gptr)(lane_src + 4 * step), (lptr)(dst + 4096), 16, 0, 0);
-}
-
-template <int CTRL>
-__device__ __forceinline__ float dpp_mov(float x) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
 }
 
 template <bool STEP>

@@ -37,4 +37,11 @@ __device__ __forceinline__ float sum_over_lane_groups(float x) {
     return q.a + q.b;
 }
 
+// x of the lane a DPP control names (row_ror:4 = 0x124, row_ror:8 = 0x128, quad_perm broadcasts
+// 0x00 / 0x55 / 0xAA / 0xFF), within the lane's row of 16
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
+}
+
 }  // namespace bkv

@@ -26,8 +26,18 @@
 // The V operand needs four cells of one head-dim column per lane: each lane loads 16 bytes
 // (8 columns) of four rows and regroups them in registers; the 8 MFMAs that use them produce
 // columns 8i + t of the output, i = the MFMA row, t = 0..7.
+//
+// Pools with q8_0 V ([f32 scale][32 x i8] blocks, qsa_attn_apply_gqa.comp:53-77) take the same
+// walk with work-groups of eight waves: the threads that fetch a V page dequantise it once for
+// all eight, on its way into LDS, into two f16 images whose sum is the value to 22 bits
+//   E[cell]    = exponent of the largest of the cell's 8 block scales (clamped to +-120),
+//   a[cell][d] = code * (scale * 2^-E[cell]) = hi + lo,
+// and the softmax runs over logit + E with weights exp2(logit + E - M) (the denominator sums
+// exp2(logit - M)), as in the decode kernel for this layout: the largest terms have weights near
+// 1 whatever the magnitude of their values.  P.V is then hi.p_hi + hi.p_lo + lo.p_hi.
 #include "bkv_internal.hpp"
 #include "lane_groups.hpp"
+#include "quant_decode.hpp"
 
 namespace bkv {
 
@@ -36,10 +46,7 @@ namespace {
 constexpr int kHd = 256;
 constexpr int kPage = 16;
 constexpr int kRowsPerWave = 16;
-constexpr int kWavesPerWg = 4;
-constexpr int kThreads = 64 * kWavesPerWg;
-constexpr int kChunks = kPage * kHd * 2 / 16 / kThreads;  // 16-byte chunks of a K (or V) page image per thread
-constexpr int kRowsPerWg = kRowsPerWave * kWavesPerWg;
+constexpr int kQ8vRow = kHd / 32 * 36;              // bytes of a q8_0 row
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kLdsRow = kHd + 8;  // halves per row of a page image in LDS (528 bytes)
 
@@ -71,7 +78,32 @@ __device__ __forceinline__ void split_f16(float x, _Float16& hi, _Float16& lo) {
     lo = (_Float16)(x - (float)hi);
 }
 
-__global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const PrefillKernelParams P) {
+// What a thread carries of one page between its fetch and its deposit into LDS.
+template <bool Q8V>
+struct PageStage;
+template <>
+struct PageStage<false> {
+    v4u k[2], v[2];  // chunks tid and tid + 256 of either image
+};
+template <>
+struct PageStage<true> {
+    v4u k;                   // chunk tid of the K image
+    unsigned scale, c0, c1;  // of V: row tid / 32, block tid / 4 % 8, codes 8 (tid % 4) .. + 7 of it
+    int pg;
+};
+
+template <bool Q8V>
+struct PrefillLds {
+    // [buffer][K | V (q8_0: high parts, low parts)][16 rows][264 halves]
+    _Float16 img[4][Q8V ? 3 : 2][kPage][kLdsRow];
+    float e[Q8V ? 4 : 1][kPage];  // q8_0: E of the buffer's cells
+};
+
+template <bool Q8V>
+__global__ __launch_bounds__(Q8V ? 512 : 256, Q8V ? 1 : 2) void prefill_attn_kernel(const PrefillKernelParams P) {
+    constexpr int kWavesPerWg = Q8V ? 8 : 4;
+    constexpr int kThreads = 64 * kWavesPerWg;
+    constexpr int kRowsPerWg = kRowsPerWave * kWavesPerWg;
     // ---- which (entry, kv head, block of 64 query rows) ---------------------------------
     int e = 0;
     while (e + 1 < P.b.n && (int)blockIdx.x >= P.b.wg_base[e + 1]) ++e;
@@ -101,12 +133,15 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
     const int n_pages = wave_live ? pos_max / kPage + 1 : 0;
     // pages the work-group walks: those of its last row
     const int wg_last_row = min(rb * kRowsPerWg + kRowsPerWg, n_rows) - 1;
-    const int wg_pages = (P.b.pos0[e] + wg_last_row / P.group) / kPage + 1;
+    const int wg_pos_max = P.b.pos0[e] + wg_last_row / P.group;
+    const int wg_pages = wg_pos_max / kPage + 1;
 
     typedef const __attribute__((address_space(4))) int32_t* table_ptr;
     const table_ptr bt = (table_ptr)(uintptr_t)(P.tables + (size_t)P.b.row[e] * (size_t)P.max_pages_per_seq);
     const size_t page_bytes = (size_t)P.n_kv * kPage * kHd * 2;
     const size_t head_off = (size_t)kvh * kPage * kHd * 2;
+    const size_t v_page_bytes = Q8V ? (size_t)P.n_kv * kPage * kQ8vRow : page_bytes;
+    const size_t v_head_off = Q8V ? (size_t)kvh * kPage * kQ8vRow : head_off;
 
     // ---- q fragments: lane (c, g) holds q[row][32 m + 8 g + 0..7], m = 0..7, as hi + lo f16 ----
     h8 qhi[8], qlo[8];
@@ -143,37 +178,80 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
     float m_run = -INFINITY;  // running max of this lane's query (base-2 logits), same in all 4 g lanes
     float l_run = 0.0f;       // this lane's share (its 4 cells per page) of the denominator
 
-    // ---- pages through LDS: [buffer][K | V][16 rows][264 halves] -------------------------------
+    // ---- pages through LDS -----------------------------------------------------------------------
     // Rows are padded to 528 bytes so that the 16-byte fragment reads of the 64 lanes spread
-    // evenly over the banks.  A page image is 2 x 512 chunks of 16 bytes: thread t moves chunk
-    // t (+ kThreads, ...) of K and of V.  Pages are taken two at a time (one softmax update, one
+    // evenly over the banks.  An f16 page image is 512 chunks of 16 bytes: thread t moves chunk
+    // t (+ 256) of it.  Pages are taken two at a time (one softmax update, one
     // barrier and P.V MFMAs that contract over the 32 cells of the pair): four buffers, the pair
     // being multiplied and the pair being filled.
-    __shared__ __attribute__((aligned(16))) _Float16 lds[4][2][kPage][kLdsRow];
+    __shared__ __attribute__((aligned(16))) PrefillLds<Q8V> L;
     const int tid = threadIdx.x;
-    const auto fetch = [&](int pg, v4u (&stage)[2 * kChunks]) {
+    // q8_0 V: this thread's part of a page
+    const int v_row = tid >> 5, v_blk = (tid >> 2) & 7, v_j = tid & 3;
+    const auto fetch = [&](int pg, PageStage<Q8V>& st) {
         const int32_t phys = bt[pg];
         const uint8_t* kp = P.kpool + (size_t)phys * page_bytes + head_off;
-        const uint8_t* vp = P.vpool + (size_t)phys * page_bytes + head_off;
+        const uint8_t* vp = P.vpool + (size_t)phys * v_page_bytes + v_head_off;
+        if constexpr (Q8V) {
+            st.k = *reinterpret_cast<const v4u*>(kp + (size_t)tid * 16);
+            const uint8_t* blk = vp + v_row * kQ8vRow + v_blk * 36;
+            st.scale = *reinterpret_cast<const unsigned*>(blk);
+            st.c0 = *reinterpret_cast<const unsigned*>(blk + 4 + v_j * 8);
+            st.c1 = *reinterpret_cast<const unsigned*>(blk + 8 + v_j * 8);
+            st.pg = pg;
+        } else {
 #pragma unroll
-        for (int j = 0; j < kChunks; ++j) {
-            stage[j] = *reinterpret_cast<const v4u*>(kp + (size_t)(tid + j * kThreads) * 16);
-            stage[kChunks + j] = *reinterpret_cast<const v4u*>(vp + (size_t)(tid + j * kThreads) * 16);
+            for (int j = 0; j < 2; ++j) {
+                st.k[j] = *reinterpret_cast<const v4u*>(kp + (size_t)(tid + j * kThreads) * 16);
+                st.v[j] = *reinterpret_cast<const v4u*>(vp + (size_t)(tid + j * kThreads) * 16);
+            }
         }
     };
-    const auto deposit = [&](int buf, const v4u (&stage)[2 * kChunks]) {
+    const auto deposit = [&](int buf, const PageStage<Q8V>& st) {
         // chunk q of a page image: row q / 32, halves (q % 32) * 8 ..
+        if constexpr (Q8V) {
+            *reinterpret_cast<v4u*>(&L.img[buf][0][tid >> 5][(tid & 31) * 8]) = st.k;
+            // Rows past the work-group's last position were never written for these queries and
+            // may hold anything: scale 1 for the row's exponent, zeros for its values.
+            const bool dead = st.pg * kPage + v_row > wg_pos_max;
+            const float sc = __builtin_bit_cast(float, st.scale);
+            // the largest scale of the row: over the lanes that differ in the block bits (2..4)
+            float smax = dead ? 1.0f : sc;
+            smax = fmaxf(smax, dpp_mov<0x124>(smax));  // row_ror:4
+            smax = fmaxf(smax, dpp_mov<0x128>(smax));  // row_ror:8
+            {
+                const LanePair o = swap_rows(smax);
+                smax = fmaxf(o.a, o.b);
+            }
+            int ee = (int)((__builtin_bit_cast(unsigned, smax) >> 23) & 0xffu) - 127;
+            ee = min(max(ee, -120), 120);
+            const float down = __builtin_bit_cast(float, (unsigned)(127 - ee) << 23);  // 2^-E
+            _Float16 s_hi, s_lo;
+            split_f16(dead ? 0.0f : sc * down, s_hi, s_lo);
+            const h2m sh = h2m{s_hi, s_hi}, sl = h2m{s_lo, s_lo};
+            h2m cd[4], hi[4], lo[4];
+            codes_to_f16(st.c0, cd[0], cd[1]);
+            codes_to_f16(st.c1, cd[2], cd[3]);
 #pragma unroll
-        for (int j = 0; j < kChunks; ++j) {
-            const int q = tid + j * kThreads;
-            *reinterpret_cast<v4u*>(&lds[buf][0][q >> 5][(q & 31) * 8]) = stage[j];
-            *reinterpret_cast<v4u*>(&lds[buf][1][q >> 5][(q & 31) * 8]) = stage[kChunks + j];
+            for (int i = 0; i < 4; ++i) scaled_hi_lo(cd[i], sh, sl, hi[i], lo[i]);
+            const h8 vh = h8{hi[0][0], hi[0][1], hi[1][0], hi[1][1], hi[2][0], hi[2][1], hi[3][0], hi[3][1]};
+            const h8 vl = h8{lo[0][0], lo[0][1], lo[1][0], lo[1][1], lo[2][0], lo[2][1], lo[3][0], lo[3][1]};
+            *reinterpret_cast<h8*>(&L.img[buf][1][v_row][v_blk * 32 + v_j * 8]) = vh;
+            *reinterpret_cast<h8*>(&L.img[buf][2][v_row][v_blk * 32 + v_j * 8]) = vl;
+            if ((tid & 31) == 0) L.e[buf][v_row] = (float)ee;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int q = tid + j * kThreads;
+                *reinterpret_cast<v4u*>(&L.img[buf][0][q >> 5][(q & 31) * 8]) = st.k[j];
+                *reinterpret_cast<v4u*>(&L.img[buf][1][q >> 5][(q & 31) * 8]) = st.v[j];
+            }
         }
     };
 
     // scores of one page: s[r] = q[row c] . k[cell 4 g + r], masked and in base 2
     const auto scores = [&](int pg, int buf, float (&t4)[4]) {
-        const _Float16* ks = &lds[buf][0][0][0];
+        const _Float16* ks = &L.img[buf][0][0][0];
         // K: row c, 16 bytes at element 32 m + 8 g (the same split of the head dim as q): the 8
         // halves of a lane are the 8 contraction steps it feeds to the 32-deep MFMA
         h8 kf[8];
@@ -210,9 +288,24 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
 #pragma unroll
             for (int r = 0; r < 4; ++r) tb[r] = -INFINITY;
         }
+        // q8_0 V: the softmax runs over logit + E of the cell (wa, wb); dead cells stay at -inf
+        float wa[4], wb[4];
+        if constexpr (Q8V) {
+            const f4 ea = *reinterpret_cast<const f4*>(&L.e[buf][4 * g]);
+            f4 eb = f4{0.0f, 0.0f, 0.0f, 0.0f};
+            if (second) eb = *reinterpret_cast<const f4*>(&L.e[buf + 1][4 * g]);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                wa[r] = ta[r] + ea[r];
+                wb[r] = tb[r] + eb[r];
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) wa[r] = ta[r], wb[r] = tb[r];
+        }
 
         // ---- online softmax for this lane's query, over the pair's 32 cells ---------------------------
-        float pm = fmaxf(fmaxf(fmaxf(ta[0], ta[1]), fmaxf(ta[2], ta[3])), fmaxf(fmaxf(tb[0], tb[1]), fmaxf(tb[2], tb[3])));
+        float pm = fmaxf(fmaxf(fmaxf(wa[0], wa[1]), fmaxf(wa[2], wa[3])), fmaxf(fmaxf(wb[0], wb[1]), fmaxf(wb[2], wb[3])));
         pm = max_over_lane_groups(pm);
         const float m_new = fmaxf(m_run, pm);
         // a query with no live cell yet keeps m = -inf: exp2(-inf - -inf) would be NaN
@@ -222,9 +315,14 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
         float psum = 0.0f;
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
-            const float tt = r < 4 ? ta[r & 3] : tb[r & 3];
-            const float p = none_yet ? 0.0f : __builtin_amdgcn_exp2f(tt - m_new);
-            psum += p;
+            const float ww = r < 4 ? wa[r & 3] : wb[r & 3];
+            const float p = none_yet ? 0.0f : __builtin_amdgcn_exp2f(ww - m_new);
+            if constexpr (Q8V) {
+                const float tt = r < 4 ? ta[r & 3] : tb[r & 3];
+                psum += none_yet ? 0.0f : __builtin_amdgcn_exp2f(tt - m_new);
+            } else {
+                psum += p;
+            }
             _Float16 hi, lo;
             split_f16(p, hi, lo);
             ph[r] = hi;
@@ -246,41 +344,46 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
         // V: rows 4 g + r of either page, 16 bytes at element 128 half + 8 c.  Rows past the last
         // position of this wave were never written for these queries and may hold anything (even
         // NaN): they are made exact zeros before they meet a zero probability.
-        const _Float16* va_s = &lds[buf][1][0][0];
-        const _Float16* vb_s = &lds[buf + 1][1][0][0];
         const bool a_last = pg == n_pages - 1, b_last = pg + 1 == n_pages - 1;
+        // q8_0 V: the image of high parts meets p's high and low parts, the image of low parts p's
+        // high parts
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            v4u fa[4], fb[4];
+        for (int img = 1; img < (Q8V ? 3 : 2); ++img) {
+            const _Float16* va_s = &L.img[buf][img][0][0];
+            const _Float16* vb_s = &L.img[buf + 1][img][0][0];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                fa[r] = *reinterpret_cast<const v4u*>(va_s + (4 * g + r) * kLdsRow + h * 128 + c * 8);
-                fb[r] = *reinterpret_cast<const v4u*>(vb_s + (4 * g + r) * kLdsRow + h * 128 + c * 8);
-            }
-            if (a_last || b_last || !second) {
+            for (int h = 0; h < 2; ++h) {
+                v4u fa[4], fb[4];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    if (a_last && pg * kPage + 4 * g + r > pos_max) fa[r] = v4u{0u, 0u, 0u, 0u};
-                    if (!second || (b_last && (pg + 1) * kPage + 4 * g + r > pos_max)) fb[r] = v4u{0u, 0u, 0u, 0u};
+                    fa[r] = *reinterpret_cast<const v4u*>(va_s + (4 * g + r) * kLdsRow + h * 128 + c * 8);
+                    fb[r] = *reinterpret_cast<const v4u*>(vb_s + (4 * g + r) * kLdsRow + h * 128 + c * 8);
                 }
-            }
-            const h8 a0 = __builtin_bit_cast(h8, fa[0]), a1 = __builtin_bit_cast(h8, fa[1]);
-            const h8 a2 = __builtin_bit_cast(h8, fa[2]), a3 = __builtin_bit_cast(h8, fa[3]);
-            const h8 b0 = __builtin_bit_cast(h8, fb[0]), b1 = __builtin_bit_cast(h8, fb[1]);
-            const h8 b2 = __builtin_bit_cast(h8, fb[2]), b3 = __builtin_bit_cast(h8, fb[3]);
+                if (a_last || b_last || !second) {
 #pragma unroll
-            for (int t = 0; t < 8; ++t) {
-                // column 128 h + 8 c + t of the pair's cells 4 g .. of either page
-                const h8 vv = h8{a0[t], a1[t], a2[t], a3[t], b0[t], b1[t], b2[t], b3[t]};
-                o[h][t] = mfma32(vv, ph, o[h][t]);
-                o[h][t] = mfma32(vv, pl, o[h][t]);
+                    for (int r = 0; r < 4; ++r) {
+                        if (a_last && pg * kPage + 4 * g + r > pos_max) fa[r] = v4u{0u, 0u, 0u, 0u};
+                        if (!second || (b_last && (pg + 1) * kPage + 4 * g + r > pos_max)) fb[r] = v4u{0u, 0u, 0u, 0u};
+                    }
+                }
+                const h8 a0 = __builtin_bit_cast(h8, fa[0]), a1 = __builtin_bit_cast(h8, fa[1]);
+                const h8 a2 = __builtin_bit_cast(h8, fa[2]), a3 = __builtin_bit_cast(h8, fa[3]);
+                const h8 b0 = __builtin_bit_cast(h8, fb[0]), b1 = __builtin_bit_cast(h8, fb[1]);
+                const h8 b2 = __builtin_bit_cast(h8, fb[2]), b3 = __builtin_bit_cast(h8, fb[3]);
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    // column 128 h + 8 c + t of the pair's cells 4 g .. of either page
+                    const h8 vv = h8{a0[t], a1[t], a2[t], a3[t], b0[t], b1[t], b2[t], b3[t]};
+                    o[h][t] = mfma32(vv, ph, o[h][t]);
+                    if (img == 1) o[h][t] = mfma32(vv, pl, o[h][t]);
+                }
             }
         }
     };
 
     // Two pairs are in flight behind the one being multiplied: one in the other two LDS buffers,
     // one in the staging registers (past the end they carry the last page again).
-    v4u stage_a[2 * kChunks], stage_b[2 * kChunks];
+    PageStage<Q8V> stage_a, stage_b;
     const int last_pg = wg_pages - 1;
     fetch(0, stage_a);
     fetch(min(1, last_pg), stage_b);
@@ -337,7 +440,7 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
 
 }  // namespace
 
-int32_t prefill_rows_per_wg() { return kRowsPerWg; }
+int32_t prefill_rows_per_wg(int32_t layout) { return kRowsPerWave * (layout == BKV_LAYOUT_Q8V ? 8 : 4); }
 
 hipError_t launch_prefill_attn(bkv_pool* p, int32_t layer, const PrefillBatch& b, const AttnArgs& a,
                                hipStream_t stream) {
@@ -359,7 +462,10 @@ hipError_t launch_prefill_attn(bkv_pool* p, int32_t layer, const PrefillBatch& b
     const int32_t grid = b.wg_base[b.n];
     if (grid == 0) return hipSuccess;
     StageScope timed(p, BKV_STAGE_ATTN_SPLIT, stream);
-    prefill_attn_kernel<<<grid, kThreads, 0, stream>>>(kp);
+    if (p->g.layout == BKV_LAYOUT_Q8V)
+        prefill_attn_kernel<true><<<grid, 512, 0, stream>>>(kp);
+    else
+        prefill_attn_kernel<false><<<grid, 256, 0, stream>>>(kp);
     return hipGetLastError();
 }
 

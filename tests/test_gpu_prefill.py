@@ -37,12 +37,13 @@ def prefill(tw, layer, seqs, pos0, q_list, n_head, gate_list=None):
     return outs
 
 
+@pytest.mark.parametrize("layout", [L.LAYOUT_F16, L.LAYOUT_Q8V])
 @pytest.mark.parametrize("n_q", [16, 24])
-def test_chunks_match_the_oracle_token_by_token(n_q):
+def test_chunks_match_the_oracle_token_by_token(n_q, layout):
     rng = np.random.Generator(np.random.PCG64(1000 + n_q))
     # (cells before the chunk, chunk length): from scratch, on a prefix, single token, page edges
     cases = [(0, 100), (517, 300), (64, 1), (15, 17), (2048, 130)]
-    with Twin(n_pages=400, max_seqs=8) as tw:
+    with Twin(n_pages=400, max_seqs=8, layout=layout) as tw:
         tw.pool.set_free_order(rng.permutation(400).astype(np.int32))
         seqs = [tw.pool.seq_create() for _ in cases]
         for s, (before, t) in zip(seqs, cases):
@@ -64,6 +65,54 @@ def test_chunks_match_the_oracle_token_by_token(n_q):
         pos = list(range(before + t - 40, before + t))
         dec = tw.decode_attn(0, [s] * 40, pos, qs[1][-40:], n_q, scale=1.0 / 16.0, gate=gates[1][-40:])
         assert max_abs(dec, outs[1][-40:]) < 5e-6
+
+
+@pytest.mark.parametrize("v_mag", [1.2e-2, 1.0, 900.0])
+def test_q8v_chunks_across_the_scale_range(v_mag):
+    # q8_0 V with block scales from near 2^-14 up to 7, blocks of one row and rows of one page on
+    # different scales: the result stays at the reference's bar relative to the largest output
+    rng = np.random.Generator(np.random.PCG64(1020))
+    with Twin(n_pages=80, max_seqs=2, layout=L.LAYOUT_Q8V) as tw:
+        s = tw.pool.seq_create()
+        n = 1203
+        tw.pool.seq_reserve(s, n)
+        k = rng.standard_normal((n, 2, 256)).astype(np.float32)
+        v = (rng.standard_normal((n, 2, 256)) * v_mag).astype(np.float32)
+        v[:, :, 64:96] *= 0.37
+        v[5::7] *= 0.11
+        v[40:60] *= 1.0e-3      # a page and a half of very quiet rows
+        tw.append(0, [s], [0], [k], [v])
+        q = rng.standard_normal((203, 16, 256)).astype(np.float32)
+        out = prefill(tw, 0, [s], [1000], [q], 16)[0]
+        for i in (0, 57, 101, 202):
+            want = tw.oracle_attend(0, s, 1000 + i, q[i], 16)
+            rel = max_abs(out[i], want) / float(np.max(np.abs(want)))
+            assert rel <= REF_BAR_MAX_REL, (i, rel)
+        # a short context made of the quiet rows and their neighbours only
+        q2 = rng.standard_normal((30, 16, 256)).astype(np.float32)
+        out2 = prefill(tw, 0, [s], [35], [q2], 16)[0]
+        for i in (0, 10, 29):
+            want = tw.oracle_attend(0, s, 35 + i, q2[i], 16)
+            rel = max_abs(out2[i], want) / float(np.max(np.abs(want)))
+            assert rel <= REF_BAR_MAX_REL, (i, rel)
+
+
+def test_q8v_prefill_ignores_poisoned_cells():
+    # every unwritten byte of the pools is 0xFF (NaN scales, NaN K): chunks that end inside a page
+    rng = np.random.Generator(np.random.PCG64(1021))
+    with Twin(n_pages=32, max_seqs=2, layout=L.LAYOUT_Q8V) as tw:
+        tw.pool.fill(0xFF)
+        for img in tw.images:
+            img.k[:] = 0xFF
+            img.v[:] = 0xFF
+        s = tw.pool.seq_create()
+        for n, t in ((1, 1), (17, 16), (40, 23), (200, 130), (203, 3)):
+            fill(tw, s, n, rng, chunk=64)
+            q = rng.standard_normal((t, 16, 256)).astype(np.float32)
+            out = prefill(tw, 0, [s], [n - t], [q], 16)[0]
+            assert np.all(np.isfinite(out))
+            for i in sorted({0, t // 2, t - 1}):
+                check_attn(out[i], tw.oracle_attend(0, s, n - t + i, q[i], 16), "len %d token %d" % (n, i))
 
 
 def test_prefill_ignores_poisoned_cells_and_future_tokens():
@@ -109,7 +158,7 @@ def test_prefill_errors_come_before_any_launch():
                 tw.pool.prefill_attn(**a)
             assert ei.value.status == status, kw
         z.free()
-    with Twin(n_pages=8, max_seqs=2, layout=L.LAYOUT_Q8V) as tw:
+    with Twin(n_pages=8, max_seqs=2, layout=L.LAYOUT_I8H) as tw:
         s = tw.pool.seq_create()
         tw.pool.seq_reserve(s, 40)
         z = DeviceBuffer(1 << 20)
