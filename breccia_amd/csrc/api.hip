@@ -812,9 +812,8 @@ bkv_status bkv_prefill_attn(bkv_pool* p, int32_t layer, int32_t n_seqs, const in
     if (n_q_head <= 0 || n_q_head % p->g.n_kv != 0)
         return fail(BKV_ERR_INVALID, sfmt("prefill_attn: %lld q heads over %lld kv heads (need a whole "
                                           "group)", n_q_head, p->g.n_kv));
-    if (p->g.layout == BKV_LAYOUT_I8H || p->g.hd != 256 || p->g.page_cells != 16)
-        return fail(BKV_ERR_INVALID, "prefill_attn is built for f16 K pools (f16 or q8_0 V) with head_dim "
-                                     "256 and 16-cell pages");
+    if (p->g.hd != 256 || p->g.page_cells != 16)
+        return fail(BKV_ERR_INVALID, "prefill_attn is built for head_dim 256 and 16-cell pages");
     if (n_seqs > 0 && (!seqs || !pos0 || !n_tokens))
         return fail(BKV_ERR_INVALID, "prefill_attn: NULL sequence / position / token-count array");
     PrefillBatch b{};

@@ -46,7 +46,8 @@ namespace {
 constexpr int kHd = 256;
 constexpr int kPage = 16;
 constexpr int kRowsPerWave = 16;
-constexpr int kQ8vRow = kHd / 32 * 36;              // bytes of a q8_0 row
+constexpr int kQ8vRow = kHd / 32 * 36;  // bytes of a q8_0 row
+constexpr int kI8hRow = kHd + kHd / 32 * 2;  // bytes of an int8 row: codes, then 8 f16 scales
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kLdsRow = kHd + 8;  // halves per row of a page image in LDS (528 bytes)
 
@@ -79,29 +80,41 @@ __device__ __forceinline__ void split_f16(float x, _Float16& hi, _Float16& lo) {
 }
 
 // What a thread carries of one page between its fetch and its deposit into LDS.
-template <bool Q8V>
+template <int LAY>
 struct PageStage;
 template <>
-struct PageStage<false> {
+struct PageStage<BKV_LAYOUT_F16> {
     v4u k[2], v[2];  // chunks tid and tid + 256 of either image
 };
+// the quantised layouts: thread tid owns row tid / 32, block tid / 4 % 8, codes 8 (tid % 4) .. + 7 of it
 template <>
-struct PageStage<true> {
-    v4u k;                   // chunk tid of the K image
-    unsigned scale, c0, c1;  // of V: row tid / 32, block tid / 4 % 8, codes 8 (tid % 4) .. + 7 of it
+struct PageStage<BKV_LAYOUT_Q8V> {
+    v4u k;                   // chunk tid of the f16 K image
+    unsigned scale, c0, c1;  // of V
+    int pg;
+};
+template <>
+struct PageStage<BKV_LAYOUT_I8H> {
+    unsigned kc0, kc1, vc0, vc1;
+    unsigned short kscale, vscale;
     int pg;
 };
 
-template <bool Q8V>
+template <int LAY>
 struct PrefillLds {
-    // [buffer][K | V (q8_0: high parts, low parts)][16 rows][264 halves]
-    _Float16 img[4][Q8V ? 3 : 2][kPage][kLdsRow];
-    float e[Q8V ? 4 : 1][kPage];  // q8_0: E of the buffer's cells
+    // [buffer][K | V (quantised V: high parts, low parts)][16 rows][264 halves]
+    _Float16 img[4][LAY == BKV_LAYOUT_F16 ? 2 : 3][kPage][kLdsRow];
+    float e[LAY == BKV_LAYOUT_Q8V ? 4 : 1][kPage];           // q8_0 V: E of the buffer's cells
+    _Float16 ksc[LAY == BKV_LAYOUT_I8H ? 4 : 1][8][kPage];   // int8 K: scale of [block][row]
 };
 
-template <bool Q8V>
-__global__ __launch_bounds__(Q8V ? 512 : 256, Q8V ? 1 : 2) void prefill_attn_kernel(const PrefillKernelParams P) {
-    constexpr int kWavesPerWg = Q8V ? 8 : 4;
+template <int LAY>
+__global__ __launch_bounds__(LAY == BKV_LAYOUT_F16 ? 256 : 512, LAY == BKV_LAYOUT_F16 ? 2 : 1) void prefill_attn_kernel(
+    const PrefillKernelParams P) {
+    constexpr bool Q8V = LAY == BKV_LAYOUT_Q8V;
+    constexpr bool I8H = LAY == BKV_LAYOUT_I8H;
+    constexpr bool WIDE = LAY != BKV_LAYOUT_F16;  // eight waves, V as two f16 images
+    constexpr int kWavesPerWg = WIDE ? 8 : 4;
     constexpr int kThreads = 64 * kWavesPerWg;
     constexpr int kRowsPerWg = kRowsPerWave * kWavesPerWg;
     // ---- which (entry, kv head, block of 64 query rows) ---------------------------------
@@ -138,10 +151,12 @@ __global__ __launch_bounds__(Q8V ? 512 : 256, Q8V ? 1 : 2) void prefill_attn_ker
 
     typedef const __attribute__((address_space(4))) int32_t* table_ptr;
     const table_ptr bt = (table_ptr)(uintptr_t)(P.tables + (size_t)P.b.row[e] * (size_t)P.max_pages_per_seq);
-    const size_t page_bytes = (size_t)P.n_kv * kPage * kHd * 2;
-    const size_t head_off = (size_t)kvh * kPage * kHd * 2;
-    const size_t v_page_bytes = Q8V ? (size_t)P.n_kv * kPage * kQ8vRow : page_bytes;
-    const size_t v_head_off = Q8V ? (size_t)kvh * kPage * kQ8vRow : head_off;
+    constexpr int kKRow = I8H ? kI8hRow : kHd * 2;  // bytes of a row in the K pool and in the V pool
+    constexpr int kVRow = I8H ? kI8hRow : Q8V ? kQ8vRow : kHd * 2;
+    const size_t page_bytes = (size_t)P.n_kv * kPage * kKRow;
+    const size_t head_off = (size_t)kvh * kPage * kKRow;
+    const size_t v_page_bytes = (size_t)P.n_kv * kPage * kVRow;
+    const size_t v_head_off = (size_t)kvh * kPage * kVRow;
 
     // ---- q fragments: lane (c, g) holds q[row][32 m + 8 g + 0..7], m = 0..7, as hi + lo f16 ----
     h8 qhi[8], qlo[8];
@@ -184,11 +199,11 @@ __global__ __launch_bounds__(Q8V ? 512 : 256, Q8V ? 1 : 2) void prefill_attn_ker
     // t (+ 256) of it.  Pages are taken two at a time (one softmax update, one
     // barrier and P.V MFMAs that contract over the 32 cells of the pair): four buffers, the pair
     // being multiplied and the pair being filled.
-    __shared__ __attribute__((aligned(16))) PrefillLds<Q8V> L;
+    __shared__ __attribute__((aligned(16))) PrefillLds<LAY> L;
     const int tid = threadIdx.x;
-    // q8_0 V: this thread's part of a page
+    // quantised layouts: this thread's part of a page
     const int v_row = tid >> 5, v_blk = (tid >> 2) & 7, v_j = tid & 3;
-    const auto fetch = [&](int pg, PageStage<Q8V>& st) {
+    const auto fetch = [&](int pg, PageStage<LAY>& st) {
         const int32_t phys = bt[pg];
         const uint8_t* kp = P.kpool + (size_t)phys * page_bytes + head_off;
         const uint8_t* vp = P.vpool + (size_t)phys * v_page_bytes + v_head_off;
@@ -199,6 +214,16 @@ __global__ __launch_bounds__(Q8V ? 512 : 256, Q8V ? 1 : 2) void prefill_attn_ker
             st.c0 = *reinterpret_cast<const unsigned*>(blk + 4 + v_j * 8);
             st.c1 = *reinterpret_cast<const unsigned*>(blk + 8 + v_j * 8);
             st.pg = pg;
+        } else if constexpr (I8H) {
+            const uint8_t* kr = kp + v_row * kI8hRow;
+            const uint8_t* vr = vp + v_row * kI8hRow;
+            st.kc0 = *reinterpret_cast<const unsigned*>(kr + v_blk * 32 + v_j * 8);
+            st.kc1 = *reinterpret_cast<const unsigned*>(kr + v_blk * 32 + v_j * 8 + 4);
+            st.vc0 = *reinterpret_cast<const unsigned*>(vr + v_blk * 32 + v_j * 8);
+            st.vc1 = *reinterpret_cast<const unsigned*>(vr + v_blk * 32 + v_j * 8 + 4);
+            st.kscale = *reinterpret_cast<const unsigned short*>(kr + kHd + v_blk * 2);
+            st.vscale = *reinterpret_cast<const unsigned short*>(vr + kHd + v_blk * 2);
+            st.pg = pg;
         } else {
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
@@ -207,7 +232,7 @@ __global__ __launch_bounds__(Q8V ? 512 : 256, Q8V ? 1 : 2) void prefill_attn_ker
             }
         }
     };
-    const auto deposit = [&](int buf, const PageStage<Q8V>& st) {
+    const auto deposit = [&](int buf, const PageStage<LAY>& st) {
         // chunk q of a page image: row q / 32, halves (q % 32) * 8 ..
         if constexpr (Q8V) {
             *reinterpret_cast<v4u*>(&L.img[buf][0][tid >> 5][(tid & 31) * 8]) = st.k;
@@ -239,6 +264,33 @@ __global__ __launch_bounds__(Q8V ? 512 : 256, Q8V ? 1 : 2) void prefill_attn_ker
             *reinterpret_cast<h8*>(&L.img[buf][1][v_row][v_blk * 32 + v_j * 8]) = vh;
             *reinterpret_cast<h8*>(&L.img[buf][2][v_row][v_blk * 32 + v_j * 8]) = vl;
             if ((tid & 31) == 0) L.e[buf][v_row] = (float)ee;
+        } else if constexpr (I8H) {
+            // K: the codes as the exact f16 numbers they are; their block scales apply to the
+            // blocks' partial scores.  A scale with exponent field 0 reads as zero, as everywhere.
+            h2m kd[4];
+            codes_to_f16(st.kc0, kd[0], kd[1]);
+            codes_to_f16(st.kc1, kd[2], kd[3]);
+            *reinterpret_cast<h8*>(&L.img[buf][0][v_row][v_blk * 32 + v_j * 8]) =
+                h8{kd[0][0], kd[0][1], kd[1][0], kd[1][1], kd[2][0], kd[2][1], kd[3][0], kd[3][1]};
+            if (v_j == 0) {
+                const unsigned short ks = (st.kscale & 0x7c00u) == 0 ? (unsigned short)0 : st.kscale;
+                L.ksc[buf][v_blk][v_row] = __builtin_bit_cast(_Float16, ks);
+            }
+            // V: code * scale (7 + 11 significant bits) as hi = f16(code * scale) and the exact
+            // remainder; rows past the work-group's last position become zeros
+            const bool dead = st.pg * kPage + v_row > wg_pos_max;
+            const unsigned short vs = (dead || (st.vscale & 0x7c00u) == 0) ? (unsigned short)0 : st.vscale;
+            const _Float16 vsc = __builtin_bit_cast(_Float16, vs);
+            const h2m sh = h2m{vsc, vsc}, sl = h2m{(_Float16)0.0f, (_Float16)0.0f};
+            h2m cd[4], hi[4], lo[4];
+            codes_to_f16(st.vc0, cd[0], cd[1]);
+            codes_to_f16(st.vc1, cd[2], cd[3]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) scaled_hi_lo(cd[i], sh, sl, hi[i], lo[i]);
+            *reinterpret_cast<h8*>(&L.img[buf][1][v_row][v_blk * 32 + v_j * 8]) =
+                h8{hi[0][0], hi[0][1], hi[1][0], hi[1][1], hi[2][0], hi[2][1], hi[3][0], hi[3][1]};
+            *reinterpret_cast<h8*>(&L.img[buf][2][v_row][v_blk * 32 + v_j * 8]) =
+                h8{lo[0][0], lo[0][1], lo[1][0], lo[1][1], lo[2][0], lo[2][1], lo[3][0], lo[3][1]};
         } else {
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
@@ -257,17 +309,35 @@ __global__ __launch_bounds__(Q8V ? 512 : 256, Q8V ? 1 : 2) void prefill_attn_ker
         h8 kf[8];
 #pragma unroll
         for (int m = 0; m < 8; ++m) kf[m] = *reinterpret_cast<const h8*>(ks + c * kLdsRow + m * 32 + g * 8);
-        // four independent accumulation chains: an MFMA that waits for the previous one's result
-        // costs its full latency
-        f4 s0 = f4{0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0, s2 = s0, s3 = s0;
+        f4 s;
+        if constexpr (I8H) {
+            // a 32-deep MFMA is exactly one block of 32 values: the block's scale of either cell
+            // multiplies its partial sum
+            s = f4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int m = 0; m < 8; m += 2) {
-            s0 = mfma32(kf[m], qhi[m], s0);
-            s1 = mfma32(kf[m], qlo[m], s1);
-            s2 = mfma32(kf[m + 1], qhi[m + 1], s2);
-            s3 = mfma32(kf[m + 1], qlo[m + 1], s3);
+            for (int m = 0; m < 8; ++m) {
+                const h4 ksr = *reinterpret_cast<const h4*>(&L.ksc[buf][m][4 * g]);
+                f4 part = mfma32(kf[m], qhi[m], f4{0.0f, 0.0f, 0.0f, 0.0f});
+                part = mfma32(kf[m], qlo[m], part);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) s[r] = fmaf((float)ksr[r], part[r], s[r]);
+                // four blocks' partial sums in flight are enough to hide the MFMA latency; all
+                // eight (of both pages of a pair) do not fit the register file
+                if (m == 3) __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+            // four independent accumulation chains: an MFMA that waits for the previous one's
+            // result costs its full latency
+            f4 s0 = f4{0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0, s2 = s0, s3 = s0;
+#pragma unroll
+            for (int m = 0; m < 8; m += 2) {
+                s0 = mfma32(kf[m], qhi[m], s0);
+                s1 = mfma32(kf[m], qlo[m], s1);
+                s2 = mfma32(kf[m + 1], qhi[m + 1], s2);
+                s3 = mfma32(kf[m + 1], qlo[m + 1], s3);
+            }
+            s = (s0 + s1) + (s2 + s3);
         }
-        const f4 s = (s0 + s1) + (s2 + s3);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int cell = pg * kPage + 4 * g + r;
@@ -345,10 +415,10 @@ __global__ __launch_bounds__(Q8V ? 512 : 256, Q8V ? 1 : 2) void prefill_attn_ker
         // position of this wave were never written for these queries and may hold anything (even
         // NaN): they are made exact zeros before they meet a zero probability.
         const bool a_last = pg == n_pages - 1, b_last = pg + 1 == n_pages - 1;
-        // q8_0 V: the image of high parts meets p's high and low parts, the image of low parts p's
-        // high parts
+        // quantised V: the image of high parts meets p's high and low parts, the image of low parts
+        // p's high parts
 #pragma unroll
-        for (int img = 1; img < (Q8V ? 3 : 2); ++img) {
+        for (int img = 1; img < (WIDE ? 3 : 2); ++img) {
             const _Float16* va_s = &L.img[buf][img][0][0];
             const _Float16* vb_s = &L.img[buf + 1][img][0][0];
 #pragma unroll
@@ -383,7 +453,7 @@ __global__ __launch_bounds__(Q8V ? 512 : 256, Q8V ? 1 : 2) void prefill_attn_ker
 
     // Two pairs are in flight behind the one being multiplied: one in the other two LDS buffers,
     // one in the staging registers (past the end they carry the last page again).
-    PageStage<Q8V> stage_a, stage_b;
+    PageStage<LAY> stage_a, stage_b;
     const int last_pg = wg_pages - 1;
     fetch(0, stage_a);
     fetch(min(1, last_pg), stage_b);
@@ -440,7 +510,7 @@ __global__ __launch_bounds__(Q8V ? 512 : 256, Q8V ? 1 : 2) void prefill_attn_ker
 
 }  // namespace
 
-int32_t prefill_rows_per_wg(int32_t layout) { return kRowsPerWave * (layout == BKV_LAYOUT_Q8V ? 8 : 4); }
+int32_t prefill_rows_per_wg(int32_t layout) { return kRowsPerWave * (layout == BKV_LAYOUT_F16 ? 4 : 8); }
 
 hipError_t launch_prefill_attn(bkv_pool* p, int32_t layer, const PrefillBatch& b, const AttnArgs& a,
                                hipStream_t stream) {
@@ -463,9 +533,11 @@ hipError_t launch_prefill_attn(bkv_pool* p, int32_t layer, const PrefillBatch& b
     if (grid == 0) return hipSuccess;
     StageScope timed(p, BKV_STAGE_ATTN_SPLIT, stream);
     if (p->g.layout == BKV_LAYOUT_Q8V)
-        prefill_attn_kernel<true><<<grid, 512, 0, stream>>>(kp);
+        prefill_attn_kernel<BKV_LAYOUT_Q8V><<<grid, 512, 0, stream>>>(kp);
+    else if (p->g.layout == BKV_LAYOUT_I8H)
+        prefill_attn_kernel<BKV_LAYOUT_I8H><<<grid, 512, 0, stream>>>(kp);
     else
-        prefill_attn_kernel<false><<<grid, 256, 0, stream>>>(kp);
+        prefill_attn_kernel<BKV_LAYOUT_F16><<<grid, 256, 0, stream>>>(kp);
     return hipGetLastError();
 }
 

@@ -37,7 +37,7 @@ def prefill(tw, layer, seqs, pos0, q_list, n_head, gate_list=None):
     return outs
 
 
-@pytest.mark.parametrize("layout", [L.LAYOUT_F16, L.LAYOUT_Q8V])
+@pytest.mark.parametrize("layout", [L.LAYOUT_F16, L.LAYOUT_Q8V, L.LAYOUT_I8H])
 @pytest.mark.parametrize("n_q", [16, 24])
 def test_chunks_match_the_oracle_token_by_token(n_q, layout):
     rng = np.random.Generator(np.random.PCG64(1000 + n_q))
@@ -67,12 +67,15 @@ def test_chunks_match_the_oracle_token_by_token(n_q, layout):
         assert max_abs(dec, outs[1][-40:]) < 5e-6
 
 
+@pytest.mark.parametrize("layout", [L.LAYOUT_Q8V, L.LAYOUT_I8H])
 @pytest.mark.parametrize("v_mag", [1.2e-2, 1.0, 900.0])
-def test_q8v_chunks_across_the_scale_range(v_mag):
-    # q8_0 V with block scales from near 2^-14 up to 7, blocks of one row and rows of one page on
-    # different scales: the result stays at the reference's bar relative to the largest output
+def test_quantised_chunks_across_the_scale_range(v_mag, layout):
+    # quantised V with block scales from near 2^-14 up to 7, blocks of one row and rows of one page
+    # on different scales (the quietest rows of the int8 layout have scales below 2^-14, which pool
+    # and oracle alike read as zero): the result stays at the reference's bar relative to the
+    # largest output
     rng = np.random.Generator(np.random.PCG64(1020))
-    with Twin(n_pages=80, max_seqs=2, layout=L.LAYOUT_Q8V) as tw:
+    with Twin(n_pages=80, max_seqs=2, layout=layout) as tw:
         s = tw.pool.seq_create()
         n = 1203
         tw.pool.seq_reserve(s, n)
@@ -97,10 +100,11 @@ def test_q8v_chunks_across_the_scale_range(v_mag):
             assert rel <= REF_BAR_MAX_REL, (i, rel)
 
 
-def test_q8v_prefill_ignores_poisoned_cells():
+@pytest.mark.parametrize("layout", [L.LAYOUT_Q8V, L.LAYOUT_I8H])
+def test_quantised_prefill_ignores_poisoned_cells(layout):
     # every unwritten byte of the pools is 0xFF (NaN scales, NaN K): chunks that end inside a page
     rng = np.random.Generator(np.random.PCG64(1021))
-    with Twin(n_pages=32, max_seqs=2, layout=L.LAYOUT_Q8V) as tw:
+    with Twin(n_pages=32, max_seqs=2, layout=layout) as tw:
         tw.pool.fill(0xFF)
         for img in tw.images:
             img.k[:] = 0xFF
@@ -157,12 +161,4 @@ def test_prefill_errors_come_before_any_launch():
             with pytest.raises(BkvError) as ei:
                 tw.pool.prefill_attn(**a)
             assert ei.value.status == status, kw
-        z.free()
-    with Twin(n_pages=8, max_seqs=2, layout=L.LAYOUT_I8H) as tw:
-        s = tw.pool.seq_create()
-        tw.pool.seq_reserve(s, 40)
-        z = DeviceBuffer(1 << 20)
-        with pytest.raises(BkvError) as ei:
-            tw.pool.prefill_attn(0, [s], [0], [40], 16, z, z, 0.0625)
-        assert ei.value.status == L.ERR_INVALID
         z.free()
