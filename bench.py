@@ -515,46 +515,51 @@ def bench_select(stream) -> dict:
 
 def bench_prefill(stream) -> dict:
     """BASELINE configs[3] shape on the MFMA prefill kernel: 4 sequences, 2048-token prefix in the
-    cache, a 1024-token chunk each (appended, then attended causally), 16 q / 2 kv heads."""
+    cache, a 1024-token chunk each (appended, then attended causally), 16 q / 2 kv heads; on the
+    f16 pool and on the two quantised layouts."""
+    from breccia_amd import lib as L
     from breccia_amd.kv import DeviceBuffer, Event, Pool
 
     rng = np.random.Generator(np.random.PCG64(20250007))
     n_seq, before, T = 4, 2048, 1024
-    pool = Pool(n_pages=n_seq * ((before + T) // PAGE + 2), max_seqs=n_seq + 1,
-                max_pages_per_seq=(before + T) // PAGE + 2)
-    seqs = [pool.seq_create() for _ in range(n_seq)]
     kd = DeviceBuffer.from_numpy(rng.standard_normal((before + T, N_KV, HD), dtype=np.float32))
     vd = DeviceBuffer.from_numpy(rng.standard_normal((before + T, N_KV, HD), dtype=np.float32))
-    for s in seqs:
-        pool.seq_reserve(s, before + T)
-        pool.append(0, [s], [0], [before + T], kd, vd, stream)
     q = DeviceBuffer.from_numpy(rng.standard_normal((n_seq * T, N_Q, HD), dtype=np.float32))
     out = DeviceBuffer(n_seq * T * N_Q * HD * 4)
-
-    def run(n):
-        for _ in range(n):
-            pool.prefill_attn(0, seqs, [before] * n_seq, [T] * n_seq, N_Q, q, out, 1.0 / 16.0, stream=stream)
-
-    run(3)
-    stream.sync()
-    e0, e1 = Event(), Event()
-    e0.record(stream)
-    run(10)
-    e1.record(stream)
-    stream.sync()
-    us = e0.elapsed_ms(e1) / 10 * 1e3
-    e0.close()
-    e1.close()
     pairs = n_seq * N_Q * sum(before + t + 1 for t in range(T))      # (query row, cell) pairs
     flops = pairs * HD * 4                                           # q.k and p.v, 2 flop per multiply-add
-    res = {"prefill_attn": {"workload": "BASELINE configs[3] shape: 4 sequences, prefix 2048 + chunk 1024, 16q/2kv",
-                            "us": round(us, 1), "useful_TFLOPs": round(flops / us / 1e6, 1),
-                            "issued_TFLOPs": round(2 * flops / us / 1e6, 1),
-                            "frac_of_f16_mfma_peak": round(flops / us / 1e6 / 2500.0, 4),
-                            "note": "q and p enter the MFMAs as hi + lo f16, which doubles the issued work"}}
+    res = {}
+    for name, layout in (("prefill_attn", L.LAYOUT_F16), ("prefill_attn_q8v", L.LAYOUT_Q8V),
+                         ("prefill_attn_i8h", L.LAYOUT_I8H)):
+        pool = Pool(n_pages=n_seq * ((before + T) // PAGE + 2), max_seqs=n_seq + 1,
+                    max_pages_per_seq=(before + T) // PAGE + 2, layout=layout)
+        seqs = [pool.seq_create() for _ in range(n_seq)]
+        for s in seqs:
+            pool.seq_reserve(s, before + T)
+            pool.append(0, [s], [0], [before + T], kd, vd, stream)
+
+        def run(n):
+            for _ in range(n):
+                pool.prefill_attn(0, seqs, [before] * n_seq, [T] * n_seq, N_Q, q, out, 1.0 / 16.0, stream=stream)
+
+        run(3)
+        stream.sync()
+        e0, e1 = Event(), Event()
+        e0.record(stream)
+        run(10)
+        e1.record(stream)
+        stream.sync()
+        us = e0.elapsed_ms(e1) / 10 * 1e3
+        e0.close()
+        e1.close()
+        res[name] = {"workload": "BASELINE configs[3] shape: 4 sequences, prefix 2048 + chunk 1024, 16q/2kv",
+                     "us": round(us, 1), "useful_TFLOPs": round(flops / us / 1e6, 1),
+                     "frac_of_f16_mfma_peak": round(flops / us / 1e6 / 2500.0, 4)}
+        pool.destroy()
+    res["prefill_attn"]["issued_TFLOPs"] = round(2 * flops / res["prefill_attn"]["us"] / 1e6, 1)
+    res["prefill_attn"]["note"] = "q and p enter the MFMAs as hi + lo f16, which doubles the issued work"
     for b in (kd, vd, q, out):
         b.free()
-    pool.destroy()
     return res
 
 

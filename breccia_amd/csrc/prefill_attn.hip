@@ -321,9 +321,6 @@ __global__ __launch_bounds__(LAY == BKV_LAYOUT_F16 ? 256 : 512, LAY == BKV_LAYOU
                 part = mfma32(kf[m], qlo[m], part);
 #pragma unroll
                 for (int r = 0; r < 4; ++r) s[r] = fmaf((float)ksr[r], part[r], s[r]);
-                // four blocks' partial sums in flight are enough to hide the MFMA latency; all
-                // eight (of both pages of a pair) do not fit the register file
-                if (m == 3) __builtin_amdgcn_sched_barrier(0);
             }
         } else {
             // four independent accumulation chains: an MFMA that waits for the previous one's
