@@ -3,6 +3,8 @@
 // host swap, a dequantising row gather for parity checks, and small utilities.
 // All of it is HBM-bound; the rules that matter are 16-byte accesses, whole-line
 // coalescing and several independent loads in flight per lane.
+#include <type_traits>
+
 #include "bkv_internal.hpp"
 #include "f16_rule.hpp"
 #include "quant_encode.hpp"
@@ -54,6 +56,23 @@ __device__ __forceinline__ void load8(const uint16_t* p, float (&x)[8]) {
     }
 }
 
+// Which token of the sequence and which lane of that token a thread of a one-dimensional launch
+// is: 32-bit division wherever the launch is small enough for it (a 64-bit one costs some 100
+// instructions, as much as the rest of an append lane's work).
+struct UnitOfToken {
+    int64_t t;
+    int r;
+};
+__device__ __forceinline__ UnitOfToken unit_of_token(int lanes_per_tok) {
+    if ((uint64_t)gridDim.x * kBlock < (1ull << 32)) {
+        const unsigned unit = blockIdx.x * kBlock + threadIdx.x;
+        const unsigned t = unit / (unsigned)lanes_per_tok;
+        return UnitOfToken{(int64_t)t, (int)(unit - t * (unsigned)lanes_per_tok)};
+    }
+    const int64_t unit = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    return UnitOfToken{unit / lanes_per_tok, (int)(unit % lanes_per_tok)};
+}
+
 // ---- append, f16 rows ---------------------------------------------------------
 // One lane converts 8 consecutive elements of one (token, kv head) row of K and of V:
 // two 16-byte loads and one 16-byte store per pool.  grid.y = sequence of the call.
@@ -66,16 +85,17 @@ __global__ __launch_bounds__(kBlock) void append_f16_kernel(AppendBatch b, MoveG
                                                             const SrcT* __restrict__ v) {
     const int s = blockIdx.y;
     const int lanes_per_tok = g.n_kv * g.hd / 8;
-    const int64_t unit = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    const int64_t t = unit / lanes_per_tok;
+    const UnitOfToken u = unit_of_token(lanes_per_tok);
+    const int64_t t = u.t;
     if (t >= b.n_tok[s]) return;
-    const int r = (int)(unit % lanes_per_tok);  // 8-element group within [n_kv][hd]
+    const int r = u.r;  // 8-element group within [n_kv][hd]
     const int kvh = (r * 8) / g.hd;
     const int d0 = (r * 8) % g.hd;
-    const int64_t cell = (int64_t)b.pos0[s] + t;
+    // cells are below 2^31 (pos0 and the token count are int32 and their sum is checked on the host)
+    const unsigned cell = (unsigned)b.pos0[s] + (unsigned)t;
     const int32_t phys =
-        tables[(size_t)b.row[s] * (size_t)g.max_pages_per_seq + (size_t)(cell / g.page_cells)];
-    const int in_page = (int)(cell % g.page_cells);
+        tables[(size_t)b.row[s] * (size_t)g.max_pages_per_seq + (size_t)(cell / (unsigned)g.page_cells)];
+    const int in_page = (int)(cell % (unsigned)g.page_cells);
     const size_t row = ((size_t)phys * g.n_kv + kvh) * g.page_cells + in_page;
     const size_t dst = row * (size_t)g.hd + d0;
     const size_t src = ((size_t)b.src0[s] + (size_t)t) * (size_t)(g.n_kv * g.hd) + (size_t)r * 8;
@@ -127,16 +147,16 @@ __global__ __launch_bounds__(kBlock) void append_q8v_kernel(AppendBatch b, MoveG
     const int s = blockIdx.y;
     const int blocks = g.hd / 32;
     const int lanes_per_tok = g.n_kv * blocks;
-    const int64_t unit = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    const int64_t t = unit / lanes_per_tok;
+    const UnitOfToken u = unit_of_token(lanes_per_tok);
+    const int64_t t = u.t;
     if (t >= b.n_tok[s]) return;
-    const int r = (int)(unit % lanes_per_tok);
+    const int r = u.r;
     const int kvh = r / blocks;
     const int blk = r % blocks;
-    const int64_t cell = (int64_t)b.pos0[s] + t;
+    const unsigned cell = (unsigned)b.pos0[s] + (unsigned)t;
     const int32_t phys =
-        tables[(size_t)b.row[s] * (size_t)g.max_pages_per_seq + (size_t)(cell / g.page_cells)];
-    const int in_page = (int)(cell % g.page_cells);
+        tables[(size_t)b.row[s] * (size_t)g.max_pages_per_seq + (size_t)(cell / (unsigned)g.page_cells)];
+    const int in_page = (int)(cell % (unsigned)g.page_cells);
     const size_t row = ((size_t)phys * g.n_kv + kvh) * g.page_cells + in_page;
     const size_t src = ((size_t)b.src0[s] + (size_t)t) * (size_t)(g.n_kv * g.hd) +
                        (size_t)kvh * g.hd + (size_t)blk * 32;
@@ -185,18 +205,18 @@ __global__ __launch_bounds__(kBlock) void append_i8h_kernel(AppendBatch b, MoveG
     const int s = blockIdx.y;
     const int blocks = g.hd / 32;
     const int lanes_per_tok = g.n_kv * blocks * 2;  // K and V blocks
-    const int64_t unit = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    const int64_t t = unit / lanes_per_tok;
+    const UnitOfToken u = unit_of_token(lanes_per_tok);
+    const int64_t t = u.t;
     if (t >= b.n_tok[s]) return;
-    int r = (int)(unit % lanes_per_tok);
+    int r = u.r;
     const int which = r / (g.n_kv * blocks);
     r %= g.n_kv * blocks;
     const int kvh = r / blocks;
     const int blk = r % blocks;
-    const int64_t cell = (int64_t)b.pos0[s] + t;
+    const unsigned cell = (unsigned)b.pos0[s] + (unsigned)t;
     const int32_t phys =
-        tables[(size_t)b.row[s] * (size_t)g.max_pages_per_seq + (size_t)(cell / g.page_cells)];
-    const int in_page = (int)(cell % g.page_cells);
+        tables[(size_t)b.row[s] * (size_t)g.max_pages_per_seq + (size_t)(cell / (unsigned)g.page_cells)];
+    const int in_page = (int)(cell % (unsigned)g.page_cells);
     const size_t row = ((size_t)phys * g.n_kv + kvh) * g.page_cells + in_page;
     const size_t src = ((size_t)b.src0[s] + (size_t)t) * (size_t)(g.n_kv * g.hd) +
                        (size_t)kvh * g.hd + (size_t)blk * 32;
@@ -224,12 +244,19 @@ struct KPrepParams {
 
 constexpr int kPrepRows = 16;  // (token, kv head) rows per work-group
 
+// The sum stays in element order (the reference's f64 loop, ops/cpu.rs:52-66); the row is read
+// 16 bytes at a time and several reads ahead, so that the chain of additions is all a lane waits for.
 __device__ __forceinline__ double row_sum_squares(const float* row, int n) {
 #pragma clang fp contract(off)
     double ss = 0.0;
-    for (int i = 0; i < n; ++i) {
-        const double v = (double)row[i];
-        ss += v * v;
+#pragma unroll 8
+    for (int i = 0; i < n; i += 4) {
+        const float4 x = *reinterpret_cast<const float4*>(row + i);
+        const double a = (double)x.x, b = (double)x.y, c = (double)x.z, d = (double)x.w;
+        ss += a * a;
+        ss += b * b;
+        ss += c * c;
+        ss += d * d;
     }
     return ss;
 }
@@ -242,7 +269,9 @@ __device__ __forceinline__ void rotate_pair(float& lo, float& hi, float c32, flo
     hi = (float)(as + bc);
 }
 
-template <int LAYOUT>
+// HD: the head dim as a compile-time constant (the index arithmetic of every loop divides by it),
+// or 0 for the value in the geometry.
+template <int LAYOUT, int HD>
 __global__ __launch_bounds__(kBlock) void append_kprep_kernel(AppendBatch b, MoveGeom g,
                                                               KPrepParams kp,
                                                               uint8_t* __restrict__ kpool,
@@ -250,15 +279,18 @@ __global__ __launch_bounds__(kBlock) void append_kprep_kernel(AppendBatch b, Mov
                                                               const int32_t* __restrict__ tables,
                                                               const float* __restrict__ k,
                                                               const float* __restrict__ v) {
-    extern __shared__ float prep_lds[];  // [kPrepRows][hd + 1] floats, then kPrepRows doubles
+    // [kPrepRows][hd + 4] floats, then per row: 1/rms, pool row, rotary position
+    extern __shared__ __attribute__((aligned(16))) float prep_lds[];
     const int s = blockIdx.y;
-    const int hd = g.hd;
-    const int stride = hd + 1;  // odd stride: the per-row serial sums do not collide on banks
+    const int hd = HD ? HD : g.hd;
+    // rows 16-byte aligned and 4 floats apart in the banks: the 16 lanes that sum a row each read
+    // 16 bytes of their own row per step without colliding
+    const int stride = hd + 4;
     const int rows_total = b.n_tok[s] * g.n_kv;
     const int r0 = (int)blockIdx.x * kPrepRows;
     if (r0 >= rows_total) return;
     const int nrows = min(kPrepRows, rows_total - r0);
-    double* inv_s = reinterpret_cast<double*>(prep_lds + ((kPrepRows * stride + 1) & ~1));
+    double* inv_s = reinterpret_cast<double*>(prep_lds + kPrepRows * stride);
     const size_t src_base = ((size_t)b.src0[s] * g.n_kv + (size_t)r0) * (size_t)hd;
     const int tid = threadIdx.x;
 
@@ -266,16 +298,26 @@ __global__ __launch_bounds__(kBlock) void append_kprep_kernel(AppendBatch b, Mov
     for (int idx = tid; idx < nrows * hd / 4; idx += kBlock) {
         const v4u w = ld_stream(k + src_base + (size_t)idx * 4);
         const int row = (idx * 4) / hd, col = (idx * 4) % hd;
-        float* d = prep_lds + row * stride + col;
-        d[0] = __uint_as_float(w.x);
-        d[1] = __uint_as_float(w.y);
-        d[2] = __uint_as_float(w.z);
-        d[3] = __uint_as_float(w.w);
+        *reinterpret_cast<v4u*>(prep_lds + row * stride + col) = w;
     }
     __syncthreads();
+    // While the first lanes sum their rows, a second wave works out where the rows go: the pool row
+    // of (sequence row r) = (token, kv head) and the token's rotary position.
+    uint64_t* const row_s = reinterpret_cast<uint64_t*>(inv_s + kPrepRows);
+    int32_t* const pos_s = reinterpret_cast<int32_t*>(row_s + kPrepRows);
     if (tid < nrows) {
         const double ss = row_sum_squares(prep_lds + tid * stride, hd);
         inv_s[tid] = 1.0 / sqrt(ss / (double)hd + (double)kp.eps);
+    } else if (tid >= 64 && tid - 64 < nrows) {
+        const unsigned r = (unsigned)(r0 + tid - 64);
+        const unsigned cell = (unsigned)b.pos0[s] + r / (unsigned)g.n_kv;
+        const unsigned kvh = r % (unsigned)g.n_kv;
+        const int32_t phys = tables[(size_t)b.row[s] * (size_t)g.max_pages_per_seq +
+                                    (size_t)(cell / (unsigned)g.page_cells)];
+        row_s[tid - 64] = ((uint64_t)phys * g.n_kv + kvh) * g.page_cells + (uint64_t)(cell % (unsigned)g.page_cells);
+        int64_t pos = kp.positions ? (int64_t)kp.positions[cell] : (int64_t)cell;
+        pos = pos < 0 ? 0 : (pos > kp.max_pos - 1 ? kp.max_pos - 1 : pos);
+        pos_s[tid - 64] = (int32_t)pos;
     }
     __syncthreads();
     for (int idx = tid; idx < nrows * hd; idx += kBlock) {
@@ -287,24 +329,13 @@ __global__ __launch_bounds__(kBlock) void append_kprep_kernel(AppendBatch b, Mov
     const int half = kp.n_rot / 2;
     for (int idx = tid; idx < nrows * half; idx += kBlock) {
         const int row = idx / half, j = idx % half;
-        const int64_t cell = (int64_t)b.pos0[s] + (r0 + row) / g.n_kv;
-        int64_t pos = kp.positions ? (int64_t)kp.positions[cell] : cell;
-        pos = pos < 0 ? 0 : (pos > kp.max_pos - 1 ? kp.max_pos - 1 : pos);
-        const float2 cs = reinterpret_cast<const float2*>(kp.table)[(size_t)pos * half + j];
+        const float2 cs = reinterpret_cast<const float2*>(kp.table)[(size_t)pos_s[row] * half + j];
         float* d = prep_lds + row * stride;
         rotate_pair(d[j], d[j + half], cs.x, cs.y);
     }
     __syncthreads();
 
-    // pool row of (sequence row r) = (token, kv head)
-    const auto pool_row = [&](int row) -> size_t {
-        const int r = r0 + row;
-        const int64_t cell = (int64_t)b.pos0[s] + r / g.n_kv;
-        const int kvh = r % g.n_kv;
-        const int32_t phys = tables[(size_t)b.row[s] * (size_t)g.max_pages_per_seq +
-                                    (size_t)(cell / g.page_cells)];
-        return ((size_t)phys * g.n_kv + kvh) * g.page_cells + (size_t)(cell % g.page_cells);
-    };
+    const auto pool_row = [&](int row) -> size_t { return (size_t)row_s[row]; };
     const int blocks = hd / 32;
 
     // K from LDS
@@ -600,22 +631,29 @@ hipError_t launch_append_kprep(const bkv_pool* p, int32_t layer, const AppendBat
     const KPrepParams kp{gamma, table, positions, eps, n_rot, max_pos};
     const int rows = max_tok * g.n_kv;
     dim3 grid((unsigned)((rows + kPrepRows - 1) / kPrepRows), (unsigned)b.n);
-    const size_t lds = (size_t)((kPrepRows * (g.hd + 1) + 1) & ~1) * sizeof(float) +
-                       kPrepRows * sizeof(double);
+    const size_t lds = (size_t)kPrepRows * (g.hd + 4) * sizeof(float) +
+                       kPrepRows * (sizeof(double) + sizeof(uint64_t) + sizeof(int32_t));
     uint8_t* kpl = p->k_layer[(size_t)layer];
     uint8_t* vpl = p->v_layer[(size_t)layer];
+    const auto launch = [&](auto layout_tag, auto hd_tag) {
+        append_kprep_kernel<decltype(layout_tag)::value, decltype(hd_tag)::value>
+            <<<grid, kBlock, lds, stream>>>(b, g, kp, kpl, vpl, p->table_dev, k, v);
+    };
+    const auto by_hd = [&](auto layout_tag) {
+        if (g.hd == 256)
+            launch(layout_tag, std::integral_constant<int, 256>{});
+        else
+            launch(layout_tag, std::integral_constant<int, 0>{});
+    };
     switch (p->g.layout) {
         case BKV_LAYOUT_F16:
-            append_kprep_kernel<BKV_LAYOUT_F16><<<grid, kBlock, lds, stream>>>(b, g, kp, kpl, vpl,
-                                                                              p->table_dev, k, v);
+            by_hd(std::integral_constant<int, BKV_LAYOUT_F16>{});
             break;
         case BKV_LAYOUT_Q8V:
-            append_kprep_kernel<BKV_LAYOUT_Q8V><<<grid, kBlock, lds, stream>>>(b, g, kp, kpl, vpl,
-                                                                              p->table_dev, k, v);
+            by_hd(std::integral_constant<int, BKV_LAYOUT_Q8V>{});
             break;
         default:
-            append_kprep_kernel<BKV_LAYOUT_I8H><<<grid, kBlock, lds, stream>>>(b, g, kp, kpl, vpl,
-                                                                              p->table_dev, k, v);
+            by_hd(std::integral_constant<int, BKV_LAYOUT_I8H>{});
             break;
     }
     return hipGetLastError();
