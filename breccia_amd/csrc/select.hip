@@ -41,21 +41,37 @@ struct ScoreParams {
 
 // score[b] = (1/sqrt(idx_dim)) * sum_h relu(q_h . pooled_b), -inf for a block that starts
 // after the query's position (qsa/cpu.rs:93-123).
+// DIM = 128: the indexer's usual width as a compile-time constant, rows moved and read 16 bytes
+// at a time (pooled and q must be 16-byte aligned); DIM = 0: any width, element by element (the
+// index arithmetic of its loops divides by the run-time width).  The products and the sum keep
+// the CPU's order in both.
+template <int DIM>
 __global__ __launch_bounds__(kScoreThreads) void idx_score_kernel(const ScoreParams P) {
-    __shared__ float pooled_s[kScoreTile * (kMaxIdxDim + 1)];
-    __shared__ float q_s[kMaxIdxHead * kMaxIdxDim];
+    // rows DIM + 4 (16-byte aligned, 4 banks apart: 16-byte reads of 64 rows do not collide) or
+    // D + 1 floats apart (odd: lanes walking one column of 64 rows hit 64 banks)
+    __shared__ __attribute__((aligned(16))) float pooled_s[kScoreTile * (kMaxIdxDim + 4)];
+    __shared__ __attribute__((aligned(16))) float q_s[kMaxIdxHead * kMaxIdxDim];
     __shared__ double part_s[kMaxIdxHead][kScoreTile];
     const int e = blockIdx.y;
     const int n_blocks = P.b.n_blocks[e];
     const int b0 = (int)blockIdx.x * kScoreTile;
     if (b0 >= n_blocks) return;
     const int nb = min(kScoreTile, n_blocks - b0);
-    const int D = P.idx_dim, H = P.idx_n_head;
-    const int stride = D + 1;  // odd: lanes walking one column of 64 rows hit 64 banks
+    const int D = DIM ? DIM : P.idx_dim, H = P.idx_n_head;
+    const int stride = DIM ? DIM + 4 : D + 1;
     const int tid = threadIdx.x;
     const float* pooled = P.b.pooled[e] + (size_t)b0 * D;
-    for (int i = tid; i < nb * D; i += kScoreThreads) pooled_s[(i / D) * stride + i % D] = pooled[i];
-    for (int i = tid; i < H * D; i += kScoreThreads) q_s[i] = P.q[(size_t)e * H * D + i];
+    if constexpr (DIM != 0) {
+        constexpr int kRow4 = DIM / 4;
+        for (int i = tid; i < nb * kRow4; i += kScoreThreads)
+            *reinterpret_cast<float4*>(&pooled_s[(i / kRow4) * stride + (i % kRow4) * 4]) =
+                reinterpret_cast<const float4*>(pooled)[i];
+        for (int i = tid; i < H * kRow4; i += kScoreThreads)
+            reinterpret_cast<float4*>(q_s)[i] = reinterpret_cast<const float4*>(P.q + (size_t)e * H * D)[i];
+    } else {
+        for (int i = tid; i < nb * D; i += kScoreThreads) pooled_s[(i / D) * stride + i % D] = pooled[i];
+        for (int i = tid; i < H * D; i += kScoreThreads) q_s[i] = P.q[(size_t)e * H * D + i];
+    }
     __syncthreads();
 
     const int b = tid % kScoreTile;
@@ -64,7 +80,19 @@ __global__ __launch_bounds__(kScoreThreads) void idx_score_kernel(const ScorePar
         const double scale = 1.0 / sqrt((double)D);
         for (int h = tid / kScoreTile; h < H; h += kScoreThreads / kScoreTile) {
             double dot = 0.0;
-            for (int d = 0; d < D; ++d) dot += (double)q_s[h * D + d] * (double)pooled_s[b * stride + d];
+            if constexpr (DIM != 0) {
+#pragma unroll 8
+                for (int d = 0; d < DIM; d += 4) {
+                    const float4 qv = *reinterpret_cast<const float4*>(&q_s[h * DIM + d]);
+                    const float4 pv = *reinterpret_cast<const float4*>(&pooled_s[b * stride + d]);
+                    dot += (double)qv.x * (double)pv.x;
+                    dot += (double)qv.y * (double)pv.y;
+                    dot += (double)qv.z * (double)pv.z;
+                    dot += (double)qv.w * (double)pv.w;
+                }
+            } else {
+                for (int d = 0; d < D; ++d) dot += (double)q_s[h * D + d] * (double)pooled_s[b * stride + d];
+            }
             part_s[h][b] = (dot > 0.0 ? dot : 0.0) * scale;
         }
     }
@@ -466,7 +494,12 @@ hipError_t launch_idx_score(const SelectBatch& b, const float* q, int32_t idx_n_
     sp.idx_dim = idx_dim;
     sp.idx_block = idx_block;
     dim3 grid((unsigned)((max_blocks + kScoreTile - 1) / kScoreTile), (unsigned)b.n);
-    idx_score_kernel<<<grid, kScoreThreads, 0, stream>>>(sp);
+    bool wide = idx_dim == 128 && (reinterpret_cast<uintptr_t>(q) & 15u) == 0;
+    for (int i = 0; i < b.n && wide; ++i) wide = (reinterpret_cast<uintptr_t>(b.pooled[i]) & 15u) == 0;
+    if (wide)
+        idx_score_kernel<128><<<grid, kScoreThreads, 0, stream>>>(sp);
+    else
+        idx_score_kernel<0><<<grid, kScoreThreads, 0, stream>>>(sp);
     return hipGetLastError();
 }
 

@@ -174,6 +174,24 @@ def test_score_and_select_batched_lists_are_exact():
     assert cnt[5] == 33 and 32 in ids[5, :33]
 
 
+@pytest.mark.parametrize("heads,dim", [(2, 96), (8, 64), (1, 2), (3, 128)])
+def test_score_and_select_other_indexer_shapes(heads, dim):
+    # widths other than 128 take the score kernel's element-by-element path; the lists stay exact
+    rng = np.random.Generator(np.random.PCG64(711 + heads * 131 + dim))
+    n_blocks = [3000, 65, 700]
+    pos = [4 * 3000 + 1, 259, 2000]
+    idx_q = rng.standard_normal((3, heads, dim)).astype(np.float32)
+    pooled = [rng.standard_normal((nb, dim)).astype(np.float32) * 0.05 for nb in n_blocks]
+    with Pool(n_pages=4, max_seqs=2) as pool:
+        idd, ids, cnt = gpu_select(pool, pos, idx_q, pooled, 128, 129)
+        idd.free()
+    for i in range(3):
+        sc = oracle.indexer_score(idx_q[i], pooled[i], n_blocks[i], pos[i], idx_n_head=heads, idx_dim=dim)
+        want = oracle.topk_blocks(sc, 128, pos[i] // 4)
+        assert cnt[i] == want.size, (i, cnt[i], want.size)
+        assert np.array_equal(ids[i, :cnt[i]], want), i
+
+
 def test_select_errors_come_before_any_launch():
     with Pool(n_pages=4, max_seqs=2) as pool:
         z = DeviceBuffer(1 << 16)
