@@ -161,6 +161,17 @@ AllocErr PageAllocator::release_page(int32_t page, std::string& err) {
     return AllocErr::Ok;
 }
 
+AllocErr PageAllocator::retain_fresh_page(int32_t* page_out, std::string& err) {
+    if (free_.empty()) {
+        err = "no free page";
+        return AllocErr::NoPages;
+    }
+    const int32_t p = take_page();
+    external_[(size_t)p] = 1;
+    *page_out = p;
+    return AllocErr::Ok;
+}
+
 bool PageAllocator::seq_resident(int32_t seq, int64_t n_cells) const {
     const int64_t pages = (n_cells + page_cells_ - 1) / page_cells_;
     if (pages > seqs_[(size_t)seq].n_pages) return false;

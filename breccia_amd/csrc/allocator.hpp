@@ -53,6 +53,9 @@ public:
     // References held by an owner that is not a sequence (the prefix tree).
     AllocErr retain_page(int32_t page, std::string& err);
     AllocErr release_page(int32_t page, std::string& err);
+    // A free page handed to a non-sequence owner (one external reference): where a cached page
+    // that comes back from a lower tier lands.
+    AllocErr retain_fresh_page(int32_t* page_out, std::string& err);
     int32_t external_refs(int32_t page) const { return external_[(size_t)page]; }
     AllocErr set_free_order(const int32_t* order, int32_t n, std::string& err);
     void reset();

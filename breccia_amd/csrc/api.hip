@@ -8,7 +8,11 @@
 #include <new>
 #include <unordered_map>
 
+#include <cerrno>
 #include <cmath>
+
+#include <fcntl.h>
+#include <unistd.h>
 
 #include "bkv_internal.hpp"
 
@@ -74,7 +78,21 @@ bkv_status ring_done(bkv_pool* p, int slot, hipStream_t stream) {
     return BKV_OK;
 }
 
+// Pages on their way between the prefix tree's tiers: work enqueued on `stream` from here on may
+// touch the device pages they leave or land on, so it waits for the transfers (until they are
+// known to be over).
+static bkv_status wait_for_tier_moves(bkv_pool* p, hipStream_t stream) {
+    if (!p->tiers.pending) return BKV_OK;
+    if (hipEventQuery(p->tiers.done) == hipSuccess)
+        p->tiers.pending = false;
+    else
+        BKV_HIP(hipStreamWaitEvent(stream, p->tiers.done, 0));
+    return BKV_OK;
+}
+
 bkv_status flush_tables(bkv_pool* p, hipStream_t stream) {
+    bkv_status tier_st = wait_for_tier_moves(p, stream);
+    if (tier_st != BKV_OK) return tier_st;
     std::vector<TableUpdate>& pend = p->alloc->pending();
     if (pend.empty()) return BKV_OK;
     if (p->host_only) {
@@ -160,8 +178,13 @@ static bkv_status need_device(const bkv_pool* p) {
 }
 
 static void destroy_device_side(bkv_pool* p) {
+    if (p->tiers.fd >= 0) (void)::close(p->tiers.fd);
+    p->tiers.fd = -1;
     if (p->host_only) return;
     (void)hipDeviceSynchronize();
+    if (p->tiers.host) (void)hipHostFree(p->tiers.host);
+    if (p->tiers.bounce) (void)hipHostFree(p->tiers.bounce);
+    if (p->tiers.done) (void)hipEventDestroy(p->tiers.done);
     if (p->slab) (void)hipFree(p->slab);
     if (p->table_dev) (void)hipFree(p->table_dev);
     if (p->part_o) (void)hipFree(p->part_o);
@@ -325,6 +348,8 @@ bkv_status bkv_pool_reset(bkv_pool* p, void* stream) {
         return BKV_OK;
     }
     const uint64_t layer_bytes = p->g.k_pool_bytes + p->g.v_pool_bytes;
+    bkv_status st = wait_for_tier_moves(p, S(stream));
+    if (st != BKV_OK) return st;
     BKV_HIP(launch_fill(p->slab, layer_bytes * (uint64_t)p->g.n_layers, 0u, S(stream)));
     return flush_tables(p, S(stream));
 }
@@ -352,6 +377,8 @@ bkv_status bkv_pool_fill(bkv_pool* p, int byte, void* stream) {
     const uint32_t b = (uint32_t)(byte & 0xff);
     const uint32_t word = b | (b << 8) | (b << 16) | (b << 24);
     const uint64_t layer_bytes = p->g.k_pool_bytes + p->g.v_pool_bytes;
+    st = wait_for_tier_moves(p, S(stream));
+    if (st != BKV_OK) return st;
     BKV_HIP(launch_fill(p->slab, layer_bytes * (uint64_t)p->g.n_layers, word, S(stream)));
     return BKV_OK;
 }
@@ -392,6 +419,18 @@ bkv_status bkv_seq_free(bkv_pool* p, int32_t seq) {
     return from_alloc(p->alloc->seq_free(seq, err), err);
 }
 
+// Moves the bytes behind the prefix tree's tier bookkeeping (defined with the swap path below).
+static bkv_status run_tier_moves(bkv_pool* p, const std::vector<TierMove>& moves);
+
+// Make `want` device pages free by evicting cached prefixes: demoted to the lower tiers when the
+// pool has them, dropped otherwise.
+static bkv_status prefix_make_room(bkv_pool* p, int32_t want, int32_t* freed) {
+    std::vector<TierMove> moves;
+    const int32_t n = p->prefix->evict(want, p->prefix->tiered() ? &moves : nullptr);
+    if (freed) *freed = n;
+    return run_tier_moves(p, moves);
+}
+
 bkv_status bkv_seq_reserve(bkv_pool* p, int32_t seq, int64_t new_len, bkv_page_pair* cow,
                            int32_t cow_cap, int32_t* n_cow) {
     if (!p) return fail(BKV_ERR_INVALID, "seq_reserve: NULL pool");
@@ -403,9 +442,14 @@ bkv_status bkv_seq_reserve(bkv_pool* p, int32_t seq, int64_t new_len, bkv_page_p
         // (least recently used first), then the request is tried once more.
         const int64_t grow = (new_len - p->alloc->seq_len(seq) + p->g.page_cells - 1) / p->g.page_cells + 1;
         const int64_t missing = grow - p->alloc->free_pages();
-        if (missing > 0 && p->prefix->evict((int32_t)missing) > 0) {
-            err.clear();
-            e = p->alloc->seq_reserve(seq, new_len, reinterpret_cast<PagePair*>(cow), cow_cap, n_cow, err);
+        if (missing > 0) {
+            int32_t freed = 0;
+            const bkv_status st = prefix_make_room(p, (int32_t)missing, &freed);
+            if (st != BKV_OK) return st;
+            if (freed > 0) {
+                err.clear();
+                e = p->alloc->seq_reserve(seq, new_len, reinterpret_cast<PagePair*>(cow), cow_cap, n_cow, err);
+            }
         }
     }
     return from_alloc(e, err);
@@ -423,9 +467,9 @@ bkv_status bkv_prefix_match(bkv_pool* p, const int32_t* tokens, int64_t n_tokens
                             int64_t* matched_tokens) {
     bkv_status st = prefix_args(p, "prefix_match", tokens, n_tokens);
     if (st != BKV_OK) return st;
-    std::vector<int32_t> pages;
-    p->prefix->match(tokens, n_tokens, false, pages);
-    if (matched_tokens) *matched_tokens = (int64_t)pages.size() * p->g.page_cells;
+    std::vector<PrefixTree::Node*> chain;
+    p->prefix->match_nodes(tokens, n_tokens, false, chain);
+    if (matched_tokens) *matched_tokens = (int64_t)chain.size() * p->g.page_cells;
     return BKV_OK;
 }
 
@@ -434,9 +478,28 @@ bkv_status bkv_seq_create_from_prefix(bkv_pool* p, const int32_t* tokens, int64_
     bkv_status st = prefix_args(p, "seq_create_from_prefix", tokens, n_tokens);
     if (st != BKV_OK) return st;
     if (!seq_out) return fail(BKV_ERR_INVALID, "seq_create_from_prefix: NULL output");
+    std::vector<PrefixTree::Node*> chain;
+    p->prefix->match_nodes(tokens, n_tokens, true, chain);
+    if ((int64_t)chain.size() > p->alloc->max_pages_per_seq()) chain.resize((size_t)p->alloc->max_pages_per_seq());
+    int32_t lower = 0;
+    for (const PrefixTree::Node* x : chain) lower += PrefixTree::tier_of(x) != Tier::Device;
+    if (lower > 0) {
+        // The tail of the chain lives in the lower tiers: it comes back to fresh device pages
+        // (other cached prefixes make room if they must; the chain itself is held meanwhile).
+        std::vector<TierMove> moves;
+        p->prefix->pin_nodes(chain, +1);
+        const int32_t missing = lower - p->alloc->free_pages();
+        if (missing > 0) p->prefix->evict(missing, &moves);
+        p->prefix->promote(chain, lower, moves);
+        p->prefix->pin_nodes(chain, -1);
+        st = run_tier_moves(p, moves);
+        if (st != BKV_OK) return st;
+    }
     std::vector<int32_t> pages;
-    p->prefix->match(tokens, n_tokens, true, pages);
-    if ((int64_t)pages.size() > p->alloc->max_pages_per_seq()) pages.resize((size_t)p->alloc->max_pages_per_seq());
+    for (const PrefixTree::Node* x : chain) {
+        if (PrefixTree::tier_of(x) != Tier::Device) break;
+        pages.push_back(PrefixTree::page_of(x));
+    }
     std::string err;
     st = from_alloc(p->alloc->seq_create_shared(pages.data(), (int32_t)pages.size(), seq_out, err), err);
     if (st != BKV_OK) return st;
@@ -464,9 +527,7 @@ bkv_status bkv_prefix_insert(bkv_pool* p, int32_t seq, const int32_t* tokens, in
 bkv_status bkv_prefix_evict(bkv_pool* p, int32_t want_pages, int32_t* freed) {
     if (!p) return fail(BKV_ERR_INVALID, "prefix_evict: NULL pool");
     if (want_pages < 0) return fail(BKV_ERR_INVALID, sfmt("prefix_evict: %lld pages wanted", want_pages));
-    const int32_t n = p->prefix->evict(want_pages);
-    if (freed) *freed = n;
-    return BKV_OK;
+    return prefix_make_room(p, want_pages, freed);
 }
 
 bkv_status bkv_prefix_pin(bkv_pool* p, const int32_t* tokens, int64_t n_tokens, int32_t pin,
@@ -531,6 +592,7 @@ bkv_status bkv_pool_check(const bkv_pool* p) {
     if (!p) return fail(BKV_ERR_INVALID, "pool_check: NULL pool");
     std::string err;
     if (!p->alloc->check(err)) return fail(BKV_ERR_STATE, "allocator invariant broken: " + err);
+    if (!p->prefix->check(err)) return fail(BKV_ERR_STATE, err);
     return BKV_OK;
 }
 
@@ -1014,6 +1076,8 @@ bkv_status bkv_page_copy(bkv_pool* p, const bkv_page_pair* pairs, int32_t n_pair
         return fail(BKV_ERR_INVALID, "page_copy: a destination page appears twice");
     bkv_status st = need_device(p);
     if (st != BKV_OK) return st;
+    st = wait_for_tier_moves(p, S(stream));
+    if (st != BKV_OK) return st;
     const int32_t per_launch = (int32_t)(ParamRing::kSlotBytes / sizeof(bkv_page_pair));
     for (int32_t at = 0; at < n_pairs; at += per_launch) {
         const int32_t n = std::min(per_launch, n_pairs - at);
@@ -1129,6 +1193,8 @@ bkv_status bkv_swap_out(bkv_pool* p, const int32_t* pages, int32_t n, void* pinn
     st = need_device(p);
     if (st != BKV_OK) return st;
     if (n == 0) return BKV_OK;
+    st = wait_for_tier_moves(p, S(stream));
+    if (st != BKV_OK) return st;
     return swap_move(p, pages, n, static_cast<uint8_t*>(pinned_host), true, S(stream));
 }
 
@@ -1144,6 +1210,8 @@ bkv_status bkv_swap_in(bkv_pool* p, const int32_t* pages, int32_t n, const void*
     st = need_device(p);
     if (st != BKV_OK) return st;
     if (n == 0) return BKV_OK;
+    st = wait_for_tier_moves(p, S(stream));
+    if (st != BKV_OK) return st;
     return swap_move(p, pages, n, const_cast<uint8_t*>(static_cast<const uint8_t*>(pinned_host)),
                      false, S(stream));
 }
@@ -1193,6 +1261,146 @@ bkv_status bkv_seq_restore(bkv_pool* p, int32_t seq, int32_t lp0, int32_t n,
                               S(stream));
     if (st != BKV_OK) return st;
     return flush_tables(p, S(stream));
+}
+
+// ---- lower tiers of the prefix tree ------------------------------------------------------
+// The bytes behind the tree's bookkeeping, in the order the tree listed the moves.  Transfers
+// between the device and the host arena go through the swap path on the side stream (runs of
+// consecutive slots as one transfer); the file is read and written from the host, one page at a
+// time, through the arena or the two-slot bounce buffer.  Work enqueued by later calls waits for
+// `tiers.done` (flush_tables).  A host-only pool keeps the books only.
+static bkv_status tier_io_failed(bkv_pool* p, const char* what) {
+    const std::string msg = std::string("prefix tiers: ") + what + " failed: " + std::strerror(errno) +
+                            "; the cached prefixes were dropped";
+    p->prefix->clear();
+    return fail(BKV_ERR_STATE, msg);
+}
+
+static bkv_status run_tier_moves(bkv_pool* p, const std::vector<TierMove>& moves) {
+    if (moves.empty() || p->host_only) return BKV_OK;
+    TierStore& ts = p->tiers;
+    const uint64_t slab = bkv_swap_page_bytes(p);
+    bool device_quiet = false;  // every stream's writes to the pages that leave are complete
+    bool side_idle = false;     // nothing is on its way into or out of the arena / bounce buffer
+    int bounce_half = 0;
+    bool half_in_flight[2] = {false, false};  // a copy out of that half of the bounce buffer is enqueued
+    size_t i = 0;
+    while (i < moves.size()) {
+        const TierMove& m = moves[i];
+        if (m.kind == TierMove::DeviceToHost || m.kind == TierMove::HostToDevice) {
+            size_t j = i + 1;
+            while (j < moves.size() && moves[j].kind == m.kind && moves[j].host_slot == moves[j - 1].host_slot + 1) ++j;
+            std::vector<int32_t> pages;
+            for (size_t k = i; k < j; ++k) pages.push_back(moves[k].page);
+            const bool out = m.kind == TierMove::DeviceToHost;
+            if (out && !device_quiet) {
+                // the pages were written on streams this call does not know
+                BKV_HIP(hipDeviceSynchronize());
+                device_quiet = true;
+            }
+            const bkv_status st = swap_move(p, pages.data(), (int32_t)pages.size(),
+                                            ts.host + (uint64_t)m.host_slot * slab, out, p->side);
+            if (st != BKV_OK) return st;
+            side_idle = false;
+            i = j;
+        } else if (m.kind == TierMove::HostToDisk) {
+            if (!side_idle) {
+                BKV_HIP(hipStreamSynchronize(p->side));
+                side_idle = true;
+                half_in_flight[0] = half_in_flight[1] = false;
+            }
+            const ssize_t w = ::pwrite(ts.fd, ts.host + (uint64_t)m.host_slot * slab, slab,
+                                       (off_t)((uint64_t)m.disk_slot * slab));
+            if (w != (ssize_t)slab) return tier_io_failed(p, "a write to the disk tier");
+            ++i;
+        } else {
+            // file -> bounce half -> device; the other half may still be on its way
+            uint8_t* half = ts.bounce + (uint64_t)bounce_half * slab;
+            if (half_in_flight[bounce_half]) {
+                BKV_HIP(hipStreamSynchronize(p->side));
+                side_idle = true;
+                half_in_flight[0] = half_in_flight[1] = false;
+            }
+            const ssize_t r = ::pread(ts.fd, half, slab, (off_t)((uint64_t)m.disk_slot * slab));
+            if (r != (ssize_t)slab) return tier_io_failed(p, "a read from the disk tier");
+            const bkv_status st = swap_move(p, &m.page, 1, half, false, p->side);
+            if (st != BKV_OK) return st;
+            side_idle = false;
+            half_in_flight[bounce_half] = true;
+            bounce_half ^= 1;
+            ++i;
+        }
+    }
+    BKV_HIP(hipEventRecord(ts.done, p->side));
+    ts.pending = true;
+    return BKV_OK;
+}
+
+bkv_status bkv_prefix_tiers(bkv_pool* p, uint64_t host_bytes, const char* disk_path, uint64_t disk_bytes) {
+    if (!p) return fail(BKV_ERR_INVALID, "prefix_tiers: NULL pool");
+    const uint64_t slab = bkv_swap_page_bytes(p);
+    const uint64_t cap = (uint64_t)1 << 30;
+    const uint64_t host_slots = std::min(host_bytes / slab, cap);
+    const uint64_t disk_slots = disk_path ? std::min(disk_bytes / slab, cap) : 0;
+    if (disk_slots > 0 && host_slots == 0)
+        return fail(BKV_ERR_INVALID, "prefix_tiers: the disk tier is fed from the host tier, which has no room "
+                                     "for a single page");
+    TierStore& ts = p->tiers;
+    // what the lower tiers hold now goes first
+    p->prefix->set_tiers(0, 0);
+    if (!p->host_only) {
+        BKV_HIP(hipStreamSynchronize(p->side));
+        if (ts.host) BKV_HIP(hipHostFree(ts.host));
+        if (ts.bounce) BKV_HIP(hipHostFree(ts.bounce));
+    }
+    ts.host = ts.bounce = nullptr;
+    ts.pending = false;
+    if (ts.fd >= 0) (void)::close(ts.fd);
+    ts.fd = -1;
+    ts.host_slots = ts.disk_slots = 0;
+    if (host_slots == 0) return BKV_OK;
+    if (!p->host_only) {
+        void* mem = nullptr;
+        if (hipHostMalloc(&mem, host_slots * slab, hipHostMallocDefault) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(BKV_ERR_NOMEM, sfmt("prefix_tiers: cannot pin %lld bytes of host memory",
+                                            (long long)(host_slots * slab)));
+        }
+        ts.host = static_cast<uint8_t*>(mem);
+        if (!ts.done) BKV_HIP(hipEventCreateWithFlags(&ts.done, hipEventDisableTiming));
+    }
+    if (disk_slots > 0) {
+        ts.fd = ::open(disk_path, O_RDWR | O_CREAT | O_TRUNC, 0600);
+        if (ts.fd < 0)
+            return fail(BKV_ERR_INVALID, std::string("prefix_tiers: cannot open ") + disk_path + ": " +
+                                             std::strerror(errno));
+        if (!p->host_only) {
+            void* mem = nullptr;
+            if (hipHostMalloc(&mem, 2 * slab, hipHostMallocDefault) != hipSuccess) {
+                (void)hipGetLastError();
+                return fail(BKV_ERR_NOMEM, "prefix_tiers: cannot pin the bounce buffer of the disk tier");
+            }
+            ts.bounce = static_cast<uint8_t*>(mem);
+        }
+    }
+    ts.host_slots = (int32_t)host_slots;
+    ts.disk_slots = (int32_t)disk_slots;
+    p->prefix->set_tiers(ts.host_slots, ts.disk_slots);
+    return BKV_OK;
+}
+
+bkv_status bkv_prefix_tier_stats(const bkv_pool* p, int32_t* nodes_by_tier, uint64_t* moved) {
+    if (!p) return fail(BKV_ERR_INVALID, "prefix_tier_stats: NULL pool");
+    const TierStats& st = p->prefix->stats();
+    if (nodes_by_tier)
+        for (int t = 0; t < 3; ++t) nodes_by_tier[t] = st.nodes[t];
+    if (moved) {
+        moved[0] = st.to_host;
+        moved[1] = st.to_disk;
+        moved[2] = st.promoted;
+        moved[3] = st.dropped;
+    }
+    return BKV_OK;
 }
 
 // ---- gather ------------------------------------------------------------------------------

@@ -69,6 +69,18 @@ struct SwapStage {
     int next = 0;
 };
 
+// Where the prefix tree's lower tiers keep their pages: a pinned-host arena of slots and a file,
+// slot = one page's bytes of every layer ([layer][K page | V page]).
+struct TierStore {
+    uint8_t* host = nullptr;    // host_slots slots (pinned; null on a host-only pool)
+    int32_t host_slots = 0;
+    int fd = -1;                // the file of the disk tier
+    int32_t disk_slots = 0;
+    uint8_t* bounce = nullptr;  // one pinned slot between the file and the device
+    hipEvent_t done = nullptr;  // behind the last transfer enqueued on the side stream
+    bool pending = false;       // `done` may not have completed yet
+};
+
 }  // namespace bkv
 
 struct bkv_pool {
@@ -95,6 +107,7 @@ struct bkv_pool {
     bkv::ParamRing ring;
     bkv::StageTimer timer;
     bkv::SwapStage stage;
+    bkv::TierStore tiers;
     hipStream_t side = nullptr;
     hipEvent_t side_done = nullptr;
     bool side_used = false;

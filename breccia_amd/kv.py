@@ -6,6 +6,7 @@ arrays and integers into the C calls and turns status codes into exceptions.
 from __future__ import annotations
 
 import ctypes as C
+import os
 
 import numpy as np
 
@@ -303,6 +304,18 @@ class Pool:
 
     def prefix_clear(self) -> None:
         check(lib.bkv_prefix_clear(self.handle))
+
+    def prefix_tiers(self, host_bytes: int, disk_path: str | None = None, disk_bytes: int = 0) -> None:
+        """Lower tiers for evicted prefix pages: pinned host memory, then a file."""
+        path = None if disk_path is None else os.fsencode(disk_path)
+        check(lib.bkv_prefix_tiers(self.handle, host_bytes, path, disk_bytes))
+
+    def prefix_tier_stats(self):
+        """-> ((device, host, disk) nodes, (to_host, to_disk, promoted, dropped) pages moved)"""
+        nodes = (C.c_int32 * 3)()
+        moved = (C.c_uint64 * 4)()
+        check(lib.bkv_prefix_tier_stats(self.handle, nodes, moved))
+        return tuple(int(x) for x in nodes), tuple(int(x) for x in moved)
 
     # -- hot path
     def append(self, layer: int, seqs, pos0, n_tokens, k_dev, v_dev, stream=None,

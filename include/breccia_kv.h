@@ -152,8 +152,8 @@ bkv_status bkv_pool_set_free_order(bkv_pool *pool, const int32_t *order, int32_t
  * bkv_prefix_insert: list the complete pages of the first n_tokens tokens of `seq` (whose K/V
  *   the caller has appended).  Prefixes already listed keep their pages (first publisher
  *   wins); *new_pages = nodes added.
- * bkv_prefix_match: how many leading tokens of `tokens` are covered by listed pages
- *   (a multiple of the page size); does not count as a use.
+ * bkv_prefix_match: how many leading tokens of `tokens` are covered by listed pages, in
+ *   whatever tier (a multiple of the page size); does not count as a use.
  * bkv_seq_create_from_prefix: a new sequence that shares those pages (refcount + 1 each),
  *   length = *matched_tokens; the caller appends the rest, starting on a fresh page -- a
  *   page-aligned share never needs a copy-on-write copy.
@@ -175,6 +175,34 @@ bkv_status bkv_prefix_pin(bkv_pool *pool, const int32_t *tokens, int64_t n_token
 bkv_status bkv_prefix_stats(const bkv_pool *pool, int32_t *nodes, int32_t *evictable_pages,
                             int32_t *pinned_nodes);
 bkv_status bkv_prefix_clear(bkv_pool *pool);
+
+/* Lower tiers for evicted prefixes (the design notes' T2 "pinned, hard byte cap" and T3 "NVMe,
+ * chunked read", docs/reference-engines/02-kv-and-context.md:594-596, under the movement rules
+ * of :566-572: only complete pages move, a page is in exactly one tier, promotion is chunked and
+ * never part of a decode step).  No reference implementation.
+ * bkv_prefix_tiers: host_bytes of pinned host memory (hipHostMalloc) and, when disk_path is not
+ *   NULL, disk_bytes of the file disk_path (created or truncated; it is left in place when the
+ *   pool goes) hold whole pages ([layer][K page | V page], bkv_swap_page_bytes each).  From
+ *   then on an evicted prefix page is demoted instead of dropped: device -> host; when the host
+ *   arena is full its least recently used page goes host -> disk, and when the file is full
+ *   its least recently used leaf is dropped.  Demotion works upwards from the leaves, so along
+ *   a chain of pages the tiers only go down.  bkv_prefix_match counts the pages of every tier;
+ *   bkv_seq_create_from_prefix brings the matched chain's lower part back to fresh device
+ *   pages (evicting other cached prefixes if it must) and adopts what is on the device after
+ *   that.  bkv_prefix_insert of a sequence that has recomputed a demoted page hands that page
+ *   to the tree at no transfer.  Transfers run on the pool's side stream; every later call
+ *   that enqueues work on the pool (append, attention, page copy, swap, fill, reset, gather)
+ *   waits for them on the device on its own stream -- writes through bkv_pool_layer_ptr are
+ *   the caller's to order (bkv_swap_wait) -- and the host does not block except for file I/O
+ *   and for the synchronisation before pages leave the device (the streams that wrote them
+ *   are not known to the call).  host_bytes = 0 switches the tiers off and drops what they
+ *   hold; calling it again resizes them the same way.  An I/O error on the file drops every
+ *   cached prefix and reports BKV_ERR_STATE.
+ * bkv_prefix_tier_stats: nodes_by_tier[3] = pages on the device / in host memory / on disk;
+ *   moved[4] = pages demoted to host, demoted to disk, promoted, dropped (since creation). */
+bkv_status bkv_prefix_tiers(bkv_pool *pool, uint64_t host_bytes, const char *disk_path,
+                            uint64_t disk_bytes);
+bkv_status bkv_prefix_tier_stats(const bkv_pool *pool, int32_t *nodes_by_tier, uint64_t *moved);
 
 /* ---- hot path ---------------------------------------------------------------
  * bkv_append replaces Qsa::kv_append + shaders/qsa_kv_append.comp (qsa/mod.rs:

@@ -4,6 +4,8 @@ appends only its own suffix attends exactly like a request that recomputed every
 import numpy as np
 import pytest
 
+from breccia_amd import lib as L
+from breccia_amd.kv import Stream
 from gpu_common import Twin, check_attn
 
 pytestmark = pytest.mark.gpu
@@ -69,3 +71,76 @@ def test_adopted_prefix_attends_like_a_recomputed_one():
         assert pool.prefix_evict(1000) == 127
         pool.check()
         assert np.array_equal(before, out_adopted[:1])
+
+
+@pytest.mark.parametrize("layout", [L.LAYOUT_F16, L.LAYOUT_Q8V])
+def test_demoted_prefix_comes_back_from_host_memory_and_from_disk_bit_for_bit(tmp_path, layout):
+    # 50 cached pages of a two-layer pool leave the device (40 fit the host arena, 10 go on to the
+    # file), the whole device pool is poisoned, and a request that adopts the prefix gets every
+    # byte of both layers back: same pool bytes as a request that recomputed the prefix, and
+    # bit-identical attention -- on a stream of the caller's, with no host synchronisation in
+    # between (later calls wait for the transfers on the device)
+    rng = np.random.Generator(np.random.PCG64(901 + layout))
+    prefix = rng.integers(0, 32000, size=50 * 16 + 5).astype(np.int32)
+    with Twin(n_layers=2, n_pages=128, max_seqs=8, layout=layout) as tw:
+        pool = tw.pool
+        pool.set_free_order(rng.permutation(128).astype(np.int32))
+        slab = pool.swap_page_bytes()
+        pool.prefix_tiers(40 * slab, str(tmp_path / "tier3.bin"), 64 * slab)
+        a = pool.seq_create()
+        pool.seq_reserve(a, prefix.size)
+        for layer in range(2):
+            k, v = kv_of(prefix, 0, 11 + layer)
+            tw.append(layer, [a], [0], [k], [v])
+        assert pool.prefix_insert(a, prefix) == 50
+        pool.seq_free(a)
+        assert pool.prefix_evict(50) == 50
+        assert pool.prefix_tier_stats() == ((0, 40, 10), (50, 10, 0, 0))
+        assert pool.free_pages() == 128
+        pool.fill(0xFF)
+        # control: recomputes everything; adopter: takes the 50 pages from the tiers
+        c = pool.seq_create()
+        pool.seq_reserve(c, prefix.size)
+        for layer in range(2):
+            k, v = kv_of(prefix, 0, 11 + layer)
+            tw.append(layer, [c], [0], [k], [v])
+        st = Stream()
+        s, m = pool.seq_create_from_prefix(prefix)
+        assert m == 800
+        assert pool.prefix_tier_stats() == ((50, 0, 0), (50, 10, 50, 0))
+        pool.seq_reserve(s, prefix.size)
+        for layer in range(2):
+            k, v = kv_of(prefix[800:], 800, 11 + layer)
+            tw.append(layer, [s], [800], [k], [v], stream=st)
+        q = rng.standard_normal((2, 16, 256)).astype(np.float32)
+        for layer in range(2):
+            out = tw.decode_attn(layer, [s, c], [prefix.size - 1] * 2, q[[0, 0]], 16, stream=st)
+            assert np.all(np.isfinite(out))
+            assert np.array_equal(out[0].view(np.uint32), out[1].view(np.uint32)), layer
+        ts, tc = pool.block_table(s), pool.block_table(c)
+        assert len(set(ts[:50].tolist()) & set(tc[:50].tolist())) == 0
+        for layer in range(2):
+            for which in range(2):
+                img = pool.read_layer(layer, which)
+                pb = img.size // 128
+                for i in range(50):
+                    ps, pc = int(ts[i]), int(tc[i])
+                    assert np.array_equal(img[ps * pb:(ps + 1) * pb], img[pc * pb:(pc + 1) * pb]), (layer, which, i)
+        pool.seq_free(s)
+        pool.seq_free(c)
+        pool.check()
+        # once more through the tiers, with the host arena alone (a smaller one: 30 pages are dropped)
+        pool.prefix_tiers(20 * slab)
+        assert pool.prefix_evict(50) == 50
+        nodes, _ = pool.prefix_tier_stats()
+        assert nodes == (0, 20, 0) and pool.prefix_match(prefix) == 320
+        pool.fill(0xEE)
+        s, m = pool.seq_create_from_prefix(prefix)
+        assert m == 320
+        c = pool.seq_create()
+        pool.seq_reserve(c, 320)
+        k, v = kv_of(prefix[:320], 0, 11)
+        tw.append(0, [c], [0], [k], [v])
+        out = tw.decode_attn(0, [s, c], [319, 319], q[[1, 1]], 16)
+        assert np.array_equal(out[0].view(np.uint32), out[1].view(np.uint32))
+        pool.check()

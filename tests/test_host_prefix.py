@@ -190,3 +190,155 @@ def test_randomised_tree_keeps_allocator_invariants():
             pool.check()
         nodes, evictable, pinned = pool.prefix_stats()
         assert 0 <= evictable <= nodes and 0 <= pinned <= nodes
+
+
+# ---- lower tiers: on a host-only pool the policy keeps its books, no bytes move ------------------
+def publish(pool, prompt):
+    s = pool.seq_create()
+    pool.seq_reserve(s, prompt.size)
+    pool.prefix_insert(s, prompt)
+    pool.seq_free(s)
+
+
+def test_evicted_pages_are_demoted_leaf_first_and_promoted_on_adoption(tmp_path):
+    with host_pool(n_pages=32) as pool:
+        slab = pool.swap_page_bytes()
+        pool.prefix_tiers(6 * slab, str(tmp_path / "t3.bin"), 4 * slab)
+        a, b = toks(70, 64), toks(71, 64)                       # 4 pages each
+        publish(pool, a)
+        publish(pool, b)
+        assert pool.prefix_tier_stats() == ((8, 0, 0), (0, 0, 0, 0))
+        # 4 pages go: a is the older chain, it goes to host memory from its end -- and stays listed
+        assert pool.prefix_evict(4) == 4
+        assert pool.free_pages() == 32 - 4
+        assert pool.prefix_tier_stats() == ((4, 4, 0), (4, 0, 0, 0))
+        assert pool.prefix_match(a) == 64 and pool.prefix_match(b) == 64
+        # 3 of b: the arena holds 6, so a's oldest page makes room by going to the file
+        assert pool.prefix_evict(3) == 3
+        nodes, moved = pool.prefix_tier_stats()
+        assert nodes == (1, 6, 1) and moved == (7, 1, 0, 0)
+        pool.check()
+        # adopting a brings its 4 pages back (3 from host memory, 1 from the file) onto fresh pages
+        s, m = pool.seq_create_from_prefix(a)
+        assert m == 64 and pool.seq_len(s) == 64
+        nodes, moved = pool.prefix_tier_stats()
+        assert nodes == (5, 3, 0) and moved == (7, 1, 4, 0)
+        assert len(set(pool.block_table(s)[:4].tolist())) == 4
+        assert [pool.page_refcount(int(p)) for p in pool.block_table(s)[:4]] == [2] * 4
+        pool.check()
+        # pages in use stay on the device: only b's last device page can leave
+        assert pool.prefix_evict(10) == 1
+        assert pool.prefix_tier_stats()[0] == (4, 4, 0)
+        pool.seq_free(s)
+        pool.check()
+
+
+def test_lower_tiers_fill_up_and_the_oldest_leaves_are_dropped(tmp_path):
+    with host_pool(n_pages=64) as pool:
+        slab = pool.swap_page_bytes()
+        pool.prefix_tiers(2 * slab, str(tmp_path / "t3.bin"), 3 * slab)
+        prompts = [toks(80 + i, 32) for i in range(4)]          # 2 pages each
+        for pr in prompts:
+            publish(pool, pr)
+        assert pool.prefix_evict(8) == 8                        # 8 pages into 2 + 3 slots
+        nodes, moved = pool.prefix_tier_stats()
+        assert nodes[0] == 0 and nodes[1] == 2 and nodes[2] == 3 and moved[3] == 3
+        assert sum(nodes) == 5
+        # what is left are heads of chains (a page never outlives its parent)
+        left = [pool.prefix_match(pr) for pr in prompts]
+        assert sum(left) == 5 * 16 and left[3] == 32            # the newest chain is whole
+        pool.check()
+        # without a file the host arena's oldest pages are dropped instead
+        pool.prefix_tiers(2 * slab)
+        assert pool.prefix_tier_stats()[0] == (0, 0, 0)         # resizing drops what the tiers held
+        for pr in prompts:
+            publish(pool, pr)
+        assert pool.prefix_evict(8) == 8
+        nodes, _ = pool.prefix_tier_stats()
+        assert nodes == (0, 2, 0)
+        # tiers off: eviction drops again
+        pool.prefix_tiers(0)
+        publish(pool, prompts[0])
+        assert pool.prefix_evict(2) == 2 and pool.prefix_stats()[0] == 0
+        pool.check()
+
+
+def test_reserve_demotes_and_a_republished_page_returns_without_a_transfer():
+    with host_pool(n_pages=16) as pool:
+        pool.prefix_tiers(64 * pool.swap_page_bytes())
+        cached = toks(90, 160)                                  # 10 pages
+        publish(pool, cached)
+        big = pool.seq_create()
+        pool.seq_reserve(big, 12 * 16)                          # 6 free + 6 demoted
+        nodes, moved = pool.prefix_tier_stats()
+        assert nodes[1] >= 6 and moved[0] == nodes[1] and pool.prefix_match(cached) == 160
+        pool.seq_free(big)
+        # a sequence that recomputed the whole prompt lists it again: its pages replace the host copies
+        s = pool.seq_create()
+        pool.seq_reserve(s, 160)
+        assert pool.prefix_insert(s, cached) == 0
+        nodes2, moved2 = pool.prefix_tier_stats()
+        assert nodes2 == (10, 0, 0) and moved2[2] == 0          # nothing was promoted: no transfer
+        # the pages that never left the device keep their first publisher's copies
+        assert [pool.page_refcount(int(p)) for p in pool.block_table(s)[:10]] == \
+            [1] * nodes[0] + [2] * (10 - nodes[0])
+        pool.check()
+
+
+def test_promotion_stops_where_the_device_has_no_page_left():
+    with host_pool(n_pages=8, max_seqs=4, per_seq=8) as pool:
+        pool.prefix_tiers(64 * pool.swap_page_bytes())
+        a = toks(95, 96)                                        # 6 pages
+        publish(pool, a)
+        assert pool.prefix_evict(6) == 6
+        hog = pool.seq_create()
+        pool.seq_reserve(hog, 5 * 16)                           # 3 pages stay free
+        s, m = pool.seq_create_from_prefix(a)
+        assert m == 48                                          # 3 pages came back, the chain's head
+        assert pool.prefix_tier_stats()[0] == (3, 3, 0)
+        assert pool.prefix_match(a) == 96
+        pool.check()
+
+
+def test_randomised_tiered_tree_keeps_every_invariant(tmp_path):
+    rng = np.random.Generator(np.random.PCG64(51))
+    base = [toks(160 + i, 16 * 12) for i in range(5)]
+    with host_pool(n_pages=48, max_seqs=12, per_seq=24) as pool:
+        slab = pool.swap_page_bytes()
+        pool.prefix_tiers(10 * slab, str(tmp_path / "t3.bin"), 12 * slab)
+        live = []
+        for step in range(600):
+            op = rng.integers(0, 7)
+            try:
+                if op == 0 and len(live) < 10:
+                    pr = base[rng.integers(0, 5)][:int(rng.integers(1, 12 * 16))].copy()
+                    if rng.integers(0, 3) == 0:
+                        pr[int(rng.integers(0, pr.size))] ^= 1
+                    s, m = pool.seq_create_from_prefix(pr)
+                    assert m % 16 == 0 and m <= pr.size
+                    live.append((s, pr))
+                    pool.seq_reserve(s, pr.size)
+                elif op == 1 and live:
+                    s, pr = live[rng.integers(0, len(live))]
+                    if pool.seq_len(s) >= pr.size:
+                        pool.prefix_insert(s, pr)
+                elif op == 2 and live:
+                    s, _ = live.pop(rng.integers(0, len(live)))
+                    pool.seq_free(s)
+                elif op == 3:
+                    pool.prefix_evict(int(rng.integers(0, 8)))
+                elif op == 4:
+                    pool.prefix_pin(base[rng.integers(0, 5)][:64], pin=bool(rng.integers(0, 2)))
+                elif op == 5 and live:
+                    s, pr = live[rng.integers(0, len(live))]
+                    pool.seq_reserve(s, min(pool.seq_len(s) + int(rng.integers(1, 40)), 24 * 16))
+                elif op == 6 and step % 97 == 0:
+                    pool.prefix_tiers(int(rng.integers(1, 12)) * slab, str(tmp_path / "t3.bin"),
+                                      int(rng.integers(0, 12)) * slab)
+            except BkvError as e:
+                assert e.status in (L.ERR_NO_PAGES, L.ERR_RANGE), e
+            pool.check()
+            nodes, moved = pool.prefix_tier_stats()
+            assert sum(nodes) == pool.prefix_stats()[0]
+        nodes, moved = pool.prefix_tier_stats()
+        assert moved[0] > 0 and moved[1] > 0 and moved[2] > 0
