@@ -266,6 +266,7 @@ def main() -> int:
         extra.update(bench_select(stream))
         extra.update(bench_prefill(stream))
         extra.update(bench_moves(stream))
+        extra.update(bench_prefix_tiers(stream))
 
     line = {"metric": "paged decode-attn step throughput, batch 8 mixed 1k-32k (append + attention, "
                       "algorithmic bytes / time)",
@@ -561,6 +562,51 @@ def bench_prefill(stream) -> dict:
     for b in (kd, vd, q, out):
         b.free()
     return res
+
+
+def bench_prefix_tiers(stream) -> dict:
+    """The prefix tree's lower tiers: 2048 cached pages (a 32k-token prefix, 64 MiB at one layer)
+    demoted to pinned host memory and promoted back by an adopting request; then the same with a
+    host arena of 256 pages, so that most pages go on to a file under the temporary directory
+    (page cache included: the file is not opened for direct I/O)."""
+    import tempfile
+
+    from breccia_amd.kv import DeviceBuffer, Pool
+
+    rng = np.random.Generator(np.random.PCG64(20250008))
+    n = 2048
+    tokens = rng.integers(0, 32000, size=n * PAGE).astype(np.int32)
+    pool = Pool(n_layers=1, n_pages=2 * n + 64, n_kv_head=N_KV, head_dim=HD, max_seqs=4,
+                max_pages_per_seq=n + 8)
+    slab = pool.swap_page_bytes()
+    rows = DeviceBuffer.from_numpy(rng.standard_normal((n * PAGE, N_KV, HD), dtype=np.float32))
+    res = {}
+    with tempfile.TemporaryDirectory() as tmp:
+        for name, host_pages, disk_pages in (("host", n, 0), ("host256_then_file", 256, n)):
+            pool.prefix_tiers(host_pages * slab, os.path.join(tmp, "tier3.bin") if disk_pages else None,
+                              disk_pages * slab)
+            s = pool.seq_create()
+            pool.seq_reserve(s, n * PAGE)
+            pool.append(0, [s], [0], [n * PAGE], rows, rows, stream)
+            stream.sync()
+            pool.prefix_insert(s, tokens)
+            pool.seq_free(s)
+            t0 = time.perf_counter()
+            freed = pool.prefix_evict(n)
+            pool.swap_wait()
+            t_out = time.perf_counter() - t0
+            t0 = time.perf_counter()
+            s, matched = pool.seq_create_from_prefix(tokens)
+            pool.swap_wait()
+            t_in = time.perf_counter() - t0
+            assert freed == n and matched == n * PAGE
+            res[name] = {"pages": n, "bytes": n * slab, "demote_GBps": round(n * slab / t_out / 1e9, 2),
+                         "promote_GBps": round(n * slab / t_in / 1e9, 2)}
+            pool.seq_free(s)
+            pool.prefix_clear()
+    rows.free()
+    pool.destroy()
+    return {"prefix_tiers": res}
 
 
 def bench_moves(stream) -> dict:

@@ -12,6 +12,7 @@
 #include <cmath>
 
 #include <fcntl.h>
+#include <sys/uio.h>
 #include <unistd.h>
 
 #include "bkv_internal.hpp"
@@ -1264,11 +1265,10 @@ bkv_status bkv_seq_restore(bkv_pool* p, int32_t seq, int32_t lp0, int32_t n,
 }
 
 // ---- lower tiers of the prefix tree ------------------------------------------------------
-// The bytes behind the tree's bookkeeping, in the order the tree listed the moves.  Transfers
-// between the device and the host arena go through the swap path on the side stream (runs of
-// consecutive slots as one transfer); the file is read and written from the host, one page at a
-// time, through the arena or the two-slot bounce buffer.  Work enqueued by later calls waits for
-// `tiers.done` (flush_tables).  A host-only pool keeps the books only.
+// The bytes behind the tree's bookkeeping.  Transfers between the device and the host arena go
+// through the swap path on the side stream (runs of consecutive slots as one transfer); the file
+// is written from the arena and read into a pinned bounce buffer of two halves.  Work enqueued by
+// later calls waits for `tiers.done` (wait_for_tier_moves).  A host-only pool keeps the books only.
 static bkv_status tier_io_failed(bkv_pool* p, const char* what) {
     const std::string msg = std::string("prefix tiers: ") + what + " failed: " + std::strerror(errno) +
                             "; the cached prefixes were dropped";
@@ -1276,59 +1276,135 @@ static bkv_status tier_io_failed(bkv_pool* p, const char* what) {
     return fail(BKV_ERR_STATE, msg);
 }
 
+// Device <-> arena transfers of moves[i..j), all of one kind: independent of each other, so they
+// go in slot order, every run of consecutive slots as one transfer.
+static bkv_status tier_arena_transfers(bkv_pool* p, std::vector<TierMove> run, bool out) {
+    const uint64_t slab = bkv_swap_page_bytes(p);
+    // A slot can be filled twice in one list (its first tenant was dropped again to make room):
+    // the last move into a slot is the one whose bytes stay.
+    std::stable_sort(run.begin(), run.end(),
+                     [](const TierMove& a, const TierMove& b) { return a.host_slot < b.host_slot; });
+    {
+        size_t kept = 0;
+        for (size_t i = 0; i < run.size(); ++i)
+            if (i + 1 == run.size() || run[i + 1].host_slot != run[i].host_slot) run[kept++] = run[i];
+        run.resize(kept);
+    }
+    std::vector<int32_t> pages;
+    for (size_t i = 0; i < run.size();) {
+        size_t j = i + 1;
+        while (j < run.size() && run[j].host_slot == run[j - 1].host_slot + 1) ++j;
+        pages.clear();
+        for (size_t k = i; k < j; ++k) pages.push_back(run[k].page);
+        const bkv_status st = swap_move(p, pages.data(), (int32_t)pages.size(),
+                                        p->tiers.host + (uint64_t)run[i].host_slot * slab, out, p->side);
+        if (st != BKV_OK) return st;
+        i = j;
+    }
+    return BKV_OK;
+}
+
 static bkv_status run_tier_moves(bkv_pool* p, const std::vector<TierMove>& moves) {
     if (moves.empty() || p->host_only) return BKV_OK;
     TierStore& ts = p->tiers;
     const uint64_t slab = bkv_swap_page_bytes(p);
-    bool device_quiet = false;  // every stream's writes to the pages that leave are complete
-    bool side_idle = false;     // nothing is on its way into or out of the arena / bounce buffer
-    int bounce_half = 0;
-    bool half_in_flight[2] = {false, false};  // a copy out of that half of the bounce buffer is enqueued
-    size_t i = 0;
-    while (i < moves.size()) {
-        const TierMove& m = moves[i];
-        if (m.kind == TierMove::DeviceToHost || m.kind == TierMove::HostToDevice) {
+    // The list is an eviction (arena -> file and device -> arena moves, interleaved victim by
+    // victim) followed by a promotion (arena -> device, then file -> device).  The eviction's moves
+    // are queued and go out in batches -- first the queued file writes (gathered over consecutive
+    // file slots), then the queued copies (merged over consecutive arena slots) -- which keeps the
+    // list's order wherever it matters: a slot's write before the copy that refills it.  Only a
+    // write that reads a slot a queued copy fills needs the batch out and finished first.
+    size_t n_evict = 0;
+    while (n_evict < moves.size() && (moves[n_evict].kind == TierMove::DeviceToHost ||
+                                      moves[n_evict].kind == TierMove::HostToDisk))
+        ++n_evict;
+    if (n_evict > 0) {
+        // the pages that leave were written on streams this call does not know, and the arena slots
+        // that go on to the file may still be on their way in
+        BKV_HIP(hipDeviceSynchronize());
+        std::vector<TierMove> writes, copies;
+        std::unordered_map<int32_t, int> copy_slots;
+        const auto flush = [&](bool wait) -> bkv_status {
+            for (size_t i = 0; i < writes.size();) {
+                size_t j = i + 1;
+                while (j < writes.size() && j - i < 512 && writes[j].disk_slot == writes[j - 1].disk_slot + 1) ++j;
+                std::vector<iovec> iov(j - i);
+                for (size_t k = i; k < j; ++k) {
+                    iov[k - i].iov_base = ts.host + (uint64_t)writes[k].host_slot * slab;
+                    iov[k - i].iov_len = slab;
+                }
+                const ssize_t w = ::pwritev(ts.fd, iov.data(), (int)iov.size(),
+                                            (off_t)((uint64_t)writes[i].disk_slot * slab));
+                if (w < 0) return tier_io_failed(p, "a write to the disk tier");
+                // a short write: the slots it did not finish go out one by one
+                for (size_t k = i + (size_t)w / slab; k < j; ++k)
+                    if (::pwrite(ts.fd, ts.host + (uint64_t)writes[k].host_slot * slab, slab,
+                                 (off_t)((uint64_t)writes[k].disk_slot * slab)) != (ssize_t)slab)
+                        return tier_io_failed(p, "a write to the disk tier");
+                i = j;
+            }
+            writes.clear();
+            if (!copies.empty()) {
+                const bkv_status st = tier_arena_transfers(p, copies, true);
+                if (st != BKV_OK) return st;
+                copies.clear();
+                copy_slots.clear();
+                if (wait) BKV_HIP(hipStreamSynchronize(p->side));
+            }
+            return BKV_OK;
+        };
+        for (size_t i = 0; i < n_evict; ++i) {
+            const TierMove& m = moves[i];
+            if (m.kind == TierMove::HostToDisk) {
+                if (copy_slots.count(m.host_slot)) {
+                    const bkv_status st = flush(true);
+                    if (st != BKV_OK) return st;
+                }
+                writes.push_back(m);
+            } else {
+                copies.push_back(m);
+                copy_slots[m.host_slot] = 1;
+            }
+        }
+        const bkv_status st = flush(false);
+        if (st != BKV_OK) return st;
+    }
+    // ---- promotion ---------------------------------------------------------------------------
+    std::vector<TierMove> from_host, from_disk;
+    for (size_t i = n_evict; i < moves.size(); ++i)
+        (moves[i].kind == TierMove::HostToDevice ? from_host : from_disk).push_back(moves[i]);
+    if (!from_host.empty()) {
+        const bkv_status st = tier_arena_transfers(p, from_host, false);
+        if (st != BKV_OK) return st;
+    }
+    if (!from_disk.empty()) {
+        // file -> one half of the bounce buffer -> device, runs of consecutive file slots as one
+        // read; the next read overlaps the previous half's upload
+        std::sort(from_disk.begin(), from_disk.end(),
+                  [](const TierMove& a, const TierMove& b) { return a.disk_slot < b.disk_slot; });
+        bool half_in_flight[2] = {false, false};
+        int half = 0;
+        std::vector<int32_t> pages;
+        for (size_t i = 0; i < from_disk.size();) {
             size_t j = i + 1;
-            while (j < moves.size() && moves[j].kind == m.kind && moves[j].host_slot == moves[j - 1].host_slot + 1) ++j;
-            std::vector<int32_t> pages;
-            for (size_t k = i; k < j; ++k) pages.push_back(moves[k].page);
-            const bool out = m.kind == TierMove::DeviceToHost;
-            if (out && !device_quiet) {
-                // the pages were written on streams this call does not know
-                BKV_HIP(hipDeviceSynchronize());
-                device_quiet = true;
+            while (j < from_disk.size() && j - i < (size_t)ts.bounce_slots &&
+                   from_disk[j].disk_slot == from_disk[j - 1].disk_slot + 1)
+                ++j;
+            uint8_t* buf = ts.bounce + (uint64_t)half * ts.bounce_slots * slab;
+            if (half_in_flight[half]) {
+                BKV_HIP(hipStreamSynchronize(p->side));
+                half_in_flight[0] = half_in_flight[1] = false;
             }
-            const bkv_status st = swap_move(p, pages.data(), (int32_t)pages.size(),
-                                            ts.host + (uint64_t)m.host_slot * slab, out, p->side);
+            const uint64_t bytes = (uint64_t)(j - i) * slab;
+            if (::pread(ts.fd, buf, bytes, (off_t)((uint64_t)from_disk[i].disk_slot * slab)) != (ssize_t)bytes)
+                return tier_io_failed(p, "a read from the disk tier");
+            pages.clear();
+            for (size_t k = i; k < j; ++k) pages.push_back(from_disk[k].page);
+            const bkv_status st = swap_move(p, pages.data(), (int32_t)pages.size(), buf, false, p->side);
             if (st != BKV_OK) return st;
-            side_idle = false;
+            half_in_flight[half] = true;
+            half ^= 1;
             i = j;
-        } else if (m.kind == TierMove::HostToDisk) {
-            if (!side_idle) {
-                BKV_HIP(hipStreamSynchronize(p->side));
-                side_idle = true;
-                half_in_flight[0] = half_in_flight[1] = false;
-            }
-            const ssize_t w = ::pwrite(ts.fd, ts.host + (uint64_t)m.host_slot * slab, slab,
-                                       (off_t)((uint64_t)m.disk_slot * slab));
-            if (w != (ssize_t)slab) return tier_io_failed(p, "a write to the disk tier");
-            ++i;
-        } else {
-            // file -> bounce half -> device; the other half may still be on its way
-            uint8_t* half = ts.bounce + (uint64_t)bounce_half * slab;
-            if (half_in_flight[bounce_half]) {
-                BKV_HIP(hipStreamSynchronize(p->side));
-                side_idle = true;
-                half_in_flight[0] = half_in_flight[1] = false;
-            }
-            const ssize_t r = ::pread(ts.fd, half, slab, (off_t)((uint64_t)m.disk_slot * slab));
-            if (r != (ssize_t)slab) return tier_io_failed(p, "a read from the disk tier");
-            const bkv_status st = swap_move(p, &m.page, 1, half, false, p->side);
-            if (st != BKV_OK) return st;
-            side_idle = false;
-            half_in_flight[bounce_half] = true;
-            bounce_half ^= 1;
-            ++i;
         }
     }
     BKV_HIP(hipEventRecord(ts.done, p->side));
@@ -1376,7 +1452,9 @@ bkv_status bkv_prefix_tiers(bkv_pool* p, uint64_t host_bytes, const char* disk_p
                                              std::strerror(errno));
         if (!p->host_only) {
             void* mem = nullptr;
-            if (hipHostMalloc(&mem, 2 * slab, hipHostMallocDefault) != hipSuccess) {
+            // two halves of up to 4 MiB
+            ts.bounce_slots = (int32_t)std::max<uint64_t>(1, std::min<uint64_t>(((uint64_t)4 << 20) / slab, disk_slots));
+            if (hipHostMalloc(&mem, 2 * (uint64_t)ts.bounce_slots * slab, hipHostMallocDefault) != hipSuccess) {
                 (void)hipGetLastError();
                 return fail(BKV_ERR_NOMEM, "prefix_tiers: cannot pin the bounce buffer of the disk tier");
             }

@@ -76,7 +76,8 @@ struct TierStore {
     int32_t host_slots = 0;
     int fd = -1;                // the file of the disk tier
     int32_t disk_slots = 0;
-    uint8_t* bounce = nullptr;  // one pinned slot between the file and the device
+    uint8_t* bounce = nullptr;  // pinned, between the file and the device: two halves of
+    int32_t bounce_slots = 0;   // bounce_slots slots each
     hipEvent_t done = nullptr;  // behind the last transfer enqueued on the side stream
     bool pending = false;       // `done` may not have completed yet
 };

@@ -116,10 +116,17 @@ void PrefixTree::release_place(Node* n) {
     n->slot = -1;
 }
 
+// Chains are as deep as a sequence is long (one node per page), so nothing here recurses: the
+// nodes below n are listed parents first and then released, and destroyed, from the far end.
 void PrefixTree::release_children(Node* n) {
-    for (auto& kv : n->children) {
-        release_children(kv.second.get());
-        release_place(kv.second.get());
+    std::vector<Node*> below;
+    walk(n, [&](Node* c) {
+        below.push_back(c);
+        return true;
+    });
+    for (size_t i = below.size(); i-- > 0;) {
+        release_place(below[i]);
+        below[i]->children.clear();  // its own children are gone already
     }
     n->children.clear();
 }
@@ -145,42 +152,81 @@ bool PrefixTree::device_candidate(const Node* n) const {
            !has_child_in(n, Tier::Device);
 }
 
-void PrefixTree::collect_device_candidates(Node* n, std::vector<Node*>& out) {
-    for (auto& kv : n->children) {
-        Node* c = kv.second.get();
-        if (c->tier != Tier::Device) continue;  // nothing on the device below a lower tier
-        if (device_candidate(c)) out.push_back(c);
-        collect_device_candidates(c, out);
+// f(node) for every node below `from`, parents before children; f returns whether to go below
+// the node it was given.
+template <typename F>
+void PrefixTree::walk(Node* from, F f) const {
+    std::vector<Node*> stack;
+    for (auto& kv : from->children) stack.push_back(kv.second.get());
+    while (!stack.empty()) {
+        Node* c = stack.back();
+        stack.pop_back();
+        if (!f(c)) continue;
+        for (auto& kv : c->children) stack.push_back(kv.second.get());
     }
 }
 
-template <typename Pred>
-void PrefixTree::oldest_where(Node* n, Pred pred, Node*& best) {
-    for (auto& kv : n->children) {
-        Node* c = kv.second.get();
-        if (pred(c) && (!best || c->last_use < best->last_use)) best = c;
-        oldest_where(c, pred, best);
-    }
+void PrefixTree::collect_device_candidates(Node* n, std::vector<Node*>& out) {
+    walk(n, [&](Node* c) {
+        if (c->tier != Tier::Device) return false;  // nothing on the device below a lower tier
+        if (device_candidate(c)) out.push_back(c);
+        return true;
+    });
+}
+
+// Least-recently-used first.
+static bool newer(const PrefixTree::Node* a, const PrefixTree::Node* b) { return a->last_use > b->last_use; }
+
+bool PrefixTree::host_candidate(const Node* c) const {
+    return c->tier == Tier::Host && c->pins == 0 && !has_child_in(c, Tier::Host);
+}
+static bool disk_leaf(const PrefixTree::Node* c) {
+    return c->tier == Tier::Disk && c->pins == 0 && c->children.empty();
+}
+
+// The lower tiers' candidates of one evict() call, each list built by one walk when it is first
+// needed and kept up to date after that: a node only ever becomes a candidate during the call
+// (its last host child left, it arrived without one), and leaves the lists when it is taken.
+void PrefixTree::LowerQueues::build(PrefixTree& t) {
+    host.clear();
+    disk.clear();
+    t.walk(&t.root_, [&](Node* c) {
+        if (t.host_candidate(c)) host.push_back(c);
+        if (disk_leaf(c)) disk.push_back(c);
+        return true;
+    });
+    std::make_heap(host.begin(), host.end(), newer);
+    std::make_heap(disk.begin(), disk.end(), newer);
+    built = true;
+}
+void PrefixTree::LowerQueues::push(std::vector<Node*>& heap, Node* n) {
+    heap.push_back(n);
+    std::push_heap(heap.begin(), heap.end(), newer);
+}
+PrefixTree::Node* PrefixTree::LowerQueues::pop(std::vector<Node*>& heap) {
+    if (heap.empty()) return nullptr;
+    std::pop_heap(heap.begin(), heap.end(), newer);
+    Node* n = heap.back();
+    heap.pop_back();
+    return n;
 }
 
 // One free slot in the host arena: its least recently used node without a host child goes to
 // the file (whose own least recently used leaf is dropped when it is full), or is dropped with
 // what hangs below it when there is no file to take it.
-bool PrefixTree::make_host_room(std::vector<TierMove>& moves) {
-    Node* h = nullptr;
-    oldest_where(&root_, [this](const Node* c) {
-        return c->tier == Tier::Host && c->pins == 0 && !has_child_in(c, Tier::Host);
-    }, h);
+bool PrefixTree::make_host_room(std::vector<TierMove>& moves, LowerQueues& q) {
+    if (!q.built) q.build(*this);
+    Node* h = q.pop(q.host);
     if (!h) return false;
+    Node* parent = h->parent;
+    bool moved = false;
     if (disk_.capacity() > 0) {
         int32_t d = disk_.take();
         if (d < 0) {
-            Node* leaf = nullptr;
-            oldest_where(&root_, [](const Node* c) {
-                return c->tier == Tier::Disk && c->pins == 0 && c->children.empty();
-            }, leaf);
-            if (leaf) {
+            if (Node* leaf = q.pop(q.disk)) {
+                Node* lp = leaf->parent;
                 drop_subtree(leaf);
+                if (lp != &root_ && disk_leaf(lp)) q.push(q.disk, lp);
                 d = disk_.take();
             }
         }
@@ -192,10 +238,16 @@ bool PrefixTree::make_host_room(std::vector<TierMove>& moves) {
             ++stats_.to_disk;
             h->tier = Tier::Disk;
             h->slot = d;
-            return true;
+            if (disk_leaf(h)) q.push(q.disk, h);
+            moved = true;
         }
     }
-    drop_subtree(h);
+    if (!moved) {
+        // what hangs below h may sit in the lists: they are rebuilt when next needed
+        if (!h->children.empty()) q.built = false;
+        drop_subtree(h);
+    }
+    if (q.built && parent != &root_ && host_candidate(parent)) q.push(q.host, parent);
     return true;
 }
 
@@ -207,6 +259,7 @@ int32_t PrefixTree::evict(int32_t want, std::vector<TierMove>* moves) {
     std::vector<Node*> heap;
     collect_device_candidates(&root_, heap);
     std::make_heap(heap.begin(), heap.end(), older);
+    LowerQueues lower;
     while (freed < want && !heap.empty()) {
         std::pop_heap(heap.begin(), heap.end(), older);
         Node* victim = heap.back();
@@ -215,7 +268,7 @@ int32_t PrefixTree::evict(int32_t want, std::vector<TierMove>* moves) {
         int32_t slot = -1;
         if (demote) {
             slot = host_.take();
-            if (slot < 0 && make_host_room(*moves)) slot = host_.take();
+            if (slot < 0 && make_host_room(*moves, lower)) slot = host_.take();
         }
         if (slot >= 0) {
             std::string err;
@@ -227,7 +280,9 @@ int32_t PrefixTree::evict(int32_t want, std::vector<TierMove>* moves) {
             victim->tier = Tier::Host;
             victim->page = -1;
             victim->slot = slot;
+            if (lower.built && host_candidate(victim)) lower.push(lower.host, victim);
         } else {
+            if (!victim->children.empty()) lower.built = false;
             drop_subtree(victim);
         }
         ++freed;
@@ -290,15 +345,11 @@ void PrefixTree::pin_nodes(const std::vector<Node*>& chain, int delta) {
 void PrefixTree::drop_lower_tiers() {
     // tiers only go down along a chain: a lower-tier node's whole subtree goes with it
     std::vector<Node*> tops;
-    const std::function<void(Node*)> walk = [&](Node* n) {
-        for (auto& kv : n->children) {
-            if (kv.second->tier != Tier::Device)
-                tops.push_back(kv.second.get());
-            else
-                walk(kv.second.get());
-        }
-    };
-    walk(&root_);
+    walk(&root_, [&](Node* c) {
+        if (c->tier == Tier::Device) return true;
+        tops.push_back(c);
+        return false;
+    });
     for (Node* t : tops) drop_subtree(t);
 }
 
@@ -315,12 +366,11 @@ void PrefixTree::clear() {
 
 // ---- counts and checks ------------------------------------------------------------------------
 void PrefixTree::count(const Node* n, int32_t& pinned, int32_t& evictable) const {
-    for (const auto& kv : n->children) {
-        const Node* c = kv.second.get();
+    walk(const_cast<Node*>(n), [&](Node* c) {
         if (c->pins > 0) ++pinned;
         if (c->tier == Tier::Device && c->pins == 0 && alloc_->refcount(c->page) == 1) ++evictable;
-        count(c, pinned, evictable);
-    }
+        return true;
+    });
 }
 
 int32_t PrefixTree::pinned_nodes() const {
@@ -335,36 +385,31 @@ int32_t PrefixTree::evictable_pages() const {
     return e;
 }
 
-bool PrefixTree::check_node(const Node* n, std::vector<int>& host_seen, std::vector<int>& disk_seen,
-                            int32_t (&by_tier)[3], std::string& err) const {
-    for (const auto& kv : n->children) {
-        const Node* c = kv.second.get();
+bool PrefixTree::check(std::string& err) const {
+    std::vector<int> host_seen((size_t)host_.capacity(), 0), disk_seen((size_t)disk_.capacity(), 0);
+    int32_t by_tier[3] = {0, 0, 0};
+    bool ok = true;
+    walk(const_cast<Node*>(&root_), [&](Node* c) {
+        if (!ok) return false;
         ++by_tier[(int)c->tier];
-        if (n != &root_ && (int)c->tier < (int)n->tier) {
+        if (c->parent != &root_ && (int)c->tier < (int)c->parent->tier) {
             err = "prefix tree: a node sits in a higher tier than its parent";
-            return false;
-        }
-        if (c->tier == Tier::Device) {
+            ok = false;
+        } else if (c->tier == Tier::Device) {
             if (c->page < 0 || c->page >= alloc_->n_pages() || alloc_->external_refs(c->page) < 1) {
                 err = "prefix tree: a device node's page holds no reference of the tree";
-                return false;
+                ok = false;
             }
         } else {
             std::vector<int>& seen = c->tier == Tier::Host ? host_seen : disk_seen;
             if (c->slot < 0 || c->slot >= (int32_t)seen.size() || seen[(size_t)c->slot]++) {
                 err = "prefix tree: a lower-tier slot is out of range or listed twice";
-                return false;
+                ok = false;
             }
         }
-        if (!check_node(c, host_seen, disk_seen, by_tier, err)) return false;
-    }
-    return true;
-}
-
-bool PrefixTree::check(std::string& err) const {
-    std::vector<int> host_seen((size_t)host_.capacity(), 0), disk_seen((size_t)disk_.capacity(), 0);
-    int32_t by_tier[3] = {0, 0, 0};
-    if (!check_node(&root_, host_seen, disk_seen, by_tier, err)) return false;
+        return ok;
+    });
+    if (!ok) return false;
     for (int t = 0; t < 3; ++t)
         if (by_tier[t] != stats_.nodes[t]) {
             err = "prefix tree: the per-tier node counts are off";

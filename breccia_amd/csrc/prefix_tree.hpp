@@ -124,15 +124,21 @@ private:
     bool has_child_in(const Node* n, Tier t) const;
     bool device_candidate(const Node* n) const;
     void collect_device_candidates(Node* n, std::vector<Node*>& out);
-    template <typename Pred>
-    void oldest_where(Node* n, Pred pred, Node*& best);
-    bool make_host_room(std::vector<TierMove>& moves);
+    template <typename F>
+    void walk(Node* from, F f) const;
+    struct LowerQueues {
+        bool built = false;
+        std::vector<Node*> host, disk;  // heaps, least recently used on top
+        void build(PrefixTree& t);
+        static void push(std::vector<Node*>& heap, Node* n);
+        static Node* pop(std::vector<Node*>& heap);
+    };
+    bool host_candidate(const Node* c) const;
+    bool make_host_room(std::vector<TierMove>& moves, LowerQueues& q);
     void drop_subtree(Node* n);  // n and everything below it; n is erased from its parent
     void release_place(Node* n);
     void count(const Node* n, int32_t& pinned, int32_t& evictable) const;
     void release_children(Node* n);
-    bool check_node(const Node* n, std::vector<int>& host_seen, std::vector<int>& disk_seen, int32_t (&by_tier)[3],
-                    std::string& err) const;
 
     PageAllocator* alloc_;
     int32_t page_cells_;

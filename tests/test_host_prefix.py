@@ -342,3 +342,22 @@ def test_randomised_tiered_tree_keeps_every_invariant(tmp_path):
             assert sum(nodes) == pool.prefix_stats()[0]
         nodes, moved = pool.prefix_tier_stats()
         assert moved[0] > 0 and moved[1] > 0 and moved[2] > 0
+
+
+def test_a_very_long_chain_is_walked_without_recursion():
+    # one node per page: a 480k-token prompt is a chain 30000 nodes deep
+    n = 30000
+    with host_pool(n_pages=n + 8, max_seqs=2, per_seq=n + 8) as pool:
+        pool.prefix_tiers(n * pool.swap_page_bytes())
+        prompt = toks(99, n * 16)
+        publish(pool, prompt)
+        assert pool.prefix_stats() == (n, n, 0)
+        pool.check()
+        assert pool.prefix_evict(n) == n
+        assert pool.prefix_tier_stats()[0] == (0, n, 0)
+        s, m = pool.seq_create_from_prefix(prompt)
+        assert m == n * 16
+        pool.seq_free(s)
+        pool.check()
+        pool.prefix_clear()
+        assert pool.prefix_stats() == (0, 0, 0) and pool.free_pages() == n + 8
