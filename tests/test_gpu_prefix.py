@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 from breccia_amd import lib as L
-from breccia_amd.kv import Stream
+from breccia_amd.kv import BkvError, Stream
 from gpu_common import Twin, check_attn
 
 pytestmark = pytest.mark.gpu
@@ -144,3 +144,64 @@ def test_demoted_prefix_comes_back_from_host_memory_and_from_disk_bit_for_bit(tm
         out = tw.decode_attn(0, [s, c], [319, 319], q[[1, 1]], 16)
         assert np.array_equal(out[0].view(np.uint32), out[1].view(np.uint32))
         pool.check()
+
+
+def test_randomised_requests_through_the_tiers_always_read_their_own_bytes(tmp_path):
+    # Requests over a few prompts with shared heads come and go on a pool too small for them, with
+    # a small host arena and a small file below it, so that pages are demoted, spilled, dropped,
+    # promoted and republished in every order.  Whatever a request adopts must hold exactly the
+    # K/V of its own tokens: every gathered row is compared with the rows the first computation of
+    # that (token, position) stored.
+    rng = np.random.Generator(np.random.PCG64(902))
+    heads = [rng.integers(0, 32000, size=16 * 6).astype(np.int32) for _ in range(2)]
+    prompts = []
+    for i in range(6):
+        tail = rng.integers(0, 32000, size=16 * int(rng.integers(4, 12)) + int(rng.integers(0, 16))).astype(np.int32)
+        prompts.append(np.concatenate([heads[i % 2], tail]))
+    with Twin(n_layers=2, n_pages=40, max_seqs=6, max_pages_per_seq=24) as tw:
+        pool = tw.pool
+        slab = pool.swap_page_bytes()
+        pool.prefix_tiers(14 * slab, str(tmp_path / "tier3.bin"), 20 * slab)
+        stored = {}                                    # (layer, prompt, page) -> (k rows, v rows) as gathered
+
+        def serve(i):
+            pr = prompts[i]
+            s, m = pool.seq_create_from_prefix(pr)
+            assert m % 16 == 0 and m <= pr.size
+            try:
+                pool.seq_reserve(s, pr.size)
+            except BkvError:
+                pool.seq_free(s)                       # no room for the rest of it: the request goes away
+                raise
+            for layer in range(2):
+                if m < pr.size:
+                    k, v = kv_of(pr[m:], m, 21 + layer)
+                    tw.append(layer, [s], [m], [k], [v])
+                gk, gv = pool.gather(layer, s, 0, pr.size - pr.size % 16)
+                for pg in range(pr.size // 16):
+                    rows = (gk[16 * pg:16 * pg + 16], gv[16 * pg:16 * pg + 16])
+                    key = (layer, tuple(pr[:16 * pg + 16].tolist()))
+                    if key not in stored:
+                        assert pg * 16 >= m, "an adopted page nobody computed"
+                        stored[key] = (rows[0].copy(), rows[1].copy())
+                    else:
+                        assert np.array_equal(rows[0], stored[key][0]) and np.array_equal(rows[1], stored[key][1]), \
+                            (i, layer, pg, m)
+            pool.prefix_insert(s, pr)
+            return s
+
+        live = []
+        for step in range(80):
+            op = int(rng.integers(0, 4))
+            try:
+                if op <= 1 and len(live) < 3:
+                    live.append(serve(int(rng.integers(0, 6))))
+                elif op == 2 and live:
+                    pool.seq_free(live.pop(int(rng.integers(0, len(live)))))
+                elif op == 3:
+                    pool.prefix_evict(int(rng.integers(1, 12)))
+            except BkvError as e:
+                assert e.status == L.ERR_NO_PAGES, e
+            pool.check()
+        nodes, moved = pool.prefix_tier_stats()
+        assert moved[0] > 20 and moved[1] > 0 and moved[2] > 20, moved
