@@ -11,7 +11,7 @@ rotate so that consecutive steps never touch the same pool bytes.
 
 Prints ONE JSON line.  `value` = algorithmic bytes of a step / wall time of a step, inputs
 resident in HBM.  `roofline` prices the split-K attention kernel alone from HIP events on
-its stream.  `cpu_baseline` is the CPU oracle (a restatement of the reference's scalar f64
+its stream, attached to each of its dispatches (the kernel's own begin and end).  `cpu_baseline` is the CPU oracle (a restatement of the reference's scalar f64
 CPU path) timed on this host on the same workload.  `extra` carries the batch-1 config and
 the byte-move kernels.
 """
@@ -189,7 +189,7 @@ def main() -> int:
     step_bytes = attn_bytes + len(seqs) * APPEND_BYTES_PER_TOKEN
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
-    # ---- roofline: the split-K kernel alone, HIP events on its stream -------------------
+    # ---- roofline: the split-K kernel alone, HIP events attached to its dispatches ---------
     pool.timing_reset()
     pool.timing_enable(True)
     first = args.warmup + args.steps

@@ -123,24 +123,35 @@ bkv_status flush_tables(bkv_pool* p, hipStream_t stream) {
     return BKV_OK;
 }
 
+static hipEvent_t timer_take_event(StageTimer& t) {
+    if (!t.idle.empty()) {
+        hipEvent_t e = t.idle.back();
+        t.idle.pop_back();
+        return e;
+    }
+    hipEvent_t e = nullptr;
+    if (hipEventCreate(&e) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    return e;
+}
+
+bool timer_dispatch_events(bkv_pool* p, int stage, hipEvent_t* start, hipEvent_t* stop) {
+    StageTimer& t = p->timer;
+    if (!t.on) return false;
+    *start = timer_take_event(t);
+    *stop = timer_take_event(t);
+    if (!*start || !*stop) return false;
+    t.open.push_back(StageTimer::Pair{stage, *start, *stop});
+    return true;
+}
+
 StageScope::StageScope(bkv_pool* p, int stage, hipStream_t stream) : stream_(stream) {
     StageTimer& t = p->timer;
     if (!t.on) return;
-    auto take = [&t]() -> hipEvent_t {
-        if (!t.idle.empty()) {
-            hipEvent_t e = t.idle.back();
-            t.idle.pop_back();
-            return e;
-        }
-        hipEvent_t e = nullptr;
-        if (hipEventCreate(&e) != hipSuccess) {
-            (void)hipGetLastError();
-            return nullptr;
-        }
-        return e;
-    };
-    hipEvent_t start = take();
-    hipEvent_t stop = take();
+    hipEvent_t start = timer_take_event(t);
+    hipEvent_t stop = timer_take_event(t);
     if (!start || !stop) return;
     if (hipEventRecord(start, stream) != hipSuccess) {
         (void)hipGetLastError();

@@ -136,6 +136,10 @@ private:
     hipStream_t stream_;
     hipEvent_t stop_ = nullptr;
 };
+// While the pool's timer is on: an event pair registered for `stage` that the caller attaches to
+// one dispatch (hipExtLaunchKernelGGL), which then reports the kernel's own duration, without
+// the event records' own time on the queue.  False (and nothing registered) while it is off.
+bool timer_dispatch_events(bkv_pool* p, int stage, hipEvent_t* start, hipEvent_t* stop);
 bkv_status timer_collect(bkv_pool* p);
 
 // ---- kernel launchers (each validates nothing: callers have checked) ---------

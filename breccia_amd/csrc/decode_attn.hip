@@ -799,7 +799,14 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
     const int32_t total = b.wg_base[b.n];
     const int32_t n_units = total / kp.n_hc;
     const int32_t grid = (n_units + 7) / 8 * 8 * kp.n_hc;
-    {
+    if (a.mfma) {
+        // one work-group per unit, every head of the kv head in it (checked by the caller); while the
+        // pool times its kernels, the events ride on the dispatch
+        hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+        (void)timer_dispatch_events(p, BKV_STAGE_ATTN_SPLIT, &ev_start, &ev_stop);
+        const hipError_t e = launch_decode_attn_mfma(kp, p->g.layout, step, sel, total, stream, ev_start, ev_stop);
+        if (e != hipSuccess) return e;
+    } else {
         StageScope timed(p, BKV_STAGE_ATTN_SPLIT, stream);
         const int layout = p->g.layout;
 #define BKV_LAUNCH(HGV, KE, VE)                                                  \
@@ -809,11 +816,7 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
         else                                                                    \
             decode_attn_kernel<HGV, KE, VE, false><<<grid, kBlock, 0, stream>>>(kp); \
     } while (0)
-        if (a.mfma) {
-            // one work-group per unit, every head of the kv head in it (checked by the caller)
-            const hipError_t e = launch_decode_attn_mfma(kp, layout, step, sel, total, stream);
-            if (e != hipSuccess) return e;
-        } else if (step) {
+        if (step) {
             // f16 pools, dense selection (checked by the caller)
             if (hg == 8)
                 decode_attn_kernel<8, kRowF16, kRowF16, false, true><<<grid, kBlock, 0, stream>>>(kp);

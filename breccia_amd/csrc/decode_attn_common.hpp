@@ -73,7 +73,8 @@ __device__ __forceinline__ bool block_cell_live(uint32_t id, int r, int pos) {
 
 // The split-K kernels on the matrix cores (decode_attn_mfma.hip); `total` work-groups, one per
 // (entry, kv head, page range).
+// `start` / `stop`: optional events attached to the dispatch (its own begin and end time stamps)
 hipError_t launch_decode_attn_mfma(const AttnKernelParams& kp, int layout, bool step, bool sel, int32_t total,
-                                   hipStream_t stream);
+                                   hipStream_t stream, hipEvent_t start = nullptr, hipEvent_t stop = nullptr);
 
 }  // namespace bkv

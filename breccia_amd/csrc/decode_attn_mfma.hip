@@ -2,6 +2,8 @@
 // int8 K/V with f16 block scales and for f16 K + q8_0 V.  Same work decomposition, partial layout
 // and merge kernel as the VALU formulation in decode_attn.hip; must agree with the reference's
 // f64 CPU attend (crates/breccia-kernels/src/qsa/cpu.rs:197-246).
+#include <hip/hip_ext.h>
+
 #include "decode_attn_common.hpp"
 #include "f16_rule.hpp"
 #include "lane_groups.hpp"
@@ -968,24 +970,35 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
 
 }  // namespace
 
+// With `start` / `stop` the two events are attached to the dispatch itself (they take the kernel's
+// own begin and end time stamps, what a profiler's kernel trace reports), otherwise a plain launch.
+template <typename K>
+static void launch_one(K kernel, const AttnKernelParams& kp, int32_t total, hipStream_t stream, hipEvent_t start,
+                       hipEvent_t stop) {
+    if (start && stop)
+        hipExtLaunchKernelGGL(kernel, dim3((unsigned)total), dim3(kBlock), 0, stream, start, stop, 0, kp);
+    else
+        kernel<<<total, kBlock, 0, stream>>>(kp);
+}
+
 hipError_t launch_decode_attn_mfma(const AttnKernelParams& kp, int layout, bool step, bool sel, int32_t total,
-                                   hipStream_t stream) {
+                                   hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
     if (layout == BKV_LAYOUT_I8H) {
         if (step)
-            decode_attn_mfma_i8h_kernel<true><<<total, kBlock, 0, stream>>>(kp);
+            launch_one(decode_attn_mfma_i8h_kernel<true>, kp, total, stream, start, stop);
         else
-            decode_attn_mfma_i8h_kernel<false><<<total, kBlock, 0, stream>>>(kp);
+            launch_one(decode_attn_mfma_i8h_kernel<false>, kp, total, stream, start, stop);
     } else if (layout == BKV_LAYOUT_Q8V) {
         if (step)
-            decode_attn_mfma_q8v_kernel<true><<<total, kBlock, 0, stream>>>(kp);
+            launch_one(decode_attn_mfma_q8v_kernel<true>, kp, total, stream, start, stop);
         else
-            decode_attn_mfma_q8v_kernel<false><<<total, kBlock, 0, stream>>>(kp);
+            launch_one(decode_attn_mfma_q8v_kernel<false>, kp, total, stream, start, stop);
     } else if (step)
-        decode_attn_mfma_kernel<true><<<total, kBlock, 0, stream>>>(kp);
+        launch_one(decode_attn_mfma_kernel<true, false>, kp, total, stream, start, stop);
     else if (sel)
-        decode_attn_mfma_kernel<false, true><<<total, kBlock, 0, stream>>>(kp);
+        launch_one(decode_attn_mfma_kernel<false, true>, kp, total, stream, start, stop);
     else
-        decode_attn_mfma_kernel<false><<<total, kBlock, 0, stream>>>(kp);
+        launch_one(decode_attn_mfma_kernel<false, false>, kp, total, stream, start, stop);
     return hipGetLastError();
 }
 
