@@ -147,26 +147,6 @@ bool timer_dispatch_events(bkv_pool* p, int stage, hipEvent_t* start, hipEvent_t
     return true;
 }
 
-StageScope::StageScope(bkv_pool* p, int stage, hipStream_t stream) : stream_(stream) {
-    StageTimer& t = p->timer;
-    if (!t.on) return;
-    hipEvent_t start = timer_take_event(t);
-    hipEvent_t stop = timer_take_event(t);
-    if (!start || !stop) return;
-    if (hipEventRecord(start, stream) != hipSuccess) {
-        (void)hipGetLastError();
-        return;
-    }
-    stop_ = stop;
-    t.open.push_back(StageTimer::Pair{stage, start, stop});
-}
-
-StageScope::~StageScope() {
-    if (stop_) {
-        if (hipEventRecord(stop_, stream_) != hipSuccess) (void)hipGetLastError();
-    }
-}
-
 bkv_status timer_collect(bkv_pool* p) {
     StageTimer& t = p->timer;
     for (const StageTimer::Pair& pr : t.open) {
@@ -673,10 +653,7 @@ static bkv_status append_rows(bkv_pool* p, int32_t layer, int32_t n_seqs, const 
                                      "aligned");
     st = flush_tables(p, S(stream));
     if (st != BKV_OK) return st;
-    {
-        StageScope timed(p, BKV_STAGE_APPEND, S(stream));
-        BKV_HIP(launch_append(p, layer, b, max_tok, k_dev, v_dev, src_is_f16, S(stream)));
-    }
+    BKV_HIP(launch_append(p, layer, b, max_tok, k_dev, v_dev, src_is_f16, S(stream)));
     if (p->timer.open.size() > 8192) return timer_collect(p);
     return BKV_OK;
 }
@@ -718,11 +695,8 @@ bkv_status bkv_append_kprep(bkv_pool* p, int32_t layer, int32_t n_seqs, const in
                                      "device pointers (table 8-byte aligned)");
     st = flush_tables(p, S(stream));
     if (st != BKV_OK) return st;
-    {
-        StageScope timed(p, BKV_STAGE_APPEND, S(stream));
-        BKV_HIP(launch_append_kprep(p, layer, b, max_tok, k_dev, v_dev, k_gamma_dev, eps,
-                                    rope_table_dev, n_rot, max_pos, positions_dev, S(stream)));
-    }
+    BKV_HIP(launch_append_kprep(p, layer, b, max_tok, k_dev, v_dev, k_gamma_dev, eps,
+                                rope_table_dev, n_rot, max_pos, positions_dev, S(stream)));
     if (p->timer.open.size() > 8192) return timer_collect(p);
     return BKV_OK;
 }
@@ -1097,10 +1071,7 @@ bkv_status bkv_page_copy(bkv_pool* p, const bkv_page_pair* pairs, int32_t n_pair
         int slot;
         st = ring_upload(p, pairs + at, (size_t)n * sizeof(bkv_page_pair), S(stream), &dev, &slot);
         if (st != BKV_OK) return st;
-        {
-            StageScope timed(p, BKV_STAGE_PAGE_COPY, S(stream));
-            BKV_HIP(launch_page_copy(p, static_cast<const bkv_page_pair*>(dev), n, S(stream)));
-        }
+        BKV_HIP(launch_page_copy(p, static_cast<const bkv_page_pair*>(dev), n, S(stream)));
         st = ring_done(p, slot, S(stream));
         if (st != BKV_OK) return st;
     }

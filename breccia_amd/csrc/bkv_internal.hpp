@@ -1,6 +1,7 @@
 // Internal declarations shared by the translation units of libbreccia_kv.so.
 #pragma once
 
+#include <hip/hip_ext.h>
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -125,22 +126,23 @@ bkv_status ring_upload(bkv_pool* p, const void* host_src, size_t bytes, hipStrea
                        void** dev_out, int* slot_out);
 bkv_status ring_done(bkv_pool* p, int slot, hipStream_t stream);
 
-// RAII bracket: records a start event now and a stop event when it goes out of scope,
-// only while the pool's timer is on.
-class StageScope {
-public:
-    StageScope(bkv_pool* p, int stage, hipStream_t stream);
-    ~StageScope();
-
-private:
-    hipStream_t stream_;
-    hipEvent_t stop_ = nullptr;
-};
 // While the pool's timer is on: an event pair registered for `stage` that the caller attaches to
 // one dispatch (hipExtLaunchKernelGGL), which then reports the kernel's own duration, without
 // the event records' own time on the queue.  False (and nothing registered) while it is off.
 bool timer_dispatch_events(bkv_pool* p, int stage, hipEvent_t* start, hipEvent_t* stop);
 bkv_status timer_collect(bkv_pool* p);
+
+// One kernel launch of a timed stage: a plain launch, or, while the pool times its kernels, one
+// that carries an event pair on the dispatch.
+template <typename K, typename... Args>
+inline void launch_staged(bkv_pool* p, int stage, K kernel, dim3 grid, dim3 block, uint32_t lds,
+                          hipStream_t stream, Args... args) {
+    hipEvent_t start = nullptr, stop = nullptr;
+    if (timer_dispatch_events(p, stage, &start, &stop))
+        hipExtLaunchKernelGGL(kernel, grid, block, lds, stream, start, stop, 0, args...);
+    else
+        hipLaunchKernelGGL(kernel, grid, block, lds, stream, args...);
+}
 
 // ---- kernel launchers (each validates nothing: callers have checked) ---------
 struct AppendBatch {
@@ -150,10 +152,10 @@ struct AppendBatch {
     int32_t n_tok[BKV_MAX_BATCH];    // tokens of this sequence
     int32_t src0[BKV_MAX_BATCH];     // first source row in k/v
 };
-hipError_t launch_append(const bkv_pool* p, int32_t layer, const AppendBatch& b, int32_t max_tok,
+hipError_t launch_append(bkv_pool* p, int32_t layer, const AppendBatch& b, int32_t max_tok,
                          const void* k, const void* v, bool src_is_f16, hipStream_t stream);
 
-hipError_t launch_append_kprep(const bkv_pool* p, int32_t layer, const AppendBatch& b, int32_t max_tok,
+hipError_t launch_append_kprep(bkv_pool* p, int32_t layer, const AppendBatch& b, int32_t max_tok,
                                const float* k, const float* v, const float* gamma, float eps,
                                const float* table, int32_t n_rot, int32_t max_pos,
                                const int32_t* positions, hipStream_t stream);
@@ -226,7 +228,7 @@ hipError_t launch_prefill_attn(bkv_pool* p, int32_t layer, const PrefillBatch& b
 // heads one wave carries for a given q-heads-per-kv-head group
 int32_t attn_heads_per_wave(int32_t group);
 
-hipError_t launch_page_copy(const bkv_pool* p, const bkv_page_pair* pairs_dev, int32_t n_pairs,
+hipError_t launch_page_copy(bkv_pool* p, const bkv_page_pair* pairs_dev, int32_t n_pairs,
                             hipStream_t stream);
 // Gather (to_stage=1) / scatter (to_stage=0) whole pages between the pools and a
 // contiguous staging buffer laid out [page][layer][K bytes | V bytes].

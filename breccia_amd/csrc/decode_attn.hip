@@ -807,21 +807,23 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
         const hipError_t e = launch_decode_attn_mfma(kp, p->g.layout, step, sel, total, stream, ev_start, ev_stop);
         if (e != hipSuccess) return e;
     } else {
-        StageScope timed(p, BKV_STAGE_ATTN_SPLIT, stream);
         const int layout = p->g.layout;
-#define BKV_LAUNCH(HGV, KE, VE)                                                  \
-    do {                                                                        \
-        if (sel)                                                                \
-            decode_attn_kernel<HGV, KE, VE, true><<<grid, kBlock, 0, stream>>>(kp);  \
-        else                                                                    \
-            decode_attn_kernel<HGV, KE, VE, false><<<grid, kBlock, 0, stream>>>(kp); \
+        const auto go = [&](auto kernel) {
+            launch_staged(p, BKV_STAGE_ATTN_SPLIT, kernel, dim3((unsigned)grid), dim3(kBlock), 0, stream, kp);
+        };
+#define BKV_LAUNCH(HGV, KE, VE)                              \
+    do {                                                    \
+        if (sel)                                            \
+            go(decode_attn_kernel<HGV, KE, VE, true, false>);  \
+        else                                                \
+            go(decode_attn_kernel<HGV, KE, VE, false, false>); \
     } while (0)
         if (step) {
             // f16 pools, dense selection (checked by the caller)
             if (hg == 8)
-                decode_attn_kernel<8, kRowF16, kRowF16, false, true><<<grid, kBlock, 0, stream>>>(kp);
+                go(decode_attn_kernel<8, kRowF16, kRowF16, false, true>);
             else
-                decode_attn_kernel<4, kRowF16, kRowF16, false, true><<<grid, kBlock, 0, stream>>>(kp);
+                go(decode_attn_kernel<4, kRowF16, kRowF16, false, true>);
         } else if (layout == BKV_LAYOUT_F16) {
             if (hg == 8) BKV_LAUNCH(8, kRowF16, kRowF16); else BKV_LAUNCH(4, kRowF16, kRowF16);
         } else if (layout == BKV_LAYOUT_Q8V) {
@@ -845,10 +847,8 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
     mp.n_q = a.n_q_head;
     mp.group = group;
     mp.hg = hg;
-    {
-        StageScope timed(p, BKV_STAGE_ATTN_MERGE, stream);
-        decode_attn_merge_kernel<<<b.n * a.n_q_head, 64 * kMergeGroups, 0, stream>>>(mp);
-    }
+    launch_staged(p, BKV_STAGE_ATTN_MERGE, decode_attn_merge_kernel, dim3((unsigned)(b.n * a.n_q_head)),
+                  dim3(64 * kMergeGroups), 0, stream, mp);
     return hipGetLastError();
 }
 

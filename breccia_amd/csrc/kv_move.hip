@@ -586,7 +586,7 @@ PoolPtrs pool_ptrs(const bkv_pool* p) {
 }  // namespace
 
 template <typename SrcT>
-static hipError_t launch_append_from(const bkv_pool* p, int32_t layer, const AppendBatch& b,
+static hipError_t launch_append_from(bkv_pool* p, int32_t layer, const AppendBatch& b,
                                      int32_t max_tok, const SrcT* k, const SrcT* v,
                                      hipStream_t stream) {
     const MoveGeom g = move_geom(p);
@@ -602,28 +602,29 @@ static hipError_t launch_append_from(const bkv_pool* p, int32_t layer, const App
     uint8_t* vp = p->v_layer[(size_t)layer];
     switch (p->g.layout) {
         case BKV_LAYOUT_F16:
-            append_f16_kernel<SrcT><<<grid, kBlock, 0, stream>>>(b, g, (uint16_t*)kp, (uint16_t*)vp,
-                                                                p->table_dev, k, v);
+            launch_staged(p, BKV_STAGE_APPEND, append_f16_kernel<SrcT>, grid, dim3(kBlock), 0, stream, b, g,
+                          (uint16_t*)kp, (uint16_t*)vp, (const int32_t*)p->table_dev, k, v);
             break;
         case BKV_LAYOUT_Q8V:
-            append_q8v_kernel<SrcT><<<grid, kBlock, 0, stream>>>(b, g, (uint16_t*)kp, (uint32_t*)vp,
-                                                                p->table_dev, k, v);
+            launch_staged(p, BKV_STAGE_APPEND, append_q8v_kernel<SrcT>, grid, dim3(kBlock), 0, stream, b, g,
+                          (uint16_t*)kp, (uint32_t*)vp, (const int32_t*)p->table_dev, k, v);
             break;
         default:
-            append_i8h_kernel<SrcT><<<grid, kBlock, 0, stream>>>(b, g, kp, vp, p->table_dev, k, v);
+            launch_staged(p, BKV_STAGE_APPEND, append_i8h_kernel<SrcT>, grid, dim3(kBlock), 0, stream, b, g, kp, vp,
+                          (const int32_t*)p->table_dev, k, v);
             break;
     }
     return hipGetLastError();
 }
 
-hipError_t launch_append(const bkv_pool* p, int32_t layer, const AppendBatch& b, int32_t max_tok,
+hipError_t launch_append(bkv_pool* p, int32_t layer, const AppendBatch& b, int32_t max_tok,
                          const void* k, const void* v, bool src_is_f16, hipStream_t stream) {
     if (src_is_f16)
         return launch_append_from(p, layer, b, max_tok, (const uint16_t*)k, (const uint16_t*)v, stream);
     return launch_append_from(p, layer, b, max_tok, (const float*)k, (const float*)v, stream);
 }
 
-hipError_t launch_append_kprep(const bkv_pool* p, int32_t layer, const AppendBatch& b, int32_t max_tok,
+hipError_t launch_append_kprep(bkv_pool* p, int32_t layer, const AppendBatch& b, int32_t max_tok,
                                const float* k, const float* v, const float* gamma, float eps,
                                const float* table, int32_t n_rot, int32_t max_pos,
                                const int32_t* positions, hipStream_t stream) {
@@ -636,8 +637,8 @@ hipError_t launch_append_kprep(const bkv_pool* p, int32_t layer, const AppendBat
     uint8_t* kpl = p->k_layer[(size_t)layer];
     uint8_t* vpl = p->v_layer[(size_t)layer];
     const auto launch = [&](auto layout_tag, auto hd_tag) {
-        append_kprep_kernel<decltype(layout_tag)::value, decltype(hd_tag)::value>
-            <<<grid, kBlock, lds, stream>>>(b, g, kp, kpl, vpl, p->table_dev, k, v);
+        launch_staged(p, BKV_STAGE_APPEND, append_kprep_kernel<decltype(layout_tag)::value, decltype(hd_tag)::value>,
+                      grid, dim3(kBlock), (uint32_t)lds, stream, b, g, kp, kpl, vpl, (const int32_t*)p->table_dev, k, v);
     };
     const auto by_hd = [&](auto layout_tag) {
         if (g.hd == 256)
@@ -659,7 +660,7 @@ hipError_t launch_append_kprep(const bkv_pool* p, int32_t layer, const AppendBat
     return hipGetLastError();
 }
 
-hipError_t launch_page_copy(const bkv_pool* p, const bkv_page_pair* pairs_dev, int32_t n_pairs,
+hipError_t launch_page_copy(bkv_pool* p, const bkv_page_pair* pairs_dev, int32_t n_pairs,
                             hipStream_t stream) {
     const PoolPtrs pp = pool_ptrs(p);
     const uint32_t chunks_k = (uint32_t)((pp.k_page_bytes / 16 + 4 * kBlock - 1) / (4 * kBlock));
@@ -668,8 +669,8 @@ hipError_t launch_page_copy(const bkv_pool* p, const bkv_page_pair* pairs_dev, i
     uint64_t grid = total;
     const uint64_t cap = (uint64_t)(p->n_cu > 0 ? p->n_cu : 256) * 32;
     if (grid > cap) grid = cap;
-    page_copy_kernel<<<(unsigned)grid, kBlock, 0, stream>>>(pp, pairs_dev, (uint32_t)n_pairs, chunks_k,
-                                                         chunks_v);
+    launch_staged(p, BKV_STAGE_PAGE_COPY, page_copy_kernel, dim3((unsigned)grid), dim3(kBlock), 0, stream, pp,
+                  pairs_dev, (uint32_t)n_pairs, chunks_k, chunks_v);
     return hipGetLastError();
 }
 

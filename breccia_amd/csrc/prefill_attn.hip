@@ -528,13 +528,15 @@ hipError_t launch_prefill_attn(bkv_pool* p, int32_t layer, const PrefillBatch& b
     kp.scale_log2e = a.scale * kLog2e;
     const int32_t grid = b.wg_base[b.n];
     if (grid == 0) return hipSuccess;
-    StageScope timed(p, BKV_STAGE_ATTN_SPLIT, stream);
     if (p->g.layout == BKV_LAYOUT_Q8V)
-        prefill_attn_kernel<BKV_LAYOUT_Q8V><<<grid, 512, 0, stream>>>(kp);
+        launch_staged(p, BKV_STAGE_ATTN_SPLIT, prefill_attn_kernel<BKV_LAYOUT_Q8V>, dim3((unsigned)grid), dim3(512), 0,
+                      stream, kp);
     else if (p->g.layout == BKV_LAYOUT_I8H)
-        prefill_attn_kernel<BKV_LAYOUT_I8H><<<grid, 512, 0, stream>>>(kp);
+        launch_staged(p, BKV_STAGE_ATTN_SPLIT, prefill_attn_kernel<BKV_LAYOUT_I8H>, dim3((unsigned)grid), dim3(512), 0,
+                      stream, kp);
     else
-        prefill_attn_kernel<BKV_LAYOUT_F16><<<grid, 256, 0, stream>>>(kp);
+        launch_staged(p, BKV_STAGE_ATTN_SPLIT, prefill_attn_kernel<BKV_LAYOUT_F16>, dim3((unsigned)grid), dim3(256), 0,
+                      stream, kp);
     return hipGetLastError();
 }
 

@@ -411,12 +411,11 @@ bkv_status bkv_gather(bkv_pool *pool, int32_t layer, int32_t seq, int64_t cell0,
 /* ---- per-kernel GPU timing ------------------------------------------------------
  * The analogue of Qsa::stage_timings / Pipe::run_timed (qsa/mod.rs:1733-1970,
  * ops/mod.rs:251-274): while enabled, every hot-path call times each of its kernels
- * with events on the call's stream: the matrix-core attention kernels carry their pair
- * on the dispatch itself (the kernel's own begin and end time stamps, what a profiler's
- * kernel trace reports), every other kernel is bracketed by two event records, which
- * add 2-4 us of queue time to what they measure.  bkv_timing_read waits for the events
- * and returns launches and summed milliseconds of one stage since the last reset.
- * Adds gaps between kernels: do not leave it on in production. */
+ * with an event pair that rides on the kernel's dispatch (hipExtLaunchKernelGGL): it
+ * reads the kernel's own begin and end time stamps, what a profiler's kernel trace
+ * reports, free of the queue time that event records around a launch would add.
+ * bkv_timing_read waits for the events and returns launches and summed milliseconds of
+ * one stage since the last reset.  Debug / benchmark only. */
 typedef enum bkv_stage {
     BKV_STAGE_APPEND = 0,
     BKV_STAGE_ATTN_SPLIT = 1, /* split-K online-softmax kernel (the dominant one) */
