@@ -74,5 +74,19 @@ def build_cpp_mirror_test(verbose: bool = False) -> str:
     return out
 
 
+def build_tree_sanitize_test(verbose: bool = False) -> str:
+    """The randomised allocator / prefix-tree exercise (tests/cpp), host code only, built with the
+    address and undefined-behaviour sanitizers."""
+    root = os.path.abspath(os.path.join(HERE, ".."))
+    out = os.path.join(root, "tests", "cpp", "tree_sanitize_test")
+    cmd = ["g++", "-std=c++17", "-O1", "-g", "-Wall", "-fsanitize=address,undefined", "-fno-omit-frame-pointer",
+           os.path.join(root, "tests", "cpp", "tree_sanitize_test.cpp"), os.path.join(CSRC, "allocator.cpp"),
+           os.path.join(CSRC, "prefix_tree.cpp"), "-o", out]
+    if verbose:
+        print(" ".join(cmd))
+    _run(cmd)
+    return out
+
+
 if __name__ == "__main__":
     print(build(verbose=True))
