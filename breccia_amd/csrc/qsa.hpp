@@ -16,7 +16,8 @@
 // apply() launches the split-K kernel plus the merge (which applies sigmoid(gate) read in
 // place from q_full at h*2*head_dim + head_dim + d, as shaders/qsa_attn_apply.comp does);
 // apply() attends the lists in ws.ids / ws.counts once select() or topk_dense() has filled
-// them, and every cell 0..=pos otherwise.
+// them, and every cell 0..=pos otherwise -- through the chunk kernel from GQA_MIN_TOKENS tokens
+// on, as the reference switches to its kv-head-group kernels there (qsa/mod.rs:132-143).
 #pragma once
 
 #include <cstddef>
@@ -38,6 +39,7 @@ constexpr int IDX_N_HEAD = 4;         // qsa/mod.rs:77
 constexpr int IDX_DIM = 128;          // qsa/mod.rs:79
 constexpr int IDX_BLOCK = 4;          // qsa/mod.rs:81
 constexpr int IDX_TOPK_BLOCKS = 512;  // qsa/mod.rs:85 (IDX_TOP_K 2048 cells / IDX_BLOCK)
+constexpr int GQA_MIN_TOKENS = 16;    // qsa/mod.rs:135: calls of at least this many tokens take the chunk kernels
 constexpr int MODEL_N_ROT = 64;       // ops/mod.rs:454
 constexpr float MODEL_RMS_EPS = 1e-6f;  // ops/mod.rs:316
 
@@ -228,8 +230,8 @@ public:
             throw Error(BKV_ERR_RANGE, "attend: cells " + std::to_string(pos0) + ".." +
                                            std::to_string(pos0 + ws.tokens) + " exceed the cache's " +
                                            std::to_string(state.capacity_cells));
-        if (ws.tokens > BKV_MAX_BATCH)
-            throw Error(BKV_ERR_INVALID, "attend: decode shapes only (tokens <= " +
+        if (ws.selected && ws.tokens > BKV_MAX_BATCH)
+            throw Error(BKV_ERR_INVALID, "attend: selection lists are a decode shape (tokens <= " +
                                              std::to_string(BKV_MAX_BATCH) + ")");
     }
 
@@ -246,6 +248,16 @@ public:
                                          ws.q, ws.q_full + hd, (int64_t)n_head_ * 2 * hd, 2 * hd, 0.0625f,
                                          ws.ids, (int64_t)ws.max_ids, ws.counts, (int32_t)ws.max_ids,
                                          ws.attn_out, stream_));
+            return;
+        }
+        if (ws.tokens >= (size_t)GQA_MIN_TOKENS) {
+            // a chunk: the reference's kv-head-group kernels (qsa/mod.rs:132-143), here the
+            // matrix-core chunk kernel -- one call, every row of the chunk, K/V read once per block
+            // of query rows
+            const int64_t p0 = (int64_t)pos0;
+            const int32_t n = (int32_t)ws.tokens;
+            check(bkv_prefill_attn(state.pool, 0, 1, &state.seq, &p0, &n, n_head_, ws.q, ws.q_full + hd,
+                                   (int64_t)n_head_ * 2 * hd, 2 * hd, 0.0625f, ws.attn_out, stream_));
             return;
         }
         check(bkv_decode_attn(state.pool, 0, (int32_t)ws.tokens, seqs.data(), pos.data(), n_head_, ws.q,

@@ -122,9 +122,10 @@ static void test_layout_recipe() {
     state.release();
 }
 
-static void test_attention() {
-    // 24 heads, gate read in place from q_full, T = 3 decode tokens after a 61-cell prefill
-    const int cells = 64, T = 3, H = MODEL_N_HEAD, hd = MODEL_HEAD_DIM;
+static void test_attention(const int T, const size_t pos0) {
+    // 24 heads, gate read in place from q_full: T = 3 decode tokens after a 61-cell prefill, and a
+    // chunk of 40 tokens at cells 24.., which apply() sends through the chunk kernel
+    const int cells = 64, H = MODEL_N_HEAD, hd = MODEL_HEAD_DIM;
     QsaState state = QsaState::create(cells, 64);
     Qsa qsa;
     const bkvo_geom g{2, 256, 16};
@@ -141,7 +142,6 @@ static void test_attention() {
     QsaWorkspace ws = qsa.workspace(T, cells);
     upload(ws.q, q);
     upload(ws.q_full, q_full);
-    const size_t pos0 = 61;
     qsa.attend(state, ws, pos0);
     qsa.apply(state, ws, pos0);
     check(bkv_device_sync());
@@ -171,7 +171,7 @@ static void test_attention() {
 
     bool threw = false;
     try {
-        qsa.apply(state, ws, 62);  // 62 + 3 tokens > 64 cells
+        qsa.apply(state, ws, pos0 + 1);  // one cell past the cache's 64
     } catch (const Error& e) {
         threw = e.status == BKV_ERR_RANGE;
     }
@@ -304,7 +304,8 @@ int main() {
     try {
         test_errors();
         test_layout_recipe();
-        test_attention();
+        test_attention(3, 61);
+        test_attention(40, 24);
         test_k_prep_append();
         test_selection_then_attention();
     } catch (const Error& e) {
