@@ -195,7 +195,9 @@ bkv_status bkv_prefix_clear(bkv_pool *pool);
  *   waits for them on the device on its own stream -- writes through bkv_pool_layer_ptr are
  *   the caller's to order (bkv_swap_wait) -- and the host does not block except for file I/O
  *   and for the synchronisation before pages leave the device (the streams that wrote them
- *   are not known to the call).  host_bytes = 0 switches the tiers off and drops what they
+ *   are not known to the call) -- so with tiers configured bkv_seq_reserve, bkv_prefix_evict
+ *   and bkv_seq_create_from_prefix must not be called while a stream is being captured
+ *   into a graph.  host_bytes = 0 switches the tiers off and drops what they
  *   hold; calling it again resizes them the same way.  An I/O error on the file drops every
  *   cached prefix and reports BKV_ERR_STATE.
  * bkv_prefix_tier_stats: nodes_by_tier[3] = pages on the device / in host memory / on disk;
