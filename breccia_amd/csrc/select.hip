@@ -30,6 +30,8 @@ constexpr int kMaxIdxDim = 128;
 
 constexpr int kTopkThreads = 1024;
 constexpr int kMaxTopk = 2048;    // candidates the sort network holds in LDS
+constexpr int kHistCopies = 16;   // copies of the radix histogram (a power of two)
+constexpr int kRankKeys = 256;    // keys of a radix bin that are ranked directly instead of split further
 
 struct ScoreParams {
     SelectBatch b;
@@ -252,13 +254,19 @@ struct TopkParams {
 // context), 32 up to 32768 (128k); longer lists re-read their scores on every pass.
 template <typename T, int kRegKeys>
 __global__ __launch_bounds__(kTopkThreads) void topk_blocks_kernel(const TopkParams P) {
-    __shared__ int hist[256];
+    // kHistCopies copies of the 256 bins, a lane adds to copy lane % kHistCopies: scores cluster in a
+    // few bins of the first digit (its top bits are exponent bits), and LDS atomics of one wave on
+    // one address run one after the other.  257 ints per copy put equal bins of different copies in
+    // different banks.
+    __shared__ int hist[kHistCopies][257];
     __shared__ int wave_sums[kTopkThreads / 64];
     __shared__ uint64_t cand_key[kMaxTopk];
     __shared__ uint32_t cand_idx[kMaxTopk];
     __shared__ uint64_t wave_min[kTopkThreads / 64], wave_max[kTopkThreads / 64];
     __shared__ uint64_t sh_prefix;
-    __shared__ int sh_rem, sh_done;
+    __shared__ int sh_rem, sh_done, sh_cnt;
+    __shared__ uint64_t small_key[kRankKeys + 4];
+    __shared__ int small_n;
     __shared__ int sh_present;
 
     const int e = blockIdx.x;
@@ -344,14 +352,14 @@ __global__ __launch_bounds__(kTopkThreads) void topk_blocks_kernel(const TopkPar
             while (!resolved) {
                 const int width = min(8, hi_bit - KeyBits<T>::kLowShift + 1);
                 const int shift = hi_bit - width + 1;
-                if (tid < 256) hist[tid] = 0;
+                for (int i = tid; i < kHistCopies * 257; i += kTopkThreads) (&hist[0][0])[i] = 0;
                 __syncthreads();
                 const uint64_t prefix = sh_prefix;
                 const int rem = sh_rem;
                 for_keys([&](int, uint64_t k) {
                     const bool match = hi_bit == 63 || ((k ^ prefix) >> (hi_bit + 1)) == 0;
                     if (k != 0 && match)
-                        atomicAdd(&hist[(int)((k >> shift) & ((1u << width) - 1u))], 1);
+                        atomicAdd(&hist[tid & (kHistCopies - 1)][(int)((k >> shift) & ((1u << width) - 1u))], 1);
                 });
                 __syncthreads();
                 // The digit of the rem-th largest matching key: wave 0 walks the bins from the top,
@@ -361,7 +369,9 @@ __global__ __launch_bounds__(kTopkThreads) void topk_blocks_kernel(const TopkPar
                     int c[4], mine = 0;
 #pragma unroll
                     for (int u = 0; u < 4; ++u) {
-                        c[u] = hist[255 - 4 * tid - u];
+                        c[u] = 0;
+#pragma unroll
+                        for (int cp = 0; cp < kHistCopies; ++cp) c[u] += hist[cp][255 - 4 * tid - u];
                         mine += c[u];
                     }
                     int inc = mine;
@@ -377,6 +387,7 @@ __global__ __launch_bounds__(kTopkThreads) void topk_blocks_kernel(const TopkPar
                             sh_rem = rem - above;
                             sh_prefix = prefix | ((uint64_t)(255 - 4 * tid - u) << shift);
                             sh_done = above + c[u] == rem;  // the whole bin is wanted
+                            sh_cnt = c[u];
                         }
                         above += c[u];
                     }
@@ -385,6 +396,43 @@ __global__ __launch_bounds__(kTopkThreads) void topk_blocks_kernel(const TopkPar
                 hi_bit = shift - 1;
                 resolved = hi_bit < KeyBits<T>::kLowShift;
                 if (sh_done) break;
+                if (!resolved && sh_cnt <= kRankKeys) {
+                    // Few keys are left in the chosen bin (after one pass over a few thousand spread
+                    // scores, a few dozen): they are listed, every thread ranks one of them against
+                    // the others, and the one that rem of them reach is the threshold -- instead of
+                    // six more passes over the remaining bits.  The list's order is whatever the
+                    // atomics made it; the threshold's value does not depend on it.
+                    if (tid == 0) small_n = 0;
+                    if (tid < kRankKeys + 4) small_key[tid] = 0;
+                    __syncthreads();
+                    const uint64_t chosen = sh_prefix;
+                    const int left = sh_rem;
+                    for_keys([&](int, uint64_t k) {
+                        if (k != 0 && ((k ^ chosen) >> shift) == 0) small_key[atomicAdd(&small_n, 1)] = k;
+                    });
+                    __syncthreads();
+                    const int c = small_n;
+                    if (tid < c) {
+                        const uint64_t mine = small_key[tid];
+                        int greater = 0, equal = 0;
+                        // four independent reads at a time (the list is padded with zeros, which
+                        // rank below every live key)
+                        for (int i = 0; i < c; i += 4) {
+                            const uint64_t o0 = small_key[i], o1 = small_key[i + 1];
+                            const uint64_t o2 = small_key[i + 2], o3 = small_key[i + 3];
+                            greater += (o0 > mine) + (o1 > mine) + (o2 > mine) + (o3 > mine);
+                            equal += (o0 == mine) + (o1 == mine) + (o2 == mine) + (o3 == mine);
+                        }
+                        // equal keys all write the same pair
+                        if (greater < left && left <= greater + equal) {
+                            sh_prefix = mine;
+                            sh_rem = left - greater;
+                        }
+                    }
+                    __syncthreads();
+                    resolved = true;
+                    break;
+                }
             }
             if (resolved && !sh_done) {
                 kth = sh_prefix;
@@ -431,6 +479,42 @@ __global__ __launch_bounds__(kTopkThreads) void topk_blocks_kernel(const TopkPar
             cand_idx[i] = 0xffffffffu;
         }
         __syncthreads();
+        if (padded <= kTopkThreads) {
+            // One candidate per thread, kept in registers: partners less than a wave apart swap
+            // through lane shuffles, the others through LDS.  Same network, same order.
+            uint64_t key = tid < padded ? cand_key[tid] : 0;
+            uint32_t idx = tid < padded ? cand_idx[tid] : 0xffffffffu;
+            for (int k2 = 2; k2 <= padded; k2 <<= 1) {
+                for (int j2 = k2 >> 1; j2 > 0; j2 >>= 1) {
+                    uint64_t pkey;
+                    uint32_t pidx;
+                    if (j2 < 64) {
+                        pkey = (uint64_t)__shfl_xor((unsigned long long)key, j2, 64);
+                        pidx = (uint32_t)__shfl_xor((int)idx, j2, 64);
+                    } else {
+                        __syncthreads();  // the partners of the previous LDS stage have read
+                        if (tid < padded) {
+                            cand_key[tid] = key;
+                            cand_idx[tid] = idx;
+                        }
+                        __syncthreads();
+                        pkey = tid < padded ? cand_key[tid ^ j2] : 0;
+                        pidx = tid < padded ? cand_idx[tid ^ j2] : 0xffffffffu;
+                    }
+                    // a run is in order (first to last) when its k2 bit is clear, reversed otherwise;
+                    // the lower position of a pair keeps the element that comes first in the run's order
+                    const bool in_order = (tid & k2) == 0;
+                    const bool low = (tid & j2) == 0;
+                    const bool mine_first = key > pkey || (key == pkey && idx < pidx);
+                    if (mine_first != (low == in_order)) {
+                        key = pkey;
+                        idx = pidx;
+                    }
+                }
+            }
+            __syncthreads();
+            if (tid < padded) cand_idx[tid] = idx;
+        } else {
         const auto exchange = [&](int a, int b, bool reversed_run) {
             const uint64_t ka = cand_key[a], kb = cand_key[b];
             const uint32_t ia = cand_idx[a], ib = cand_idx[b];
@@ -458,6 +542,7 @@ __global__ __launch_bounds__(kTopkThreads) void topk_blocks_kernel(const TopkPar
                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
                 }
             }
+        }
         }
         __syncthreads();
     }

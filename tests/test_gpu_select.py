@@ -95,6 +95,13 @@ def test_topk_edge_cases():
         got = gpu_topk(pool, sc, [0, 3999], 2048, 2049)
         for i, p in enumerate([0, 3999]):
             assert np.array_equal(got[i], oracle_topk_f32(sc[i], 2048, p // 4, 2049)), i
+        # lists longer than the work-group (more than one candidate per thread in the sort): 1500 and
+        # 2048 kept, scores with ties
+        sc = (rng.integers(0, 4000, size=(2, 6000)).astype(np.float32) - 1000) / 16
+        for keep in (1500, 2048):
+            got = gpu_topk(pool, sc, [4 * 6000, 4 * 6000], keep, keep + 1)
+            for i in range(2):
+                assert np.array_equal(got[i], oracle_topk_f32(sc[i], keep, 6000, keep + 1)), (keep, i)
         # dense: every visible block ascending, own appended when it lies beyond n_blocks
         d = gpu_topk(pool, np.zeros((3, 515), np.float32), [2061, 100, 2059], 512, 600, dense=True)
         assert list(d[0]) == list(range(515)) + [515]
