@@ -465,28 +465,48 @@ bkv_status bkv_prefix_match(bkv_pool* p, const int32_t* tokens, int64_t n_tokens
     return BKV_OK;
 }
 
+// The chain of listed pages that matches tokens[0..n), with its lower part brought back to fresh
+// device pages as far as pages can be had (other cached prefixes make room if they must; the
+// chain itself is held meanwhile).  The transfers are enqueued, not awaited.
+static bkv_status promote_matched_chain(bkv_pool* p, const int32_t* tokens, int64_t n_tokens,
+                                        std::vector<PrefixTree::Node*>& chain) {
+    p->prefix->match_nodes(tokens, n_tokens, true, chain);
+    if ((int64_t)chain.size() > p->alloc->max_pages_per_seq()) chain.resize((size_t)p->alloc->max_pages_per_seq());
+    int32_t lower = 0;
+    for (const PrefixTree::Node* x : chain) lower += PrefixTree::tier_of(x) != Tier::Device;
+    if (lower == 0) return BKV_OK;
+    std::vector<TierMove> moves;
+    p->prefix->pin_nodes(chain, +1);
+    const int32_t missing = lower - p->alloc->free_pages();
+    if (missing > 0) p->prefix->evict(missing, &moves);
+    p->prefix->promote(chain, lower, moves);
+    p->prefix->pin_nodes(chain, -1);
+    return run_tier_moves(p, moves);
+}
+
+bkv_status bkv_prefix_prefetch(bkv_pool* p, const int32_t* tokens, int64_t n_tokens, int64_t* device_tokens) {
+    bkv_status st = prefix_args(p, "prefix_prefetch", tokens, n_tokens);
+    if (st != BKV_OK) return st;
+    std::vector<PrefixTree::Node*> chain;
+    st = promote_matched_chain(p, tokens, n_tokens, chain);
+    if (st != BKV_OK) return st;
+    int64_t on_device = 0;
+    for (const PrefixTree::Node* x : chain) {
+        if (PrefixTree::tier_of(x) != Tier::Device) break;
+        ++on_device;
+    }
+    if (device_tokens) *device_tokens = on_device * p->g.page_cells;
+    return BKV_OK;
+}
+
 bkv_status bkv_seq_create_from_prefix(bkv_pool* p, const int32_t* tokens, int64_t n_tokens,
                                       int32_t* seq_out, int64_t* matched_tokens) {
     bkv_status st = prefix_args(p, "seq_create_from_prefix", tokens, n_tokens);
     if (st != BKV_OK) return st;
     if (!seq_out) return fail(BKV_ERR_INVALID, "seq_create_from_prefix: NULL output");
     std::vector<PrefixTree::Node*> chain;
-    p->prefix->match_nodes(tokens, n_tokens, true, chain);
-    if ((int64_t)chain.size() > p->alloc->max_pages_per_seq()) chain.resize((size_t)p->alloc->max_pages_per_seq());
-    int32_t lower = 0;
-    for (const PrefixTree::Node* x : chain) lower += PrefixTree::tier_of(x) != Tier::Device;
-    if (lower > 0) {
-        // The tail of the chain lives in the lower tiers: it comes back to fresh device pages
-        // (other cached prefixes make room if they must; the chain itself is held meanwhile).
-        std::vector<TierMove> moves;
-        p->prefix->pin_nodes(chain, +1);
-        const int32_t missing = lower - p->alloc->free_pages();
-        if (missing > 0) p->prefix->evict(missing, &moves);
-        p->prefix->promote(chain, lower, moves);
-        p->prefix->pin_nodes(chain, -1);
-        st = run_tier_moves(p, moves);
-        if (st != BKV_OK) return st;
-    }
+    st = promote_matched_chain(p, tokens, n_tokens, chain);
+    if (st != BKV_OK) return st;
     std::vector<int32_t> pages;
     for (const PrefixTree::Node* x : chain) {
         if (PrefixTree::tier_of(x) != Tier::Device) break;

@@ -310,6 +310,13 @@ class Pool:
         path = None if disk_path is None else os.fsencode(disk_path)
         check(lib.bkv_prefix_tiers(self.handle, host_bytes, path, disk_bytes))
 
+    def prefix_prefetch(self, tokens) -> int:
+        """Bring the matched chain's lower tiers back to the device; -> tokens on the device."""
+        tokens, pt = _i32(tokens)
+        m = C.c_int64()
+        check(lib.bkv_prefix_prefetch(self.handle, pt, tokens.size, C.byref(m)))
+        return int(m.value)
+
     def prefix_tier_stats(self):
         """-> ((device, host, disk) nodes, (to_host, to_disk, promoted, dropped) pages moved)"""
         nodes = (C.c_int32 * 3)()

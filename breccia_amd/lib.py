@@ -85,6 +85,7 @@ _SIGNATURES = {
     "bkv_prefix_clear": (C.c_int, [_vp]),
     "bkv_prefix_tiers": (C.c_int, [_vp, _u64, C.c_char_p, _u64]),
     "bkv_prefix_tier_stats": (C.c_int, [_vp, _pi32, C.POINTER(C.c_uint64)]),
+    "bkv_prefix_prefetch": (C.c_int, [_vp, _pi32, _i64, _pi64]),
     "bkv_timing_enable": (C.c_int, [_vp, C.c_int]),
     "bkv_timing_reset": (C.c_int, [_vp]),
     "bkv_timing_read": (C.c_int, [_vp, C.c_int, C.POINTER(_u64), C.POINTER(C.c_double)]),

@@ -205,6 +205,13 @@ bkv_status bkv_prefix_clear(bkv_pool *pool);
 bkv_status bkv_prefix_tiers(bkv_pool *pool, uint64_t host_bytes, const char *disk_path,
                             uint64_t disk_bytes);
 bkv_status bkv_prefix_tier_stats(const bkv_pool *pool, int32_t *nodes_by_tier, uint64_t *moved);
+/* Promotion ahead of a request (the notes' "async, never on the decode critical path", :570-572):
+ * brings the lower part of the chain that matches `tokens` back to device pages, as
+ * bkv_seq_create_from_prefix would, without creating a sequence; the transfers are enqueued on
+ * the side stream and not awaited.  Counts as a use of the chain.  *device_tokens = leading
+ * tokens whose pages are on the device once the transfers are done. */
+bkv_status bkv_prefix_prefetch(bkv_pool *pool, const int32_t *tokens, int64_t n_tokens,
+                               int64_t *device_tokens);
 
 /* ---- hot path ---------------------------------------------------------------
  * bkv_append replaces Qsa::kv_append + shaders/qsa_kv_append.comp (qsa/mod.rs:

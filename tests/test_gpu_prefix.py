@@ -135,8 +135,11 @@ def test_demoted_prefix_comes_back_from_host_memory_and_from_disk_bit_for_bit(tm
         nodes, _ = pool.prefix_tier_stats()
         assert nodes == (0, 20, 0) and pool.prefix_match(prefix) == 320
         pool.fill(0xEE)
+        # promotion ahead of the request: the request then finds its pages on the device
+        assert pool.prefix_prefetch(prefix) == 320
+        promoted = pool.prefix_tier_stats()[1][2]
         s, m = pool.seq_create_from_prefix(prefix)
-        assert m == 320
+        assert m == 320 and pool.prefix_tier_stats()[1][2] == promoted
         c = pool.seq_create()
         pool.seq_reserve(c, 320)
         k, v = kv_of(prefix[:320], 0, 11)

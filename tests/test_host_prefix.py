@@ -300,6 +300,27 @@ def test_promotion_stops_where_the_device_has_no_page_left():
         pool.check()
 
 
+def test_prefetch_promotes_ahead_of_the_request():
+    with host_pool(n_pages=16, max_seqs=4, per_seq=16) as pool:
+        pool.prefix_tiers(64 * pool.swap_page_bytes())
+        a, b = toks(96, 80), toks(97, 80)                       # 5 pages each
+        publish(pool, a)
+        publish(pool, b)
+        assert pool.prefix_evict(10) == 10 and pool.prefix_tier_stats()[0] == (0, 10, 0)
+        assert pool.prefix_prefetch(a) == 80                    # a is back on the device, nobody holds it
+        assert pool.prefix_tier_stats()[0] == (5, 5, 0) and pool.prefix_stats()[1] == 5
+        assert pool.prefix_prefetch(a[:40]) == 32               # already there: nothing moves
+        assert pool.prefix_tier_stats()[1][2] == 5
+        s, m = pool.seq_create_from_prefix(a)                   # the request finds it on the device
+        assert m == 80 and pool.prefix_tier_stats()[1][2] == 5
+        # with 11 pages held elsewhere only part of b can come back
+        hog = pool.seq_create()
+        pool.seq_reserve(hog, 9 * 16)
+        assert pool.prefix_prefetch(b) == 32
+        assert pool.prefix_match(b) == 80
+        pool.check()
+
+
 def test_randomised_tiered_tree_keeps_every_invariant(tmp_path):
     rng = np.random.Generator(np.random.PCG64(51))
     base = [toks(160 + i, 16 * 12) for i in range(5)]
