@@ -102,10 +102,10 @@ struct PageStage<BKV_LAYOUT_I8H> {
 
 template <int LAY>
 struct PrefillLds {
-    // [buffer][K | V (quantised V: high parts, low parts)][16 rows][264 halves]
-    _Float16 img[4][LAY == BKV_LAYOUT_F16 ? 2 : 3][kPage][kLdsRow];
-    float e[LAY == BKV_LAYOUT_Q8V ? 4 : 1][kPage];           // q8_0 V: E of the buffer's cells
-    _Float16 ksc[LAY == BKV_LAYOUT_I8H ? 4 : 1][8][kPage];   // int8 K: scale of [block][row]
+    // [buffer][image][16 rows][264 halves]; images: K, V -- with q8_0 V: K, V high parts, V low
+    // parts -- with int8 K and V: K high, V high, V low, K low parts
+    _Float16 img[4][LAY == BKV_LAYOUT_F16 ? 2 : LAY == BKV_LAYOUT_Q8V ? 3 : 4][kPage][kLdsRow];
+    float e[LAY == BKV_LAYOUT_Q8V ? 4 : 1][kPage];  // q8_0 V: E of the buffer's cells
 };
 
 template <int LAY>
@@ -265,16 +265,21 @@ __global__ __launch_bounds__(LAY == BKV_LAYOUT_F16 ? 256 : 512, LAY == BKV_LAYOU
             *reinterpret_cast<h8*>(&L.img[buf][2][v_row][v_blk * 32 + v_j * 8]) = vl;
             if ((tid & 31) == 0) L.e[buf][v_row] = (float)ee;
         } else if constexpr (I8H) {
-            // K: the codes as the exact f16 numbers they are; their block scales apply to the
-            // blocks' partial scores.  A scale with exponent field 0 reads as zero, as everywhere.
-            h2m kd[4];
-            codes_to_f16(st.kc0, kd[0], kd[1]);
-            codes_to_f16(st.kc1, kd[2], kd[3]);
-            *reinterpret_cast<h8*>(&L.img[buf][0][v_row][v_blk * 32 + v_j * 8]) =
-                h8{kd[0][0], kd[0][1], kd[1][0], kd[1][1], kd[2][0], kd[2][1], kd[3][0], kd[3][1]};
-            if (v_j == 0) {
+            // K: code * scale (7 + 11 significant bits) as hi = f16(code * scale) and the exact
+            // remainder, like V below.  A scale with exponent field 0 reads as zero, as everywhere.
+            {
                 const unsigned short ks = (st.kscale & 0x7c00u) == 0 ? (unsigned short)0 : st.kscale;
-                L.ksc[buf][v_blk][v_row] = __builtin_bit_cast(_Float16, ks);
+                const _Float16 ksc = __builtin_bit_cast(_Float16, ks);
+                const h2m sh = h2m{ksc, ksc}, sl = h2m{(_Float16)0.0f, (_Float16)0.0f};
+                h2m kd[4], hi[4], lo[4];
+                codes_to_f16(st.kc0, kd[0], kd[1]);
+                codes_to_f16(st.kc1, kd[2], kd[3]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) scaled_hi_lo(kd[i], sh, sl, hi[i], lo[i]);
+                *reinterpret_cast<h8*>(&L.img[buf][0][v_row][v_blk * 32 + v_j * 8]) =
+                    h8{hi[0][0], hi[0][1], hi[1][0], hi[1][1], hi[2][0], hi[2][1], hi[3][0], hi[3][1]};
+                *reinterpret_cast<h8*>(&L.img[buf][3][v_row][v_blk * 32 + v_j * 8]) =
+                    h8{lo[0][0], lo[0][1], lo[1][0], lo[1][1], lo[2][0], lo[2][1], lo[3][0], lo[3][1]};
             }
             // V: code * scale (7 + 11 significant bits) as hi = f16(code * scale) and the exact
             // remainder; rows past the work-group's last position become zeros
@@ -311,17 +316,17 @@ __global__ __launch_bounds__(LAY == BKV_LAYOUT_F16 ? 256 : 512, LAY == BKV_LAYOU
         for (int m = 0; m < 8; ++m) kf[m] = *reinterpret_cast<const h8*>(ks + c * kLdsRow + m * 32 + g * 8);
         f4 s;
         if constexpr (I8H) {
-            // a 32-deep MFMA is exactly one block of 32 values: the block's scale of either cell
-            // multiplies its partial sum
-            s = f4{0.0f, 0.0f, 0.0f, 0.0f};
+            // K = hi + lo: hi meets q's high and low parts, lo q's high parts; three chains
+            const _Float16* kl = &L.img[buf][3][0][0];
+            f4 s0 = f4{0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0, s2 = s0;
 #pragma unroll
             for (int m = 0; m < 8; ++m) {
-                const h4 ksr = *reinterpret_cast<const h4*>(&L.ksc[buf][m][4 * g]);
-                f4 part = mfma32(kf[m], qhi[m], f4{0.0f, 0.0f, 0.0f, 0.0f});
-                part = mfma32(kf[m], qlo[m], part);
-#pragma unroll
-                for (int r = 0; r < 4; ++r) s[r] = fmaf((float)ksr[r], part[r], s[r]);
+                const h8 klo = *reinterpret_cast<const h8*>(kl + c * kLdsRow + m * 32 + g * 8);
+                s0 = mfma32(kf[m], qhi[m], s0);
+                s1 = mfma32(kf[m], qlo[m], s1);
+                s2 = mfma32(klo, qhi[m], s2);
             }
+            s = (s0 + s1) + s2;
         } else {
             // four independent accumulation chains: an MFMA that waits for the previous one's
             // result costs its full latency

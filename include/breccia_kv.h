@@ -290,8 +290,7 @@ bkv_status bkv_decode_attn(bkv_pool *pool, int32_t layer, int32_t n, const int32
  * as the exact f16 the cache holds; q and the probabilities are f32 split into two f16 parts,
  * so accuracy is that of f32 accumulation.  q8_0 V blocks (BRECCIA_KV_Q8V in
  * qsa_attn_apply_gqa.comp:53-77) are dequantised once per work-group into two f16 terms whose
- * sum carries code * scale to 22 bits; int8 K codes enter as the exact f16 numbers they are
- * and their block scales multiply the blocks' partial scores.  All three layouts, head_dim
+ * sum carries code * scale to 22 bits, and so are int8 K blocks.  All three layouts, head_dim
  * 256, 16-cell pages.  Written
  * for chunks of tens to thousands of tokens; a handful of tokens is bkv_decode_attn's case. */
 bkv_status bkv_prefill_attn(bkv_pool *pool, int32_t layer, int32_t n_seqs, const int32_t *seqs,
