@@ -35,6 +35,9 @@
 // and the softmax runs over logit + E with weights exp2(logit + E - M) (the denominator sums
 // exp2(logit - M)), as in the decode kernel for this layout: the largest terms have weights near
 // 1 whatever the magnitude of their values.  P.V is then hi.p_hi + hi.p_lo + lo.p_hi.
+// Int8 pools (codes with an f16 scale per 32 values, K and V alike) are dequantised the same way,
+// without the exponent: both K and V become hi/lo image pairs, and the scores are
+// K_hi.q_hi + K_hi.q_lo + K_lo.q_hi.
 #include "bkv_internal.hpp"
 #include "lane_groups.hpp"
 #include "quant_decode.hpp"
