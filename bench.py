@@ -696,21 +696,11 @@ def bench_moves(stream) -> dict:
     ms = timed(lambda: pool.page_copy(pairs[:1], stream), 200)
     res["page_copy_one_us"] = round(ms * 1e3, 2)
 
-    # plain device copy of the same volume (ceiling of a read+write stream on this box)
-    a = DeviceBuffer(512 << 20)
-    c = DeviceBuffer(512 << 20)
-    ms = timed(lambda: check(lib.bkv_copy_probe(c.ptr, a.ptr, 512 << 20, stream.handle)), 10)
-    res["device_copy_probe"] = {"bytes_moved": 2 * (512 << 20), "ms": round(ms, 4),
-                                "GBps": round(2 * (512 << 20) / ms / 1e6, 1)}
-    a.free()
-    c.free()
-
     # swap: 25 % of the live pages out to pinned host and back
     n_swap = 4096
     host = pool.host_alloc(n_swap * pool.swap_page_bytes())
     pages = used[:n_swap].astype(np.int32)
-    # once untimed: the first pass through both staging halves and the side stream pays one-time
-    # costs (a first out-swap reads 29 GB/s, every later one 54)
+    # once untimed: the first pass through the staging halves and the side stream pays one-time costs
     pool.swap_out(pages, host, stream)
     pool.swap_wait()
     pool.swap_in(pages, host, stream)
@@ -729,6 +719,18 @@ def bench_moves(stream) -> dict:
     res["swap"] = {"pages": n_swap, "bytes": b, "out_GBps": round(b / t_out / 1e9, 2),
                    "in_GBps": round(b / t_in / 1e9, 2)}
     host.free()
+
+    # plain device copy of the same volume (ceiling of a read+write stream on this box); after the
+    # swap, because for some tens of milliseconds after large device buffers are freed
+    # device-to-host copies run at half their rate
+    a = DeviceBuffer(512 << 20)
+    c = DeviceBuffer(512 << 20)
+    ms = timed(lambda: check(lib.bkv_copy_probe(c.ptr, a.ptr, 512 << 20, stream.handle)), 10)
+    res["device_copy_probe"] = {"bytes_moved": 2 * (512 << 20), "ms": round(ms, 4),
+                                "GBps": round(2 * (512 << 20) / ms / 1e6, 1)}
+    a.free()
+    c.free()
+
     pool.destroy()
     return res
 
