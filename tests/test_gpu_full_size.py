@@ -5,7 +5,9 @@ configs[4] (batch 16, contexts 8k..128k, int8 K/V with f16 scales): the oracle a
 rows read back through bkv_gather for a seeded subset of sequences (shortest, median, longest --
 all 16 heads each; the full f64 oracle over all 16 sequences is ~10^10 MACs), plus
 size-independent properties on all of them: the batched call equals the per-sequence call to
-1e-6, and every output is a convex combination of V rows (bounded by the largest |v|)."""
+1e-6, and every output is a convex combination of V rows (bounded by the largest |v|).
+configs[3] shape (4 sequences, 2048-token prefix + 1024-token chunk) through the chunk kernel on
+all three layouts: sampled tokens against the oracle, the chunk's tail against the decode kernel."""
 import numpy as np
 import pytest
 
@@ -119,5 +121,49 @@ def test_config5_batch16_int8_8k_128k():
         for i in range(16):
             alone = run_attn(pool, [seqs[i]], [pos[i]], q[i:i + 1])
             assert max_abs(alone[0], out[i]) < 1e-6, i
+    finally:
+        pool.destroy()
+
+
+@pytest.mark.parametrize("layout", [L.LAYOUT_F16, L.LAYOUT_Q8V, L.LAYOUT_I8H])
+def test_config4_shape_prefill_of_1024_token_chunks_on_2048_token_prefixes(layout):
+    # BASELINE configs[3] at full size through the chunk kernel: 4 sequences, a 2048-token prefix in
+    # the cache, a 1024-token chunk each, one call.  Sampled tokens of every sequence against the
+    # oracle (over the rows read back through bkv_gather) at the reference's bar; the chunk's last 64
+    # positions of one sequence against the decode kernel; every output bounded by the largest |v|.
+    rng = np.random.Generator(np.random.PCG64(20250004 + layout))
+    before, t = 2048, 1024
+    ctx = [before + t] * 4
+    live = sum((c + 15) // 16 for c in ctx)
+    pool = Pool(n_layers=1, n_pages=int(np.ceil(live / 0.6)), n_kv_head=N_KV, head_dim=HD, layout=layout,
+                max_seqs=5, max_pages_per_seq=ctx[0] // 16 + 2)
+    pool.set_free_order(rng.permutation(pool.desc.n_pages).astype(np.int32))
+    try:
+        seqs = [pool.seq_create() for _ in ctx]
+        for s in seqs:
+            pool.seq_reserve(s, ctx[0])
+        fill_tiled(pool, seqs, ctx, rng, tile=1024)
+        q = rng.standard_normal((4 * t, N_Q, HD), dtype=np.float32)
+        qd, od = DeviceBuffer.from_numpy(q), DeviceBuffer(q.nbytes)
+        pool.prefill_attn(0, seqs, [before] * 4, [t] * 4, N_Q, qd, od, 1.0 / 16.0)
+        device_sync()
+        out = od.download(np.float32).reshape(4, t, N_Q, HD)
+        assert np.all(np.isfinite(out))
+        worst = 0.0
+        for i, s in enumerate(seqs):
+            k, v = pool.gather(0, s, 0, ctx[i])
+            assert np.abs(out[i]).max() <= np.abs(v).max()
+            for tok in sorted({0, t - 1, t // 2, int(rng.integers(0, t)), int(rng.integers(0, t))}):
+                pos = before + tok
+                want = oracle.attend(q[i * t + tok], k[:pos + 1], v[:pos + 1], oracle.dense_cells(pos), pos, N_Q,
+                                     N_KV, HD, threads=8)
+                _, rel = check_attn(out[i, tok], want, "config4 seq %d token %d" % (i, tok))
+                worst = max(worst, rel)
+        assert worst <= REF_BAR_MAX_REL, worst
+        tail = list(range(ctx[2] - 64, ctx[2]))
+        dec = run_attn(pool, [seqs[2]] * 64, tail, q[2 * t + t - 64:3 * t])
+        assert max_abs(dec, out[2, -64:]) < 5e-6
+        qd.free()
+        od.free()
     finally:
         pool.destroy()
