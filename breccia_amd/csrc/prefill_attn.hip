@@ -445,23 +445,12 @@ __global__ __launch_bounds__(LAY == BKV_LAYOUT_F16 ? 256 : 512, LAY == BKV_LAYOU
                 const h8 a2 = __builtin_bit_cast(h8, fa[2]), a3 = __builtin_bit_cast(h8, fa[3]);
                 const h8 b0 = __builtin_bit_cast(h8, fb[0]), b1 = __builtin_bit_cast(h8, fb[1]);
                 const h8 b2 = __builtin_bit_cast(h8, fb[2]), b3 = __builtin_bit_cast(h8, fb[3]);
-                // four columns at a time: their MFMAs against p's high parts, then those against its
-                // low parts, so that no MFMA follows the one whose sum it adds to
 #pragma unroll
-                for (int t0 = 0; t0 < 8; t0 += 4) {
-                    h8 vv[4];
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        // column 128 h + 8 c + t of the pair's cells 4 g .. of either page
-                        const int t = t0 + j;
-                        vv[j] = h8{a0[t], a1[t], a2[t], a3[t], b0[t], b1[t], b2[t], b3[t]};
-                    }
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) o[h][t0 + j] = mfma32(vv[j], ph, o[h][t0 + j]);
-                    if (img == 1) {
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) o[h][t0 + j] = mfma32(vv[j], pl, o[h][t0 + j]);
-                    }
+                for (int t = 0; t < 8; ++t) {
+                    // column 128 h + 8 c + t of the pair's cells 4 g .. of either page
+                    const h8 vv = h8{a0[t], a1[t], a2[t], a3[t], b0[t], b1[t], b2[t], b3[t]};
+                    o[h][t] = mfma32(vv, ph, o[h][t]);
+                    if (img == 1) o[h][t] = mfma32(vv, pl, o[h][t]);
                 }
             }
         }
