@@ -162,3 +162,50 @@ def test_prefill_errors_come_before_any_launch():
                 tw.pool.prefill_attn(**a)
             assert ei.value.status == status, kw
         z.free()
+
+
+@pytest.mark.parametrize("layout", [L.LAYOUT_F16, L.LAYOUT_Q8V, L.LAYOUT_I8H])
+def test_the_largest_batch_of_chunks_in_one_call(layout):
+    # 64 chunks (the limit of one call) over 8 sequences, lengths 0..70 tokens, several chunks of
+    # one sequence in the same call: every token agrees with the decode kernel at its position, and
+    # a sample with the oracle; 65 chunks are refused
+    rng = np.random.Generator(np.random.PCG64(1030 + layout))
+    with Twin(n_pages=300, max_seqs=10, layout=layout) as tw:
+        tw.pool.set_free_order(rng.permutation(300).astype(np.int32))
+        lens = [int(x) for x in rng.integers(200, 520, size=8)]
+        seqs = [tw.pool.seq_create() for _ in lens]
+        for s, n in zip(seqs, lens):
+            fill(tw, s, n, rng, chunk=256)
+        ent_seq, pos0, n_tok = [], [], []
+        for i in range(64):
+            j = i % 8
+            t = [0, 1, 15, 16, 17, 33, 64, 70][(i // 8 + j) % 8]
+            p0 = int(rng.integers(0, lens[j] - t + 1))
+            ent_seq.append(seqs[j])
+            pos0.append(p0)
+            n_tok.append(t)
+        qs = [rng.standard_normal((t, 16, 256)).astype(np.float32) for t in n_tok]
+        outs = prefill(tw, 0, ent_seq, pos0, qs, 16)
+        checked = 0
+        for i in range(64):
+            t = n_tok[i]
+            if t == 0:
+                assert outs[i].shape[0] == 0
+                continue
+            for at in range(0, t, 64):
+                m = min(64, t - at)
+                dec = tw.decode_attn(0, [ent_seq[i]] * m, list(range(pos0[i] + at, pos0[i] + at + m)),
+                                     qs[i][at:at + m], 16, scale=1.0 / 16.0)
+                assert max_abs(dec, outs[i][at:at + m]) < 5e-6, (i, at)
+            if i % 9 == 0:
+                tok = t - 1
+                want = tw.oracle_attend(0, ent_seq[i], pos0[i] + tok, qs[i][tok], 16)
+                _, rel = check_attn(outs[i][tok], want, "chunk %d" % i)
+                assert rel <= REF_BAR_MAX_REL, (i, rel)
+                checked += 1
+        assert checked >= 5
+        z = DeviceBuffer(1 << 16)
+        with pytest.raises(BkvError) as ei:
+            tw.pool.prefill_attn(0, ent_seq + [seqs[0]], pos0 + [0], [1] * 65, 16, z, z, 0.0625)
+        assert ei.value.status == L.ERR_INVALID
+        z.free()
