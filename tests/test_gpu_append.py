@@ -236,3 +236,59 @@ def test_reset_zeroes_the_pools_and_frees_every_sequence():
         tw.pool.fill(0xFF)
         device_sync()
         assert (tw.pool.read_layer(0, 1) == 0xFF).all()
+
+
+@pytest.mark.parametrize("layout", [L.LAYOUT_F16, L.LAYOUT_Q8V, L.LAYOUT_I8H])
+@pytest.mark.parametrize("n_kv,hd", [(3, 96), (1, 32), (8, 128), (5, 256)])
+def test_other_geometries_append_bit_exact(layout, n_kv, hd):
+    # the append kernels (plain and with the K preparation fused in) take any head count and any
+    # head dim that is a multiple of 32 (the int8 layout: head dim 256 only): every pool byte
+    # against the oracle, chunked and one token at a time, through a permuted table
+    from breccia_amd.kv import rope_table
+    if layout == L.LAYOUT_I8H and hd != 256:
+        with pytest.raises(BkvError) as ei:
+            Twin(n_pages=8, n_kv=n_kv, hd=hd, layout=layout, max_seqs=2)
+        assert ei.value.status == L.ERR_INVALID
+        return
+    rng = np.random.Generator(np.random.PCG64(40 + layout + 7 * n_kv + hd))
+    n_rot = min(64, hd)
+    gamma = (1.0 + 0.3 * rng.standard_normal(hd)).astype(np.float32)
+    table = rope_table(1e7, n_rot, 512)
+    gd, td = DeviceBuffer.from_numpy(gamma), DeviceBuffer.from_numpy(table)
+    with Twin(n_pages=64, n_kv=n_kv, hd=hd, layout=layout, max_seqs=4) as tw:
+        tw.pool.set_free_order(rng.permutation(64).astype(np.int32))
+        a, b = tw.pool.seq_create(), tw.pool.seq_create()
+        n = 203
+        for s in (a, b):
+            tw.pool.seq_reserve(s, n)
+        k = (rng.standard_normal((n, n_kv, hd)) * rng.uniform(0.01, 20, size=(n, n_kv, 1))).astype(np.float32)
+        v = (rng.standard_normal((n, n_kv, hd)) * rng.uniform(0.01, 20, size=(n, n_kv, 1))).astype(np.float32)
+        # plain append: a chunk, then token by token
+        tw.append(0, [a], [0], [k[:190]], [v[:190]])
+        for t in range(190, n):
+            tw.append(0, [a], [t], [k[t:t + 1]], [v[t:t + 1]])
+        tw.assert_pools_equal()
+        # fused K preparation on the second sequence: two chunks
+        for lo, hi in ((0, 150), (150, n)):
+            kd = DeviceBuffer.from_numpy(np.concatenate([k[lo:hi].reshape(-1), np.zeros(4, np.float32)]))
+            vd = DeviceBuffer.from_numpy(np.concatenate([v[lo:hi].reshape(-1), np.zeros(4, np.float32)]))
+            tw.pool.append_kprep(0, [b], [lo], [hi - lo], kd, vd, gd, 1e-6, td, n_rot, 512, None)
+            device_sync()
+            kd.free()
+            vd.free()
+            want_k = oracle.k_prep(k[lo:hi], n_kv, hd, gamma, 1e-6, table, n_rot, np.arange(lo, hi))
+            assert tw.images[0].append(tw.pool.block_table(b), lo, want_k, v[lo:hi],
+                                       capacity_cells=tw.pool.seq_capacity(b)) == 0
+        tw.assert_pools_equal()
+        tw.pool.check()
+        if hd != 256:
+            # the attention kernels are built for head dim 256: refused, not launched
+            z = DeviceBuffer(1 << 16)
+            for call in (lambda: tw.pool.decode_attn(0, [a], [n - 1], 2 * n_kv, z, z, 0.0625),
+                         lambda: tw.pool.prefill_attn(0, [a], [0], [n], 2 * n_kv, z, z, 0.0625)):
+                with pytest.raises(BkvError) as ei:
+                    call()
+                assert ei.value.status == L.ERR_INVALID
+            z.free()
+    gd.free()
+    td.free()
