@@ -10,7 +10,7 @@ import pytest
 
 import oracle
 from breccia_amd import lib as L
-from breccia_amd.kv import device_sync
+from breccia_amd.kv import DeviceBuffer, device_sync
 from gpu_common import REF_BAR_MAX_REL, Twin, check_attn
 from helpers import max_abs
 
@@ -289,3 +289,57 @@ def test_layers_are_independent():
             tw.assert_pools_equal(layer)
             out = tw.decode_attn(layer, [s], [199], q, 16)
             check_attn(out[0], tw.oracle_attend(layer, s, 199, q[0], 16), "layer %d" % layer)
+
+
+@pytest.mark.parametrize("layout", [L.LAYOUT_F16, L.LAYOUT_Q8V, L.LAYOUT_I8H])
+@pytest.mark.parametrize("n_kv,n_q", [(1, 16), (3, 12), (8, 32), (4, 4), (5, 60)])
+def test_other_head_counts(layout, n_kv, n_q):
+    # kv head counts other than the model's 2, groups of 1, 4, 12 and 16 q heads per kv head: decode
+    # attention, the fused step and the chunk kernel against the oracle
+    rng = np.random.Generator(np.random.PCG64(150 + 17 * n_kv + n_q + layout))
+    with Twin(n_pages=96, n_kv=n_kv, layout=layout, max_seqs=4) as tw:
+        tw.pool.set_free_order(rng.permutation(96).astype(np.int32))
+        lens = [333, 70]
+        seqs = [tw.pool.seq_create() for _ in lens]
+        for s, n in zip(seqs, lens):
+            tw.pool.seq_reserve(s, n + 1)
+            k = rng.standard_normal((n, n_kv, 256)).astype(np.float32)
+            v = rng.standard_normal((n, n_kv, 256)).astype(np.float32)
+            tw.append(0, [s], [0], [k], [v])
+        q = rng.standard_normal((2, n_q, 256)).astype(np.float32)
+        pos = [n - 1 for n in lens]
+        out = tw.decode_attn(0, seqs, pos, q, n_q)
+        for i in range(2):
+            _, rel = check_attn(out[i], tw.oracle_attend(0, seqs[i], pos[i], q[i], n_q), "decode %d" % i)
+            assert rel <= REF_BAR_MAX_REL, rel
+        # the chunk kernel over the last 40 tokens of the first sequence
+        qc = rng.standard_normal((40, n_q, 256)).astype(np.float32)
+        qd, od = DeviceBuffer.from_numpy(qc), DeviceBuffer(qc.nbytes)
+        tw.pool.prefill_attn(0, [seqs[0]], [lens[0] - 40], [40], n_q, qd, od, 1.0 / 16.0)
+        device_sync()
+        oc = od.download(np.float32).reshape(40, n_q, 256)
+        qd.free()
+        od.free()
+        for t in (0, 17, 39):
+            _, rel = check_attn(oc[t], tw.oracle_attend(0, seqs[0], lens[0] - 40 + t, qc[t], n_q), "chunk %d" % t)
+            assert rel <= REF_BAR_MAX_REL, rel
+        # the fused step (one more token per sequence), where this pool has it: pool bytes as an
+        # append would leave them, outputs against the oracle
+        import gpu_common
+        if layout == L.LAYOUT_F16 or not gpu_common.DEFAULT_ATTN_VALU:
+            k1 = rng.standard_normal((2, n_kv, 256)).astype(np.float32)
+            v1 = rng.standard_normal((2, n_kv, 256)).astype(np.float32)
+            kd, vd = DeviceBuffer.from_numpy(k1), DeviceBuffer.from_numpy(v1)
+            qd, od = DeviceBuffer.from_numpy(q), DeviceBuffer(q.nbytes)
+            tw.pool.decode_step(0, seqs, lens, kd, vd, n_q, qd, od, 1.0 / 16.0)
+            device_sync()
+            os_ = od.download(np.float32).reshape(2, n_q, 256)
+            for b in (kd, vd, qd, od):
+                b.free()
+            for i, s in enumerate(seqs):
+                assert tw.images[0].append(tw.pool.block_table(s), lens[i], k1[i:i + 1], v1[i:i + 1],
+                                           capacity_cells=tw.pool.seq_capacity(s)) == 0
+            tw.assert_pools_equal()
+            for i in range(2):
+                _, rel = check_attn(os_[i], tw.oracle_attend(0, seqs[i], lens[i], q[i], n_q), "step %d" % i)
+                assert rel <= REF_BAR_MAX_REL, rel
