@@ -192,3 +192,28 @@ def test_select_errors_come_before_any_launch():
                 call(**kw)
             assert ei.value.status == status, kw
         z.free()
+
+
+@pytest.mark.parametrize("layout", [L.LAYOUT_F16, L.LAYOUT_Q8V, L.LAYOUT_I8H])
+@pytest.mark.parametrize("n_kv,n_q", [(1, 16), (3, 12), (8, 32), (5, 60)])
+def test_selection_lists_with_other_head_counts(layout, n_kv, n_q):
+    rng = np.random.Generator(np.random.PCG64(950 + 13 * n_kv + n_q + layout))
+    with Twin(n_pages=64, n_kv=n_kv, layout=layout, max_seqs=4) as tw:
+        tw.pool.set_free_order(rng.permutation(64).astype(np.int32))
+        n = 413
+        s = tw.pool.seq_create()
+        tw.pool.seq_reserve(s, n)
+        k = rng.standard_normal((n, n_kv, 256)).astype(np.float32)
+        v = rng.standard_normal((n, n_kv, 256)).astype(np.float32)
+        tw.append(0, [s], [0], [k], [v])
+        pos = [n - 1, 200]
+        lists = [sorted(rng.choice((p + 1 + 3) // 4, size=min(37, (p + 4) // 4), replace=False).tolist()) for p in pos]
+        q = rng.standard_normal((2, n_q, 256)).astype(np.float32)
+        out = select_attn(tw, 0, [s, s], pos, q, n_q, lists)
+        table = tw.pool.block_table(s)
+        for i in range(2):
+            kk, vv = tw.images[0].gather(table, 0, pos[i] + 1)
+            cells = oracle.cells_of(np.asarray(lists[i], dtype=np.uint32))
+            want = oracle.attend(q[i], kk, vv, cells, pos[i], n_q, n_kv, 256, threads=4)
+            _, rel = check_attn(out[i], want, "list %d" % i)
+            assert rel <= REF_BAR_MAX_REL, rel
