@@ -7,7 +7,9 @@ all 16 heads each; the full f64 oracle over all 16 sequences is ~10^10 MACs), pl
 size-independent properties on all of them: the batched call equals the per-sequence call to
 1e-6, and every output is a convex combination of V rows (bounded by the largest |v|).
 configs[3] shape (4 sequences, 2048-token prefix + 1024-token chunk) through the chunk kernel on
-all three layouts: sampled tokens against the oracle, the chunk's tail against the decode kernel."""
+all three layouts: sampled tokens against the oracle, the chunk's tail against the decode kernel.
+A 300k-page pool with a sequence on the highest page ids (byte offsets past 2^32): every kernel of the
+path there against a twin on the lowest pages and the oracle."""
 import numpy as np
 import pytest
 
@@ -165,5 +167,109 @@ def test_config4_shape_prefill_of_1024_token_chunks_on_2048_token_prefixes(layou
         assert max_abs(dec, out[2, -64:]) < 5e-6
         qd.free()
         od.free()
+    finally:
+        pool.destroy()
+
+
+@pytest.mark.parametrize("layout", [L.LAYOUT_F16, L.LAYOUT_Q8V, L.LAYOUT_I8H])
+def test_pages_beyond_4_gib_into_a_pool(layout):
+    # A pool of 300k pages (4.9 GB of K and as much of V on the f16 layout): one sequence lives on
+    # the highest page ids, byte offsets past 2^32 into either pool.  Append, decode attention,
+    # chunk attention, the fused step and a copy-on-write page copy there, against the oracle over
+    # the rows read back through bkv_gather (a separate kernel with its own address arithmetic) and
+    # against a twin sequence on the lowest page ids that holds the same rows.
+    rng = np.random.Generator(np.random.PCG64(20250009 + layout))
+    n_pages, n = 300000, 517
+    pool = Pool(n_layers=1, n_pages=n_pages, n_kv_head=N_KV, head_dim=HD, layout=layout, max_seqs=6,
+                max_pages_per_seq=64)
+    try:
+        pool.set_free_order(np.arange(n_pages - 1, -1, -1, dtype=np.int32))          # highest first
+        hi = pool.seq_create()
+        pool.seq_reserve(hi, n + 1)                                                  # 33 pages
+        assert int(pool.block_table(hi)[:33].min()) == n_pages - 33
+        pool.set_free_order(np.arange(0, n_pages - 33, dtype=np.int32))              # lowest first
+        lo = pool.seq_create()
+        pool.seq_reserve(lo, n + 1)
+        assert int(pool.block_table(lo)[:33].max()) == 32
+        k = rng.standard_normal((n + 1, N_KV, HD), dtype=np.float32)
+        v = rng.standard_normal((n + 1, N_KV, HD), dtype=np.float32)
+        kd, vd = DeviceBuffer.from_numpy(k), DeviceBuffer.from_numpy(v)
+        pool.append(0, [hi], [0], [n], kd, vd)
+        pool.append(0, [lo], [0], [n], kd, vd)
+        device_sync()
+        ghk, ghv = pool.gather(0, hi, 0, n)
+        glk, glv = pool.gather(0, lo, 0, n)
+        assert np.array_equal(ghk, glk) and np.array_equal(ghv, glv)
+        assert np.abs(ghk).max() > 1.0                           # not the zeros of an untouched pool
+        q = rng.standard_normal((2, N_Q, HD), dtype=np.float32)
+        out = run_attn(pool, [hi, lo], [n - 1, n - 1], q[[0, 0]])
+        assert np.array_equal(out[0].view(np.uint32), out[1].view(np.uint32))
+        want = oracle.attend(q[0], ghk, ghv, oracle.dense_cells(n - 1), n - 1, N_Q, N_KV, HD, threads=8)
+        _, rel = check_attn(out[0], want, "decode on the highest pages")
+        assert rel <= REF_BAR_MAX_REL, rel
+        # chunk attention over the last 100 tokens of both
+        qc = rng.standard_normal((100, N_Q, HD), dtype=np.float32)
+        qd, od = DeviceBuffer.from_numpy(np.concatenate([qc, qc])), DeviceBuffer(2 * qc.nbytes)
+        pool.prefill_attn(0, [hi, lo], [n - 100, n - 100], [100, 100], N_Q, qd, od, 1.0 / 16.0)
+        device_sync()
+        oc = od.download(np.float32).reshape(2, 100, N_Q, HD)
+        assert np.array_equal(oc[0].view(np.uint32), oc[1].view(np.uint32))
+        for t in (0, 99):
+            p = n - 100 + t
+            want = oracle.attend(qc[t], ghk[:p + 1], ghv[:p + 1], oracle.dense_cells(p), p, N_Q, N_KV, HD, threads=8)
+            _, rel = check_attn(oc[0, t], want, "chunk on the highest pages, token %d" % t)
+            assert rel <= REF_BAR_MAX_REL, rel
+        qd.free()
+        od.free()
+        # the fused step appends row n on both and attends
+        k1 = DeviceBuffer.from_numpy(np.ascontiguousarray(k[n:n + 1].repeat(2, 0)))
+        v1 = DeviceBuffer.from_numpy(np.ascontiguousarray(v[n:n + 1].repeat(2, 0)))
+        qd, od = DeviceBuffer.from_numpy(np.ascontiguousarray(q[[1, 1]])), DeviceBuffer(q.nbytes)
+        pool.decode_step(0, [hi, lo], [n, n], k1, v1, N_Q, qd, od, 1.0 / 16.0)
+        device_sync()
+        os_ = od.download(np.float32).reshape(2, N_Q, HD)
+        assert np.array_equal(os_[0].view(np.uint32), os_[1].view(np.uint32))
+        ghk, ghv = pool.gather(0, hi, 0, n + 1)
+        want = oracle.attend(q[1], ghk, ghv, oracle.dense_cells(n), n, N_Q, N_KV, HD, threads=8)
+        _, rel = check_attn(os_[0], want, "step on the highest pages")
+        assert rel <= REF_BAR_MAX_REL, rel
+        for b in (k1, v1, qd, od):
+            b.free()
+        # selection lists (every block, ascending) through the list kernel
+        n_ids = (n + 1 + 3) // 4
+        ids = np.tile(np.arange(n_ids, dtype=np.uint32), (2, 1))
+        idd, cd = DeviceBuffer.from_numpy(ids), DeviceBuffer.from_numpy(np.full(2, n_ids, dtype=np.uint32))
+        qd, od = DeviceBuffer.from_numpy(np.ascontiguousarray(q[[1, 1]])), DeviceBuffer(q.nbytes)
+        pool.decode_attn_select(0, [hi, lo], [n, n], N_Q, qd, od, 1.0 / 16.0, idd, n_ids, cd, n_ids)
+        device_sync()
+        osel = od.download(np.float32).reshape(2, N_Q, HD)
+        assert np.array_equal(osel[0].view(np.uint32), osel[1].view(np.uint32))
+        _, rel = check_attn(osel[0], want, "selection lists on the highest pages")
+        assert rel <= REF_BAR_MAX_REL, rel
+        for b in (idd, cd, qd, od):
+            b.free()
+        # the complete pages of `hi` go to host memory and come back onto other high pages
+        pool.set_free_order(np.arange(n_pages - 34, 32, -1, dtype=np.int32))
+        host = pool.host_alloc(32 * pool.swap_page_bytes())
+        pool.seq_evict(hi, 0, 32, host)
+        pool.swap_wait()
+        pool.seq_restore(hi, 0, 32, host)
+        device_sync()
+        pool.swap_wait()
+        assert int(pool.block_table(hi)[:32].min()) >= n_pages - 100
+        grk, grv = pool.gather(0, hi, 0, n + 1)
+        assert np.array_equal(grk, ghk) and np.array_equal(grv, ghv)
+        host.free()
+        # a fork of `hi` that writes copies the shared, partly filled last page to another high page
+        child = pool.seq_fork(hi, n + 1)
+        pairs = pool.seq_reserve(child, n + 2)
+        assert len(pairs) == 1 and pairs[0][0] == n_pages - 33 and pairs[0][1] >= n_pages - 100
+        pool.page_copy(pairs)
+        device_sync()
+        gck, gcv = pool.gather(0, child, 0, n + 1)
+        assert np.array_equal(gck, ghk) and np.array_equal(gcv, ghv)
+        kd.free()
+        vd.free()
+        pool.check()
     finally:
         pool.destroy()
