@@ -273,3 +273,28 @@ def test_pages_beyond_4_gib_into_a_pool(layout):
         pool.check()
     finally:
         pool.destroy()
+
+
+def test_one_sequence_of_400k_tokens():
+    # far past BASELINE's longest context (128k): 25000 pages in one block-table row, hundreds of
+    # split-K ranges per head for the merge; decode attention and the fused step against the oracle
+    rng = np.random.Generator(np.random.PCG64(20250010))
+    ctx = [400003]
+    pool, seqs, _ = build(rng, 1, ctx[0], ctx[0], L.LAYOUT_F16, occupancy=0.9)
+    try:
+        fill_tiled(pool, seqs, ctx, rng)
+        q = rng.standard_normal((1, N_Q, HD), dtype=np.float32)
+        out = run_attn(pool, seqs, [ctx[0] - 1], q)
+        want, v = oracle_for(pool, seqs[0], ctx[0] - 1, q[0])
+        _, rel = check_attn(out[0], want, "400k tokens")
+        assert rel <= REF_BAR_MAX_REL, rel
+        assert np.abs(out[0]).max() <= np.abs(v).max()
+        # a T = 3 decode (three positions of the same sequence) equals three single calls
+        pos = [ctx[0] - 1, ctx[0] // 2, 12345]
+        q3 = rng.standard_normal((3, N_Q, HD), dtype=np.float32)
+        together = run_attn(pool, seqs * 3, pos, q3)
+        for i in range(3):
+            alone = run_attn(pool, seqs, [pos[i]], q3[i:i + 1])
+            assert max_abs(alone[0], together[i]) < 1e-6, i
+    finally:
+        pool.destroy()
