@@ -91,6 +91,25 @@ static bkv_status wait_for_tier_moves(bkv_pool* p, hipStream_t stream) {
     return BKV_OK;
 }
 
+// A pool has one split-K workspace and one score workspace.  Calls on one stream use them in turn
+// by themselves; a call that arrives on another stream than the last one is ordered behind it
+// with an event recorded there now (behind everything that stream has been given).
+static bkv_status order_workspace(WorkspaceOrder& w, hipStream_t stream) {
+    if (w.used && w.last != stream) {
+        if (!w.ev) BKV_HIP(hipEventCreateWithFlags(&w.ev, hipEventDisableTiming));
+        if (hipEventRecord(w.ev, w.last) == hipSuccess) {
+            BKV_HIP(hipStreamWaitEvent(stream, w.ev, 0));
+        } else {
+            // the stream is gone: whatever it was given is ordered by a full synchronisation
+            (void)hipGetLastError();
+            BKV_HIP(hipDeviceSynchronize());
+        }
+    }
+    w.last = stream;
+    w.used = true;
+    return BKV_OK;
+}
+
 bkv_status flush_tables(bkv_pool* p, hipStream_t stream) {
     bkv_status tier_st = wait_for_tier_moves(p, stream);
     if (tier_st != BKV_OK) return tier_st;
@@ -177,6 +196,8 @@ static void destroy_device_side(bkv_pool* p) {
     if (p->tiers.host) (void)hipHostFree(p->tiers.host);
     if (p->tiers.bounce) (void)hipHostFree(p->tiers.bounce);
     if (p->tiers.done) (void)hipEventDestroy(p->tiers.done);
+    if (p->attn_ws.ev) (void)hipEventDestroy(p->attn_ws.ev);
+    if (p->sel_ws.ev) (void)hipEventDestroy(p->sel_ws.ev);
     if (p->slab) (void)hipFree(p->slab);
     if (p->table_dev) (void)hipFree(p->table_dev);
     if (p->part_o) (void)hipFree(p->part_o);
@@ -833,6 +854,8 @@ static bkv_status decode_attn_common(bkv_pool* p, int32_t layer, int32_t n, cons
         a.new_k = new_k_dev;
         a.new_v = new_v_dev;
     }
+    st = order_workspace(p->attn_ws, S(stream));
+    if (st != BKV_OK) return st;
     BKV_HIP(launch_decode_attn(p, layer, b, a, S(stream)));
     if (p->timer.open.size() > 8192) return timer_collect(p);
     return BKV_OK;
@@ -1054,6 +1077,8 @@ bkv_status bkv_select_blocks(bkv_pool* p, int32_t n, const int64_t* pos, const f
         BKV_HIP(hipMalloc(reinterpret_cast<void**>(&p->sel_scores), cap * sizeof(double)));
         p->sel_scores_cap = cap;
     }
+    const bkv_status ws = order_workspace(p->sel_ws, S(stream));
+    if (ws != BKV_OK) return ws;
     if (max_blocks > 0)
         BKV_HIP(launch_idx_score(b, idx_q_dev, idx_n_head, idx_dim, 4, p->sel_scores, (int64_t)stride,
                                  max_blocks, S(stream)));

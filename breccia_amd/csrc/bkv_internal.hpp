@@ -70,6 +70,13 @@ struct SwapStage {
     int next = 0;
 };
 
+// Which stream used a pool-owned workspace last, and an event to order the next one behind it.
+struct WorkspaceOrder {
+    hipStream_t last = nullptr;
+    bool used = false;
+    hipEvent_t ev = nullptr;
+};
+
 // Where the prefix tree's lower tiers keep their pages: a pinned-host arena of slots and a file,
 // slot = one page's bytes of every layer ([layer][K page | V page]).
 struct TierStore {
@@ -105,6 +112,10 @@ struct bkv_pool {
     // block selection: f64 indexer scores [entry][block], grown on demand
     double* sel_scores = nullptr;
     uint64_t sel_scores_cap = 0;  // doubles
+
+    // Streams that used the split-K workspace and the score workspace last: a call on another
+    // stream is ordered behind them first (the workspaces are one per pool).
+    bkv::WorkspaceOrder attn_ws, sel_ws;
 
     bkv::ParamRing ring;
     bkv::StageTimer timer;

@@ -11,6 +11,12 @@
  * reference recording into a device's open batch, crates/breccia-kernels/src/
  * ops/mod.rs:205-222): results are visible to later work on the same stream.
  * `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ * One pool may be driven from several streams (by one host thread at a time: the
+ * pool itself is not thread-safe).  What the pool owns and every call shares --
+ * the argument ring, the block tables, the split-K and score workspaces, the swap
+ * staging -- it orders across streams by itself with events; the order between the
+ * caller's own data (an append before the attention that reads its rows, on another
+ * stream) is the caller's to keep, as with any work on streams.
  *
  * Reference items each group replaces are cited per declaration; paths are
  * relative to the reference tree, `qsa/` = crates/breccia-kernels/src/qsa/.

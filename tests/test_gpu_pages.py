@@ -138,3 +138,68 @@ def test_evict_and_restore_through_the_allocator():
         assert np.array_equal(ka, kb) and np.array_equal(va, vb)
         tw.pool.check()
         host.free()
+
+
+def test_two_streams_interleave_on_one_pool_without_host_synchronisation():
+    # Two request streams share a pool: each grows its own sequence (2000 tokens to begin with) one
+    # token at a time (a table update, an append and a decode attention per step) and forks it
+    # every 16 steps (a copy-on-write page copy), 150 steps each, the calls of the two interleaved
+    # and nothing synchronised on the host until the end -- the parameter ring and the block-table
+    # uploads wrap around several times, and the attention calls of the two streams, which share
+    # the pool's split-K workspace, would overlap on the device if the pool did not order them.
+    # Every output and the final K/V rows equal what the same work gives when it is run on one
+    # stream with a synchronisation after every call.
+    from breccia_amd.kv import DeviceBuffer, Pool, Stream, device_sync
+
+    def run(async_two_streams):
+        rng = np.random.Generator(np.random.PCG64(444))
+        pool = Pool(n_pages=400, max_seqs=40)
+        pool.set_free_order(rng.permutation(400).astype(np.int32))
+        streams = [Stream(), Stream()] if async_two_streams else [Stream()] * 2
+        seqs = [pool.seq_create(), pool.seq_create()]
+        steps, base = 150, 2000
+        head = DeviceBuffer.from_numpy(rng.standard_normal((base, 2, 256), dtype=np.float32))
+        for s in seqs:
+            pool.seq_reserve(s, base)
+            pool.append(0, [s], [0], [base], head, head, streams[0])
+        streams[0].sync()
+        k = [DeviceBuffer.from_numpy(rng.standard_normal((steps, 2, 256), dtype=np.float32)) for _ in range(2)]
+        v = [DeviceBuffer.from_numpy(rng.standard_normal((steps, 2, 256), dtype=np.float32)) for _ in range(2)]
+        q = [DeviceBuffer.from_numpy(rng.standard_normal((steps, 16, 256), dtype=np.float32)) for _ in range(2)]
+        out = [DeviceBuffer(steps * 16 * 256 * 4) for _ in range(2)]
+        row, qrow = 2 * 256 * 4, 16 * 256 * 4
+        for t in range(steps):
+            for i in range(2):
+                st = streams[i]
+                if t and t % 16 == 5:
+                    # fork inside a page and drop the parent: the child's next write copies the page
+                    child = pool.seq_fork(seqs[i], base + t)
+                    old = seqs[i]
+                    seqs[i] = child
+                    pairs = pool.seq_reserve(child, base + t + 1)
+                    assert len(pairs) == 1
+                    pool.page_copy(pairs, st)
+                    pool.seq_free(old)
+                else:
+                    pool.seq_reserve(seqs[i], base + t + 1)
+                pool.append(0, [seqs[i]], [base + t], [1], k[i].at(t * row), v[i].at(t * row), st)
+                pool.decode_attn(0, [seqs[i]], [base + t], 16, q[i].at(t * qrow), out[i].at(t * qrow), 1.0 / 16.0, stream=st)
+                if not async_two_streams:
+                    st.sync()
+        for st in set(streams):
+            st.sync()
+        device_sync()
+        res = [o.download(np.float32) for o in out]
+        rows = [pool.gather(0, s, 0, base + steps) for s in seqs]
+        pool.check()
+        for b in k + v + q + out + [head]:
+            b.free()
+        pool.destroy()
+        return res, rows
+
+    a_out, a_rows = run(True)
+    b_out, b_rows = run(False)
+    for i in range(2):
+        assert np.array_equal(a_out[i].view(np.uint32), b_out[i].view(np.uint32)), i
+        assert np.array_equal(a_rows[i][0], b_rows[i][0]) and np.array_equal(a_rows[i][1], b_rows[i][1]), i
+        assert np.abs(a_out[i]).max() > 0
