@@ -113,6 +113,15 @@ static bkv_status order_workspace(WorkspaceOrder& w, hipStream_t stream) {
 bkv_status flush_tables(bkv_pool* p, hipStream_t stream) {
     bkv_status tier_st = wait_for_tier_moves(p, stream);
     if (tier_st != BKV_OK) return tier_st;
+    // Block-table updates are scattered on whichever stream brings the next call.  A call on
+    // another stream reads the same table: it waits for the last scatter (until that is known to
+    // be over).
+    if (p->table_sync.used && p->table_sync.last != stream) {
+        if (hipEventQuery(p->table_sync.ev) == hipSuccess)
+            p->table_sync.used = false;
+        else
+            BKV_HIP(hipStreamWaitEvent(stream, p->table_sync.ev, 0));
+    }
     std::vector<TableUpdate>& pend = p->alloc->pending();
     if (pend.empty()) return BKV_OK;
     if (p->host_only) {
@@ -139,6 +148,10 @@ bkv_status flush_tables(bkv_pool* p, hipStream_t stream) {
         if (st != BKV_OK) return st;
     }
     pend.clear();
+    if (!p->table_sync.ev) BKV_HIP(hipEventCreateWithFlags(&p->table_sync.ev, hipEventDisableTiming));
+    BKV_HIP(hipEventRecord(p->table_sync.ev, stream));
+    p->table_sync.last = stream;
+    p->table_sync.used = true;
     return BKV_OK;
 }
 
@@ -198,6 +211,7 @@ static void destroy_device_side(bkv_pool* p) {
     if (p->tiers.done) (void)hipEventDestroy(p->tiers.done);
     if (p->attn_ws.ev) (void)hipEventDestroy(p->attn_ws.ev);
     if (p->sel_ws.ev) (void)hipEventDestroy(p->sel_ws.ev);
+    if (p->table_sync.ev) (void)hipEventDestroy(p->table_sync.ev);
     if (p->slab) (void)hipFree(p->slab);
     if (p->table_dev) (void)hipFree(p->table_dev);
     if (p->part_o) (void)hipFree(p->part_o);

@@ -116,6 +116,8 @@ struct bkv_pool {
     // Streams that used the split-K workspace and the score workspace last: a call on another
     // stream is ordered behind them first (the workspaces are one per pool).
     bkv::WorkspaceOrder attn_ws, sel_ws;
+    // the stream of the last block-table scatter, and the event behind it
+    bkv::WorkspaceOrder table_sync;
 
     bkv::ParamRing ring;
     bkv::StageTimer timer;

@@ -203,3 +203,45 @@ def test_two_streams_interleave_on_one_pool_without_host_synchronisation():
         assert np.array_equal(a_out[i].view(np.uint32), b_out[i].view(np.uint32)), i
         assert np.array_equal(a_rows[i][0], b_rows[i][0]) and np.array_equal(a_rows[i][1], b_rows[i][1]), i
         assert np.abs(a_out[i]).max() > 0
+
+
+def test_table_updates_flushed_on_one_stream_are_seen_on_another():
+    # The block-table changes of two sequences are pushed to the device by whichever call comes
+    # next -- here a call on stream 1, queued behind a long append -- and the other sequence's
+    # append and attention follow at once on stream 0: they wait for that push on the device.
+    from breccia_amd.kv import DeviceBuffer, Pool, Stream, device_sync
+    rng = np.random.Generator(np.random.PCG64(445))
+    s0, s1 = Stream(), Stream()
+    with Pool(n_pages=1200, max_seqs=8, max_pages_per_seq=600) as pool:
+        pool.set_free_order(rng.permutation(1200).astype(np.int32))
+        big_rows = DeviceBuffer.from_numpy(rng.standard_normal((8192, 2, 256), dtype=np.float32))
+        rows = rng.standard_normal((40, 2, 256), dtype=np.float32)
+        rd = DeviceBuffer.from_numpy(rows)
+        q = rng.standard_normal((1, 16, 256), dtype=np.float32)
+        qd, od = DeviceBuffer.from_numpy(q), DeviceBuffer(q.nbytes)
+        c = pool.seq_create()
+        pool.seq_reserve(c, 8192)
+        for rep in range(5):
+            a, b = pool.seq_create(), pool.seq_create()
+            pool.append(0, [c], [0], [8192], big_rows, big_rows, s1)     # long work on stream 1
+            pool.seq_reserve(a, 40)
+            pool.seq_reserve(b, 40)
+            pool.append(0, [b], [0], [40], rd, rd, s1)                   # pushes both tables, on stream 1
+            pool.append(0, [a], [0], [40], rd, rd, s0)                   # stream 0, nothing left to push
+            pool.decode_attn(0, [a], [39], 16, qd, od, 1.0 / 16.0, stream=s0)
+            s0.sync()
+            out_a = od.download(np.float32, stream=s0).copy()
+            s1.sync()
+            ka, va = pool.gather(0, a, 0, 40)
+            kb, vb = pool.gather(0, b, 0, 40)
+            assert np.array_equal(ka, kb) and np.array_equal(va, vb) and np.abs(ka).max() > 1.0
+            pool.decode_attn(0, [b], [39], 16, qd, od, 1.0 / 16.0, stream=s1)
+            s1.sync()
+            out_b = od.download(np.float32, stream=s1)
+            assert np.array_equal(out_a.view(np.uint32), out_b.view(np.uint32))
+            pool.seq_free(a)
+            pool.seq_free(b)
+            pool.check()
+        device_sync()
+        for x in (big_rows, rd, qd, od):
+            x.free()
