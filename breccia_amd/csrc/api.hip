@@ -1423,6 +1423,8 @@ static bkv_status run_tier_moves(bkv_pool* p, const std::vector<TierMove>& moves
         // read; the next read overlaps the previous half's upload
         std::sort(from_disk.begin(), from_disk.end(),
                   [](const TierMove& a, const TierMove& b) { return a.disk_slot < b.disk_slot; });
+        // an earlier call's upload may still be reading the bounce buffer
+        BKV_HIP(hipStreamSynchronize(p->side));
         bool half_in_flight[2] = {false, false};
         int half = 0;
         std::vector<int32_t> pages;
