@@ -56,7 +56,6 @@ struct StageTimer {
     };
     bool on = false;
     std::vector<Pair> open;       // recorded, not yet read
-    std::vector<hipEvent_t> idle; // events to reuse
     uint64_t launches[BKV_STAGE_COUNT] = {};
     double total_ms[BKV_STAGE_COUNT] = {};
 };
