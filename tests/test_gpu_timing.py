@@ -1,0 +1,77 @@
+"""The per-kernel timers (bkv_timing_*): launches are attributed to their stages, the durations are
+those of the kernels (positive, and together no longer than the stream time around them), results
+do not depend on whether the timers are on, and a reset starts from zero."""
+import numpy as np
+import pytest
+
+from breccia_amd import lib as L
+from breccia_amd.kv import Event, Stream
+from gpu_common import Twin, check_attn
+from test_gpu_attn import fill
+
+pytestmark = pytest.mark.gpu
+
+STAGES = (L.STAGE_APPEND, L.STAGE_ATTN_SPLIT, L.STAGE_ATTN_MERGE, L.STAGE_PAGE_COPY)
+
+
+def read_all(pool):
+    return {s: pool.timing_read(s) for s in STAGES}
+
+
+def test_timers_count_each_stage_and_leave_results_alone():
+    rng = np.random.Generator(np.random.PCG64(4711))
+    with Twin(n_pages=256, max_seqs=4) as tw:
+        st = Stream()
+        a, b = tw.pool.seq_create(), tw.pool.seq_create()
+        fill(tw, a, 1500, rng)
+        fill(tw, b, 333, rng)
+        q = rng.standard_normal((2, 16, 256)).astype(np.float32)
+        pos = [1499, 332]
+        plain = tw.decode_attn(0, [a, b], pos, q, 16, stream=st)
+        # off: nothing is counted
+        assert all(n == 0 and ms == 0.0 for n, ms in read_all(tw.pool).values())
+
+        tw.pool.timing_enable(True)
+        e0, e1 = Event(), Event()
+        e0.record(st)
+        timed = tw.decode_attn(0, [a, b], pos, q, 16, stream=st)
+        k = rng.standard_normal((7, 2, 256)).astype(np.float32)
+        tw.pool.seq_reserve(a, 1507)
+        tw.append(0, [a], [1500], [k], [k], stream=st)
+        free = [p for p in range(256) if tw.pool.page_refcount(p) == 0][:3]
+        pairs = [(int(tw.pool.block_table(a)[i]), free[i]) for i in range(3)]
+        tw.pool.page_copy(pairs, st)
+        for img in tw.images:
+            img.page_copy(pairs)
+        e1.record(st)
+        st.sync()
+        wall = e0.elapsed_ms(e1)
+        tw.pool.timing_enable(False)
+        got = read_all(tw.pool)
+        assert got[L.STAGE_ATTN_SPLIT][0] == 1 and got[L.STAGE_ATTN_MERGE][0] == 1
+        assert got[L.STAGE_APPEND][0] == 1 and got[L.STAGE_PAGE_COPY][0] == 1
+        total = sum(ms for _, ms in got.values())
+        assert all(ms > 0.0 for _, ms in got.values())
+        assert total < wall, "kernels %.4f ms, stream time around them %.4f ms" % (total, wall)
+        # the same bytes with the timers on or off, and both are the oracle's answer
+        assert np.array_equal(plain.view(np.uint32), timed.view(np.uint32))
+        for i, s in enumerate([a, b]):
+            check_attn(timed[i], tw.oracle_attend(0, s, pos[i], q[i], 16), "seq %d" % s)
+        tw.assert_pools_equal()
+
+        # off again: later launches are not counted; a reset starts from zero
+        tw.decode_attn(0, [a, b], pos, q, 16, stream=st)
+        assert read_all(tw.pool) == got
+        tw.pool.timing_reset()
+        assert all(n == 0 and ms == 0.0 for n, ms in read_all(tw.pool).values())
+
+        # many launches in one session, read while still enabled
+        tw.pool.timing_enable(True)
+        for _ in range(50):
+            tw.decode_attn(0, [a, b], pos, q, 16, stream=st)
+        n, ms = tw.pool.timing_read(L.STAGE_ATTN_SPLIT)
+        assert n == 50 and 0.0 < ms / n < 1.0
+        tw.pool.timing_enable(False)
+        e0.close()
+        e1.close()
+        st.close()
