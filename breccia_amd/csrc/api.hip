@@ -180,12 +180,15 @@ bool timer_dispatch_events(bkv_pool* p, int stage, hipEvent_t* start, hipEvent_t
 
 bkv_status timer_collect(bkv_pool* p) {
     StageTimer& t = p->timer;
+    hipError_t err = hipSuccess;
     for (const StageTimer::Pair& pr : t.open) {
-        BKV_HIP(hipEventSynchronize(pr.stop));
         float ms = 0.0f;
-        BKV_HIP(hipEventElapsedTime(&ms, pr.start, pr.stop));
-        t.launches[pr.stage] += 1;
-        t.total_ms[pr.stage] += (double)ms;
+        if (err == hipSuccess) err = hipEventSynchronize(pr.stop);
+        if (err == hipSuccess) err = hipEventElapsedTime(&ms, pr.start, pr.stop);
+        if (err == hipSuccess) {
+            t.launches[pr.stage] += 1;
+            t.total_ms[pr.stage] += (double)ms;
+        }
         // Events are not kept for reuse.  A recorded event holds on to its dispatch, and with it, as
         // measured, to the buffers the dispatch was given: with a pool of idle events, buffers that the
         // caller had freed since were only unmapped when those events were recorded again, and the
@@ -194,6 +197,7 @@ bkv_status timer_collect(bkv_pool* p) {
         (void)hipEventDestroy(pr.stop);
     }
     t.open.clear();
+    BKV_HIP(err);
     return BKV_OK;
 }
 
