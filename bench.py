@@ -142,6 +142,21 @@ def time_steps(pool, seqs, ctx0, n_layers, steps, warmup, bufs, stream, first_st
     return wall_ms, ev_ms
 
 
+PREHEAT_MS = 40.0
+
+
+def preheat(pool, seqs, ctx0, n_layers, bufs, stream, ms: float, first_step: int = 0):
+    """Run the step for about `ms` milliseconds of wall time (in bursts of 50, synchronised);
+    returns (steps run, milliseconds spent).  Not part of the warm-up or of the timed steps."""
+    t0 = time.perf_counter()
+    done = 0
+    while (time.perf_counter() - t0) * 1e3 < ms:
+        run_steps(pool, seqs, ctx0, n_layers, 50, *bufs, stream, first_step=first_step + done)
+        stream.sync()
+        done += 50
+    return done, (time.perf_counter() - t0) * 1e3
+
+
 def make_step_buffers(n_seqs, rng, slots=64):
     from breccia_amd.kv import DeviceBuffer
 
@@ -158,9 +173,7 @@ def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
-    # the first ~20 ms after the set-up phase run at lower clocks (81 vs 70 us per step measured):
-    # the default warm-up is long enough to leave that ramp outside the timed region
-    ap.add_argument("--warmup", type=int, default=300)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-extra", action="store_true", help="skip batch-1 / byte-move extras")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
@@ -180,11 +193,15 @@ def main() -> int:
     host_kv = fill_layers(pool, seqs, ctx, n_layers, rng, stream, keep_host_layer0=not args.no_cpu)
     q_host, bufs = make_step_buffers(len(seqs), rng)
 
+    # ---- clock ramp: the same step, untimed and uncounted, for a fixed wall time -----------
+    # (the first tens of milliseconds after the set-up phase run at lower clocks whatever --warmup is)
+    pre_steps, pre_ms = preheat(pool, seqs, ctx, n_layers, bufs, stream, PREHEAT_MS)
+
     # ---- headline: K steps, whole path ------------------------------------------------
-    wall_ms, ev_ms = time_steps(pool, seqs, ctx, n_layers, args.steps, args.warmup, bufs, stream)
+    wall_ms, ev_ms = time_steps(pool, seqs, ctx, n_layers, args.steps, args.warmup, bufs, stream,
+                                first_step=pre_steps)
     ms_per_step = wall_ms / args.steps
-    tokens_done = (args.warmup + args.steps + n_layers - 1) // n_layers
-    ctx_mid = [c + 1 + (args.warmup + args.steps // 2) // n_layers for c in ctx]
+    ctx_mid = [c + 1 + (pre_steps + args.warmup + args.steps // 2) // n_layers for c in ctx]
     attn_bytes = attn_algorithmic_bytes(ctx_mid)
     step_bytes = attn_bytes + len(seqs) * APPEND_BYTES_PER_TOKEN
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
@@ -192,7 +209,7 @@ def main() -> int:
     # ---- roofline: the split-K kernel alone, HIP events attached to its dispatches ---------
     pool.timing_reset()
     pool.timing_enable(True)
-    first = args.warmup + args.steps
+    first = pre_steps + args.warmup + args.steps
     run_steps(pool, seqs, ctx, n_layers, args.steps, *bufs, stream, first_step=first)
     stream.sync()
     pool.timing_enable(False)
@@ -207,6 +224,9 @@ def main() -> int:
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                 "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                 "traffic": MEASURED_TRAFFIC["fetch_bytes"] + MEASURED_TRAFFIC["write_bytes"],
+                "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE profile of this command (seed %d), "
+                                  "profiles/hbm_traffic_all_kernels.md; a constant of this file, not measured "
+                                  "by this run" % MEASURED_TRAFFIC["seed"],
                 "kernel": "decode_attn_mfma_kernel<true> (f16 K/V, all 8 q heads of a kv head per pass on the "
                           "matrix cores, new row taken in flight)",
                 "avg_us": round(split_us, 2),
@@ -220,7 +240,7 @@ def main() -> int:
 
         out = bufs[1].download(np.float32, stream=stream).reshape(len(seqs), N_Q, HD)
         # shortest sequence, layer of the last step
-        last = first + args.steps + max(args.steps // 2, 1) + 4 - 1
+        last = first + args.steps + max(args.steps // 2, 1) + 4 - 1   # `first` counts the preheat steps
         layer = last % n_layers
         i = int(np.argmin(ctx))
         pos = ctx[i] + last // n_layers
@@ -242,7 +262,12 @@ def main() -> int:
         for j in range(len(seqs)):
             oracle.attend(q_host[j], kf[j], vf[j], cells[j], ctx[j] - 1, N_Q, N_KV, HD, threads=nthr)
         cpu_mt_s = time.perf_counter() - t0
+        try:
+            affinity = len(os.sched_getaffinity(0))
+        except AttributeError:
+            affinity = None
         cpu = {"value": round(cpu_bytes / cpu_s / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+               "nproc": os.cpu_count(), "affinity": affinity,
                "sample": "one full batch-8 decode-attention step (all 8 sequences, 16 heads, "
                          "%d cells) in the scalar f64 oracle: %.2f s" % (sum(ctx), cpu_s),
                "us_per_layer": round(cpu_s * 1e6, 0),
@@ -253,6 +278,7 @@ def main() -> int:
     extra = {"attn_split_us": round(split_us, 2), "attn_merge_us": round(ms_merge / max(n_merge, 1) * 1e3, 2),
              "two_call_us_per_layer": round(two_call_us, 2),
              "step_event_ms": round(ev_ms / args.steps, 4),
+             "preheat_ms": round(pre_ms, 1), "preheat_steps": pre_steps,
              "contexts": ctx, "pool_pages": pool.desc.n_pages, "device": dev_name, "cus": n_cu,
              "oracle_check_max_abs": checked}
     pool.destroy()
@@ -260,7 +286,7 @@ def main() -> int:
         b.free()
 
     if not args.no_extra:
-        extra.update(bench_batch1(stream))
+        extra.update(bench_batch1(stream, check=not args.no_cpu))
         extra.update(bench_valu_formulation(stream))
         extra.update(bench_quantised(stream))
         extra.update(bench_select(stream))
@@ -284,7 +310,7 @@ def main() -> int:
     return 0
 
 
-def bench_batch1(stream) -> dict:
+def bench_batch1(stream, check: bool = True) -> dict:
     """BASELINE configs[1]: one sequence at 4096 context, pages scattered over a 64k-page pool,
     12 layers with independent contents; per-layer latency."""
     from breccia_amd import lib as L
@@ -307,7 +333,7 @@ def bench_batch1(stream) -> dict:
         stream.sync()
     kd.free()
     vd.free()
-    _, bufs = make_step_buffers(1, rng)
+    q_host, bufs = make_step_buffers(1, rng)
     steps, warm = 600, 60
     wall_ms, ev_ms = time_steps(pool, [s], [ctx], n_layers, steps, warm, bufs, stream)
     pool.timing_reset()
@@ -321,13 +347,31 @@ def bench_batch1(stream) -> dict:
                            first_step=2 * steps + warm, fused=False)
     bytes_step = attn_algorithmic_bytes([ctx + 1 + (warm + steps // 2) // n_layers])
     us = wall_ms / steps * 1e3
+    checked = None
+    if check:
+        # the last step's output (two-call form) and the last fused step's, against the oracle
+        import oracle
+
+        def against_oracle(step_index):
+            layer, pos = step_index % n_layers, ctx + step_index // n_layers
+            got = bufs[1].download(np.float32, stream=stream).reshape(N_Q, HD)
+            k, v = pool.gather(layer, s, 0, pos + 1, stream)
+            want = oracle.attend(q_host[0], k, v, oracle.dense_cells(pos), pos, N_Q, N_KV, HD, threads=8)
+            return float(np.max(np.abs(got.astype(np.float64) - want)))
+
+        two_call = against_oracle(2 * steps + warm + steps // 2 + 12 - 1)
+        nxt = 2 * steps + warm + steps // 2 + 12
+        run_steps(pool, [s], [ctx], n_layers, 1, *bufs, stream, first_step=nxt)
+        stream.sync()
+        checked = max(two_call, against_oracle(nxt))
     out = {"batch1": {"workload": "BASELINE configs[1]: 1 sequence, ctx 4096, 64k-page pool, 12 layers",
                       "us_per_layer": round(us, 2), "GBps": round(bytes_step / (us * 1e-6) / 1e9, 1),
                       "frac_of_hbm_peak": round(bytes_step / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
                       "attn_split_us": round(ms_split / max(n_split, 1) * 1e3, 2),
                       "attn_merge_us": round(ms_merge / max(n_merge, 1) * 1e3, 2),
                       "two_call_us_per_layer": round(two_ms / (steps // 2) * 1e3, 2),
-                      "ms_per_token_12_layers": round(us * 12 / 1e3, 4)}}
+                      "ms_per_token_12_layers": round(us * 12 / 1e3, 4),
+                      "oracle_check_max_abs": checked}}
     pool.destroy()
     for b in bufs:
         b.free()
@@ -508,6 +552,15 @@ def bench_select(stream) -> dict:
                                    "us": round(e0.elapsed_ms(e1) / 50 * 1e3, 2)}
     e0.close()
     e1.close()
+    pool.timing_reset()
+    pool.timing_enable(True)
+    run_sel(20)
+    stream.sync()
+    pool.timing_enable(False)
+    n_sc, ms_sc = pool.timing_read(L.STAGE_IDX_SCORE)
+    n_tk, ms_tk = pool.timing_read(L.STAGE_TOPK)
+    res["select_blocks_batch8"]["idx_score_us"] = round(ms_sc / max(n_sc, 1) * 1e3, 2)
+    res["select_blocks_batch8"]["topk_us"] = round(ms_tk / max(n_tk, 1) * 1e3, 2)
     for x in [idd, cd, q, out, iq] + pooled:
         x.free()
     pool.destroy()
@@ -553,8 +606,15 @@ def bench_prefill(stream) -> dict:
         us = e0.elapsed_ms(e1) / 10 * 1e3
         e0.close()
         e1.close()
+        pool.timing_reset()
+        pool.timing_enable(True)
+        run(5)
+        stream.sync()
+        pool.timing_enable(False)
+        n_k, ms_k = pool.timing_read(L.STAGE_PREFILL_ATTN)
         res[name] = {"workload": "BASELINE configs[3] shape: 4 sequences, prefix 2048 + chunk 1024, 16q/2kv",
-                     "us": round(us, 1), "useful_TFLOPs": round(flops / us / 1e6, 1),
+                     "us": round(us, 1), "kernel_us": round(ms_k / max(n_k, 1) * 1e3, 1),
+                     "useful_TFLOPs": round(flops / us / 1e6, 1),
                      "frac_of_f16_mfma_peak": round(flops / us / 1e6 / 2500.0, 4)}
         pool.destroy()
     res["prefill_attn"]["issued_TFLOPs"] = round(2 * flops / res["prefill_attn"]["us"] / 1e6, 1)
@@ -667,6 +727,14 @@ def bench_moves(stream) -> dict:
     ms = timed(lambda: pool.append_kprep(0, seqs, [7] * 4, [1] * 4, kd, vd, gd, 1e-6, td, 64, T,
                                          stream=stream), 200)
     res["append_kprep_decode_us"] = round(ms * 1e3, 2)
+    pool.timing_reset()
+    pool.timing_enable(True)
+    for _ in range(5):
+        pool.append_kprep(0, seqs, [0] * 4, [T] * 4, kd, vd, gd, 1e-6, td, 64, T, stream=stream)
+    stream.sync()
+    pool.timing_enable(False)
+    n_k, ms_k = pool.timing_read(L.STAGE_APPEND_KPREP)
+    res["append_kprep_bulk"]["kernel_ms"] = round(ms_k / max(n_k, 1), 4)
     gd.free()
     td.free()
     kd.free()
@@ -718,6 +786,15 @@ def bench_moves(stream) -> dict:
     b = n_swap * pool.swap_page_bytes()
     res["swap"] = {"pages": n_swap, "bytes": b, "out_GBps": round(b / t_out / 1e9, 2),
                    "in_GBps": round(b / t_in / 1e9, 2)}
+    # the device-side gather / scatter of the same pages (page_stage_kernel), by the stage timer
+    pool.timing_reset()
+    pool.timing_enable(True)
+    pool.swap_out(pages, host, stream)
+    pool.swap_wait()
+    pool.timing_enable(False)
+    n_ps, ms_ps = pool.timing_read(L.STAGE_PAGE_STAGE)
+    res["swap"]["page_stage_launches"] = n_ps
+    res["swap"]["page_stage_GBps"] = round(2 * b / max(ms_ps, 1e-9) / 1e6, 1)
     host.free()
 
     # plain device copy of the same volume (ceiling of a read+write stream on this box); after the
@@ -728,6 +805,15 @@ def bench_moves(stream) -> dict:
     ms = timed(lambda: check(lib.bkv_copy_probe(c.ptr, a.ptr, 512 << 20, stream.handle)), 10)
     res["device_copy_probe"] = {"bytes_moved": 2 * (512 << 20), "ms": round(ms, 4),
                                 "GBps": round(2 * (512 << 20) / ms / 1e6, 1)}
+    # read-only stream of the same buffer: in address order, and as 8 KiB chunks in a scattered order
+    # (what a shuffled pool looks like to the attention kernels) -- the ceiling a read-only kernel
+    # can be held against on this box
+    sink = DeviceBuffer(16)
+    for name, scattered in (("device_read_probe_linear", 0), ("device_read_probe_scattered", 1)):
+        ms = timed(lambda: check(lib.bkv_read_probe(a.ptr, 512 << 20, scattered, sink.ptr, stream.handle)), 20)
+        res[name] = {"bytes_read": 512 << 20, "ms": round(ms, 4), "GBps": round((512 << 20) / ms / 1e6, 1),
+                     "frac_of_hbm_peak": round((512 << 20) / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    sink.free()
     a.free()
     c.free()
 

@@ -258,6 +258,9 @@ bkv_status bkv_pool_create(const bkv_pool_desc* d, bkv_pool** out) {
         return fail(BKV_ERR_INVALID,
                     "pool_create: n_layers, n_pages, n_kv_head, max_seqs and max_pages_per_seq "
                     "must all be > 0 (a cache needs capacity > 0)");
+    if (d->n_kv_head > BKV_MAX_KV_HEAD)
+        return fail(BKV_ERR_INVALID, sfmt("pool_create: %lld kv heads; the kernels are built and tested for "
+                                          "at most %lld", d->n_kv_head, BKV_MAX_KV_HEAD));
     if (d->head_dim <= 0 || d->head_dim % 32 != 0 || d->head_dim > 256)
         return fail(BKV_ERR_INVALID, sfmt("pool_create: head_dim %lld must be a multiple of 32 "
                                           "(the q8 block) and at most 256", d->head_dim));
@@ -276,6 +279,7 @@ bkv_status bkv_pool_create(const bkv_pool_desc* d, bkv_pool** out) {
     if (!p) return fail(BKV_ERR_NOMEM, "pool_create: out of host memory");
     p->desc = *d;
     p->host_only = (d->flags & BKV_POOL_HOST_ONLY) != 0;
+    p->max_wgs = kMaxWgs;
     Geom& g = p->g;
     g.n_layers = d->n_layers, g.n_pages = d->n_pages, g.n_kv = d->n_kv_head, g.hd = d->head_dim;
     g.page_cells = d->page_cells, g.layout = d->layout;
@@ -339,7 +343,6 @@ bkv_status bkv_pool_create(const bkv_pool_desc* d, bkv_pool** out) {
     BKV_TRY(hipMalloc(reinterpret_cast<void**>(&p->table_dev), (table_bytes + 15u) & ~15ull));
     BKV_TRY(launch_fill(p->table_dev, (table_bytes + 15u) & ~15ull, 0xffffffffu, nullptr));
 
-    p->max_wgs = 4096;
     BKV_TRY(hipMalloc(reinterpret_cast<void**>(&p->part_o), (uint64_t)p->max_wgs * 8u * 256u * 4u));
     BKV_TRY(hipMalloc(reinterpret_cast<void**>(&p->part_ml), (uint64_t)p->max_wgs * 8u * 2u * 4u));
 
@@ -650,6 +653,32 @@ bkv_status bkv_pool_check(const bkv_pool* p) {
 }
 
 // ---- append ------------------------------------------------------------------------
+// Cells [c0, c1) of a live sequence may be written only when they have been reserved
+// (bkv_seq_reserve moved the sequence's length past them) and every page they lie on is on the
+// device and held by this sequence alone: a page that a fork, a cached prefix or another
+// sequence still shares would change under its other holders.  bkv_seq_reserve is what replaces
+// such a page (and reports the copy to make); writing without it is a state error here, before
+// anything is launched.
+static bkv_status check_writable(const bkv_pool* p, const char* what, int32_t seq, int64_t c0, int64_t c1) {
+    const int64_t len = p->alloc->seq_len(seq);
+    if (c1 > len)
+        return fail(BKV_ERR_RANGE, std::string(what) + sfmt(" would write cells %lld..%lld of sequence %lld but "
+                                                            "only %lld are reserved (bkv_seq_reserve first)",
+                                                            c0, c1, seq, len));
+    const int32_t* row = p->alloc->seq_table(seq);
+    for (int64_t c = c0 / p->g.page_cells; c <= (c1 - 1) / p->g.page_cells; ++c) {
+        if (row[c] < 0)
+            return fail(BKV_ERR_STATE, std::string(what) + sfmt(": logical page %lld of sequence %lld is "
+                                                                "swapped out", c, seq));
+        if (p->alloc->refcount(row[c]) != 1)
+            return fail(BKV_ERR_STATE, std::string(what) + sfmt(": logical page %lld of sequence %lld (page %lld) "
+                                                                "has %lld holders; bkv_seq_reserve replaces a "
+                                                                "shared page before it is written",
+                                                                c, seq, row[c], p->alloc->refcount(row[c])));
+    }
+    return BKV_OK;
+}
+
 // Range checks shared by the append entry points (qsa/mod.rs:1108-1116: a write past the
 // cache is an error before anything is launched) and the per-sequence launch arguments.
 static bkv_status build_append_batch(bkv_pool* p, int32_t layer, int32_t n_seqs, const int32_t* seqs,
@@ -681,11 +710,8 @@ static bkv_status build_append_batch(bkv_pool* p, int32_t layer, int32_t n_seqs,
                              "%lld (a write past the block table would land on an unmapped page)",
                              pos0[i], end, seqs[i], cap));
         if (n_tokens[i] > 0) {
-            const int32_t* row = p->alloc->seq_table(seqs[i]);
-            for (int64_t c = pos0[i] / p->g.page_cells; c <= (end - 1) / p->g.page_cells; ++c)
-                if (row[c] < 0)
-                    return fail(BKV_ERR_STATE, sfmt("append: logical page %lld of sequence %lld is "
-                                                    "swapped out", c, seqs[i]));
+            bkv_status wst = check_writable(p, "append", seqs[i], pos0[i], end);
+            if (wst != BKV_OK) return wst;
         }
         b.row[i] = seqs[i];
         b.pos0[i] = (int32_t)pos0[i];
@@ -826,6 +852,10 @@ static bkv_status decode_attn_common(bkv_pool* p, int32_t layer, int32_t n, cons
         if (!p->alloc->seq_resident(seqs[i], pos[i] + 1))
             return fail(BKV_ERR_STATE, sfmt("decode_attn: sequence %lld has swapped-out pages "
                                             "below position %lld", seqs[i], pos[i]));
+        if (step) {
+            const bkv_status wst = check_writable(p, "decode_step", seqs[i], pos[i], pos[i] + 1);
+            if (wst != BKV_OK) return wst;
+        }
         if (step)
             for (int j = 0; j < i; ++j)
                 if (seqs[j] == seqs[i])
@@ -852,9 +882,15 @@ static bkv_status decode_attn_common(bkv_pool* p, int32_t layer, int32_t n, cons
         return fail(BKV_ERR_INVALID, "decode_step on a quantised pool is served by the matrix-core kernels "
                                      "only (at most 16 q heads per kv head, pool without "
                                      "BKV_POOL_ATTN_VALU); append and attend in two calls instead");
+    // the cut into work-groups comes before anything is enqueued: a batch it cannot serve is an
+    // error like any other size violation
+    if (plan_attn(p, n_q_head, b, select ? (max_ids + 3) / 4 : 0, mfma) < 0)
+        return fail(BKV_ERR_INVALID,
+                    sfmt("decode_attn: %lld entries x %lld kv heads need more work-groups than the "
+                         "partial-result workspace holds (%lld); use smaller batches", n, p->g.n_kv,
+                         attn_plan_limits(p->n_cu, p->max_wgs, p->g.n_kv, n_q_head / p->g.n_kv, mfma).max_wgs));
     st = flush_tables(p, S(stream));
     if (st != BKV_OK) return st;
-    plan_attn(p, n_q_head, b, select ? (max_ids + 3) / 4 : 0, mfma);
     AttnArgs a;
     a.mfma = mfma;
     a.n_q_head = n_q_head;
@@ -878,6 +914,37 @@ static bkv_status decode_attn_common(bkv_pool* p, int32_t layer, int32_t n, cons
     if (st != BKV_OK) return st;
     BKV_HIP(launch_decode_attn(p, layer, b, a, S(stream)));
     if (p->timer.open.size() > 8192) return timer_collect(p);
+    return BKV_OK;
+}
+
+bkv_status bkv_attn_plan(int32_t n_cu, int32_t n_kv_head, int32_t n_q_head, int32_t n, const int64_t* pos,
+                         int32_t sel_groups, int32_t matrix_cores, int32_t* splits_out, int32_t* pps_out,
+                         int32_t* total_out) {
+    if (n_cu <= 0 || n_kv_head <= 0 || n_kv_head > BKV_MAX_KV_HEAD)
+        return fail(BKV_ERR_INVALID, sfmt("attn_plan: %lld compute units, %lld kv heads", n_cu, n_kv_head));
+    if (n_q_head <= 0 || n_q_head % n_kv_head != 0 || n_q_head / n_kv_head > BKV_MAX_HEAD_GROUP)
+        return fail(BKV_ERR_INVALID, sfmt("attn_plan: %lld q heads over %lld kv heads (need a whole group of "
+                                          "at most %lld)", n_q_head, n_kv_head, BKV_MAX_HEAD_GROUP));
+    if (n < 0 || n > BKV_MAX_BATCH || (n > 0 && !pos) || sel_groups < 0)
+        return fail(BKV_ERR_INVALID, sfmt("attn_plan: %lld entries (limit %lld), sel_groups %lld", n,
+                                          BKV_MAX_BATCH, sel_groups));
+    AttnBatch b{};
+    b.n = n;
+    for (int i = 0; i < n; ++i) {
+        if (pos[i] < 0 || pos[i] > 0x7ffffff0)
+            return fail(BKV_ERR_RANGE, sfmt("attn_plan: position %lld of entry %lld", pos[i], i));
+        b.pos[i] = (int32_t)pos[i];
+    }
+    const AttnPlanLimits lim = attn_plan_limits(n_cu, kMaxWgs, n_kv_head, n_q_head / n_kv_head, matrix_cores != 0);
+    const int32_t total = plan_attn_ranges(lim, 16, sel_groups, b);
+    if (total < 0)
+        return fail(BKV_ERR_INVALID, sfmt("attn_plan: %lld entries x %lld kv heads need more work-groups than "
+                                          "the partial-result workspace holds (%lld)", n, n_kv_head, lim.max_wgs));
+    for (int i = 0; i < n; ++i) {
+        if (splits_out) splits_out[i] = b.splits[i];
+        if (pps_out) pps_out[i] = b.pps[i];
+    }
+    if (total_out) *total_out = total;
     return BKV_OK;
 }
 
@@ -1030,7 +1097,7 @@ bkv_status bkv_idx_pool(bkv_pool* p, float* pooled_dev, int32_t max_blocks, floa
     if (tokens == 0) return BKV_OK;
     if (!pooled_dev || !tail_dev || !idx_k_dev || !gamma_dev || !rope_table_dev)
         return fail(BKV_ERR_INVALID, "idx_pool: NULL device pointer");
-    BKV_HIP(launch_idx_pool(idx_k_dev, tail_dev, gamma_dev, rope_table_dev, pooled_dev, (int32_t)pos0, tokens,
+    BKV_HIP(launch_idx_pool(p, idx_k_dev, tail_dev, gamma_dev, rope_table_dev, pooled_dev, (int32_t)pos0, tokens,
                             idx_dim, 4, n_rot, max_pos, eps, S(stream)));
     return BKV_OK;
 }
@@ -1052,7 +1119,7 @@ bkv_status bkv_topk_blocks(bkv_pool* p, int32_t n, const int64_t* pos, const flo
         b.pos[i] = (int32_t)pos[i];
         b.n_blocks[i] = n_blocks;
     }
-    BKV_HIP(launch_topk_blocks(b, scores_dev, false, n_blocks, topk_blocks, 4, dense != 0, ids_dev,
+    BKV_HIP(launch_topk_blocks(p, b, scores_dev, false, n_blocks, topk_blocks, 4, dense != 0, ids_dev,
                                id_stride, counts_dev, max_ids, S(stream)));
     return BKV_OK;
 }
@@ -1100,9 +1167,9 @@ bkv_status bkv_select_blocks(bkv_pool* p, int32_t n, const int64_t* pos, const f
     const bkv_status ws = order_workspace(p->sel_ws, S(stream));
     if (ws != BKV_OK) return ws;
     if (max_blocks > 0)
-        BKV_HIP(launch_idx_score(b, idx_q_dev, idx_n_head, idx_dim, 4, p->sel_scores, (int64_t)stride,
+        BKV_HIP(launch_idx_score(p, b, idx_q_dev, idx_n_head, idx_dim, 4, p->sel_scores, (int64_t)stride,
                                  max_blocks, S(stream)));
-    BKV_HIP(launch_topk_blocks(b, p->sel_scores, true, (int64_t)stride, topk_blocks, 4, false, ids_dev,
+    BKV_HIP(launch_topk_blocks(p, b, p->sel_scores, true, (int64_t)stride, topk_blocks, 4, false, ids_dev,
                                id_stride, counts_dev, max_ids, S(stream)));
     return BKV_OK;
 }
@@ -1189,7 +1256,10 @@ static bkv_status swap_move(bkv_pool* p, const int32_t* pages, int32_t n, uint8_
         void* pages_dev;
         int slot;
         if (out) {
+            // the half is free once its last transfer (side stream) and its last unpack kernel (a
+            // swap-in, possibly on another caller stream) are over
             BKV_HIP(hipStreamWaitEvent(stream, sg.ev_side[h], 0));
+            BKV_HIP(hipStreamWaitEvent(stream, sg.ev_stream[h], 0));
             bkv_status st = ring_upload(p, pages + at, (size_t)m * 4, stream, &pages_dev, &slot);
             if (st != BKV_OK) return st;
             BKV_HIP(launch_page_stage(p, static_cast<const int32_t*>(pages_dev), m, sg.dev[h], 1,
@@ -1674,6 +1744,20 @@ bkv_status bkv_copy_probe(void* dst_dev, const void* src_dev, uint64_t bytes, vo
     if (!dst_dev || !src_dev || !aligned16(dst_dev) || !aligned16(src_dev) || bytes % 16)
         return fail(BKV_ERR_INVALID, "copy_probe: pointers and size must be 16-byte multiples");
     BKV_HIP(launch_copy_probe(dst_dev, src_dev, bytes, S(stream)));
+    return BKV_OK;
+}
+
+bkv_status bkv_read_probe(const void* src_dev, uint64_t bytes, int32_t scattered, void* sink_dev, void* stream) {
+    if (!src_dev || !sink_dev || !aligned16(src_dev) || ((uintptr_t)sink_dev & 3u))
+        return fail(BKV_ERR_INVALID, "read_probe: NULL or misaligned pointer");
+    const uint64_t chunks = bytes / 8192;
+    if (bytes % 8192 != 0 || chunks == 0 || chunks > 0x7fffffffull || (chunks & (chunks - 1)) != 0)
+        return fail(BKV_ERR_INVALID, sfmt("read_probe: %lld bytes; need a power-of-two number of 8 KiB chunks",
+                                          (long long)bytes));
+    int dev = 0, n_cu = 0;
+    BKV_HIP(hipGetDevice(&dev));
+    BKV_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
+    BKV_HIP(launch_read_probe(src_dev, bytes, scattered != 0, sink_dev, n_cu, S(stream)));
     return BKV_OK;
 }
 

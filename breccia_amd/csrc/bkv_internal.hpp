@@ -11,6 +11,7 @@
 
 #include "../../include/breccia_kv.h"
 #include "allocator.hpp"
+#include "attn_plan.hpp"
 #include "prefix_tree.hpp"
 
 namespace bkv {
@@ -25,6 +26,9 @@ bkv_status hip_fail(hipError_t e, const char* what);
         hipError_t e__ = (call);                                      \
         if (e__ != hipSuccess) return ::bkv::hip_fail(e__, #call);    \
     } while (0)
+
+// work-groups the split-K partial-result workspace is sized for (x 8 head rows of 256 floats)
+constexpr int32_t kMaxWgs = 4096;
 
 // ---- geometry ----------------------------------------------------------------
 struct Geom {
@@ -179,28 +183,20 @@ struct SelectBatch {
     int32_t n_blocks[BKV_MAX_BATCH];  // pooled / scored blocks of the entry
     const float* pooled[BKV_MAX_BATCH];  // [n_blocks][idx_dim] (score kernel only)
 };
-hipError_t launch_idx_score(const SelectBatch& b, const float* q, int32_t idx_n_head, int32_t idx_dim,
+hipError_t launch_idx_score(bkv_pool* p, const SelectBatch& b, const float* q, int32_t idx_n_head, int32_t idx_dim,
                             int32_t idx_block, double* scores, int64_t score_stride, int32_t max_blocks,
                             hipStream_t stream);
-hipError_t launch_topk_blocks(const SelectBatch& b, const void* scores, bool scores_f64,
+hipError_t launch_topk_blocks(bkv_pool* p, const SelectBatch& b, const void* scores, bool scores_f64,
                               int64_t score_stride, int32_t topk_blocks, int32_t idx_block, bool dense,
                               uint32_t* ids, int64_t id_stride, uint32_t* counts, int32_t max_ids,
                               hipStream_t stream);
-hipError_t launch_idx_pool(const float* raw, float* tail, const float* gamma, const float* table,
+hipError_t launch_idx_pool(bkv_pool* p, const float* raw, float* tail, const float* gamma, const float* table,
                            float* pooled, int32_t pos0, int32_t tokens, int32_t idx_dim, int32_t idx_block,
                            int32_t n_rot, int32_t max_pos, float eps, hipStream_t stream);
 int32_t select_max_topk();
 int32_t select_max_idx_head();
 int32_t select_max_idx_dim();
 
-struct AttnBatch {
-    int32_t n;
-    int32_t row[BKV_MAX_BATCH];       // block-table row
-    int32_t pos[BKV_MAX_BATCH];       // last visible cell
-    int32_t wg_base[BKV_MAX_BATCH + 1];  // first work-group of the entry; [n] = total
-    int32_t splits[BKV_MAX_BATCH];    // page ranges the entry is cut into
-    int32_t pps[BKV_MAX_BATCH];       // pages per split
-};
 struct AttnArgs {
     int32_t n_q_head;
     const float* q;
@@ -218,8 +214,10 @@ struct AttnArgs {
     const float* new_v = nullptr;
     bool mfma = false;  // dense f16 call routed to the MFMA kernel (all heads of a group at once)
 };
-// Fills wg_base/splits/pps from row/pos; returns the total work-group count.  sel_groups > 0:
+// Fills wg_base/splits/pps from row/pos (attn_plan.hpp); returns the total work-group count, -1
+// when the batch cannot be cut into as few work-groups as the workspace holds.  sel_groups > 0:
 // every entry is planned for that many groups of four selected blocks instead of its pages.
+AttnPlanLimits attn_plan_limits(int32_t n_cu, int32_t max_wgs, int32_t n_kv, int32_t group, bool mfma);
 int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b, int32_t sel_groups = 0,
                   bool mfma = false);
 bool attn_on_mfma(const bkv_pool* p, int32_t group, bool dense);
@@ -244,7 +242,7 @@ hipError_t launch_page_copy(bkv_pool* p, const bkv_page_pair* pairs_dev, int32_t
                             hipStream_t stream);
 // Gather (to_stage=1) / scatter (to_stage=0) whole pages between the pools and a
 // contiguous staging buffer laid out [page][layer][K bytes | V bytes].
-hipError_t launch_page_stage(const bkv_pool* p, const int32_t* pages_dev, int32_t n_pages,
+hipError_t launch_page_stage(bkv_pool* p, const int32_t* pages_dev, int32_t n_pages,
                              uint8_t* stage, int to_stage, hipStream_t stream);
 hipError_t launch_gather(const bkv_pool* p, int32_t layer, int32_t row, int64_t cell0, int64_t n,
                          float* k_out, float* v_out, hipStream_t stream);
@@ -252,5 +250,7 @@ hipError_t launch_table_scatter(int32_t* table, const TableUpdate* upd_dev, int3
                                 hipStream_t stream);
 hipError_t launch_fill(void* dst, uint64_t bytes, uint32_t word, hipStream_t stream);
 hipError_t launch_copy_probe(void* dst, const void* src, uint64_t bytes, hipStream_t stream);
+hipError_t launch_read_probe(const void* src, uint64_t bytes, bool scattered, void* sink, int32_t n_cu,
+                             hipStream_t stream);
 
 }  // namespace bkv

@@ -728,43 +728,27 @@ bool attn_on_mfma(const bkv_pool* p, int32_t group, bool dense) {
     return p->g.layout == BKV_LAYOUT_F16 || dense;
 }
 
-int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b, int32_t sel_groups, bool mfma) {
-    const int32_t n_kv = p->g.n_kv;
-    const int32_t group = n_q_head / n_kv;
+// The limits a plan of this pool geometry works under.  The partial-result workspace holds
+// max_wgs x 8 head rows: a work-group of the matrix-core kernels writes `group` rows, one of the
+// VALU kernel 8 or 4.
+AttnPlanLimits attn_plan_limits(int32_t n_cu, int32_t max_wgs, int32_t n_kv, int32_t group, bool mfma) {
     const int32_t hg = mfma ? group : attn_heads_per_wave(group);
     const int32_t n_hc = (group + hg - 1) / hg;
-    const int64_t per_page = (int64_t)n_kv * n_hc;
-    int64_t total_pages = 0;
-    // loop iterations of an entry: its pages, or (selection lists, whose true lengths only the
-    // device knows) the most groups of four blocks a list can hold
-    const auto iters = [&](int i) -> int64_t { return sel_groups > 0 ? sel_groups : b.pos[i] / kPage + 1; };
-    for (int i = 0; i < b.n; ++i) total_pages += iters(i);
+    AttnPlanLimits lim;
+    lim.per_page = n_kv * n_hc;
+    lim.gran = kWaves;
     // All work-groups should be resident at once (one generation): a handful of left-over
     // work-groups would run alone after the rest and double the kernel's time.  `resident`
     // follows from the register budget of the kernel variant that will run.
-    const int64_t resident = (mfma || hg == 8) ? 2 : 3;
-    int64_t target = (int64_t)(p->n_cu > 0 ? p->n_cu : 256) * resident;
-    if (target > p->max_wgs) target = p->max_wgs;
-    int64_t pps = (total_pages * per_page + target - 1) / target;
-    pps = ((pps + kWaves - 1) / kWaves) * kWaves;
-    if (pps < kWaves) pps = kWaves;
-    for (;;) {
-        int64_t total = 0;
-        for (int i = 0; i < b.n; ++i) {
-            const int64_t pages = iters(i);
-            const int64_t splits = (pages + pps - 1) / pps;
-            // even the ranges out inside the entry, keeping whole groups of kWaves pages
-            int64_t each = (pages + splits - 1) / splits;
-            each = ((each + kWaves - 1) / kWaves) * kWaves;
-            b.splits[i] = (int32_t)((pages + each - 1) / each);
-            b.pps[i] = (int32_t)each;
-            b.wg_base[i] = (int32_t)total;
-            total += (int64_t)b.splits[i] * per_page;
-        }
-        b.wg_base[b.n] = (int32_t)total;
-        if (total <= target) return (int32_t)total;
-        pps += kWaves;
-    }
+    const int32_t resident = (mfma || hg == 8) ? 2 : 3;
+    lim.target = (n_cu > 0 ? n_cu : 256) * resident;
+    lim.max_wgs = hg > 8 ? (int32_t)((int64_t)max_wgs * 8 / hg) : max_wgs;
+    return lim;
+}
+
+int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b, int32_t sel_groups, bool mfma) {
+    const AttnPlanLimits lim = attn_plan_limits(p->n_cu, p->max_wgs, p->g.n_kv, n_q_head / p->g.n_kv, mfma);
+    return plan_attn_ranges(lim, kPage, sel_groups, b);
 }
 
 hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, const AttnArgs& a,

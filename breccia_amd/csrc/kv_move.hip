@@ -568,6 +568,34 @@ __global__ __launch_bounds__(kBlock) void copy_probe_kernel(uint4* __restrict__ 
     for (; i < n_vec; i += stride) dst[i] = src[i];
 }
 
+// Read-only bandwidth probe: every wave reads 8 KiB chunks (8 wave-loads of 1 KiB, the shape of
+// one (page, kv head) run of a pool) and folds them into a value nothing depends on.  Chunk c of
+// the walk is chunk c of the buffer, or, scattered, chunk (c * odd) mod n_chunks of it (n_chunks a
+// power of two: a bijection), which is how a shuffled pool looks to the attention kernels.
+typedef unsigned probe_v4u __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(kBlock) void read_probe_kernel(const probe_v4u* __restrict__ src, uint32_t n_chunks,
+                                                            uint32_t scatter_mul, uint32_t* __restrict__ sink) {
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = (blockIdx.x * kBlock + threadIdx.x) >> 6;
+    const uint32_t n_waves = gridDim.x * (kBlock / 64);
+    probe_v4u acc = probe_v4u{0u, 0u, 0u, 0u};
+    for (uint32_t c = wave; c < n_chunks; c += 2 * n_waves) {
+        const uint32_t c1 = c + n_waves < n_chunks ? c + n_waves : c;
+        const probe_v4u* a = src + (size_t)((c * scatter_mul) & (n_chunks - 1u)) * 512u + lane;
+        const probe_v4u* b = src + (size_t)((c1 * scatter_mul) & (n_chunks - 1u)) * 512u + lane;
+        probe_v4u r[16];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) r[i] = __builtin_nontemporal_load(a + i * 64);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) r[8 + i] = __builtin_nontemporal_load(b + i * 64);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            acc ^= r[i];
+        }
+    }
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u) sink[0] = 1u;  // keeps the loads alive
+}
+
 MoveGeom move_geom(const bkv_pool* p) {
     return MoveGeom{p->g.n_kv, p->g.hd, p->g.page_cells, p->desc.max_pages_per_seq};
 }
@@ -637,7 +665,7 @@ hipError_t launch_append_kprep(bkv_pool* p, int32_t layer, const AppendBatch& b,
     uint8_t* kpl = p->k_layer[(size_t)layer];
     uint8_t* vpl = p->v_layer[(size_t)layer];
     const auto launch = [&](auto layout_tag, auto hd_tag) {
-        launch_staged(p, BKV_STAGE_APPEND, append_kprep_kernel<decltype(layout_tag)::value, decltype(hd_tag)::value>,
+        launch_staged(p, BKV_STAGE_APPEND_KPREP, append_kprep_kernel<decltype(layout_tag)::value, decltype(hd_tag)::value>,
                       grid, dim3(kBlock), (uint32_t)lds, stream, b, g, kp, kpl, vpl, (const int32_t*)p->table_dev, k, v);
     };
     const auto by_hd = [&](auto layout_tag) {
@@ -674,13 +702,13 @@ hipError_t launch_page_copy(bkv_pool* p, const bkv_page_pair* pairs_dev, int32_t
     return hipGetLastError();
 }
 
-hipError_t launch_page_stage(const bkv_pool* p, const int32_t* pages_dev, int32_t n_pages,
+hipError_t launch_page_stage(bkv_pool* p, const int32_t* pages_dev, int32_t n_pages,
                              uint8_t* stage, int to_stage, hipStream_t stream) {
     const PoolPtrs pp = pool_ptrs(p);
     const uint64_t pb = pp.k_page_bytes > pp.v_page_bytes ? pp.k_page_bytes : pp.v_page_bytes;
     const unsigned chunks = (unsigned)((pb / 16 + 4 * kBlock - 1) / (4 * kBlock));
     dim3 grid(chunks, (unsigned)n_pages * (unsigned)pp.n_layers * 2u);
-    page_stage_kernel<<<grid, kBlock, 0, stream>>>(pp, pages_dev, stage, to_stage);
+    launch_staged(p, BKV_STAGE_PAGE_STAGE, page_stage_kernel, grid, dim3(kBlock), 0, stream, pp, pages_dev, stage, to_stage);
     return hipGetLastError();
 }
 
@@ -718,6 +746,18 @@ hipError_t launch_copy_probe(void* dst, const void* src, uint64_t bytes, hipStre
     uint64_t blocks = (n_vec + 4 * kBlock - 1) / (4 * kBlock);
     if (blocks > 8192) blocks = 8192;
     copy_probe_kernel<<<(unsigned)blocks, kBlock, 0, stream>>>((uint4*)dst, (const uint4*)src, n_vec);
+    return hipGetLastError();
+}
+
+hipError_t launch_read_probe(const void* src, uint64_t bytes, bool scattered, void* sink, int32_t n_cu,
+                             hipStream_t stream) {
+    const uint32_t n_chunks = (uint32_t)(bytes / 8192);
+    if (n_chunks == 0) return hipSuccess;
+    // two resident generations of 4-wave work-groups at the decode kernels' occupancy
+    uint32_t blocks = (uint32_t)(n_cu > 0 ? n_cu : 256) * 4u;
+    if (blocks * (kBlock / 64) > n_chunks) blocks = (n_chunks + kBlock / 64 - 1) / (kBlock / 64);
+    read_probe_kernel<<<blocks, kBlock, 0, stream>>>((const probe_v4u*)src, n_chunks, scattered ? 0x9e3779b1u : 1u,
+                                                     (uint32_t*)sink);
     return hipGetLastError();
 }
 

@@ -537,13 +537,13 @@ hipError_t launch_prefill_attn(bkv_pool* p, int32_t layer, const PrefillBatch& b
     const int32_t grid = b.wg_base[b.n];
     if (grid == 0) return hipSuccess;
     if (p->g.layout == BKV_LAYOUT_Q8V)
-        launch_staged(p, BKV_STAGE_ATTN_SPLIT, prefill_attn_kernel<BKV_LAYOUT_Q8V>, dim3((unsigned)grid), dim3(512), 0,
+        launch_staged(p, BKV_STAGE_PREFILL_ATTN, prefill_attn_kernel<BKV_LAYOUT_Q8V>, dim3((unsigned)grid), dim3(512), 0,
                       stream, kp);
     else if (p->g.layout == BKV_LAYOUT_I8H)
-        launch_staged(p, BKV_STAGE_ATTN_SPLIT, prefill_attn_kernel<BKV_LAYOUT_I8H>, dim3((unsigned)grid), dim3(512), 0,
+        launch_staged(p, BKV_STAGE_PREFILL_ATTN, prefill_attn_kernel<BKV_LAYOUT_I8H>, dim3((unsigned)grid), dim3(512), 0,
                       stream, kp);
     else
-        launch_staged(p, BKV_STAGE_ATTN_SPLIT, prefill_attn_kernel<BKV_LAYOUT_F16>, dim3((unsigned)grid), dim3(256), 0,
+        launch_staged(p, BKV_STAGE_PREFILL_ATTN, prefill_attn_kernel<BKV_LAYOUT_F16>, dim3((unsigned)grid), dim3(256), 0,
                       stream, kp);
     return hipGetLastError();
 }

@@ -567,7 +567,7 @@ __global__ __launch_bounds__(kTopkThreads) void topk_blocks_kernel(const TopkPar
 
 }  // namespace
 
-hipError_t launch_idx_score(const SelectBatch& b, const float* q, int32_t idx_n_head, int32_t idx_dim,
+hipError_t launch_idx_score(bkv_pool* p, const SelectBatch& b, const float* q, int32_t idx_n_head, int32_t idx_dim,
                             int32_t idx_block, double* scores, int64_t score_stride, int32_t max_blocks,
                             hipStream_t stream) {
     ScoreParams sp;
@@ -582,13 +582,13 @@ hipError_t launch_idx_score(const SelectBatch& b, const float* q, int32_t idx_n_
     bool wide = idx_dim == 128 && (reinterpret_cast<uintptr_t>(q) & 15u) == 0;
     for (int i = 0; i < b.n && wide; ++i) wide = (reinterpret_cast<uintptr_t>(b.pooled[i]) & 15u) == 0;
     if (wide)
-        idx_score_kernel<128><<<grid, kScoreThreads, 0, stream>>>(sp);
+        launch_staged(p, BKV_STAGE_IDX_SCORE, idx_score_kernel<128>, grid, dim3(kScoreThreads), 0, stream, sp);
     else
-        idx_score_kernel<0><<<grid, kScoreThreads, 0, stream>>>(sp);
+        launch_staged(p, BKV_STAGE_IDX_SCORE, idx_score_kernel<0>, grid, dim3(kScoreThreads), 0, stream, sp);
     return hipGetLastError();
 }
 
-hipError_t launch_topk_blocks(const SelectBatch& b, const void* scores, bool scores_f64,
+hipError_t launch_topk_blocks(bkv_pool* p, const SelectBatch& b, const void* scores, bool scores_f64,
                               int64_t score_stride, int32_t topk_blocks, int32_t idx_block, bool dense,
                               uint32_t* ids, int64_t id_stride, uint32_t* counts, int32_t max_ids,
                               hipStream_t stream) {
@@ -608,19 +608,19 @@ hipError_t launch_topk_blocks(const SelectBatch& b, const void* scores, bool sco
     const bool few = longest <= 8 * kTopkThreads;
     if (scores_f64) {
         if (few)
-            topk_blocks_kernel<double, 8><<<b.n, kTopkThreads, 0, stream>>>(tp);
+            launch_staged(p, BKV_STAGE_TOPK, topk_blocks_kernel<double, 8>, dim3((unsigned)b.n), dim3(kTopkThreads), 0, stream, tp);
         else
-            topk_blocks_kernel<double, 32><<<b.n, kTopkThreads, 0, stream>>>(tp);
+            launch_staged(p, BKV_STAGE_TOPK, topk_blocks_kernel<double, 32>, dim3((unsigned)b.n), dim3(kTopkThreads), 0, stream, tp);
     } else {
         if (few)
-            topk_blocks_kernel<float, 8><<<b.n, kTopkThreads, 0, stream>>>(tp);
+            launch_staged(p, BKV_STAGE_TOPK, topk_blocks_kernel<float, 8>, dim3((unsigned)b.n), dim3(kTopkThreads), 0, stream, tp);
         else
-            topk_blocks_kernel<float, 32><<<b.n, kTopkThreads, 0, stream>>>(tp);
+            launch_staged(p, BKV_STAGE_TOPK, topk_blocks_kernel<float, 32>, dim3((unsigned)b.n), dim3(kTopkThreads), 0, stream, tp);
     }
     return hipGetLastError();
 }
 
-hipError_t launch_idx_pool(const float* raw, float* tail, const float* gamma, const float* table,
+hipError_t launch_idx_pool(bkv_pool* p, const float* raw, float* tail, const float* gamma, const float* table,
                            float* pooled, int32_t pos0, int32_t tokens, int32_t idx_dim, int32_t idx_block,
                            int32_t n_rot, int32_t max_pos, float eps, hipStream_t stream) {
     PoolKeysParams pp;
@@ -639,13 +639,14 @@ hipError_t launch_idx_pool(const float* raw, float* tail, const float* gamma, co
     pp.max_pos = max_pos;
     pp.eps = eps;
     if (pp.n_new > 0) {
-        idx_pool_kernel<<<pp.n_new, kMaxIdxDim, 0, stream>>>(pp);
+        launch_staged(p, BKV_STAGE_IDX_POOL, idx_pool_kernel, dim3((unsigned)pp.n_new), dim3(kMaxIdxDim), 0, stream, pp);
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
     // the tail is read by the pooling above and rewritten here: stream order keeps them apart
     const int total = tokens * idx_dim;
-    idx_tail_kernel<<<(total + 255) / 256, 256, 0, stream>>>(raw, tail, tokens, pos0, idx_dim, idx_block);
+    launch_staged(p, BKV_STAGE_IDX_POOL, idx_tail_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, raw, tail, tokens, pos0,
+                  idx_dim, idx_block);
     return hipGetLastError();
 }
 

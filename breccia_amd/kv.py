@@ -73,6 +73,19 @@ def rope_table(freq_base: float, n_rot: int, max_pos: int) -> np.ndarray:
     return out
 
 
+def attn_plan(n_cu: int, n_kv_head: int, n_q_head: int, pos, sel_groups: int = 0, matrix_cores: bool = True):
+    """How the library would cut a decode-attention batch into work-groups on a device of n_cu
+    compute units -> (splits per entry, pages per split, total work-groups).  Host only."""
+    pos, pp = _i64(pos)
+    splits = np.zeros(max(pos.size, 1), dtype=np.int32)
+    pps = np.zeros(max(pos.size, 1), dtype=np.int32)
+    total = C.c_int32()
+    check(lib.bkv_attn_plan(n_cu, n_kv_head, n_q_head, pos.size, pp, sel_groups, 1 if matrix_cores else 0,
+                            splits.ctypes.data_as(C.POINTER(C.c_int32)), pps.ctypes.data_as(C.POINTER(C.c_int32)),
+                            C.byref(total)))
+    return splits[:pos.size], pps[:pos.size], int(total.value)
+
+
 def device_sync() -> None:
     check(lib.bkv_device_sync())
 

@@ -18,7 +18,9 @@ LAYOUT_F16, LAYOUT_Q8V, LAYOUT_I8H = 0, 1, 2
 POOL_HOST_ONLY = 1
 POOL_ATTN_VALU = 2
 MAX_BATCH = 64
-STAGE_APPEND, STAGE_ATTN_SPLIT, STAGE_ATTN_MERGE, STAGE_PAGE_COPY = range(4)
+MAX_KV_HEAD = 16
+(STAGE_APPEND, STAGE_ATTN_SPLIT, STAGE_ATTN_MERGE, STAGE_PAGE_COPY, STAGE_PREFILL_ATTN, STAGE_APPEND_KPREP,
+ STAGE_IDX_POOL, STAGE_IDX_SCORE, STAGE_TOPK, STAGE_PAGE_STAGE) = range(10)
 
 
 class BkvError(RuntimeError):
@@ -96,6 +98,7 @@ _SIGNATURES = {
     "bkv_rope_table": (C.c_int, [C.c_double, _i32, _i32, _vp]),
     "bkv_decode_attn": (C.c_int, [_vp, _i32, _i32, _pi32, _pi64, _i32, _vp, _vp, _i64, _i64, _f32,
                                   _vp, _vp]),
+    "bkv_attn_plan": (C.c_int, [_i32, _i32, _i32, _i32, _pi64, _i32, _i32, _pi32, _pi32, _pi32]),
     "bkv_prefill_attn": (C.c_int, [_vp, _i32, _i32, _pi32, _pi64, _pi32, _i32, _vp, _vp, _i64, _i64, _f32,
                                    _vp, _vp]),
     "bkv_decode_step": (C.c_int, [_vp, _i32, _i32, _pi32, _pi64, _vp, _vp, _i32, _vp, _vp, _i64, _i64, _f32,
@@ -132,6 +135,7 @@ _SIGNATURES = {
     "bkv_event_elapsed_ms": (C.c_int, [_vp, _vp, C.POINTER(C.c_float)]),
     "bkv_device_info": (C.c_int, [C.c_char_p, _i32, _pi32, C.POINTER(_u64)]),
     "bkv_copy_probe": (C.c_int, [_vp, _vp, _u64, _vp]),
+    "bkv_read_probe": (C.c_int, [_vp, _u64, _i32, _vp, _vp]),
 }
 
 for _name, (_res, _args) in _SIGNATURES.items():

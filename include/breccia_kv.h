@@ -61,6 +61,7 @@ enum {
 
 #define BKV_MAX_BATCH 64      /* (sequence, position) entries per append / attention call */
 #define BKV_MAX_HEAD_GROUP 16 /* q heads per kv head */
+#define BKV_MAX_KV_HEAD 16    /* kv heads of a pool */
 
 /* Pool geometry.  One pool = n_layers x (K pool, V pool), each laid out exactly as
  * the reference's k_pool / v_pool (qsa/mod.rs:20-35):
@@ -71,7 +72,7 @@ enum {
 typedef struct bkv_pool_desc {
     int32_t n_layers;
     int32_t n_pages;
-    int32_t n_kv_head;
+    int32_t n_kv_head;          /* 1 .. BKV_MAX_KV_HEAD */
     int32_t head_dim;           /* multiple of 32, <= 256; kernels are tuned for 256 */
     int32_t page_cells;         /* 16 */
     int32_t layout;             /* bkv_layout */
@@ -422,6 +423,19 @@ bkv_status bkv_seq_restore(bkv_pool *pool, int32_t seq, int32_t lp0, int32_t n,
 bkv_status bkv_gather(bkv_pool *pool, int32_t layer, int32_t seq, int64_t cell0, int64_t n,
                       float *k_out_dev, float *v_out_dev, void *stream);
 
+/* How a decode-attention batch would be cut into work-groups on a device of n_cu compute units:
+ * the planning step of bkv_decode_attn / bkv_decode_step / bkv_decode_attn_select alone, on the
+ * host, nothing launched (no pool or device needed).  pos[n] as for those calls; sel_groups > 0
+ * plans every entry for that many groups of four listed blocks (a selection list of
+ * 4 * sel_groups ids) instead of its pages; matrix_cores != 0 plans for the matrix-core
+ * kernels, 0 for the VALU formulation.  splits_out[n], pps_out[n]: page ranges per entry and
+ * pages per range; *total_out: work-groups of the launch.  BKV_ERR_INVALID when the batch needs
+ * more work-groups than the partial-result workspace holds -- the error the attention calls
+ * themselves return, before anything is enqueued (qsa/mod.rs:1108-1116). */
+bkv_status bkv_attn_plan(int32_t n_cu, int32_t n_kv_head, int32_t n_q_head, int32_t n, const int64_t *pos,
+                         int32_t sel_groups, int32_t matrix_cores, int32_t *splits_out, int32_t *pps_out,
+                         int32_t *total_out);
+
 /* ---- per-kernel GPU timing ------------------------------------------------------
  * The analogue of Qsa::stage_timings / Pipe::run_timed (qsa/mod.rs:1733-1970,
  * ops/mod.rs:251-274): while enabled, every hot-path call times each of its kernels
@@ -435,7 +449,13 @@ typedef enum bkv_stage {
     BKV_STAGE_ATTN_SPLIT = 1, /* split-K online-softmax kernel (the dominant one) */
     BKV_STAGE_ATTN_MERGE = 2,
     BKV_STAGE_PAGE_COPY = 3,
-    BKV_STAGE_COUNT = 4
+    BKV_STAGE_PREFILL_ATTN = 4, /* chunk attention (bkv_prefill_attn) */
+    BKV_STAGE_APPEND_KPREP = 5, /* norm + rotary + append in one kernel */
+    BKV_STAGE_IDX_POOL = 6,     /* pooled indexer keys + rolling tail */
+    BKV_STAGE_IDX_SCORE = 7,
+    BKV_STAGE_TOPK = 8,
+    BKV_STAGE_PAGE_STAGE = 9,   /* gather / scatter of whole pages for swap and the prefix tiers */
+    BKV_STAGE_COUNT = 10
 } bkv_stage;
 bkv_status bkv_timing_enable(bkv_pool *pool, int on);
 bkv_status bkv_timing_reset(bkv_pool *pool);
@@ -461,6 +481,13 @@ bkv_status bkv_device_info(char *name_out, int32_t name_cap, int32_t *cu_out,
 /* Reference bandwidth probe: a plain 16-byte-vector device copy of `bytes` bytes
  * (used to scale profiler byte counters and to report the copy ceiling). */
 bkv_status bkv_copy_probe(void *dst_dev, const void *src_dev, uint64_t bytes, void *stream);
+/* Read-only bandwidth probe: reads `bytes` (a power-of-two number of 8 KiB chunks -- the size of
+ * one (page, kv head) run of an f16 pool) once, 8 KiB per wave at a time, in address order or
+ * (scattered != 0) in a fixed pseudo-random order of chunks, as the attention kernels see a
+ * shuffled pool; nothing is written except, never in practice, one word at sink_dev.  The rate
+ * it reaches is the ceiling a read-only kernel can be held against on a given box. */
+bkv_status bkv_read_probe(const void *src_dev, uint64_t bytes, int32_t scattered, void *sink_dev,
+                          void *stream);
 
 #ifdef __cplusplus
 }

@@ -21,6 +21,7 @@ def test_reference_layout_recipe_on_the_gpu():
     r = GOLD["layout_recipe"]
     with Twin(n_pages=3, max_seqs=2) as tw:
         s = tw.pool.seq_create_identity(3)
+        tw.pool.seq_reserve(s, 48)      # capacity 40 rounded up to whole pages
         i = np.arange(512)
         for t in range(r["n_tokens"]):
             cell = r["start_cell"] + t

@@ -298,3 +298,90 @@ def test_one_sequence_of_400k_tokens():
             assert max_abs(alone[0], together[i]) < 1e-6, i
     finally:
         pool.destroy()
+
+
+def test_config2_single_stream_ctx4096_on_a_64k_page_pool_12_layers():
+    """BASELINE configs[1]: one sequence of 4096 tokens on pages drawn by a seeded shuffle from a
+    65 536-page pool (1 GiB K + 1 GiB V per layer), 12 layers with independent seeded K/V/q; the step
+    of every layer is append-then-attend at position 4096 (the reference's per-layer loop,
+    crates/breccia-engine/src/graph.rs:5899-5966 -> crates/breccia-kernels/src/qsa/mod.rs:1617-1641).
+    The step runs in both forms -- one bkv_decode_step on the sequence, bkv_append + bkv_decode_attn on
+    a fork that shares its 256 full pages -- and per layer the rows the sequence holds are compared bit
+    for bit with the oracle's image (through bkv_gather, and the new row's raw pool bytes at the page
+    the shuffle gave it), the outputs with the oracle at the reference's 1e-5 bar and with each other
+    bit for bit."""
+    n_layers, n_pages, ctx = 12, 65536, 4096
+    rng = np.random.Generator(np.random.PCG64(20250002))
+    pool = Pool(n_layers=n_layers, n_pages=n_pages, n_kv_head=N_KV, head_dim=HD, max_seqs=4,
+                max_pages_per_seq=ctx // 16 + 2)
+    bufs = []
+    try:
+        pool.set_free_order(rng.permutation(n_pages).astype(np.int32))
+        seq = pool.seq_create()
+        pool.seq_reserve(seq, ctx)
+        g = oracle.Geom(N_KV, HD, 16)
+        compact = np.arange(ctx // 16 + 1, dtype=np.int32)      # the oracle keeps the pages side by side
+        images = []
+        for layer in range(n_layers):
+            k = rng.standard_normal((ctx, N_KV, HD), dtype=np.float32)
+            v = rng.standard_normal((ctx, N_KV, HD), dtype=np.float32)
+            kd, vd = DeviceBuffer.from_numpy(k), DeviceBuffer.from_numpy(v)
+            pool.append(layer, [seq], [0], [ctx], kd, vd)
+            device_sync()
+            kd.free()
+            vd.free()
+            img = oracle.PoolImage(g, compact.size)
+            assert img.append(compact, 0, k, v) == 0
+            images.append(img)
+        twin = pool.seq_fork(seq, ctx)                          # 256 full pages shared: no copy to make
+        assert pool.seq_reserve(seq, ctx + 1) == [] and pool.seq_reserve(twin, ctx + 1) == []
+        tab, tab2 = pool.block_table(seq), pool.block_table(twin)
+        assert np.array_equal(tab[:256], tab2[:256]) and tab[256] != tab2[256]
+        assert len(set(tab.tolist())) == 257 and tab.max() > n_pages // 2      # scattered over the pool
+        worst = 0.0
+        for layer in range(n_layers):
+            k1 = rng.standard_normal((1, N_KV, HD), dtype=np.float32)
+            v1 = rng.standard_normal((1, N_KV, HD), dtype=np.float32)
+            q = rng.standard_normal((1, N_Q, HD), dtype=np.float32)
+            kd, vd, qd = DeviceBuffer.from_numpy(k1), DeviceBuffer.from_numpy(v1), DeviceBuffer.from_numpy(q)
+            o1, o2 = DeviceBuffer(q.nbytes), DeviceBuffer(q.nbytes)
+            bufs = [kd, vd, qd, o1, o2]
+            pool.decode_step(layer, [seq], [ctx], kd, vd, N_Q, qd, o1, 1.0 / 16.0)
+            pool.append(layer, [twin], [ctx], [1], kd, vd)
+            pool.decode_attn(layer, [twin], [ctx], N_Q, qd, o2, 1.0 / 16.0)
+            device_sync()
+            fused = o1.download(np.float32).reshape(N_Q, HD)
+            twocall = o2.download(np.float32).reshape(N_Q, HD)
+            img = images[layer]
+            assert img.append(compact, ctx, k1, v1) == 0
+            wk, wv = img.gather(compact, 0, ctx + 1)
+            for s, t in ((seq, tab), (twin, tab2)):
+                gk, gv = pool.gather(layer, s, 0, ctx + 1)
+                assert np.array_equal(gk.view(np.uint32), wk.view(np.uint32)), (layer, s)
+                assert np.array_equal(gv.view(np.uint32), wv.view(np.uint32)), (layer, s)
+                # the new row's bytes where the block table says they are: page t[256], cell 0, both kv heads
+                for which, image in ((0, img.k), (1, img.v)):
+                    base, _ = pool.layer_ptr(layer, which)
+                    for kvh in range(N_KV):
+                        row = np.empty(HD * 2, dtype=np.uint8)
+                        off = ((int(t[256]) * N_KV + kvh) * 16) * HD * 2
+                        from breccia_amd.kv import check, lib
+                        import ctypes as C
+                        check(lib.bkv_memcpy_d2h(row.ctypes.data, C.c_void_p(base.value + off), row.nbytes, None))
+                        check(lib.bkv_stream_sync(None))
+                        woff = ((256 * N_KV + kvh) * 16) * HD * 2
+                        assert np.array_equal(row, image[woff:woff + HD * 2]), (layer, s, which, kvh)
+            want = oracle.attend(q[0], wk, wv, oracle.dense_cells(ctx), ctx, N_Q, N_KV, HD, threads=8)
+            _, rel = check_attn(fused, want, "configs[1] layer %d fused step" % layer)
+            _, rel2 = check_attn(twocall, want, "configs[1] layer %d two calls" % layer)
+            worst = max(worst, rel, rel2)
+            assert np.array_equal(fused.view(np.uint32), twocall.view(np.uint32)), layer
+            for b in bufs:
+                b.free()
+            bufs = []
+        assert worst <= REF_BAR_MAX_REL, worst
+        pool.check()
+    finally:
+        for b in bufs:
+            b.free()
+        pool.destroy()

@@ -269,3 +269,95 @@ def test_rope_table_is_the_reference_formula():
         with pytest.raises(BkvError) as ei:
             rope_table(*bad)
         assert ei.value.status == L.ERR_INVALID
+
+
+def test_attention_planning_terminates_and_fits_for_every_batch_shape():
+    """The cut of a batch into work-groups must come back for every shape the calls accept (a batch
+    whose one-range-per-entry cut already exceeds what is resident at once used to spin on the
+    host), cover every page, and fit the partial-result workspace -- or be refused as a size
+    error before anything is enqueued (crates/breccia-kernels/src/qsa/mod.rs:1108-1116)."""
+    rng = np.random.Generator(np.random.PCG64(77))
+    checked = refused = 0
+    for mc in (True, False):
+        for n_cu in (256, 64, 8):
+            for n_kv in range(1, L.MAX_KV_HEAD + 1):
+                for group in range(1, 17):
+                    hg = group if mc else (8 if group % 8 == 0 else 4)
+                    n_hc = (group + hg - 1) // hg
+                    cap = 4096 * 8 // hg if hg > 8 else 4096
+                    for n in (1, 2, 7, 33, 64):
+                        for sel_groups in (0, 129):
+                            pos = rng.integers(0, 40000, size=n)
+                            if n >= 33:
+                                pos[: n // 2] = rng.integers(0, 64, size=n // 2)   # many one-page entries
+                            if n * n_kv * n_hc > cap:
+                                expect(L.ERR_INVALID, kv.attn_plan, n_cu, n_kv, n_kv * group, pos, sel_groups, mc)
+                                refused += 1
+                                continue
+                            splits, pps, total = kv.attn_plan(n_cu, n_kv, n_kv * group, pos, sel_groups, mc)
+                            pages = np.full(n, sel_groups) if sel_groups else pos // 16 + 1
+                            assert total == int(splits.sum()) * n_kv * n_hc <= cap
+                            assert np.all(pps % 4 == 0) and np.all(splits >= 1)
+                            assert np.all(splits * pps >= pages) and np.all((splits - 1) * pps < pages)
+                            resident = n_cu * (2 if (mc or hg == 8) else 3)
+                            # one generation whenever one is possible at all
+                            assert total <= max(resident, n * n_kv * n_hc)
+                            checked += 1
+    # with at most 64 entries, 16 kv heads and 4 head chunks the workspace (4096 work-groups) always suffices
+    assert checked > 5000 and refused == 0
+
+
+def test_attention_batches_larger_than_one_generation_are_planned_not_spun_on():
+    with host_pool(n_pages=64, n_kv_head=16, max_seqs=64, max_pages_per_seq=2) as p:
+        seqs = [p.seq_create() for _ in range(64)]
+        for s in seqs:
+            p.seq_reserve(s, 4)
+        z = C.c_void_p(0)
+        # 64 entries x 16 kv heads x 4 head chunks of the VALU formulation's 13-head groups = 4096: accepted
+        # as a plan (and then refused for lack of a device); one more kv head cannot exist
+        expect(L.ERR_NO_DEVICE, p.decode_attn, 0, seqs, [3] * 64, 16 * 13, z, z, 0.0625)
+    expect(L.ERR_INVALID, host_pool, n_kv_head=L.MAX_KV_HEAD + 1)
+    expect(L.ERR_INVALID, kv.attn_plan, 256, L.MAX_KV_HEAD + 1, 17, [5], 0, True)
+    # the largest accepted shapes are planned as one range per entry, in more than one generation
+    splits, pps, total = kv.attn_plan(256, 16, 16 * 16, [5] * 64, 0, True)
+    assert total == 1024 and np.all(splits == 1)
+    splits, pps, total = kv.attn_plan(256, 9, 9, [70000] * 64, 0, True)      # 576 > 512 resident: used to spin
+    assert total == 576 and np.all(splits == 1) and np.all(pps >= 70000 // 16 + 1)
+
+
+def test_writes_need_reserved_cells_on_pages_the_sequence_holds_alone():
+    """bkv_append / bkv_append_kprep / bkv_decode_step write only cells that bkv_seq_reserve has
+    made the sequence's own: past the reserved length is a range error, a page another holder
+    still shares is a state error (the copy-on-write pair was never asked for), and nothing
+    changes -- tables, lengths and refcounts stay as they were."""
+    with host_pool(n_pages=32, max_seqs=4, max_pages_per_seq=8) as p:
+        z = C.c_void_p(0)
+        parent = p.seq_create()
+        p.seq_reserve(parent, 40)                      # pages 0, 1 full, page 2 half full
+        child = p.seq_fork(parent, 40)
+        before = (p.block_table(parent).tolist(), p.block_table(child).tolist(), p.free_pages())
+        shared = int(p.block_table(child)[2])
+        assert p.page_refcount(shared) == 2
+        # the child appends at its length without a reserve: capacity (48) would allow it
+        msg = expect(L.ERR_RANGE, p.append, 0, [child], [40], [1], z, z)
+        assert "reserve" in msg
+        expect(L.ERR_RANGE, p.decode_step, 0, [child], [40], z, z, 16, z, z, 0.0625)
+        # rewriting cells it does hold, on a page the parent still shares
+        msg = expect(L.ERR_STATE, p.append, 0, [child], [33], [2], z, z)
+        assert "holders" in msg
+        expect(L.ERR_STATE, p.append, 0, [parent], [0], [40], z, z)
+        expect(L.ERR_STATE, p.decode_step, 0, [parent], [39], z, z, 16, z, z, 0.0625)
+        assert (p.block_table(parent).tolist(), p.block_table(child).tolist(), p.free_pages()) == before
+        assert p.seq_len(child) == 40 and p.seq_len(parent) == 40 and p.page_refcount(shared) == 2
+        p.check()
+        # with the reserve the child gets its own copy of the half page; both may then write
+        pairs = p.seq_reserve(child, 41)
+        assert pairs == [(shared, int(p.block_table(child)[2]))] and p.page_refcount(shared) == 1
+        expect(L.ERR_NO_DEVICE, p.append, 0, [child], [40], [1], z, z)       # passes every host check
+        p.seq_reserve(parent, 41)                                            # sole holder again: in place
+        expect(L.ERR_NO_DEVICE, p.append, 0, [parent], [40], [1], z, z)
+        expect(L.ERR_NO_DEVICE, p.decode_step, 0, [parent], [40], z, z, 16, z, z, 0.0625)
+        # a page a cached prefix lists is shared too
+        p.prefix_insert(parent, np.arange(32))
+        expect(L.ERR_STATE, p.append, 0, [parent], [16], [4], z, z)
+        p.check()
