@@ -343,3 +343,27 @@ def test_other_head_counts(layout, n_kv, n_q):
             for i in range(2):
                 _, rel = check_attn(os_[i], tw.oracle_attend(0, seqs[i], lens[i], q[i], n_q), "step %d" % i)
                 assert rel <= REF_BAR_MAX_REL, rel
+
+
+@pytest.mark.parametrize("layout", [L.LAYOUT_F16, L.LAYOUT_Q8V, L.LAYOUT_I8H])
+def test_batches_that_need_more_than_one_generation_of_work_groups(layout):
+    # 64 entries x 9 kv heads = 576 units even with one range per entry: more than the 512 work-groups
+    # that are resident at once.  Planned as one range per entry (the host used to spin on this shape),
+    # run in two generations, and still the oracle's answer.
+    n_kv, n_q = 9, 18
+    rng = np.random.Generator(np.random.PCG64(9100 + layout))
+    with Twin(n_pages=64 * 6, n_kv=n_kv, layout=layout, max_seqs=64, max_pages_per_seq=8) as tw:
+        tw.pool.set_free_order(rng.permutation(64 * 6).astype(np.int32))
+        lens = [int(x) for x in rng.integers(1, 90, size=64)]
+        seqs = [tw.pool.seq_create() for _ in lens]
+        for s, n in zip(seqs, lens):
+            tw.pool.seq_reserve(s, n)
+        ks = [rng.standard_normal((n, n_kv, 256)).astype(np.float32) for n in lens]
+        vs = [rng.standard_normal((n, n_kv, 256)).astype(np.float32) for n in lens]
+        tw.append(0, seqs, [0] * 64, ks, vs)
+        q = rng.standard_normal((64, n_q, 256)).astype(np.float32)
+        pos = [n - 1 for n in lens]
+        out = tw.decode_attn(0, seqs, pos, q, n_q)
+        for i in range(64):
+            _, rel = check_attn(out[i], tw.oracle_attend(0, seqs[i], pos[i], q[i], n_q), "entry %d" % i)
+            assert rel <= REF_BAR_MAX_REL, (i, rel)
