@@ -362,6 +362,12 @@ bkv_status bkv_pool_create(const bkv_pool_desc* d, bkv_pool** out) {
     }
     BKV_TRY(hipStreamCreateWithFlags(&p->side, hipStreamNonBlocking));
     BKV_TRY(hipEventCreateWithFlags(&p->side_done, hipEventDisableTiming));
+    // created here rather than on first use: the calls that order work with them create nothing
+    BKV_TRY(hipEventCreateWithFlags(&p->attn_ws.ev, hipEventDisableTiming));
+    BKV_TRY(hipEventCreateWithFlags(&p->sel_ws.ev, hipEventDisableTiming));
+    BKV_TRY(hipEventCreateWithFlags(&p->table_sync.ev, hipEventDisableTiming));
+    // this device's copy of the static scratch of bkv_decode_attn_static
+    BKV_TRY(attn_static_scratch_init(p->device));
     BKV_TRY(hipDeviceSynchronize());
 #undef BKV_TRY
     *out = p;
@@ -813,7 +819,7 @@ static bkv_status decode_attn_common(bkv_pool* p, int32_t layer, int32_t n, cons
                                      int64_t id_stride, const uint32_t* counts_dev, int32_t max_ids,
                                      bool select, float* out_dev, void* stream,
                                      const float* new_k_dev = nullptr, const float* new_v_dev = nullptr,
-                                     bool step = false) {
+                                     bool step = false, bool static_ws = false) {
     if (!p) return fail(BKV_ERR_INVALID, "decode_attn: NULL pool");
     if (layer < 0 || layer >= p->g.n_layers)
         return fail(BKV_ERR_RANGE, sfmt("decode_attn: layer %lld is outside 0..%lld", layer,
@@ -884,14 +890,23 @@ static bkv_status decode_attn_common(bkv_pool* p, int32_t layer, int32_t n, cons
                                      "BKV_POOL_ATTN_VALU); append and attend in two calls instead");
     // the cut into work-groups comes before anything is enqueued: a batch it cannot serve is an
     // error like any other size violation
-    if (plan_attn(p, n_q_head, b, select ? (max_ids + 3) / 4 : 0, mfma) < 0)
+    const int32_t ws_wgs = static_ws ? kStaticWgs : p->max_wgs;
+    if (plan_attn(p, n_q_head, b, select ? (max_ids + 3) / 4 : 0, mfma, ws_wgs) < 0)
         return fail(BKV_ERR_INVALID,
-                    sfmt("decode_attn: %lld entries x %lld kv heads need more work-groups than the "
-                         "partial-result workspace holds (%lld); use smaller batches", n, p->g.n_kv,
-                         attn_plan_limits(p->n_cu, p->max_wgs, p->g.n_kv, n_q_head / p->g.n_kv, mfma).max_wgs));
+                    sfmt(static_ws ? "decode_attn_static: %lld entries x %lld kv heads need more work-groups than "
+                                     "the static scratch holds (%lld); use smaller batches or bkv_decode_attn"
+                                   : "decode_attn: %lld entries x %lld kv heads need more work-groups than the "
+                                     "partial-result workspace holds (%lld); use smaller batches",
+                         n, p->g.n_kv,
+                         attn_plan_limits(p->n_cu, ws_wgs, p->g.n_kv, n_q_head / p->g.n_kv, mfma).max_wgs));
+    AttnArgs a;
+    if (static_ws) {
+        if (!attn_static_scratch(p->device, &a.ws_o, &a.ws_ml))
+            return fail(BKV_ERR_STATE, "decode_attn_static: the static scratch of this device was not set up");
+        a.timed = false;
+    }
     st = flush_tables(p, S(stream));
     if (st != BKV_OK) return st;
-    AttnArgs a;
     a.mfma = mfma;
     a.n_q_head = n_q_head;
     a.q = q_dev;
@@ -910,8 +925,12 @@ static bkv_status decode_attn_common(bkv_pool* p, int32_t layer, int32_t n, cons
         a.new_k = new_k_dev;
         a.new_v = new_v_dev;
     }
-    st = order_workspace(p->attn_ws, S(stream));
-    if (st != BKV_OK) return st;
+    // the pool's own workspace is ordered across streams; the static scratch is the device's, shared by
+    // every pool, and overlapping calls on it are the caller's to avoid
+    if (!static_ws) {
+        st = order_workspace(p->attn_ws, S(stream));
+        if (st != BKV_OK) return st;
+    }
     BKV_HIP(launch_decode_attn(p, layer, b, a, S(stream)));
     if (p->timer.open.size() > 8192) return timer_collect(p);
     return BKV_OK;
@@ -954,6 +973,15 @@ bkv_status bkv_decode_attn(bkv_pool* p, int32_t layer, int32_t n, const int32_t*
                            int64_t gate_head_stride, float scale, float* out_dev, void* stream) {
     return decode_attn_common(p, layer, n, seqs, pos, n_q_head, q_dev, gate_dev, gate_seq_stride,
                               gate_head_stride, scale, nullptr, 0, nullptr, 0, false, out_dev, stream);
+}
+
+bkv_status bkv_decode_attn_static(bkv_pool* p, int32_t layer, int32_t n, const int32_t* seqs,
+                                  const int64_t* pos, int32_t n_q_head, const float* q_dev,
+                                  const float* gate_dev, int64_t gate_seq_stride,
+                                  int64_t gate_head_stride, float scale, float* out_dev, void* stream) {
+    return decode_attn_common(p, layer, n, seqs, pos, n_q_head, q_dev, gate_dev, gate_seq_stride,
+                              gate_head_stride, scale, nullptr, 0, nullptr, 0, false, out_dev, stream,
+                              nullptr, nullptr, false, true);
 }
 
 bkv_status bkv_decode_step(bkv_pool* p, int32_t layer, int32_t n, const int32_t* seqs, const int64_t* pos,

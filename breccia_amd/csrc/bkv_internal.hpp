@@ -29,6 +29,8 @@ bkv_status hip_fail(hipError_t e, const char* what);
 
 // work-groups the split-K partial-result workspace is sized for (x 8 head rows of 256 floats)
 constexpr int32_t kMaxWgs = 4096;
+// work-groups (x 8 head rows) the static device scratch of bkv_decode_attn_static is sized for
+constexpr int32_t kStaticWgs = 1024;
 
 // ---- geometry ----------------------------------------------------------------
 struct Geom {
@@ -213,13 +215,21 @@ struct AttnArgs {
     const float* new_k = nullptr;
     const float* new_v = nullptr;
     bool mfma = false;  // dense f16 call routed to the MFMA kernel (all heads of a group at once)
+    // partial-result workspace other than the pool's own (the static device scratch); nullptr = the pool's
+    float* ws_o = nullptr;
+    float* ws_ml = nullptr;
+    bool timed = true;  // kernels carry stage-timer events while the pool's timer is on
 };
 // Fills wg_base/splits/pps from row/pos (attn_plan.hpp); returns the total work-group count, -1
 // when the batch cannot be cut into as few work-groups as the workspace holds.  sel_groups > 0:
 // every entry is planned for that many groups of four selected blocks instead of its pages.
 AttnPlanLimits attn_plan_limits(int32_t n_cu, int32_t max_wgs, int32_t n_kv, int32_t group, bool mfma);
 int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b, int32_t sel_groups = 0,
-                  bool mfma = false);
+                  bool mfma = false, int32_t max_wgs = 0);
+// The static device scratch of bkv_decode_attn_static: looked up once per device (which must be
+// the current one) at pool creation; false from the accessor when that has not happened.
+hipError_t attn_static_scratch_init(int device);
+bool attn_static_scratch(int device, float** o, float** ml);
 bool attn_on_mfma(const bkv_pool* p, int32_t group, bool dense);
 hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, const AttnArgs& a,
                               hipStream_t stream);

@@ -746,9 +746,47 @@ AttnPlanLimits attn_plan_limits(int32_t n_cu, int32_t max_wgs, int32_t n_kv, int
     return lim;
 }
 
-int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b, int32_t sel_groups, bool mfma) {
-    const AttnPlanLimits lim = attn_plan_limits(p->n_cu, p->max_wgs, p->g.n_kv, n_q_head / p->g.n_kv, mfma);
+int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b, int32_t sel_groups, bool mfma,
+                  int32_t max_wgs) {
+    const AttnPlanLimits lim =
+        attn_plan_limits(p->n_cu, max_wgs > 0 ? max_wgs : p->max_wgs, p->g.n_kv, n_q_head / p->g.n_kv, mfma);
     return plan_attn_ranges(lim, kPage, sel_groups, b);
+}
+
+// ---- partial results without an allocation -----------------------------------------------------
+// For callers that may not allocate device memory (a stream under capture, a tight serving loop):
+// the split-K partials of bkv_decode_attn_static live in this array, one copy per GPU, held from
+// the moment the library is loaded until the process ends.  Host code never uses the array's name
+// as an address: each device's copy has its own address, looked up once per device below.
+struct AttnStaticScratch {
+    float o[(size_t)kStaticWgs * 8 * kHd];
+    float ml[(size_t)kStaticWgs * 8 * 2];
+};
+static __device__ __align__(256) unsigned char scratch[sizeof(AttnStaticScratch)];
+
+constexpr int kMaxDevices = 64;
+static void* g_scratch_ptr[kMaxDevices] = {};
+
+hipError_t attn_static_scratch_init(int device) {
+    if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+    if (g_scratch_ptr[device]) return hipSuccess;
+    int current = -1;
+    hipError_t e = hipGetDevice(&current);
+    if (e != hipSuccess) return e;
+    if (current != device) return hipErrorInvalidDevice;
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    g_scratch_ptr[device] = ptr;
+    return hipSuccess;
+}
+
+bool attn_static_scratch(int device, float** o, float** ml) {
+    if (device < 0 || device >= kMaxDevices || !g_scratch_ptr[device]) return false;
+    AttnStaticScratch* s = static_cast<AttnStaticScratch*>(g_scratch_ptr[device]);
+    *o = s->o;
+    *ml = s->ml;
+    return true;
 }
 
 hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, const AttnArgs& a,
@@ -762,8 +800,8 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
     kp.vpool = p->v_layer[(size_t)layer];
     kp.tables = p->table_dev;
     kp.q = a.q;
-    kp.part_o = p->part_o;
-    kp.part_ml = p->part_ml;
+    kp.part_o = a.ws_o ? a.ws_o : p->part_o;
+    kp.part_ml = a.ws_ml ? a.ws_ml : p->part_ml;
     kp.max_pages_per_seq = p->desc.max_pages_per_seq;
     kp.n_kv = n_kv;
     kp.n_q = a.n_q_head;
@@ -787,13 +825,16 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
         // one work-group per unit, every head of the kv head in it (checked by the caller); while the
         // pool times its kernels, the events ride on the dispatch
         hipEvent_t ev_start = nullptr, ev_stop = nullptr;
-        (void)timer_dispatch_events(p, BKV_STAGE_ATTN_SPLIT, &ev_start, &ev_stop);
+        if (a.timed) (void)timer_dispatch_events(p, BKV_STAGE_ATTN_SPLIT, &ev_start, &ev_stop);
         const hipError_t e = launch_decode_attn_mfma(kp, p->g.layout, step, sel, total, stream, ev_start, ev_stop);
         if (e != hipSuccess) return e;
     } else {
         const int layout = p->g.layout;
         const auto go = [&](auto kernel) {
-            launch_staged(p, BKV_STAGE_ATTN_SPLIT, kernel, dim3((unsigned)grid), dim3(kBlock), 0, stream, kp);
+            if (a.timed)
+                launch_staged(p, BKV_STAGE_ATTN_SPLIT, kernel, dim3((unsigned)grid), dim3(kBlock), 0, stream, kp);
+            else
+                hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kBlock), 0, stream, kp);
         };
 #define BKV_LAUNCH(HGV, KE, VE)                              \
     do {                                                    \
@@ -821,8 +862,8 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
     if (err != hipSuccess) return err;
     MergeParams mp;
     mp.b = b;
-    mp.part_o = p->part_o;
-    mp.part_ml = p->part_ml;
+    mp.part_o = kp.part_o;
+    mp.part_ml = kp.part_ml;
     mp.gate = a.gate;
     mp.out = a.out;
     mp.gate_seq_stride = a.gate_seq_stride;
@@ -831,8 +872,12 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
     mp.n_q = a.n_q_head;
     mp.group = group;
     mp.hg = hg;
-    launch_staged(p, BKV_STAGE_ATTN_MERGE, decode_attn_merge_kernel, dim3((unsigned)(b.n * a.n_q_head)),
-                  dim3(64 * kMergeGroups), 0, stream, mp);
+    if (a.timed)
+        launch_staged(p, BKV_STAGE_ATTN_MERGE, decode_attn_merge_kernel, dim3((unsigned)(b.n * a.n_q_head)),
+                      dim3(64 * kMergeGroups), 0, stream, mp);
+    else
+        hipLaunchKernelGGL(decode_attn_merge_kernel, dim3((unsigned)(b.n * a.n_q_head)), dim3(64 * kMergeGroups),
+                           0, stream, mp);
     return hipGetLastError();
 }
 

@@ -370,6 +370,16 @@ class Pool:
                                   _ptr(gate_dev), gate_seq_stride, gate_head_stride, scale,
                                   _ptr(out_dev), _sh(stream)))
 
+    def decode_attn_static(self, layer: int, seqs, pos, n_q_head: int, q_dev, out_dev, scale: float,
+                           gate_dev=None, gate_seq_stride: int = 0, gate_head_stride: int = 0,
+                           stream=None) -> None:
+        seqs, ps = _i32(seqs)
+        pos, pp = _i64(pos)
+        assert seqs.size == pos.size
+        check(lib.bkv_decode_attn_static(self.handle, layer, seqs.size, ps, pp, n_q_head, _ptr(q_dev),
+                                         _ptr(gate_dev), gate_seq_stride, gate_head_stride, scale,
+                                         _ptr(out_dev), _sh(stream)))
+
     def prefill_attn(self, layer: int, seqs, pos0, n_tokens, n_q_head: int, q_dev, out_dev, scale: float,
                      gate_dev=None, gate_tok_stride: int = 0, gate_head_stride: int = 0, stream=None) -> None:
         """Causal attention of whole chunks (token t of chunk i sees cells 0..pos0[i]+t), on MFMA."""

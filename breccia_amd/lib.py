@@ -19,6 +19,7 @@ POOL_HOST_ONLY = 1
 POOL_ATTN_VALU = 2
 MAX_BATCH = 64
 MAX_KV_HEAD = 16
+STATIC_WGS = 1024
 (STAGE_APPEND, STAGE_ATTN_SPLIT, STAGE_ATTN_MERGE, STAGE_PAGE_COPY, STAGE_PREFILL_ATTN, STAGE_APPEND_KPREP,
  STAGE_IDX_POOL, STAGE_IDX_SCORE, STAGE_TOPK, STAGE_PAGE_STAGE) = range(10)
 
@@ -98,6 +99,8 @@ _SIGNATURES = {
     "bkv_rope_table": (C.c_int, [C.c_double, _i32, _i32, _vp]),
     "bkv_decode_attn": (C.c_int, [_vp, _i32, _i32, _pi32, _pi64, _i32, _vp, _vp, _i64, _i64, _f32,
                                   _vp, _vp]),
+    "bkv_decode_attn_static": (C.c_int, [_vp, _i32, _i32, _pi32, _pi64, _i32, _vp, _vp, _i64, _i64, _f32,
+                                         _vp, _vp]),
     "bkv_attn_plan": (C.c_int, [_i32, _i32, _i32, _i32, _pi64, _i32, _i32, _pi32, _pi32, _pi32]),
     "bkv_prefill_attn": (C.c_int, [_vp, _i32, _i32, _pi32, _pi64, _pi32, _i32, _vp, _vp, _i64, _i64, _f32,
                                    _vp, _vp]),

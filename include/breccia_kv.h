@@ -287,6 +287,25 @@ bkv_status bkv_decode_attn(bkv_pool *pool, int32_t layer, int32_t n, const int32
                            const float *gate_dev, int64_t gate_seq_stride,
                            int64_t gate_head_stride, float scale, float *out_dev, void *stream);
 
+/* bkv_decode_attn for callers that cannot allocate device memory (a stream being captured into a
+ * graph, a tight serving loop, a harness that forbids hipMalloc).  No counterpart in the
+ * reference.  Same arguments, checks, kernels and results (bit for bit) as bkv_decode_attn, but the
+ * split-K partial results live in a static device array inside the library instead of a
+ * workspace the pool allocated, and the call itself allocates nothing on the device, creates no
+ * event and attaches no stage timer.  The array is sized for BKV_STATIC_WGS work-groups of 8 head
+ * rows (8.06 MiB, one copy per GPU, held from library load to process end): a batch whose cut
+ * needs more -- more than BKV_STATIC_WGS (entry, kv head) pairs at up to 8 q heads per kv head,
+ * half as many at 9 to 16 -- is rejected with BKV_ERR_INVALID before anything is enqueued.
+ * Every pool and every call on one GPU shares that GPU's array: calls that overlap on one GPU
+ * (different streams, different pools) race; calls on one stream are ordered by the stream.
+ * Nothing in the array has to start at zero.  Block-table changes still pending from allocator
+ * calls are uploaded first, as in every other call (host heap and the pinned argument ring only). */
+#define BKV_STATIC_WGS 1024
+bkv_status bkv_decode_attn_static(bkv_pool *pool, int32_t layer, int32_t n, const int32_t *seqs,
+                                  const int64_t *pos, int32_t n_q_head, const float *q_dev,
+                                  const float *gate_dev, int64_t gate_seq_stride,
+                                  int64_t gate_head_stride, float scale, float *out_dev, void *stream);
+
 /* Causal attention for chunks of many query tokens (prefill), on the matrix cores: the
  * reference's GQA pair for T >= 16 (shaders/qsa_attn_scores_gqa.comp, qsa_attn_apply_gqa.comp;
  * qsa/mod.rs:116-150), same contract as bkv_decode_attn (oracle qsa/cpu.rs:197-246, dense
