@@ -106,7 +106,13 @@ uint64_t bkv_page_bytes(const bkv_pool *pool, int which);   /* one layer; 0 = K,
  * knob fills with NaN words, qsa/mod.rs:509-523; 0xff bytes are NaN in f16 and f32). */
 bkv_status bkv_pool_fill(bkv_pool *pool, int byte, void *stream);
 /* Raw device base of one layer's K (which=0) or V (which=1) pool, for callers that
- * dump or diff pool bytes (the reference's BRECCIA_DUMP_*, graph.rs:2204-2229). */
+ * dump or diff pool bytes (the reference's BRECCIA_DUMP_*, graph.rs:2204-2229).
+ * Bytes written through this pointer (or swapped in from a foreign dump) bypass the append
+ * path's store rule.  One consequence is part of the contract: an f16 code with exponent field 0
+ * (a subnormal) is never stored by any append entry point; if foreign bytes hold one, bkv_gather
+ * and the int8 layout's scale load read it as zero (the reference's load rule,
+ * shaders/f16_storage.glsl:58-69) while the attention kernels multiply it as the IEEE value it
+ * encodes.  Pools written only through this library read the same everywhere. */
 bkv_status bkv_pool_layer_ptr(const bkv_pool *pool, int32_t layer, int which, void **dev_ptr,
                               uint64_t *bytes);
 

@@ -367,3 +367,41 @@ def test_batches_that_need_more_than_one_generation_of_work_groups(layout):
         for i in range(64):
             _, rel = check_attn(out[i], tw.oracle_attend(0, seqs[i], pos[i], q[i], n_q), "entry %d" % i)
             assert rel <= REF_BAR_MAX_REL, (i, rel)
+
+
+def test_foreign_f16_subnormals_attend_with_their_ieee_value_and_gather_as_zero():
+    """The append path never stores an f16 code with exponent field 0; bytes written behind its
+    back (bkv_pool_layer_ptr, a restored foreign dump) may hold them.  The documented split: the
+    attention kernels multiply such codes as the IEEE subnormals they are, bkv_gather reads them
+    as zero (the reference's load rule, crates/breccia-kernels/shaders/f16_storage.glsl:58-69)."""
+    rng = np.random.Generator(np.random.PCG64(6060))
+    n, n_q = 45, 16
+    with Twin(n_pages=8) as tw:
+        s = tw.pool.seq_create()
+        fill(tw, s, n, rng)
+        table = tw.pool.block_table(s)
+        kb = tw.pool.read_layer(0, 0).view(np.uint16).copy()
+        vb = tw.pool.read_layer(0, 1).view(np.uint16).copy()
+        codes = {}
+        for cell, kvh in ((5, 0), (17, 1), (44, 0)):
+            row = (int(table[cell // 16]) * 2 + kvh) * 16 + cell % 16
+            for name, buf in (("k", kb), ("v", vb)):
+                c = (rng.integers(1, 0x400, size=256) | (rng.integers(0, 2, size=256) << 15)).astype(np.uint16)
+                buf[row * 256:(row + 1) * 256] = c
+                codes[(name, cell, kvh)] = c
+        tw.pool.write_layer(0, 0, kb)
+        tw.pool.write_layer(0, 1, vb)
+        # what the kernels are documented to see: every code as its IEEE value
+        k_img, v_img = tw.images[0].gather(table, 0, n)
+        k_ieee, v_ieee = k_img.copy().reshape(n, 2, 256), v_img.copy().reshape(n, 2, 256)
+        for (name, cell, kvh), c in codes.items():
+            (k_ieee if name == "k" else v_ieee)[cell, kvh] = c.view(np.float16).astype(np.float32)
+        # large q so that the subnormal K rows move the logits by a visible amount
+        q = (rng.standard_normal((1, n_q, 256)) * 300.0).astype(np.float32)
+        got = tw.decode_attn(0, [s], [n - 1], q, n_q)[0]
+        want = oracle.attend(q[0], k_ieee, v_ieee, oracle.dense_cells(n - 1), n - 1, n_q, 2, 256)
+        _, rel = check_attn(got, want, "subnormal rows as IEEE values")
+        assert rel <= REF_BAR_MAX_REL, rel
+        gk, gv = tw.pool.gather(0, s, 0, n)
+        for (name, cell, kvh), _c in codes.items():
+            assert not np.any((gk if name == "k" else gv)[cell, kvh]), (name, cell, kvh)

@@ -29,6 +29,21 @@ def test_library_exports_every_declared_symbol():
     assert sorted(L._SIGNATURES) == names
 
 
+def test_rust_binding_text_lists_every_declaration_with_its_argument_count():
+    """The Rust `extern "C"` block a maintainer would add (source only, no Rust
+    toolchain here) names every function of the header with as many arguments as the header gives it."""
+    doc = open(os.path.join(os.path.dirname(__file__), "..", "INTEGRATION.md")).read()
+    rust = dict((m.group(1), m.group(2)) for m in re.finditer(r"pub fn (bkv_[a-z0-9_]+)\(([^;]*?)\)(?: -> [^;]+)?;", doc, re.S))
+    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    header = dict((m.group(1), m.group(2)) for m in re.finditer(r"\b(bkv_[a-z0-9_]+)\s*\(([^;{}]*?)\);", text, re.S))
+    assert sorted(header) == declared_functions()
+    assert sorted(rust) == sorted(header)
+    for name, args in header.items():
+        n_c = 0 if args.strip() in ("", "void") else args.count(",") + 1
+        n_rust = 0 if not rust[name].strip() else rust[name].count(":")
+        assert n_c == n_rust, (name, n_c, n_rust)
+
+
 def test_header_structs_match_the_binding():
     text = open(HEADER).read()
     body = re.search(r"typedef struct bkv_pool_desc \{(.*?)\} bkv_pool_desc;", text, re.S).group(1)
