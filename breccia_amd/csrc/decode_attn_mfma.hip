@@ -122,6 +122,22 @@ __device__ __forceinline__ void mfma_fold_and_store(const AttnKernelParams& P, M
     }
 }
 
+// K fragments as fetched (see k_addr in the kernel): of the pair (2 p, 2 p + 1), lane c < 8 holds its own
+// fragment 2 p and fragment 2 p of lane c + 8, lane c >= 8 holds fragment 2 p + 1 of lane c - 8 and its own
+// fragment 2 p + 1.  One masked DPP move per register (row_ror:8 is lane ^ 8 inside a row of 16; the bank
+// mask picks the half of the row that takes the neighbour's value) puts every fragment where its MFMA reads it.
+__device__ __forceinline__ void k_pair_home(const v4u& lo_rows, const v4u& hi_rows, half8& even, half8& odd) {
+    v4u e, o;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int a = (int)lo_rows[j], b = (int)hi_rows[j];
+        e[j] = (unsigned)__builtin_amdgcn_update_dpp(a, b, 0x128, 0xf, 0xc, false);
+        o[j] = (unsigned)__builtin_amdgcn_update_dpp(b, a, 0x128, 0xf, 0x3, false);
+    }
+    even = __builtin_bit_cast(half8, e);
+    odd = __builtin_bit_cast(half8, o);
+}
+
 // STEP: the row of cell pos comes from the caller's f32 K/V (stored under the f16 rule into the
 // pool on the way), as in decode_attn_kernel<..., STEP = true>.
 // SEL: the 16 rows of an iteration are four listed 4-cell blocks instead of a page, as in
@@ -187,15 +203,22 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
     const auto pick = [](const auto (&a)[SEL ? 4 : 1], int j) {
         if constexpr (SEL) return j == 0 ? a[0] : j == 1 ? a[1] : j == 2 ? a[2] : a[3]; else return a[0];
     };
-    // this lane's K row (row c of the iteration) and the first of its four V rows (row 4 g)
-    const auto k_row = [&](const RowRuns<SEL>& rr) {
-        return SEL ? pick(rr.k, c >> 2) + (size_t)(c & 3) * (kHd * 2) : rr.k[0] + (size_t)c * (kHd * 2);
+    // K rows are fetched in whole 128-byte cache lines: for the pair of fragments (2 p, 2 p + 1) -- bytes
+    // 128 p .. 128 p + 127 of a row -- one instruction reads rows 0..7 and one rows 8..15 of the iteration,
+    // eight lanes to a row (lane (c, g) takes segment g + 4 (c / 8) of row c % 8, or of row 8 + c % 8).
+    // Half of what a lane receives is its neighbour's eight columns away (c ^ 8); the two trade
+    // places before use (k_fragments_home).  Fetched four lanes to a row, fragment by fragment, every
+    // line was requested twice, half a line at a time, and the kernel streamed 4 to 7 % slower.
+    const int c7 = c & 7;
+    const auto k_row_of = [&](const RowRuns<SEL>& rr, int row) {
+        return SEL ? pick(rr.k, row >> 2) + (size_t)(row & 3) * (kHd * 2) : rr.k[0] + (size_t)row * (kHd * 2);
     };
+    const auto k_addr = [&](const uint8_t* row, int p) {
+        return reinterpret_cast<const v4u*>(row + (size_t)(128 * p + 16 * (g + 4 * (c >> 3))));
+    };
+    // the first of this lane's four V rows (row 4 g)
     const auto v_rows = [&](const RowRuns<SEL>& rr) {
         return SEL ? pick(rr.v, g) : rr.v[0] + (size_t)(4 * g) * (kHd * 2);
-    };
-    const auto k_addr = [&](const uint8_t* row, int m) {
-        return reinterpret_cast<const v4u*>(row + (size_t)(m * 32 + g * 8) * 2);
     };
     const auto v_addr = [&](const uint8_t* rows, int h, int r) {
         return reinterpret_cast<const v4u*>(rows + (size_t)r * (kHd * 2) + (size_t)(h * 128 + c * 8) * 2);
@@ -206,10 +229,14 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
     RowRuns<SEL> cur{};
     if (pg < pg1) {
         locate(pg, cur);
-        const uint8_t* kp = k_row(cur);
+        const uint8_t* kp_lo = k_row_of(cur, c7);
+        const uint8_t* kp_hi = k_row_of(cur, 8 + c7);
         const uint8_t* vp = v_rows(cur);
 #pragma unroll
-        for (int m = 0; m < 8; ++m) kf[m] = __builtin_nontemporal_load(k_addr(kp, m));
+        for (int p = 0; p < 4; ++p) {
+            kf[2 * p] = __builtin_nontemporal_load(k_addr(kp_lo, p));
+            kf[2 * p + 1] = __builtin_nontemporal_load(k_addr(kp_hi, p));
+        }
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
@@ -234,11 +261,13 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
         const int pg_next = pg + kWaves;
         const bool more = pg_next < pg1;
         RowRuns<SEL> nxt{};
-        const uint8_t* kp_next = nullptr;
+        const uint8_t* kp_lo_next = nullptr;
+        const uint8_t* kp_hi_next = nullptr;
         const uint8_t* vp_next = nullptr;
         if (more) {
             locate(pg_next, nxt);
-            kp_next = k_row(nxt);
+            kp_lo_next = k_row_of(nxt, c7);
+            kp_hi_next = k_row_of(nxt, 8 + c7);
             vp_next = v_rows(nxt);
         }
 
@@ -258,12 +287,15 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
                     w.z = f16_store_pair(b.x, b.y), w.w = f16_store_pair(b.z, b.w);
                     return w;
                 };
+                // K registers hold rows as fetched: row r sits in the lanes with c % 8 == r % 8, in the
+                // register of rows 0..7 or of rows 8..15, segment g + 4 (c / 8) of each 128-byte line
+                const int seg = g + 4 * (c >> 3);
 #pragma unroll
-                for (int m = 0; m < 8; ++m) {
-                    const v4u w = row_slice(nk + m * 32 + g * 8);
-                    if (c == r) {
-                        kf[m] = w;
-                        *reinterpret_cast<v4u*>(P.kpool_w + here + (size_t)(m * 32 + g * 8) * 2) = w;
+                for (int p = 0; p < 4; ++p) {
+                    const v4u w = row_slice(nk + p * 64 + seg * 8);
+                    if (c7 == (r & 7)) {
+                        if (r < 8) kf[2 * p] = w; else kf[2 * p + 1] = w;
+                        *reinterpret_cast<v4u*>(P.kpool_w + here + (size_t)(p * 64 + seg * 8) * 2) = w;
                     }
                 }
 #pragma unroll
@@ -283,15 +315,15 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
         f4 s0 = f4{0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0, s2 = s0, s3 = s0;
 #pragma unroll
         for (int m = 0; m < 8; m += 2) {
-            const half8 ka = __builtin_bit_cast(half8, kf[m]);
-            const half8 kb = __builtin_bit_cast(half8, kf[m + 1]);
+            half8 ka, kb;
+            k_pair_home(kf[m], kf[m + 1], ka, kb);
             s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qhi[m], s0, 0, 0, 0);
             s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qlo[m], s1, 0, 0, 0);
             s2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kb, qhi[m + 1], s2, 0, 0, 0);
             s3 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kb, qlo[m + 1], s3, 0, 0, 0);
             if (more) {
-                kf[m] = __builtin_nontemporal_load(k_addr(kp_next, m));
-                kf[m + 1] = __builtin_nontemporal_load(k_addr(kp_next, m + 1));
+                kf[m] = __builtin_nontemporal_load(k_addr(kp_lo_next, m >> 1));
+                kf[m + 1] = __builtin_nontemporal_load(k_addr(kp_hi_next, m >> 1));
             }
         }
         const f4 s = (s0 + s1) + (s2 + s3);  // s[r] = q[head c] . k[cell 4 g + r]

@@ -22,7 +22,7 @@ def attn_formulation(request):
     """Every case runs in both formulations of f16 decode attention (matrix cores / VALU)."""
     import gpu_common
     gpu_common.DEFAULT_ATTN_VALU = request.param == "valu"
-    yield
+    yield request.param
     gpu_common.DEFAULT_ATTN_VALU = False
 
 
@@ -373,7 +373,9 @@ def test_foreign_f16_subnormals_attend_with_their_ieee_value_and_gather_as_zero(
     """The append path never stores an f16 code with exponent field 0; bytes written behind its
     back (bkv_pool_layer_ptr, a restored foreign dump) may hold them.  The documented split: the
     attention kernels multiply such codes as the IEEE subnormals they are, bkv_gather reads them
-    as zero (the reference's load rule, crates/breccia-kernels/shaders/f16_storage.glsl:58-69)."""
+    as zero (the reference's load rule, crates/breccia-kernels/shaders/f16_storage.glsl:58-69).
+    kv head 0 gets subnormal V rows (outputs of the size of a subnormal, not zero), kv head 1
+    subnormal K rows under a large q (logits that move the weights by about a percent)."""
     rng = np.random.Generator(np.random.PCG64(6060))
     n, n_q = 45, 16
     with Twin(n_pages=8) as tw:
@@ -382,26 +384,63 @@ def test_foreign_f16_subnormals_attend_with_their_ieee_value_and_gather_as_zero(
         table = tw.pool.block_table(s)
         kb = tw.pool.read_layer(0, 0).view(np.uint16).copy()
         vb = tw.pool.read_layer(0, 1).view(np.uint16).copy()
-        codes = {}
-        for cell, kvh in ((5, 0), (17, 1), (44, 0)):
-            row = (int(table[cell // 16]) * 2 + kvh) * 16 + cell % 16
-            for name, buf in (("k", kb), ("v", vb)):
-                c = (rng.integers(1, 0x400, size=256) | (rng.integers(0, 2, size=256) << 15)).astype(np.uint16)
-                buf[row * 256:(row + 1) * 256] = c
-                codes[(name, cell, kvh)] = c
-        tw.pool.write_layer(0, 0, kb)
-        tw.pool.write_layer(0, 1, vb)
-        # what the kernels are documented to see: every code as its IEEE value
         k_img, v_img = tw.images[0].gather(table, 0, n)
         k_ieee, v_ieee = k_img.copy().reshape(n, 2, 256), v_img.copy().reshape(n, 2, 256)
-        for (name, cell, kvh), c in codes.items():
-            (k_ieee if name == "k" else v_ieee)[cell, kvh] = c.view(np.float16).astype(np.float32)
-        # large q so that the subnormal K rows move the logits by a visible amount
-        q = (rng.standard_normal((1, n_q, 256)) * 300.0).astype(np.float32)
+        for cell in range(n):
+            for buf, kvh, img in ((vb, 0, v_ieee), (kb, 1, k_ieee)):
+                row = (int(table[cell // 16]) * 2 + kvh) * 16 + cell % 16
+                c = (rng.integers(1, 0x400, size=256) | (rng.integers(0, 2, size=256) << 15)).astype(np.uint16)
+                buf[row * 256:(row + 1) * 256] = c
+                img[cell, kvh] = c.view(np.float16).astype(np.float32)
+        tw.pool.write_layer(0, 0, kb)
+        tw.pool.write_layer(0, 1, vb)
+        q = rng.standard_normal((1, n_q, 256)).astype(np.float32)
+        q[0, 8:] *= 300.0
         got = tw.decode_attn(0, [s], [n - 1], q, n_q)[0]
         want = oracle.attend(q[0], k_ieee, v_ieee, oracle.dense_cells(n - 1), n - 1, n_q, 2, 256)
-        _, rel = check_attn(got, want, "subnormal rows as IEEE values")
+        # heads of kv head 0: weighted means of subnormals
+        top = float(np.max(np.abs(want[:8])))
+        assert 1e-6 < top < 1e-4, top
+        assert max_abs(got[:8], want[:8]) <= 1e-3 * top
+        # heads of kv head 1: the reference bar, and visibly not the uniform weights of an all-zero K
+        _, rel = check_attn(got[8:], want[8:], "subnormal K rows as IEEE values")
         assert rel <= REF_BAR_MAX_REL, rel
+        uniform = v_ieee[:, 1, :].astype(np.float64).mean(axis=0)
+        assert max_abs(got[8:], np.broadcast_to(uniform, (8, 256))) > 1e-4
         gk, gv = tw.pool.gather(0, s, 0, n)
-        for (name, cell, kvh), _c in codes.items():
-            assert not np.any((gk if name == "k" else gv)[cell, kvh]), (name, cell, kvh)
+        assert not np.any(gv[:, 0]) and not np.any(gk[:, 1])
+        assert np.array_equal(gk[:, 0], k_img.reshape(n, 2, 256)[:, 0])
+
+
+@pytest.mark.parametrize("layout", [L.LAYOUT_F16, L.LAYOUT_Q8V, L.LAYOUT_I8H])
+def test_repeated_launches_of_one_batch_return_identical_bits(layout):
+    """The cut into page ranges and the order in which the partial results are combined are a
+    function of the batch alone: 100 launches of one batch (ranges of 1 to 40 pages per
+    work-group, 1 to 33 of them per head) return identical bits, and those are the oracle's answer."""
+    rng = np.random.Generator(np.random.PCG64(8800 + layout))
+    lens = [5000, 16, 2100, 333, 90, 1]
+    n_q = 16
+    with Twin(n_pages=520, layout=layout, max_seqs=8, max_pages_per_seq=320) as tw:
+        tw.pool.set_free_order(rng.permutation(520).astype(np.int32))
+        seqs = [tw.pool.seq_create() for _ in lens]
+        for s, n in zip(seqs, lens):
+            fill(tw, s, n, rng, chunk=1024)
+        pos = [n - 1 for n in lens]
+        q = rng.standard_normal((len(lens), n_q, 256)).astype(np.float32)
+        gate = rng.standard_normal((len(lens), n_q, 256)).astype(np.float32)
+        qd, gd = DeviceBuffer.from_numpy(q), DeviceBuffer.from_numpy(gate)
+        od = DeviceBuffer(q.nbytes)
+        first = None
+        for it in range(100):
+            tw.pool.decode_attn(0, seqs, pos, n_q, qd, od, 1.0 / 16.0, gate_dev=gd, gate_seq_stride=n_q * 256,
+                                gate_head_stride=256)
+            out = od.download(np.float32).reshape(len(lens), n_q, 256)
+            if first is None:
+                first = out.copy()
+                for i in range(len(lens)):
+                    _, rel = check_attn(out[i], tw.oracle_attend(0, seqs[i], pos[i], q[i], n_q, gate=gate[i]), "entry %d" % i)
+                    assert rel <= REF_BAR_MAX_REL, (i, rel)
+            else:
+                assert np.array_equal(first.view(np.uint32), out.view(np.uint32)), "launch %d differs" % it
+        for b in (qd, gd, od):
+            b.free()
