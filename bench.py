@@ -142,6 +142,40 @@ def time_steps(pool, seqs, ctx0, n_layers, steps, warmup, bufs, stream, first_st
     return wall_ms, ev_ms
 
 
+def time_replay(pool, seqs, n_layers, tokens, bufs, stream):
+    """The same step through a step plan: one token (n_layers x bkv_step_plan_decode + one advance)
+    captured into a graph and replayed `tokens` times after a few untimed replays.  Returns
+    microseconds per layer.  The sequences go on from their current lengths."""
+    from breccia_amd.kv import Graph, StepPlan
+
+    q_dev, out_dev, newk, newv = bufs
+    n = len(seqs)
+    warm = 4
+    pos = [pool.seq_len(s) for s in seqs]
+    for s, p in zip(seqs, pos):
+        pool.seq_reserve(s, p + tokens + warm + 1)
+    plan = StepPlan(pool, seqs, pos, tokens + warm + 1, N_Q, stream=stream)
+    g = Graph(stream)
+    for layer in range(n_layers):
+        off = layer * n * N_KV * HD * 4
+        plan.decode(layer, newk.at(off), newv.at(off), q_dev, out_dev, 1.0 / 16.0, stream=stream)
+    plan.advance(stream)
+    g.end()
+    for _ in range(warm):
+        g.launch(stream)
+    stream.sync()
+    t0 = time.perf_counter()
+    for _ in range(tokens):
+        g.launch(stream)
+    stream.sync()
+    us = (time.perf_counter() - t0) * 1e6 / (tokens * n_layers)
+    _, steps, status = plan.state(stream)
+    assert steps == tokens + warm and status == 0, (steps, status)
+    g.destroy()
+    plan.destroy()
+    return us
+
+
 PREHEAT_MS = 40.0
 
 
@@ -275,8 +309,11 @@ def main() -> int:
                           "seconds": round(cpu_mt_s, 3)}}
         del kf, vf, host_kv
 
+    # and as one token (4 layers + advance) captured into a graph and replayed
+    replay_us = time_replay(pool, seqs, n_layers, max(args.steps // n_layers, 5), bufs, stream)
     extra = {"attn_split_us": round(split_us, 2), "attn_merge_us": round(ms_merge / max(n_merge, 1) * 1e3, 2),
              "two_call_us_per_layer": round(two_call_us, 2),
+             "graph_replay_us_per_layer": round(replay_us, 2),
              "step_event_ms": round(ev_ms / args.steps, 4),
              "preheat_ms": round(pre_ms, 1), "preheat_steps": pre_steps,
              "contexts": ctx, "pool_pages": pool.desc.n_pages, "device": dev_name, "cus": n_cu,
@@ -364,12 +401,14 @@ def bench_batch1(stream, check: bool = True) -> dict:
         run_steps(pool, [s], [ctx], n_layers, 1, *bufs, stream, first_step=nxt)
         stream.sync()
         checked = max(two_call, against_oracle(nxt))
+    replay_us = time_replay(pool, [s], n_layers, 50, bufs, stream)
     out = {"batch1": {"workload": "BASELINE configs[1]: 1 sequence, ctx 4096, 64k-page pool, 12 layers",
                       "us_per_layer": round(us, 2), "GBps": round(bytes_step / (us * 1e-6) / 1e9, 1),
                       "frac_of_hbm_peak": round(bytes_step / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
                       "attn_split_us": round(ms_split / max(n_split, 1) * 1e3, 2),
                       "attn_merge_us": round(ms_merge / max(n_merge, 1) * 1e3, 2),
                       "two_call_us_per_layer": round(two_ms / (steps // 2) * 1e3, 2),
+                      "graph_replay_us_per_layer": round(replay_us, 2),
                       "ms_per_token_12_layers": round(us * 12 / 1e3, 4),
                       "oracle_check_max_abs": checked}}
     pool.destroy()

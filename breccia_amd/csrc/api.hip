@@ -993,6 +993,166 @@ bkv_status bkv_decode_step(bkv_pool* p, int32_t layer, int32_t n, const int32_t*
                               k_new_dev, v_new_dev, true);
 }
 
+// ---- step plans: a decode step whose batch lives on the device -------------------------------
+struct bkv_step_plan {
+    bkv_pool* pool = nullptr;
+    StepDesc* dev = nullptr;
+    float* part_o = nullptr;  // the plan's own split-K workspace: no sharing, nothing to order
+    float* part_ml = nullptr;
+    int32_t n = 0, n_q_head = 0, grid = 0;
+    AttnPlanLimits lim{};
+};
+
+bkv_status bkv_step_plan_create(bkv_pool* p, int32_t n, const int32_t* seqs, const int64_t* pos,
+                                int32_t horizon, int32_t n_q_head, void* stream, bkv_step_plan** out) {
+    if (!p || !out) return fail(BKV_ERR_INVALID, "step_plan_create: NULL argument");
+    *out = nullptr;
+    if (n <= 0 || n > BKV_MAX_BATCH || !seqs || !pos)
+        return fail(BKV_ERR_INVALID, sfmt("step_plan_create: %lld entries (1..%lld) or NULL seqs / pos", n,
+                                          BKV_MAX_BATCH));
+    if (horizon <= 0) return fail(BKV_ERR_INVALID, sfmt("step_plan_create: a horizon of %lld tokens", horizon));
+    if (n_q_head <= 0 || n_q_head % p->g.n_kv != 0 || n_q_head / p->g.n_kv > BKV_MAX_HEAD_GROUP)
+        return fail(BKV_ERR_INVALID, sfmt("step_plan_create: %lld q heads over %lld kv heads (need a whole group "
+                                          "of at most %lld)", n_q_head, p->g.n_kv, BKV_MAX_HEAD_GROUP));
+    if (p->g.hd != 256)
+        return fail(BKV_ERR_INVALID, sfmt("step_plan_create: built for head_dim 256, pool has %lld", p->g.hd));
+    StepDesc host{};
+    for (int i = 0; i < n; ++i) {
+        if (!p->alloc->seq_valid(seqs[i]))
+            return fail(BKV_ERR_RANGE, sfmt("step_plan_create: sequence %lld is not live", seqs[i]));
+        for (int j = 0; j < i; ++j)
+            if (seqs[j] == seqs[i])
+                return fail(BKV_ERR_INVALID, sfmt("step_plan_create: sequence %lld appears twice; one new token "
+                                                  "per sequence and step", seqs[i]));
+        const int64_t last = pos[i] + horizon - 1;  // the last cell a step of this plan may write and attend
+        if (pos[i] < 0 || last >= p->alloc->seq_capacity(seqs[i]))
+            return fail(BKV_ERR_RANGE, sfmt("step_plan_create: cells %lld..%lld of sequence %lld are outside its "
+                                            "addressable cells", pos[i], last, seqs[i]));
+        if (!p->alloc->seq_resident(seqs[i], last + 1))
+            return fail(BKV_ERR_STATE, sfmt("step_plan_create: sequence %lld has swapped-out pages below position "
+                                            "%lld", seqs[i], last));
+        const bkv_status wst = check_writable(p, "step_plan_create", seqs[i], pos[i], last + 1);
+        if (wst != BKV_OK) return wst;
+        host.b.row[i] = seqs[i];
+        host.b.pos[i] = (int32_t)pos[i];
+        host.horizon[i] = (int32_t)last;
+    }
+    host.b.n = n;
+    bkv_status st = need_device(p);
+    if (st != BKV_OK) return st;
+    const int32_t group = n_q_head / p->g.n_kv;
+    if (!attn_on_mfma(p, group, true))
+        return fail(BKV_ERR_INVALID, "step_plan_create: step plans are served by the matrix-core kernels");
+    const AttnPlanLimits lim = attn_plan_limits(p->n_cu, p->max_wgs, p->g.n_kv, group, true);
+    if (plan_attn_ranges(lim, p->g.page_cells, 0, host.b) < 0)
+        return fail(BKV_ERR_INVALID, sfmt("step_plan_create: %lld entries x %lld kv heads need more work-groups "
+                                          "than the partial-result workspace holds (%lld)", n, p->g.n_kv,
+                                          lim.max_wgs));
+    bkv_step_plan* pl = new (std::nothrow) bkv_step_plan();
+    if (!pl) return fail(BKV_ERR_NOMEM, "step_plan_create: out of host memory");
+    pl->pool = p;
+    pl->n = n;
+    pl->n_q_head = n_q_head;
+    pl->lim = lim;
+    // no cut of this batch, at any position, has more work-groups than this
+    pl->grid = std::max<int32_t>(std::min(lim.target, lim.max_wgs), n * lim.per_page);
+    auto bail = [&](bkv_status err) {
+        const std::string keep = g_last_error;
+        (void)bkv_step_plan_destroy(pl);
+        g_last_error = keep;
+        return err;
+    };
+    hipError_t e = hipMalloc(reinterpret_cast<void**>(&pl->dev), sizeof(StepDesc));
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&pl->part_o), (size_t)pl->grid * group * 256 * 4);
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&pl->part_ml), (size_t)pl->grid * group * 2 * 4);
+    if (e != hipSuccess) return bail(hip_fail(e, "hipMalloc (step plan)"));
+    st = flush_tables(p, S(stream));
+    if (st != BKV_OK) return bail(st);
+    void* staged;
+    int slot;
+    st = ring_upload(p, &host, sizeof(host), S(stream), &staged, &slot);
+    if (st != BKV_OK) return bail(st);
+    e = hipMemcpyAsync(pl->dev, staged, sizeof(host), hipMemcpyDeviceToDevice, S(stream));
+    if (e != hipSuccess) return bail(hip_fail(e, "hipMemcpyAsync (step plan)"));
+    st = ring_done(p, slot, S(stream));
+    if (st != BKV_OK) return bail(st);
+    *out = pl;
+    return BKV_OK;
+}
+
+bkv_status bkv_step_plan_destroy(bkv_step_plan* pl) {
+    if (!pl) return fail(BKV_ERR_INVALID, "step_plan_destroy: NULL plan");
+    (void)hipDeviceSynchronize();
+    if (pl->dev) (void)hipFree(pl->dev);
+    if (pl->part_o) (void)hipFree(pl->part_o);
+    if (pl->part_ml) (void)hipFree(pl->part_ml);
+    delete pl;
+    return BKV_OK;
+}
+
+bkv_status bkv_step_plan_decode(bkv_step_plan* pl, int32_t layer, const float* k_new_dev, const float* v_new_dev,
+                                const float* q_dev, const float* gate_dev, int64_t gate_seq_stride,
+                                int64_t gate_head_stride, float scale, float* out_dev, void* stream) {
+    if (!pl) return fail(BKV_ERR_INVALID, "step_plan_decode: NULL plan");
+    bkv_pool* p = pl->pool;
+    if (layer < 0 || layer >= p->g.n_layers)
+        return fail(BKV_ERR_RANGE, sfmt("step_plan_decode: layer %lld is outside 0..%lld", layer, p->g.n_layers));
+    if (!q_dev || !out_dev || !k_new_dev || !v_new_dev || !aligned16(q_dev) || !aligned16(out_dev) ||
+        !aligned16(k_new_dev) || !aligned16(v_new_dev))
+        return fail(BKV_ERR_INVALID, "step_plan_decode: q / out / k / v device pointers must be non-NULL and "
+                                     "16-byte aligned");
+    // Block-table changes made since the last call still travel the usual way, which a stream under
+    // capture cannot record (it waits on the host for a free ring slot): make them before capturing.
+    if (!p->alloc->pending().empty() || p->tiers.pending) {
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        if (stream && hipStreamIsCapturing(S(stream), &cs) == hipSuccess && cs != hipStreamCaptureStatusNone)
+            return fail(BKV_ERR_STATE, "step_plan_decode: block-table changes are pending while the stream is being "
+                                       "captured; make allocator calls, then any eager call, before the capture");
+        (void)hipGetLastError();
+        const bkv_status st = flush_tables(p, S(stream));
+        if (st != BKV_OK) return st;
+    }
+    AttnBatch b{};
+    b.n = pl->n;
+    AttnArgs a;
+    a.mfma = true;
+    a.n_q_head = pl->n_q_head;
+    a.q = q_dev;
+    a.gate = gate_dev;
+    a.gate_seq_stride = gate_seq_stride;
+    a.gate_head_stride = gate_head_stride;
+    a.scale = scale;
+    a.out = out_dev;
+    a.new_k = k_new_dev;
+    a.new_v = v_new_dev;
+    a.ws_o = pl->part_o;
+    a.ws_ml = pl->part_ml;
+    a.timed = false;
+    a.desc = &pl->dev->b;
+    a.desc_grid = pl->grid;
+    BKV_HIP(launch_decode_attn(p, layer, b, a, S(stream)));
+    return BKV_OK;
+}
+
+bkv_status bkv_step_plan_advance(bkv_step_plan* pl, void* stream) {
+    if (!pl) return fail(BKV_ERR_INVALID, "step_plan_advance: NULL plan");
+    BKV_HIP(launch_step_advance(pl->dev, pl->lim, pl->pool->g.page_cells, S(stream)));
+    return BKV_OK;
+}
+
+bkv_status bkv_step_plan_state(bkv_step_plan* pl, void* stream, int64_t* pos_out, uint32_t* steps_out,
+                               int32_t* status_out) {
+    if (!pl) return fail(BKV_ERR_INVALID, "step_plan_state: NULL plan");
+    StepDesc host;
+    BKV_HIP(hipStreamSynchronize(S(stream)));
+    BKV_HIP(hipMemcpy(&host, pl->dev, sizeof(host), hipMemcpyDeviceToHost));
+    if (pos_out)
+        for (int i = 0; i < pl->n; ++i) pos_out[i] = host.b.pos[i];
+    if (steps_out) *steps_out = host.steps;
+    if (status_out) *status_out = host.status;
+    return BKV_OK;
+}
+
 bkv_status bkv_decode_attn_select(bkv_pool* p, int32_t layer, int32_t n, const int32_t* seqs,
                                   const int64_t* pos, int32_t n_q_head, const float* q_dev,
                                   const float* gate_dev, int64_t gate_seq_stride,
@@ -1711,6 +1871,37 @@ bkv_status bkv_memcpy_d2h(void* host, const void* dev, uint64_t bytes, void* str
     BKV_HIP(hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, S(stream)));
     return BKV_OK;
 }
+bkv_status bkv_graph_begin_capture(void* stream) {
+    if (!stream) return fail(BKV_ERR_INVALID, "graph_begin_capture: the NULL stream cannot be captured");
+    BKV_HIP(hipStreamBeginCapture(S(stream), hipStreamCaptureModeThreadLocal));
+    return BKV_OK;
+}
+
+bkv_status bkv_graph_end_capture(void* stream, void** graph_exec_out) {
+    if (!stream || !graph_exec_out) return fail(BKV_ERR_INVALID, "graph_end_capture: NULL argument");
+    *graph_exec_out = nullptr;
+    hipGraph_t graph = nullptr;
+    BKV_HIP(hipStreamEndCapture(S(stream), &graph));
+    hipGraphExec_t exec = nullptr;
+    const hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) return hip_fail(e, "hipGraphInstantiate");
+    *graph_exec_out = exec;
+    return BKV_OK;
+}
+
+bkv_status bkv_graph_launch(void* graph_exec, void* stream) {
+    if (!graph_exec) return fail(BKV_ERR_INVALID, "graph_launch: NULL graph");
+    BKV_HIP(hipGraphLaunch(static_cast<hipGraphExec_t>(graph_exec), S(stream)));
+    return BKV_OK;
+}
+
+bkv_status bkv_graph_destroy(void* graph_exec) {
+    if (!graph_exec) return fail(BKV_ERR_INVALID, "graph_destroy: NULL graph");
+    BKV_HIP(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec)));
+    return BKV_OK;
+}
+
 bkv_status bkv_stream_create(void** stream_out) {
     if (!stream_out) return fail(BKV_ERR_INVALID, "stream_create: NULL out pointer");
     hipStream_t s;

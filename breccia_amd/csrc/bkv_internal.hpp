@@ -219,7 +219,21 @@ struct AttnArgs {
     float* ws_o = nullptr;
     float* ws_ml = nullptr;
     bool timed = true;  // kernels carry stage-timer events while the pool's timer is on
+    // the batch lives in a device-resident descriptor (a step plan): the kernels read it there and the
+    // split-K launch has this fixed grid
+    const AttnBatch* desc = nullptr;
+    int32_t desc_grid = 0;
 };
+
+// Device-resident state of a step plan (bkv_step_plan_*): the batch as the kernels read it, the last
+// cell each entry was checked for, and what the advances did.
+struct StepDesc {
+    AttnBatch b;
+    int32_t horizon[kMaxBatch];
+    int32_t status;  // 0, or 1 once an advance was refused at the horizon
+    uint32_t steps;  // advances done
+};
+hipError_t launch_step_advance(StepDesc* d, const AttnPlanLimits& lim, int32_t page_cells, hipStream_t stream);
 // Fills wg_base/splits/pps from row/pos (attn_plan.hpp); returns the total work-group count, -1
 // when the batch cannot be cut into as few work-groups as the workspace holds.  sel_groups > 0:
 // every entry is planned for that many groups of four selected blocks instead of its pages.

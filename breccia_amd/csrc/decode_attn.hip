@@ -592,6 +592,7 @@ __global__ __launch_bounds__(kBlock, HG == 8 ? 2 : 3) void decode_attn_kernel(co
 
 struct MergeParams {
     AttnBatch b;
+    const AttnBatch* bd;  // DESC: the batch is read from this device-resident copy
     const float* part_o;
     const float* part_ml;
     const float* gate;
@@ -607,6 +608,7 @@ constexpr int kMergeInFlight = 8;  // partial rows (16 bytes a lane) a wave requ
 // 4 d4 .. 4 d4 + 3 of splits g, g + 16, ...; it requests its first 8 partial rows straight away,
 // and only then are the per-split (m, l) pairs staged in LDS and the maximum agreed, so the two
 // round trips to memory overlap.  One round covers 128 splits.
+template <bool DESC>
 __global__ __launch_bounds__(64 * kMergeGroups) void decode_attn_merge_kernel(const MergeParams P) {
     constexpr int kMaxStaged = 1024;
     constexpr int kThreads = 64 * kMergeGroups;
@@ -621,8 +623,16 @@ __global__ __launch_bounds__(64 * kMergeGroups) void decode_attn_merge_kernel(co
     const int hl = h % P.group;
     const int hc = hl / P.hg;
     const int hh = hl % P.hg;
-    const int splits = P.b.splits[e];
-    const int wg0 = P.b.wg_base[e] + hc * splits * P.n_kv + kvh;
+    int splits, base;
+    if constexpr (DESC) {
+        const batch_desc_ptr D = (batch_desc_ptr)(uintptr_t)P.bd;
+        splits = D->splits[e];
+        base = D->wg_base[e];
+    } else {
+        splits = P.b.splits[e];
+        base = P.b.wg_base[e];
+    }
+    const int wg0 = base + hc * splits * P.n_kv + kvh;
     const int d4 = threadIdx.x & 63;
     const int g = threadIdx.x >> 6;
     const size_t ostride = (size_t)P.n_kv * P.hg * kHd;  // floats between consecutive splits
@@ -796,6 +806,7 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
     const int32_t hg = a.mfma ? group : attn_heads_per_wave(group);
     AttnKernelParams kp;
     kp.b = b;
+    kp.bd = a.desc;
     kp.kpool = p->k_layer[(size_t)layer];
     kp.vpool = p->v_layer[(size_t)layer];
     kp.tables = p->table_dev;
@@ -818,7 +829,7 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
     kp.vpool_w = p->v_layer[(size_t)layer];
     const bool sel = a.ids != nullptr;
     const bool step = a.new_k != nullptr;
-    const int32_t total = b.wg_base[b.n];
+    const int32_t total = a.desc ? a.desc_grid : b.wg_base[b.n];
     const int32_t n_units = total / kp.n_hc;
     const int32_t grid = (n_units + 7) / 8 * 8 * kp.n_hc;
     if (a.mfma) {
@@ -862,6 +873,7 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
     if (err != hipSuccess) return err;
     MergeParams mp;
     mp.b = b;
+    mp.bd = a.desc;
     mp.part_o = kp.part_o;
     mp.part_ml = kp.part_ml;
     mp.gate = a.gate;
@@ -872,12 +884,37 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
     mp.n_q = a.n_q_head;
     mp.group = group;
     mp.hg = hg;
-    if (a.timed)
-        launch_staged(p, BKV_STAGE_ATTN_MERGE, decode_attn_merge_kernel, dim3((unsigned)(b.n * a.n_q_head)),
-                      dim3(64 * kMergeGroups), 0, stream, mp);
+    const dim3 mgrid((unsigned)(b.n * a.n_q_head)), mblock(64 * kMergeGroups);
+    if (a.desc)
+        hipLaunchKernelGGL(decode_attn_merge_kernel<true>, mgrid, mblock, 0, stream, mp);
+    else if (a.timed)
+        launch_staged(p, BKV_STAGE_ATTN_MERGE, decode_attn_merge_kernel<false>, mgrid, mblock, 0, stream, mp);
     else
-        hipLaunchKernelGGL(decode_attn_merge_kernel, dim3((unsigned)(b.n * a.n_q_head)), dim3(64 * kMergeGroups),
-                           0, stream, mp);
+        hipLaunchKernelGGL(decode_attn_merge_kernel<false>, mgrid, mblock, 0, stream, mp);
+    return hipGetLastError();
+}
+
+// ---- a decode step that re-plans itself on the device ------------------------------------------
+// One thread: every entry moves on by one cell and the batch is cut again, by the same function the
+// host uses, so that a replayed launch reads what a fresh call would have been given.  An entry
+// that would pass the last cell the plan was checked for stops the advance (nothing moves, the
+// status word says so).
+__global__ void step_advance_kernel(StepDesc* d, AttnPlanLimits lim, int32_t page_cells) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    AttnBatch b = d->b;
+    for (int i = 0; i < b.n; ++i)
+        if (b.pos[i] + 1 > d->horizon[i]) {
+            d->status = 1;
+            return;
+        }
+    for (int i = 0; i < b.n; ++i) b.pos[i] += 1;
+    (void)plan_attn_ranges(lim, page_cells, 0, b);
+    d->b = b;
+    d->steps += 1u;
+}
+
+hipError_t launch_step_advance(StepDesc* d, const AttnPlanLimits& lim, int32_t page_cells, hipStream_t stream) {
+    hipLaunchKernelGGL(step_advance_kernel, dim3(1), dim3(64), 0, stream, d, lim, page_cells);
     return hipGetLastError();
 }
 

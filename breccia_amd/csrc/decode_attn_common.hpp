@@ -18,6 +18,9 @@ typedef float f4 __attribute__((ext_vector_type(4)));
 
 struct AttnKernelParams {
     AttnBatch b;
+    // kernels instantiated with DESC read the batch from this device-resident copy instead of `b`: a
+    // launch recorded once (in a graph) then serves whatever batch the descriptor holds when it runs
+    const AttnBatch* bd;
     const uint8_t* kpool;
     const uint8_t* vpool;
     const int32_t* tables;
@@ -40,6 +43,35 @@ struct AttnKernelParams {
     uint8_t* kpool_w;
     uint8_t* vpool_w;
 };
+
+// Which unit of work a work-group of the matrix-core kernels has: entry e, its rem-th work-group
+// (page range x kv head), and the entry's position, block-table row and pages per range.  With DESC the
+// batch is read from device memory through the constant address space (uniform addresses: scalar
+// loads), and a work-group past the end of the current cut reports false: such a launch has a fixed grid.
+typedef const __attribute__((address_space(4))) AttnBatch* batch_desc_ptr;
+template <bool DESC>
+__device__ __forceinline__ bool unit_of_work_group(const AttnKernelParams& P, int unit, int& e, int& rem, int& pos,
+                                                   int& row, int& pps) {
+    if constexpr (DESC) {
+        const batch_desc_ptr D = (batch_desc_ptr)(uintptr_t)P.bd;
+        const int n = D->n;
+        if (unit >= D->wg_base[n]) return false;
+        e = 0;
+        while (e + 1 < n && unit >= D->wg_base[e + 1]) ++e;
+        rem = unit - D->wg_base[e];
+        pos = D->pos[e];
+        row = D->row[e];
+        pps = D->pps[e];
+    } else {
+        e = 0;
+        while (e + 1 < P.b.n && unit >= P.b.wg_base[e + 1]) ++e;
+        rem = unit - P.b.wg_base[e];
+        pos = P.b.pos[e];
+        row = P.b.row[e];
+        pps = P.b.pps[e];
+    }
+    return true;
+}
 
 // Row encodings of the K and V pools:
 //   kRowF16   256 f16
@@ -74,6 +106,7 @@ __device__ __forceinline__ bool block_cell_live(uint32_t id, int r, int pos) {
 // The split-K kernels on the matrix cores (decode_attn_mfma.hip); `total` work-groups, one per
 // (entry, kv head, page range).
 // `start` / `stop`: optional events attached to the dispatch (its own begin and end time stamps)
+// kp.bd != nullptr: the step kernels that read the batch from the descriptor (`total` is then the fixed grid).
 hipError_t launch_decode_attn_mfma(const AttnKernelParams& kp, int layout, bool step, bool sel, int32_t total,
                                    hipStream_t stream, hipEvent_t start = nullptr, hipEvent_t stop = nullptr);
 

@@ -143,23 +143,21 @@ __device__ __forceinline__ void k_pair_home(const v4u& lo_rows, const v4u& hi_ro
 // SEL: the 16 rows of an iteration are four listed 4-cell blocks instead of a page, as in
 // decode_attn_kernel<..., SEL = true> (block g supplies the V rows of lane group g, block c / 4
 // the K row of lane c).
-template <bool STEP, bool SEL = false>
+template <bool STEP, bool SEL = false, bool DESC = false>
 __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnKernelParams P) {
     static_assert(!(STEP && SEL), "the fused step attends the dense selection");
     __shared__ __attribute__((aligned(16))) MfmaFoldLds lds;
 
     // ---- which (entry, kv head, page range); one work-group per unit (no head chunks) --------
     const int unit = blockIdx.x;
-    int e = 0;
-    while (e + 1 < P.b.n && unit >= P.b.wg_base[e + 1]) ++e;
-    const int rem = unit - P.b.wg_base[e];
+    int e, rem, pos, row, pps;
+    if (!unit_of_work_group<DESC>(P, unit, e, rem, pos, row, pps)) return;
     const int split = rem / P.n_kv;
     const int kvh = rem - split * P.n_kv;
     const int wg = unit;
-    const int pos = P.b.pos[e];
     typedef const __attribute__((address_space(4))) int32_t* table_ptr;
     typedef const __attribute__((address_space(4))) uint32_t* list_ptr;
-    const table_ptr bt = (table_ptr)(uintptr_t)(P.tables + (size_t)P.b.row[e] * (size_t)P.max_pages_per_seq);
+    const table_ptr bt = (table_ptr)(uintptr_t)(P.tables + (size_t)row * (size_t)P.max_pages_per_seq);
     uint32_t n_sel = 0;
     list_ptr sel = nullptr;
     if constexpr (SEL) {
@@ -168,7 +166,6 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
     }
     // loop iterations of this entry: pages, or groups of four selected blocks
     const int n_pages = SEL ? (int)((n_sel + 3u) >> 2) : pos / kPage + 1;
-    const int pps = P.b.pps[e];
     const int pg0 = split * pps;
     const int pg1 = min(pg0 + pps, n_pages);
 
@@ -460,7 +457,7 @@ __device__ __forceinline__ void i8h_unit_to_lds(const uint8_t* src, bool real, u
     if (lane < 16) __builtin_amdgcn_global_load_lds((gptr)(lane_src + 4 * step), (lptr)(dst + 4096), 16, 0, 0);
 }
 
-template <bool STEP>
+template <bool STEP, bool DESC = false>
 __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const AttnKernelParams P) {
     // slot 0 and slot 1 of the four waves; the fold staging of the epilogue reuses their memory
     __shared__ __attribute__((aligned(16))) uint8_t ring[2 * kWaves * kI8hSlot];
@@ -470,19 +467,16 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
     constexpr int kRow = row_bytes_of(kRowI8H);  // 272
 
     const int unit = blockIdx.x;
-    int e = 0;
-    while (e + 1 < P.b.n && unit >= P.b.wg_base[e + 1]) ++e;
-    const int rem = unit - P.b.wg_base[e];
+    int e, rem, pos, row, pps;
+    if (!unit_of_work_group<DESC>(P, unit, e, rem, pos, row, pps)) return;
     const int split = rem / P.n_kv;
     const int kvh = rem - split * P.n_kv;
     const int wg = unit;
-    const int pos = P.b.pos[e];
     const int n_pages = pos / kPage + 1;
-    const int pps = P.b.pps[e];
     const int pg0 = split * pps;
     const int pg1 = min(pg0 + pps, n_pages);
     typedef const __attribute__((address_space(4))) int32_t* table_ptr;
-    const table_ptr bt = (table_ptr)(uintptr_t)(P.tables + (size_t)P.b.row[e] * (size_t)P.max_pages_per_seq);
+    const table_ptr bt = (table_ptr)(uintptr_t)(P.tables + (size_t)row * (size_t)P.max_pages_per_seq);
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
@@ -748,7 +742,7 @@ __device__ __forceinline__ void q8v_unit_to_lds(const uint8_t* src, bool real, u
     if (lane < 32) __builtin_amdgcn_global_load_lds((gptr)(lane_src + 4 * step), (lptr)(dst + 4096), 16, 0, 0);
 }
 
-template <bool STEP>
+template <bool STEP, bool DESC = false>
 __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const AttnKernelParams P) {
     // per wave one K slot and two V slots during the loop, the fold staging after it
     constexpr int kWaveLds = kQ8vKSlot + 2 * kQ8vUnit;
@@ -756,19 +750,16 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
     __shared__ __attribute__((aligned(16))) uint8_t smem[kLds];
 
     const int unit = blockIdx.x;
-    int e = 0;
-    while (e + 1 < P.b.n && unit >= P.b.wg_base[e + 1]) ++e;
-    const int rem = unit - P.b.wg_base[e];
+    int e, rem, pos, row, pps;
+    if (!unit_of_work_group<DESC>(P, unit, e, rem, pos, row, pps)) return;
     const int split = rem / P.n_kv;
     const int kvh = rem - split * P.n_kv;
     const int wg = unit;
-    const int pos = P.b.pos[e];
     const int n_pages = pos / kPage + 1;
-    const int pps = P.b.pps[e];
     const int pg0 = split * pps;
     const int pg1 = min(pg0 + pps, n_pages);
     typedef const __attribute__((address_space(4))) int32_t* table_ptr;
-    const table_ptr bt = (table_ptr)(uintptr_t)(P.tables + (size_t)P.b.row[e] * (size_t)P.max_pages_per_seq);
+    const table_ptr bt = (table_ptr)(uintptr_t)(P.tables + (size_t)row * (size_t)P.max_pages_per_seq);
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
@@ -1015,6 +1006,17 @@ static void launch_one(K kernel, const AttnKernelParams& kp, int32_t total, hipS
 
 hipError_t launch_decode_attn_mfma(const AttnKernelParams& kp, int layout, bool step, bool sel, int32_t total,
                                    hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
+    if (kp.bd) {
+        // the batch comes from the device-resident descriptor: the fused step only
+        if (!step || sel) return hipErrorInvalidValue;
+        if (layout == BKV_LAYOUT_I8H)
+            launch_one(decode_attn_mfma_i8h_kernel<true, true>, kp, total, stream, start, stop);
+        else if (layout == BKV_LAYOUT_Q8V)
+            launch_one(decode_attn_mfma_q8v_kernel<true, true>, kp, total, stream, start, stop);
+        else
+            launch_one(decode_attn_mfma_kernel<true, false, true>, kp, total, stream, start, stop);
+        return hipGetLastError();
+    }
     if (layout == BKV_LAYOUT_I8H) {
         if (step)
             launch_one(decode_attn_mfma_i8h_kernel<true>, kp, total, stream, start, stop);

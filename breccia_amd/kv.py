@@ -491,6 +491,64 @@ class Pool:
         check(lib.bkv_seq_restore(self.handle, seq, lp0, n, host.ptr, _sh(stream)))
 
 
+class StepPlan:
+    """A decode step whose batch lives on the device (bkv_step_plan_*): capturable and replayable."""
+
+    def __init__(self, pool: Pool, seqs, pos, horizon: int, n_q_head: int, stream=None):
+        seqs, ps = _i32(seqs)
+        pos, pp = _i64(pos)
+        assert seqs.size == pos.size
+        self.n = int(seqs.size)
+        self.handle = C.c_void_p()
+        check(lib.bkv_step_plan_create(pool.handle, self.n, ps, pp, horizon, n_q_head, _sh(stream),
+                                       C.byref(self.handle)))
+
+    def decode(self, layer: int, k_new_dev, v_new_dev, q_dev, out_dev, scale: float, gate_dev=None,
+               gate_seq_stride: int = 0, gate_head_stride: int = 0, stream=None) -> None:
+        check(lib.bkv_step_plan_decode(self.handle, layer, _ptr(k_new_dev), _ptr(v_new_dev), _ptr(q_dev),
+                                       _ptr(gate_dev), gate_seq_stride, gate_head_stride, scale, _ptr(out_dev),
+                                       _sh(stream)))
+
+    def advance(self, stream=None) -> None:
+        check(lib.bkv_step_plan_advance(self.handle, _sh(stream)))
+
+    def state(self, stream=None):
+        """(positions, advances done, status) once `stream` has drained."""
+        pos = np.zeros(self.n, dtype=np.int64)
+        steps, status = C.c_uint32(), C.c_int32()
+        check(lib.bkv_step_plan_state(self.handle, _sh(stream), pos.ctypes.data_as(C.POINTER(C.c_int64)),
+                                      C.byref(steps), C.byref(status)))
+        return pos, int(steps.value), int(status.value)
+
+    def destroy(self) -> None:
+        if self.handle:
+            check(lib.bkv_step_plan_destroy(self.handle))
+            self.handle = None
+
+
+class Graph:
+    """Work captured from a stream (bkv_graph_*)."""
+
+    def __init__(self, stream: Stream):
+        self.stream = stream
+        self.exec = None
+        check(lib.bkv_graph_begin_capture(stream.handle))
+
+    def end(self) -> "Graph":
+        ex = C.c_void_p()
+        check(lib.bkv_graph_end_capture(self.stream.handle, C.byref(ex)))
+        self.exec = ex
+        return self
+
+    def launch(self, stream=None) -> None:
+        check(lib.bkv_graph_launch(self.exec, _sh(stream if stream is not None else self.stream)))
+
+    def destroy(self) -> None:
+        if self.exec:
+            check(lib.bkv_graph_destroy(self.exec))
+            self.exec = None
+
+
 class PinnedBuffer:
     """hipHostMalloc'd memory owned through the pool, viewable as a numpy array."""
 

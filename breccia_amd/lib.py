@@ -106,6 +106,11 @@ _SIGNATURES = {
                                    _vp, _vp]),
     "bkv_decode_step": (C.c_int, [_vp, _i32, _i32, _pi32, _pi64, _vp, _vp, _i32, _vp, _vp, _i64, _i64, _f32,
                                   _vp, _vp]),
+    "bkv_step_plan_create": (C.c_int, [_vp, _i32, _pi32, _pi64, _i32, _i32, _vp, C.POINTER(_vp)]),
+    "bkv_step_plan_destroy": (C.c_int, [_vp]),
+    "bkv_step_plan_decode": (C.c_int, [_vp, _i32, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _vp, _vp]),
+    "bkv_step_plan_advance": (C.c_int, [_vp, _vp]),
+    "bkv_step_plan_state": (C.c_int, [_vp, _vp, _pi64, C.POINTER(C.c_uint32), _pi32]),
     "bkv_decode_attn_select": (C.c_int, [_vp, _i32, _i32, _pi32, _pi64, _i32, _vp, _vp, _i64, _i64, _f32,
                                          _vp, _i64, _vp, _i32, _vp, _vp]),
     "bkv_select_blocks": (C.c_int, [_vp, _i32, _pi64, _vp, C.POINTER(_vp), _pi32, _i32, _i32, _i32, _vp,
@@ -128,6 +133,10 @@ _SIGNATURES = {
     "bkv_memcpy_h2d": (C.c_int, [_vp, _vp, _u64, _vp]),
     "bkv_memcpy_d2h": (C.c_int, [_vp, _vp, _u64, _vp]),
     "bkv_stream_create": (C.c_int, [C.POINTER(_vp)]),
+    "bkv_graph_begin_capture": (C.c_int, [_vp]),
+    "bkv_graph_end_capture": (C.c_int, [_vp, C.POINTER(_vp)]),
+    "bkv_graph_launch": (C.c_int, [_vp, _vp]),
+    "bkv_graph_destroy": (C.c_int, [_vp]),
     "bkv_stream_destroy": (C.c_int, [_vp]),
     "bkv_stream_sync": (C.c_int, [_vp]),
     "bkv_device_sync": (C.c_int, []),

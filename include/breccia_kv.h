@@ -347,6 +347,45 @@ bkv_status bkv_decode_step(bkv_pool *pool, int32_t layer, int32_t n, const int32
                            int64_t gate_seq_stride, int64_t gate_head_stride, float scale,
                            float *out_dev, void *stream);
 
+/* ---- step plans: a decode step that can be recorded once and replayed ------------------------
+ * The reference records every stage of a layer into one open batch and submits once
+ * (crates/breccia-kernels/src/ops/mod.rs:205-222, src/dispatch_batch.rs:46-59; contract test
+ * tests/batching.rs:27-88: batched == unbatched bit for bit).  The HIP analogue is a graph: the
+ * calls of one token are captured from a stream once and replayed for the tokens that follow.
+ * bkv_decode_step cannot be captured usefully -- positions, block-table rows and the cut into
+ * work-groups travel as kernel arguments, so a replay would repeat one token.  A step plan keeps
+ * that batch in device memory instead:
+ *   bkv_step_plan_create   checks, for every listed sequence, the `horizon` cells pos[i] ..
+ *                          pos[i] + horizon - 1 the way bkv_decode_step checks one (reserved, on
+ *                          the device, held by this sequence alone; each sequence once), pushes
+ *                          pending block-table changes and writes the descriptor on `stream`.
+ *   bkv_step_plan_decode   bkv_decode_step for the plan's batch at its current positions on one
+ *                          layer: same kernels, same bytes in the pool, same output bits.  It
+ *                          reads positions and the cut from the descriptor, uses a workspace of the
+ *                          plan's own, copies nothing from the host, allocates nothing and attaches
+ *                          no timer: it can be captured, any number of layers per token.
+ *   bkv_step_plan_advance  one small kernel: every position moves on by one cell and the batch is
+ *                          cut again on the device by the function the host uses (so a replayed
+ *                          step sums its partial results in the order a fresh call would).  An
+ *                          advance past the checked cells changes nothing and sets status 1.
+ *   bkv_step_plan_state    waits for `stream`, then reports positions, advances done and status.
+ * Between creation and the last replay the caller leaves the listed sequences alone (no free,
+ * fork, truncate, evict); allocator calls for OTHER sequences are fine but must be followed by an
+ * eager call on the pool before a capture begins, since their block-table changes cannot be
+ * recorded.  Destroy a pool's plans before the pool.  Matrix-core pools only (no
+ * BKV_POOL_ATTN_VALU), all three layouts. */
+typedef struct bkv_step_plan bkv_step_plan;
+bkv_status bkv_step_plan_create(bkv_pool *pool, int32_t n, const int32_t *seqs, const int64_t *pos,
+                                int32_t horizon, int32_t n_q_head, void *stream, bkv_step_plan **out);
+bkv_status bkv_step_plan_destroy(bkv_step_plan *plan);
+bkv_status bkv_step_plan_decode(bkv_step_plan *plan, int32_t layer, const float *k_new_dev,
+                                const float *v_new_dev, const float *q_dev, const float *gate_dev,
+                                int64_t gate_seq_stride, int64_t gate_head_stride, float scale,
+                                float *out_dev, void *stream);
+bkv_status bkv_step_plan_advance(bkv_step_plan *plan, void *stream);
+bkv_status bkv_step_plan_state(bkv_step_plan *plan, void *stream, int64_t *pos_out, uint32_t *steps_out,
+                               int32_t *status_out);
+
 /* The same attention over a selection list instead of every cell: the reference's real
  * long-context form (Qsa::attend / Qsa::apply read ws.ids [T, max_ids] and ws.counts [T],
  * qsa/mod.rs:1382-1462; shaders/qsa_attn_scores_small.comp; oracle qsa/cpu.rs:197-257).
@@ -492,6 +531,12 @@ bkv_status bkv_dev_free(void *dev);
 bkv_status bkv_memcpy_h2d(void *dev, const void *host, uint64_t bytes, void *stream);
 bkv_status bkv_memcpy_d2h(void *host, const void *dev, uint64_t bytes, void *stream);
 bkv_status bkv_stream_create(void **stream_out);
+/* Stream capture into a graph (hipStreamBeginCapture / EndCapture + hipGraphInstantiate, thread-local
+ * capture mode) and its replay; `stream` must not be NULL. */
+bkv_status bkv_graph_begin_capture(void *stream);
+bkv_status bkv_graph_end_capture(void *stream, void **graph_exec_out);
+bkv_status bkv_graph_launch(void *graph_exec, void *stream);
+bkv_status bkv_graph_destroy(void *graph_exec);
 bkv_status bkv_stream_destroy(void *stream);
 bkv_status bkv_stream_sync(void *stream);
 bkv_status bkv_device_sync(void);

@@ -376,3 +376,33 @@ def test_writes_need_reserved_cells_on_pages_the_sequence_holds_alone():
         p.prefix_insert(parent, np.arange(32))
         expect(L.ERR_STATE, p.append, 0, [parent], [16], [4], z, z)
         p.check()
+
+
+def test_step_plan_checks_come_before_any_device_work():
+    """bkv_step_plan_create validates like bkv_decode_step, for every cell of the horizon, on the host:
+    a host-only pool gets as far as the device check and no further."""
+    import ctypes as C
+    from breccia_amd.kv import StepPlan
+
+    with host_pool(n_pages=16, max_seqs=4) as pool:
+        s = pool.seq_create()
+        pool.seq_reserve(s, 30)
+        for kw, status in ((dict(seqs=[s], pos=[25], horizon=6), L.ERR_RANGE),      # cell 30 is not reserved
+                           (dict(seqs=[s, s], pos=[1, 2], horizon=2), L.ERR_INVALID),
+                           (dict(seqs=[7], pos=[0], horizon=1), L.ERR_RANGE),
+                           (dict(seqs=[s], pos=[0], horizon=0), L.ERR_INVALID),
+                           (dict(seqs=[s], pos=[0], horizon=4, n_q=17), L.ERR_INVALID),
+                           (dict(seqs=[s], pos=[20], horizon=10), L.ERR_NO_DEVICE)):  # valid: stops at the device
+            with pytest.raises(BkvError) as ei:
+                StepPlan(pool, kw["seqs"], kw["pos"], kw["horizon"], kw.get("n_q", 16))
+            assert ei.value.status == status, (kw, ei.value)
+        child = pool.seq_fork(s, 20)
+        with pytest.raises(BkvError) as ei:       # the page of cells 16..31 is shared now
+            StepPlan(pool, [s], [20], 5, 16)
+        assert ei.value.status == L.ERR_STATE
+        pool.seq_free(child)
+        for fn in ("bkv_step_plan_destroy",):
+            assert getattr(L.lib, fn)(None) == L.ERR_INVALID
+        assert L.lib.bkv_step_plan_decode(None, 0, None, None, None, None, 0, 0, C.c_float(1.0), None, None) == L.ERR_INVALID
+        assert L.lib.bkv_step_plan_advance(None, None) == L.ERR_INVALID
+        assert L.lib.bkv_graph_begin_capture(None) == L.ERR_INVALID
