@@ -734,8 +734,8 @@ int32_t attn_heads_per_wave(int32_t group) { return group % 8 == 0 ? 8 : 4; }
 // created with BKV_POOL_ATTN_VALU (the VALU formulation, kept for comparison).
 bool attn_on_mfma(const bkv_pool* p, int32_t group, bool dense) {
     if (group > 16 || (p->desc.flags & BKV_POOL_ATTN_VALU) != 0) return false;
-    // f16 rows: every call; the quantised layouts: the dense selection
-    return p->g.layout == BKV_LAYOUT_F16 || dense;
+    (void)dense;
+    return true;
 }
 
 // The limits a plan of this pool geometry works under.  The partial-result workspace holds

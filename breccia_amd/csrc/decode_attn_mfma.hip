@@ -443,22 +443,70 @@ __device__ __forceinline__ half8 codes8_to_f16(v2u w) {
 constexpr int kI8hUnit = kPage * row_bytes_of(kRowI8H);  // 4352
 constexpr int kI8hSlot = 2 * kI8hUnit;                    // K unit, then V unit
 
+// Where the 16 rows of one K or V unit come from: one run (a page's rows of one kv head), or, for a
+// selection list, four runs of four rows (the listed blocks; crates/breccia-kernels/src/qsa/cpu.rs:
+// 248-257).  In LDS the unit looks the same either way: a 16-byte piece at byte `off` of the unit
+// comes from run off / RUN (row lengths are multiples of 16 bytes, so a piece never straddles runs).
+template <bool SEL>
+struct UnitSrc {
+    const uint8_t* run[SEL ? 4 : 1];
+};
+template <bool SEL, int RUN>
+__device__ __forceinline__ const uint8_t* unit_piece(const UnitSrc<SEL>& u, int off) {
+    if constexpr (SEL) {
+        const uint8_t* base = off >= 3 * RUN ? u.run[3] : off >= 2 * RUN ? u.run[2] : off >= RUN ? u.run[1] : u.run[0];
+        const int j = (off >= RUN) + (off >= 2 * RUN) + (off >= 3 * RUN);
+        return base + (off - j * RUN);
+    } else {
+        return u.run[0] + off;
+    }
+}
+// The four listed blocks of loop iteration `it` of a selection list: ids for the causal test
+// (0xffffffff past the end of the list) and, clamped to the blocks at or below `pos` before any
+// address is formed, the byte offset of each block's rows inside a pool whose pages are
+// `page_bytes` long and whose rows are `row_bytes` long.
+typedef const __attribute__((address_space(4))) uint32_t* sel_list_ptr;
+typedef const __attribute__((address_space(4))) int32_t* block_table_ptr;
+__device__ __forceinline__ void listed_blocks(sel_list_ptr sel, uint32_t n_sel, block_table_ptr bt, int it, int pos,
+                                              size_t page_bytes, size_t head_off, int row_bytes, uint32_t (&id)[4],
+                                              size_t (&off)[4]) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t at = (uint32_t)it * 4u + (uint32_t)j;
+        const uint32_t raw = sel[min(at, n_sel - 1u)];
+        id[j] = at < n_sel ? raw : 0xffffffffu;
+        const uint32_t idc = min(raw, (uint32_t)pos >> 2);
+        off[j] = (size_t)bt[idc >> 2] * page_bytes + head_off + (size_t)(idc & 3u) * 4u * (size_t)row_bytes;
+    }
+}
+__device__ __forceinline__ uint32_t pick4(const uint32_t (&a)[4], int j) {
+    return j == 0 ? a[0] : j == 1 ? a[1] : j == 2 ? a[2] : a[3];
+}
+
 // 4352 bytes = 4 x 1024 + 256: four full instructions and one of 16 lanes.  `real` false issues the
 // same five instructions on one 16-byte location (the data is never used): the number of loads
 // in flight, which the waits count, then does not depend on where in its range a wave is.
-__device__ __forceinline__ void i8h_unit_to_lds(const uint8_t* src, bool real, uint8_t* dst, int lane) {
+template <bool SEL>
+__device__ __forceinline__ void i8h_unit_to_lds(const UnitSrc<SEL>& src, bool real, uint8_t* dst, int lane) {
     typedef const __attribute__((address_space(1))) void* gptr;
     typedef __attribute__((address_space(3))) void* lptr;
-    const uint8_t* lane_src = src + (real ? lane * 16 : 0);
-    const int step = real ? 1024 : 0;
+    constexpr int kRun = 4 * row_bytes_of(kRowI8H);
 #pragma unroll
-    for (int n = 0; n < 4; ++n)
-        __builtin_amdgcn_global_load_lds((gptr)(lane_src + n * step), (lptr)(dst + n * 1024), 16, 0, 0);
-    if (lane < 16) __builtin_amdgcn_global_load_lds((gptr)(lane_src + 4 * step), (lptr)(dst + 4096), 16, 0, 0);
+    for (int n = 0; n < 4; ++n) {
+        const uint8_t* a = real ? unit_piece<SEL, kRun>(src, n * 1024 + lane * 16) : src.run[0];
+        __builtin_amdgcn_global_load_lds((gptr)a, (lptr)(dst + n * 1024), 16, 0, 0);
+    }
+    if (lane < 16) {
+        const uint8_t* a = real ? unit_piece<SEL, kRun>(src, 4096 + lane * 16) : src.run[0];
+        __builtin_amdgcn_global_load_lds((gptr)a, (lptr)(dst + 4096), 16, 0, 0);
+    }
 }
 
-template <bool STEP, bool DESC = false>
+// SEL: an iteration's 16 rows are four listed 4-cell blocks (see decode_attn_mfma_kernel); the
+// work is planned for max_ids blocks, a work-group past the end of the list has nothing to do.
+template <bool STEP, bool DESC = false, bool SEL = false>
 __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const AttnKernelParams P) {
+    static_assert(!(STEP && SEL), "the fused step attends the dense selection");
     // slot 0 and slot 1 of the four waves; the fold staging of the epilogue reuses their memory
     __shared__ __attribute__((aligned(16))) uint8_t ring[2 * kWaves * kI8hSlot];
     static_assert(sizeof(MfmaFoldLds) <= sizeof(ring), "fold staging must fit the slots");
@@ -472,11 +520,17 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
     const int split = rem / P.n_kv;
     const int kvh = rem - split * P.n_kv;
     const int wg = unit;
-    const int n_pages = pos / kPage + 1;
+    const block_table_ptr bt = (block_table_ptr)(uintptr_t)(P.tables + (size_t)row * (size_t)P.max_pages_per_seq);
+    uint32_t n_sel = 0;
+    sel_list_ptr sel = nullptr;
+    if constexpr (SEL) {
+        n_sel = min(((sel_list_ptr)(uintptr_t)P.counts)[e], (uint32_t)P.max_ids);
+        sel = (sel_list_ptr)(uintptr_t)(P.ids + (size_t)e * (size_t)P.id_stride);
+    }
+    // loop iterations of this entry: pages, or groups of four selected blocks
+    const int n_pages = SEL ? (int)((n_sel + 3u) >> 2) : pos / kPage + 1;
     const int pg0 = split * pps;
     const int pg1 = min(pg0 + pps, n_pages);
-    typedef const __attribute__((address_space(4))) int32_t* table_ptr;
-    const table_ptr bt = (table_ptr)(uintptr_t)(P.tables + (size_t)row * (size_t)P.max_pages_per_seq);
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
@@ -494,10 +548,32 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
     const auto unit_off = [&](int i) -> size_t {
         return (size_t)bt[min(pg0 + wave + kWaves * i, pg1 - 1)] * page_bytes + head_off;
     };
-    i8h_unit_to_lds(P.kpool + unit_off(0), n_steps > 0, slot0, lane);
-    i8h_unit_to_lds(P.vpool + unit_off(0), n_steps > 0, slot0 + kI8hUnit, lane);
-    i8h_unit_to_lds(P.kpool + unit_off(1), n_steps > 1, slot1, lane);
-    i8h_unit_to_lds(P.vpool + unit_off(1), n_steps > 1, slot1 + kI8hUnit, lane);
+    // the K and the V unit of step i (both pools have the same geometry in this layout)
+    const auto unit_src = [&](int i, const uint8_t* pool, UnitSrc<SEL>& u) {
+        if constexpr (SEL) {
+            if (i < n_steps) {
+                uint32_t id[4];
+                size_t off[4];
+                listed_blocks(sel, n_sel, bt, pg0 + wave + kWaves * i, pos, page_bytes, head_off, kRow, id, off);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) u.run[j] = pool + off[j];
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) u.run[j] = pool;
+            }
+        } else {
+            u.run[0] = pool + (n_steps > 0 ? unit_off(i) : 0);
+        }
+    };
+    const auto request = [&](int i, const uint8_t* pool, uint8_t* dst) {
+        UnitSrc<SEL> u;
+        unit_src(i, pool, u);
+        i8h_unit_to_lds<SEL>(u, i < n_steps, dst, lane);
+    };
+    request(0, P.kpool, slot0);
+    request(0, P.vpool, slot0 + kI8hUnit);
+    request(1, P.kpool, slot1);
+    request(1, P.vpool, slot1 + kI8hUnit);
 
     half8 qhi[8], qlo[8];
     load_q_fragments(P, e, kvh, c, g, qhi, qlo);
@@ -545,7 +621,19 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
         const int pg = pg0 + wave + kWaves * i;
         const uint8_t* ks = slot;
         const uint8_t* vs = slot + kI8hUnit;
-        const size_t off_next = unit_off(i + 2);
+        // which of the lane's four cells are attended: up to `pos`, or the live cells of listed blocks
+        bool live[4];
+        if constexpr (SEL) {
+            uint32_t id[4];
+            size_t unused[4];
+            listed_blocks(sel, n_sel, bt, pg, pos, page_bytes, head_off, kRow, id, unused);
+            const uint32_t mine = pick4(id, g);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) live[r] = block_cell_live(mine, r, pos);
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) live[r] = pg * kPage + 4 * g + r <= pos;
+        }
 
         // ---- scores: per block, codes . q on the matrix core, then the block's scale ----------------
         __builtin_amdgcn_s_waitcnt(0x0F7F);  // vmcnt(15): this page's K unit has landed
@@ -581,7 +669,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
 #pragma unroll
             for (int r = 0; r < 4; ++r) s[r] = fmaf((float)ksc[r][m], part[r], s[r]);
         }
-        i8h_unit_to_lds(P.kpool + off_next, i + 2 < n_steps, slot, lane);
+        request(i + 2, P.kpool, slot);
 
         // ---- this page's V fragments are requested before the softmax, whose chain of dependent
         // instructions then has the dequantisation to overlap with -----------------------------------
@@ -608,18 +696,20 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
         float pm = -INFINITY;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const bool live = pg * kPage + 4 * g + r <= pos;
-            t4[r] = live ? s[r] * P.scale_log2e : -INFINITY;
+            t4[r] = live[r] ? s[r] * P.scale_log2e : -INFINITY;
             pm = fmaxf(pm, t4[r]);
         }
         pm = max_over_lane_groups(pm);
-        const float m_new = fmaxf(m_run, pm);  // finite: every page of a range holds a live cell
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        // dense: finite, every page of a range holds a live cell; a group of listed blocks may be dead
+        // as a whole, and exp2(-inf - -inf) would be NaN
+        const float m_new = fmaxf(m_run, pm);
+        const bool none_yet = SEL && m_new == -INFINITY;
+        const float alpha = none_yet ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
         float p[4];
         float psum = 0.0f;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            p[r] = __builtin_amdgcn_exp2f(t4[r] - m_new);
+            p[r] = none_yet ? 0.0f : __builtin_amdgcn_exp2f(t4[r] - m_new);
             psum += p[r];
         }
         l_run = l_run * alpha + psum;
@@ -641,13 +731,13 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
         const half8 phh = half8{phi[0], phi[1], phi[2], phi[3], phi[0], phi[1], phi[2], phi[3]};
         const half8 pll = half8{plo[0], plo[1], plo[2], plo[3], plo[0], plo[1], plo[2], plo[3]};
         // ---- P.V: dequantise into the exact (hi, lo) pair, two 32-deep MFMAs per 16 columns ---------------
-        const bool last_page = pg == n_pages - 1;
+        const bool last_page = SEL || pg == n_pages - 1;
         if (last_page || __builtin_amdgcn_ballot_w64(has_zero_exponent(v_screen)) != 0) {
 #pragma unroll
             for (int h = 0; h < 2; ++h)
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
-                    if ((vsb[h][r] & 0x7c00u) == 0 || pg * kPage + 4 * g + r > pos) vsb[h][r] = 0;
+                    if ((vsb[h][r] & 0x7c00u) == 0 || !live[r]) vsb[h][r] = 0;
         }
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
@@ -683,7 +773,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
                 o[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahl, pll, o[h][t], 0, 0, 0);
             }
         }
-        i8h_unit_to_lds(P.vpool + off_next, i + 2 < n_steps, slot + kI8hUnit, lane);
+        request(i + 2, P.vpool, slot + kI8hUnit);
     };
 
     for (int i = 0; i < n_steps; ++i) one_page((i & 1) ? slot1 : slot0, i);
@@ -718,32 +808,43 @@ constexpr int kQ8vUnit = kPage * kQ8vRow;      // 4608
 // fragment read touches spread over the banks.
 constexpr int kQ8vKStep = 1024 + 32;
 constexpr int kQ8vKSlot = 8 * kQ8vKStep;  // 8448
-__device__ __forceinline__ void q8v_k_unit_to_lds(const uint8_t* src, bool real, uint8_t* dst, int lane) {
+template <bool SEL>
+__device__ __forceinline__ void q8v_k_unit_to_lds(const UnitSrc<SEL>& src, bool real, uint8_t* dst, int lane) {
     typedef const __attribute__((address_space(1))) void* gptr;
     typedef __attribute__((address_space(3))) void* lptr;
-    const uint8_t* lane_src = src + (real ? lane * 16 : 0);
-    const int step = real ? 1024 : 0;
 #pragma unroll
-    for (int n = 0; n < 8; ++n)
-        __builtin_amdgcn_global_load_lds((gptr)(lane_src + n * step), (lptr)(dst + n * kQ8vKStep), 16, 0, 0);
+    for (int n = 0; n < 8; ++n) {
+        // instruction n moves rows 2 n and 2 n + 1: of a selection list, half of block n / 2
+        const uint8_t* a = !real ? src.run[0]
+                           : SEL ? src.run[SEL ? n >> 1 : 0] + (n & 1) * 1024 + lane * 16
+                                 : src.run[0] + n * 1024 + lane * 16;
+        __builtin_amdgcn_global_load_lds((gptr)a, (lptr)(dst + n * kQ8vKStep), 16, 0, 0);
+    }
 }
 
 // 4608 bytes = 4 x 1024 + 512: four full instructions and one of 32 lanes.  `real` false issues the
 // same five instructions on one 16-byte location (the data is never used): the number of loads
 // in flight, which the waits count, then does not depend on where in its range a wave is.
-__device__ __forceinline__ void q8v_unit_to_lds(const uint8_t* src, bool real, uint8_t* dst, int lane) {
+template <bool SEL>
+__device__ __forceinline__ void q8v_unit_to_lds(const UnitSrc<SEL>& src, bool real, uint8_t* dst, int lane) {
     typedef const __attribute__((address_space(1))) void* gptr;
     typedef __attribute__((address_space(3))) void* lptr;
-    const uint8_t* lane_src = src + (real ? lane * 16 : 0);
-    const int step = real ? 1024 : 0;
+    constexpr int kRun = 4 * kQ8vRow;
 #pragma unroll
-    for (int n = 0; n < 4; ++n)
-        __builtin_amdgcn_global_load_lds((gptr)(lane_src + n * step), (lptr)(dst + n * 1024), 16, 0, 0);
-    if (lane < 32) __builtin_amdgcn_global_load_lds((gptr)(lane_src + 4 * step), (lptr)(dst + 4096), 16, 0, 0);
+    for (int n = 0; n < 4; ++n) {
+        const uint8_t* a = real ? unit_piece<SEL, kRun>(src, n * 1024 + lane * 16) : src.run[0];
+        __builtin_amdgcn_global_load_lds((gptr)a, (lptr)(dst + n * 1024), 16, 0, 0);
+    }
+    if (lane < 32) {
+        const uint8_t* a = real ? unit_piece<SEL, kRun>(src, 4096 + lane * 16) : src.run[0];
+        __builtin_amdgcn_global_load_lds((gptr)a, (lptr)(dst + 4096), 16, 0, 0);
+    }
 }
 
-template <bool STEP, bool DESC = false>
+// SEL: an iteration's 16 rows are four listed 4-cell blocks, as in the int8 kernel.
+template <bool STEP, bool DESC = false, bool SEL = false>
 __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const AttnKernelParams P) {
+    static_assert(!(STEP && SEL), "the fused step attends the dense selection");
     // per wave one K slot and two V slots during the loop, the fold staging after it
     constexpr int kWaveLds = kQ8vKSlot + 2 * kQ8vUnit;
     constexpr int kLds = kWaves * kWaveLds > (int)sizeof(MfmaFoldLds) ? kWaves * kWaveLds : (int)sizeof(MfmaFoldLds);
@@ -755,11 +856,16 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
     const int split = rem / P.n_kv;
     const int kvh = rem - split * P.n_kv;
     const int wg = unit;
-    const int n_pages = pos / kPage + 1;
+    const block_table_ptr bt = (block_table_ptr)(uintptr_t)(P.tables + (size_t)row * (size_t)P.max_pages_per_seq);
+    uint32_t n_sel = 0;
+    sel_list_ptr sel = nullptr;
+    if constexpr (SEL) {
+        n_sel = min(((sel_list_ptr)(uintptr_t)P.counts)[e], (uint32_t)P.max_ids);
+        sel = (sel_list_ptr)(uintptr_t)(P.ids + (size_t)e * (size_t)P.id_stride);
+    }
+    const int n_pages = SEL ? (int)((n_sel + 3u) >> 2) : pos / kPage + 1;
     const int pg0 = split * pps;
     const int pg1 = min(pg0 + pps, n_pages);
-    typedef const __attribute__((address_space(4))) int32_t* table_ptr;
-    const table_ptr bt = (table_ptr)(uintptr_t)(P.tables + (size_t)row * (size_t)P.max_pages_per_seq);
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
@@ -782,11 +888,38 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
     // i there is V(i+1) = 5 loads; behind V(i) where step i needs it there are K(i), V(i+1), K(i+1)
     // = 8 + 5 + 8.  Steps that do not exist are requested all the same, as loads of one location,
     // so that these counts hold everywhere.
-    const auto k_unit = [&](int i) { return P.kpool + phys(i) * k_page_bytes + k_head_off; };
-    const auto v_unit = [&](int i) { return P.vpool + phys(i) * v_page_bytes + v_head_off; };
-    q8v_unit_to_lds(v_unit(0), n_steps > 0, slots, lane);
-    q8v_k_unit_to_lds(k_unit(0), n_steps > 0, kslot, lane);
-    q8v_unit_to_lds(v_unit(1), n_steps > 1, slots + kQ8vUnit, lane);
+    const auto unit_src = [&](int i, bool is_k, UnitSrc<SEL>& u) {
+        const uint8_t* pool = is_k ? P.kpool : P.vpool;
+        if constexpr (SEL) {
+            if (i < n_steps) {
+                uint32_t id[4];
+                size_t off[4];
+                listed_blocks(sel, n_sel, bt, pg0 + wave + kWaves * i, pos, is_k ? k_page_bytes : v_page_bytes,
+                              is_k ? k_head_off : v_head_off, is_k ? kHd * 2 : kQ8vRow, id, off);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) u.run[j] = pool + off[j];
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) u.run[j] = pool;
+            }
+        } else {
+            u.run[0] = n_steps > 0 ? pool + phys(i) * (is_k ? k_page_bytes : v_page_bytes) + (is_k ? k_head_off : v_head_off)
+                                   : pool;
+        }
+    };
+    const auto request_k = [&](int i) {
+        UnitSrc<SEL> u;
+        unit_src(i, true, u);
+        q8v_k_unit_to_lds<SEL>(u, i < n_steps, kslot, lane);
+    };
+    const auto request_v = [&](int i, uint8_t* dst) {
+        UnitSrc<SEL> u;
+        unit_src(i, false, u);
+        q8v_unit_to_lds<SEL>(u, i < n_steps, dst, lane);
+    };
+    request_v(0, slots);
+    request_k(0);
+    request_v(1, slots + kQ8vUnit);
 
     half8 qhi[8], qlo[8];
     load_q_fragments(P, e, kvh, c, g, qhi, qlo);
@@ -849,7 +982,21 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
     for (int i = 0; i < n_steps; ++i) {
         const int pg = pg0 + wave + kWaves * i;
         const uint8_t* vs = slots + (i & 1) * kQ8vUnit;
-        const int behind = n_steps - 1 - i;  // steps after this one
+        bool live[4];       // the lane's cells 4 g + r
+        bool live_mine;     // cell 4 g + c % 4
+        if constexpr (SEL) {
+            uint32_t id[4];
+            size_t unused[4];
+            listed_blocks(sel, n_sel, bt, pg, pos, k_page_bytes, k_head_off, kHd * 2, id, unused);
+            const uint32_t mine = pick4(id, g);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) live[r] = block_cell_live(mine, r, pos);
+            live_mine = block_cell_live(mine, c & 3, pos);
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) live[r] = pg * kPage + 4 * g + r <= pos;
+            live_mine = pg * kPage + 4 * g + (c & 3) <= pos;
+        }
 
         // ---- S^T = K . q^T: four independent accumulation chains ------------------------------
         __builtin_amdgcn_s_waitcnt(0x0F75);  // vmcnt(5): this page's K unit has landed
@@ -875,7 +1022,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
             s3 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kb, qlo[m + 1], s3, 0, 0, 0);
         }
         const f4 s = (s0 + s1) + (s2 + s3);  // s[r] = q[head c] . k[cell 4 g + r]
-        q8v_k_unit_to_lds(k_unit(i + 1), behind >= 1, kslot, lane);
+        request_k(i + 1);
 
         // ---- this page's V unit: scales first -------------------------------------------------
         __builtin_amdgcn_s_waitcnt(0x4F75);  // vmcnt(21): K(i), V(i+1), K(i+1) behind V(i)
@@ -884,7 +1031,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
         }
         // lane (c, g): scale of blocks 2 (c / 4), + 1 of row 4 g + c % 4, the row's maximum over the
         // lanes c, c ^ 4, c ^ 8, c ^ 12, then the four rows' maxima from the lanes of the quad
-        const bool last_page = pg == n_pages - 1;
+        const bool last_page = SEL || pg == n_pages - 1;
         float smax;
         {
             const uint8_t* rp = vs + (4 * g + (c & 3)) * kQ8vRow + (c >> 2) * 72;
@@ -892,7 +1039,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
             const float b = *reinterpret_cast<const float*>(rp + 36);
             smax = fmaxf(a, b);
             // rows past `pos` may hold anything: they count as scale 1 here and as zeros below
-            if (last_page && pg * kPage + 4 * g + (c & 3) > pos) smax = 1.0f;
+            if (last_page && !live_mine) smax = 1.0f;
             smax = fmaxf(smax, dpp_mov<0x124>(smax));  // row_ror:4
             smax = fmaxf(smax, dpp_mov<0x128>(smax));  // row_ror:8
         }
@@ -916,20 +1063,22 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
         float pm = -INFINITY;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const bool live = pg * kPage + 4 * g + r <= pos;
-            t4[r] = live ? s[r] * P.scale_log2e : -INFINITY;
+            t4[r] = live[r] ? s[r] * P.scale_log2e : -INFINITY;
             tw[r] = t4[r] + (float)ex[r];
             pm = fmaxf(pm, tw[r]);
         }
         pm = max_over_lane_groups(pm);
-        const float m_new = fmaxf(m_run, pm);  // finite: every page of a range holds a live cell
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        // dense: finite, every page of a range holds a live cell; a group of listed blocks may be dead
+        // as a whole, and exp2(-inf - -inf) would be NaN
+        const float m_new = fmaxf(m_run, pm);
+        const bool none_yet = SEL && m_new == -INFINITY;
+        const float alpha = none_yet ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
         h4m whi, wlo;
         float psum = 0.0f;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const float w = __builtin_amdgcn_exp2f(tw[r] - m_new);
-            psum += __builtin_amdgcn_exp2f(t4[r] - m_new);
+            const float w = none_yet ? 0.0f : __builtin_amdgcn_exp2f(tw[r] - m_new);
+            psum += none_yet ? 0.0f : __builtin_amdgcn_exp2f(t4[r] - m_new);
             _Float16 hi, lo;
             split_hi_lo(w, hi, lo);
             whi[r] = hi;
@@ -955,7 +1104,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
             for (int r = 0; r < 4; ++r) {
                 const uint8_t* blk = vs + (4 * g + r) * kQ8vRow + (4 * h + my_block) * 36;
                 float sc = *reinterpret_cast<const float*>(blk) * down[r];
-                if (last_page && pg * kPage + 4 * g + r > pos) sc = 0.0f;
+                if (last_page && !live[r]) sc = 0.0f;
                 split_hi_lo(sc, shi[r], slo[r]);
                 const unsigned* cw = reinterpret_cast<const unsigned*>(blk + 4 + (c & 3) * 8);
                 wx[r] = cw[0] ^ 0x80808080u;
@@ -982,7 +1131,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
                 o[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahl, wll, o[h][t], 0, 0, 0);
             }
         }
-        q8v_unit_to_lds(v_unit(i + 2), behind >= 2, slots + (i & 1) * kQ8vUnit, lane);
+        request_v(i + 2, slots + (i & 1) * kQ8vUnit);
     }
 
     // no load may still be on its way into the slots when the fold staging takes their place
@@ -1020,11 +1169,15 @@ hipError_t launch_decode_attn_mfma(const AttnKernelParams& kp, int layout, bool 
     if (layout == BKV_LAYOUT_I8H) {
         if (step)
             launch_one(decode_attn_mfma_i8h_kernel<true>, kp, total, stream, start, stop);
+        else if (sel)
+            launch_one(decode_attn_mfma_i8h_kernel<false, false, true>, kp, total, stream, start, stop);
         else
             launch_one(decode_attn_mfma_i8h_kernel<false>, kp, total, stream, start, stop);
     } else if (layout == BKV_LAYOUT_Q8V) {
         if (step)
             launch_one(decode_attn_mfma_q8v_kernel<true>, kp, total, stream, start, stop);
+        else if (sel)
+            launch_one(decode_attn_mfma_q8v_kernel<false, false, true>, kp, total, stream, start, stop);
         else
             launch_one(decode_attn_mfma_q8v_kernel<false>, kp, total, stream, start, stop);
     } else if (step)
