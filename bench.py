@@ -51,7 +51,7 @@ def attn_algorithmic_bytes(ctx_after: list[int], row_bytes: int = ROW_BYTES) -> 
 
 
 def build_batched(pool_mod, rng, n_seqs: int, lo: int, hi: int, n_layers: int, occupancy: float,
-                  layout: int = 0, attn_valu: bool = False):
+                  layout: int = 0):
     from breccia_amd.kv import Pool
 
     ctx = []
@@ -63,7 +63,7 @@ def build_batched(pool_mod, rng, n_seqs: int, lo: int, hi: int, n_layers: int, o
     live_pages = sum((c + PAGE) // PAGE + 1 for c in ctx)
     n_pages = int(np.ceil(live_pages / occupancy))
     pool = Pool(n_layers=n_layers, n_pages=n_pages, n_kv_head=N_KV, head_dim=HD, max_seqs=n_seqs + 1,
-                max_pages_per_seq=max(ctx) // PAGE + 64, layout=layout, attn_valu=attn_valu)
+                max_pages_per_seq=max(ctx) // PAGE + 64, layout=layout)
     pool.set_free_order(rng.permutation(n_pages).astype(np.int32))
     seqs = [pool.seq_create() for _ in ctx]
     # deal the shuffled pages round-robin: one page per sequence per turn
@@ -324,7 +324,7 @@ def main() -> int:
 
     if not args.no_extra:
         extra.update(bench_batch1(stream, check=not args.no_cpu))
-        extra.update(bench_valu_formulation(stream))
+        extra.update(bench_head_counts(stream))
         extra.update(bench_quantised(stream))
         extra.update(bench_select(stream))
         extra.update(bench_prefill(stream))
@@ -467,46 +467,44 @@ def bench_quantised(stream) -> dict:
     return res
 
 
-def bench_valu_formulation(stream) -> dict:
-    """The headline batch with f16 decode attention in the VALU formulation (pool flag
-    BKV_POOL_ATTN_VALU), at 16 and at the reference model's 24 q heads, beside the MFMA one."""
+def bench_head_counts(stream) -> dict:
+    """The headline batch through bkv_decode_attn (no append) at 16 q heads and at the reference
+    model's 24: every head of a kv head shares one pass over the K/V rows."""
     from breccia_amd import lib as L
     from breccia_amd.kv import DeviceBuffer
 
     res = {}
-    for valu in (False, True):
-        rng = np.random.Generator(np.random.PCG64(20250003))
-        pool, seqs, ctx = build_batched(None, rng, 8, 1024, 32768, 4, 0.6, attn_valu=valu)
-        kd = DeviceBuffer.from_numpy(rng.standard_normal((8192, N_KV, HD), dtype=np.float32))
-        for layer in range(4):
-            for s, c in zip(seqs, ctx):
-                for at in range(0, c, 8192):
-                    pool.append(layer, [s], [at], [min(8192, c - at)], kd, kd, stream)
+    rng = np.random.Generator(np.random.PCG64(20250003))
+    pool, seqs, ctx = build_batched(None, rng, 8, 1024, 32768, 4, 0.6)
+    kd = DeviceBuffer.from_numpy(rng.standard_normal((8192, N_KV, HD), dtype=np.float32))
+    for layer in range(4):
+        for s, c in zip(seqs, ctx):
+            for at in range(0, c, 8192):
+                pool.append(layer, [s], [at], [min(8192, c - at)], kd, kd, stream)
+    stream.sync()
+    kd.free()
+    pos = [c - 1 for c in ctx]
+    b = attn_algorithmic_bytes(ctx)
+    for n_q in (16, 24):
+        q = DeviceBuffer.from_numpy(rng.standard_normal((8, n_q, HD), dtype=np.float32))
+        out = DeviceBuffer(8 * n_q * HD * 4)
+        for i in range(200):
+            pool.decode_attn(i % 4, seqs, pos, n_q, q, out, 1.0 / 16.0, stream=stream)
         stream.sync()
-        kd.free()
-        pos = [c - 1 for c in ctx]
-        b = attn_algorithmic_bytes(ctx)
-        for n_q in (16, 24):
-            q = DeviceBuffer.from_numpy(rng.standard_normal((8, n_q, HD), dtype=np.float32))
-            out = DeviceBuffer(8 * n_q * HD * 4)
-            for i in range(200):
-                pool.decode_attn(i % 4, seqs, pos, n_q, q, out, 1.0 / 16.0, stream=stream)
-            stream.sync()
-            pool.timing_reset()
-            pool.timing_enable(True)
-            for i in range(100):
-                pool.decode_attn(i % 4, seqs, pos, n_q, q, out, 1.0 / 16.0, stream=stream)
-            stream.sync()
-            pool.timing_enable(False)
-            n, ms = pool.timing_read(L.STAGE_ATTN_SPLIT)
-            us = ms / max(n, 1) * 1e3
-            res["%s_%dq" % ("valu" if valu else "mfma", n_q)] = {
-                "attn_split_us": round(us, 2), "split_GBps": round(b / us / 1e3, 1),
-                "frac_of_hbm_peak": round(b / us / 1e3 / HBM_PEAK_GBPS, 4)}
-            q.free()
-            out.free()
-        pool.destroy()
-    return {"attn_formulations_batch8": res}
+        pool.timing_reset()
+        pool.timing_enable(True)
+        for i in range(100):
+            pool.decode_attn(i % 4, seqs, pos, n_q, q, out, 1.0 / 16.0, stream=stream)
+        stream.sync()
+        pool.timing_enable(False)
+        n, ms = pool.timing_read(L.STAGE_ATTN_SPLIT)
+        us = ms / max(n, 1) * 1e3
+        res["%dq" % n_q] = {"attn_split_us": round(us, 2), "split_GBps": round(b / us / 1e3, 1),
+                            "frac_of_hbm_peak": round(b / us / 1e3 / HBM_PEAK_GBPS, 4)}
+        q.free()
+        out.free()
+    pool.destroy()
+    return {"attn_head_counts_batch8": res}
 
 
 def bench_select(stream) -> dict:

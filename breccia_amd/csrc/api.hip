@@ -883,22 +883,17 @@ static bkv_status decode_attn_common(bkv_pool* p, int32_t layer, int32_t n, cons
     if (select && (!ids_dev || !counts_dev || ((uintptr_t)ids_dev & 3u) || ((uintptr_t)counts_dev & 3u)))
         return fail(BKV_ERR_INVALID, "decode_attn_select: ids/counts device pointers must be "
                                      "non-NULL and 4-byte aligned");
-    const bool mfma = attn_on_mfma(p, n_q_head / p->g.n_kv, !select);
-    if (step && !mfma && p->g.layout != BKV_LAYOUT_F16)
-        return fail(BKV_ERR_INVALID, "decode_step on a quantised pool is served by the matrix-core kernels "
-                                     "only (at most 16 q heads per kv head, pool without "
-                                     "BKV_POOL_ATTN_VALU); append and attend in two calls instead");
     // the cut into work-groups comes before anything is enqueued: a batch it cannot serve is an
     // error like any other size violation
     const int32_t ws_wgs = static_ws ? kStaticWgs : p->max_wgs;
-    if (plan_attn(p, n_q_head, b, select ? (max_ids + 3) / 4 : 0, mfma, ws_wgs) < 0)
+    if (plan_attn(p, n_q_head, b, select ? (max_ids + 3) / 4 : 0, ws_wgs) < 0)
         return fail(BKV_ERR_INVALID,
                     sfmt(static_ws ? "decode_attn_static: %lld entries x %lld kv heads need more work-groups than "
                                      "the static scratch holds (%lld); use smaller batches or bkv_decode_attn"
                                    : "decode_attn: %lld entries x %lld kv heads need more work-groups than the "
                                      "partial-result workspace holds (%lld); use smaller batches",
                          n, p->g.n_kv,
-                         attn_plan_limits(p->n_cu, ws_wgs, p->g.n_kv, n_q_head / p->g.n_kv, mfma).max_wgs));
+                         attn_plan_limits(p->n_cu, ws_wgs, p->g.n_kv, n_q_head / p->g.n_kv).max_wgs));
     AttnArgs a;
     if (static_ws) {
         if (!attn_static_scratch(p->device, &a.ws_o, &a.ws_ml))
@@ -907,7 +902,6 @@ static bkv_status decode_attn_common(bkv_pool* p, int32_t layer, int32_t n, cons
     }
     st = flush_tables(p, S(stream));
     if (st != BKV_OK) return st;
-    a.mfma = mfma;
     a.n_q_head = n_q_head;
     a.q = q_dev;
     a.gate = gate_dev;
@@ -937,8 +931,7 @@ static bkv_status decode_attn_common(bkv_pool* p, int32_t layer, int32_t n, cons
 }
 
 bkv_status bkv_attn_plan(int32_t n_cu, int32_t n_kv_head, int32_t n_q_head, int32_t n, const int64_t* pos,
-                         int32_t sel_groups, int32_t matrix_cores, int32_t* splits_out, int32_t* pps_out,
-                         int32_t* total_out) {
+                         int32_t sel_groups, int32_t* splits_out, int32_t* pps_out, int32_t* total_out) {
     if (n_cu <= 0 || n_kv_head <= 0 || n_kv_head > BKV_MAX_KV_HEAD)
         return fail(BKV_ERR_INVALID, sfmt("attn_plan: %lld compute units, %lld kv heads", n_cu, n_kv_head));
     if (n_q_head <= 0 || n_q_head % n_kv_head != 0 || n_q_head / n_kv_head > BKV_MAX_HEAD_GROUP)
@@ -954,7 +947,7 @@ bkv_status bkv_attn_plan(int32_t n_cu, int32_t n_kv_head, int32_t n_q_head, int3
             return fail(BKV_ERR_RANGE, sfmt("attn_plan: position %lld of entry %lld", pos[i], i));
         b.pos[i] = (int32_t)pos[i];
     }
-    const AttnPlanLimits lim = attn_plan_limits(n_cu, kMaxWgs, n_kv_head, n_q_head / n_kv_head, matrix_cores != 0);
+    const AttnPlanLimits lim = attn_plan_limits(n_cu, kMaxWgs, n_kv_head, n_q_head / n_kv_head);
     const int32_t total = plan_attn_ranges(lim, 16, sel_groups, b);
     if (total < 0)
         return fail(BKV_ERR_INVALID, sfmt("attn_plan: %lld entries x %lld kv heads need more work-groups than "
@@ -1041,9 +1034,7 @@ bkv_status bkv_step_plan_create(bkv_pool* p, int32_t n, const int32_t* seqs, con
     bkv_status st = need_device(p);
     if (st != BKV_OK) return st;
     const int32_t group = n_q_head / p->g.n_kv;
-    if (!attn_on_mfma(p, group, true))
-        return fail(BKV_ERR_INVALID, "step_plan_create: step plans are served by the matrix-core kernels");
-    const AttnPlanLimits lim = attn_plan_limits(p->n_cu, p->max_wgs, p->g.n_kv, group, true);
+    const AttnPlanLimits lim = attn_plan_limits(p->n_cu, p->max_wgs, p->g.n_kv, group);
     if (plan_attn_ranges(lim, p->g.page_cells, 0, host.b) < 0)
         return fail(BKV_ERR_INVALID, sfmt("step_plan_create: %lld entries x %lld kv heads need more work-groups "
                                           "than the partial-result workspace holds (%lld)", n, p->g.n_kv,
@@ -1115,7 +1106,6 @@ bkv_status bkv_step_plan_decode(bkv_step_plan* pl, int32_t layer, const float* k
     AttnBatch b{};
     b.n = pl->n;
     AttnArgs a;
-    a.mfma = true;
     a.n_q_head = pl->n_q_head;
     a.q = q_dev;
     a.gate = gate_dev;

@@ -214,7 +214,6 @@ struct AttnArgs {
     // fused decode step: new rows [n][n_kv][head_dim] f32; nullptr = plain attention
     const float* new_k = nullptr;
     const float* new_v = nullptr;
-    bool mfma = false;  // dense f16 call routed to the MFMA kernel (all heads of a group at once)
     // partial-result workspace other than the pool's own (the static device scratch); nullptr = the pool's
     float* ws_o = nullptr;
     float* ws_ml = nullptr;
@@ -237,14 +236,12 @@ hipError_t launch_step_advance(StepDesc* d, const AttnPlanLimits& lim, int32_t p
 // Fills wg_base/splits/pps from row/pos (attn_plan.hpp); returns the total work-group count, -1
 // when the batch cannot be cut into as few work-groups as the workspace holds.  sel_groups > 0:
 // every entry is planned for that many groups of four selected blocks instead of its pages.
-AttnPlanLimits attn_plan_limits(int32_t n_cu, int32_t max_wgs, int32_t n_kv, int32_t group, bool mfma);
-int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b, int32_t sel_groups = 0,
-                  bool mfma = false, int32_t max_wgs = 0);
+AttnPlanLimits attn_plan_limits(int32_t n_cu, int32_t max_wgs, int32_t n_kv, int32_t group);
+int32_t plan_attn(const bkv_pool* p, int32_t n_q_head, AttnBatch& b, int32_t sel_groups = 0, int32_t max_wgs = 0);
 // The static device scratch of bkv_decode_attn_static: looked up once per device (which must be
 // the current one) at pool creation; false from the accessor when that has not happened.
 hipError_t attn_static_scratch_init(int device);
 bool attn_static_scratch(int device, float** o, float** ml);
-bool attn_on_mfma(const bkv_pool* p, int32_t group, bool dense);
 hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, const AttnArgs& a,
                               hipStream_t stream);
 // Prefill attention (prefill_attn.hip): one entry per sequence chunk.
@@ -259,8 +256,6 @@ struct PrefillBatch {
 int32_t prefill_rows_per_wg(int32_t layout);  // query rows one work-group owns
 hipError_t launch_prefill_attn(bkv_pool* p, int32_t layer, const PrefillBatch& b, const AttnArgs& a,
                                hipStream_t stream);
-// heads one wave carries for a given q-heads-per-kv-head group
-int32_t attn_heads_per_wave(int32_t group);
 
 hipError_t launch_page_copy(bkv_pool* p, const bkv_page_pair* pairs_dev, int32_t n_pairs,
                             hipStream_t stream);

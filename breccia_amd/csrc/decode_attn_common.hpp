@@ -28,16 +28,16 @@ struct AttnKernelParams {
     float* part_o;
     float* part_ml;
     int32_t max_pages_per_seq;
-    int32_t n_kv, n_q, group, n_hc;
+    int32_t n_kv, n_q, group;
     float scale_log2e;
-    // selection lists (decode_attn_kernel<..., true> only): entry e attends the 4-cell blocks
+    // selection lists (kernels instantiated with SEL only): entry e attends the 4-cell blocks
     // ids[e * id_stride + 0 .. min(counts[e], max_ids))
     const uint32_t* ids;
     const uint32_t* counts;
     int64_t id_stride;
     int32_t max_ids;
-    // fused decode step (decode_attn_kernel<..., STEP = true> only): the K/V row of cell pos of
-    // entry e comes from new_k / new_v [n][n_kv][head_dim] f32 and is stored into the pool on the way
+    // fused decode step (kernels instantiated with STEP only): the K/V row of cell pos of entry e
+    // comes from new_k / new_v [n][n_kv][head_dim] f32 and is stored into the pool on the way
     const float* new_k;
     const float* new_v;
     uint8_t* kpool_w;

@@ -1,6 +1,6 @@
-// Paged decode attention for gfx950 on the matrix cores: the split-K kernels for f16 pools, for
-// int8 K/V with f16 block scales and for f16 K + q8_0 V.  Same work decomposition, partial layout
-// and merge kernel as the VALU formulation in decode_attn.hip; must agree with the reference's
+// Paged decode attention for gfx950: the split-K online-softmax kernels, on the matrix cores, for
+// f16 pools, for int8 K/V with f16 block scales and for f16 K + q8_0 V.  The cut into work-groups,
+// the merge kernel and the launch are in decode_attn.hip; results must agree with the reference's
 // f64 CPU attend (crates/breccia-kernels/src/qsa/cpu.rs:197-246).
 #include <hip/hip_ext.h>
 
@@ -15,18 +15,20 @@ namespace bkv {
 namespace {
 
 // ---- decode attention on the matrix cores -----------------------------------------------------
-// The same split-K decomposition and the same partial-result layout as decode_attn_kernel, for
-// f16 pools and head groups the 8- or 4-head VALU kernel would have to walk in several chunks
-// (the reference's own 24 q / 2 kv heads = 12 per group; 32 / 2 = 16): a 16-column MFMA tile
-// holds up to 16 heads of a kv head at once, every K/V row is still read once, and the VALU
+// Decode attention is an HBM-bound stream (every K/V row is read once and used by the `group` q
+// heads of its kv head), but at the edge of the HBM roofline a formulation that multiplies on the
+// VALU is co-limited by instruction issue -- and has to walk the rows once per chunk of 8 or 4
+// heads (the reference's own 24 q / 2 kv heads = 12 per group).  A 16-column MFMA tile holds up
+// to 16 heads of a kv head at once, every K/V row is read once whatever the group, and the VALU
 // only does the softmax.  Lane (c = lane % 16, g = lane / 16) of a wave owns head c; per page:
 //   S^T[cell][head] = K[cell][:] . q[head][:]          v_mfma_f32_16x16x32_f16, A = K, B = q
 //   O^T[d][head]   += V^T[d][cell] . P^T[cell][head]   v_mfma_f32_16x16x32_f16, A = V regrouped
 // with q and p split into a high and a low f16 part (K and V are exact f16), as in the prefill
 // kernel: two MFMAs per K fragment, and for P.V one MFMA whose 32-deep contraction runs over the
-// page's 16 cells twice, against p's high parts and against its low parts.  K fragment m of a lane is the 16 bytes at element 32 m + 8 g of row c; V fragments
-// are the 16 bytes at element 128 h + 8 c of rows 4 g + r.  Every fragment register is
-// refilled with the next page's data right after its last use.
+// page's 16 cells twice, against p's high parts and against its low parts.  K fragment m of a
+// lane is the 16 bytes at element 32 m + 8 g of row c; V fragments are the 16 bytes at element
+// 128 h + 8 c of rows 4 g + r.  Every fragment register is refilled with the next page's data
+// right after its last use.
 typedef _Float16 h4m __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ void split_hi_lo(float x, _Float16& hi, _Float16& lo) {
@@ -139,10 +141,9 @@ __device__ __forceinline__ void k_pair_home(const v4u& lo_rows, const v4u& hi_ro
 }
 
 // STEP: the row of cell pos comes from the caller's f32 K/V (stored under the f16 rule into the
-// pool on the way), as in decode_attn_kernel<..., STEP = true>.
-// SEL: the 16 rows of an iteration are four listed 4-cell blocks instead of a page, as in
-// decode_attn_kernel<..., SEL = true> (block g supplies the V rows of lane group g, block c / 4
-// the K row of lane c).
+// pool on the way): the pool ends up as bkv_append would leave it, the output as append + attend.
+// SEL: the 16 rows of an iteration are four listed 4-cell blocks instead of a page (block g
+// supplies the V rows of lane group g, block c / 4 the K row of lane c).
 template <bool STEP, bool SEL = false, bool DESC = false>
 __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnKernelParams P) {
     static_assert(!(STEP && SEL), "the fused step attends the dense selection");
@@ -176,7 +177,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
     const size_t page_bytes = (size_t)P.n_kv * kPage * kHd * 2;
     const size_t head_off = (size_t)kvh * kPage * kHd * 2;
 
-    // Row runs of iteration i (see decode_attn_kernel): a page, or four listed blocks whose ids
+    // Row runs of iteration i: a page, or four listed blocks whose ids
     // are clamped to the blocks at or below `pos` before any address is formed.
     const auto locate = [&](int i, RowRuns<SEL>& rr) {
         if constexpr (SEL) {
@@ -418,8 +419,8 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
 //           scale 2^e * f, so it is a representable f16 number, subnormal at worst); the three
 //           products (hi + lo).(p_hi + p_lo) then carry the result to f32 accuracy.  A lane's 8 columns lie in one block (4 h + c / 4), so it
 //           needs one scale per V row and half.
-// The VALU formulation of this layout is bound by instruction issue (conversions and FMAs, 40 %
-// of the HBM roofline on long contexts); here the VALU only converts and scales.
+// (Multiplied on the VALU, this layout is bound by instruction issue: conversions and FMAs, 40 %
+// of the HBM roofline on long contexts; here the VALU only converts and scales.)
 // whether either f16 of a dword has exponent field 0 (the values the cache reads as zero)
 __device__ __forceinline__ bool has_zero_exponent(unsigned two_halves) {
     const unsigned t = two_halves & 0x7c007c00u;

@@ -73,14 +73,14 @@ def rope_table(freq_base: float, n_rot: int, max_pos: int) -> np.ndarray:
     return out
 
 
-def attn_plan(n_cu: int, n_kv_head: int, n_q_head: int, pos, sel_groups: int = 0, matrix_cores: bool = True):
+def attn_plan(n_cu: int, n_kv_head: int, n_q_head: int, pos, sel_groups: int = 0):
     """How the library would cut a decode-attention batch into work-groups on a device of n_cu
     compute units -> (splits per entry, pages per split, total work-groups).  Host only."""
     pos, pp = _i64(pos)
     splits = np.zeros(max(pos.size, 1), dtype=np.int32)
     pps = np.zeros(max(pos.size, 1), dtype=np.int32)
     total = C.c_int32()
-    check(lib.bkv_attn_plan(n_cu, n_kv_head, n_q_head, pos.size, pp, sel_groups, 1 if matrix_cores else 0,
+    check(lib.bkv_attn_plan(n_cu, n_kv_head, n_q_head, pos.size, pp, sel_groups,
                             splits.ctypes.data_as(C.POINTER(C.c_int32)), pps.ctypes.data_as(C.POINTER(C.c_int32)),
                             C.byref(total)))
     return splits[:pos.size], pps[:pos.size], int(total.value)
@@ -148,11 +148,10 @@ class Pool:
     """bkv_pool handle.  Method names follow the C entry points."""
 
     def __init__(self, n_layers=1, n_pages=512, n_kv_head=2, head_dim=256, page_cells=16,
-                 layout=L.LAYOUT_F16, max_seqs=16, max_pages_per_seq=None, host_only=False,
-                 attn_valu=False):
+                 layout=L.LAYOUT_F16, max_seqs=16, max_pages_per_seq=None, host_only=False):
         if max_pages_per_seq is None:
             max_pages_per_seq = n_pages
-        flags = (L.POOL_HOST_ONLY if host_only else 0) | (L.POOL_ATTN_VALU if attn_valu else 0)
+        flags = L.POOL_HOST_ONLY if host_only else 0
         self.desc = PoolDesc(n_layers, n_pages, n_kv_head, head_dim, page_cells, layout, max_seqs,
                              max_pages_per_seq, flags)
         h = C.c_void_p()

@@ -16,7 +16,6 @@ OK, ERR_INVALID, ERR_RANGE, ERR_NO_PAGES, ERR_STATE, ERR_NO_DEVICE, ERR_HIP, ERR
 STATUS_NAMES = ["OK", "INVALID", "RANGE", "NO_PAGES", "STATE", "NO_DEVICE", "HIP", "NOMEM"]
 LAYOUT_F16, LAYOUT_Q8V, LAYOUT_I8H = 0, 1, 2
 POOL_HOST_ONLY = 1
-POOL_ATTN_VALU = 2
 MAX_BATCH = 64
 MAX_KV_HEAD = 16
 STATIC_WGS = 1024
@@ -101,7 +100,7 @@ _SIGNATURES = {
                                   _vp, _vp]),
     "bkv_decode_attn_static": (C.c_int, [_vp, _i32, _i32, _pi32, _pi64, _i32, _vp, _vp, _i64, _i64, _f32,
                                          _vp, _vp]),
-    "bkv_attn_plan": (C.c_int, [_i32, _i32, _i32, _i32, _pi64, _i32, _i32, _pi32, _pi32, _pi32]),
+    "bkv_attn_plan": (C.c_int, [_i32, _i32, _i32, _i32, _pi64, _i32, _pi32, _pi32, _pi32]),
     "bkv_prefill_attn": (C.c_int, [_vp, _i32, _i32, _pi32, _pi64, _pi32, _i32, _vp, _vp, _i64, _i64, _f32,
                                    _vp, _vp]),
     "bkv_decode_step": (C.c_int, [_vp, _i32, _i32, _pi32, _pi64, _vp, _vp, _i32, _vp, _vp, _i64, _i64, _f32,

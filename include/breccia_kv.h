@@ -52,11 +52,8 @@ typedef enum bkv_layout {
 } bkv_layout;
 
 enum {
-    BKV_POOL_HOST_ONLY = 1u, /* allocator + block tables only; device calls fail with
-                                BKV_ERR_NO_DEVICE (for hosts without a GPU) */
-    BKV_POOL_ATTN_VALU = 2u  /* decode attention in the VALU formulation (chunks of 8 or 4 heads,
-                                no MFMA) instead of the MFMA one; same results, kept for
-                                comparison */
+    BKV_POOL_HOST_ONLY = 1u /* allocator + block tables only; device calls fail with
+                               BKV_ERR_NO_DEVICE (for hosts without a GPU) */
 };
 
 #define BKV_MAX_BATCH 64      /* (sequence, position) entries per append / attention call */
@@ -285,9 +282,7 @@ bkv_status bkv_rope_table(double freq_base, int32_t n_rot, int32_t max_pos, floa
  * workspace the pool owns.  The split-K kernel multiplies on the matrix cores (all heads of a
  * kv head, up to 16, in one pass over the K/V rows; q and the probabilities as high + low f16
  * parts, quantised values as exact high + low f16 parts, so accuracy is that of f32
- * accumulation): on f16 pools always, also for selection lists and the fused step; on the
- * quantised pools for this call, while their selection lists use the VALU kernel (heads in
- * chunks of 8 or 4). */
+ * accumulation), on every layout, for this call, for selection lists and for the fused step. */
 bkv_status bkv_decode_attn(bkv_pool *pool, int32_t layer, int32_t n, const int32_t *seqs,
                            const int64_t *pos, int32_t n_q_head, const float *q_dev,
                            const float *gate_dev, int64_t gate_seq_stride,
@@ -339,8 +334,7 @@ bkv_status bkv_prefill_attn(bkv_pool *pool, int32_t layer, int32_t n_seqs, const
  * the pool afterwards holds exactly what bkv_append would have written -- and uses it in
  * place of the stale pool row; the output is bit-identical to the two-call sequence.  Every
  * sequence at most once per call; the cell must have been reserved (bkv_seq_reserve) like for
- * bkv_append.  On quantised pools the step is served by the matrix-core kernels only (at most
- * 16 q heads per kv head, pool without BKV_POOL_ATTN_VALU; BKV_ERR_INVALID otherwise). */
+ * bkv_append. */
 bkv_status bkv_decode_step(bkv_pool *pool, int32_t layer, int32_t n, const int32_t *seqs,
                            const int64_t *pos, const float *k_new_dev, const float *v_new_dev,
                            int32_t n_q_head, const float *q_dev, const float *gate_dev,
@@ -372,8 +366,7 @@ bkv_status bkv_decode_step(bkv_pool *pool, int32_t layer, int32_t n, const int32
  * Between creation and the last replay the caller leaves the listed sequences alone (no free,
  * fork, truncate, evict); allocator calls for OTHER sequences are fine but must be followed by an
  * eager call on the pool before a capture begins, since their block-table changes cannot be
- * recorded.  Destroy a pool's plans before the pool.  Matrix-core pools only (no
- * BKV_POOL_ATTN_VALU), all three layouts. */
+ * recorded.  Destroy a pool's plans before the pool.  All three layouts. */
 typedef struct bkv_step_plan bkv_step_plan;
 bkv_status bkv_step_plan_create(bkv_pool *pool, int32_t n, const int32_t *seqs, const int64_t *pos,
                                 int32_t horizon, int32_t n_q_head, void *stream, bkv_step_plan **out);
@@ -491,14 +484,12 @@ bkv_status bkv_gather(bkv_pool *pool, int32_t layer, int32_t seq, int64_t cell0,
  * the planning step of bkv_decode_attn / bkv_decode_step / bkv_decode_attn_select alone, on the
  * host, nothing launched (no pool or device needed).  pos[n] as for those calls; sel_groups > 0
  * plans every entry for that many groups of four listed blocks (a selection list of
- * 4 * sel_groups ids) instead of its pages; matrix_cores != 0 plans for the matrix-core
- * kernels, 0 for the VALU formulation.  splits_out[n], pps_out[n]: page ranges per entry and
+ * 4 * sel_groups ids) instead of its pages.  splits_out[n], pps_out[n]: page ranges per entry and
  * pages per range; *total_out: work-groups of the launch.  BKV_ERR_INVALID when the batch needs
  * more work-groups than the partial-result workspace holds -- the error the attention calls
  * themselves return, before anything is enqueued (qsa/mod.rs:1108-1116). */
 bkv_status bkv_attn_plan(int32_t n_cu, int32_t n_kv_head, int32_t n_q_head, int32_t n, const int64_t *pos,
-                         int32_t sel_groups, int32_t matrix_cores, int32_t *splits_out, int32_t *pps_out,
-                         int32_t *total_out);
+                         int32_t sel_groups, int32_t *splits_out, int32_t *pps_out, int32_t *total_out);
 
 /* ---- per-kernel GPU timing ------------------------------------------------------
  * The analogue of Qsa::stage_timings / Pipe::run_timed (qsa/mod.rs:1733-1970,

@@ -16,19 +16,13 @@ ATTN_MAX_REL = 1e-3
 REF_BAR_MAX_REL = 1e-5
 
 
-# f16 pools run dense decode attention on the matrix cores unless created with
-# BKV_POOL_ATTN_VALU; test modules flip this default to run every case in both formulations
-DEFAULT_ATTN_VALU = False
-
-
 class Twin:
     """A device pool plus one oracle PoolImage per layer, kept in step."""
 
     def __init__(self, n_layers=1, n_pages=512, n_kv=2, hd=256, layout=L.LAYOUT_F16, max_seqs=16,
-                 max_pages_per_seq=None, attn_valu=None):
+                 max_pages_per_seq=None):
         self.pool = Pool(n_layers=n_layers, n_pages=n_pages, n_kv_head=n_kv, head_dim=hd,
-                         layout=layout, max_seqs=max_seqs, max_pages_per_seq=max_pages_per_seq,
-                         attn_valu=DEFAULT_ATTN_VALU if attn_valu is None else attn_valu)
+                         layout=layout, max_seqs=max_seqs, max_pages_per_seq=max_pages_per_seq)
         self.g = oracle.Geom(n_kv, hd, 16)
         self.layout = layout
         self.images = [oracle.PoolImage(self.g, n_pages, ORACLE_LAYOUT[layout]) for _ in range(n_layers)]

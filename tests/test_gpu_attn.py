@@ -17,15 +17,6 @@ from helpers import max_abs
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(autouse=True, params=["mfma", "valu"])
-def attn_formulation(request):
-    """Every case runs in both formulations of f16 decode attention (matrix cores / VALU)."""
-    import gpu_common
-    gpu_common.DEFAULT_ATTN_VALU = request.param == "valu"
-    yield request.param
-    gpu_common.DEFAULT_ATTN_VALU = False
-
-
 GOLD = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_kats.json")))
 
 
@@ -323,26 +314,24 @@ def test_other_head_counts(layout, n_kv, n_q):
         for t in (0, 17, 39):
             _, rel = check_attn(oc[t], tw.oracle_attend(0, seqs[0], lens[0] - 40 + t, qc[t], n_q), "chunk %d" % t)
             assert rel <= REF_BAR_MAX_REL, rel
-        # the fused step (one more token per sequence), where this pool has it: pool bytes as an
-        # append would leave them, outputs against the oracle
-        import gpu_common
-        if layout == L.LAYOUT_F16 or not gpu_common.DEFAULT_ATTN_VALU:
-            k1 = rng.standard_normal((2, n_kv, 256)).astype(np.float32)
-            v1 = rng.standard_normal((2, n_kv, 256)).astype(np.float32)
-            kd, vd = DeviceBuffer.from_numpy(k1), DeviceBuffer.from_numpy(v1)
-            qd, od = DeviceBuffer.from_numpy(q), DeviceBuffer(q.nbytes)
-            tw.pool.decode_step(0, seqs, lens, kd, vd, n_q, qd, od, 1.0 / 16.0)
-            device_sync()
-            os_ = od.download(np.float32).reshape(2, n_q, 256)
-            for b in (kd, vd, qd, od):
-                b.free()
-            for i, s in enumerate(seqs):
-                assert tw.images[0].append(tw.pool.block_table(s), lens[i], k1[i:i + 1], v1[i:i + 1],
-                                           capacity_cells=tw.pool.seq_capacity(s)) == 0
-            tw.assert_pools_equal()
-            for i in range(2):
-                _, rel = check_attn(os_[i], tw.oracle_attend(0, seqs[i], lens[i], q[i], n_q), "step %d" % i)
-                assert rel <= REF_BAR_MAX_REL, rel
+        # the fused step (one more token per sequence): pool bytes as an append would leave them,
+        # outputs against the oracle
+        k1 = rng.standard_normal((2, n_kv, 256)).astype(np.float32)
+        v1 = rng.standard_normal((2, n_kv, 256)).astype(np.float32)
+        kd, vd = DeviceBuffer.from_numpy(k1), DeviceBuffer.from_numpy(v1)
+        qd, od = DeviceBuffer.from_numpy(q), DeviceBuffer(q.nbytes)
+        tw.pool.decode_step(0, seqs, lens, kd, vd, n_q, qd, od, 1.0 / 16.0)
+        device_sync()
+        os_ = od.download(np.float32).reshape(2, n_q, 256)
+        for b in (kd, vd, qd, od):
+            b.free()
+        for i, s in enumerate(seqs):
+            assert tw.images[0].append(tw.pool.block_table(s), lens[i], k1[i:i + 1], v1[i:i + 1],
+                                       capacity_cells=tw.pool.seq_capacity(s)) == 0
+        tw.assert_pools_equal()
+        for i in range(2):
+            _, rel = check_attn(os_[i], tw.oracle_attend(0, seqs[i], lens[i], q[i], n_q), "step %d" % i)
+            assert rel <= REF_BAR_MAX_REL, rel
 
 
 @pytest.mark.parametrize("layout", [L.LAYOUT_F16, L.LAYOUT_Q8V, L.LAYOUT_I8H])

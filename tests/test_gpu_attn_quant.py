@@ -16,15 +16,6 @@ from test_gpu_attn import fill, score_spread_case
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(autouse=True, params=["mfma", "valu"])
-def attn_formulation(request):
-    """Every case runs in both formulations of dense decode attention (matrix cores / VALU)."""
-    import gpu_common
-    gpu_common.DEFAULT_ATTN_VALU = request.param == "valu"
-    yield
-    gpu_common.DEFAULT_ATTN_VALU = False
-
-
 def test_reference_q8v_recipe_64_cells():
     # attn_conformance.rs:1355-1452: normalish seeds 0xF1..0xF4, one append of 64 cells, 24 heads,
     # gate from q_full; dense list instead of the reference's sparse ids [0,5,9,15]

@@ -15,15 +15,6 @@ from test_gpu_attn import fill
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(autouse=True, params=["mfma", "valu"])
-def attn_formulation(request):
-    """f16 pools run every case in both formulations of decode attention (matrix cores / VALU)."""
-    import gpu_common
-    gpu_common.DEFAULT_ATTN_VALU = request.param == "valu"
-    yield
-    gpu_common.DEFAULT_ATTN_VALU = False
-
-
 def select_attn(tw, layer, seqs, pos, q, n_head, id_lists, max_ids=None, id_stride=None, gate=None,
                 gate_strides=None, counts=None, pad=0xDEADBEEF):
     """q: [n, n_head, 256]; id_lists: one list of block ids per entry.  The unused tail of every

@@ -12,15 +12,6 @@ from test_gpu_attn import fill
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(autouse=True, params=["mfma", "valu"])
-def attn_formulation(request):
-    """Every case runs in both formulations of f16 decode attention (matrix cores / VALU)."""
-    import gpu_common
-    gpu_common.DEFAULT_ATTN_VALU = request.param == "valu"
-    yield
-    gpu_common.DEFAULT_ATTN_VALU = False
-
-
 def step(tw, layer, seqs, pos, k_new, v_new, q, n_head, gate=None):
     n = len(seqs)
     kd, vd = DeviceBuffer.from_numpy(k_new), DeviceBuffer.from_numpy(v_new)
@@ -39,20 +30,8 @@ def step(tw, layer, seqs, pos, k_new, v_new, q, n_head, gate=None):
 @pytest.mark.parametrize("layout", [L.LAYOUT_F16, L.LAYOUT_Q8V, L.LAYOUT_I8H])
 @pytest.mark.parametrize("n_q", [16, 24])
 def test_fused_step_equals_append_then_attend(n_q, layout):
-    import gpu_common
     rng = np.random.Generator(np.random.PCG64(800 + n_q + 7 * layout))
     lens = [37, 512, 1000, 2048, 15, 16, 1, 0, 4099]      # page edges, an empty sequence, long
-    if layout != L.LAYOUT_F16 and gpu_common.DEFAULT_ATTN_VALU:
-        # on quantised pools the step exists on the matrix-core path only: refused, pool untouched
-        with Twin(n_pages=16, max_seqs=4, layout=layout) as tw:
-            s = tw.pool.seq_create()
-            tw.pool.seq_reserve(s, 20)
-            z = DeviceBuffer(1 << 16)
-            with pytest.raises(BkvError) as ei:
-                tw.pool.decode_step(0, [s], [19], z, z, n_q, z, z, 0.0625)
-            assert ei.value.status == L.ERR_INVALID
-            z.free()
-        return
     with Twin(n_pages=700, max_seqs=24, layout=layout) as tw:
         tw.pool.set_free_order(rng.permutation(700).astype(np.int32))
         fused = [tw.pool.seq_create() for _ in lens]

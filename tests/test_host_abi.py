@@ -292,34 +292,27 @@ def test_attention_planning_terminates_and_fits_for_every_batch_shape():
     host), cover every page, and fit the partial-result workspace -- or be refused as a size
     error before anything is enqueued (crates/breccia-kernels/src/qsa/mod.rs:1108-1116)."""
     rng = np.random.Generator(np.random.PCG64(77))
-    checked = refused = 0
-    for mc in (True, False):
-        for n_cu in (256, 64, 8):
-            for n_kv in range(1, L.MAX_KV_HEAD + 1):
-                for group in range(1, 17):
-                    hg = group if mc else (8 if group % 8 == 0 else 4)
-                    n_hc = (group + hg - 1) // hg
-                    cap = 4096 * 8 // hg if hg > 8 else 4096
-                    for n in (1, 2, 7, 33, 64):
-                        for sel_groups in (0, 129):
-                            pos = rng.integers(0, 40000, size=n)
-                            if n >= 33:
-                                pos[: n // 2] = rng.integers(0, 64, size=n // 2)   # many one-page entries
-                            if n * n_kv * n_hc > cap:
-                                expect(L.ERR_INVALID, kv.attn_plan, n_cu, n_kv, n_kv * group, pos, sel_groups, mc)
-                                refused += 1
-                                continue
-                            splits, pps, total = kv.attn_plan(n_cu, n_kv, n_kv * group, pos, sel_groups, mc)
-                            pages = np.full(n, sel_groups) if sel_groups else pos // 16 + 1
-                            assert total == int(splits.sum()) * n_kv * n_hc <= cap
-                            assert np.all(pps % 4 == 0) and np.all(splits >= 1)
-                            assert np.all(splits * pps >= pages) and np.all((splits - 1) * pps < pages)
-                            resident = n_cu * (2 if (mc or hg == 8) else 3)
-                            # one generation whenever one is possible at all
-                            assert total <= max(resident, n * n_kv * n_hc)
-                            checked += 1
-    # with at most 64 entries, 16 kv heads and 4 head chunks the workspace (4096 work-groups) always suffices
-    assert checked > 5000 and refused == 0
+    checked = 0
+    for n_cu in (256, 64, 8):
+        for n_kv in range(1, L.MAX_KV_HEAD + 1):
+            for group in range(1, 17):
+                # a work-group writes `group` head rows of a workspace that holds 4096 x 8
+                cap = 4096 * 8 // group if group > 8 else 4096
+                for n in (1, 2, 7, 33, 64):
+                    for sel_groups in (0, 129):
+                        pos = rng.integers(0, 40000, size=n)
+                        if n >= 33:
+                            pos[: n // 2] = rng.integers(0, 64, size=n // 2)   # many one-page entries
+                        assert n * n_kv <= cap    # 64 entries x 16 kv heads always fit
+                        splits, pps, total = kv.attn_plan(n_cu, n_kv, n_kv * group, pos, sel_groups)
+                        pages = np.full(n, sel_groups) if sel_groups else pos // 16 + 1
+                        assert total == int(splits.sum()) * n_kv <= cap
+                        assert np.all(pps % 4 == 0) and np.all(splits >= 1)
+                        assert np.all(splits * pps >= pages) and np.all((splits - 1) * pps < pages)
+                        # one generation (two work-groups per compute unit) whenever one is possible at all
+                        assert total <= max(2 * n_cu, n * n_kv)
+                        checked += 1
+    assert checked > 5000
 
 
 def test_attention_batches_larger_than_one_generation_are_planned_not_spun_on():
@@ -328,15 +321,15 @@ def test_attention_batches_larger_than_one_generation_are_planned_not_spun_on():
         for s in seqs:
             p.seq_reserve(s, 4)
         z = C.c_void_p(0)
-        # 64 entries x 16 kv heads x 4 head chunks of the VALU formulation's 13-head groups = 4096: accepted
-        # as a plan (and then refused for lack of a device); one more kv head cannot exist
+        # 64 entries x 16 kv heads of 13 q heads each = 1024 work-groups: accepted as a plan (and then
+        # refused for lack of a device); one more kv head cannot exist
         expect(L.ERR_NO_DEVICE, p.decode_attn, 0, seqs, [3] * 64, 16 * 13, z, z, 0.0625)
     expect(L.ERR_INVALID, host_pool, n_kv_head=L.MAX_KV_HEAD + 1)
-    expect(L.ERR_INVALID, kv.attn_plan, 256, L.MAX_KV_HEAD + 1, 17, [5], 0, True)
+    expect(L.ERR_INVALID, kv.attn_plan, 256, L.MAX_KV_HEAD + 1, 17, [5], 0)
     # the largest accepted shapes are planned as one range per entry, in more than one generation
-    splits, pps, total = kv.attn_plan(256, 16, 16 * 16, [5] * 64, 0, True)
+    splits, pps, total = kv.attn_plan(256, 16, 16 * 16, [5] * 64, 0)
     assert total == 1024 and np.all(splits == 1)
-    splits, pps, total = kv.attn_plan(256, 9, 9, [70000] * 64, 0, True)      # 576 > 512 resident: used to spin
+    splits, pps, total = kv.attn_plan(256, 9, 9, [70000] * 64, 0)      # 576 > 512 resident: used to spin
     assert total == 576 and np.all(splits == 1) and np.all(pps >= 70000 // 16 + 1)
 
 
