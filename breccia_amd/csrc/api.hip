@@ -3,6 +3,7 @@
 // before anything reaches the GPU (the reference's contract, crates/breccia-kernels/
 // src/qsa/mod.rs:1108-1116).
 #include <algorithm>
+#include <chrono>
 #include <cstdio>
 #include <cstring>
 #include <new>
@@ -1903,7 +1904,18 @@ bkv_status bkv_stream_destroy(void* stream) {
     if (stream) BKV_HIP(hipStreamDestroy(S(stream)));
     return BKV_OK;
 }
+// The host polls the stream for a few milliseconds before it blocks: a thread that sleeps in
+// hipStreamSynchronize is woken some tens of microseconds after the stream has drained, which a
+// decode loop that synchronises per token would pay every time.
 bkv_status bkv_stream_sync(void* stream) {
+    const auto t0 = std::chrono::steady_clock::now();
+    for (;;) {
+        const hipError_t e = hipStreamQuery(S(stream));
+        if (e == hipSuccess) return BKV_OK;
+        if (e != hipErrorNotReady) return hip_fail(e, "hipStreamQuery");
+        (void)hipGetLastError();
+        if (std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(4)) break;
+    }
     BKV_HIP(hipStreamSynchronize(S(stream)));
     return BKV_OK;
 }
