@@ -265,22 +265,75 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
 }
 
 // ---- a decode step that re-plans itself on the device ------------------------------------------
-// One thread: every entry moves on by one cell and the batch is cut again, by the same function the
-// host uses, so that a replayed launch reads what a fresh call would have been given.  An entry
-// that would pass the last cell the plan was checked for stops the advance (nothing moves, the
-// status word says so).
-__global__ void step_advance_kernel(StepDesc* d, AttnPlanLimits lim, int32_t page_cells) {
-    if (threadIdx.x != 0 || blockIdx.x != 0) return;
-    AttnBatch b = d->b;
-    for (int i = 0; i < b.n; ++i)
-        if (b.pos[i] + 1 > d->horizon[i]) {
-            d->status = 1;
-            return;
+// One wave, lane i = entry i: every entry moves on by one cell and the batch is cut again with the
+// arithmetic of plan_attn_ranges (attn_plan.hpp) -- the sums and the running offsets as wave
+// reductions -- so that a replayed launch reads what a fresh call would have been given, bit for
+// bit.  An entry that would pass the last cell the plan was checked for stops the advance
+// (nothing moves, the status word says so).
+__device__ __forceinline__ long long wave_sum(long long v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+__device__ __forceinline__ long long wave_max(long long v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const long long o = __shfl_xor(v, off, 64);
+        v = o > v ? o : v;
+    }
+    return v;
+}
+__global__ __launch_bounds__(64) void step_advance_kernel(StepDesc* d, AttnPlanLimits lim, int32_t page_cells) {
+    static_assert(kMaxBatch <= 64, "one lane per entry");
+    const int i = threadIdx.x;
+    const int n = d->b.n;
+    const bool live = i < n;
+    int pos = live ? d->b.pos[i] : 0;
+    const bool past = live && pos + 1 > d->horizon[i];
+    if (__builtin_amdgcn_ballot_w64(past) != 0) {
+        if (i == 0) d->status = 1;
+        return;
+    }
+    pos += 1;
+    const long long per_page = lim.per_page, gran = lim.gran;
+    const long long min_total = (long long)n * per_page;
+    long long target = lim.target < lim.max_wgs ? lim.target : lim.max_wgs;
+    if (target < min_total) target = min_total;
+    const long long pages = live ? pos / page_cells + 1 : 0;
+    const long long total_pages = wave_sum(pages), max_pages = wave_max(pages);
+    long long pps = (total_pages * per_page + target - 1) / target;
+    pps = (pps + gran - 1) / gran * gran;
+    if (pps < gran) pps = gran;
+    long long my_splits = 0, each = gran, total = 0;
+    for (;;) {
+        if (live) {
+            const long long splits = (pages + pps - 1) / pps;
+            // even the ranges out inside the entry, keeping whole groups of `gran` pages
+            each = (pages + splits - 1) / splits;
+            each = (each + gran - 1) / gran * gran;
+            my_splits = (pages + each - 1) / each;
         }
-    for (int i = 0; i < b.n; ++i) b.pos[i] += 1;
-    (void)plan_attn_ranges(lim, page_cells, 0, b);
-    d->b = b;
-    d->steps += 1u;
+        total = wave_sum(my_splits * per_page);
+        if (total <= target || pps >= max_pages) break;
+        pps += gran;
+    }
+    // first work-group of every entry: the sum over the entries before it
+    long long incl = my_splits * per_page;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const long long o = __shfl_up(incl, off, 64);
+        if (i >= off) incl += o;
+    }
+    if (live) {
+        d->b.pos[i] = pos;
+        d->b.splits[i] = (int32_t)my_splits;
+        d->b.pps[i] = (int32_t)each;
+        d->b.wg_base[i] = (int32_t)(incl - my_splits * per_page);
+    }
+    if (i == 0) {
+        d->b.wg_base[n] = (int32_t)total;
+        d->steps += 1u;
+    }
 }
 
 hipError_t launch_step_advance(StepDesc* d, const AttnPlanLimits& lim, int32_t page_cells, hipStream_t stream) {

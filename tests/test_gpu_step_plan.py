@@ -132,3 +132,49 @@ def test_plan_creation_checks_the_whole_horizon():
         tw.pool.seq_free(child)
         plan = StepPlan(tw.pool, [a, b], [30, 20], 10, 16)
         plan.destroy()
+
+
+def test_the_device_cuts_a_large_ragged_batch_as_the_host_does():
+    """The advance kernel re-plans on the device with the host planner's arithmetic: over 40 advances
+    of 64 sequences of very different lengths (page edges crossed all the time, the cut changing with
+    them), a step replayed from the plan returns the bits of bkv_decode_step at the same positions."""
+    n, n_q, n_tok = 64, 16, 40
+    rng = np.random.Generator(np.random.PCG64(9400))
+    lens = [int(x) for x in rng.integers(0, 70, size=40)] + [int(x) for x in rng.integers(200, 3000, size=24)]
+    order = rng.permutation(4096).astype(np.int32)
+    st = Stream()
+    with Twin(n_pages=4096, max_seqs=64, max_pages_per_seq=200) as a, \
+            Twin(n_pages=4096, max_seqs=64, max_pages_per_seq=200) as b:
+        seqs = None
+        for tw in (a, b):
+            r2 = np.random.Generator(np.random.PCG64(5))
+            tw.pool.set_free_order(order)
+            ss = [tw.pool.seq_create() for _ in lens]
+            for s, c in zip(ss, lens):
+                if c:
+                    fill(tw, s, c, r2, chunk=1024)
+                tw.pool.seq_reserve(s, c + n_tok + 1)
+            assert seqs is None or seqs == ss
+            seqs = ss
+        kn = rng.standard_normal((n_tok, n, 2, 256)).astype(np.float32)
+        q = rng.standard_normal((n, n_q, 256)).astype(np.float32)
+        kd, qd = DeviceBuffer(kn[0].nbytes), DeviceBuffer.from_numpy(q)
+        oe, op = DeviceBuffer(q.nbytes), DeviceBuffer(q.nbytes)
+        plan = StepPlan(b.pool, seqs, lens, n_tok + 1, n_q, stream=st)
+        for t in range(n_tok):
+            kd.upload(kn[t])
+            device_sync()
+            a.pool.decode_step(0, seqs, [c + t for c in lens], kd, kd, n_q, qd, oe, 1.0 / 16.0)
+            plan.decode(0, kd, kd, qd, op, 1.0 / 16.0, stream=st)
+            plan.advance(st)
+            st.sync()
+            device_sync()
+            if t % 3 == 0 or t == n_tok - 1:
+                assert np.array_equal(oe.download(np.uint32), op.download(np.uint32)), "token %d" % t
+        pos, steps, status = plan.state(st)
+        assert steps == n_tok and status == 0 and list(pos) == [c + n_tok for c in lens]
+        assert np.array_equal(a.pool.read_layer(0, 0), b.pool.read_layer(0, 0))
+        plan.destroy()
+        for x in (kd, qd, oe, op):
+            x.free()
+    st.close()
