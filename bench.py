@@ -38,7 +38,7 @@ ROW_BYTES_I8H = N_KV * 2 * (HD // 32 * 34)        # 1088
 # HBM traffic of one launch of the split-K kernel on the default seeded workload, from
 # rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this file, each scaled by what the same counter
 # reads for the plain copy probe (profiles/hbm_traffic_all_kernels.md)
-MEASURED_TRAFFIC = {"seed": 20250003, "fetch_bytes": 328.68e6, "write_bytes": 4.18e6}
+MEASURED_TRAFFIC = {"seed": 20250003, "fetch_bytes": 328.36e6, "write_bytes": 4.19e6}
 APPEND_BYTES_PER_TOKEN = N_KV * HD * (4 + 2) * 2  # f32 in + f16 out, K and V = 6144
 
 
@@ -300,7 +300,7 @@ def main() -> int:
                 "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE profile of this command (seed %d), "
                                   "profiles/hbm_traffic_all_kernels.md; a constant of this file, not measured "
                                   "by this run" % MEASURED_TRAFFIC["seed"],
-                "kernel": "decode_attn_mfma_kernel<true> (f16 K/V, all 8 q heads of a kv head per pass on the "
+                "kernel": "decode_attn_mfma_kernel<true, false, false> (f16 K/V, all 8 q heads of a kv head per pass on the "
                           "matrix cores, new row taken in flight)",
                 "avg_us": round(split_us, 2),
                 "launches": n_split, "algorithmic_bytes": attn_bytes}
