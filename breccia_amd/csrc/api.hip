@@ -137,6 +137,12 @@ bkv_status flush_tables(bkv_pool* p, hipStream_t stream) {
     flat.reserve(last.size());
     for (const auto& kv : last) flat.push_back(TableUpdate{kv.first, kv.second});
     const size_t per_slot = ParamRing::kSlotBytes / sizeof(TableUpdate);
+    if (flat.size() <= (size_t)kTableUpdatesInArgs) {
+        // the usual case of a decode loop (a sequence or two opened a page): the updates ride in the
+        // arguments of the scatter launch, no upload
+        BKV_HIP(launch_table_scatter_args(p->table_dev, flat.data(), (int32_t)flat.size(), stream));
+        flat.clear();
+    }
     for (size_t at = 0; at < flat.size(); at += per_slot) {
         const size_t n = std::min(per_slot, flat.size() - at);
         void* dev;

@@ -267,6 +267,9 @@ hipError_t launch_gather(const bkv_pool* p, int32_t layer, int32_t row, int64_t 
                          float* k_out, float* v_out, hipStream_t stream);
 hipError_t launch_table_scatter(int32_t* table, const TableUpdate* upd_dev, int32_t n,
                                 hipStream_t stream);
+// up to kTableUpdatesInArgs updates, given on the host, as arguments of one small launch
+constexpr int32_t kTableUpdatesInArgs = 32;
+hipError_t launch_table_scatter_args(int32_t* table, const TableUpdate* upd_host, int32_t n, hipStream_t stream);
 hipError_t launch_fill(void* dst, uint64_t bytes, uint32_t word, hipStream_t stream);
 hipError_t launch_copy_probe(void* dst, const void* src, uint64_t bytes, hipStream_t stream);
 hipError_t launch_read_probe(const void* src, uint64_t bytes, bool scattered, void* sink, int32_t n_cu,

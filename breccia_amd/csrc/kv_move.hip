@@ -544,6 +544,16 @@ __global__ __launch_bounds__(kBlock) void table_scatter_kernel(int32_t* __restri
     if (i < n) table[upd[i].offset] = upd[i].value;
 }
 
+// A handful of updates travel as kernel arguments: no upload, no ring slot.
+struct TableUpdateArgs {
+    TableUpdate u[kTableUpdatesInArgs];
+};
+__global__ __launch_bounds__(64) void table_scatter_args_kernel(int32_t* __restrict__ table, TableUpdateArgs a,
+                                                               int32_t n) {
+    const int i = threadIdx.x;
+    if (i < n) table[a.u[i].offset] = a.u[i].value;
+}
+
 __global__ __launch_bounds__(kBlock) void fill_kernel(uint4* __restrict__ dst, uint64_t n_vec,
                                                       uint32_t word) {
     const uint4 w = make_uint4(word, word, word, word);
@@ -728,6 +738,15 @@ hipError_t launch_table_scatter(int32_t* table, const TableUpdate* upd_dev, int3
                                 hipStream_t stream) {
     if (n == 0) return hipSuccess;
     table_scatter_kernel<<<(n + kBlock - 1) / kBlock, kBlock, 0, stream>>>(table, upd_dev, n);
+    return hipGetLastError();
+}
+
+hipError_t launch_table_scatter_args(int32_t* table, const TableUpdate* upd_host, int32_t n, hipStream_t stream) {
+    if (n == 0) return hipSuccess;
+    if (n > kTableUpdatesInArgs) return hipErrorInvalidValue;
+    TableUpdateArgs a{};
+    for (int i = 0; i < n; ++i) a.u[i] = upd_host[i];
+    table_scatter_args_kernel<<<1, 64, 0, stream>>>(table, a, n);
     return hipGetLastError();
 }
 
