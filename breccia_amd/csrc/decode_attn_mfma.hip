@@ -492,6 +492,18 @@ __device__ __forceinline__ void i8h_unit_to_lds(const UnitSrc<SEL>& src, bool re
     typedef const __attribute__((address_space(1))) void* gptr;
     typedef __attribute__((address_space(3))) void* lptr;
     constexpr int kRun = 4 * row_bytes_of(kRowI8H);
+    if constexpr (!SEL) {
+        // one run: a single address, the pieces as immediate offsets of the instruction (they move the
+        // place in memory and the place in LDS alike); a wave past its last page asks for five
+        // pieces at the head of the unit it last read
+        const uint8_t* a = src.run[0] + (real ? lane * 16 : 0);
+        __builtin_amdgcn_global_load_lds((gptr)a, (lptr)dst, 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gptr)a, (lptr)dst, 16, 1024, 0);
+        __builtin_amdgcn_global_load_lds((gptr)a, (lptr)dst, 16, 2048, 0);
+        __builtin_amdgcn_global_load_lds((gptr)a, (lptr)dst, 16, 3072, 0);
+        if (lane < 16) __builtin_amdgcn_global_load_lds((gptr)(a + 4096), (lptr)(dst + 4096), 16, 0, 0);
+        return;
+    }
 #pragma unroll
     for (int n = 0; n < 4; ++n) {
         const uint8_t* a = real ? unit_piece<SEL, kRun>(src, n * 1024 + lane * 16) : src.run[0];
@@ -831,6 +843,16 @@ __device__ __forceinline__ void q8v_unit_to_lds(const UnitSrc<SEL>& src, bool re
     typedef const __attribute__((address_space(1))) void* gptr;
     typedef __attribute__((address_space(3))) void* lptr;
     constexpr int kRun = 4 * kQ8vRow;
+    if constexpr (!SEL) {
+        // one run: a single address and immediate offsets, as in i8h_unit_to_lds
+        const uint8_t* a = src.run[0] + (real ? lane * 16 : 0);
+        __builtin_amdgcn_global_load_lds((gptr)a, (lptr)dst, 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gptr)a, (lptr)dst, 16, 1024, 0);
+        __builtin_amdgcn_global_load_lds((gptr)a, (lptr)dst, 16, 2048, 0);
+        __builtin_amdgcn_global_load_lds((gptr)a, (lptr)dst, 16, 3072, 0);
+        if (lane < 32) __builtin_amdgcn_global_load_lds((gptr)(a + 4096), (lptr)(dst + 4096), 16, 0, 0);
+        return;
+    }
 #pragma unroll
     for (int n = 0; n < 4; ++n) {
         const uint8_t* a = real ? unit_piece<SEL, kRun>(src, n * 1024 + lane * 16) : src.run[0];
