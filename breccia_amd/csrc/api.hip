@@ -1001,7 +1001,30 @@ struct bkv_step_plan {
     float* part_ml = nullptr;
     int32_t n = 0, n_q_head = 0, grid = 0;
     AttnPlanLimits lim{};
+    // what the plan was checked for: cells first[i]..last[i] of sequence seq[i]
+    int32_t seq[kMaxBatch] = {};
+    int64_t first[kMaxBatch] = {}, last[kMaxBatch] = {};
 };
+
+// The cells a plan was created for must still be what they were then (reserved, on the device, held
+// by the sequence alone): a host call that enqueues the plan's kernels looks again, so that a
+// sequence freed, forked, truncated or evicted in between is an error here and not a write into
+// somebody else's page.  (A replayed graph makes no host call; there the rule is the caller's.)
+static bkv_status plan_cells_unchanged(const bkv_step_plan* pl, const char* what) {
+    const bkv_pool* p = pl->pool;
+    for (int i = 0; i < pl->n; ++i) {
+        if (!p->alloc->seq_valid(pl->seq[i]))
+            return fail(BKV_ERR_STATE, std::string(what) + sfmt(": sequence %lld of the plan is no longer live",
+                                                                pl->seq[i]));
+        if (pl->last[i] >= p->alloc->seq_capacity(pl->seq[i]) || !p->alloc->seq_resident(pl->seq[i], pl->last[i] + 1))
+            return fail(BKV_ERR_STATE, std::string(what) + sfmt(": sequence %lld of the plan lost pages below cell "
+                                                                "%lld since the plan was made", pl->seq[i],
+                                                                pl->last[i]));
+        const bkv_status wst = check_writable(p, what, pl->seq[i], pl->first[i], pl->last[i] + 1);
+        if (wst != BKV_OK) return wst == BKV_ERR_RANGE ? fail(BKV_ERR_STATE, g_last_error) : wst;
+    }
+    return BKV_OK;
+}
 
 bkv_status bkv_step_plan_create(bkv_pool* p, int32_t n, const int32_t* seqs, const int64_t* pos,
                                 int32_t horizon, int32_t n_q_head, void* stream, bkv_step_plan** out) {
@@ -1052,6 +1075,11 @@ bkv_status bkv_step_plan_create(bkv_pool* p, int32_t n, const int32_t* seqs, con
     pl->n = n;
     pl->n_q_head = n_q_head;
     pl->lim = lim;
+    for (int i = 0; i < n; ++i) {
+        pl->seq[i] = seqs[i];
+        pl->first[i] = pos[i];
+        pl->last[i] = host.horizon[i];
+    }
     // no cut of this batch, at any position, has more work-groups than this
     pl->grid = std::max<int32_t>(std::min(lim.target, lim.max_wgs), n * lim.per_page);
     auto bail = [&](bkv_status err) {
@@ -1099,6 +1127,8 @@ bkv_status bkv_step_plan_decode(bkv_step_plan* pl, int32_t layer, const float* k
         !aligned16(k_new_dev) || !aligned16(v_new_dev))
         return fail(BKV_ERR_INVALID, "step_plan_decode: q / out / k / v device pointers must be non-NULL and "
                                      "16-byte aligned");
+    const bkv_status still = plan_cells_unchanged(pl, "step_plan_decode");
+    if (still != BKV_OK) return still;
     // Block-table changes made since the last call still travel the usual way, which a stream under
     // capture cannot record (it waits on the host for a free ring slot): make them before capturing.
     if (!p->alloc->pending().empty() || p->tiers.pending) {

@@ -364,7 +364,9 @@ bkv_status bkv_decode_step(bkv_pool *pool, int32_t layer, int32_t n, const int32
  *                          advance past the checked cells changes nothing and sets status 1.
  *   bkv_step_plan_state    waits for `stream`, then reports positions, advances done and status.
  * Between creation and the last replay the caller leaves the listed sequences alone (no free,
- * fork, truncate, evict); allocator calls for OTHER sequences are fine but must be followed by an
+ * fork, truncate, evict): bkv_step_plan_decode looks at the plan's cells again on every call and
+ * returns BKV_ERR_STATE when they are no longer reserved, resident and unshared, but a replayed
+ * graph makes no such call.  Allocator calls for OTHER sequences are fine but must be followed by an
  * eager call on the pool before a capture begins, since their block-table changes cannot be
  * recorded.  Destroy a pool's plans before the pool.  All three layouts. */
 typedef struct bkv_step_plan bkv_step_plan;

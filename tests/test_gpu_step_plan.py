@@ -134,6 +134,47 @@ def test_plan_creation_checks_the_whole_horizon():
         plan.destroy()
 
 
+def test_a_plan_whose_sequences_changed_is_refused_at_the_next_call():
+    """Between creation and the last use the plan's sequences are to be left alone; a host call that
+    enqueues the plan's kernels looks again, and a sequence that was forked (its page now shared),
+    truncated or freed since is an error before anything is launched."""
+    rng = np.random.Generator(np.random.PCG64(9400))
+    with Twin(n_pages=32, max_seqs=4) as tw:
+        a, b = tw.pool.seq_create(), tw.pool.seq_create()
+        fill(tw, a, 30, rng)
+        fill(tw, b, 20, rng)
+        tw.pool.seq_reserve(a, 40)
+        tw.pool.seq_reserve(b, 40)
+        plan = StepPlan(tw.pool, [a, b], [30, 20], 10, 16)
+        kn = DeviceBuffer.from_numpy(rng.standard_normal((2, 2, 256)).astype(np.float32))
+        q = DeviceBuffer.from_numpy(rng.standard_normal((2, 16, 256)).astype(np.float32))
+        out = DeviceBuffer(2 * 16 * 256 * 4)
+        plan.decode(0, kn, kn, q, out, 1.0 / 16.0)      # as made: fine
+        device_sync()
+        before = tw.pool.read_layer(0, 0).copy()
+        child = tw.pool.seq_fork(a, 35)                  # a's third page is shared now
+        with pytest.raises(BkvError) as ei:
+            plan.decode(0, kn, kn, q, out, 1.0 / 16.0)
+        assert ei.value.status == L.ERR_STATE
+        tw.pool.seq_free(child)
+        plan.decode(0, kn, kn, q, out, 1.0 / 16.0)      # sole holder again
+        tw.pool.seq_truncate(b, 25)                      # cells 25..29 of b are no longer reserved
+        with pytest.raises(BkvError) as ei:
+            plan.decode(0, kn, kn, q, out, 1.0 / 16.0)
+        assert ei.value.status == L.ERR_STATE
+        tw.pool.seq_reserve(b, 40)
+        tw.pool.seq_free(a)
+        with pytest.raises(BkvError) as ei:
+            plan.decode(0, kn, kn, q, out, 1.0 / 16.0)
+        assert ei.value.status == L.ERR_STATE
+        device_sync()
+        # the refused calls wrote nothing (the two accepted ones rewrote the same row)
+        assert np.array_equal(before, tw.pool.read_layer(0, 0))
+        plan.destroy()
+        for x in (kn, q, out):
+            x.free()
+
+
 def test_the_device_cuts_a_large_ragged_batch_as_the_host_does():
     """The advance kernel re-plans on the device with the host planner's arithmetic: over 40 advances
     of 64 sequences of very different lengths (page edges crossed all the time, the cut changing with
