@@ -383,6 +383,9 @@ bkv_status bkv_pool_create(const bkv_pool_desc* d, bkv_pool** out) {
 
 bkv_status bkv_pool_destroy(bkv_pool* p) {
     if (!p) return fail(BKV_ERR_INVALID, "pool_destroy: NULL pool");
+    if (p->live_plans > 0)
+        return fail(BKV_ERR_STATE, sfmt("pool_destroy: %lld step plans of this pool are still alive; destroy them "
+                                        "first (they point into the pool)", p->live_plans));
     destroy_device_side(p);
     delete p;
     return BKV_OK;
@@ -1072,6 +1075,7 @@ bkv_status bkv_step_plan_create(bkv_pool* p, int32_t n, const int32_t* seqs, con
     bkv_step_plan* pl = new (std::nothrow) bkv_step_plan();
     if (!pl) return fail(BKV_ERR_NOMEM, "step_plan_create: out of host memory");
     pl->pool = p;
+    ++p->live_plans;
     pl->n = n;
     pl->n_q_head = n_q_head;
     pl->lim = lim;
@@ -1112,6 +1116,7 @@ bkv_status bkv_step_plan_destroy(bkv_step_plan* pl) {
     if (pl->dev) (void)hipFree(pl->dev);
     if (pl->part_o) (void)hipFree(pl->part_o);
     if (pl->part_ml) (void)hipFree(pl->part_ml);
+    if (pl->pool) --pl->pool->live_plans;
     delete pl;
     return BKV_OK;
 }

@@ -114,6 +114,7 @@ struct bkv_pool {
     float* part_o = nullptr;
     float* part_ml = nullptr;
     int32_t max_wgs = 0;
+    int32_t live_plans = 0;  // step plans made from this pool and not yet destroyed
     // block selection: f64 indexer scores [entry][block], grown on demand
     double* sel_scores = nullptr;
     uint64_t sel_scores_cap = 0;  // doubles

@@ -368,7 +368,8 @@ bkv_status bkv_decode_step(bkv_pool *pool, int32_t layer, int32_t n, const int32
  * returns BKV_ERR_STATE when they are no longer reserved, resident and unshared, but a replayed
  * graph makes no such call.  Allocator calls for OTHER sequences are fine but must be followed by an
  * eager call on the pool before a capture begins, since their block-table changes cannot be
- * recorded.  Destroy a pool's plans before the pool.  All three layouts. */
+ * recorded.  Destroy a pool's plans before the pool (bkv_pool_destroy returns BKV_ERR_STATE while
+ * one is alive).  All three layouts. */
 typedef struct bkv_step_plan bkv_step_plan;
 bkv_status bkv_step_plan_create(bkv_pool *pool, int32_t n, const int32_t *seqs, const int64_t *pos,
                                 int32_t horizon, int32_t n_q_head, void *stream, bkv_step_plan **out);

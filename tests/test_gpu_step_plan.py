@@ -131,6 +131,9 @@ def test_plan_creation_checks_the_whole_horizon():
         assert ei.value.status == L.ERR_STATE
         tw.pool.seq_free(child)
         plan = StepPlan(tw.pool, [a, b], [30, 20], 10, 16)
+        with pytest.raises(BkvError) as ei:          # a plan points into its pool
+            tw.pool.destroy()
+        assert ei.value.status == L.ERR_STATE
         plan.destroy()
 
 
