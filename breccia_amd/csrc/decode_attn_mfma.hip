@@ -241,6 +241,30 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
             for (int r = 0; r < 4; ++r) vf[h][r] = __builtin_nontemporal_load(v_addr(vp, h, r));
     }
 
+    // STEP: the wave that will hold the page of cell pos (in its last iteration) takes the new row now,
+    // while its first pages are on their way: lane l < 32 converts slice l (8 values) of the K row, lane
+    // 32 + l slice l of the V row, stores it into the pool (whole rows, 16 bytes a lane) and parks it in
+    // the wave's part of the fold staging, which nothing else uses before the loop is over.  Fetched at
+    // the last page instead, the row would add a trip to memory to the end of that work-group's walk.
+    v4u* const new_row = reinterpret_cast<v4u*>(&lds.ow[wave][0][0]);
+    if constexpr (STEP) {
+        const int last = n_pages - 1;
+        if (last >= pg0 && last < pg1 && ((last - pg0) & (kWaves - 1)) == wave) {
+            const bool is_k = lane < 32;
+            const int sl = lane & 31;
+            const float* src = (is_k ? P.new_k : P.new_v) + ((size_t)e * P.n_kv + (size_t)kvh) * kHd + sl * 8;
+            const float4 a = *reinterpret_cast<const float4*>(src);
+            const float4 b = *reinterpret_cast<const float4*>(src + 4);
+            v4u w;
+            w.x = f16_store_pair(a.x, a.y), w.y = f16_store_pair(a.z, a.w);
+            w.z = f16_store_pair(b.x, b.y), w.w = f16_store_pair(b.z, b.w);
+            const size_t here = (size_t)bt[last] * page_bytes + head_off + (size_t)(pos & (kPage - 1)) * (kHd * 2);
+            *reinterpret_cast<v4u*>((is_k ? P.kpool_w : P.vpool_w) + here + (size_t)sl * 16) = w;
+            new_row[lane] = w;
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        }
+    }
+
     half8 qhi[8], qlo[8];
     load_q_fragments(P, e, kvh, c, g, qhi, qlo);
 
@@ -271,39 +295,27 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
 
         if constexpr (STEP) {
             if (pg == n_pages - 1) {
-                // This wave holds the page of cell pos; its pool row is stale.  Every lane converts
-                // its slices of the new row; the lanes whose fragments are that row keep and store them.
+                // This wave holds the page of cell pos; its pool row was stale when it was fetched.  The
+                // lanes whose fragments are that row take the slices parked before the loop.
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
                 const int r = pos & (kPage - 1);
-                const size_t here = (size_t)(cur.k[0] - P.kpool) + (size_t)r * (kHd * 2);
-                const float* nk = P.new_k + ((size_t)e * P.n_kv + (size_t)kvh) * kHd;
-                const float* nv = P.new_v + ((size_t)e * P.n_kv + (size_t)kvh) * kHd;
-                const auto row_slice = [](const float* src) {
-                    const float4 a = *reinterpret_cast<const float4*>(src);
-                    const float4 b = *reinterpret_cast<const float4*>(src + 4);
-                    v4u w;
-                    w.x = f16_store_pair(a.x, a.y), w.y = f16_store_pair(a.z, a.w);
-                    w.z = f16_store_pair(b.x, b.y), w.w = f16_store_pair(b.z, b.w);
-                    return w;
-                };
                 // K registers hold rows as fetched: row r sits in the lanes with c % 8 == r % 8, in the
                 // register of rows 0..7 or of rows 8..15, segment g + 4 (c / 8) of each 128-byte line
                 const int seg = g + 4 * (c >> 3);
 #pragma unroll
                 for (int p = 0; p < 4; ++p) {
-                    const v4u w = row_slice(nk + p * 64 + seg * 8);
+                    const v4u w = new_row[p * 8 + seg];
                     if (c7 == (r & 7)) {
                         if (r < 8) kf[2 * p] = w; else kf[2 * p + 1] = w;
-                        *reinterpret_cast<v4u*>(P.kpool_w + here + (size_t)(p * 64 + seg * 8) * 2) = w;
                     }
                 }
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
-                    const v4u w = row_slice(nv + h * 128 + c * 8);
+                    const v4u w = new_row[32 + h * 16 + c];
                     if (g == (r >> 2)) {
 #pragma unroll
                         for (int rr = 0; rr < 4; ++rr)
                             if (rr == (r & 3)) vf[h][rr] = w;
-                        *reinterpret_cast<v4u*>(P.vpool_w + here + (size_t)(h * 128 + c * 8) * 2) = w;
                     }
                 }
             }
@@ -526,6 +538,8 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
     uint8_t* const ring0 = ring;
     uint8_t* const ring1 = ring + kWaves * kI8hSlot;
     constexpr int kRow = row_bytes_of(kRowI8H);  // 272
+    // STEP: the new K row and the new V row of the entry, encoded; one wave of a work-group at most
+    __shared__ __attribute__((aligned(16))) uint8_t parked[STEP ? 2 * kRow : 16];
 
     const int unit = blockIdx.x;
     int e, rem, pos, row, pps;
@@ -588,8 +602,54 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
     request(1, P.kpool, slot1);
     request(1, P.vpool, slot1 + kI8hUnit);
 
+    // STEP: the wave that will hold the page of cell pos (in its last step) takes the new rows before the
+    // loop, while its first units are on their way: the raw values are requested ahead of the q fragments
+    // (one wait covers both), then lanes 0..7 encode the K row and lanes 8..15 the V row with the append
+    // kernel's encoder, one lane per 32-value block, into the pool and into two parking rows in LDS.  In
+    // its last step the wave copies a parked row into the unit that has just landed (an LDS move instead
+    // of a trip to memory and an encode at the end of the work-group's walk).
+    const auto wave_lds_fence = [&]() {
+        // the wave's own LDS writes are in order with its later reads; keep the compiler from
+        // moving those reads up
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+    const bool takes_new_row = STEP && n_steps > 0 && pg0 + wave + kWaves * (n_steps - 1) == n_pages - 1;
+    float new_x[32];
+    if constexpr (STEP) {
+        if (takes_new_row && lane < 16) {
+            const float* src = (lane < 8 ? P.new_k : P.new_v) + ((size_t)e * P.n_kv + (size_t)kvh) * kHd + (lane & 7) * 32;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float4 a = *reinterpret_cast<const float4*>(src + 4 * j);
+                new_x[4 * j] = a.x, new_x[4 * j + 1] = a.y, new_x[4 * j + 2] = a.z, new_x[4 * j + 3] = a.w;
+            }
+        }
+    }
+
     half8 qhi[8], qlo[8];
     load_q_fragments(P, e, kvh, c, g, qhi, qlo);
+
+    if constexpr (STEP) {
+        if (takes_new_row) {
+            if (lane < 16) {
+                uint32_t w[8], hb;
+                i8h_block_words(new_x, w, hb);
+                const int r = pos & (kPage - 1);
+                const int blk = lane & 7;
+                uint8_t* const pool_row = (lane < 8 ? P.kpool_w : P.vpool_w) + unit_off(n_steps - 1) + (size_t)r * kRow;
+                uint8_t* const rows[2] = {parked + (lane < 8 ? 0 : kRow), pool_row};
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    *reinterpret_cast<v4u*>(rows[t] + blk * 32) = v4u{w[0], w[1], w[2], w[3]};
+                    *reinterpret_cast<v4u*>(rows[t] + blk * 32 + 16) = v4u{w[4], w[5], w[6], w[7]};
+                    *reinterpret_cast<unsigned short*>(rows[t] + kHd + 2 * blk) = (unsigned short)hb;
+                }
+            }
+            wave_lds_fence();
+        }
+    }
 
     f4 o[2][8];
 #pragma unroll
@@ -599,34 +659,13 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
     float m_run = -INFINITY;
     float l_run = 0.0f;
 
-    // STEP: the wave that holds the page of cell pos (always in its last step) encodes the new row
-    // with the append kernel's encoder, one lane per 32-value block, into the LDS unit that has
-    // just landed and into the pool.
-    const auto take_new_row = [&](const float* new_rows, uint8_t* lds_unit, uint8_t* pool_unit) {
-        if (lane < 8) {
-            float x[32];
-            const float* src = new_rows + ((size_t)e * P.n_kv + (size_t)kvh) * kHd + lane * 32;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const float4 a = *reinterpret_cast<const float4*>(src + 4 * j);
-                x[4 * j] = a.x, x[4 * j + 1] = a.y, x[4 * j + 2] = a.z, x[4 * j + 3] = a.w;
-            }
-            uint32_t w[8], hb;
-            i8h_block_words(x, w, hb);
-            const int r = pos & (kPage - 1);
-            uint8_t* const rows[2] = {lds_unit + r * kRow, pool_unit + (size_t)r * kRow};
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                *reinterpret_cast<v4u*>(rows[t] + lane * 32) = v4u{w[0], w[1], w[2], w[3]};
-                *reinterpret_cast<v4u*>(rows[t] + lane * 32 + 16) = v4u{w[4], w[5], w[6], w[7]};
-                *reinterpret_cast<unsigned short*>(rows[t] + kHd + 2 * lane) = (unsigned short)hb;
-            }
-        }
-        // the wave's own LDS writes are in order with its later reads; keep the compiler from
-        // moving those reads up
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // the parked row `which` (0 = K, 1 = V) into row pos % 16 of the unit that has just landed
+    const auto take_new_row = [&](int which, uint8_t* lds_unit) {
+        const int r = pos & (kPage - 1);
+        if (lane < kRow / 16)
+            *reinterpret_cast<v4u*>(lds_unit + r * kRow + lane * 16) =
+                *reinterpret_cast<const v4u*>(parked + which * kRow + lane * 16);
+        wave_lds_fence();
     };
 
     // One page: step i of the wave, resident in `slot`; the slot is refilled with step i + 2.
@@ -651,7 +690,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
         // ---- scores: per block, codes . q on the matrix core, then the block's scale ----------------
         __builtin_amdgcn_s_waitcnt(0x0F7F);  // vmcnt(15): this page's K unit has landed
         if constexpr (STEP) {
-            if (pg == n_pages - 1) take_new_row(P.new_k, slot, P.kpool_w + unit_off(i));
+            if (pg == n_pages - 1) take_new_row(0, slot);
         }
         f4 s = f4{0.0f, 0.0f, 0.0f, 0.0f};
         // all fragments of the unit are requested from LDS in one batch, ahead of the first use
@@ -688,7 +727,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
         // instructions then has the dequantisation to overlap with -----------------------------------
         __builtin_amdgcn_s_waitcnt(0x0F7F);  // vmcnt(15): this page's V unit has landed
         if constexpr (STEP) {
-            if (pg == n_pages - 1) take_new_row(P.new_v, slot + kI8hUnit, P.vpool_w + unit_off(i));
+            if (pg == n_pages - 1) take_new_row(1, slot + kI8hUnit);
         }
         // Scales of the lane's rows 4 g + r for its block of either half.  Rows past `pos` may hold
         // anything: their probabilities are exact zeros already, and their scales are made zeros
@@ -872,6 +911,8 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
     constexpr int kWaveLds = kQ8vKSlot + 2 * kQ8vUnit;
     constexpr int kLds = kWaves * kWaveLds > (int)sizeof(MfmaFoldLds) ? kWaves * kWaveLds : (int)sizeof(MfmaFoldLds);
     __shared__ __attribute__((aligned(16))) uint8_t smem[kLds];
+    // STEP: the new row of the entry, encoded (512 bytes of K, 288 of V); one wave of a work-group at most
+    __shared__ __attribute__((aligned(16))) uint8_t parked[STEP ? 512 + kQ8vRow : 16];
 
     const int unit = blockIdx.x;
     int e, rem, pos, row, pps;
@@ -944,8 +985,81 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
     request_k(0);
     request_v(1, slots + kQ8vUnit);
 
+    // STEP: the wave that will hold the page of cell pos (in its last step) encodes the new row before
+    // the loop, while its first units are on their way, as the append kernel does -- K under the f16
+    // rule, 8 values a lane; V as q8_0 blocks, one lane per block -- into the pool and into a parking
+    // row in LDS; in its last step it copies the parked row into the unit that has just landed (two LDS
+    // moves instead of a trip to memory and an encode at the end of the work-group's walk).
+    const auto wave_lds_fence = [&]() {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+    // the raw values are requested ahead of the q fragments (one wait covers both) and encoded after them
+    const bool takes_new_row = STEP && n_steps > 0 && pg0 + wave + kWaves * (n_steps - 1) == n_pages - 1;
+    float new_x[32];
+    if constexpr (STEP) {
+        if (takes_new_row) {
+            if (lane < 32) {
+                const float* src = P.new_k + ((size_t)e * P.n_kv + (size_t)kvh) * kHd + lane * 8;
+                const float4 a = *reinterpret_cast<const float4*>(src);
+                const float4 b = *reinterpret_cast<const float4*>(src + 4);
+                new_x[0] = a.x, new_x[1] = a.y, new_x[2] = a.z, new_x[3] = a.w;
+                new_x[4] = b.x, new_x[5] = b.y, new_x[6] = b.z, new_x[7] = b.w;
+            } else if (lane < 40) {
+                const float* src = P.new_v + ((size_t)e * P.n_kv + (size_t)kvh) * kHd + (lane - 32) * 32;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float4 a = *reinterpret_cast<const float4*>(src + 4 * j);
+                    new_x[4 * j] = a.x, new_x[4 * j + 1] = a.y, new_x[4 * j + 2] = a.z, new_x[4 * j + 3] = a.w;
+                }
+            }
+        }
+    }
+
     half8 qhi[8], qlo[8];
     load_q_fragments(P, e, kvh, c, g, qhi, qlo);
+
+    if constexpr (STEP) {
+        if (takes_new_row) {
+            const int r = pos & (kPage - 1);
+            const int i = n_steps - 1;
+            if (lane < 32) {
+                v4u w;
+                w.x = f16_store_pair(new_x[0], new_x[1]), w.y = f16_store_pair(new_x[2], new_x[3]);
+                w.z = f16_store_pair(new_x[4], new_x[5]), w.w = f16_store_pair(new_x[6], new_x[7]);
+                *reinterpret_cast<v4u*>(parked + lane * 16) = w;
+                *reinterpret_cast<v4u*>(P.kpool_w + phys(i) * k_page_bytes + k_head_off + (size_t)r * 512 + lane * 16) = w;
+            } else if (lane < 40) {
+                const int blk = lane - 32;
+                uint32_t w[9];
+                q8v_block_words(new_x, w);
+                uint32_t* const ld = reinterpret_cast<uint32_t*>(parked + 512 + blk * 36);
+                uint32_t* const gd = reinterpret_cast<uint32_t*>(P.vpool_w + phys(i) * v_page_bytes + v_head_off +
+                                                                  (size_t)r * kQ8vRow + blk * 36);
+#pragma unroll
+                for (int j = 0; j < 9; ++j) {
+                    ld[j] = w[j];
+                    gd[j] = w[j];
+                }
+            }
+            wave_lds_fence();
+        }
+    }
+    const auto take_new_k = [&]() {
+        const int r = pos & (kPage - 1);
+        if (lane < 32)
+            *reinterpret_cast<v4u*>(kslot + (r >> 1) * kQ8vKStep + (r & 1) * 512 + lane * 16) =
+                *reinterpret_cast<const v4u*>(parked + lane * 16);
+        wave_lds_fence();
+    };
+    const auto take_new_v = [&](uint8_t* lds_unit) {
+        const int r = pos & (kPage - 1);
+        if (lane < kQ8vRow / 16)
+            *reinterpret_cast<v4u*>(lds_unit + r * kQ8vRow + lane * 16) =
+                *reinterpret_cast<const v4u*>(parked + 512 + lane * 16);
+        wave_lds_fence();
+    };
 
     f4 o[2][8];
 #pragma unroll
@@ -955,52 +1069,6 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
     float m_run = -INFINITY;  // running maximum of logit + E (base 2)
     float l_run = 0.0f;       // this lane's share of sum exp2(logit - m_run)
     const int my_block = c >> 2;  // which of the 4 blocks of a half this lane's 8 columns lie in
-
-    // STEP: the wave that holds the page of cell pos (always in its last step) stores the new row
-    // as the append kernel does -- K under the f16 rule, 8 values a lane; V as q8_0 blocks, one lane
-    // per block -- into the LDS units that have just landed and into the pool.
-    const auto wave_lds_fence = [&]() {
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    };
-    const auto take_new_k = [&](int i) {
-        const int r = pos & (kPage - 1);
-        if (lane < 32) {
-            const float* src = P.new_k + ((size_t)e * P.n_kv + (size_t)kvh) * kHd + lane * 8;
-            const float4 a = *reinterpret_cast<const float4*>(src);
-            const float4 b = *reinterpret_cast<const float4*>(src + 4);
-            v4u w;
-            w.x = f16_store_pair(a.x, a.y), w.y = f16_store_pair(a.z, a.w);
-            w.z = f16_store_pair(b.x, b.y), w.w = f16_store_pair(b.z, b.w);
-            *reinterpret_cast<v4u*>(kslot + (r >> 1) * kQ8vKStep + (r & 1) * 512 + lane * 16) = w;
-            *reinterpret_cast<v4u*>(P.kpool_w + phys(i) * k_page_bytes + k_head_off + (size_t)r * 512 + lane * 16) = w;
-        }
-        wave_lds_fence();
-    };
-    const auto take_new_v = [&](int i, uint8_t* lds_unit) {
-        const int r = pos & (kPage - 1);
-        if (lane < 8) {
-            float x[32];
-            const float* src = P.new_v + ((size_t)e * P.n_kv + (size_t)kvh) * kHd + lane * 32;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const float4 a = *reinterpret_cast<const float4*>(src + 4 * j);
-                x[4 * j] = a.x, x[4 * j + 1] = a.y, x[4 * j + 2] = a.z, x[4 * j + 3] = a.w;
-            }
-            uint32_t w[9];
-            q8v_block_words(x, w);
-            uint32_t* const ld = reinterpret_cast<uint32_t*>(lds_unit + r * kQ8vRow + lane * 36);
-            uint32_t* const gd = reinterpret_cast<uint32_t*>(P.vpool_w + phys(i) * v_page_bytes + v_head_off +
-                                                              (size_t)r * kQ8vRow + lane * 36);
-#pragma unroll
-            for (int j = 0; j < 9; ++j) {
-                ld[j] = w[j];
-                gd[j] = w[j];
-            }
-        }
-        wave_lds_fence();
-    };
 
     for (int i = 0; i < n_steps; ++i) {
         const int pg = pg0 + wave + kWaves * i;
@@ -1024,7 +1092,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
         // ---- S^T = K . q^T: four independent accumulation chains ------------------------------
         __builtin_amdgcn_s_waitcnt(0x0F75);  // vmcnt(5): this page's K unit has landed
         if constexpr (STEP) {
-            if (pg == n_pages - 1) take_new_k(i);
+            if (pg == n_pages - 1) take_new_k();
         }
         v4u kf[8];
         {
@@ -1050,7 +1118,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
         // ---- this page's V unit: scales first -------------------------------------------------
         __builtin_amdgcn_s_waitcnt(0x4F75);  // vmcnt(21): K(i), V(i+1), K(i+1) behind V(i)
         if constexpr (STEP) {
-            if (pg == n_pages - 1) take_new_v(i, slots + (i & 1) * kQ8vUnit);
+            if (pg == n_pages - 1) take_new_v(slots + (i & 1) * kQ8vUnit);
         }
         // lane (c, g): scale of blocks 2 (c / 4), + 1 of row 4 g + c % 4, the row's maximum over the
         // lanes c, c ^ 4, c ^ 8, c ^ 12, then the four rows' maxima from the lanes of the quad
