@@ -25,6 +25,7 @@ struct MergeParams {
     float* out;
     int64_t gate_seq_stride, gate_head_stride;
     int32_t n_kv, n_q, group;
+    uint32_t inv_group16;  // small_divisor_inverse(group)
 };
 
 constexpr int kMergeGroups = 16;   // waves of a work-group; wave g sums splits g, g + 16, ...
@@ -43,10 +44,11 @@ __global__ __launch_bounds__(64 * kMergeGroups) void decode_attn_merge_kernel(co
     __shared__ __attribute__((aligned(16))) float red[kMergeGroups][kHd];
     __shared__ float red_l[kMergeGroups];
     __shared__ float wave_max[kMergeGroups];
-    const int e = blockIdx.x / P.n_q;
-    const int h = blockIdx.x % P.n_q;
-    const int kvh = h / P.group;
-    const int hl = h % P.group;
+    // grid (q heads, entries): no division at the head of a kernel that is all latency
+    const int e = blockIdx.y;
+    const int h = blockIdx.x;
+    const int kvh = small_div(h, P.inv_group16);
+    const int hl = h - kvh * P.group;
     int splits, base;
     if constexpr (DESC) {
         const batch_desc_ptr D = (batch_desc_ptr)(uintptr_t)P.bd;
@@ -70,6 +72,11 @@ __global__ __launch_bounds__(64 * kMergeGroups) void decode_attn_merge_kernel(co
         const int s = g + u * kMergeGroups;
         v[u] = s < splits ? *reinterpret_cast<const f4*>(po + (size_t)s * ostride) : f4{0.0f, 0.0f, 0.0f, 0.0f};
     }
+    // the gate of the element this thread writes at the end is requested with the partial rows, not after
+    // the sums (a trip to memory at the tail of a kernel that is all latency)
+    float gt = 0.0f;
+    if (P.gate && threadIdx.x < kHd)
+        gt = P.gate[(size_t)e * P.gate_seq_stride + (size_t)h * P.gate_head_stride + threadIdx.x];
     // stage (m, l) and agree on the maximum: per-thread max over its splits, wave reduction,
     // then one LDS slot per wave (a serial scan over the splits would cost a dependent LDS
     // round trip per split)
@@ -135,7 +142,6 @@ __global__ __launch_bounds__(64 * kMergeGroups) void decode_attn_merge_kernel(co
     }
     r = lt > 0.0f ? r / lt : 0.0f;
     if (P.gate) {
-        const float gt = P.gate[(size_t)e * P.gate_seq_stride + (size_t)h * P.gate_head_stride + d];
         // sigmoid in the overflow-free form of the reference (qsa/cpu.rs:84-91)
         float sg;
         if (gt >= 0.0f) {
@@ -224,6 +230,7 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
     kp.n_kv = n_kv;
     kp.n_q = a.n_q_head;
     kp.group = group;
+    kp.inv_kv16 = small_divisor_inverse(n_kv);
     kp.scale_log2e = a.scale * kLog2e;
     kp.ids = a.ids;
     kp.counts = a.counts;
@@ -254,7 +261,8 @@ hipError_t launch_decode_attn(bkv_pool* p, int32_t layer, const AttnBatch& b, co
     mp.n_kv = n_kv;
     mp.n_q = a.n_q_head;
     mp.group = group;
-    const dim3 mgrid((unsigned)(b.n * a.n_q_head)), mblock(64 * kMergeGroups);
+    mp.inv_group16 = small_divisor_inverse(group);
+    const dim3 mgrid((unsigned)a.n_q_head, (unsigned)b.n), mblock(64 * kMergeGroups);
     if (a.desc)
         hipLaunchKernelGGL(decode_attn_merge_kernel<true>, mgrid, mblock, 0, stream, mp);
     else if (a.timed)

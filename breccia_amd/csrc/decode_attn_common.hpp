@@ -29,6 +29,7 @@ struct AttnKernelParams {
     float* part_ml;
     int32_t max_pages_per_seq;
     int32_t n_kv, n_q, group;
+    uint32_t inv_kv16;  // small_divisor_inverse(n_kv): a work-group's index splits into (page range, kv head) without a division
     float scale_log2e;
     // selection lists (kernels instantiated with SEL only): entry e attends the 4-cell blocks
     // ids[e * id_stride + 0 .. min(counts[e], max_ids))
@@ -43,6 +44,15 @@ struct AttnKernelParams {
     uint8_t* kpool_w;
     uint8_t* vpool_w;
 };
+
+// x / d for the small numbers of this launch geometry, as a multiplication by ceil(2^16 / d): exact while
+// x * d < 2^16 (work-group indices stay below kMaxWgs = 4096, head indices below 256, divisors are kv head
+// counts and head groups of at most 16).  An integer division by a run-time value is some forty dependent
+// instructions at the head of kernels whose first microsecond is all latency.
+static_assert((int64_t)kMaxWgs * BKV_MAX_KV_HEAD <= 65536 && 256 * BKV_MAX_HEAD_GROUP <= 65536,
+              "small_div is exact only while x * d < 2^16");
+inline uint32_t small_divisor_inverse(int32_t d) { return (65536u + (uint32_t)d - 1u) / (uint32_t)d; }
+__device__ __forceinline__ int small_div(int x, uint32_t inv16) { return (int)(((uint32_t)x * inv16) >> 16); }
 
 // Which unit of work a work-group of the matrix-core kernels has: entry e, its rem-th work-group
 // (page range x kv head), and the entry's position, block-table row and pages per range.  With DESC the

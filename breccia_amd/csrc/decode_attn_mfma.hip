@@ -153,7 +153,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
     const int unit = blockIdx.x;
     int e, rem, pos, row, pps;
     if (!unit_of_work_group<DESC>(P, unit, e, rem, pos, row, pps)) return;
-    const int split = rem / P.n_kv;
+    const int split = small_div(rem, P.inv_kv16);
     const int kvh = rem - split * P.n_kv;
     const int wg = unit;
     typedef const __attribute__((address_space(4))) int32_t* table_ptr;
@@ -544,7 +544,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
     const int unit = blockIdx.x;
     int e, rem, pos, row, pps;
     if (!unit_of_work_group<DESC>(P, unit, e, rem, pos, row, pps)) return;
-    const int split = rem / P.n_kv;
+    const int split = small_div(rem, P.inv_kv16);
     const int kvh = rem - split * P.n_kv;
     const int wg = unit;
     const block_table_ptr bt = (block_table_ptr)(uintptr_t)(P.tables + (size_t)row * (size_t)P.max_pages_per_seq);
@@ -917,7 +917,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
     const int unit = blockIdx.x;
     int e, rem, pos, row, pps;
     if (!unit_of_work_group<DESC>(P, unit, e, rem, pos, row, pps)) return;
-    const int split = rem / P.n_kv;
+    const int split = small_div(rem, P.inv_kv16);
     const int kvh = rem - split * P.n_kv;
     const int wg = unit;
     const block_table_ptr bt = (block_table_ptr)(uintptr_t)(P.tables + (size_t)row * (size_t)P.max_pages_per_seq);
