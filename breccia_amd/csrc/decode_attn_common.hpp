@@ -73,6 +73,9 @@ __device__ __forceinline__ bool unit_of_work_group(const AttnKernelParams& P, in
         row = D->row[e];
         pps = D->pps[e];
     } else {
+        // entry 0's fields are asked for alongside n: their cache lines (sixteen entries each) are then on
+        // their way before the entry is known
+        asm volatile("" ::"s"(P.b.pos[0]), "s"(P.b.pps[0]), "s"(P.b.row[0]), "s"(P.b.wg_base[0]));
         e = 0;
         while (e + 1 < P.b.n && unit >= P.b.wg_base[e + 1]) ++e;
         rem = unit - P.b.wg_base[e];
