@@ -445,14 +445,14 @@ __device__ __forceinline__ half8 codes8_to_f16(v2u w) {
     return half8{a[0], a[1], b[0], b[1], c2[0], c2[1], d[0], d[1]};
 }
 
-// Data path: rows reach the matrix cores through LDS, not through registers.  Every wave owns two
-// slots of 2 x 4352 bytes (the K unit and the V unit of one page and kv head, scales included)
-// and fills them with 16-byte global->LDS loads, 64 lanes x 16 contiguous bytes per instruction
-// (whole cache lines, nothing fetched twice), two pages ahead of the page it computes: the K half
-// of a slot is refilled right after the scores that read it, the V half right after P.V (whose
-// fragments are requested before the softmax, so that their dequantisation overlaps it).  A
-// wave has 20 such loads in flight in a fixed order (K, V of the next page, K, V of the one
-// after), so "the oldest five have landed" is s_waitcnt vmcnt(15) at both points of use.
+// Data path: rows reach the matrix cores through LDS, because a lane's MFMA fragments are scattered
+// over a row of codes and scales, but they travel there through registers: a wave fetches the K
+// unit and the V unit of its next page (2 x 4352 bytes: one page and kv head, scales included) with
+// ordinary coalesced loads -- 64 lanes x 16 contiguous bytes per instruction, whole cache lines, 17
+// registers a unit -- while it multiplies the page before, and deposits them into its one LDS slot
+// when it gets there.  (Direct global->LDS loads save the registers and the deposit, and stream
+// 10 % slower on this chip: 6.0 against 6.7 TB/s for the same random 4 KiB chunks in this launch
+// shape, measured with a probe; the kernel had been bound by that, not by its arithmetic.)
 constexpr int kI8hUnit = kPage * row_bytes_of(kRowI8H);  // 4352
 constexpr int kI8hSlot = 2 * kI8hUnit;                    // K unit, then V unit
 
@@ -496,35 +496,23 @@ __device__ __forceinline__ uint32_t pick4(const uint32_t (&a)[4], int j) {
     return j == 0 ? a[0] : j == 1 ? a[1] : j == 2 ? a[2] : a[3];
 }
 
-// 4352 bytes = 4 x 1024 + 256: four full instructions and one of 16 lanes.  `real` false issues the
-// same five instructions on one 16-byte location (the data is never used): the number of loads
-// in flight, which the waits count, then does not depend on where in its range a wave is.
+// One unit between memory and LDS: 4352 bytes = 64 lanes x (4 x 16 + 4).
+struct I8hUnitRegs {
+    v4u q[4];
+    unsigned tail;
+};
 template <bool SEL>
-__device__ __forceinline__ void i8h_unit_to_lds(const UnitSrc<SEL>& src, bool real, uint8_t* dst, int lane) {
-    typedef const __attribute__((address_space(1))) void* gptr;
-    typedef __attribute__((address_space(3))) void* lptr;
+__device__ __forceinline__ void i8h_unit_fetch(const UnitSrc<SEL>& src, int lane, I8hUnitRegs& r) {
     constexpr int kRun = 4 * row_bytes_of(kRowI8H);
-    if constexpr (!SEL) {
-        // one run: a single address, the pieces as immediate offsets of the instruction (they move the
-        // place in memory and the place in LDS alike); a wave past its last page asks for five
-        // pieces at the head of the unit it last read
-        const uint8_t* a = src.run[0] + (real ? lane * 16 : 0);
-        __builtin_amdgcn_global_load_lds((gptr)a, (lptr)dst, 16, 0, 0);
-        __builtin_amdgcn_global_load_lds((gptr)a, (lptr)dst, 16, 1024, 0);
-        __builtin_amdgcn_global_load_lds((gptr)a, (lptr)dst, 16, 2048, 0);
-        __builtin_amdgcn_global_load_lds((gptr)a, (lptr)dst, 16, 3072, 0);
-        if (lane < 16) __builtin_amdgcn_global_load_lds((gptr)(a + 4096), (lptr)(dst + 4096), 16, 0, 0);
-        return;
-    }
 #pragma unroll
-    for (int n = 0; n < 4; ++n) {
-        const uint8_t* a = real ? unit_piece<SEL, kRun>(src, n * 1024 + lane * 16) : src.run[0];
-        __builtin_amdgcn_global_load_lds((gptr)a, (lptr)(dst + n * 1024), 16, 0, 0);
-    }
-    if (lane < 16) {
-        const uint8_t* a = real ? unit_piece<SEL, kRun>(src, 4096 + lane * 16) : src.run[0];
-        __builtin_amdgcn_global_load_lds((gptr)a, (lptr)(dst + 4096), 16, 0, 0);
-    }
+    for (int n = 0; n < 4; ++n)
+        r.q[n] = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(unit_piece<SEL, kRun>(src, n * 1024 + lane * 16)));
+    r.tail = __builtin_nontemporal_load(reinterpret_cast<const unsigned*>(unit_piece<SEL, kRun>(src, 4096 + lane * 4)));
+}
+__device__ __forceinline__ void i8h_unit_deposit(const I8hUnitRegs& r, uint8_t* dst, int lane) {
+#pragma unroll
+    for (int n = 0; n < 4; ++n) *reinterpret_cast<v4u*>(dst + n * 1024 + lane * 16) = r.q[n];
+    *reinterpret_cast<unsigned*>(dst + 4096 + lane * 4) = r.tail;
 }
 
 // SEL: an iteration's 16 rows are four listed 4-cell blocks (see decode_attn_mfma_kernel); the
@@ -532,11 +520,9 @@ __device__ __forceinline__ void i8h_unit_to_lds(const UnitSrc<SEL>& src, bool re
 template <bool STEP, bool DESC = false, bool SEL = false>
 __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const AttnKernelParams P) {
     static_assert(!(STEP && SEL), "the fused step attends the dense selection");
-    // slot 0 and slot 1 of the four waves; the fold staging of the epilogue reuses their memory
-    __shared__ __attribute__((aligned(16))) uint8_t ring[2 * kWaves * kI8hSlot];
-    static_assert(sizeof(MfmaFoldLds) <= sizeof(ring), "fold staging must fit the slots");
-    uint8_t* const ring0 = ring;
-    uint8_t* const ring1 = ring + kWaves * kI8hSlot;
+    // one slot per wave; the fold staging of the epilogue reuses the memory
+    constexpr int kRing = kWaves * kI8hSlot > (int)sizeof(MfmaFoldLds) ? kWaves * kI8hSlot : (int)sizeof(MfmaFoldLds);
+    __shared__ __attribute__((aligned(16))) uint8_t ring[kRing];
     constexpr int kRow = row_bytes_of(kRowI8H);  // 272
     // STEP: the new K row and the new V row of the entry, encoded; one wave of a work-group at most
     __shared__ __attribute__((aligned(16))) uint8_t parked[STEP ? 2 * kRow : 16];
@@ -566,11 +552,9 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
     const int my_block = c >> 2;  // which of the 4 blocks of a half this lane's 8 columns lie in
     const size_t page_bytes = (size_t)P.n_kv * kI8hUnit;
     const size_t head_off = (size_t)kvh * kI8hUnit;
-    uint8_t* const slot0 = ring0 + wave * kI8hSlot;
-    uint8_t* const slot1 = ring1 + wave * kI8hSlot;
+    uint8_t* const slot = ring + wave * kI8hSlot;
 
-    // unit of pipeline step i of this wave; steps past the wave's last are requested all the same,
-    // as loads of one location, so that the number of loads in flight stays what the waits assume
+    // pipeline steps of this wave: pages pg0 + wave, + kWaves, ...
     const int n_steps = pg0 + wave < pg1 ? (pg1 - pg0 - wave + kWaves - 1) / kWaves : 0;
     const auto unit_off = [&](int i) -> size_t {
         return (size_t)bt[min(pg0 + wave + kWaves * i, pg1 - 1)] * page_bytes + head_off;
@@ -592,15 +576,16 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
             u.run[0] = pool + (n_steps > 0 ? unit_off(i) : 0);
         }
     };
-    const auto request = [&](int i, const uint8_t* pool, uint8_t* dst) {
+    // the page in flight: requested while the page before is multiplied
+    I8hUnitRegs k_regs, v_regs;
+    const auto fetch = [&](int i) {
         UnitSrc<SEL> u;
-        unit_src(i, pool, u);
-        i8h_unit_to_lds<SEL>(u, i < n_steps, dst, lane);
+        unit_src(i, P.kpool, u);
+        i8h_unit_fetch<SEL>(u, lane, k_regs);
+        unit_src(i, P.vpool, u);
+        i8h_unit_fetch<SEL>(u, lane, v_regs);
     };
-    request(0, P.kpool, slot0);
-    request(0, P.vpool, slot0 + kI8hUnit);
-    request(1, P.kpool, slot1);
-    request(1, P.vpool, slot1 + kI8hUnit);
+    if (n_steps > 0) fetch(0);
 
     // STEP: the wave that will hold the page of cell pos (in its last step) takes the new rows before the
     // loop, while its first units are on their way: the raw values are requested ahead of the q fragments
@@ -668,11 +653,22 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
         wave_lds_fence();
     };
 
-    // One page: step i of the wave, resident in `slot`; the slot is refilled with step i + 2.
-    const auto one_page = [&](uint8_t* slot, int i) __attribute__((always_inline)) {
+    // One page: step i of the wave.  Its units arrive in the registers; they go into the slot and the
+    // registers take the request for step i + 1.
+    const auto one_page = [&](int i) __attribute__((always_inline)) {
         const int pg = pg0 + wave + kWaves * i;
         const uint8_t* ks = slot;
         const uint8_t* vs = slot + kI8hUnit;
+        i8h_unit_deposit(k_regs, slot, lane);
+        i8h_unit_deposit(v_regs, slot + kI8hUnit, lane);
+        if (i + 1 < n_steps) fetch(i + 1);
+        wave_lds_fence();
+        if constexpr (STEP) {
+            if (pg == n_pages - 1) {
+                take_new_row(0, slot);
+                take_new_row(1, slot + kI8hUnit);
+            }
+        }
         // which of the lane's four cells are attended: up to `pos`, or the live cells of listed blocks
         bool live[4];
         if constexpr (SEL) {
@@ -688,10 +684,6 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
         }
 
         // ---- scores: per block, codes . q on the matrix core, then the block's scale ----------------
-        __builtin_amdgcn_s_waitcnt(0x0F7F);  // vmcnt(15): this page's K unit has landed
-        if constexpr (STEP) {
-            if (pg == n_pages - 1) take_new_row(0, slot);
-        }
         f4 s = f4{0.0f, 0.0f, 0.0f, 0.0f};
         // all fragments of the unit are requested from LDS in one batch, ahead of the first use
         half8 ksc[4];
@@ -721,14 +713,9 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
 #pragma unroll
             for (int r = 0; r < 4; ++r) s[r] = fmaf((float)ksc[r][m], part[r], s[r]);
         }
-        request(i + 2, P.kpool, slot);
 
         // ---- this page's V fragments are requested before the softmax, whose chain of dependent
         // instructions then has the dequantisation to overlap with -----------------------------------
-        __builtin_amdgcn_s_waitcnt(0x0F7F);  // vmcnt(15): this page's V unit has landed
-        if constexpr (STEP) {
-            if (pg == n_pages - 1) take_new_row(1, slot + kI8hUnit);
-        }
         // Scales of the lane's rows 4 g + r for its block of either half.  Rows past `pos` may hold
         // anything: their probabilities are exact zeros already, and their scales are made zeros
         // too, so that 0 * (garbage scale) cannot produce a NaN (any int8 code is a finite number).
@@ -825,13 +812,11 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
                 o[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahl, pll, o[h][t], 0, 0, 0);
             }
         }
-        request(i + 2, P.vpool, slot + kI8hUnit);
     };
 
-    for (int i = 0; i < n_steps; ++i) one_page((i & 1) ? slot1 : slot0, i);
+    for (int i = 0; i < n_steps; ++i) one_page(i);
 
-    // no load may still be on its way into the slots when the fold staging takes their place
-    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0)
+    // every wave is done with its slot before the fold staging takes their place
     __syncthreads();
     mfma_fold_and_store(P, *reinterpret_cast<MfmaFoldLds*>(ring), wg, wave, c, g, o, m_run, l_run);
 }
