@@ -823,10 +823,10 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
 
 // ---- decode attention on the matrix cores, f16 K and q8_0 V -----------------------------------
 // The MFMA decomposition of decode_attn_mfma_kernel with both operands staged through LDS like the
-// int8 kernel's units (every load of the loop is then a global->LDS load, which keeps the count of
-// loads in flight, and with it every wait, exact): the f16 K unit of the next page is requested
-// when the scores have used this page's, the V units ([f32 scale][32 x i8] blocks, 288 bytes a
-// row) two pages ahead.  A q8_0 value is code * scale with an f32 scale, so it takes a per-cell
+// int8 kernel's units: the f16 K unit (8 KiB) and the V unit ([f32 scale][32 x i8] blocks, 288
+// bytes a row) of the next page are fetched into registers with coalesced loads while this page
+// is multiplied, and deposited into the wave's slot when the page is reached.  A q8_0 value is
+// code * scale with an f32 scale, so it takes a per-cell
 // power of two out first to stay inside f16:
 //   E[cell]  = exponent of the largest of the cell's 8 block scales (clamped to +-120),
 //   a[cell][d] = code * (scale * 2^-E[cell])       |a| < 256; split into hi + lo f16 as below,
@@ -845,55 +845,46 @@ constexpr int kQ8vUnit = kPage * kQ8vRow;      // 4608
 // fragment read touches spread over the banks.
 constexpr int kQ8vKStep = 1024 + 32;
 constexpr int kQ8vKSlot = 8 * kQ8vKStep;  // 8448
+// A K unit between memory and LDS: instruction n moves rows 2 n and 2 n + 1 (of a selection list,
+// half of block n / 2).
 template <bool SEL>
-__device__ __forceinline__ void q8v_k_unit_to_lds(const UnitSrc<SEL>& src, bool real, uint8_t* dst, int lane) {
-    typedef const __attribute__((address_space(1))) void* gptr;
-    typedef __attribute__((address_space(3))) void* lptr;
+__device__ __forceinline__ void q8v_k_unit_fetch(const UnitSrc<SEL>& src, int lane, v4u (&r)[8]) {
 #pragma unroll
     for (int n = 0; n < 8; ++n) {
-        // instruction n moves rows 2 n and 2 n + 1: of a selection list, half of block n / 2
-        const uint8_t* a = !real ? src.run[0]
-                           : SEL ? src.run[SEL ? n >> 1 : 0] + (n & 1) * 1024 + lane * 16
-                                 : src.run[0] + n * 1024 + lane * 16;
-        __builtin_amdgcn_global_load_lds((gptr)a, (lptr)(dst + n * kQ8vKStep), 16, 0, 0);
+        const uint8_t* a = SEL ? src.run[SEL ? n >> 1 : 0] + (n & 1) * 1024 + lane * 16 : src.run[0] + n * 1024 + lane * 16;
+        r[n] = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(a));
     }
 }
-
-// 4608 bytes = 4 x 1024 + 512: four full instructions and one of 32 lanes.  `real` false issues the
-// same five instructions on one 16-byte location (the data is never used): the number of loads
-// in flight, which the waits count, then does not depend on where in its range a wave is.
-template <bool SEL>
-__device__ __forceinline__ void q8v_unit_to_lds(const UnitSrc<SEL>& src, bool real, uint8_t* dst, int lane) {
-    typedef const __attribute__((address_space(1))) void* gptr;
-    typedef __attribute__((address_space(3))) void* lptr;
-    constexpr int kRun = 4 * kQ8vRow;
-    if constexpr (!SEL) {
-        // one run: a single address and immediate offsets, as in i8h_unit_to_lds
-        const uint8_t* a = src.run[0] + (real ? lane * 16 : 0);
-        __builtin_amdgcn_global_load_lds((gptr)a, (lptr)dst, 16, 0, 0);
-        __builtin_amdgcn_global_load_lds((gptr)a, (lptr)dst, 16, 1024, 0);
-        __builtin_amdgcn_global_load_lds((gptr)a, (lptr)dst, 16, 2048, 0);
-        __builtin_amdgcn_global_load_lds((gptr)a, (lptr)dst, 16, 3072, 0);
-        if (lane < 32) __builtin_amdgcn_global_load_lds((gptr)(a + 4096), (lptr)(dst + 4096), 16, 0, 0);
-        return;
-    }
+__device__ __forceinline__ void q8v_k_unit_deposit(const v4u (&r)[8], uint8_t* dst, int lane) {
 #pragma unroll
-    for (int n = 0; n < 4; ++n) {
-        const uint8_t* a = real ? unit_piece<SEL, kRun>(src, n * 1024 + lane * 16) : src.run[0];
-        __builtin_amdgcn_global_load_lds((gptr)a, (lptr)(dst + n * 1024), 16, 0, 0);
-    }
-    if (lane < 32) {
-        const uint8_t* a = real ? unit_piece<SEL, kRun>(src, 4096 + lane * 16) : src.run[0];
-        __builtin_amdgcn_global_load_lds((gptr)a, (lptr)(dst + 4096), 16, 0, 0);
-    }
+    for (int n = 0; n < 8; ++n) *reinterpret_cast<v4u*>(dst + n * kQ8vKStep + lane * 16) = r[n];
+}
+
+// A V unit: 4608 bytes = 64 lanes x (4 x 16 + 8).
+struct Q8vUnitRegs {
+    v4u q[4];
+    v2u tail;
+};
+template <bool SEL>
+__device__ __forceinline__ void q8v_unit_fetch(const UnitSrc<SEL>& src, int lane, Q8vUnitRegs& r) {
+    constexpr int kRun = 4 * kQ8vRow;
+#pragma unroll
+    for (int n = 0; n < 4; ++n)
+        r.q[n] = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(unit_piece<SEL, kRun>(src, n * 1024 + lane * 16)));
+    r.tail = __builtin_nontemporal_load(reinterpret_cast<const v2u*>(unit_piece<SEL, kRun>(src, 4096 + lane * 8)));
+}
+__device__ __forceinline__ void q8v_unit_deposit(const Q8vUnitRegs& r, uint8_t* dst, int lane) {
+#pragma unroll
+    for (int n = 0; n < 4; ++n) *reinterpret_cast<v4u*>(dst + n * 1024 + lane * 16) = r.q[n];
+    *reinterpret_cast<v2u*>(dst + 4096 + lane * 8) = r.tail;
 }
 
 // SEL: an iteration's 16 rows are four listed 4-cell blocks, as in the int8 kernel.
 template <bool STEP, bool DESC = false, bool SEL = false>
 __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const AttnKernelParams P) {
     static_assert(!(STEP && SEL), "the fused step attends the dense selection");
-    // per wave one K slot and two V slots during the loop, the fold staging after it
-    constexpr int kWaveLds = kQ8vKSlot + 2 * kQ8vUnit;
+    // per wave one K slot and one V slot during the loop, the fold staging after it
+    constexpr int kWaveLds = kQ8vKSlot + kQ8vUnit;
     constexpr int kLds = kWaves * kWaveLds > (int)sizeof(MfmaFoldLds) ? kWaves * kWaveLds : (int)sizeof(MfmaFoldLds);
     __shared__ __attribute__((aligned(16))) uint8_t smem[kLds];
     // STEP: the new row of the entry, encoded (512 bytes of K, 288 of V); one wave of a work-group at most
@@ -932,11 +923,6 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
     // physical page of step i; past the wave's last step the answer is not used for its data
     const auto phys = [&](int i) -> size_t { return (size_t)bt[min(pg0 + wave + kWaves * i, pg1 - 1)]; };
 
-    // Loads complete in order.  Issue order per step: K(i+1) when the scores of step i are done,
-    // V(i+2) at its end; the prologue keeps that order (V0, K0, V1).  Behind K(i) at the top of step
-    // i there is V(i+1) = 5 loads; behind V(i) where step i needs it there are K(i), V(i+1), K(i+1)
-    // = 8 + 5 + 8.  Steps that do not exist are requested all the same, as loads of one location,
-    // so that these counts hold everywhere.
     const auto unit_src = [&](int i, bool is_k, UnitSrc<SEL>& u) {
         const uint8_t* pool = is_k ? P.kpool : P.vpool;
         if constexpr (SEL) {
@@ -956,19 +942,17 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
                                    : pool;
         }
     };
-    const auto request_k = [&](int i) {
+    // the page in flight: requested while the page before is multiplied
+    v4u k_regs[8];
+    Q8vUnitRegs v_regs;
+    const auto fetch = [&](int i) {
         UnitSrc<SEL> u;
         unit_src(i, true, u);
-        q8v_k_unit_to_lds<SEL>(u, i < n_steps, kslot, lane);
-    };
-    const auto request_v = [&](int i, uint8_t* dst) {
-        UnitSrc<SEL> u;
+        q8v_k_unit_fetch<SEL>(u, lane, k_regs);
         unit_src(i, false, u);
-        q8v_unit_to_lds<SEL>(u, i < n_steps, dst, lane);
+        q8v_unit_fetch<SEL>(u, lane, v_regs);
     };
-    request_v(0, slots);
-    request_k(0);
-    request_v(1, slots + kQ8vUnit);
+    if (n_steps > 0) fetch(0);
 
     // STEP: the wave that will hold the page of cell pos (in its last step) encodes the new row before
     // the loop, while its first units are on their way, as the append kernel does -- K under the f16
@@ -1057,7 +1041,19 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
 
     for (int i = 0; i < n_steps; ++i) {
         const int pg = pg0 + wave + kWaves * i;
-        const uint8_t* vs = slots + (i & 1) * kQ8vUnit;
+        const uint8_t* vs = slots;
+        // this page's units arrive in the registers: into the slots with them, and the registers take
+        // the request for the next page
+        q8v_k_unit_deposit(k_regs, kslot, lane);
+        q8v_unit_deposit(v_regs, slots, lane);
+        if (i + 1 < n_steps) fetch(i + 1);
+        wave_lds_fence();
+        if constexpr (STEP) {
+            if (pg == n_pages - 1) {
+                take_new_k();
+                take_new_v(slots);
+            }
+        }
         bool live[4];       // the lane's cells 4 g + r
         bool live_mine;     // cell 4 g + c % 4
         if constexpr (SEL) {
@@ -1075,10 +1071,6 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
         }
 
         // ---- S^T = K . q^T: four independent accumulation chains ------------------------------
-        __builtin_amdgcn_s_waitcnt(0x0F75);  // vmcnt(5): this page's K unit has landed
-        if constexpr (STEP) {
-            if (pg == n_pages - 1) take_new_k();
-        }
         v4u kf[8];
         {
             // row c: two rows per 1056-byte step; fragment m of lane group g at 64 m + 16 g
@@ -1098,13 +1090,8 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
             s3 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kb, qlo[m + 1], s3, 0, 0, 0);
         }
         const f4 s = (s0 + s1) + (s2 + s3);  // s[r] = q[head c] . k[cell 4 g + r]
-        request_k(i + 1);
 
         // ---- this page's V unit: scales first -------------------------------------------------
-        __builtin_amdgcn_s_waitcnt(0x4F75);  // vmcnt(21): K(i), V(i+1), K(i+1) behind V(i)
-        if constexpr (STEP) {
-            if (pg == n_pages - 1) take_new_v(slots + (i & 1) * kQ8vUnit);
-        }
         // lane (c, g): scale of blocks 2 (c / 4), + 1 of row 4 g + c % 4, the row's maximum over the
         // lanes c, c ^ 4, c ^ 8, c ^ 12, then the four rows' maxima from the lanes of the quad
         const bool last_page = SEL || pg == n_pages - 1;
@@ -1207,11 +1194,9 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
                 o[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahl, wll, o[h][t], 0, 0, 0);
             }
         }
-        request_v(i + 2, slots + (i & 1) * kQ8vUnit);
     }
 
-    // no load may still be on its way into the slots when the fold staging takes their place
-    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0)
+    // every wave is done with its slots before the fold staging takes their place
     __syncthreads();
     mfma_fold_and_store(P, *reinterpret_cast<MfmaFoldLds*>(smem), wg, wave, c, g, o, m_run, l_run);
 }
