@@ -899,7 +899,8 @@ def bench_moves(stream) -> dict:
     # (what a shuffled pool looks like to the attention kernels) -- the ceiling a read-only kernel
     # can be held against on this box
     sink = DeviceBuffer(16)
-    for name, scattered in (("device_read_probe_linear", 0), ("device_read_probe_scattered", 1)):
+    for name, scattered in (("device_read_probe_linear", 0), ("device_read_probe_scattered", 1),
+                            ("device_read_probe_scattered_via_lds_loads", 2)):
         ms = timed(lambda: check(lib.bkv_read_probe(a.ptr, 512 << 20, scattered, sink.ptr, stream.handle)), 20)
         res[name] = {"bytes_read": 512 << 20, "ms": round(ms, 4), "GBps": round((512 << 20) / ms / 1e6, 1),
                      "frac_of_hbm_peak": round((512 << 20) / ms / 1e6 / HBM_PEAK_GBPS, 4)}

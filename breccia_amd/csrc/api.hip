@@ -2016,10 +2016,13 @@ bkv_status bkv_read_probe(const void* src_dev, uint64_t bytes, int32_t scattered
     if (bytes % 8192 != 0 || chunks == 0 || chunks > 0x7fffffffull || (chunks & (chunks - 1)) != 0)
         return fail(BKV_ERR_INVALID, sfmt("read_probe: %lld bytes; need a power-of-two number of 8 KiB chunks",
                                           (long long)bytes));
+    if (scattered < 0 || scattered > 2)
+        return fail(BKV_ERR_INVALID, sfmt("read_probe: order %lld (0 = address order, 1 = scattered, 2 = scattered "
+                                          "through global->LDS loads)", scattered));
     int dev = 0, n_cu = 0;
     BKV_HIP(hipGetDevice(&dev));
     BKV_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
-    BKV_HIP(launch_read_probe(src_dev, bytes, scattered != 0, sink_dev, n_cu, S(stream)));
+    BKV_HIP(launch_read_probe(src_dev, bytes, scattered, sink_dev, n_cu, S(stream)));
     return BKV_OK;
 }
 

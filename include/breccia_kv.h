@@ -546,10 +546,13 @@ bkv_status bkv_device_info(char *name_out, int32_t name_cap, int32_t *cu_out,
  * (used to scale profiler byte counters and to report the copy ceiling). */
 bkv_status bkv_copy_probe(void *dst_dev, const void *src_dev, uint64_t bytes, void *stream);
 /* Read-only bandwidth probe: reads `bytes` (a power-of-two number of 8 KiB chunks -- the size of
- * one (page, kv head) run of an f16 pool) once, 8 KiB per wave at a time, in address order or
- * (scattered != 0) in a fixed pseudo-random order of chunks, as the attention kernels see a
- * shuffled pool; nothing is written except, never in practice, one word at sink_dev.  The rate
- * it reaches is the ceiling a read-only kernel can be held against on a given box. */
+ * one (page, kv head) run of an f16 pool) once, 8 KiB per wave at a time, in address order
+ * (scattered = 0), in a fixed pseudo-random order of chunks (1), as the attention kernels see a
+ * shuffled pool, or in that order with every chunk fetched by global->LDS loads instead of loads
+ * into registers (2: the slower of the two ways a row can reach LDS on this chip, kept so that the
+ * comparison behind the quantised kernels' data path can be repeated); nothing is written
+ * except, never in practice, one word at sink_dev.  The rate it reaches is the ceiling a
+ * read-only kernel can be held against on a given box. */
 bkv_status bkv_read_probe(const void *src_dev, uint64_t bytes, int32_t scattered, void *sink_dev,
                           void *stream);
 

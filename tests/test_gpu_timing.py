@@ -127,8 +127,13 @@ def test_read_probe_accepts_whole_power_of_two_chunk_counts_only():
     from breccia_amd.kv import BkvError, DeviceBuffer, check, device_sync, lib
 
     buf, sink = DeviceBuffer(1 << 20), DeviceBuffer(16)
-    for scattered in (0, 1):
+    for scattered in (0, 1, 2):
         check(lib.bkv_read_probe(buf.ptr, 1 << 20, scattered, sink.ptr, None))
+    check(lib.bkv_read_probe(buf.ptr, 8192, 2, sink.ptr, None))
+    for bad_order in (-1, 3):
+        with pytest.raises(BkvError) as ei:
+            check(lib.bkv_read_probe(buf.ptr, 1 << 20, bad_order, sink.ptr, None))
+        assert ei.value.status == L.ERR_INVALID
     check(lib.bkv_read_probe(buf.ptr, 8192, 1, sink.ptr, None))
     device_sync()
     for bad in (0, 8191, 3 * 8192, (1 << 20) + 16):
