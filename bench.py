@@ -827,8 +827,29 @@ def bench_moves(stream) -> dict:
     res["append_kprep_bulk"]["kernel_ms"] = round(ms_k / max(n_k, 1), 4)
     gd.free()
     td.free()
-    kd.free()
-    vd.free()
+    # the quantised layouts on the same bulk shape: f32 rows in, and raw f16 rows in (BASELINE
+    # configs[4]: "quantized from N(0,1) f16 on append")
+    k16 = DeviceBuffer.from_numpy(rng.standard_normal((4 * T, N_KV, HD), dtype=np.float32).astype(np.float16))
+    v16 = DeviceBuffer.from_numpy(rng.standard_normal((4 * T, N_KV, HD), dtype=np.float32).astype(np.float16))
+    for tag, layout, out_bytes in (("q8v", L.LAYOUT_Q8V, ROW_BYTES_Q8V), ("i8h", L.LAYOUT_I8H, ROW_BYTES_I8H)):
+        qp = Pool(n_layers=1, n_pages=4 * T // PAGE + 8, n_kv_head=N_KV, head_dim=HD, max_seqs=8,
+                  max_pages_per_seq=T // PAGE + 8, layout=layout)
+        qp.set_free_order(rng.permutation(4 * T // PAGE + 8).astype(np.int32))
+        qs = [qp.seq_create() for _ in range(4)]
+        for s in qs:
+            qp.seq_reserve(s, T)
+        for name, f16_rows, in_bytes in (("append_bulk_" + tag, False, N_KV * HD * 4 * 2),
+                                         ("append_bulk_%s_f16_rows" % tag, True, N_KV * HD * 2 * 2)):
+            ks, vs = (k16, v16) if f16_rows else (kd, vd)
+            ms = timed(lambda: qp.append(0, qs, [0] * 4, [T] * 4, ks, vs, stream, f16_rows=f16_rows), 20)
+            b = 4 * T * (in_bytes + out_bytes)
+            res[name] = {"tokens": 4 * T, "bytes_per_token": in_bytes + out_bytes, "ms": round(ms, 4),
+                         "GBps": round(b / ms / 1e6, 1), "frac_of_hbm_peak": round(b / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+        ms = timed(lambda: qp.append(0, qs, [7] * 4, [1] * 4, kd, vd, stream), 200)
+        res["append_decode_%s_us" % tag] = round(ms * 1e3, 2)
+        qp.destroy()
+    for x in (kd, vd, k16, v16):
+        x.free()
 
     # page copy: 16384 pairs = 512 MiB read + 512 MiB written
     used = np.concatenate([pool.block_table(s) for s in seqs])

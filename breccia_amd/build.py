@@ -88,5 +88,16 @@ def build_tree_sanitize_test(verbose: bool = False) -> str:
     return out
 
 
+def build_quant_arith_test(verbose: bool = False) -> str:
+    """The exhaustive CPU check of the int8 append's code arithmetic for binary16 rows (tests/cpp)."""
+    root = os.path.abspath(os.path.join(HERE, ".."))
+    out = os.path.join(root, "tests", "cpp", "i8h_f16_codes_exhaustive")
+    cmd = ["gcc", "-O2", "-fopenmp", "-ffp-contract=off", out + ".c", "-o", out, "-lm"]
+    if verbose:
+        print(" ".join(cmd))
+    _run(cmd)
+    return out
+
+
 if __name__ == "__main__":
     print(build(verbose=True))

@@ -46,37 +46,105 @@ __device__ __forceinline__ void load8(const float* p, float (&x)[8]) {
     x[6] = __uint_as_float(b.z);
     x[7] = __uint_as_float(b.w);
 }
+// The load rule on the hardware convert: v_cvt_f32_f16 is exact (subnormals included), and a code
+// whose exponent field is 0 -- magnitude below 2^-14 -- reads as a signed zero.
+__device__ __forceinline__ float f16_widen(uint32_t h) {
+    const float x = (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+    return fabsf(x) < 0x1p-14f ? __uint_as_float((h & 0x8000u) << 16) : x;
+}
 __device__ __forceinline__ void load8(const uint16_t* p, float (&x)[8]) {
     const v4u a = ld_stream(p);
     const unsigned w[4] = {a.x, a.y, a.z, a.w};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        x[2 * i] = f16_load(w[i] & 0xffffu);
-        x[2 * i + 1] = f16_load(w[i] >> 16);
+        x[2 * i] = f16_widen(w[i] & 0xffffu);
+        x[2 * i + 1] = f16_widen(w[i] >> 16);
     }
 }
 
-// Which token of the sequence and which lane of that token a thread of a one-dimensional launch
-// is: 32-bit division wherever the launch is small enough for it (a 64-bit one costs some 100
-// instructions, as much as the rest of an append lane's work).
-struct UnitOfToken {
-    int64_t t;
-    int r;
-};
-__device__ __forceinline__ UnitOfToken unit_of_token(int lanes_per_tok) {
-    if ((uint64_t)gridDim.x * kBlock < (1ull << 32)) {
-        const unsigned unit = blockIdx.x * kBlock + threadIdx.x;
-        const unsigned t = unit / (unsigned)lanes_per_tok;
-        return UnitOfToken{(int64_t)t, (int)(unit - t * (unsigned)lanes_per_tok)};
+// For the quantising kernels: the values as the hardware converts them (subnormal codes keep
+// their value), and the load rule's flush as a separate step.  Where a block's amax is above 2^-6
+// the flush changes neither the amax nor a code (|x| < 2^-14 quantises to 0 against a scale above
+// 2^-6 / 127 either way), so those kernels only flush when a block is below that.
+__device__ __forceinline__ void load8_unflushed(const float* p, float (&x)[8]) { load8(p, x); }
+__device__ __forceinline__ void load8_unflushed(const uint16_t* p, float (&x)[8]) {
+    typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+    const h8 h = __builtin_bit_cast(h8, ld_stream(p));
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] = (float)h[i];
+}
+template <typename SrcT>
+__device__ __forceinline__ void flush8(float (&x)[8]) {
+    if (std::is_same<SrcT, uint16_t>::value) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] = fabsf(x[i]) < 0x1p-14f ? __builtin_copysignf(0.0f, x[i]) : x[i];
     }
-    const int64_t unit = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    return UnitOfToken{unit / lanes_per_tok, (int)(unit % lanes_per_tok)};
+}
+
+// Eight consecutive source values as the f16 codes the cache stores for them.
+__device__ __forceinline__ v4u codes8(const float* p) {
+    float x[8];
+    load8(p, x);
+    v4u o;
+    o.x = pack2(x[0], x[1]);
+    o.y = pack2(x[2], x[3]);
+    o.z = pack2(x[4], x[5]);
+    o.w = pack2(x[6], x[7]);
+    return o;
+}
+// A binary16 source goes through the load rule and then the store rule: a code with exponent field
+// 0 becomes a signed zero and a NaN a signed infinity, every other code is stored as it is -- that
+// is, codes with exponent field 0 or 31 lose their mantissa bits.  Two codes a word, no conversion:
+// e + 0x0400 has none of the bits 0x7800 exactly for those two exponent fields.
+// (The packed 16-bit min and multiply are written as instructions: the vector forms crash this
+// compiler's instruction selection.)
+__device__ __forceinline__ uint32_t f16_rule_pair(uint32_t w) {
+    const uint32_t t = ((w & 0x7c007c00u) + 0x04000400u) & 0x78007800u;
+    uint32_t ordinary, keep;  // per half: 1 where the mantissa stays, then its mask
+    asm("v_pk_min_u16 %0, %1, %2" : "=v"(ordinary) : "v"(t), "v"(0x00010001u));
+    asm("v_pk_mul_lo_u16 %0, %1, %2" : "=v"(keep) : "v"(ordinary), "v"(0x03ff03ffu));
+    return w & (0xfc00fc00u | keep);
+}
+__device__ __forceinline__ v4u codes8(const uint16_t* p) {
+    v4u a = ld_stream(p);
+    a.x = f16_rule_pair(a.x);
+    a.y = f16_rule_pair(a.y);
+    a.z = f16_rule_pair(a.z);
+    a.w = f16_rule_pair(a.w);
+    return a;
+}
+
+// Pages hold 16 cells (bkv_pool_create accepts nothing else), so cell -> (page, row in page) is a
+// shift and a mask; the kernels are compiled for head dim 256 and once more for any other, and the
+// usual power-of-two kv head counts divide by a shift: a division by a run-time value is some 25
+// instructions (a 64-bit one 100), as much as the rest of an append lane's work.
+constexpr unsigned kPageShift = 4, kPageMask = 15;
+
+struct RowOfSeq {
+    unsigned t, kvh;  // token within the sequence's rows of this call, kv head
+};
+__device__ __forceinline__ RowOfSeq split_row(uint64_t r, unsigned n_kv, bool fits32) {
+    unsigned t;
+    if ((n_kv & (n_kv - 1u)) == 0u)
+        t = (unsigned)(r >> (31 - __builtin_clz(n_kv)));
+    else
+        t = fits32 ? (unsigned)r / n_kv : (unsigned)(r / n_kv);
+    return RowOfSeq{t, (unsigned)(r - (uint64_t)t * n_kv)};
+}
+// the pool row of (sequence s of the call, token t, kv head)
+__device__ __forceinline__ size_t pool_row_of(const AppendBatch& b, const MoveGeom& g, const int32_t* tables, int s,
+                                              RowOfSeq rs) {
+    // cells are below 2^31 (pos0 and the token count are int32 and their sum is checked on the host)
+    const unsigned cell = (unsigned)b.pos0[s] + rs.t;
+    const int32_t phys = tables[(size_t)b.row[s] * (size_t)g.max_pages_per_seq + (size_t)(cell >> kPageShift)];
+    return (((size_t)phys * g.n_kv + rs.kvh) << kPageShift) + (size_t)(cell & kPageMask);
 }
 
 // ---- append, f16 rows ---------------------------------------------------------
 // One lane converts 8 consecutive elements of one (token, kv head) row of K and of V:
-// two 16-byte loads and one 16-byte store per pool.  grid.y = sequence of the call.
-template <typename SrcT>
+// two 16-byte loads and one 16-byte store per pool.  grid.y = sequence of the call; the rows of a
+// sequence are contiguous in the source, so unit u of a sequence is simply its u-th 8-element group.
+template <typename SrcT, int HD>
 __global__ __launch_bounds__(kBlock) void append_f16_kernel(AppendBatch b, MoveGeom g,
                                                             uint16_t* __restrict__ kpool,
                                                             uint16_t* __restrict__ vpool,
@@ -84,34 +152,18 @@ __global__ __launch_bounds__(kBlock) void append_f16_kernel(AppendBatch b, MoveG
                                                             const SrcT* __restrict__ k,
                                                             const SrcT* __restrict__ v) {
     const int s = blockIdx.y;
-    const int lanes_per_tok = g.n_kv * g.hd / 8;
-    const UnitOfToken u = unit_of_token(lanes_per_tok);
-    const int64_t t = u.t;
-    if (t >= b.n_tok[s]) return;
-    const int r = u.r;  // 8-element group within [n_kv][hd]
-    const int kvh = (r * 8) / g.hd;
-    const int d0 = (r * 8) % g.hd;
-    // cells are below 2^31 (pos0 and the token count are int32 and their sum is checked on the host)
-    const unsigned cell = (unsigned)b.pos0[s] + (unsigned)t;
-    const int32_t phys =
-        tables[(size_t)b.row[s] * (size_t)g.max_pages_per_seq + (size_t)(cell / (unsigned)g.page_cells)];
-    const int in_page = (int)(cell % (unsigned)g.page_cells);
-    const size_t row = ((size_t)phys * g.n_kv + kvh) * g.page_cells + in_page;
-    const size_t dst = row * (size_t)g.hd + d0;
-    const size_t src = ((size_t)b.src0[s] + (size_t)t) * (size_t)(g.n_kv * g.hd) + (size_t)r * 8;
-
-    float kx[8], vx[8];
-    load8(k + src, kx);
-    load8(v + src, vx);
-    v4u ko, vo;
-    ko.x = pack2(kx[0], kx[1]);
-    ko.y = pack2(kx[2], kx[3]);
-    ko.z = pack2(kx[4], kx[5]);
-    ko.w = pack2(kx[6], kx[7]);
-    vo.x = pack2(vx[0], vx[1]);
-    vo.y = pack2(vx[2], vx[3]);
-    vo.z = pack2(vx[4], vx[5]);
-    vo.w = pack2(vx[6], vx[7]);
+    const unsigned hd = HD ? HD : g.hd;
+    const unsigned lpr = hd / 8;  // lanes of a row
+    const int64_t rows_total = (int64_t)b.n_tok[s] * g.n_kv;
+    const bool fits32 = rows_total * lpr < (1ll << 32);
+    const uint64_t unit = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    const uint64_t r = HD ? unit / lpr : (fits32 ? (uint64_t)((unsigned)unit / lpr) : unit / lpr);
+    if ((int64_t)r >= rows_total) return;
+    const unsigned li = (unsigned)(unit - r * lpr);
+    const size_t row = pool_row_of(b, g, tables, s, split_row(r, (unsigned)g.n_kv, fits32));
+    const size_t dst = row * (size_t)hd + (size_t)li * 8;
+    const size_t src = (size_t)b.src0[s] * (size_t)(g.n_kv * hd) + (size_t)unit * 8;
+    const v4u ko = codes8(k + src), vo = codes8(v + src);
     st_stream(kpool + dst, ko);
     st_stream(vpool + dst, vo);
 }
@@ -135,47 +187,6 @@ __device__ __forceinline__ void q8v_encode(const float (&x)[32], uint32_t* vd) {
     for (int j = 0; j < 9; ++j) vd[j] = w[j];
 }
 
-// ---- append, reference q8_0-V rows: K f16, V [f32 scale][32 x i8] per 32 values ---
-// One lane per (token, kv head, 32-element block), as the reference shader does.
-template <typename SrcT>
-__global__ __launch_bounds__(kBlock) void append_q8v_kernel(AppendBatch b, MoveGeom g,
-                                                            uint16_t* __restrict__ kpool,
-                                                            uint32_t* __restrict__ vpool,
-                                                            const int32_t* __restrict__ tables,
-                                                            const SrcT* __restrict__ k,
-                                                            const SrcT* __restrict__ v) {
-    const int s = blockIdx.y;
-    const int blocks = g.hd / 32;
-    const int lanes_per_tok = g.n_kv * blocks;
-    const UnitOfToken u = unit_of_token(lanes_per_tok);
-    const int64_t t = u.t;
-    if (t >= b.n_tok[s]) return;
-    const int r = u.r;
-    const int kvh = r / blocks;
-    const int blk = r % blocks;
-    const unsigned cell = (unsigned)b.pos0[s] + (unsigned)t;
-    const int32_t phys =
-        tables[(size_t)b.row[s] * (size_t)g.max_pages_per_seq + (size_t)(cell / (unsigned)g.page_cells)];
-    const int in_page = (int)(cell % (unsigned)g.page_cells);
-    const size_t row = ((size_t)phys * g.n_kv + kvh) * g.page_cells + in_page;
-    const size_t src = ((size_t)b.src0[s] + (size_t)t) * (size_t)(g.n_kv * g.hd) +
-                       (size_t)kvh * g.hd + (size_t)blk * 32;
-    float x[32];
-    load32(k + src, x);
-    uint4* kd = reinterpret_cast<uint4*>(kpool + row * (size_t)g.hd + (size_t)blk * 32);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        uint4 o;
-        o.x = pack2(x[i * 8 + 0], x[i * 8 + 1]);
-        o.y = pack2(x[i * 8 + 2], x[i * 8 + 3]);
-        o.z = pack2(x[i * 8 + 4], x[i * 8 + 5]);
-        o.w = pack2(x[i * 8 + 6], x[i * 8 + 7]);
-        kd[i] = o;
-    }
-    load32(v + src, x);
-    q8v_encode(x, vpool + (row * (size_t)blocks + (size_t)blk) * 9u);
-}
-
 // ---- append, int8 K and V with f16 scales: row = [hd x i8][hd/32 x f16] -----------
 // The q8_0 rule with the scale stored through the cache's f16 encoding; a scale the
 // f16 rule would flush is raised to 2^-14.  (No reference counterpart.)
@@ -188,40 +199,133 @@ __device__ __forceinline__ void i8h_encode(const float (&x)[32], uint8_t* row_ba
     *reinterpret_cast<uint16_t*>(row_base + hd + blk * 2) = (uint16_t)hb;
 }
 
-template <typename SrcT>
-__device__ __forceinline__ void i8h_block(const SrcT* src, uint8_t* row_base, int hd, int blk) {
-    float x[32];
-    load32(src, x);
-    i8h_encode(x, row_base, hd, blk);
-}
-
-template <typename SrcT>
-__global__ __launch_bounds__(kBlock) void append_i8h_kernel(AppendBatch b, MoveGeom g,
-                                                            uint8_t* __restrict__ kpool,
-                                                            uint8_t* __restrict__ vpool,
-                                                            const int32_t* __restrict__ tables,
-                                                            const SrcT* __restrict__ k,
-                                                            const SrcT* __restrict__ v) {
+// ---- append, quantised rows -----------------------------------------------------------
+// Q8V (the reference's BRECCIA_KV_Q8V, shaders/qsa_kv_append.comp:87-133): K f16, V
+// [f32 scale][32 x i8] per 32 values.  I8H: K and V rows of [hd x i8][hd/32 x f16 scale].
+// A lane takes 8 consecutive elements of one (token, kv head) row of K and of V, like the f16
+// kernel (a wave's loads are contiguous 16-byte pieces); the four lanes of a quad share a
+// 32-value block and agree its amax by DPP.  The encoded rows are put together in LDS and
+// leave as whole contiguous rows, one 16-byte piece a lane (4-byte pieces when the head dim
+// makes rows that are not 16-byte multiples).  A work-group owns 256 / (hd / 8) consecutive
+// rows of one sequence of the call (grid.y).
+template <int LAYOUT, typename SrcT, int HD>
+__global__ __launch_bounds__(kBlock) void append_quant_kernel(AppendBatch b, MoveGeom g,
+                                                              uint8_t* __restrict__ kpool,
+                                                              uint8_t* __restrict__ vpool,
+                                                              const int32_t* __restrict__ tables,
+                                                              const SrcT* __restrict__ k,
+                                                              const SrcT* __restrict__ v) {
+    // at most 64 rows (hd 32) of at most 288 bytes (hd 256): rows x row bytes <= 2304 per image
+    __shared__ __attribute__((aligned(16))) uint8_t image[2 * 2304];
+    __shared__ uint64_t row_s[64];
     const int s = blockIdx.y;
-    const int blocks = g.hd / 32;
-    const int lanes_per_tok = g.n_kv * blocks * 2;  // K and V blocks
-    const UnitOfToken u = unit_of_token(lanes_per_tok);
-    const int64_t t = u.t;
-    if (t >= b.n_tok[s]) return;
-    int r = u.r;
-    const int which = r / (g.n_kv * blocks);
-    r %= g.n_kv * blocks;
-    const int kvh = r / blocks;
-    const int blk = r % blocks;
-    const unsigned cell = (unsigned)b.pos0[s] + (unsigned)t;
-    const int32_t phys =
-        tables[(size_t)b.row[s] * (size_t)g.max_pages_per_seq + (size_t)(cell / (unsigned)g.page_cells)];
-    const int in_page = (int)(cell % (unsigned)g.page_cells);
-    const size_t row = ((size_t)phys * g.n_kv + kvh) * g.page_cells + in_page;
-    const size_t src = ((size_t)b.src0[s] + (size_t)t) * (size_t)(g.n_kv * g.hd) +
-                       (size_t)kvh * g.hd + (size_t)blk * 32;
-    const size_t row_bytes = (size_t)g.hd + (size_t)blocks * 2;
-    i8h_block((which ? v : k) + src, (which ? vpool : kpool) + row * row_bytes, g.hd, blk);
+    const int hd = HD ? HD : g.hd;
+    const int lpr = hd / 8;           // lanes of a row
+    const int rows_wg = kBlock / lpr;
+    const int blocks = hd / 32;
+    const int64_t rows_total = (int64_t)b.n_tok[s] * g.n_kv;
+    const int64_t r0 = (int64_t)blockIdx.x * rows_wg;
+    if (r0 >= rows_total) return;
+    const int nrows = (int)(rows_total - r0 < rows_wg ? rows_total - r0 : rows_wg);
+    const int tid = threadIdx.x;
+    const int rl = tid / lpr, li = tid - rl * lpr;
+    const bool active = rl < nrows;
+    const uint32_t row_bytes = LAYOUT == BKV_LAYOUT_Q8V ? (uint32_t)blocks * 36u : (uint32_t)hd + (uint32_t)blocks * 2u;
+    uint8_t* const v_image = image + (LAYOUT == BKV_LAYOUT_I8H ? rows_wg * row_bytes : 0u);
+
+    float kx[8], vx[8];
+    v4u ko = v4u{0u, 0u, 0u, 0u};
+    size_t row = 0;
+    if (active) {
+        const uint64_t r = (uint64_t)(r0 + rl);
+        row = pool_row_of(b, g, tables, s, split_row(r, (unsigned)g.n_kv, rows_total < (1ll << 32)));
+        // the rows of a sequence are contiguous in the source
+        const size_t src = ((size_t)b.src0[s] * g.n_kv + (size_t)r) * (size_t)hd + (size_t)li * 8;
+        if (LAYOUT == BKV_LAYOUT_Q8V)
+            ko = codes8(k + src);
+        else
+            load8_unflushed(k + src, kx);
+        load8_unflushed(v + src, vx);
+        if (li == 0) row_s[rl] = (uint64_t)row;
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) kx[i] = vx[i] = 0.0f;
+    }
+    // quads never straddle rows (lanes of a row are a multiple of four), so a quad is active as a whole
+    const int blk = li >> 2, quarter = li & 3;
+    constexpr bool kSrcF16 = std::is_same<SrcT, uint16_t>::value;
+    if (LAYOUT == BKV_LAYOUT_Q8V) {
+        if (active) st_stream(reinterpret_cast<uint16_t*>(kpool) + row * (size_t)hd + (size_t)li * 8, ko);
+        float amax = quad_max(amax8(vx));
+        float scale = q8v_scale(amax);
+        uint32_t w0, w1, doubt = (kSrcF16 && !(amax > 0x1p-6f)) ? 0x7fc00000u : 0u;
+        codes8_on_reciprocal(vx, scale, w0, w1, doubt);
+        if (__any(codes_in_doubt(doubt))) {  // the rule as written, for the whole wave
+            flush8<SrcT>(vx);
+            scale = q8v_scale(quad_max(amax8(vx)));
+            q8_codes8(vx, scale, w0, w1);
+        }
+        if (active) {
+            uint32_t* blk_words = reinterpret_cast<uint32_t*>(v_image + rl * row_bytes + blk * 36);
+            if (quarter == 0) blk_words[0] = __float_as_uint(scale);
+            blk_words[1 + 2 * quarter] = w0;
+            blk_words[2 + 2 * quarter] = w1;
+        }
+    } else {
+        const float ka = quad_max(amax8(kx)), va = quad_max(amax8(vx));
+        uint32_t kb = i8h_scale_bits(ka), vb = i8h_scale_bits(va);
+        uint32_t k0, k1, v0, v1;
+        bool redo;
+        if (kSrcF16) {
+            // a NaN survives any sum; an infinity shows in the amax
+            const float sum = ((kx[0] + kx[1]) + (kx[2] + kx[3])) + ((kx[4] + kx[5]) + (kx[6] + kx[7])) +
+                              ((vx[0] + vx[1]) + (vx[2] + vx[3])) + ((vx[4] + vx[5]) + (vx[6] + vx[7]));
+            redo = !(ka > 0x1p-6f && va > 0x1p-6f && ka <= 65504.0f && va <= 65504.0f) || sum != sum;
+            codes8_f16_on_biased_reciprocal(kx, __builtin_amdgcn_rcpf(f16_normal_value(kb)) * kTieBias, k0, k1);
+            codes8_f16_on_biased_reciprocal(vx, __builtin_amdgcn_rcpf(f16_normal_value(vb)) * kTieBias, v0, v1);
+        } else {
+            uint32_t doubt = 0u;
+            codes8_on_reciprocal(kx, f16_normal_value(kb), k0, k1, doubt);
+            codes8_on_reciprocal(vx, f16_normal_value(vb), v0, v1, doubt);
+            redo = codes_in_doubt(doubt);
+        }
+        if (__any(redo)) {  // the rule as written, for the whole wave
+            flush8<SrcT>(kx);
+            flush8<SrcT>(vx);
+            kb = i8h_scale_bits(quad_max(amax8(kx)));
+            vb = i8h_scale_bits(quad_max(amax8(vx)));
+            i8h_codes8(kx, f16_load(kb), k0, k1);
+            i8h_codes8(vx, f16_load(vb), v0, v1);
+        }
+        if (active) {
+            uint8_t* kr = image + rl * row_bytes;
+            uint8_t* vr = v_image + rl * row_bytes;
+            *reinterpret_cast<uint2*>(kr + li * 8) = make_uint2(k0, k1);
+            *reinterpret_cast<uint2*>(vr + li * 8) = make_uint2(v0, v1);
+            if (quarter == 0) {
+                *reinterpret_cast<uint16_t*>(kr + hd + blk * 2) = (uint16_t)kb;
+                *reinterpret_cast<uint16_t*>(vr + hd + blk * 2) = (uint16_t)vb;
+            }
+        }
+    }
+    __syncthreads();
+    // whole rows out: piece p of the work-group's image goes to the same offset of its pool row
+    constexpr uint32_t kPiece = HD == 256 ? 16u : 4u;
+    const uint32_t ppr = row_bytes / kPiece;  // pieces of a row
+    const uint32_t n_pieces = (uint32_t)nrows * ppr;
+    const int n_images = LAYOUT == BKV_LAYOUT_I8H ? 2 : 1;
+    for (int im = 0; im < n_images; ++im) {
+        const uint8_t* src_image = im ? v_image : image;
+        uint8_t* pool = (LAYOUT == BKV_LAYOUT_I8H && im == 0) ? kpool : vpool;
+        for (uint32_t p = (uint32_t)tid; p < n_pieces; p += kBlock) {
+            const uint32_t pr = p / ppr, off = (p - pr * ppr) * kPiece;
+            uint8_t* dst = pool + (size_t)row_s[pr] * row_bytes + off;
+            if (kPiece == 16)
+                st_stream(dst, *reinterpret_cast<const v4u*>(src_image + pr * row_bytes + off));
+            else
+                *reinterpret_cast<uint32_t*>(dst) = *reinterpret_cast<const uint32_t*>(src_image + pr * row_bytes + off);
+        }
+    }
 }
 
 // ---- K preparation fused into the append ------------------------------------------
@@ -312,9 +416,8 @@ __global__ __launch_bounds__(kBlock) void append_kprep_kernel(AppendBatch b, Mov
         const unsigned r = (unsigned)(r0 + tid - 64);
         const unsigned cell = (unsigned)b.pos0[s] + r / (unsigned)g.n_kv;
         const unsigned kvh = r % (unsigned)g.n_kv;
-        const int32_t phys = tables[(size_t)b.row[s] * (size_t)g.max_pages_per_seq +
-                                    (size_t)(cell / (unsigned)g.page_cells)];
-        row_s[tid - 64] = ((uint64_t)phys * g.n_kv + kvh) * g.page_cells + (uint64_t)(cell % (unsigned)g.page_cells);
+        const int32_t phys = tables[(size_t)b.row[s] * (size_t)g.max_pages_per_seq + (size_t)(cell >> kPageShift)];
+        row_s[tid - 64] = (((uint64_t)phys * g.n_kv + kvh) << kPageShift) + (uint64_t)(cell & kPageMask);
         int64_t pos = kp.positions ? (int64_t)kp.positions[cell] : (int64_t)cell;
         pos = pos < 0 ? 0 : (pos > kp.max_pos - 1 ? kp.max_pos - 1 : pos);
         pos_s[tid - 64] = (int32_t)pos;
@@ -664,30 +767,32 @@ static hipError_t launch_append_from(bkv_pool* p, int32_t layer, const AppendBat
                                      int32_t max_tok, const SrcT* k, const SrcT* v,
                                      hipStream_t stream) {
     const MoveGeom g = move_geom(p);
-    int lanes_per_tok;
-    switch (p->g.layout) {
-        case BKV_LAYOUT_F16: lanes_per_tok = g.n_kv * g.hd / 8; break;
-        case BKV_LAYOUT_Q8V: lanes_per_tok = g.n_kv * g.hd / 32; break;
-        default: lanes_per_tok = g.n_kv * g.hd / 32 * 2; break;
-    }
-    const int64_t lanes = (int64_t)max_tok * lanes_per_tok;
-    dim3 grid((unsigned)((lanes + kBlock - 1) / kBlock), (unsigned)b.n);
     uint8_t* kp = p->k_layer[(size_t)layer];
     uint8_t* vp = p->v_layer[(size_t)layer];
-    switch (p->g.layout) {
-        case BKV_LAYOUT_F16:
-            launch_staged(p, BKV_STAGE_APPEND, append_f16_kernel<SrcT>, grid, dim3(kBlock), 0, stream, b, g,
-                          (uint16_t*)kp, (uint16_t*)vp, (const int32_t*)p->table_dev, k, v);
-            break;
-        case BKV_LAYOUT_Q8V:
-            launch_staged(p, BKV_STAGE_APPEND, append_q8v_kernel<SrcT>, grid, dim3(kBlock), 0, stream, b, g,
-                          (uint16_t*)kp, (uint32_t*)vp, (const int32_t*)p->table_dev, k, v);
-            break;
-        default:
-            launch_staged(p, BKV_STAGE_APPEND, append_i8h_kernel<SrcT>, grid, dim3(kBlock), 0, stream, b, g, kp, vp,
-                          (const int32_t*)p->table_dev, k, v);
-            break;
+    const int32_t* tables = p->table_dev;
+    if (p->g.layout == BKV_LAYOUT_F16) {
+        const int64_t lanes = (int64_t)max_tok * (g.n_kv * g.hd / 8);
+        dim3 grid((unsigned)((lanes + kBlock - 1) / kBlock), (unsigned)b.n);
+        if (g.hd == 256)
+            launch_staged(p, BKV_STAGE_APPEND, append_f16_kernel<SrcT, 256>, grid, dim3(kBlock), 0, stream, b, g,
+                          (uint16_t*)kp, (uint16_t*)vp, tables, k, v);
+        else
+            launch_staged(p, BKV_STAGE_APPEND, append_f16_kernel<SrcT, 0>, grid, dim3(kBlock), 0, stream, b, g,
+                          (uint16_t*)kp, (uint16_t*)vp, tables, k, v);
+        return hipGetLastError();
     }
+    const int rows_wg = kBlock / (g.hd / 8);
+    const int64_t rows = (int64_t)max_tok * g.n_kv;
+    dim3 grid((unsigned)((rows + rows_wg - 1) / rows_wg), (unsigned)b.n);
+    if (p->g.layout == BKV_LAYOUT_I8H)  // pools of this layout have head dim 256
+        launch_staged(p, BKV_STAGE_APPEND, append_quant_kernel<BKV_LAYOUT_I8H, SrcT, 256>, grid, dim3(kBlock), 0,
+                      stream, b, g, kp, vp, tables, k, v);
+    else if (g.hd == 256)
+        launch_staged(p, BKV_STAGE_APPEND, append_quant_kernel<BKV_LAYOUT_Q8V, SrcT, 256>, grid, dim3(kBlock), 0,
+                      stream, b, g, kp, vp, tables, k, v);
+    else
+        launch_staged(p, BKV_STAGE_APPEND, append_quant_kernel<BKV_LAYOUT_Q8V, SrcT, 0>, grid, dim3(kBlock), 0,
+                      stream, b, g, kp, vp, tables, k, v);
     return hipGetLastError();
 }
 

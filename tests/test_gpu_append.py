@@ -149,6 +149,44 @@ def test_quantised_append_is_bit_exact(layout):
         assert np.array_equal(gk, ok) and np.array_equal(gv, ov)
 
 
+@pytest.mark.parametrize("f16_rows", [False, True])
+@pytest.mark.parametrize("layout", [L.LAYOUT_Q8V, L.LAYOUT_I8H])
+def test_quantised_bulk_append_with_ties_is_bit_exact(layout, f16_rows):
+    # The bulk kernels take the codes from a reciprocal of the scale where that provably gives the
+    # rule's round-half-away(clamp(x / scale)) (qsa/cpu.rs:65-82) and from the division itself
+    # elsewhere: 3000 tokens (most waves on the short cut, some not), blocks of exact ties
+    # (scale 1 and 1/4: values k + 1/2 and (k + 1/2) / 4, both signs), values one ulp either side
+    # of a tie, blocks below 2^-6 (f16 rows are flushed there), an all-zero block, a lone large value.
+    rng = np.random.Generator(np.random.PCG64(300 + 2 * layout + int(f16_rows)))
+    T = 3000
+    k = (rng.standard_normal((T, 2, 256)) * rng.uniform(0.05, 30, size=(T, 2, 1))).astype(np.float32)
+    v = (rng.standard_normal((T, 2, 256)) * rng.uniform(0.05, 30, size=(T, 2, 1))).astype(np.float32)
+    halves = (np.arange(32, dtype=np.float32) * 7.0) % 126.0 + 0.5
+    halves[::2] *= -1.0
+    for x in (k, v):
+        x[10, 0, 0:32] = halves
+        x[10, 0, 0] = 127.0                         # amax 127: scale exactly 1
+        x[11, 1, 64:96] = halves / 4.0
+        x[11, 1, 64] = -127.0 / 4.0                 # scale exactly 1/4
+        x[12, 0, 32:64] = np.nextafter(halves, np.float32(1000.0))
+        x[12, 0, 32] = 127.0
+        x[13, 1, 32:64] = np.nextafter(halves, np.float32(-1000.0))
+        x[13, 1, 32] = 127.0
+        x[14, 0, 96:128] = rng.standard_normal(32).astype(np.float32) * 1e-3     # amax below 2^-6
+        x[15, 1, 0:32] = rng.standard_normal(32).astype(np.float32) * 3e-5       # around 2^-14 and below
+        x[16, 0, 128:160] = 0.0
+        x[17, 1, 160:192] = 1e-4
+        x[17, 1, 161] = 5e4
+    if f16_rows:
+        with np.errstate(over="ignore"):
+            k, v = k.astype(np.float16).view(np.uint16), v.astype(np.float16).view(np.uint16)
+    with Twin(n_pages=T // 16 + 8, layout=layout, max_seqs=4) as tw:
+        s = tw.pool.seq_create()
+        tw.pool.seq_reserve(s, T + 5)
+        tw.append(0, [s], [5], [k], [v], f16_rows=f16_rows)
+        tw.assert_pools_equal()
+
+
 @pytest.mark.parametrize("layout", [L.LAYOUT_F16, L.LAYOUT_Q8V, L.LAYOUT_I8H])
 def test_f16_rows_append_like_their_widened_f32_rows(layout):
     # bkv_append_f16: raw binary16 rows, read under the cache's load rule
