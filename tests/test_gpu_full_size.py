@@ -8,6 +8,15 @@ size-independent properties on all of them: the batched call equals the per-sequ
 1e-6, and every output is a convex combination of V rows (bounded by the largest |v|).
 configs[3] shape (4 sequences, 2048-token prefix + 1024-token chunk) through the chunk kernel on
 all three layouts: sampled tokens against the oracle, the chunk's tail against the decode kernel.
+The fused step (bkv_decode_step) on configs[2] (f16 and f16 K + q8_0 V) and on configs[4] at the same
+sizes: outputs bit-identical to bkv_append + bkv_decode_attn, the new rows' pool bytes against the
+oracle's encoders.  configs[3] end to end on one pool: shared 2040-token prefix, binary16 chunks
+through bkv_append_f16, the copy-on-write copies, a seeded quarter of the pages out to pinned host
+memory, poisoned, back, every pool byte against the oracle's image.
+In the attention checks of this file the oracle attends over the rows read back through bkv_gather
+(its own kernel and address arithmetic) unless a test says it keeps an oracle image: the appends
+that stored those rows are compared byte for byte with the oracle's image elsewhere
+(tests/test_gpu_append.py, the configs[1] and configs[3] tests below).
 A 300k-page pool with a sequence on the highest page ids (byte offsets past 2^32): every kernel of the
 path there against a twin on the lowest pages and the oracle."""
 import numpy as np
@@ -102,6 +111,169 @@ def test_config3_batch8_mixed_1k_32k_all_heads():
         nd.free()
     finally:
         pool.destroy()
+
+
+def read_page(pool, which, page):
+    """Raw bytes of one page of layer 0's K (0) or V (1) pool."""
+    import ctypes as C
+
+    from breccia_amd.kv import check, lib
+
+    base, _ = pool.layer_ptr(0, which)
+    n = pool.page_bytes(which)
+    out = np.empty(n, dtype=np.uint8)
+    check(lib.bkv_memcpy_d2h(out.ctypes.data, C.c_void_p(base.value + page * n), n, None))
+    check(lib.bkv_stream_sync(None))
+    return out
+
+
+def step_both_ways(pool, layout, seqs, ctx, rng):
+    """One decode step at positions ctx, as bkv_append + bkv_decode_attn and then -- after the new
+    cells have been overwritten with other rows -- as one bkv_decode_step.  Checks that the two forms
+    return the same bits and leave the same pool bytes in the pages they wrote, and that the new
+    rows' bytes are the oracle encoders'.  Returns (q, outputs)."""
+    n = len(seqs)
+    for s, c in zip(seqs, ctx):
+        pool.seq_reserve(s, c + 1)
+    new_k = rng.standard_normal((n, N_KV, HD), dtype=np.float32)
+    new_v = rng.standard_normal((n, N_KV, HD), dtype=np.float32)
+    junk = rng.standard_normal((n, N_KV, HD), dtype=np.float32)
+    q = rng.standard_normal((n, N_Q, HD), dtype=np.float32)
+    kd, vd, jd = DeviceBuffer.from_numpy(new_k), DeviceBuffer.from_numpy(new_v), DeviceBuffer.from_numpy(junk)
+    qd, od = DeviceBuffer.from_numpy(q), DeviceBuffer(q.nbytes)
+    try:
+        pool.append(0, seqs, ctx, [1] * n, kd, vd)
+        two = run_attn(pool, seqs, ctx, q)
+        last_pages = [int(pool.block_table(s)[c // 16]) for s, c in zip(seqs, ctx)]
+        pages_two = [(read_page(pool, 0, p), read_page(pool, 1, p)) for p in last_pages]
+        pool.append(0, seqs, ctx, [1] * n, jd, jd)          # other rows in the new cells
+        assert not np.array_equal(read_page(pool, 0, last_pages[0]), pages_two[0][0])
+        pool.decode_step(0, seqs, ctx, kd, vd, N_Q, qd, od, 1.0 / 16.0)
+        device_sync()
+        fused = od.download(np.float32).reshape(n, N_Q, HD)
+        assert np.array_equal(fused.view(np.uint32), two.view(np.uint32))
+        g = oracle.Geom(N_KV, HD, 16)
+        from gpu_common import ORACLE_LAYOUT
+        for i, (p, c) in enumerate(zip(last_pages, ctx)):
+            pk, pv = read_page(pool, 0, p), read_page(pool, 1, p)
+            assert np.array_equal(pk, pages_two[i][0]) and np.array_equal(pv, pages_two[i][1]), i
+            img = oracle.PoolImage(g, 1, ORACLE_LAYOUT[layout])
+            assert img.append(np.zeros(1, dtype=np.int32), c % 16, new_k[i], new_v[i]) == 0
+            for which, page, image in ((0, pk, img.k), (1, pv, img.v)):
+                rb = image.size // (N_KV * 16)
+                for kvh in range(N_KV):
+                    at = (kvh * 16 + c % 16) * rb
+                    assert np.array_equal(page[at:at + rb], image[at:at + rb]), (i, which, kvh)
+    finally:
+        for b in (kd, vd, jd, qd, od):
+            b.free()
+    return q, fused
+
+
+@pytest.mark.parametrize("layout", [L.LAYOUT_F16, L.LAYOUT_Q8V])
+def test_config3_batch8_fused_step_all_heads(layout):
+    # the benchmark's headline call at the benchmark's size (and its q8_0-V variant): every (sequence,
+    # head) pair of the fused step against the oracle at the reference's bar
+    rng = np.random.Generator(np.random.PCG64(20250003))
+    pool, seqs, ctx = build(rng, 8, 1024, 32768, layout)
+    try:
+        fill_tiled(pool, seqs, ctx, rng)
+        q, out = step_both_ways(pool, layout, seqs, ctx, rng)
+        worst = 0.0
+        for i, s in enumerate(seqs):
+            want, _ = oracle_for(pool, s, ctx[i], q[i])
+            _, rel = check_attn(out[i], want, "config3 fused step, layout %d, seq %d (ctx %d)" % (layout, i, ctx[i]))
+            worst = max(worst, rel)
+        assert worst <= REF_BAR_MAX_REL, worst
+    finally:
+        pool.destroy()
+
+
+def test_config5_batch16_int8_fused_step():
+    # configs[4] through bkv_decode_step, the call the benchmark times on this layout: bit-identical to
+    # append + attend on all 16 sequences, the oracle on the shortest, the median and the longest
+    rng = np.random.Generator(np.random.PCG64(20250005))
+    pool, seqs, ctx = build(rng, 16, 8192, 131072, L.LAYOUT_I8H)
+    try:
+        fill_tiled(pool, seqs, ctx, rng)
+        q, out = step_both_ways(pool, L.LAYOUT_I8H, seqs, ctx, rng)
+        order = np.argsort(ctx)
+        for i in (int(order[0]), int(order[8]), int(order[-1])):
+            want, v = oracle_for(pool, seqs[i], ctx[i], q[i])
+            _, rel = check_attn(out[i], want, "config5 fused step seq %d (ctx %d)" % (i, ctx[i]))
+            assert rel <= REF_BAR_MAX_REL, rel
+            assert np.abs(out[i]).max() <= np.abs(v).max()
+    finally:
+        pool.destroy()
+
+
+def test_config4_end_to_end_shared_prefix_f16_chunks_cow_and_swap():
+    """BASELINE configs[3] as worded, on one pool: four sequences share a prefix through shared page ids
+    with refcounts (2040 tokens: 127 full pages and a partial one); each appends a distinct 1024-token
+    chunk of binary16 K/V (bkv_append_f16), which makes all writers but the last copy the shared
+    partial page first; then a seeded 25 % of the pages in use go to pinned host memory, are
+    overwritten in VRAM, and come back.  The oracle keeps its own image of the pool throughout
+    (append of the widened rows, page copies): every pool byte is compared after the appends and after
+    the swap, and decode attention runs against the oracle over its own image."""
+    from breccia_amd.kv import Stream
+    from gpu_common import Twin
+
+    rng = np.random.Generator(np.random.PCG64(20250004))
+    prefix, chunk = 2040, 1024
+    with Twin(n_pages=640, max_seqs=8) as tw:
+        tw.pool.set_free_order(rng.permutation(640).astype(np.int32))
+        root = tw.pool.seq_create()
+        tw.pool.seq_reserve(root, prefix)
+        pk = rng.standard_normal((prefix, N_KV, HD)).astype(np.float16).view(np.uint16)
+        pv = rng.standard_normal((prefix, N_KV, HD)).astype(np.float16).view(np.uint16)
+        tw.append(0, [root], [0], [pk], [pv], f16_rows=True)
+        kids = [tw.pool.seq_fork(root, prefix) for _ in range(3)]
+        seqs = [root] + kids
+        shared = tw.pool.block_table(root).copy()
+        assert shared.size == 128 and all(tw.pool.page_refcount(int(p)) == 4 for p in shared)
+        n_copies = 0
+        for s in seqs:
+            pairs = tw.pool.seq_reserve(s, prefix + chunk)
+            n_copies += len(pairs)
+            tw.pool.page_copy(pairs)
+            tw.images[0].page_copy(pairs)
+            ck = rng.standard_normal((chunk, N_KV, HD)).astype(np.float16).view(np.uint16)
+            cv = rng.standard_normal((chunk, N_KV, HD)).astype(np.float16).view(np.uint16)
+            tw.append(0, [s], [prefix], [ck], [cv], f16_rows=True)
+        assert n_copies == 3
+        tw.assert_pools_equal()
+        tw.pool.check()
+        assert all(np.array_equal(tw.pool.block_table(s)[:127], shared[:127]) for s in seqs)
+        assert len({int(tw.pool.block_table(s)[127]) for s in seqs}) == 4
+        # a seeded quarter of the pages in use: out, poisoned, back
+        used = np.unique(np.concatenate([tw.pool.block_table(s) for s in seqs]))
+        cold = rng.choice(used, size=used.size // 4, replace=False).astype(np.int32)
+        slab = tw.pool.swap_page_bytes()
+        host = tw.pool.host_alloc(cold.size * slab)
+        st = Stream()
+        tw.pool.swap_out(cold, host, st)
+        tw.pool.swap_wait()
+        hv = host.view().reshape(cold.size, 2, 16384)
+        for i, p in enumerate(cold):
+            assert np.array_equal(hv[i, 0], tw.images[0].k.reshape(-1, 16384)[p])
+            assert np.array_equal(hv[i, 1], tw.images[0].v.reshape(-1, 16384)[p])
+        junk = int(np.setdiff1d(np.arange(640, dtype=np.int32), used)[0])
+        tw.pool.page_copy([(junk, int(p)) for p in cold], st)
+        st.sync()
+        assert not np.array_equal(tw.pool.read_layer(0, 0), tw.images[0].k)
+        tw.pool.swap_in(cold, host, st)
+        tw.pool.swap_fence(st)
+        st.sync()
+        tw.assert_pools_equal()
+        host.free()
+        q = rng.standard_normal((4, N_Q, HD)).astype(np.float32)
+        pos = [prefix + chunk - 1] * 4
+        out = tw.decode_attn(0, seqs, pos, q, N_Q)
+        worst = 0.0
+        for i, s in enumerate(seqs):
+            _, rel = check_attn(out[i], tw.oracle_attend(0, s, pos[i], q[i], N_Q, threads=8), "configs[3] seq %d" % i)
+            worst = max(worst, rel)
+        assert worst <= REF_BAR_MAX_REL, worst
 
 
 def test_config5_batch16_int8_8k_128k():
