@@ -213,6 +213,7 @@ def time_replay(pool, seqs, n_layers, tokens, bufs, stream):
 
 
 PREHEAT_MS = 40.0
+REGIONS = 5           # timed regions of --steps steps; the median is reported
 CPU_SAMPLE_S = 10.0   # CPU time spent on the one-thread baseline
 
 
@@ -269,10 +270,16 @@ def main() -> int:
     pre_steps, pre_ms = preheat(pool, seqs, ctx, n_layers, bufs, stream, PREHEAT_MS)
 
     # ---- headline: K steps, whole path ------------------------------------------------
-    wall_ms, _ = time_steps(pool, seqs, ctx, n_layers, args.steps, args.warmup, bufs, stream,
-                            first_step=pre_steps)
-    ms_per_step = wall_ms / args.steps
-    ctx_mid = [c + 1 + (pre_steps + args.warmup + args.steps // 2) // n_layers for c in ctx]
+    # REGIONS consecutive timed regions of --steps steps each (every one bracketed by host
+    # synchronisations); ms_per_step is the median region's, the spread goes into `extra`
+    region_ms = []
+    for r in range(REGIONS):
+        wall_ms, _ = time_steps(pool, seqs, ctx, n_layers, args.steps, args.warmup if r == 0 else 0, bufs, stream,
+                                first_step=pre_steps + (args.warmup + r * args.steps if r else 0))
+        region_ms.append(wall_ms / args.steps)
+    ms_per_step = float(np.median(region_ms))
+    ctx_mid = [c + 1 + (pre_steps + args.warmup + REGIONS * args.steps // 2) // n_layers for c in ctx]
+    pre_steps += (REGIONS - 1) * args.steps          # steps taken so far = pre_steps + warmup + steps, as below
     attn_bytes = attn_algorithmic_bytes(ctx_mid)
     step_bytes = attn_bytes + len(seqs) * APPEND_BYTES_PER_TOKEN
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
@@ -362,6 +369,11 @@ def main() -> int:
              "two_call_us_per_layer": round(two_call_us, 2),
              "graph_replay_us_per_layer": round(replay_us, 2),
              "step_event_ms": round(ev_ms / args.steps, 4),
+             "timed_regions": {"count": REGIONS, "steps_each": args.steps, "reported": "median",
+                               "ms_per_step": [round(x, 5) for x in region_ms],
+                               "min_ms_per_step": round(min(region_ms), 5), "max_ms_per_step": round(max(region_ms), 5),
+                               "frac_of_hbm_peak_min_max": [round(step_bytes / (max(region_ms) * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                                                            round(step_bytes / (min(region_ms) * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)]},
              "preheat_ms": round(pre_ms, 1), "preheat_steps": pre_steps,
              "contexts": ctx, "pool_pages": pool.desc.n_pages, "device": dev_name, "cus": n_cu,
              "oracle_check_max_abs": checked}
@@ -377,6 +389,8 @@ def main() -> int:
         extra.update(bench_prefill(stream))
         extra.update(bench_moves(stream))
         extra.update(bench_prefix_tiers(stream))
+        extra.update(bench_reference_cell(stream))
+        extra.update(bench_config3_scenario(stream))
 
     line = {"metric": "paged decode-attn step throughput, batch 8 mixed 1k-32k (append + attention, "
                       "algorithmic bytes / time)",
@@ -712,6 +726,169 @@ def bench_prefill(stream) -> dict:
     for b in (kd, vd, q, out):
         b.free()
     return res
+
+
+def bench_reference_cell(stream) -> dict:
+    """The one cell the reference publishes stage times for (crates/breccia-kernels/src/qsa/bench.rs:28-33,
+    numbers docs/phase-4/01-forward-pass.md:4650-4664, RX 6950 XT): one sequence, T = 1, 24 q / 2 kv
+    heads, 512 selected blocks + the token's own block = 2051 cells, gate on, f16 and q8_0 V.  Stages
+    here: kv-append (T = 1), selection (indexer score over every pooled block + exact top-512), attention
+    over the list (split-K + merge, gate applied in the merge), and the three enqueued back to back."""
+    from breccia_amd import lib as L
+    from breccia_amd.kv import DeviceBuffer, Event, Pool
+
+    n_q, ctx = 24, 16387                 # pos 16386: the own block holds 3 cells -> 512 * 4 + 3 = 2051
+    pos, max_ids = ctx - 1, 513
+    rng = np.random.Generator(np.random.PCG64(20250011))
+    published = {"hardware": "RX 6950 XT (the reference's own GPU; context, not a like-for-like target)",
+                 "source": "docs/phase-4/01-forward-pass.md:4650-4664",
+                 "kv_append_us": {"f16": 2.11, "q8v": 6.29}, "attn_scores_softmax_us": 1945.1,
+                 "attn_apply_gate_us": {"f16": 649.0, "q8v": 622.4}, "layer_total_us": {"f16": 2707.8, "q8v": 2693.9}}
+    res = {"workload": "1 sequence at ctx %d, T = 1, 24 q / 2 kv heads, 512 selected blocks + own block = 2051 "
+                       "cells, gate on" % ctx, "reference_published": published}
+    rows = DeviceBuffer.from_numpy(rng.standard_normal((ctx, N_KV, HD), dtype=np.float32))
+    new = DeviceBuffer.from_numpy(rng.standard_normal((1, N_KV, HD), dtype=np.float32))
+    q = DeviceBuffer.from_numpy(rng.standard_normal((1, n_q, HD), dtype=np.float32))
+    gate = DeviceBuffer.from_numpy(rng.standard_normal((1, n_q, HD), dtype=np.float32))
+    out = DeviceBuffer(n_q * HD * 4)
+    n_blocks = pos // 4
+    pooled = DeviceBuffer.from_numpy(rng.standard_normal((n_blocks, 128), dtype=np.float32))
+    iq = DeviceBuffer.from_numpy(rng.standard_normal((1, 4, 128), dtype=np.float32))
+    ids = DeviceBuffer(max_ids * 4)
+    cnt = DeviceBuffer(16)
+
+    def timed(fn, reps=200):
+        for _ in range(20):
+            fn()
+        stream.sync()
+        e0, e1 = Event(), Event()
+        e0.record(stream)
+        for _ in range(reps):
+            fn()
+        e1.record(stream)
+        stream.sync()
+        us = e0.elapsed_ms(e1) / reps * 1e3
+        e0.close()
+        e1.close()
+        return round(us, 2)
+
+    for tag, layout in (("f16", L.LAYOUT_F16), ("q8v", L.LAYOUT_Q8V)):
+        pool = Pool(n_layers=1, n_pages=ctx // PAGE + 64, n_kv_head=N_KV, head_dim=HD, max_seqs=2,
+                    max_pages_per_seq=ctx // PAGE + 8, layout=layout)
+        pool.set_free_order(rng.permutation(ctx // PAGE + 64).astype(np.int32))
+        s = pool.seq_create()
+        pool.seq_reserve(s, ctx)
+        pool.append(0, [s], [0], [ctx], rows, rows, stream)
+        stream.sync()
+
+        def append():
+            pool.append(0, [s], [pos], [1], new, new, stream)
+
+        def select():
+            pool.select_blocks([pos], iq, [pooled], [n_blocks], 4, 128, 512, ids, max_ids, cnt, max_ids, stream=stream)
+
+        def attend():
+            pool.decode_attn_select(0, [s], [pos], n_q, q, out, 1.0 / 16.0, ids, max_ids, cnt, max_ids,
+                                    gate_dev=gate, gate_seq_stride=n_q * HD, gate_head_stride=HD, stream=stream)
+
+        def layer():
+            append()
+            select()
+            attend()
+
+        select()
+        stream.sync()
+        n_sel = int(cnt.download(np.uint32, 1, stream)[0])
+        r = {"selected_blocks": n_sel, "kv_append_us": timed(append), "select_us": timed(select),
+             "attn_over_list_us": timed(attend), "layer_total_us": timed(layer)}
+        pool.timing_reset()
+        pool.timing_enable(True)
+        for _ in range(50):
+            layer()
+        stream.sync()
+        pool.timing_enable(False)
+        for name, stage in (("append", L.STAGE_APPEND), ("idx_score", L.STAGE_IDX_SCORE), ("topk", L.STAGE_TOPK),
+                            ("attn_split", L.STAGE_ATTN_SPLIT), ("attn_merge", L.STAGE_ATTN_MERGE)):
+            n_k, ms_k = pool.timing_read(stage)
+            r[name + "_kernel_us"] = round(ms_k / max(n_k, 1) * 1e3, 2)
+        res[tag] = r
+        pool.destroy()
+    for b in (rows, new, q, gate, out, pooled, iq, ids, cnt):
+        b.free()
+    return {"reference_cell": res}
+
+
+def bench_config3_scenario(stream) -> dict:
+    """BASELINE configs[3] as worded, timed end to end on one pool: four sequences share a 2040-token
+    prefix (127 full pages + a partial one) through refcounts; each appends a distinct 1024-token chunk of
+    binary16 K/V (bkv_append_f16), which costs the writers that still share the partial page one
+    copy-on-write page copy each; then a seeded 25 % of the pages in use go to pinned host memory and come
+    back.  12 layers (the model's full-attention layers), so that a page is 12 x 32 KiB.  At these sizes the
+    append and the copies are launch-bound; the bulk legs of bench_moves price the kernels."""
+    from breccia_amd.kv import DeviceBuffer, Event, Pool
+
+    rng = np.random.Generator(np.random.PCG64(20250004))
+    n_layers, prefix, chunk, n_pages = 12, 2040, 1024, 1024
+    pool = Pool(n_layers=n_layers, n_pages=n_pages, n_kv_head=N_KV, head_dim=HD, max_seqs=8,
+                max_pages_per_seq=(prefix + chunk) // PAGE + 4)
+    pool.set_free_order(rng.permutation(n_pages).astype(np.int32))
+    k16 = DeviceBuffer.from_numpy(rng.standard_normal((prefix + 4 * chunk, N_KV, HD), dtype=np.float32).astype(np.float16))
+    v16 = DeviceBuffer.from_numpy(rng.standard_normal((prefix + 4 * chunk, N_KV, HD), dtype=np.float32).astype(np.float16))
+    row = N_KV * HD * 2
+    root = pool.seq_create()
+    pool.seq_reserve(root, prefix)
+    for layer in range(n_layers):
+        pool.append(0 + layer, [root], [0], [prefix], k16, v16, stream, f16_rows=True)
+    seqs = [root] + [pool.seq_fork(root, prefix) for _ in range(3)]
+    stream.sync()
+    e = [Event() for _ in range(4)]
+    pairs_all = [pool.seq_reserve(s, prefix + chunk) for s in seqs]
+    # copy-on-write copies (all layers of a page in one call), then the four chunks, layer by layer
+    e[0].record(stream)
+    for pairs in pairs_all:
+        pool.page_copy(pairs, stream)
+    e[1].record(stream)
+    for layer in range(n_layers):
+        for i, s in enumerate(seqs):
+            off = (prefix + i * chunk) * row
+            pool.append(layer, [s], [prefix], [chunk], k16.at(off), v16.at(off), stream, f16_rows=True)
+    e[2].record(stream)
+    stream.sync()
+    n_copies = sum(len(p) for p in pairs_all)
+    copy_ms, append_ms = e[0].elapsed_ms(e[1]), e[1].elapsed_ms(e[2])
+    used = np.unique(np.concatenate([pool.block_table(s) for s in seqs]))
+    cold = rng.choice(used, size=used.size // 4, replace=False).astype(np.int32)
+    slab = pool.swap_page_bytes()
+    host = pool.host_alloc(cold.size * slab)
+    pool.swap_out(cold[:8], host, stream)       # the staging halves' and the side stream's one-time costs
+    pool.swap_wait()
+    t0 = time.perf_counter()
+    pool.swap_out(cold, host, stream)
+    pool.swap_wait()
+    t_out = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    pool.swap_in(cold, host, stream)
+    pool.swap_fence(stream)
+    stream.sync()
+    t_in = time.perf_counter() - t0
+    app_bytes = 4 * chunk * n_layers * N_KV * HD * (2 + 2) * 2
+    copy_bytes = n_copies * n_layers * 2 * 32768
+    res = {"workload": "BASELINE configs[3]: 4 sequences on a shared 2040-token prefix, 1024-token f16 chunks "
+                       "(bkv_append_f16), copy-on-write of the partial page, 25 % of pages out and back; 12 layers",
+           "cow_copies": n_copies, "cow_copy_us_each": round(copy_ms * 1e3 / max(n_copies, 1), 2),
+           "cow_copy_GBps": round(copy_bytes / max(copy_ms, 1e-9) / 1e6, 1),
+           "append_calls": 4 * n_layers, "append_us_per_call": round(append_ms * 1e3 / (4 * n_layers), 2),
+           "append_GBps": round(app_bytes / append_ms / 1e6, 1),
+           "swap_pages": int(cold.size), "swap_bytes": int(cold.size * slab),
+           "swap_out_GBps": round(cold.size * slab / t_out / 1e9, 2),
+           "swap_in_GBps": round(cold.size * slab / t_in / 1e9, 2)}
+    host.free()
+    for x in e:
+        x.close()
+    k16.free()
+    v16.free()
+    pool.destroy()
+    return {"config3_scenario": res}
 
 
 def bench_prefix_tiers(stream) -> dict:

@@ -14,6 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libbreccia_kv.so")
+BENCH_LIB = os.path.join(HERE, "libbreccia_kv_bench.so")
 
 SOURCES = ["allocator.cpp", "prefix_tree.cpp", "api.hip", "kv_move.hip", "decode_attn.hip", "decode_attn_mfma.hip", "prefill_attn.hip", "select.hip"]
 ARCH = "gfx950"
@@ -56,6 +57,11 @@ def build(verbose: bool = False) -> str:
     if verbose:
         print(" ".join(cmd))
     _run(cmd)
+    # the tests' and the benchmark's device plumbing and bandwidth probes: a library of its own
+    obj = os.path.join(OBJ, "bench_support.o")
+    _run([hipcc] + HIP_FLAGS + ["-I", os.path.join(HERE, "..", "include"), "-c",
+                                os.path.join(CSRC, "bench_support.hip"), "-o", obj])
+    _run([hipcc, "-shared", "-fPIC", "--offload-arch=" + ARCH, obj, "-o", BENCH_LIB])
     return LIB
 
 
@@ -65,7 +71,7 @@ def build_cpp_mirror_test(verbose: bool = False) -> str:
     src = os.path.join(root, "tests", "cpp", "qsa_mirror_test.cpp")
     out = os.path.join(root, "tests", "cpp", "qsa_mirror_test")
     cmd = ["g++", "-std=c++17", "-O2", "-Wall", src, "-o", out,
-           "-L" + HERE, "-lbreccia_kv", "-L" + os.path.join(root, "oracle"), "-lbkv_oracle",
+           "-L" + HERE, "-lbreccia_kv", "-lbreccia_kv_bench", "-L" + os.path.join(root, "oracle"), "-lbkv_oracle",
            "-Wl,-rpath,$ORIGIN/../../breccia_amd", "-Wl,-rpath,$ORIGIN/../../oracle",
            "-Wl,-rpath,/opt/rocm/lib"]
     if verbose:

@@ -3,10 +3,12 @@
 // before anything reaches the GPU (the reference's contract, crates/breccia-kernels/
 // src/qsa/mod.rs:1108-1116).
 #include <algorithm>
+#include <atomic>
 #include <chrono>
 #include <cstdio>
 #include <cstring>
 #include <new>
+#include <thread>
 #include <unordered_map>
 
 #include <cerrno>
@@ -54,6 +56,46 @@ static bkv_status from_alloc(AllocErr e, const std::string& msg) {
 
 static inline hipStream_t S(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
+// ---- bounded host waits ---------------------------------------------------------------
+// The reference never waits on its device without a deadline (crates/breccia-vk/src/ctx.rs:
+// 1545-1553: WAIT_TIMEOUT_NS = 10 s, then a diagnostic instead of a hang).  Every host-side wait
+// of this library -- for a stream, for an event -- polls the HIP query call up to a deadline and
+// returns BKV_ERR_TIMEOUT with what it was waiting for; nothing is aborted, the work stays
+// enqueued and a later wait can succeed.  The first `poll_us` microseconds of a wait spin on the
+// query (a thread that sleeps in hipStreamSynchronize is woken some tens of microseconds after the
+// stream has drained, which a decode loop that waits per token would pay every time); after that
+// the thread naps 50 us between queries.  Process-wide settings (bkv_wait_options).
+static std::atomic<int64_t> g_wait_timeout_ms{10000};
+static std::atomic<int64_t> g_wait_poll_us{4000};
+
+template <typename Query>
+static bkv_status bounded_wait(Query query, int64_t timeout_ms, const char* call, const std::string& what) {
+    const auto t0 = std::chrono::steady_clock::now();
+    const auto spin = std::chrono::microseconds(g_wait_poll_us.load(std::memory_order_relaxed));
+    for (;;) {
+        const hipError_t e = query();
+        if (e == hipSuccess) return BKV_OK;
+        if (e != hipErrorNotReady) return hip_fail(e, call);
+        (void)hipGetLastError();
+        const auto waited = std::chrono::steady_clock::now() - t0;
+        if (timeout_ms >= 0 && waited >= std::chrono::milliseconds(timeout_ms))
+            return fail(BKV_ERR_TIMEOUT, sfmt("timed out after %lld ms waiting for ", timeout_ms) + what +
+                                             ": the work is still enqueued, nothing was cancelled");
+        if (waited < spin)
+            __builtin_ia32_pause();
+        else
+            std::this_thread::sleep_for(std::chrono::microseconds(50));
+    }
+}
+static bkv_status wait_stream(hipStream_t stream, int64_t timeout_ms, const std::string& what) {
+    return bounded_wait([&] { return hipStreamQuery(stream); }, timeout_ms, "hipStreamQuery", what);
+}
+static bkv_status wait_event(hipEvent_t ev, const std::string& what) {
+    return bounded_wait([&] { return hipEventQuery(ev); }, g_wait_timeout_ms.load(std::memory_order_relaxed),
+                        "hipEventQuery", what);
+}
+static int64_t default_timeout_ms() { return g_wait_timeout_ms.load(std::memory_order_relaxed); }
+
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // ---- parameter ring ---------------------------------------------------------------
@@ -64,7 +106,10 @@ bkv_status ring_upload(bkv_pool* p, const void* host_src, size_t bytes, hipStrea
         return fail(BKV_ERR_INVALID, "internal: parameter list larger than a ring slot");
     const int slot = r.next;
     r.next = (r.next + 1) % ParamRing::kSlots;
-    if (r.used[slot]) BKV_HIP(hipEventSynchronize(r.ev[slot]));
+    if (r.used[slot]) {
+        const bkv_status ws = wait_event(r.ev[slot], "the last reader of an argument-ring slot");
+        if (ws != BKV_OK) return ws;
+    }
     uint8_t* h = r.host + (size_t)slot * ParamRing::kSlotBytes;
     uint8_t* d = r.dev + (size_t)slot * ParamRing::kSlotBytes;
     std::memcpy(h, host_src, bytes);
@@ -111,18 +156,26 @@ static bkv_status order_workspace(WorkspaceOrder& w, hipStream_t stream) {
     return BKV_OK;
 }
 
+// Block-table updates are scattered on whichever stream brings the next call.  A call on another
+// stream reads the same table: it waits for the last scatter (until that is known to be over).
+// `may_query` false: only the wait is enqueued, no host-side look at the event (for streams that
+// may be under capture).
+static bkv_status wait_for_table_scatter(bkv_pool* p, hipStream_t stream, bool may_query) {
+    if (!p->table_sync.used || p->table_sync.last == stream) return BKV_OK;
+    if (may_query && hipEventQuery(p->table_sync.ev) == hipSuccess) {
+        p->table_sync.used = false;
+        return BKV_OK;
+    }
+    (void)hipGetLastError();
+    BKV_HIP(hipStreamWaitEvent(stream, p->table_sync.ev, 0));
+    return BKV_OK;
+}
+
 bkv_status flush_tables(bkv_pool* p, hipStream_t stream) {
     bkv_status tier_st = wait_for_tier_moves(p, stream);
     if (tier_st != BKV_OK) return tier_st;
-    // Block-table updates are scattered on whichever stream brings the next call.  A call on
-    // another stream reads the same table: it waits for the last scatter (until that is known to
-    // be over).
-    if (p->table_sync.used && p->table_sync.last != stream) {
-        if (hipEventQuery(p->table_sync.ev) == hipSuccess)
-            p->table_sync.used = false;
-        else
-            BKV_HIP(hipStreamWaitEvent(stream, p->table_sync.ev, 0));
-    }
+    const bkv_status ts = wait_for_table_scatter(p, stream, true);
+    if (ts != BKV_OK) return ts;
     std::vector<TableUpdate>& pend = p->alloc->pending();
     if (pend.empty()) return BKV_OK;
     if (p->host_only) {
@@ -188,11 +241,12 @@ bool timer_dispatch_events(bkv_pool* p, int stage, hipEvent_t* start, hipEvent_t
 bkv_status timer_collect(bkv_pool* p) {
     StageTimer& t = p->timer;
     hipError_t err = hipSuccess;
+    bool timed_out = false;  // the event pairs are dropped either way; the error text is wait_event's
     for (const StageTimer::Pair& pr : t.open) {
         float ms = 0.0f;
-        if (err == hipSuccess) err = hipEventSynchronize(pr.stop);
-        if (err == hipSuccess) err = hipEventElapsedTime(&ms, pr.start, pr.stop);
-        if (err == hipSuccess) {
+        if (err == hipSuccess && !timed_out) timed_out = wait_event(pr.stop, "a timed kernel") != BKV_OK;
+        if (err == hipSuccess && !timed_out) err = hipEventElapsedTime(&ms, pr.start, pr.stop);
+        if (err == hipSuccess && !timed_out) {
             t.launches[pr.stage] += 1;
             t.total_ms[pr.stage] += (double)ms;
         }
@@ -204,6 +258,7 @@ bkv_status timer_collect(bkv_pool* p) {
         (void)hipEventDestroy(pr.stop);
     }
     t.open.clear();
+    if (timed_out) return BKV_ERR_TIMEOUT;
     BKV_HIP(err);
     return BKV_OK;
 }
@@ -1004,6 +1059,10 @@ struct bkv_step_plan {
     float* part_ml = nullptr;
     int32_t n = 0, n_q_head = 0, grid = 0;
     AttnPlanLimits lim{};
+    // The descriptor is uploaded on the stream of bkv_step_plan_create, rewritten by every advance
+    // and read by every decode: a call that arrives on another stream than the plan's last one is
+    // ordered behind it with an event recorded there at that moment.
+    WorkspaceOrder order;
     // what the plan was checked for: cells first[i]..last[i] of sequence seq[i]
     int32_t seq[kMaxBatch] = {};
     int64_t first[kMaxBatch] = {}, last[kMaxBatch] = {};
@@ -1106,6 +1165,8 @@ bkv_status bkv_step_plan_create(bkv_pool* p, int32_t n, const int32_t* seqs, con
     if (e != hipSuccess) return bail(hip_fail(e, "hipMemcpyAsync (step plan)"));
     st = ring_done(p, slot, S(stream));
     if (st != BKV_OK) return bail(st);
+    pl->order.last = S(stream);
+    pl->order.used = true;
     *out = pl;
     return BKV_OK;
 }
@@ -1113,6 +1174,7 @@ bkv_status bkv_step_plan_create(bkv_pool* p, int32_t n, const int32_t* seqs, con
 bkv_status bkv_step_plan_destroy(bkv_step_plan* pl) {
     if (!pl) return fail(BKV_ERR_INVALID, "step_plan_destroy: NULL plan");
     (void)hipDeviceSynchronize();
+    if (pl->order.ev) (void)hipEventDestroy(pl->order.ev);
     if (pl->dev) (void)hipFree(pl->dev);
     if (pl->part_o) (void)hipFree(pl->part_o);
     if (pl->part_ml) (void)hipFree(pl->part_ml);
@@ -1145,6 +1207,12 @@ bkv_status bkv_step_plan_decode(bkv_step_plan* pl, int32_t layer, const float* k
         const bkv_status st = flush_tables(p, S(stream));
         if (st != BKV_OK) return st;
     }
+    // Nothing pending does not mean nothing in flight: the last scatter may still run on another
+    // stream (the wait is a stream operation a capture can record), and so may the plan's own last
+    // upload or advance.
+    bkv_status ord = wait_for_table_scatter(p, S(stream), false);
+    if (ord == BKV_OK) ord = order_workspace(pl->order, S(stream));
+    if (ord != BKV_OK) return ord;
     AttnBatch b{};
     b.n = pl->n;
     AttnArgs a;
@@ -1168,6 +1236,8 @@ bkv_status bkv_step_plan_decode(bkv_step_plan* pl, int32_t layer, const float* k
 
 bkv_status bkv_step_plan_advance(bkv_step_plan* pl, void* stream) {
     if (!pl) return fail(BKV_ERR_INVALID, "step_plan_advance: NULL plan");
+    const bkv_status ord = order_workspace(pl->order, S(stream));
+    if (ord != BKV_OK) return ord;
     BKV_HIP(launch_step_advance(pl->dev, pl->lim, pl->pool->g.page_cells, S(stream)));
     return BKV_OK;
 }
@@ -1176,7 +1246,10 @@ bkv_status bkv_step_plan_state(bkv_step_plan* pl, void* stream, int64_t* pos_out
                                int32_t* status_out) {
     if (!pl) return fail(BKV_ERR_INVALID, "step_plan_state: NULL plan");
     StepDesc host;
-    BKV_HIP(hipStreamSynchronize(S(stream)));
+    const bkv_status ord = order_workspace(pl->order, S(stream));
+    if (ord != BKV_OK) return ord;
+    const bkv_status ws = wait_stream(S(stream), default_timeout_ms(), "the stream of a step plan");
+    if (ws != BKV_OK) return ws;
     BKV_HIP(hipMemcpy(&host, pl->dev, sizeof(host), hipMemcpyDeviceToHost));
     if (pos_out)
         for (int i = 0; i < pl->n; ++i) pos_out[i] = host.b.pos[i];
@@ -1554,10 +1627,34 @@ bkv_status bkv_swap_in(bkv_pool* p, const int32_t* pages, int32_t n, const void*
                      false, S(stream));
 }
 
-bkv_status bkv_swap_wait(bkv_pool* p) {
+static bkv_status wait_side(bkv_pool* p, int64_t timeout_ms) {
+    return wait_stream(p->side, timeout_ms, "the pool's side stream (page transfers to or from host memory)");
+}
+
+bkv_status bkv_swap_wait_for(bkv_pool* p, int64_t timeout_ms) {
     bkv_status st = need_device(p);
     if (st != BKV_OK) return st;
-    BKV_HIP(hipStreamSynchronize(p->side));
+    return wait_side(p, timeout_ms);
+}
+
+bkv_status bkv_swap_wait(bkv_pool* p) { return bkv_swap_wait_for(p, default_timeout_ms()); }
+
+bkv_status bkv_stream_wait(void* stream, int64_t timeout_ms) {
+    return wait_stream(S(stream), timeout_ms, "a caller stream");
+}
+
+bkv_status bkv_wait_options(int64_t timeout_ms, int64_t poll_us) {
+    if (timeout_ms == 0) return fail(BKV_ERR_INVALID, "wait_options: a default timeout of 0 ms would fail every wait; "
+                                                      "negative = no deadline");
+    if (poll_us < 0) return fail(BKV_ERR_INVALID, "wait_options: the spin window cannot be negative");
+    g_wait_timeout_ms.store(timeout_ms, std::memory_order_relaxed);
+    g_wait_poll_us.store(poll_us, std::memory_order_relaxed);
+    return BKV_OK;
+}
+
+bkv_status bkv_wait_options_get(int64_t* timeout_ms, int64_t* poll_us) {
+    if (timeout_ms) *timeout_ms = g_wait_timeout_ms.load(std::memory_order_relaxed);
+    if (poll_us) *poll_us = g_wait_poll_us.load(std::memory_order_relaxed);
     return BKV_OK;
 }
 
@@ -1686,7 +1783,10 @@ static bkv_status run_tier_moves(bkv_pool* p, const std::vector<TierMove>& moves
                 if (st != BKV_OK) return st;
                 copies.clear();
                 copy_slots.clear();
-                if (wait) BKV_HIP(hipStreamSynchronize(p->side));
+                if (wait) {
+                    const bkv_status ws = wait_side(p, default_timeout_ms());
+                    if (ws != BKV_OK) return ws;
+                }
             }
             return BKV_OK;
         };
@@ -1720,7 +1820,10 @@ static bkv_status run_tier_moves(bkv_pool* p, const std::vector<TierMove>& moves
         std::sort(from_disk.begin(), from_disk.end(),
                   [](const TierMove& a, const TierMove& b) { return a.disk_slot < b.disk_slot; });
         // an earlier call's upload may still be reading the bounce buffer
-        BKV_HIP(hipStreamSynchronize(p->side));
+        {
+            const bkv_status ws = wait_side(p, default_timeout_ms());
+            if (ws != BKV_OK) return ws;
+        }
         bool half_in_flight[2] = {false, false};
         int half = 0;
         std::vector<int32_t> pages;
@@ -1731,7 +1834,8 @@ static bkv_status run_tier_moves(bkv_pool* p, const std::vector<TierMove>& moves
                 ++j;
             uint8_t* buf = ts.bounce + (uint64_t)half * ts.bounce_slots * slab;
             if (half_in_flight[half]) {
-                BKV_HIP(hipStreamSynchronize(p->side));
+                const bkv_status ws = wait_side(p, default_timeout_ms());
+                if (ws != BKV_OK) return ws;
                 half_in_flight[0] = half_in_flight[1] = false;
             }
             const uint64_t bytes = (uint64_t)(j - i) * slab;
@@ -1764,7 +1868,8 @@ bkv_status bkv_prefix_tiers(bkv_pool* p, uint64_t host_bytes, const char* disk_p
     // what the lower tiers hold now goes first
     p->prefix->set_tiers(0, 0);
     if (!p->host_only) {
-        BKV_HIP(hipStreamSynchronize(p->side));
+        const bkv_status ws = wait_side(p, default_timeout_ms());
+        if (ws != BKV_OK) return ws;
         if (ts.host) BKV_HIP(hipHostFree(ts.host));
         if (ts.bounce) BKV_HIP(hipHostFree(ts.bounce));
     }
@@ -1882,147 +1987,6 @@ bkv_status bkv_timing_read(bkv_pool* p, int stage, uint64_t* launches, double* t
     if (st != BKV_OK) return st;
     if (launches) *launches = p->timer.launches[stage];
     if (total_ms) *total_ms = p->timer.total_ms[stage];
-    return BKV_OK;
-}
-
-// ---- device plumbing ------------------------------------------------------------------
-bkv_status bkv_dev_alloc(uint64_t bytes, void** dev_out) {
-    if (!dev_out) return fail(BKV_ERR_INVALID, "dev_alloc: NULL out pointer");
-    BKV_HIP(hipMalloc(dev_out, bytes ? bytes : 16));
-    return BKV_OK;
-}
-bkv_status bkv_dev_free(void* dev) {
-    if (dev) BKV_HIP(hipFree(dev));
-    return BKV_OK;
-}
-bkv_status bkv_memcpy_h2d(void* dev, const void* host, uint64_t bytes, void* stream) {
-    BKV_HIP(hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, S(stream)));
-    return BKV_OK;
-}
-bkv_status bkv_memcpy_d2h(void* host, const void* dev, uint64_t bytes, void* stream) {
-    BKV_HIP(hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, S(stream)));
-    return BKV_OK;
-}
-bkv_status bkv_graph_begin_capture(void* stream) {
-    if (!stream) return fail(BKV_ERR_INVALID, "graph_begin_capture: the NULL stream cannot be captured");
-    BKV_HIP(hipStreamBeginCapture(S(stream), hipStreamCaptureModeThreadLocal));
-    return BKV_OK;
-}
-
-bkv_status bkv_graph_end_capture(void* stream, void** graph_exec_out) {
-    if (!stream || !graph_exec_out) return fail(BKV_ERR_INVALID, "graph_end_capture: NULL argument");
-    *graph_exec_out = nullptr;
-    hipGraph_t graph = nullptr;
-    BKV_HIP(hipStreamEndCapture(S(stream), &graph));
-    hipGraphExec_t exec = nullptr;
-    const hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
-    (void)hipGraphDestroy(graph);
-    if (e != hipSuccess) return hip_fail(e, "hipGraphInstantiate");
-    *graph_exec_out = exec;
-    return BKV_OK;
-}
-
-bkv_status bkv_graph_launch(void* graph_exec, void* stream) {
-    if (!graph_exec) return fail(BKV_ERR_INVALID, "graph_launch: NULL graph");
-    BKV_HIP(hipGraphLaunch(static_cast<hipGraphExec_t>(graph_exec), S(stream)));
-    return BKV_OK;
-}
-
-bkv_status bkv_graph_destroy(void* graph_exec) {
-    if (!graph_exec) return fail(BKV_ERR_INVALID, "graph_destroy: NULL graph");
-    BKV_HIP(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec)));
-    return BKV_OK;
-}
-
-bkv_status bkv_stream_create(void** stream_out) {
-    if (!stream_out) return fail(BKV_ERR_INVALID, "stream_create: NULL out pointer");
-    hipStream_t s;
-    BKV_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
-    *stream_out = s;
-    return BKV_OK;
-}
-bkv_status bkv_stream_destroy(void* stream) {
-    if (stream) BKV_HIP(hipStreamDestroy(S(stream)));
-    return BKV_OK;
-}
-// The host polls the stream for a few milliseconds before it blocks: a thread that sleeps in
-// hipStreamSynchronize is woken some tens of microseconds after the stream has drained, which a
-// decode loop that synchronises per token would pay every time.
-bkv_status bkv_stream_sync(void* stream) {
-    const auto t0 = std::chrono::steady_clock::now();
-    for (;;) {
-        const hipError_t e = hipStreamQuery(S(stream));
-        if (e == hipSuccess) return BKV_OK;
-        if (e != hipErrorNotReady) return hip_fail(e, "hipStreamQuery");
-        (void)hipGetLastError();
-        if (std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(4)) break;
-    }
-    BKV_HIP(hipStreamSynchronize(S(stream)));
-    return BKV_OK;
-}
-bkv_status bkv_device_sync(void) {
-    BKV_HIP(hipDeviceSynchronize());
-    return BKV_OK;
-}
-bkv_status bkv_event_create(void** event_out) {
-    if (!event_out) return fail(BKV_ERR_INVALID, "event_create: NULL out pointer");
-    hipEvent_t e;
-    BKV_HIP(hipEventCreate(&e));
-    *event_out = e;
-    return BKV_OK;
-}
-bkv_status bkv_event_destroy(void* event) {
-    if (event) BKV_HIP(hipEventDestroy(reinterpret_cast<hipEvent_t>(event)));
-    return BKV_OK;
-}
-bkv_status bkv_event_record(void* event, void* stream) {
-    BKV_HIP(hipEventRecord(reinterpret_cast<hipEvent_t>(event), S(stream)));
-    return BKV_OK;
-}
-bkv_status bkv_event_sync(void* event) {
-    BKV_HIP(hipEventSynchronize(reinterpret_cast<hipEvent_t>(event)));
-    return BKV_OK;
-}
-bkv_status bkv_event_elapsed_ms(void* start, void* stop, float* ms_out) {
-    if (!ms_out) return fail(BKV_ERR_INVALID, "event_elapsed_ms: NULL out pointer");
-    BKV_HIP(hipEventElapsedTime(ms_out, reinterpret_cast<hipEvent_t>(start),
-                                reinterpret_cast<hipEvent_t>(stop)));
-    return BKV_OK;
-}
-bkv_status bkv_device_info(char* name_out, int32_t name_cap, int32_t* cu_out,
-                           uint64_t* mem_bytes_out) {
-    int dev = 0;
-    BKV_HIP(hipGetDevice(&dev));
-    hipDeviceProp_t prop;
-    BKV_HIP(hipGetDeviceProperties(&prop, dev));
-    if (name_out && name_cap > 0) {
-        std::snprintf(name_out, (size_t)name_cap, "%s (%s)", prop.name, prop.gcnArchName);
-    }
-    if (cu_out) *cu_out = prop.multiProcessorCount;
-    if (mem_bytes_out) *mem_bytes_out = prop.totalGlobalMem;
-    return BKV_OK;
-}
-bkv_status bkv_copy_probe(void* dst_dev, const void* src_dev, uint64_t bytes, void* stream) {
-    if (!dst_dev || !src_dev || !aligned16(dst_dev) || !aligned16(src_dev) || bytes % 16)
-        return fail(BKV_ERR_INVALID, "copy_probe: pointers and size must be 16-byte multiples");
-    BKV_HIP(launch_copy_probe(dst_dev, src_dev, bytes, S(stream)));
-    return BKV_OK;
-}
-
-bkv_status bkv_read_probe(const void* src_dev, uint64_t bytes, int32_t scattered, void* sink_dev, void* stream) {
-    if (!src_dev || !sink_dev || !aligned16(src_dev) || ((uintptr_t)sink_dev & 3u))
-        return fail(BKV_ERR_INVALID, "read_probe: NULL or misaligned pointer");
-    const uint64_t chunks = bytes / 8192;
-    if (bytes % 8192 != 0 || chunks == 0 || chunks > 0x7fffffffull || (chunks & (chunks - 1)) != 0)
-        return fail(BKV_ERR_INVALID, sfmt("read_probe: %lld bytes; need a power-of-two number of 8 KiB chunks",
-                                          (long long)bytes));
-    if (scattered < 0 || scattered > 2)
-        return fail(BKV_ERR_INVALID, sfmt("read_probe: order %lld (0 = address order, 1 = scattered, 2 = scattered "
-                                          "through global->LDS loads)", scattered));
-    int dev = 0, n_cu = 0;
-    BKV_HIP(hipGetDevice(&dev));
-    BKV_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
-    BKV_HIP(launch_read_probe(src_dev, bytes, scattered, sink_dev, n_cu, S(stream)));
     return BKV_OK;
 }
 

@@ -272,8 +272,5 @@ hipError_t launch_table_scatter(int32_t* table, const TableUpdate* upd_dev, int3
 constexpr int32_t kTableUpdatesInArgs = 32;
 hipError_t launch_table_scatter_args(int32_t* table, const TableUpdate* upd_host, int32_t n, hipStream_t stream);
 hipError_t launch_fill(void* dst, uint64_t bytes, uint32_t word, hipStream_t stream);
-hipError_t launch_copy_probe(void* dst, const void* src, uint64_t bytes, hipStream_t stream);
-hipError_t launch_read_probe(const void* src, uint64_t bytes, int32_t mode, void* sink, int32_t n_cu,
-                             hipStream_t stream);
 
 }  // namespace bkv

@@ -665,86 +665,6 @@ __global__ __launch_bounds__(kBlock) void fill_kernel(uint4* __restrict__ dst, u
         dst[i] = w;
 }
 
-__global__ __launch_bounds__(kBlock) void copy_probe_kernel(uint4* __restrict__ dst,
-                                                            const uint4* __restrict__ src,
-                                                            uint64_t n_vec) {
-    const uint64_t stride = (uint64_t)gridDim.x * kBlock;
-    uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
-    for (; i + 3 * stride < n_vec; i += 4 * stride) {
-        const uint4 a = src[i], b = src[i + stride], c = src[i + 2 * stride],
-                    d = src[i + 3 * stride];
-        dst[i] = a;
-        dst[i + stride] = b;
-        dst[i + 2 * stride] = c;
-        dst[i + 3 * stride] = d;
-    }
-    for (; i < n_vec; i += stride) dst[i] = src[i];
-}
-
-// Read-only bandwidth probe: every wave reads 8 KiB chunks (8 wave-loads of 1 KiB, the shape of
-// one (page, kv head) run of a pool) and folds them into a value nothing depends on.  Chunk c of
-// the walk is chunk c of the buffer, or, scattered, chunk (c * odd) mod n_chunks of it (n_chunks a
-// power of two: a bijection), which is how a shuffled pool looks to the attention kernels.
-typedef unsigned probe_v4u __attribute__((ext_vector_type(4)));
-__global__ __launch_bounds__(kBlock) void read_probe_kernel(const probe_v4u* __restrict__ src, uint32_t n_chunks,
-                                                            uint32_t scatter_mul, uint32_t* __restrict__ sink) {
-    const uint32_t lane = threadIdx.x & 63u;
-    const uint32_t wave = (blockIdx.x * kBlock + threadIdx.x) >> 6;
-    const uint32_t n_waves = gridDim.x * (kBlock / 64);
-    probe_v4u acc = probe_v4u{0u, 0u, 0u, 0u};
-    for (uint32_t c = wave; c < n_chunks; c += 2 * n_waves) {
-        const uint32_t c1 = c + n_waves < n_chunks ? c + n_waves : c;
-        const probe_v4u* a = src + (size_t)((c * scatter_mul) & (n_chunks - 1u)) * 512u + lane;
-        const probe_v4u* b = src + (size_t)((c1 * scatter_mul) & (n_chunks - 1u)) * 512u + lane;
-        probe_v4u r[16];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) r[i] = __builtin_nontemporal_load(a + i * 64);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) r[8 + i] = __builtin_nontemporal_load(b + i * 64);
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            acc ^= r[i];
-        }
-    }
-    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u) sink[0] = 1u;  // keeps the loads alive
-}
-
-// The scattered walk again, every chunk fetched with 16-byte global->LDS loads instead of loads into
-// registers (two 8 KiB slots per wave, the next chunk in flight while one word a lane of the landed
-// one is folded): the mechanism the quantised attention kernels used first.  It streams about a tenth
-// slower than the register path on this chip, which is why they moved off it; the probe keeps that
-// comparison reproducible.
-__global__ __launch_bounds__(kBlock) void read_probe_lds_kernel(const probe_v4u* __restrict__ src, uint32_t n_chunks,
-                                                                uint32_t scatter_mul, uint32_t* __restrict__ sink) {
-    typedef const __attribute__((address_space(1))) void* gptr;
-    typedef __attribute__((address_space(3))) void* lptr;
-    __shared__ __attribute__((aligned(16))) probe_v4u stage[(kBlock / 64) * 2 * 512];
-    const uint32_t lane = threadIdx.x & 63u;
-    const uint32_t wv = threadIdx.x >> 6;
-    const uint32_t wave = (blockIdx.x * kBlock + threadIdx.x) >> 6;
-    const uint32_t n_waves = gridDim.x * (kBlock / 64);
-    probe_v4u* const mine = stage + wv * 2 * 512;
-    const auto request = [&](uint32_t c, uint32_t slot) {
-        const probe_v4u* a = src + (size_t)((c * scatter_mul) & (n_chunks - 1u)) * 512u + lane;
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-            __builtin_amdgcn_global_load_lds((gptr)(a + i * 64), (lptr)(mine + slot * 512 + i * 64), 16, 0, 0);
-    };
-    probe_v4u acc = probe_v4u{0u, 0u, 0u, 0u};
-    uint32_t slot = 0;
-    if (wave < n_chunks) request(wave, 0);
-    for (uint32_t c = wave; c < n_chunks; c += n_waves) {
-        // the next chunk (or this one again past the end: the count of loads in flight stays 16)
-        const uint32_t nx = c + n_waves < n_chunks ? c + n_waves : c;
-        request(nx, slot ^ 1u);
-        __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): the older eight have landed
-        acc ^= mine[slot * 512 + lane];
-        slot ^= 1u;
-    }
-    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0): nothing may land in LDS after the wave has gone
-    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u) sink[0] = 1u;
-}
-
 MoveGeom move_geom(const bkv_pool* p) {
     return MoveGeom{p->g.n_kv, p->g.hd, p->g.page_cells, p->desc.max_pages_per_seq};
 }
@@ -897,34 +817,6 @@ hipError_t launch_fill(void* dst, uint64_t bytes, uint32_t word, hipStream_t str
     uint64_t blocks = (n_vec + kBlock - 1) / kBlock;
     if (blocks > 16384) blocks = 16384;
     fill_kernel<<<(unsigned)blocks, kBlock, 0, stream>>>((uint4*)dst, n_vec, word);
-    return hipGetLastError();
-}
-
-hipError_t launch_copy_probe(void* dst, const void* src, uint64_t bytes, hipStream_t stream) {
-    const uint64_t n_vec = bytes / 16;
-    if (n_vec == 0) return hipSuccess;
-    uint64_t blocks = (n_vec + 4 * kBlock - 1) / (4 * kBlock);
-    if (blocks > 8192) blocks = 8192;
-    copy_probe_kernel<<<(unsigned)blocks, kBlock, 0, stream>>>((uint4*)dst, (const uint4*)src, n_vec);
-    return hipGetLastError();
-}
-
-hipError_t launch_read_probe(const void* src, uint64_t bytes, int32_t mode, void* sink, int32_t n_cu,
-                             hipStream_t stream) {
-    const uint32_t n_chunks = (uint32_t)(bytes / 8192);
-    if (n_chunks == 0) return hipSuccess;
-    if (mode == 2) {
-        // the decode kernels' launch shape: two 4-wave work-groups per compute unit, all resident
-        uint32_t blocks = (uint32_t)(n_cu > 0 ? n_cu : 256) * 2u;
-        if (blocks * (kBlock / 64) > n_chunks) blocks = (n_chunks + kBlock / 64 - 1) / (kBlock / 64);
-        read_probe_lds_kernel<<<blocks, kBlock, 0, stream>>>((const probe_v4u*)src, n_chunks, 0x9e3779b1u, (uint32_t*)sink);
-        return hipGetLastError();
-    }
-    // two resident generations of 4-wave work-groups at the decode kernels' occupancy
-    uint32_t blocks = (uint32_t)(n_cu > 0 ? n_cu : 256) * 4u;
-    if (blocks * (kBlock / 64) > n_chunks) blocks = (n_chunks + kBlock / 64 - 1) / (kBlock / 64);
-    read_probe_kernel<<<blocks, kBlock, 0, stream>>>((const probe_v4u*)src, n_chunks, mode ? 0x9e3779b1u : 1u,
-                                                     (uint32_t*)sink);
     return hipGetLastError();
 }
 

@@ -27,6 +27,7 @@
 #include <vector>
 
 #include "../../include/breccia_kv.h"
+#include "../../include/breccia_kv_bench.h"  // device allocation for the workspace (the reference: its Vulkan context)
 
 namespace breccia {
 namespace qsa {

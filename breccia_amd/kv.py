@@ -33,6 +33,10 @@ class Stream:
     def sync(self) -> None:
         check(lib.bkv_stream_sync(self.handle))
 
+    def wait(self, timeout_ms: int) -> None:
+        """The library's bounded wait (bkv_stream_wait): BkvError with ERR_TIMEOUT past the deadline."""
+        check(lib.bkv_stream_wait(self.handle, timeout_ms))
+
     def close(self) -> None:
         if self.handle:
             check(lib.bkv_stream_destroy(self.handle))
@@ -84,6 +88,17 @@ def attn_plan(n_cu: int, n_kv_head: int, n_q_head: int, pos, sel_groups: int = 0
                             splits.ctypes.data_as(C.POINTER(C.c_int32)), pps.ctypes.data_as(C.POINTER(C.c_int32)),
                             C.byref(total)))
     return splits[:pos.size], pps[:pos.size], int(total.value)
+
+
+def wait_options(timeout_ms: int | None = None, poll_us: int | None = None):
+    """Set (where given) and return the process-wide (deadline in ms, spin window in us) of the library's waits."""
+    t, p = C.c_int64(), C.c_int64()
+    check(lib.bkv_wait_options_get(C.byref(t), C.byref(p)))
+    if timeout_ms is not None or poll_us is not None:
+        check(lib.bkv_wait_options(t.value if timeout_ms is None else timeout_ms,
+                                   p.value if poll_us is None else poll_us))
+        check(lib.bkv_wait_options_get(C.byref(t), C.byref(p)))
+    return int(t.value), int(p.value)
 
 
 def device_sync() -> None:
@@ -477,6 +492,9 @@ class Pool:
 
     def swap_wait(self) -> None:
         check(lib.bkv_swap_wait(self.handle))
+
+    def swap_wait_for(self, timeout_ms: int) -> None:
+        check(lib.bkv_swap_wait_for(self.handle, timeout_ms))
 
     def swap_fence(self, stream=None) -> None:
         check(lib.bkv_swap_fence(self.handle, _sh(stream)))

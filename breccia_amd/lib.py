@@ -10,10 +10,12 @@ import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libbreccia_kv.so")
+BENCH_LIB_PATH = os.path.join(HERE, "libbreccia_kv_bench.so")
 HEADER_PATH = os.path.join(HERE, "..", "include", "breccia_kv.h")
+BENCH_HEADER_PATH = os.path.join(HERE, "..", "include", "breccia_kv_bench.h")
 
-OK, ERR_INVALID, ERR_RANGE, ERR_NO_PAGES, ERR_STATE, ERR_NO_DEVICE, ERR_HIP, ERR_NOMEM = range(8)
-STATUS_NAMES = ["OK", "INVALID", "RANGE", "NO_PAGES", "STATE", "NO_DEVICE", "HIP", "NOMEM"]
+OK, ERR_INVALID, ERR_RANGE, ERR_NO_PAGES, ERR_STATE, ERR_NO_DEVICE, ERR_HIP, ERR_NOMEM, ERR_TIMEOUT = range(9)
+STATUS_NAMES = ["OK", "INVALID", "RANGE", "NO_PAGES", "STATE", "NO_DEVICE", "HIP", "NOMEM", "TIMEOUT"]
 LAYOUT_F16, LAYOUT_Q8V, LAYOUT_I8H = 0, 1, 2
 POOL_HOST_ONLY = 1
 MAX_BATCH = 64
@@ -40,15 +42,16 @@ class PagePair(C.Structure):
     _fields_ = [("src", C.c_int32), ("dst", C.c_int32)]
 
 
-def _load() -> C.CDLL:
-    if not os.path.exists(LIB_PATH):
+def _load(path: str) -> C.CDLL:
+    if not os.path.exists(path):
         raise ImportError(
-            "libbreccia_kv.so is not built (%s). Build it with `python -m breccia_amd.build` "
-            "(needs hipcc); there is no CPU fallback." % LIB_PATH)
-    return C.CDLL(LIB_PATH)
+            "%s is not built (%s). Build it with `python -m breccia_amd.build` "
+            "(needs hipcc); there is no CPU fallback." % (os.path.basename(path), path))
+    return C.CDLL(path)
 
 
-lib = _load()
+_product = _load(LIB_PATH)        # the paged-KV library: include/breccia_kv.h
+_bench = _load(BENCH_LIB_PATH)    # device plumbing and probes for tests and bench: include/breccia_kv_bench.h
 
 _vp, _i32, _i64, _u64, _f32 = C.c_void_p, C.c_int32, C.c_int64, C.c_uint64, C.c_float
 _pi32, _pi64 = C.POINTER(C.c_int32), C.POINTER(C.c_int64)
@@ -123,10 +126,18 @@ _SIGNATURES = {
     "bkv_swap_out": (C.c_int, [_vp, _pi32, _i32, _vp, _vp]),
     "bkv_swap_in": (C.c_int, [_vp, _pi32, _i32, _vp, _vp]),
     "bkv_swap_wait": (C.c_int, [_vp]),
+    "bkv_swap_wait_for": (C.c_int, [_vp, _i64]),
+    "bkv_stream_wait": (C.c_int, [_vp, _i64]),
+    "bkv_wait_options": (C.c_int, [_i64, _i64]),
+    "bkv_wait_options_get": (C.c_int, [_pi64, _pi64]),
     "bkv_swap_fence": (C.c_int, [_vp, _vp]),
     "bkv_seq_evict": (C.c_int, [_vp, _i32, _i32, _i32, _vp, _vp]),
     "bkv_seq_restore": (C.c_int, [_vp, _i32, _i32, _i32, _vp, _vp]),
     "bkv_gather": (C.c_int, [_vp, _i32, _i32, _i64, _i64, _vp, _vp, _vp]),
+}
+
+_BENCH_SIGNATURES = {
+    "bkv_bench_last_error": (C.c_char_p, []),
     "bkv_dev_alloc": (C.c_int, [_u64, C.POINTER(_vp)]),
     "bkv_dev_free": (C.c_int, [_vp]),
     "bkv_memcpy_h2d": (C.c_int, [_vp, _vp, _u64, _vp]),
@@ -149,16 +160,42 @@ _SIGNATURES = {
     "bkv_read_probe": (C.c_int, [_vp, _u64, _i32, _vp, _vp]),
 }
 
+_bench_error = None   # message of the last failed call into the bench library, until check() takes it
+
+
+def _bench_call(fn):
+    def call(*args):
+        global _bench_error
+        status = fn(*args)
+        if status != OK:
+            _bench_error = _bench.bkv_bench_last_error().decode("utf-8", "replace")
+        return status
+    return call
+
+
+class _Both:
+    """Every entry point of the two libraries under one name space (the names do not overlap)."""
+
+
+lib = _Both()
 for _name, (_res, _args) in _SIGNATURES.items():
-    _fn = getattr(lib, _name)
+    _fn = getattr(_product, _name)
     _fn.restype = _res
     _fn.argtypes = _args
+    setattr(lib, _name, _fn)
+for _name, (_res, _args) in _BENCH_SIGNATURES.items():
+    _fn = getattr(_bench, _name)
+    _fn.restype = _res
+    _fn.argtypes = _args
+    setattr(lib, _name, _bench_call(_fn) if _res is C.c_int else _fn)
 
 
 def last_error() -> str:
-    return lib.bkv_last_error().decode("utf-8", "replace")
+    return _product.bkv_last_error().decode("utf-8", "replace")
 
 
 def check(status: int) -> None:
+    global _bench_error
     if status != OK:
-        raise BkvError(status, last_error())
+        msg, _bench_error = (_bench_error, None) if _bench_error is not None else (last_error(), None)
+        raise BkvError(status, msg)

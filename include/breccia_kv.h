@@ -11,8 +11,11 @@
  * reference recording into a device's open batch, crates/breccia-kernels/src/
  * ops/mod.rs:205-222): results are visible to later work on the same stream.
  * `stream` is a hipStream_t passed as void* (NULL = the default stream).
- * One pool may be driven from several streams (by one host thread at a time: the
- * pool itself is not thread-safe).  What the pool owns and every call shares --
+ * One pool may be driven from several streams, by one host thread at a time: a pool is
+ * not thread-safe and takes no lock of its own (the reference guards its queue with a
+ * mutex, crates/breccia-vk/src/ctx.rs:565; here that lock belongs to the owner of the pool --
+ * a Rust wrapper is Send and not Sync).  Different pools may be used from different threads;
+ * bkv_last_error and the wait options are the only process-wide state.  What the pool owns and every call shares --
  * the argument ring, the block tables, the split-K and score workspaces, the swap
  * staging -- it orders across streams by itself with events; the order between the
  * caller's own data (an append before the attention that reads its rows, on another
@@ -39,7 +42,9 @@ typedef enum bkv_status {
     BKV_ERR_STATE = 4,      /* refcount / ownership / residency rule violated */
     BKV_ERR_NO_DEVICE = 5,  /* pool was created host-only, or HIP is unusable */
     BKV_ERR_HIP = 6,        /* a HIP runtime call failed (message names it) */
-    BKV_ERR_NOMEM = 7       /* host or pinned-host allocation failed */
+    BKV_ERR_NOMEM = 7,      /* host or pinned-host allocation failed */
+    BKV_ERR_TIMEOUT = 8     /* a bounded host wait ran out (message names what it waited for);
+                               the work is still enqueued, nothing was cancelled */
 } bkv_status;
 
 /* How K and V rows are stored.  qsa/mod.rs:242-254 (VLayout). */
@@ -466,8 +471,28 @@ bkv_status bkv_swap_out(bkv_pool *pool, const int32_t *pages, int32_t n, void *p
                         void *stream);
 bkv_status bkv_swap_in(bkv_pool *pool, const int32_t *pages, int32_t n, const void *pinned_host,
                        void *stream);
-bkv_status bkv_swap_wait(bkv_pool *pool);
+bkv_status bkv_swap_wait(bkv_pool *pool); /* bkv_swap_wait_for with the default deadline */
 bkv_status bkv_swap_fence(bkv_pool *pool, void *stream);
+
+/* ---- bounded host waits ---------------------------------------------------------
+ * The reference never waits on its device without a deadline: crates/breccia-vk/src/ctx.rs:
+ * 1545-1553 (WAIT_TIMEOUT_NS = 10 s, then a diagnostic instead of a hang).  The same here: every
+ * host-side wait of the library for a stream or an event -- bkv_swap_wait, the transfers between
+ * the prefix tiers, a free argument-ring slot, bkv_step_plan_state, bkv_timing_read -- polls the
+ * HIP query call up to a deadline and then returns BKV_ERR_TIMEOUT with what it was waiting for.
+ * Nothing is aborted or cancelled: the work stays enqueued and a later wait can succeed.
+ * bkv_stream_wait is that wait for a caller's stream (timeout_ms < 0: no deadline; 0: a query).
+ * bkv_wait_options sets, for the process, the deadline of the library's internal waits
+ * (default 10000 ms; negative = none) and how long a wait spins on the query before it starts
+ * napping 50 us between queries (default 4000 us: a thread asleep in hipStreamSynchronize is
+ * woken tens of microseconds late, which a decode loop that waits per token would pay every
+ * time; 0 = never spin).  The exceptions are the device-wide synchronisations HIP offers no
+ * query for: pool destruction and reset, growing the selection workspace, and the one before
+ * prefix pages leave the device. */
+bkv_status bkv_stream_wait(void *stream, int64_t timeout_ms);
+bkv_status bkv_swap_wait_for(bkv_pool *pool, int64_t timeout_ms);
+bkv_status bkv_wait_options(int64_t timeout_ms, int64_t poll_us);
+bkv_status bkv_wait_options_get(int64_t *timeout_ms_out, int64_t *poll_us_out);
 /* Allocator-aware eviction of logical pages [lp0, lp0+n) of a sequence: each must be
  * complete and held only by this sequence; bytes go to pinned_host, the physical
  * pages return to the free list and the table entries become -1.  Restore allocates
@@ -518,43 +543,6 @@ typedef enum bkv_stage {
 bkv_status bkv_timing_enable(bkv_pool *pool, int on);
 bkv_status bkv_timing_reset(bkv_pool *pool);
 bkv_status bkv_timing_read(bkv_pool *pool, int stage, uint64_t *launches, double *total_ms);
-
-/* ---- device plumbing for hosts without their own HIP bindings ---------------- */
-bkv_status bkv_dev_alloc(uint64_t bytes, void **dev_out);
-bkv_status bkv_dev_free(void *dev);
-bkv_status bkv_memcpy_h2d(void *dev, const void *host, uint64_t bytes, void *stream);
-bkv_status bkv_memcpy_d2h(void *host, const void *dev, uint64_t bytes, void *stream);
-bkv_status bkv_stream_create(void **stream_out);
-/* Stream capture into a graph (hipStreamBeginCapture / EndCapture + hipGraphInstantiate, thread-local
- * capture mode) and its replay; `stream` must not be NULL. */
-bkv_status bkv_graph_begin_capture(void *stream);
-bkv_status bkv_graph_end_capture(void *stream, void **graph_exec_out);
-bkv_status bkv_graph_launch(void *graph_exec, void *stream);
-bkv_status bkv_graph_destroy(void *graph_exec);
-bkv_status bkv_stream_destroy(void *stream);
-bkv_status bkv_stream_sync(void *stream);
-bkv_status bkv_device_sync(void);
-bkv_status bkv_event_create(void **event_out);
-bkv_status bkv_event_destroy(void *event);
-bkv_status bkv_event_record(void *event, void *stream);
-bkv_status bkv_event_sync(void *event);
-bkv_status bkv_event_elapsed_ms(void *start, void *stop, float *ms_out);
-/* name (<= 255 chars), compute units, total device memory */
-bkv_status bkv_device_info(char *name_out, int32_t name_cap, int32_t *cu_out,
-                           uint64_t *mem_bytes_out);
-/* Reference bandwidth probe: a plain 16-byte-vector device copy of `bytes` bytes
- * (used to scale profiler byte counters and to report the copy ceiling). */
-bkv_status bkv_copy_probe(void *dst_dev, const void *src_dev, uint64_t bytes, void *stream);
-/* Read-only bandwidth probe: reads `bytes` (a power-of-two number of 8 KiB chunks -- the size of
- * one (page, kv head) run of an f16 pool) once, 8 KiB per wave at a time, in address order
- * (scattered = 0), in a fixed pseudo-random order of chunks (1), as the attention kernels see a
- * shuffled pool, or in that order with every chunk fetched by global->LDS loads instead of loads
- * into registers (2: the slower of the two ways a row can reach LDS on this chip, kept so that the
- * comparison behind the quantised kernels' data path can be repeated); nothing is written
- * except, never in practice, one word at sink_dev.  The rate it reaches is the ceiling a
- * read-only kernel can be held against on a given box. */
-bkv_status bkv_read_probe(const void *src_dev, uint64_t bytes, int32_t scattered, void *sink_dev,
-                          void *stream);
 
 #ifdef __cplusplus
 }

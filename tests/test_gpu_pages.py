@@ -245,3 +245,47 @@ def test_table_updates_flushed_on_one_stream_are_seen_on_another():
         device_sync()
         for x in (big_rows, rd, qd, od):
             x.free()
+
+
+def test_bounded_waits_time_out_and_the_work_still_completes():
+    """crates/breccia-vk/src/ctx.rs:1545-1553: the reference's device waits have a deadline and report
+    instead of hanging.  A stream with a queue of bulk appends behind it: a wait with a deadline of 0 ms
+    is a query and returns TIMEOUT (with what it waited for), nothing is cancelled, a wait with a real
+    deadline then succeeds and the pool holds every appended byte.  The same on the pool's side stream
+    with page transfers in flight."""
+    from breccia_amd.kv import DeviceBuffer
+
+    rng = np.random.Generator(np.random.PCG64(77))
+    T = 8192
+    with Twin(n_pages=T // 16 + 600, max_seqs=4, max_pages_per_seq=T // 16 + 8) as tw:
+        s = tw.pool.seq_create()
+        tw.pool.seq_reserve(s, T)
+        k = rng.standard_normal((T, 2, 256)).astype(np.float32)
+        v = rng.standard_normal((T, 2, 256)).astype(np.float32)
+        kd, vd = DeviceBuffer.from_numpy(k), DeviceBuffer.from_numpy(v)
+        st = Stream()
+        st.wait(0)                                              # an idle stream: a query succeeds
+        for _ in range(400):                                    # some 10 ms of device work, enqueued in less
+            tw.pool.append(0, [s], [0], [T], kd, vd, st)
+        with pytest.raises(BkvError) as ei:
+            st.wait(0)
+        assert ei.value.status == L.ERR_TIMEOUT and "caller stream" in ei.value.message
+        assert "nothing was cancelled" in ei.value.message
+        st.wait(10000)
+        assert tw.images[0].append(tw.pool.block_table(s), 0, k, v) == 0
+        tw.assert_pools_equal()
+        # the side stream: 512 pages out to pinned host memory
+        pages = tw.pool.block_table(s)[:512].astype(np.int32)
+        host = tw.pool.host_alloc(512 * tw.pool.swap_page_bytes())
+        for _ in range(200):                                    # the transfers queue up behind these
+            tw.pool.append(0, [s], [0], [T], kd, vd, st)
+        tw.pool.swap_out(pages, host, st)
+        with pytest.raises(BkvError) as ei:
+            tw.pool.swap_wait_for(0)
+        assert ei.value.status == L.ERR_TIMEOUT and "side stream" in ei.value.message
+        tw.pool.swap_wait()
+        hv = host.view().reshape(512, 2, 16384)
+        assert np.array_equal(hv[511, 0], tw.images[0].k.reshape(-1, 16384)[pages[511]])
+        host.free()
+        kd.free()
+        vd.free()

@@ -114,6 +114,65 @@ def test_captured_token_replayed_32_times_equals_eager_steps(layout):
     st.close()
 
 
+def test_a_plan_made_on_one_stream_and_driven_from_others_needs_no_host_synchronisation():
+    # The plan's descriptor is uploaded on the stream of its creation, behind whatever that stream
+    # still has to do (here: bulk appends and the scatter of freshly reserved pages' table entries);
+    # decode arrives on a second stream and advance on a third, with no host synchronisation in
+    # between.  The library orders them (events, on the device): outputs and pool bytes equal the eager
+    # steps' of a twin pool, bit for bit.
+    n_q, lens, n_tok = 16, [333, 47], 5
+    rng = np.random.Generator(np.random.PCG64(9400))
+    a, b, c = Stream(), Stream(), Stream()
+    with Twin(n_pages=2200, max_seqs=8, max_pages_per_seq=1100) as eager, \
+            Twin(n_pages=2200, max_seqs=8, max_pages_per_seq=1100) as planned:
+        rng_a, rng_b = np.random.Generator(np.random.PCG64(5)), np.random.Generator(np.random.PCG64(5))
+        order = rng.permutation(2200).astype(np.int32)
+        seqs = grow(eager, lens, rng_a, order)
+        assert grow(planned, lens, rng_b, order) == seqs
+        kn = rng.standard_normal((n_tok, 2, 2, 256)).astype(np.float32)
+        vn = rng.standard_normal((n_tok, 2, 2, 256)).astype(np.float32)
+        q = rng.standard_normal((n_tok, 2, n_q, 256)).astype(np.float32)
+        kd, vd, qd = DeviceBuffer.from_numpy(kn), DeviceBuffer.from_numpy(vn), DeviceBuffer.from_numpy(q)
+        od = DeviceBuffer(q.nbytes)
+        step_kv, step_q = 2 * 2 * 256 * 4, 2 * n_q * 256 * 4
+        want = np.zeros_like(q)
+        for t in range(n_tok):
+            for s, n in zip(seqs, lens):
+                eager.pool.seq_reserve(s, n + t + 1)
+            eager.pool.decode_step(0, seqs, [n + t for n in lens], kd.at(t * step_kv), vd.at(t * step_kv), n_q,
+                                   qd.at(t * step_q), od.at(t * step_q), 1.0 / 16.0)
+        device_sync()
+        want = od.download(np.float32).reshape(q.shape)
+        od.upload(np.zeros_like(q))
+        # the planned pool: a long tail of work on stream a (a third sequence filled with 16384 tokens, in
+        # four calls), the step's pages reserved (their table entries pending), then the plan on stream a
+        big = planned.pool.seq_create()
+        planned.pool.seq_reserve(big, 16384)
+        rows = DeviceBuffer.from_numpy(rng.standard_normal((4096, 2, 256)).astype(np.float32))
+        for s, n in zip(seqs, lens):
+            planned.pool.seq_reserve(s, n + n_tok + 1)
+        for i in range(4):
+            planned.pool.append(0, [big], [4096 * i], [4096], rows, rows, a)
+        plan = StepPlan(planned.pool, seqs, lens, n_tok + 1, n_q, stream=a)
+        for t in range(n_tok):
+            plan.decode(0, kd.at(t * step_kv), vd.at(t * step_kv), qd.at(t * step_q), od.at(t * step_q), 1.0 / 16.0,
+                        stream=b)
+            plan.advance(c)
+        pos, steps, status = plan.state(b)
+        assert steps == n_tok and status == 0 and pos.tolist() == [n + n_tok for n in lens]
+        got = od.download(np.float32).reshape(q.shape)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+        device_sync()
+        planned.pool.seq_free(big)
+        for s in seqs:
+            ge, gp = eager.pool.gather(0, s, 0, lens[seqs.index(s)] + n_tok), planned.pool.gather(0, s, 0, lens[seqs.index(s)] + n_tok)
+            assert np.array_equal(ge[0].view(np.uint32), gp[0].view(np.uint32))
+            assert np.array_equal(ge[1].view(np.uint32), gp[1].view(np.uint32))
+        plan.destroy()
+        for x in (kd, vd, qd, od, rows):
+            x.free()
+
+
 def test_plan_creation_checks_the_whole_horizon():
     with Twin(n_pages=32, max_seqs=4) as tw:
         a, b = tw.pool.seq_create(), tw.pool.seq_create()

@@ -12,10 +12,11 @@ from breccia_amd import kv, lib as L
 from breccia_amd.kv import BkvError, Pool
 
 HEADER = os.path.join(os.path.dirname(__file__), "..", "include", "breccia_kv.h")
+BENCH_HEADER = os.path.join(os.path.dirname(__file__), "..", "include", "breccia_kv_bench.h")
 
 
-def declared_functions():
-    text = open(HEADER).read()
+def declared_functions(header=HEADER):
+    text = open(header).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(bkv_[a-z0-9_]+)\s*\(", text)))
 
@@ -24,9 +25,31 @@ def test_library_exports_every_declared_symbol():
     names = declared_functions()
     assert len(names) >= 45
     for name in names:
-        assert hasattr(L.lib, name), "libbreccia_kv.so does not export " + name
+        assert hasattr(L._product, name), "libbreccia_kv.so does not export " + name
     # and the Python binding covers each of them
     assert sorted(L._SIGNATURES) == names
+
+
+def test_the_product_library_carries_no_probe_or_plumbing_entry_point():
+    # device allocation, copies, streams, events, graphs and the bandwidth probes live in
+    # libbreccia_kv_bench.so (include/breccia_kv_bench.h): what an integration links has the path only
+    bench = declared_functions(BENCH_HEADER)
+    assert "bkv_copy_probe" in bench and "bkv_dev_alloc" in bench and "bkv_graph_launch" in bench
+    assert sorted(L._BENCH_SIGNATURES) == bench
+    for name in bench:
+        assert hasattr(L._bench, name), "libbreccia_kv_bench.so does not export " + name
+        assert not hasattr(L._product, name), "libbreccia_kv.so still exports " + name
+    assert not set(bench) & set(declared_functions())
+
+
+def test_wait_options_round_trip_and_reject_a_zero_deadline():
+    # crates/breccia-vk/src/ctx.rs:1545-1553: the reference's waits have a 10 s deadline; so have these
+    assert kv.wait_options() == (10000, 4000)
+    assert kv.wait_options(timeout_ms=250, poll_us=0) == (250, 0)
+    assert kv.wait_options(timeout_ms=-1) == (-1, 0)
+    expect(L.ERR_INVALID, kv.wait_options, 0, 100)
+    expect(L.ERR_INVALID, kv.wait_options, 100, -5)
+    assert kv.wait_options(10000, 4000) == (10000, 4000)
 
 
 def test_rust_binding_text_lists_every_declaration_with_its_argument_count():
