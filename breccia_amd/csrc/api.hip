@@ -234,6 +234,9 @@ bool timer_dispatch_events(bkv_pool* p, int stage, hipEvent_t* start, hipEvent_t
         if (*stop) (void)hipEventDestroy(*stop);
         return false;
     }
+    // every timed launch comes through here: a caller that never reads the timer (bkv_timing_read)
+    // must not grow the list of open event pairs without bound
+    if (t.open.size() >= 8192) (void)timer_collect(p);
     t.open.push_back(StageTimer::Pair{stage, *start, *stop});
     return true;
 }
@@ -812,7 +815,6 @@ static bkv_status append_rows(bkv_pool* p, int32_t layer, int32_t n_seqs, const 
     st = flush_tables(p, S(stream));
     if (st != BKV_OK) return st;
     BKV_HIP(launch_append(p, layer, b, max_tok, k_dev, v_dev, src_is_f16, S(stream)));
-    if (p->timer.open.size() > 8192) return timer_collect(p);
     return BKV_OK;
 }
 
@@ -855,7 +857,6 @@ bkv_status bkv_append_kprep(bkv_pool* p, int32_t layer, int32_t n_seqs, const in
     if (st != BKV_OK) return st;
     BKV_HIP(launch_append_kprep(p, layer, b, max_tok, k_dev, v_dev, k_gamma_dev, eps,
                                 rope_table_dev, n_rot, max_pos, positions_dev, S(stream)));
-    if (p->timer.open.size() > 8192) return timer_collect(p);
     return BKV_OK;
 }
 
@@ -964,6 +965,16 @@ static bkv_status decode_attn_common(bkv_pool* p, int32_t layer, int32_t n, cons
         if (!attn_static_scratch(p->device, &a.ws_o, &a.ws_ml))
             return fail(BKV_ERR_STATE, "decode_attn_static: the static scratch of this device was not set up");
         a.timed = false;
+        // A stream under capture cannot record the usual way block-table changes travel (it may wait on
+        // the host for a free ring slot): as for step plans, they are made before the capture.
+        if (!p->alloc->pending().empty() || p->tiers.pending) {
+            hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+            if (stream && hipStreamIsCapturing(S(stream), &cs) == hipSuccess && cs != hipStreamCaptureStatusNone)
+                return fail(BKV_ERR_STATE, "decode_attn_static: block-table changes are pending while the stream is "
+                                           "being captured; make allocator calls, then any eager call, before the "
+                                           "capture");
+            (void)hipGetLastError();
+        }
     }
     st = flush_tables(p, S(stream));
     if (st != BKV_OK) return st;
@@ -991,7 +1002,6 @@ static bkv_status decode_attn_common(bkv_pool* p, int32_t layer, int32_t n, cons
         if (st != BKV_OK) return st;
     }
     BKV_HIP(launch_decode_attn(p, layer, b, a, S(stream)));
-    if (p->timer.open.size() > 8192) return timer_collect(p);
     return BKV_OK;
 }
 
@@ -1335,7 +1345,6 @@ bkv_status bkv_prefill_attn(bkv_pool* p, int32_t layer, int32_t n_seqs, const in
     a.scale = scale;
     a.out = out_dev;
     BKV_HIP(launch_prefill_attn(p, layer, b, a, S(stream)));
-    if (p->timer.open.size() > 8192) return timer_collect(p);
     return BKV_OK;
 }
 

@@ -255,6 +255,13 @@ bkv_status bkv_device_info(char* name_out, int32_t name_cap, int32_t* cu_out,
     if (mem_bytes_out) *mem_bytes_out = prop.totalGlobalMem;
     return BKV_OK;
 }
+bkv_status bkv_device_mem_info(uint64_t* free_out, uint64_t* total_out) {
+    size_t f = 0, t = 0;
+    BKV_HIP(hipMemGetInfo(&f, &t));
+    if (free_out) *free_out = f;
+    if (total_out) *total_out = t;
+    return BKV_OK;
+}
 bkv_status bkv_copy_probe(void* dst_dev, const void* src_dev, uint64_t bytes, void* stream) {
     if (!dst_dev || !src_dev || !aligned16(dst_dev) || !aligned16(src_dev) || bytes % 16)
         return fail(BKV_ERR_INVALID, "copy_probe: pointers and size must be 16-byte multiples");

@@ -10,6 +10,8 @@
 // head, page range); a wave owns whole pages (16 cells); the four waves' running (m, l, O) are
 // folded in LDS and written as one partial per work-group; the merge kernel combines the page
 // ranges of a head and applies sigmoid(gate).
+#include <atomic>
+
 #include "decode_attn_common.hpp"
 
 namespace bkv {
@@ -189,25 +191,38 @@ struct AttnStaticScratch {
 static __device__ __align__(256) unsigned char scratch[sizeof(AttnStaticScratch)];
 
 constexpr int kMaxDevices = 64;
-static void* g_scratch_ptr[kMaxDevices] = {};
+// One address per device, looked up once; pools may be created from several threads at once, so the
+// table is atomic (two threads that race on one device store the same address).
+static std::atomic<void*> g_scratch_ptr[kMaxDevices];
 
+// Makes `device` current for the lookup (every GPU holds its own copy of the array at its own
+// address) and restores the caller's device afterwards.
 hipError_t attn_static_scratch_init(int device) {
     if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
-    if (g_scratch_ptr[device]) return hipSuccess;
+    if (g_scratch_ptr[device].load(std::memory_order_acquire)) return hipSuccess;
     int current = -1;
     hipError_t e = hipGetDevice(&current);
     if (e != hipSuccess) return e;
-    if (current != device) return hipErrorInvalidDevice;
+    if (current != device) {
+        e = hipSetDevice(device);
+        if (e != hipSuccess) return e;
+    }
     void* ptr = nullptr;
     e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (current != device) {
+        const hipError_t back = hipSetDevice(current);
+        if (e == hipSuccess) e = back;
+    }
     if (e != hipSuccess) return e;
-    g_scratch_ptr[device] = ptr;
+    g_scratch_ptr[device].store(ptr, std::memory_order_release);
     return hipSuccess;
 }
 
 bool attn_static_scratch(int device, float** o, float** ml) {
-    if (device < 0 || device >= kMaxDevices || !g_scratch_ptr[device]) return false;
-    AttnStaticScratch* s = static_cast<AttnStaticScratch*>(g_scratch_ptr[device]);
+    if (device < 0 || device >= kMaxDevices) return false;
+    void* ptr = g_scratch_ptr[device].load(std::memory_order_acquire);
+    if (!ptr) return false;
+    AttnStaticScratch* s = static_cast<AttnStaticScratch*>(ptr);
     *o = s->o;
     *ml = s->ml;
     return true;

@@ -113,6 +113,12 @@ def device_info():
     return name.value.decode(), int(cu.value), int(mem.value)
 
 
+def device_mem_free() -> int:
+    f = C.c_uint64()
+    check(lib.bkv_device_mem_info(C.byref(f), None))
+    return int(f.value)
+
+
 class DeviceBuffer:
     """A hipMalloc'd region with numpy upload/download."""
 

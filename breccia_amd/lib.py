@@ -156,6 +156,7 @@ _BENCH_SIGNATURES = {
     "bkv_event_sync": (C.c_int, [_vp]),
     "bkv_event_elapsed_ms": (C.c_int, [_vp, _vp, C.POINTER(C.c_float)]),
     "bkv_device_info": (C.c_int, [C.c_char_p, _i32, _pi32, C.POINTER(_u64)]),
+    "bkv_device_mem_info": (C.c_int, [C.POINTER(_u64), C.POINTER(_u64)]),
     "bkv_copy_probe": (C.c_int, [_vp, _vp, _u64, _vp]),
     "bkv_read_probe": (C.c_int, [_vp, _u64, _i32, _vp, _vp]),
 }

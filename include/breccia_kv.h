@@ -305,7 +305,10 @@ bkv_status bkv_decode_attn(bkv_pool *pool, int32_t layer, int32_t n, const int32
  * Every pool and every call on one GPU shares that GPU's array: calls that overlap on one GPU
  * (different streams, different pools) race; calls on one stream are ordered by the stream.
  * Nothing in the array has to start at zero.  Block-table changes still pending from allocator
- * calls are uploaded first, as in every other call (host heap and the pinned argument ring only). */
+ * calls are uploaded first, as in every other call (host heap and the pinned argument ring only)
+ * -- except on a stream that is being captured, which cannot record that upload: there the call
+ * returns BKV_ERR_STATE; make the allocator calls and any eager call before the capture (the rule
+ * of step plans). */
 #define BKV_STATIC_WGS 1024
 bkv_status bkv_decode_attn_static(bkv_pool *pool, int32_t layer, int32_t n, const int32_t *seqs,
                                   const int64_t *pos, int32_t n_q_head, const float *q_dev,
@@ -373,8 +376,12 @@ bkv_status bkv_decode_step(bkv_pool *pool, int32_t layer, int32_t n, const int32
  * returns BKV_ERR_STATE when they are no longer reserved, resident and unshared, but a replayed
  * graph makes no such call.  Allocator calls for OTHER sequences are fine but must be followed by an
  * eager call on the pool before a capture begins, since their block-table changes cannot be
- * recorded.  Destroy a pool's plans before the pool (bkv_pool_destroy returns BKV_ERR_STATE while
- * one is alive).  All three layouts. */
+ * recorded.  Streams: the calls of a plan may come on any stream; a call that arrives on another
+ * stream than the plan's previous one (creation included) is ordered behind it by the library, with
+ * an event recorded there at that moment, and behind the last block-table scatter wherever that
+ * ran.  A replayed graph holds none of these host-made orderings: replay on the stream the capture
+ * was taken from, or order the streams yourself.  Destroy a pool's plans before the pool
+ * (bkv_pool_destroy returns BKV_ERR_STATE while one is alive).  All three layouts. */
 typedef struct bkv_step_plan bkv_step_plan;
 bkv_status bkv_step_plan_create(bkv_pool *pool, int32_t n, const int32_t *seqs, const int64_t *pos,
                                 int32_t horizon, int32_t n_q_head, void *stream, bkv_step_plan **out);

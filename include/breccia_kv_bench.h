@@ -44,6 +44,8 @@ bkv_status bkv_event_elapsed_ms(void *start, void *stop, float *ms_out);
 /* name (<= 255 chars), compute units, total device memory */
 bkv_status bkv_device_info(char *name_out, int32_t name_cap, int32_t *cu_out,
                            uint64_t *mem_bytes_out);
+/* free and total device memory (hipMemGetInfo) */
+bkv_status bkv_device_mem_info(uint64_t *free_out, uint64_t *total_out);
 /* Reference bandwidth probe: a plain 16-byte-vector device copy of `bytes` bytes
  * (used to scale profiler byte counters and to report the copy ceiling). */
 bkv_status bkv_copy_probe(void *dst_dev, const void *src_dev, uint64_t bytes, void *stream);

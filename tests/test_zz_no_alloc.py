@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 from breccia_amd import lib as L
-from breccia_amd.kv import BkvError, DeviceBuffer, device_sync
+from breccia_amd.kv import BkvError, DeviceBuffer, Graph, Stream, device_mem_free, device_sync
 from gpu_common import REF_BAR_MAX_REL, Twin, check_attn
 
 pytestmark = pytest.mark.gpu
@@ -86,3 +86,66 @@ def test_static_scratch_call_rejects_batches_beyond_the_array():
         device_sync()
         qd.free()
         od.free()
+
+
+def test_static_scratch_call_allocates_nothing_and_replays_from_a_graph():
+    # What the entry point is for: callers that cannot allocate.  Free device memory is the same
+    # before and after a run of calls (the allocating entry point's workspace was made at pool
+    # creation, so it serves as the control), and the call can be recorded into a graph: three
+    # replays, with eager work on the same pool and a synchronisation between them, each return the
+    # bits of the eager call on that replay's inputs.  Block-table changes pending at capture time
+    # are refused, as for step plans.
+    rng = np.random.Generator(np.random.PCG64(7200))
+    n_q, lens = 16, [900, 41, 2047]
+    st = Stream()
+    with Twin(n_pages=300, max_seqs=8) as tw:
+        tw.pool.set_free_order(rng.permutation(300).astype(np.int32))
+        seqs = [tw.pool.seq_create() for _ in lens]
+        for s, n in zip(seqs, lens):
+            tw.pool.seq_reserve(s, n)
+        tw.append(0, seqs, [0] * 3, [rng.standard_normal((n, 2, 256)).astype(np.float32) for n in lens],
+                  [rng.standard_normal((n, 2, 256)).astype(np.float32) for n in lens])
+        pos = [n - 1 for n in lens]
+        qd = DeviceBuffer(3 * n_q * 256 * 4)
+        o_static, o_ref = DeviceBuffer(3 * n_q * 256 * 4), DeviceBuffer(3 * n_q * 256 * 4)
+        qd.upload(rng.standard_normal((3, n_q, 256)).astype(np.float32))
+        tw.pool.decode_attn_static(0, seqs, pos, n_q, qd, o_static, 1.0 / 16.0, stream=st)
+        st.sync()
+        free0 = device_mem_free()
+        for _ in range(50):
+            tw.pool.decode_attn_static(0, seqs, pos, n_q, qd, o_static, 1.0 / 16.0, stream=st)
+        st.sync()
+        assert device_mem_free() == free0
+        # pending table changes at capture time: refused, and the capture can go on after an eager flush
+        extra = tw.pool.seq_create()
+        tw.pool.seq_reserve(extra, 20)
+        g = Graph(st)
+        with pytest.raises(BkvError) as ei:
+            tw.pool.decode_attn_static(0, seqs, pos, n_q, qd, o_static, 1.0 / 16.0, stream=st)
+        assert ei.value.status == L.ERR_STATE and "captured" in ei.value.message
+        g.end()
+        g.destroy()
+        tw.pool.decode_attn(0, seqs, pos, n_q, qd, o_ref, 1.0 / 16.0, stream=st)    # eager: flushes the tables
+        st.sync()
+        g = Graph(st)
+        tw.pool.decode_attn_static(0, seqs, pos, n_q, qd, o_static, 1.0 / 16.0, stream=st)
+        g.end()
+        free1 = None
+        for rep in range(3):
+            q = rng.standard_normal((3, n_q, 256)).astype(np.float32)
+            qd.upload(q, st)
+            tw.pool.decode_attn(0, seqs, pos, n_q, qd, o_ref, 1.0 / 16.0, stream=st)      # eager work in between
+            st.sync()
+            g.launch(st)
+            st.sync()
+            got = o_static.download(np.float32, stream=st)
+            want = o_ref.download(np.float32, stream=st)
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), rep
+            if free1 is None:
+                # instantiating a graph and launching it for the first time take device memory of the
+                # runtime's own; from then on nothing moves
+                free1 = device_mem_free()
+        assert device_mem_free() == free1
+        g.destroy()
+        for b in (qd, o_static, o_ref):
+            b.free()
