@@ -23,9 +23,13 @@
 // exact f16; q and p are f32 values split into a high and a low f16 part (two MFMAs each), so the
 // products carry ~22 significant bits and the result stays at f32-accumulate accuracy.  Pages are
 // walked two at a time: one softmax update and one barrier per pair.
-// The V operand needs four cells of one head-dim column per lane: each lane loads 16 bytes
-// (8 columns) of four rows and regroups them in registers; the 8 MFMAs that use them produce
-// columns 8i + t of the output, i = the MFMA row, t = 0..7.
+// The V operand needs, per lane, four cells of one head-dim column of either page: a column of
+// the row-major page image.  gfx950's transposing LDS read (ds_read_b64_tr_b16) delivers exactly
+// that: within a group of 16 lanes, lane L receives element L % 4 of the 8-byte pieces that lanes
+// L / 4, 4 + L / 4, 8 + L / 4 and 12 + L / 4 addressed.  With lane (c, g) addressing row 4 g + c / 4,
+// halves 4 (c % 4) .. of a tile of 16 columns, lane c receives column c of the tile for cells
+// 4 g .. 4 g + 3: the MFMA operand, no regrouping on the VALU.  The V images have rows of 544
+// bytes (8 banks apart: the 64 lanes' 8-byte pieces of such a read tile the banks exactly).
 //
 // Pools with q8_0 V ([f32 scale][32 x i8] blocks, qsa_attn_apply_gqa.comp:53-77) take the same
 // walk with work-groups of eight waves: the threads that fetch a V page dequantise it once for
@@ -52,12 +56,15 @@ constexpr int kRowsPerWave = 16;
 constexpr int kQ8vRow = kHd / 32 * 36;  // bytes of a q8_0 row
 constexpr int kI8hRow = kHd + kHd / 32 * 2;  // bytes of an int8 row: codes, then 8 f16 scales
 constexpr float kLog2e = 1.4426950408889634f;
-constexpr int kLdsRow = kHd + 8;  // halves per row of a page image in LDS (528 bytes)
+constexpr int kLdsRow = kHd + 8;    // halves per row of a K page image in LDS (528 bytes)
+constexpr int kLdsRowV = kHd + 16;  // of a V page image (544 bytes)
 
 typedef _Float16 h4 __attribute__((ext_vector_type(4)));
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
+typedef short tr_s4 __attribute__((__vector_size__(8)));  // what the transposing LDS read returns
+typedef __attribute__((address_space(3))) tr_s4* lds_tr_ptr;
 
 struct PrefillKernelParams {
     PrefillBatch b;
@@ -88,6 +95,7 @@ struct PageStage;
 template <>
 struct PageStage<BKV_LAYOUT_F16> {
     v4u k[2], v[2];  // chunks tid and tid + 256 of either image
+    int pg;
 };
 // the quantised layouts: thread tid owns row tid / 32, block tid / 4 % 8, codes 8 (tid % 4) .. + 7 of it
 template <>
@@ -105,9 +113,10 @@ struct PageStage<BKV_LAYOUT_I8H> {
 
 template <int LAY>
 struct PrefillLds {
-    // [buffer][image][16 rows][264 halves]; images: K, V -- with q8_0 V: K, V high parts, V low
-    // parts -- with int8 K and V: K high, V high, V low, K low parts
-    _Float16 img[4][LAY == BKV_LAYOUT_F16 ? 2 : LAY == BKV_LAYOUT_Q8V ? 3 : 4][kPage][kLdsRow];
+    // [buffer][image][16 rows][halves]: K (int8 pools: K high parts, K low parts) and V (quantised
+    // pools: V high parts, V low parts)
+    _Float16 kimg[4][LAY == BKV_LAYOUT_I8H ? 2 : 1][kPage][kLdsRow];
+    _Float16 vimg[4][LAY == BKV_LAYOUT_F16 ? 1 : 2][kPage][kLdsRowV];
     float e[LAY == BKV_LAYOUT_Q8V ? 4 : 1][kPage];  // q8_0 V: E of the buffer's cells
 };
 
@@ -187,12 +196,10 @@ __global__ __launch_bounds__(LAY == BKV_LAYOUT_F16 ? 256 : 512, LAY == BKV_LAYOU
         }
     }
 
-    // O^T accumulators: o[half][t][r] = out[row][128 half + 8 (4 g + r) + t]
-    f4 o[2][8];
+    // O^T accumulators: o[tile][r] = out[row][16 tile + 4 g + r]
+    f4 o[16];
 #pragma unroll
-    for (int h = 0; h < 2; ++h)
-#pragma unroll
-        for (int t = 0; t < 8; ++t) o[h][t] = f4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int t = 0; t < 16; ++t) o[t] = f4{0.0f, 0.0f, 0.0f, 0.0f};
     float m_run = -INFINITY;  // running max of this lane's query (base-2 logits), same in all 4 g lanes
     float l_run = 0.0f;       // this lane's share (its 4 cells per page) of the denominator
 
@@ -233,12 +240,13 @@ __global__ __launch_bounds__(LAY == BKV_LAYOUT_F16 ? 256 : 512, LAY == BKV_LAYOU
                 st.k[j] = *reinterpret_cast<const v4u*>(kp + (size_t)(tid + j * kThreads) * 16);
                 st.v[j] = *reinterpret_cast<const v4u*>(vp + (size_t)(tid + j * kThreads) * 16);
             }
+            st.pg = pg;
         }
     };
     const auto deposit = [&](int buf, const PageStage<LAY>& st) {
         // chunk q of a page image: row q / 32, halves (q % 32) * 8 ..
         if constexpr (Q8V) {
-            *reinterpret_cast<v4u*>(&L.img[buf][0][tid >> 5][(tid & 31) * 8]) = st.k;
+            *reinterpret_cast<v4u*>(&L.kimg[buf][0][tid >> 5][(tid & 31) * 8]) = st.k;
             // Rows past the work-group's last position were never written for these queries and
             // may hold anything: scale 1 for the row's exponent, zeros for its values.
             const bool dead = st.pg * kPage + v_row > wg_pos_max;
@@ -264,8 +272,8 @@ __global__ __launch_bounds__(LAY == BKV_LAYOUT_F16 ? 256 : 512, LAY == BKV_LAYOU
             for (int i = 0; i < 4; ++i) scaled_hi_lo(cd[i], sh, sl, hi[i], lo[i]);
             const h8 vh = h8{hi[0][0], hi[0][1], hi[1][0], hi[1][1], hi[2][0], hi[2][1], hi[3][0], hi[3][1]};
             const h8 vl = h8{lo[0][0], lo[0][1], lo[1][0], lo[1][1], lo[2][0], lo[2][1], lo[3][0], lo[3][1]};
-            *reinterpret_cast<h8*>(&L.img[buf][1][v_row][v_blk * 32 + v_j * 8]) = vh;
-            *reinterpret_cast<h8*>(&L.img[buf][2][v_row][v_blk * 32 + v_j * 8]) = vl;
+            *reinterpret_cast<h8*>(&L.vimg[buf][0][v_row][v_blk * 32 + v_j * 8]) = vh;
+            *reinterpret_cast<h8*>(&L.vimg[buf][1][v_row][v_blk * 32 + v_j * 8]) = vl;
             if ((tid & 31) == 0) L.e[buf][v_row] = (float)ee;
         } else if constexpr (I8H) {
             // K: code * scale (7 + 11 significant bits) as hi = f16(code * scale) and the exact
@@ -279,9 +287,9 @@ __global__ __launch_bounds__(LAY == BKV_LAYOUT_F16 ? 256 : 512, LAY == BKV_LAYOU
                 codes_to_f16(st.kc1, kd[2], kd[3]);
 #pragma unroll
                 for (int i = 0; i < 4; ++i) scaled_hi_lo(kd[i], sh, sl, hi[i], lo[i]);
-                *reinterpret_cast<h8*>(&L.img[buf][0][v_row][v_blk * 32 + v_j * 8]) =
+                *reinterpret_cast<h8*>(&L.kimg[buf][0][v_row][v_blk * 32 + v_j * 8]) =
                     h8{hi[0][0], hi[0][1], hi[1][0], hi[1][1], hi[2][0], hi[2][1], hi[3][0], hi[3][1]};
-                *reinterpret_cast<h8*>(&L.img[buf][3][v_row][v_blk * 32 + v_j * 8]) =
+                *reinterpret_cast<h8*>(&L.kimg[buf][1][v_row][v_blk * 32 + v_j * 8]) =
                     h8{lo[0][0], lo[0][1], lo[1][0], lo[1][1], lo[2][0], lo[2][1], lo[3][0], lo[3][1]};
             }
             // V: code * scale (7 + 11 significant bits) as hi = f16(code * scale) and the exact
@@ -295,23 +303,28 @@ __global__ __launch_bounds__(LAY == BKV_LAYOUT_F16 ? 256 : 512, LAY == BKV_LAYOU
             codes_to_f16(st.vc1, cd[2], cd[3]);
 #pragma unroll
             for (int i = 0; i < 4; ++i) scaled_hi_lo(cd[i], sh, sl, hi[i], lo[i]);
-            *reinterpret_cast<h8*>(&L.img[buf][1][v_row][v_blk * 32 + v_j * 8]) =
+            *reinterpret_cast<h8*>(&L.vimg[buf][0][v_row][v_blk * 32 + v_j * 8]) =
                 h8{hi[0][0], hi[0][1], hi[1][0], hi[1][1], hi[2][0], hi[2][1], hi[3][0], hi[3][1]};
-            *reinterpret_cast<h8*>(&L.img[buf][2][v_row][v_blk * 32 + v_j * 8]) =
+            *reinterpret_cast<h8*>(&L.vimg[buf][1][v_row][v_blk * 32 + v_j * 8]) =
                 h8{lo[0][0], lo[0][1], lo[1][0], lo[1][1], lo[2][0], lo[2][1], lo[3][0], lo[3][1]};
         } else {
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 const int q = tid + j * kThreads;
-                *reinterpret_cast<v4u*>(&L.img[buf][0][q >> 5][(q & 31) * 8]) = st.k[j];
-                *reinterpret_cast<v4u*>(&L.img[buf][1][q >> 5][(q & 31) * 8]) = st.v[j];
+                // V rows past the work-group's last position were never written for these queries and
+                // may hold anything (even NaN): exact zeros, before they meet a zero probability
+                const bool dead = st.pg * kPage + (q >> 5) > wg_pos_max;
+                *reinterpret_cast<v4u*>(&L.kimg[buf][0][q >> 5][(q & 31) * 8]) = st.k[j];
+                *reinterpret_cast<v4u*>(&L.vimg[buf][0][q >> 5][(q & 31) * 8]) = dead ? v4u{0u, 0u, 0u, 0u} : st.v[j];
             }
         }
     };
 
+    // this lane's piece of a transposing V read: row 4 g + c / 4, halves 4 (c % 4) .. of a 16-column tile
+    const int tr_off = (4 * g + (c >> 2)) * kLdsRowV + 4 * (c & 3);
     // scores of one page: s[r] = q[row c] . k[cell 4 g + r], masked and in base 2
     const auto scores = [&](int pg, int buf, float (&t4)[4]) {
-        const _Float16* ks = &L.img[buf][0][0][0];
+        const _Float16* ks = &L.kimg[buf][0][0][0];
         // K: row c, 16 bytes at element 32 m + 8 g (the same split of the head dim as q): the 8
         // halves of a lane are the 8 contraction steps it feeds to the 32-deep MFMA
         h8 kf[8];
@@ -320,7 +333,7 @@ __global__ __launch_bounds__(LAY == BKV_LAYOUT_F16 ? 256 : 512, LAY == BKV_LAYOU
         f4 s;
         if constexpr (I8H) {
             // K = hi + lo: hi meets q's high and low parts, lo q's high parts; three chains
-            const _Float16* kl = &L.img[buf][3][0][0];
+            const _Float16* kl = &L.kimg[buf][1][0][0];
             f4 s0 = f4{0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0, s2 = s0;
 #pragma unroll
             for (int m = 0; m < 8; ++m) {
@@ -410,48 +423,29 @@ __global__ __launch_bounds__(LAY == BKV_LAYOUT_F16 ? 256 : 512, LAY == BKV_LAYOU
         m_run = m_new;
         if (__builtin_amdgcn_ballot_w64(moved) != 0) {
 #pragma unroll
-            for (int h = 0; h < 2; ++h)
-#pragma unroll
-                for (int t = 0; t < 8; ++t) o[h][t] *= alpha;
+            for (int t = 0; t < 16; ++t) o[t] *= alpha;
         }
 
         // ---- O^T += V^T . P^T over the 32 cells of the pair ----------------------------------------
-        // V: rows 4 g + r of either page, 16 bytes at element 128 half + 8 c.  Rows past the last
-        // position of this wave were never written for these queries and may hold anything (even
-        // NaN): they are made exact zeros before they meet a zero probability.
-        const bool a_last = pg == n_pages - 1, b_last = pg + 1 == n_pages - 1;
+        // Per tile of 16 output columns one transposing read from either page's image: lane (c, g)
+        // receives column 16 tile + c of cells 4 g .. 4 g + 3 -- slots 0..3 and 4..7 of the operand,
+        // the order P^T has.  Rows past the work-group's last position are zeros in the image.  A
+        // second page past this wave's last one meets zero probabilities: its buffer holds a page of
+        // the work-group all the same (the last one again, past the end), never nothing, so the
+        // reads need no condition and the 32 of them can be issued ahead of the MFMAs.
         // quantised V: the image of high parts meets p's high and low parts, the image of low parts
         // p's high parts
 #pragma unroll
-        for (int img = 1; img < (WIDE ? 3 : 2); ++img) {
-            const _Float16* va_s = &L.img[buf][img][0][0];
-            const _Float16* vb_s = &L.img[buf + 1][img][0][0];
+        for (int img = 0; img < (WIDE ? 2 : 1); ++img) {
+            const _Float16* va_s = &L.vimg[buf][img][0][0] + tr_off;
+            const _Float16* vb_s = &L.vimg[buf + 1][img][0][0] + tr_off;
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                v4u fa[4], fb[4];
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    fa[r] = *reinterpret_cast<const v4u*>(va_s + (4 * g + r) * kLdsRow + h * 128 + c * 8);
-                    fb[r] = *reinterpret_cast<const v4u*>(vb_s + (4 * g + r) * kLdsRow + h * 128 + c * 8);
-                }
-                if (a_last || b_last || !second) {
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        if (a_last && pg * kPage + 4 * g + r > pos_max) fa[r] = v4u{0u, 0u, 0u, 0u};
-                        if (!second || (b_last && (pg + 1) * kPage + 4 * g + r > pos_max)) fb[r] = v4u{0u, 0u, 0u, 0u};
-                    }
-                }
-                const h8 a0 = __builtin_bit_cast(h8, fa[0]), a1 = __builtin_bit_cast(h8, fa[1]);
-                const h8 a2 = __builtin_bit_cast(h8, fa[2]), a3 = __builtin_bit_cast(h8, fa[3]);
-                const h8 b0 = __builtin_bit_cast(h8, fb[0]), b1 = __builtin_bit_cast(h8, fb[1]);
-                const h8 b2 = __builtin_bit_cast(h8, fb[2]), b3 = __builtin_bit_cast(h8, fb[3]);
-#pragma unroll
-                for (int t = 0; t < 8; ++t) {
-                    // column 128 h + 8 c + t of the pair's cells 4 g .. of either page
-                    const h8 vv = h8{a0[t], a1[t], a2[t], a3[t], b0[t], b1[t], b2[t], b3[t]};
-                    o[h][t] = mfma32(vv, ph, o[h][t]);
-                    if (img == 1) o[h][t] = mfma32(vv, pl, o[h][t]);
-                }
+            for (int t = 0; t < 16; ++t) {
+                const tr_s4 fa = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(va_s + t * 16));
+                const tr_s4 fb = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(vb_s + t * 16));
+                const h8 vv = __builtin_bit_cast(h8, __builtin_shufflevector(fa, fb, 0, 1, 2, 3, 4, 5, 6, 7));
+                o[t] = mfma32(vv, ph, o[t]);
+                if (img == 0) o[t] = mfma32(vv, pl, o[t]);
             }
         }
     };
@@ -487,30 +481,27 @@ __global__ __launch_bounds__(LAY == BKV_LAYOUT_F16 ? 256 : 512, LAY == BKV_LAYOU
                                    (size_t)head * P.gate_head_stride
                              : nullptr;
 #pragma unroll
-    for (int h = 0; h < 2; ++h)
+    for (int t = 0; t < 16; ++t) {
+        const int d0 = 16 * t + 4 * g;
+        float y[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const int d0 = h * 128 + 8 * (4 * g + r);
-            float y[8];
-#pragma unroll
-            for (int t = 0; t < 8; ++t) {
-                y[t] = o[h][t][r] * inv;
-                if (gp) {
-                    // sigmoid in the overflow-free form of the reference (qsa/cpu.rs:84-91)
-                    const float gt = gp[d0 + t];
-                    float sg;
-                    if (gt >= 0.0f) {
-                        sg = 1.0f / (1.0f + expf(-gt));
-                    } else {
-                        const float ex = expf(gt);
-                        sg = ex / (1.0f + ex);
-                    }
-                    y[t] *= sg;
+            y[r] = o[t][r] * inv;
+            if (gp) {
+                // sigmoid in the overflow-free form of the reference (qsa/cpu.rs:84-91)
+                const float gt = gp[d0 + r];
+                float sg;
+                if (gt >= 0.0f) {
+                    sg = 1.0f / (1.0f + expf(-gt));
+                } else {
+                    const float ex = expf(gt);
+                    sg = ex / (1.0f + ex);
                 }
+                y[r] *= sg;
             }
-            *reinterpret_cast<float4*>(op + d0) = make_float4(y[0], y[1], y[2], y[3]);
-            *reinterpret_cast<float4*>(op + d0 + 4) = make_float4(y[4], y[5], y[6], y[7]);
         }
+        *reinterpret_cast<float4*>(op + d0) = make_float4(y[0], y[1], y[2], y[3]);
+    }
 }
 
 }  // namespace
