@@ -42,6 +42,8 @@
 // Int8 pools (codes with an f16 scale per 32 values, K and V alike) are dequantised the same way,
 // without the exponent: both K and V become hi/lo image pairs, and the scores are
 // K_hi.q_hi + K_hi.q_lo + K_lo.q_hi.
+#include <algorithm>
+
 #include "bkv_internal.hpp"
 #include "lane_groups.hpp"
 #include "quant_decode.hpp"
@@ -56,6 +58,7 @@ constexpr int kRowsPerWave = 16;
 constexpr int kQ8vRow = kHd / 32 * 36;  // bytes of a q8_0 row
 constexpr int kI8hRow = kHd + kHd / 32 * 2;  // bytes of an int8 row: codes, then 8 f16 scales
 constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLoDown = 1.0f / 2048.0f;  // q's low parts enter the products times 2^11
 constexpr int kLdsRow = kHd + 8;    // halves per row of a K page image in LDS (528 bytes)
 constexpr int kLdsRowV = kHd + 16;  // of a V page image (544 bytes)
 
@@ -77,7 +80,15 @@ struct PrefillKernelParams {
     int64_t gate_tok_stride, gate_head_stride;
     int32_t max_pages_per_seq, n_kv, n_q, group;
     float scale_log2e;
+    int32_t by_xcd;  // work-groups are dealt to the chip's 8 dies so that each die sees few (entry, kv head) units
 };
+
+// The chip is 8 dies (XCDs), each with an L2 of its own, and work-group i runs on die i % 8.
+// Every work-group of one (entry, kv head) unit walks the same K/V pages, so the dies are given
+// whole units: with 8 or more units, die x serves units x, x + 8, ...; with fewer, unit u is
+// served by dies u, u + U, ...  A unit's pages then stay in one die's L2 (3 MiB for a 3072-token
+// chunk) instead of every die fetching every unit through the fabric.
+constexpr int kXcds = 8;
 
 // gfx950's double-depth form: 32 contraction steps, 8 halves per lane (k = 8 (lane / 16) + 0..7)
 __device__ __forceinline__ f4 mfma32(h8 a, h8 b, f4 c) {
@@ -130,14 +141,40 @@ __global__ __launch_bounds__(LAY == BKV_LAYOUT_F16 ? 256 : 512, LAY == BKV_LAYOU
     constexpr int kThreads = 64 * kWavesPerWg;
     constexpr int kRowsPerWg = kRowsPerWave * kWavesPerWg;
     // ---- which (entry, kv head, block of 64 query rows) ---------------------------------
-    int e = 0;
-    while (e + 1 < P.b.n && (int)blockIdx.x >= P.b.wg_base[e + 1]) ++e;
-    const int rem = (int)blockIdx.x - P.b.wg_base[e];
-    const int kvh = rem % P.n_kv;
+    int e = 0, kvh, idx;  // idx: which of the unit's blocks, in dispatch order
+    if (P.by_xcd) {
+        const int units = P.b.n * P.n_kv;
+        const int x = (int)blockIdx.x % kXcds;
+        int j = (int)blockIdx.x / kXcds;
+        int u;
+        if (units >= kXcds) {
+            u = x;
+            for (;;) {
+                if (u >= units) return;  // this die's share of the grid is shorter than the longest
+                const int nb = (P.b.n_tok[u / P.n_kv] * P.group + kRowsPerWg - 1) / kRowsPerWg;
+                if (j < nb) break;
+                j -= nb;
+                u += kXcds;
+            }
+            idx = j;
+        } else {
+            u = x % units;
+            const int dies = (kXcds - u + units - 1) / units;  // dies x with x % units == u
+            idx = j * dies + x / units;
+        }
+        e = u / P.n_kv;
+        kvh = u - e * P.n_kv;
+    } else {
+        while (e + 1 < P.b.n && (int)blockIdx.x >= P.b.wg_base[e + 1]) ++e;
+        const int rem = (int)blockIdx.x - P.b.wg_base[e];
+        kvh = rem % P.n_kv;
+        idx = rem / P.n_kv;
+    }
     const int n_rows = P.b.n_tok[e] * P.group;  // query rows of this kv head
     const int n_blocks = (n_rows + kRowsPerWg - 1) / kRowsPerWg;
+    if (idx >= n_blocks) return;
     // later rows attend more cells: the heaviest blocks are dispatched first
-    const int rb = n_blocks - 1 - rem / P.n_kv;
+    const int rb = n_blocks - 1 - idx;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
     const int c = lane & 15;  // query row of the tile / cell of the page / output column group
@@ -151,7 +188,11 @@ __global__ __launch_bounds__(LAY == BKV_LAYOUT_F16 ? 256 : 512, LAY == BKV_LAYOU
     const bool row_live = wave_live && row < n_rows;
     const int tok = row_live ? row / P.group : 0;
     const int head = kvh * P.group + (row_live ? row % P.group : 0);
-    const int pos_q = row_live ? P.b.pos0[e] + tok : -1;
+    // a lane without a query row (past the end of the chunk) walks along with q = 0 and every cell
+    // live: its column of the products is its own, and nothing of it is stored
+    const int pos_q = row_live ? P.b.pos0[e] + tok : 0x7fffffff;
+    // the first position any row of this wave has: pages wholly at or below it need no causal mask
+    const int pos_min = P.b.pos0[e] + (wave_live ? row0 / P.group : 0);
     // the last token any row of this wave belongs to bounds the page walk
     const int last_row = min(row0 + kRowsPerWave, n_rows) - 1;
     const int pos_max = wave_live ? P.b.pos0[e] + last_row / P.group : -1;
@@ -186,12 +227,20 @@ __global__ __launch_bounds__(LAY == BKV_LAYOUT_F16 ? 256 : 512, LAY == BKV_LAYOU
 #pragma unroll
                 for (int j = 0; j < 8; ++j) x[j] = 0.0f;
             }
+            // The softmax scale (and the change to base 2) rides on q: one rounding of q, 2^-24
+            // relative.  The low parts are kept times 2^11 and their products scaled back in f32
+            // (kLoDown), which keeps them out of the f16 subnormals' few bits.  The product is
+            // pinned as one f32 number: left to fuse it into the conversions, the compiler took the
+            // remainder against f16(x * c) rounded once and stored a high part rounded twice (x * c to
+            // f32, then to f16) -- two numbers that differ by an f16 ulp now and then, which showed as
+            // 3e-5 in short contexts.
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                _Float16 hi, lo;
-                split_f16(x[j], hi, lo);
+                float xs = x[j] * P.scale_log2e;
+                asm("" : "+v"(xs));  // the product as one f32 number: no fusing into the conversions below
+                const _Float16 hi = (_Float16)xs;
                 qhi[m][j] = hi;
-                qlo[m][j] = lo;
+                qlo[m][j] = (_Float16)((xs - (float)hi) * 2048.0f);
             }
         }
     }
@@ -308,29 +357,31 @@ __global__ __launch_bounds__(LAY == BKV_LAYOUT_F16 ? 256 : 512, LAY == BKV_LAYOU
             *reinterpret_cast<h8*>(&L.vimg[buf][1][v_row][v_blk * 32 + v_j * 8]) =
                 h8{lo[0][0], lo[0][1], lo[1][0], lo[1][1], lo[2][0], lo[2][1], lo[3][0], lo[3][1]};
         } else {
+            // V rows past the work-group's last position were never written for these queries and may
+            // hold anything (even NaN): exact zeros, before they meet a zero probability.  Only the
+            // work-group's last page has such rows.
+            const bool last_page = st.pg * kPage + kPage - 1 > wg_pos_max;
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 const int q = tid + j * kThreads;
-                // V rows past the work-group's last position were never written for these queries and
-                // may hold anything (even NaN): exact zeros, before they meet a zero probability
-                const bool dead = st.pg * kPage + (q >> 5) > wg_pos_max;
+                v4u vv = st.v[j];
+                if (last_page && st.pg * kPage + (q >> 5) > wg_pos_max) vv = v4u{0u, 0u, 0u, 0u};
                 *reinterpret_cast<v4u*>(&L.kimg[buf][0][q >> 5][(q & 31) * 8]) = st.k[j];
-                *reinterpret_cast<v4u*>(&L.vimg[buf][0][q >> 5][(q & 31) * 8]) = dead ? v4u{0u, 0u, 0u, 0u} : st.v[j];
+                *reinterpret_cast<v4u*>(&L.vimg[buf][0][q >> 5][(q & 31) * 8]) = vv;
             }
         }
     };
 
     // this lane's piece of a transposing V read: row 4 g + c / 4, halves 4 (c % 4) .. of a 16-column tile
     const int tr_off = (4 * g + (c >> 2)) * kLdsRowV + 4 * (c & 3);
-    // scores of one page: s[r] = q[row c] . k[cell 4 g + r], masked and in base 2
-    const auto scores = [&](int pg, int buf, float (&t4)[4]) {
+    // scores of one page in base 2: s[r] = scale * log2(e) * q[row c] . k[cell 4 g + r], unmasked
+    const auto scores = [&](int buf) -> f4 {
         const _Float16* ks = &L.kimg[buf][0][0][0];
         // K: row c, 16 bytes at element 32 m + 8 g (the same split of the head dim as q): the 8
         // halves of a lane are the 8 contraction steps it feeds to the 32-deep MFMA
         h8 kf[8];
 #pragma unroll
         for (int m = 0; m < 8; ++m) kf[m] = *reinterpret_cast<const h8*>(ks + c * kLdsRow + m * 32 + g * 8);
-        f4 s;
         if constexpr (I8H) {
             // K = hi + lo: hi meets q's high and low parts, lo q's high parts; three chains
             const _Float16* kl = &L.kimg[buf][1][0][0];
@@ -342,24 +393,17 @@ __global__ __launch_bounds__(LAY == BKV_LAYOUT_F16 ? 256 : 512, LAY == BKV_LAYOU
                 s1 = mfma32(kf[m], qlo[m], s1);
                 s2 = mfma32(klo, qhi[m], s2);
             }
-            s = (s0 + s1) + s2;
+            return (s0 + s2) + s1 * kLoDown;
         } else {
-            // four independent accumulation chains: an MFMA that waits for the previous one's
-            // result costs its full latency
-            f4 s0 = f4{0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0, s2 = s0, s3 = s0;
+            // two accumulation chains, q's high parts and q's low parts: an MFMA adds to the sum of the
+            // one before the last, which has left the pipeline by then
+            f4 s0 = f4{0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0;
 #pragma unroll
-            for (int m = 0; m < 8; m += 2) {
+            for (int m = 0; m < 8; ++m) {
                 s0 = mfma32(kf[m], qhi[m], s0);
                 s1 = mfma32(kf[m], qlo[m], s1);
-                s2 = mfma32(kf[m + 1], qhi[m + 1], s2);
-                s3 = mfma32(kf[m + 1], qlo[m + 1], s3);
             }
-            s = (s0 + s1) + (s2 + s3);
-        }
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int cell = pg * kPage + 4 * g + r;
-            t4[r] = cell <= pos_q ? s[r] * P.scale_log2e : -INFINITY;
+            return s0 + s1 * kLoDown;
         }
     };
 
@@ -369,12 +413,22 @@ __global__ __launch_bounds__(LAY == BKV_LAYOUT_F16 ? 256 : 512, LAY == BKV_LAYOU
     const auto process_pair = [&](int pg, int buf) {
         const bool second = pg + 1 < n_pages;
         float ta[4], tb[4];
-        scores(pg, buf, ta);
-        if (second) {
-            scores(pg + 1, buf + 1, tb);
-        } else {
+        {
+            const f4 sa = scores(buf);
+            f4 sb = f4{0.0f, 0.0f, 0.0f, 0.0f};
+            if (second) sb = scores(buf + 1);
+            if (second && (pg + 2) * kPage - 1 <= pos_min) {
+                // every cell of the pair is at or below every row's position
 #pragma unroll
-            for (int r = 0; r < 4; ++r) tb[r] = -INFINITY;
+                for (int r = 0; r < 4; ++r) ta[r] = sa[r], tb[r] = sb[r];
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int cell = pg * kPage + 4 * g + r;
+                    ta[r] = cell <= pos_q ? sa[r] : -INFINITY;
+                    tb[r] = second && cell + kPage <= pos_q ? sb[r] : -INFINITY;
+                }
+            }
         }
         // q8_0 V: the softmax runs over logit + E of the cell (wa, wb); dead cells stay at -inf
         float wa[4], wb[4];
@@ -393,33 +447,41 @@ __global__ __launch_bounds__(LAY == BKV_LAYOUT_F16 ? 256 : 512, LAY == BKV_LAYOU
         }
 
         // ---- online softmax for this lane's query, over the pair's 32 cells ---------------------------
+        // Cell 0 is live for every query, so from the first pair on the reference m_run is finite.
+        // It follows the running maximum lazily: it moves only when a pair's maximum passes it by
+        // more than kSlack (weights then reach 2^kSlack at most, far inside f16 and f32), which after
+        // the first pairs is rare -- and every move costs a rescale of the 64 accumulators.  The
+        // q8_0 weights multiply values of up to 2^8, so there the reference is the maximum itself.
+        constexpr float kSlack = Q8V ? 0.0f : 6.0f;
         float pm = fmaxf(fmaxf(fmaxf(wa[0], wa[1]), fmaxf(wa[2], wa[3])), fmaxf(fmaxf(wb[0], wb[1]), fmaxf(wb[2], wb[3])));
         pm = max_over_lane_groups(pm);
-        const float m_new = fmaxf(m_run, pm);
-        // a query with no live cell yet keeps m = -inf: exp2(-inf - -inf) would be NaN
-        const bool none_yet = m_new == -INFINITY;
-        const float alpha = none_yet ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
-        h8 ph, pl;  // slots 0..3: the first page's cells 4 g + r, slots 4..7: the second page's
+        const bool moved = pm > m_run + kSlack;  // m_run = -inf at the start: any finite maximum moves it
+        const float m_new = moved ? pm : m_run;
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // 1, or 0 at the start
+        float pv[8];
         float psum = 0.0f;
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
             const float ww = r < 4 ? wa[r & 3] : wb[r & 3];
-            const float p = none_yet ? 0.0f : __builtin_amdgcn_exp2f(ww - m_new);
+            pv[r] = __builtin_amdgcn_exp2f(ww - m_new);
             if constexpr (Q8V) {
                 const float tt = r < 4 ? ta[r & 3] : tb[r & 3];
-                psum += none_yet ? 0.0f : __builtin_amdgcn_exp2f(tt - m_new);
+                psum += __builtin_amdgcn_exp2f(tt - m_new);
             } else {
-                psum += p;
+                psum += pv[r];
             }
+        }
+        // p = hi + lo, both rounded to nearest (the matrix cores read f16 subnormals as the numbers
+        // they are, so small weights keep their low parts' few bits)
+        h8 ph, pl;  // slots 0..3: the first page's cells 4 g + r, slots 4..7: the second page's
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
             _Float16 hi, lo;
-            split_f16(p, hi, lo);
+            split_f16(pv[r], hi, lo);
             ph[r] = hi;
             pl[r] = lo;
         }
         l_run = l_run * alpha + psum;
-        // rescale only where some query's maximum moved (the test is on the maxima, not on
-        // alpha != 1: with the latter the compiler multiplies unconditionally, 64 instructions)
-        const bool moved = m_new > m_run;
         m_run = m_new;
         if (__builtin_amdgcn_ballot_w64(moved) != 0) {
 #pragma unroll
@@ -525,8 +587,33 @@ hipError_t launch_prefill_attn(bkv_pool* p, int32_t layer, const PrefillBatch& b
     kp.n_q = a.n_q_head;
     kp.group = a.n_q_head / p->g.n_kv;
     kp.scale_log2e = a.scale * kLog2e;
-    const int32_t grid = b.wg_base[b.n];
+    int32_t grid = b.wg_base[b.n];
     if (grid == 0) return hipSuccess;
+    // Deal the work-groups to the dies by unit where that costs little: the grid then holds 8 x the
+    // longest die's share, and work-groups past a shorter die's share leave at once.
+    kp.by_xcd = 0;
+    {
+        const int rows_per_wg = prefill_rows_per_wg(p->g.layout);
+        const int units = b.n * p->g.n_kv;
+        int64_t longest = 0;
+        if (units >= kXcds) {
+            int64_t share[kXcds] = {};
+            for (int u = 0; u < units; ++u)
+                share[u % kXcds] += ((int64_t)b.n_tok[u / p->g.n_kv] * kp.group + rows_per_wg - 1) / rows_per_wg;
+            for (int x = 0; x < kXcds; ++x) longest = std::max(longest, share[x]);
+        } else {
+            for (int u = 0; u < units; ++u) {
+                const int64_t nb = ((int64_t)b.n_tok[u / p->g.n_kv] * kp.group + rows_per_wg - 1) / rows_per_wg;
+                const int dies = (kXcds - u + units - 1) / units;
+                longest = std::max(longest, (nb + dies - 1) / dies);
+            }
+        }
+        const int64_t by_xcd_grid = longest * kXcds;
+        if (by_xcd_grid <= (int64_t)grid + grid / 4 + kXcds) {
+            kp.by_xcd = 1;
+            grid = (int32_t)by_xcd_grid;
+        }
+    }
     if (p->g.layout == BKV_LAYOUT_Q8V)
         launch_staged(p, BKV_STAGE_PREFILL_ATTN, prefill_attn_kernel<BKV_LAYOUT_Q8V>, dim3((unsigned)grid), dim3(512), 0,
                       stream, kp);
