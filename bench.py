@@ -114,8 +114,12 @@ def prepare_steps(pool, seqs, ctx0, n_layers, steps, q_dev, out_dev, newk, newv,
         layer, tok = i % n_layers, i // n_layers
         pos = np.ascontiguousarray([c + tok for c in ctx0], dtype=np.int64)
         off = (i % newk.n_slots) * n * N_KV * HD * 4
-        plan.append((layer, pos, pos.ctypes.data_as(C.POINTER(C.c_int64)), newk.at(off), newv.at(off)))
-    return {"plan": plan, "seq_arr": seq_arr, "ps": ps, "ones": ones,
+        plan.append((layer, [int(p) + 1 for p in pos] if layer == 0 else None,
+                     pos.ctypes.data_as(C.POINTER(C.c_int64)), newk.at(off), newv.at(off), pos))
+    from breccia_amd.kv import PagePair
+
+    return {"plan": plan, "seq_ids": [int(s) for s in seqs], "cow_pairs": (PagePair * 4)(), "n_cow": C.c_int32(),
+             "seq_arr": seq_arr, "ps": ps, "ones": ones,
             "pones": ones.ctypes.data_as(C.POINTER(C.c_int32)), "q": q_dev.ptr, "out": out_dev.ptr,
             "stream": stream.handle, "n": n}
 
@@ -126,12 +130,16 @@ def issue_steps(pool, seqs, prep, fused=True):
     from breccia_amd.kv import check, lib
 
     n, ps, st, q, out, h = prep["n"], prep["ps"], prep["stream"], prep["q"], prep["out"], pool.handle
-    for layer, pos, pp, k_new, v_new in prep["plan"]:
-        if layer == 0:
-            for s, p in zip(seqs, pos):
-                pool.seq_reserve(s, int(p) + 1)
+    ids, pairs, n_cow = prep["seq_ids"], prep["cow_pairs"], prep["n_cow"]
+    reserve, step = lib.bkv_seq_reserve, lib.bkv_decode_step
+    for layer, new_lens, pp, k_new, v_new, _pos in prep["plan"]:
+        if new_lens is not None:
+            for s, new_len in zip(ids, new_lens):
+                check(reserve(h, s, new_len, pairs, 4, n_cow))
+                if n_cow.value:  # no sequence of this workload shares a page
+                    raise RuntimeError("bkv_seq_reserve reported a copy-on-write pair in the bench workload")
         if fused:
-            check(lib.bkv_decode_step(h, layer, n, ps, pp, k_new, v_new, N_Q, q, None, 0, 0, 1.0 / 16.0, out, st))
+            check(step(h, layer, n, ps, pp, k_new, v_new, N_Q, q, None, 0, 0, 1.0 / 16.0, out, st))
         else:
             check(lib.bkv_append(h, layer, n, ps, pp, prep["pones"], k_new, v_new, st))
             check(lib.bkv_decode_attn(h, layer, n, ps, pp, N_Q, q, None, 0, 0, 1.0 / 16.0, out, st))
@@ -145,8 +153,8 @@ def run_steps(pool, seqs, ctx0, n_layers, steps, q_dev, out_dev, newk, newv, str
 
 
 def time_steps(pool, seqs, ctx0, n_layers, steps, warmup, bufs, stream, first_step=0, fused=True):
-    """(wall milliseconds of `steps` steps between two synchronisations, the same by stream events
-    in a second pass of as many steps)."""
+    """(wall milliseconds of `steps` steps between two device-wide synchronisations, the same up to the
+    synchronisation of the stream that carries them)."""
     from breccia_amd.kv import Event, device_sync
 
     q_dev, out_dev, newk, newv = bufs
@@ -157,9 +165,10 @@ def time_steps(pool, seqs, ctx0, n_layers, steps, warmup, bufs, stream, first_st
     t0 = time.perf_counter()
     issue_steps(pool, seqs, prep, fused)
     stream.sync()
-    device_sync()
+    stream_ms = (time.perf_counter() - t0) * 1e3
+    device_sync()  # nothing else is pending: every launch of the region was on `stream`
     wall_ms = (time.perf_counter() - t0) * 1e3
-    return wall_ms, None
+    return wall_ms, stream_ms
 
 
 def event_steps(pool, seqs, ctx0, n_layers, steps, bufs, stream, first_step):
@@ -272,11 +281,12 @@ def main() -> int:
     # ---- headline: K steps, whole path ------------------------------------------------
     # REGIONS consecutive timed regions of --steps steps each (every one bracketed by host
     # synchronisations); ms_per_step is the median region's, the spread goes into `extra`
-    region_ms = []
+    region_ms, region_stream_ms = [], []
     for r in range(REGIONS):
-        wall_ms, _ = time_steps(pool, seqs, ctx, n_layers, args.steps, args.warmup if r == 0 else 0, bufs, stream,
-                                first_step=pre_steps + (args.warmup + r * args.steps if r else 0))
+        wall_ms, stream_ms = time_steps(pool, seqs, ctx, n_layers, args.steps, args.warmup if r == 0 else 0, bufs, stream,
+                                     first_step=pre_steps + (args.warmup + r * args.steps if r else 0))
         region_ms.append(wall_ms / args.steps)
+        region_stream_ms.append(stream_ms / args.steps)
     ms_per_step = float(np.median(region_ms))
     ctx_mid = [c + 1 + (pre_steps + args.warmup + REGIONS * args.steps // 2) // n_layers for c in ctx]
     pre_steps += (REGIONS - 1) * args.steps          # steps taken so far = pre_steps + warmup + steps, as below
@@ -371,6 +381,8 @@ def main() -> int:
              "step_event_ms": round(ev_ms / args.steps, 4),
              "timed_regions": {"count": REGIONS, "steps_each": args.steps, "reported": "median",
                                "ms_per_step": [round(x, 5) for x in region_ms],
+                               "end_of_region": "bkv_stream_sync of the stream that carries every launch, then bkv_device_sync",
+                               "median_ms_per_step_up_to_the_stream_sync": round(float(np.median(region_stream_ms)), 5),
                                "min_ms_per_step": round(min(region_ms), 5), "max_ms_per_step": round(max(region_ms), 5),
                                "frac_of_hbm_peak_min_max": [round(step_bytes / (max(region_ms) * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
                                                             round(step_bytes / (min(region_ms) * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)]},
