@@ -1014,8 +1014,6 @@ def bench_moves(stream) -> dict:
     pool.timing_enable(False)
     n_k, ms_k = pool.timing_read(L.STAGE_APPEND_KPREP)
     res["append_kprep_bulk"]["kernel_ms"] = round(ms_k / max(n_k, 1), 4)
-    gd.free()
-    td.free()
     # the quantised layouts on the same bulk shape: f32 rows in, and raw f16 rows in (BASELINE
     # configs[4]: "quantized from N(0,1) f16 on append")
     k16 = DeviceBuffer.from_numpy(rng.standard_normal((4 * T, N_KV, HD), dtype=np.float32).astype(np.float16))
@@ -1036,8 +1034,12 @@ def bench_moves(stream) -> dict:
                          "GBps": round(b / ms / 1e6, 1), "frac_of_hbm_peak": round(b / ms / 1e6 / HBM_PEAK_GBPS, 4)}
         ms = timed(lambda: qp.append(0, qs, [7] * 4, [1] * 4, kd, vd, stream), 200)
         res["append_decode_%s_us" % tag] = round(ms * 1e3, 2)
+        ms = timed(lambda: qp.append_kprep(0, qs, [0] * 4, [T] * 4, kd, vd, gd, 1e-6, td, 64, T, stream=stream), 20)
+        b = 4 * T * (N_KV * HD * 4 * 2 + out_bytes)
+        res["append_kprep_bulk_" + tag] = {"tokens": 4 * T, "ms": round(ms, 4), "GBps": round(b / ms / 1e6, 1),
+                                           "frac_of_hbm_peak": round(b / ms / 1e6 / HBM_PEAK_GBPS, 4)}
         qp.destroy()
-    for x in (kd, vd, k16, v16):
+    for x in (kd, vd, k16, v16, gd, td):
         x.free()
 
     # page copy: 16384 pairs = 512 MiB read + 512 MiB written

@@ -168,35 +168,44 @@ __global__ __launch_bounds__(kBlock) void append_f16_kernel(AppendBatch b, MoveG
     st_stream(vpool + dst, vo);
 }
 
+// ---- 8 values at a time: the lane's share of a 32-value block whose other shares the rest of its quad holds --
+// Both return the rule's results exactly: codes on a reciprocal with a proof per value, and the rule as
+// written for the whole wave when any lane could not prove its codes.
 template <typename SrcT>
-__device__ __forceinline__ void load32(const SrcT* p, float (&x)[32]) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        float y[8];
-        load8(p + i * 8, y);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) x[i * 8 + j] = y[j];
+__device__ __forceinline__ void q8v_quarter(float (&x)[8], float& scale, uint32_t& w0, uint32_t& w1) {
+    const float amax = quad_max(amax8(x));
+    scale = q8v_scale(amax);
+    uint32_t doubt = (std::is_same<SrcT, uint16_t>::value && !(amax > 0x1p-6f)) ? 0x7fc00000u : 0u;
+    codes8_on_reciprocal(x, scale, w0, w1, doubt);
+    if (__any(codes_in_doubt(doubt))) {
+        flush8<SrcT>(x);
+        scale = q8v_scale(quad_max(amax8(x)));
+        q8_codes8(x, scale, w0, w1);
     }
 }
-
-// One q8_0 block as the V pool holds it: [f32 scale][32 x i8] = 9 words.
-__device__ __forceinline__ void q8v_encode(const float (&x)[32], uint32_t* vd) {
-    uint32_t w[9];
-    q8v_block_words(x, w);
-#pragma unroll
-    for (int j = 0; j < 9; ++j) vd[j] = w[j];
+// f32 values only (binary16 rows have a path of their own in append_quant_kernel)
+__device__ __forceinline__ void i8h_quarter(const float (&x)[8], uint32_t& scale_bits, uint32_t& w0, uint32_t& w1) {
+    scale_bits = i8h_scale_bits(quad_max(amax8(x)));
+    uint32_t doubt = 0u;
+    codes8_on_reciprocal(x, f16_normal_value(scale_bits), w0, w1, doubt);
+    if (__any(codes_in_doubt(doubt))) i8h_codes8(x, f16_load(scale_bits), w0, w1);
 }
 
-// ---- append, int8 K and V with f16 scales: row = [hd x i8][hd/32 x f16] -----------
-// The q8_0 rule with the scale stored through the cache's f16 encoding; a scale the
-// f16 rule would flush is raised to 2^-14.  (No reference counterpart.)
-__device__ __forceinline__ void i8h_encode(const float (&x)[32], uint8_t* row_base, int hd, int blk) {
-    uint32_t w[8], hb;
-    i8h_block_words(x, w, hb);
-    uint4* qd = reinterpret_cast<uint4*>(row_base + (size_t)blk * 32);
-    qd[0] = make_uint4(w[0], w[1], w[2], w[3]);
-    qd[1] = make_uint4(w[4], w[5], w[6], w[7]);
-    *reinterpret_cast<uint16_t*>(row_base + hd + blk * 2) = (uint16_t)hb;
+// Encoded rows put together in LDS leave as whole contiguous rows: piece p of the image goes to the same
+// offset of its pool row (16-byte pieces where rows are multiples of 16 bytes, else 4-byte ones).
+template <uint32_t PIECE>
+__device__ __forceinline__ void image_rows_out(const uint8_t* image, uint8_t* pool, const uint64_t* row_s, int nrows,
+                                               uint32_t row_bytes, int tid) {
+    const uint32_t ppr = row_bytes / PIECE;  // pieces of a row
+    const uint32_t n_pieces = (uint32_t)nrows * ppr;
+    for (uint32_t p = (uint32_t)tid; p < n_pieces; p += kBlock) {
+        const uint32_t pr = p / ppr, off = (p - pr * ppr) * PIECE;
+        uint8_t* dst = pool + (size_t)row_s[pr] * row_bytes + off;
+        if (PIECE == 16)
+            st_stream(dst, *reinterpret_cast<const v4u*>(image + pr * row_bytes + off));
+        else
+            *reinterpret_cast<uint32_t*>(dst) = *reinterpret_cast<const uint32_t*>(image + pr * row_bytes + off);
+    }
 }
 
 // ---- append, quantised rows -----------------------------------------------------------
@@ -256,15 +265,9 @@ __global__ __launch_bounds__(kBlock) void append_quant_kernel(AppendBatch b, Mov
     constexpr bool kSrcF16 = std::is_same<SrcT, uint16_t>::value;
     if (LAYOUT == BKV_LAYOUT_Q8V) {
         if (active) st_stream(reinterpret_cast<uint16_t*>(kpool) + row * (size_t)hd + (size_t)li * 8, ko);
-        float amax = quad_max(amax8(vx));
-        float scale = q8v_scale(amax);
-        uint32_t w0, w1, doubt = (kSrcF16 && !(amax > 0x1p-6f)) ? 0x7fc00000u : 0u;
-        codes8_on_reciprocal(vx, scale, w0, w1, doubt);
-        if (__any(codes_in_doubt(doubt))) {  // the rule as written, for the whole wave
-            flush8<SrcT>(vx);
-            scale = q8v_scale(quad_max(amax8(vx)));
-            q8_codes8(vx, scale, w0, w1);
-        }
+        float scale;
+        uint32_t w0, w1;
+        q8v_quarter<SrcT>(vx, scale, w0, w1);
         if (active) {
             uint32_t* blk_words = reinterpret_cast<uint32_t*>(v_image + rl * row_bytes + blk * 36);
             if (quarter == 0) blk_words[0] = __float_as_uint(scale);
@@ -309,23 +312,9 @@ __global__ __launch_bounds__(kBlock) void append_quant_kernel(AppendBatch b, Mov
         }
     }
     __syncthreads();
-    // whole rows out: piece p of the work-group's image goes to the same offset of its pool row
     constexpr uint32_t kPiece = HD == 256 ? 16u : 4u;
-    const uint32_t ppr = row_bytes / kPiece;  // pieces of a row
-    const uint32_t n_pieces = (uint32_t)nrows * ppr;
-    const int n_images = LAYOUT == BKV_LAYOUT_I8H ? 2 : 1;
-    for (int im = 0; im < n_images; ++im) {
-        const uint8_t* src_image = im ? v_image : image;
-        uint8_t* pool = (LAYOUT == BKV_LAYOUT_I8H && im == 0) ? kpool : vpool;
-        for (uint32_t p = (uint32_t)tid; p < n_pieces; p += kBlock) {
-            const uint32_t pr = p / ppr, off = (p - pr * ppr) * kPiece;
-            uint8_t* dst = pool + (size_t)row_s[pr] * row_bytes + off;
-            if (kPiece == 16)
-                st_stream(dst, *reinterpret_cast<const v4u*>(src_image + pr * row_bytes + off));
-            else
-                *reinterpret_cast<uint32_t*>(dst) = *reinterpret_cast<const uint32_t*>(src_image + pr * row_bytes + off);
-        }
-    }
+    if (LAYOUT == BKV_LAYOUT_I8H) image_rows_out<kPiece>(image, kpool, row_s, nrows, row_bytes, tid);
+    image_rows_out<kPiece>(v_image, vpool, row_s, nrows, row_bytes, tid);
 }
 
 // ---- K preparation fused into the append ------------------------------------------
@@ -439,20 +428,11 @@ __global__ __launch_bounds__(kBlock) void append_kprep_kernel(AppendBatch b, Mov
     __syncthreads();
 
     const auto pool_row = [&](int row) -> size_t { return (size_t)row_s[row]; };
-    const int blocks = hd / 32;
+    const int lpr = hd / 8;  // 8-value groups of a row
 
-    // K from LDS
-    if (LAYOUT == BKV_LAYOUT_I8H) {
-        const size_t row_bytes = (size_t)hd + (size_t)blocks * 2;
-        for (int idx = tid; idx < nrows * blocks; idx += kBlock) {
-            const int row = idx / blocks, blk = idx % blocks;
-            float x[32];
-#pragma unroll
-            for (int i = 0; i < 32; ++i) x[i] = prep_lds[row * stride + blk * 32 + i];
-            i8h_encode(x, kpool + pool_row(row) * row_bytes, hd, blk);
-        }
-    } else {
-        for (int idx = tid; idx < nrows * hd / 8; idx += kBlock) {
+    if (LAYOUT == BKV_LAYOUT_F16) {
+        // K from LDS, V straight from the source rows
+        for (int idx = tid; idx < nrows * lpr; idx += kBlock) {
             const int row = (idx * 8) / hd, col = (idx * 8) % hd;
             const float* x = prep_lds + row * stride + col;
             v4u o;
@@ -461,35 +441,63 @@ __global__ __launch_bounds__(kBlock) void append_kprep_kernel(AppendBatch b, Mov
             o.z = pack2(x[4], x[5]);
             o.w = pack2(x[6], x[7]);
             st_stream(reinterpret_cast<uint16_t*>(kpool) + pool_row(row) * (size_t)hd + col, o);
-        }
-    }
-
-    // V straight from the source rows
-    if (LAYOUT == BKV_LAYOUT_F16) {
-        for (int idx = tid; idx < nrows * hd / 8; idx += kBlock) {
-            const int row = (idx * 8) / hd, col = (idx * 8) % hd;
-            float x[8];
-            load8(v + src_base + (size_t)idx * 8, x);
-            v4u o;
-            o.x = pack2(x[0], x[1]);
-            o.y = pack2(x[2], x[3]);
-            o.z = pack2(x[4], x[5]);
-            o.w = pack2(x[6], x[7]);
+            float y[8];
+            load8(v + src_base + (size_t)idx * 8, y);
+            o.x = pack2(y[0], y[1]);
+            o.y = pack2(y[2], y[3]);
+            o.z = pack2(y[4], y[5]);
+            o.w = pack2(y[6], y[7]);
             st_stream(reinterpret_cast<uint16_t*>(vpool) + pool_row(row) * (size_t)hd + col, o);
         }
-    } else {
-        const size_t row_bytes = (size_t)hd + (size_t)blocks * 2;
-        for (int idx = tid; idx < nrows * blocks; idx += kBlock) {
-            const int row = idx / blocks, blk = idx % blocks;
-            float x[32];
-            load32(v + src_base + (size_t)idx * 32, x);
-            if (LAYOUT == BKV_LAYOUT_Q8V)
-                q8v_encode(x, reinterpret_cast<uint32_t*>(vpool) +
-                                  (pool_row(row) * (size_t)blocks + (size_t)blk) * 9u);
-            else
-                i8h_encode(x, vpool + pool_row(row) * row_bytes, hd, blk);
+        return;
+    }
+    // Quantised rows, as in append_quant_kernel: a lane encodes 8 consecutive values (the four lanes of a
+    // quad share a 32-value block: 8-value groups of a row are a multiple of four, so a quad is in or
+    // out of the loop as a whole), the rows are put together in LDS and leave whole.
+    __shared__ __attribute__((aligned(16))) uint8_t image[2 * kPrepRows * 288];
+    const int blocks = hd / 32;
+    const uint32_t row_bytes = LAYOUT == BKV_LAYOUT_Q8V ? (uint32_t)blocks * 36u : (uint32_t)hd + (uint32_t)blocks * 2u;
+    uint8_t* const v_image = image + (LAYOUT == BKV_LAYOUT_I8H ? kPrepRows * row_bytes : 0u);
+    for (int idx = tid; idx < nrows * lpr; idx += kBlock) {
+        const int row = idx / lpr, li = idx - row * lpr;
+        const int blk = li >> 2, quarter = li & 3;
+        const float* kxp = prep_lds + row * stride + li * 8;
+        const float4 ka = *reinterpret_cast<const float4*>(kxp), kb = *reinterpret_cast<const float4*>(kxp + 4);
+        float vx[8];
+        load8(v + src_base + (size_t)idx * 8, vx);
+        if (LAYOUT == BKV_LAYOUT_Q8V) {
+            v4u o;
+            o.x = pack2(ka.x, ka.y);
+            o.y = pack2(ka.z, ka.w);
+            o.z = pack2(kb.x, kb.y);
+            o.w = pack2(kb.z, kb.w);
+            st_stream(reinterpret_cast<uint16_t*>(kpool) + pool_row(row) * (size_t)hd + (size_t)li * 8, o);
+            float scale;
+            uint32_t w0, w1;
+            q8v_quarter<float>(vx, scale, w0, w1);
+            uint32_t* blk_words = reinterpret_cast<uint32_t*>(v_image + row * row_bytes + blk * 36);
+            if (quarter == 0) blk_words[0] = __float_as_uint(scale);
+            blk_words[1 + 2 * quarter] = w0;
+            blk_words[2 + 2 * quarter] = w1;
+        } else {
+            const float kx[8] = {ka.x, ka.y, ka.z, ka.w, kb.x, kb.y, kb.z, kb.w};
+            uint32_t ks, k0, k1, vs, v0, v1;
+            i8h_quarter(kx, ks, k0, k1);
+            i8h_quarter(vx, vs, v0, v1);
+            uint8_t* kr = image + row * row_bytes;
+            uint8_t* vr = v_image + row * row_bytes;
+            *reinterpret_cast<uint2*>(kr + li * 8) = make_uint2(k0, k1);
+            *reinterpret_cast<uint2*>(vr + li * 8) = make_uint2(v0, v1);
+            if (quarter == 0) {
+                *reinterpret_cast<uint16_t*>(kr + hd + blk * 2) = (uint16_t)ks;
+                *reinterpret_cast<uint16_t*>(vr + hd + blk * 2) = (uint16_t)vs;
+            }
         }
     }
+    __syncthreads();
+    constexpr uint32_t kPiece = HD == 256 ? 16u : 4u;
+    if (LAYOUT == BKV_LAYOUT_I8H) image_rows_out<kPiece>(image, kpool, row_s, nrows, row_bytes, tid);
+    image_rows_out<kPiece>(v_image, vpool, row_s, nrows, row_bytes, tid);
 }
 
 // ---- whole-page moves -----------------------------------------------------------

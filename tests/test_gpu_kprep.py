@@ -87,6 +87,45 @@ def test_decode_step_and_ragged_prefill_are_bit_exact(layout):
     prep.free()
 
 
+@pytest.mark.parametrize("layout", [L.LAYOUT_Q8V, L.LAYOUT_I8H])
+def test_bulk_quantised_rows_with_rounding_ties_are_bit_exact(layout):
+    # The quantised stores take their codes from a reciprocal of the scale where that provably gives
+    # the rule's round-half-away(clamp(x / scale)) (qsa/cpu.rs:65-82) and from the division elsewhere.
+    # 2000 tokens in one call; V rows pass through unprepared, so they can carry exact ties (scale 1
+    # and 1/4), values one ulp either side of a tie, tiny blocks, a zero block and a lone large value;
+    # the prepared K rows are whatever the normalisation makes of rows of very different magnitude.
+    rng = np.random.Generator(np.random.PCG64(500 + layout))
+    T = 2000
+    gamma = (1.0 + 0.3 * rng.standard_normal(HD)).astype(np.float32)
+    prep = Prep(gamma, max_pos=2048)
+    k = (rng.standard_normal((T, N_KV, HD)) * rng.uniform(1e-3, 300, size=(T, N_KV, 1))).astype(np.float32)
+    k[40, 0, :] = 0.0
+    k[41, 1, 5:] = 0.0
+    v = (rng.standard_normal((T, N_KV, HD)) * rng.uniform(0.05, 30, size=(T, N_KV, 1))).astype(np.float32)
+    halves = (np.arange(32, dtype=np.float32) * 7.0) % 126.0 + 0.5
+    halves[::2] *= -1.0
+    v[10, 0, 0:32] = halves
+    v[10, 0, 0] = 127.0
+    v[11, 1, 64:96] = halves / 4.0
+    v[11, 1, 64] = -127.0 / 4.0
+    v[12, 0, 32:64] = np.nextafter(halves, np.float32(1000.0))
+    v[12, 0, 32] = 127.0
+    v[13, 1, 32:64] = np.nextafter(halves, np.float32(-1000.0))
+    v[13, 1, 32] = 127.0
+    v[14, 0, 96:128] = rng.standard_normal(32).astype(np.float32) * 1e-3
+    v[15, 1, 0:32] = rng.standard_normal(32).astype(np.float32) * 1e-30
+    v[16, 0, 128:160] = 0.0
+    v[17, 1, 160:192] = 1e-4
+    v[17, 1, 161] = 5e4
+    with Twin(n_pages=T // 16 + 8, layout=layout, max_seqs=4) as tw:
+        tw.pool.set_free_order(rng.permutation(T // 16 + 8).astype(np.int32))
+        s = tw.pool.seq_create()
+        tw.pool.seq_reserve(s, T + 3)
+        fused_append(tw, prep, 0, [s], [3], [k], [v])
+        tw.assert_pools_equal()
+    prep.free()
+
+
 def test_fused_call_equals_the_unfused_chain_on_the_device():
     # bkv_append of the oracle-prepared K rows must land on the same bytes as the fused call
     rng = np.random.Generator(np.random.PCG64(41))
