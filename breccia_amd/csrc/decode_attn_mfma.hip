@@ -822,11 +822,12 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
 }
 
 // ---- decode attention on the matrix cores, f16 K and q8_0 V -----------------------------------
-// The MFMA decomposition of decode_attn_mfma_kernel with both operands staged through LDS like the
-// int8 kernel's units: the f16 K unit (8 KiB) and the V unit ([f32 scale][32 x i8] blocks, 288
-// bytes a row) of the next page are fetched into registers with coalesced loads while this page
-// is multiplied, and deposited into the wave's slot when the page is reached.  A q8_0 value is
-// code * scale with an f32 scale, so it takes a per-cell
+// The MFMA decomposition of decode_attn_mfma_kernel.  K is f16 and takes that kernel's way: whole
+// 128-byte lines straight into the fragment registers (k_pair_home), refilled with the next page's
+// as they are used up.  The V unit ([f32 scale][32 x i8] blocks, 288 bytes a row) is staged through
+// LDS like the int8 kernel's units: the next page's unit is fetched into registers with coalesced
+// loads while this page is multiplied, and deposited into the wave's slot when the page is reached.
+// A q8_0 value is code * scale with an f32 scale, so it takes a per-cell
 // power of two out first to stay inside f16:
 //   E[cell]  = exponent of the largest of the cell's 8 block scales (clamped to +-120),
 //   a[cell][d] = code * (scale * 2^-E[cell])       |a| < 256; split into hi + lo f16 as below,
@@ -840,25 +841,6 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
 // kernel.
 constexpr int kQ8vRow = row_bytes_of(kRowQ8);  // 288
 constexpr int kQ8vUnit = kPage * kQ8vRow;      // 4608
-
-// K unit in LDS: 8 instructions of 1024 bytes (two rows each), 32 bytes apart so that the rows a
-// fragment read touches spread over the banks.
-constexpr int kQ8vKStep = 1024 + 32;
-constexpr int kQ8vKSlot = 8 * kQ8vKStep;  // 8448
-// A K unit between memory and LDS: instruction n moves rows 2 n and 2 n + 1 (of a selection list,
-// half of block n / 2).
-template <bool SEL>
-__device__ __forceinline__ void q8v_k_unit_fetch(const UnitSrc<SEL>& src, int lane, v4u (&r)[8]) {
-#pragma unroll
-    for (int n = 0; n < 8; ++n) {
-        const uint8_t* a = SEL ? src.run[SEL ? n >> 1 : 0] + (n & 1) * 1024 + lane * 16 : src.run[0] + n * 1024 + lane * 16;
-        r[n] = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(a));
-    }
-}
-__device__ __forceinline__ void q8v_k_unit_deposit(const v4u (&r)[8], uint8_t* dst, int lane) {
-#pragma unroll
-    for (int n = 0; n < 8; ++n) *reinterpret_cast<v4u*>(dst + n * kQ8vKStep + lane * 16) = r[n];
-}
 
 // A V unit: 4608 bytes = 64 lanes x (4 x 16 + 8).
 struct Q8vUnitRegs {
@@ -883,8 +865,8 @@ __device__ __forceinline__ void q8v_unit_deposit(const Q8vUnitRegs& r, uint8_t* 
 template <bool STEP, bool DESC = false, bool SEL = false>
 __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const AttnKernelParams P) {
     static_assert(!(STEP && SEL), "the fused step attends the dense selection");
-    // per wave one K slot and one V slot during the loop, the fold staging after it
-    constexpr int kWaveLds = kQ8vKSlot + kQ8vUnit;
+    // per wave one V slot during the loop, the fold staging after it
+    constexpr int kWaveLds = kQ8vUnit;
     constexpr int kLds = kWaves * kWaveLds > (int)sizeof(MfmaFoldLds) ? kWaves * kWaveLds : (int)sizeof(MfmaFoldLds);
     __shared__ __attribute__((aligned(16))) uint8_t smem[kLds];
     // STEP: the new row of the entry, encoded (512 bytes of K, 288 of V); one wave of a work-group at most
@@ -915,8 +897,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
     const size_t k_head_off = (size_t)kvh * kPage * kHd * 2;
     const size_t v_page_bytes = (size_t)P.n_kv * kQ8vUnit;
     const size_t v_head_off = (size_t)kvh * kQ8vUnit;
-    uint8_t* const kslot = smem + wave * kWaveLds;
-    uint8_t* const slots = kslot + kQ8vKSlot;
+    uint8_t* const slots = smem + wave * kWaveLds;
 
     // pipeline steps of this wave: pages pg0 + wave, + kWaves, ...
     const int n_steps = pg0 + wave < pg1 ? (pg1 - pg0 - wave + kWaves - 1) / kWaves : 0;
@@ -942,17 +923,40 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
                                    : pool;
         }
     };
-    // the page in flight: requested while the page before is multiplied
-    v4u k_regs[8];
-    Q8vUnitRegs v_regs;
-    const auto fetch = [&](int i) {
-        UnitSrc<SEL> u;
-        unit_src(i, true, u);
-        q8v_k_unit_fetch<SEL>(u, lane, k_regs);
-        unit_src(i, false, u);
-        q8v_unit_fetch<SEL>(u, lane, v_regs);
+    // K rows are fetched in whole 128-byte lines, as in decode_attn_mfma_kernel: for the pair of fragments
+    // (2 p, 2 p + 1) one instruction reads rows 0..7 and one rows 8..15 of the page, eight lanes to a row
+    // (lane (c, g) takes segment g + 4 (c / 8) of row c % 8, or of row 8 + c % 8); k_pair_home puts the
+    // halves where their MFMAs read them.
+    const int c7 = c & 7;
+    const int kseg = g + 4 * (c >> 3);
+    const auto k_rows = [&](const UnitSrc<SEL>& u, const uint8_t*& lo, const uint8_t*& hi) {
+        if constexpr (SEL) {
+            // rows 4 j .. 4 j + 3 of the iteration are listed block j
+            const int at = (c7 & 3) * (kHd * 2) + kseg * 16;
+            lo = (c7 >> 2 ? u.run[1] : u.run[0]) + at;
+            hi = (c7 >> 2 ? u.run[3] : u.run[2]) + at;
+        } else {
+            lo = u.run[0] + c7 * (kHd * 2) + kseg * 16;
+            hi = lo + 8 * (kHd * 2);
+        }
     };
-    if (n_steps > 0) fetch(0);
+    // the page in flight: K in the fragment registers, refilled as they are used up; the V unit requested
+    // while the page before is multiplied
+    v4u kf[8];
+    Q8vUnitRegs v_regs;
+    if (n_steps > 0) {
+        UnitSrc<SEL> u;
+        const uint8_t *lo, *hi;
+        unit_src(0, true, u);
+        k_rows(u, lo, hi);
+#pragma unroll
+        for (int pp = 0; pp < 4; ++pp) {
+            kf[2 * pp] = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(lo + 128 * pp));
+            kf[2 * pp + 1] = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(hi + 128 * pp));
+        }
+        unit_src(0, false, u);
+        q8v_unit_fetch<SEL>(u, lane, v_regs);
+    }
 
     // STEP: the wave that will hold the page of cell pos (in its last step) encodes the new row before
     // the loop, while its first units are on their way, as the append kernel does -- K under the f16
@@ -1015,12 +1019,17 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
             wave_lds_fence();
         }
     }
+    // K registers hold rows as fetched: row r sits in the lanes with c % 8 == r % 8, in the register of
+    // rows 0..7 or of rows 8..15, segment g + 4 (c / 8) of each 128-byte line
     const auto take_new_k = [&]() {
         const int r = pos & (kPage - 1);
-        if (lane < 32)
-            *reinterpret_cast<v4u*>(kslot + (r >> 1) * kQ8vKStep + (r & 1) * 512 + lane * 16) =
-                *reinterpret_cast<const v4u*>(parked + lane * 16);
-        wave_lds_fence();
+#pragma unroll
+        for (int pp = 0; pp < 4; ++pp) {
+            const v4u w = *reinterpret_cast<const v4u*>(parked + (pp * 8 + kseg) * 16);
+            if (c7 == (r & 7)) {
+                if (r < 8) kf[2 * pp] = w; else kf[2 * pp + 1] = w;
+            }
+        }
     };
     const auto take_new_v = [&](uint8_t* lds_unit) {
         const int r = pos & (kPage - 1);
@@ -1042,11 +1051,19 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
     for (int i = 0; i < n_steps; ++i) {
         const int pg = pg0 + wave + kWaves * i;
         const uint8_t* vs = slots;
-        // this page's units arrive in the registers: into the slots with them, and the registers take
-        // the request for the next page
-        q8v_k_unit_deposit(k_regs, kslot, lane);
+        // this page's V unit arrives in the registers: into the slot with it, and the registers take the
+        // request for the next page's
         q8v_unit_deposit(v_regs, slots, lane);
-        if (i + 1 < n_steps) fetch(i + 1);
+        const bool more = i + 1 < n_steps;
+        const uint8_t* klo_next = nullptr;
+        const uint8_t* khi_next = nullptr;
+        if (more) {
+            UnitSrc<SEL> u;
+            unit_src(i + 1, false, u);
+            q8v_unit_fetch<SEL>(u, lane, v_regs);
+            unit_src(i + 1, true, u);
+            k_rows(u, klo_next, khi_next);
+        }
         wave_lds_fence();
         if constexpr (STEP) {
             if (pg == n_pages - 1) {
@@ -1071,23 +1088,19 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
         }
 
         // ---- S^T = K . q^T: four independent accumulation chains ------------------------------
-        v4u kf[8];
-        {
-            // row c: two rows per 1056-byte step; fragment m of lane group g at 64 m + 16 g
-            const uint8_t* kr = kslot + (c >> 1) * kQ8vKStep + (c & 1) * 512 + g * 16;
-#pragma unroll
-            for (int m = 0; m < 8; ++m) kf[m] = *reinterpret_cast<const v4u*>(kr + m * 64);
-        }
-        __builtin_amdgcn_sched_barrier(0);
         f4 s0 = f4{0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0, s2 = s0, s3 = s0;
 #pragma unroll
         for (int m = 0; m < 8; m += 2) {
-            const half8 ka = __builtin_bit_cast(half8, kf[m]);
-            const half8 kb = __builtin_bit_cast(half8, kf[m + 1]);
+            half8 ka, kb;
+            k_pair_home(kf[m], kf[m + 1], ka, kb);
             s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qhi[m], s0, 0, 0, 0);
             s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qlo[m], s1, 0, 0, 0);
             s2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kb, qhi[m + 1], s2, 0, 0, 0);
             s3 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kb, qlo[m + 1], s3, 0, 0, 0);
+            if (more) {
+                kf[m] = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(klo_next + 64 * m));
+                kf[m + 1] = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(khi_next + 64 * m));
+            }
         }
         const f4 s = (s0 + s1) + (s2 + s3);  // s[r] = q[head c] . k[cell 4 g + r]
 
