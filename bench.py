@@ -38,7 +38,7 @@ ROW_BYTES_I8H = N_KV * 2 * (HD // 32 * 34)        # 1088
 # HBM traffic of one launch of the split-K kernel on the default seeded workload, from
 # rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this file, each scaled by what the same counter
 # reads for the plain copy probe (profiles/hbm_traffic_all_kernels.md)
-MEASURED_TRAFFIC = {"seed": 20250003, "fetch_bytes": 328.36e6, "write_bytes": 4.19e6}
+MEASURED_TRAFFIC = {"seed": 20250003, "fetch_bytes": 329.24e6, "write_bytes": 4.23e6}
 APPEND_BYTES_PER_TOKEN = N_KV * HD * (4 + 2) * 2  # f32 in + f16 out, K and V = 6144
 
 
