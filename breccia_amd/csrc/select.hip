@@ -32,6 +32,8 @@ constexpr int kTopkThreads = 1024;
 constexpr int kMaxTopk = 2048;    // candidates the sort network holds in LDS
 constexpr int kHistCopies = 16;   // copies of the radix histogram (a power of two)
 constexpr int kRankKeys = 256;    // keys of a radix bin that are ranked directly instead of split further
+constexpr int kBuckets = kTopkThreads;  // buckets the selected keys are ordered through (one per thread)
+constexpr int kBucketCap = 64;    // a fuller bucket sends the list to the sorting network instead
 
 struct ScoreParams {
     SelectBatch b;
@@ -191,21 +193,36 @@ __global__ __launch_bounds__(256) void idx_tail_kernel(const float* __restrict__
 
 // ---- top-k ---------------------------------------------------------------------------
 // Keys: unsigned integers that order like the scores.  A score is dead (never selected)
-// unless it is greater than -1e29: that covers -inf, NaN and the reference shaders' own
-// dead marker -1e30 (shaders/qsa_topk.comp stops at the first best <= -1e29).  -0 is keyed
-// as +0 so that equal scores stay equal.  Live keys are never 0.
+// unless it is finite and greater than -1e29: that covers NaN, the infinities (the CPU path
+// keeps finite scores only, qsa/cpu.rs:139-143) and the reference shaders' own dead marker -1e30
+// (shaders/qsa_topk.comp stops at the first best <= -1e29).  -0 is keyed as +0 so that equal
+// scores stay equal.  Live keys are never 0.
 __device__ __forceinline__ uint64_t score_key(double s) {
-    if (!(s > -1.0e29)) return 0;
+    if (!(s > -1.0e29 && s < INFINITY)) return 0;
     if (s == 0.0) s = 0.0;
     const uint64_t u = (uint64_t)__double_as_longlong(s);
     return (u >> 63) ? ~u : (u | 0x8000000000000000ull);
 }
 __device__ __forceinline__ uint64_t score_key(float s) {
-    if (!(s > -1.0e29f)) return 0;
+    if (!(s > -1.0e29f && s < INFINITY)) return 0;
     if (s == 0.0f) s = 0.0f;
     const uint32_t u = __float_as_uint(s);
     const uint32_t k = (u >> 31) ? ~u : (u | 0x80000000u);
     return (uint64_t)k << 32;
+}
+// the score a live key stands for (-0 comes back as +0)
+template <typename T>
+__device__ __forceinline__ double key_score(uint64_t k);
+template <>
+__device__ __forceinline__ double key_score<double>(uint64_t k) {
+    const uint64_t u = (k >> 63) ? (k ^ 0x8000000000000000ull) : ~k;
+    return __longlong_as_double((long long)u);
+}
+template <>
+__device__ __forceinline__ double key_score<float>(uint64_t k) {
+    const uint32_t k32 = (uint32_t)(k >> 32);
+    const uint32_t u = (k32 >> 31) ? (k32 ^ 0x80000000u) : ~k32;
+    return (double)__uint_as_float(u);
 }
 template <typename T>
 struct KeyBits;
@@ -260,14 +277,16 @@ __global__ __launch_bounds__(kTopkThreads) void topk_blocks_kernel(const TopkPar
     // different banks.
     __shared__ int hist[kHistCopies][257];
     __shared__ int wave_sums[kTopkThreads / 64];
-    __shared__ uint64_t cand_key[kMaxTopk];
-    __shared__ uint32_t cand_idx[kMaxTopk];
+    __shared__ uint64_t cand_key[kMaxTopk + kBucketCap];  // the threshold slice may hold keys that are not kept
+    __shared__ uint32_t cand_idx[kMaxTopk + kBucketCap];
     __shared__ uint64_t wave_min[kTopkThreads / 64], wave_max[kTopkThreads / 64];
     __shared__ uint64_t sh_prefix;
     __shared__ int sh_rem, sh_done, sh_cnt;
     __shared__ uint64_t small_key[kRankKeys + 4];
     __shared__ int small_n;
-    __shared__ int sh_present;
+    __shared__ int sh_present, sh_crowded;
+    __shared__ int sh_placed;  // keys of the slices at and above the threshold slice
+    static_assert(3 * kBuckets <= kHistCopies * 257, "the bucket counters reuse the histogram");
 
     const int e = blockIdx.x;
     const int tid = threadIdx.x;
@@ -288,6 +307,7 @@ __global__ __launch_bounds__(kTopkThreads) void topk_blocks_kernel(const TopkPar
     }
 
     const T* sc = reinterpret_cast<const T*>(P.scores) + (size_t)e * P.score_stride;
+    if (tid == 0) sh_present = 0;  // read after the barriers of the scans below
     // thread t owns the contiguous index range [lo, hi): compaction keeps index order
     const int per = (N + kTopkThreads - 1) / kTopkThreads;
     const int lo = min(tid * per, N), hi = min(lo + per, N);
@@ -306,10 +326,35 @@ __global__ __launch_bounds__(kTopkThreads) void topk_blocks_kernel(const TopkPar
         }
     };
 
+    // live keys, the smallest and the largest of them: one sweep, one wave reduction each, one barrier
     int live = 0;
-    for_keys([&](int, uint64_t k) { live += k != 0; });
-    int n_live;
-    block_exclusive_scan(live, wave_sums, &n_live);
+    uint64_t kmin = ~0ull, kmax = 0;
+    for_keys([&](int, uint64_t k) {
+        if (k != 0) {
+            ++live;
+            kmin = min(kmin, k);
+            kmax = max(kmax, k);
+        }
+    });
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        live += __shfl_xor(live, off, 64);
+        kmin = min(kmin, (uint64_t)__shfl_xor((unsigned long long)kmin, off, 64));
+        kmax = max(kmax, (uint64_t)__shfl_xor((unsigned long long)kmax, off, 64));
+    }
+    if ((tid & 63) == 0) {
+        wave_sums[tid >> 6] = live;
+        wave_min[tid >> 6] = kmin;
+        wave_max[tid >> 6] = kmax;
+    }
+    if (tid == 0) sh_done = 0;
+    __syncthreads();
+    int n_live = 0;
+    for (int w = 0; w < kTopkThreads / 64; ++w) {
+        n_live += wave_sums[w];
+        kmin = min(kmin, wave_min[w]);
+        kmax = max(kmax, wave_max[w]);
+    }
     const int want = min(min(min(N, P.topk_blocks), n_live), P.max_ids);
 
     if (want > 0) {
@@ -318,28 +363,86 @@ __global__ __launch_bounds__(kTopkThreads) void topk_blocks_kernel(const TopkPar
         // largest differ (for scores of similar magnitude that is sign, exponent and more), so
         // the digits start there: the first histogram is already well spread, and the LDS
         // atomics do not pile up on one bin.
-        uint64_t kmin = ~0ull, kmax = 0;
-        for_keys([&](int, uint64_t k) {
-            if (k != 0) {
-                kmin = min(kmin, k);
-                kmax = max(kmax, k);
+        // ---- the usual case: one histogram over equal slices of the score range --------------------
+        // Slice = floor((score - least) * kBuckets / (greatest - least)), which never decreases when the
+        // score grows (a rounded difference, a rounded product and a truncation are all monotone) and is
+        // the same for equal scores.  The counts are summed from the top slice down: the slice in which
+        // the sum reaches `want` holds the threshold, every slice above it is selected whole, and a
+        // slice's keys own a run of output places.  Every key of those slices is ranked against the
+        // others of its slice -- greater keys first, equal keys in index order -- which is the place it
+        // is written to; in the threshold slice only ranks below the number still wanted are written.
+        // Selection, tie rule and order in one histogram and a handful of barriers.  Scores that crowd a
+        // slice (many equal scores, an outlier that stretches the range, a range too narrow or too wide
+        // to divide) take the general path below: a radix select on the keys' bits.
+        bool done = false;
+        {
+            int* const bcount = &hist[0][0];
+            int* const bfill = bcount + kBuckets;
+            int* const bbase = bfill + kBuckets;
+            const double least = key_score<T>(kmin);
+            const double inv_w = (double)kBuckets / (key_score<T>(kmax) - least);
+            if (kmin != kmax && inv_w > 0.0 && inv_w < 1.0e300) {
+                const auto slice_of = [&](uint64_t k) {
+                    return min(kBuckets - 1, (int)((key_score<T>(k) - least) * inv_w));
+                };
+                bcount[tid] = 0;
+                bfill[tid] = 0;
+                if (tid == 0) sh_crowded = 0;
+                __syncthreads();
+                for_keys([&](int, uint64_t k) {
+                    if (k != 0) atomicAdd(&bcount[slice_of(k)], 1);
+                });
+                __syncthreads();
+                const int sl_mine = kBuckets - 1 - tid;  // thread t sums from the top
+                const int in_mine = bcount[sl_mine];
+                int all;
+                const int above = block_exclusive_scan(in_mine, wave_sums, &all);
+                bbase[sl_mine] = above;
+                if (above < want) {
+                    if (in_mine > kBucketCap) sh_crowded = 1;
+                    if (above + in_mine >= want) {  // the threshold slice: exactly one thread
+                        sh_cnt = sl_mine;
+                        sh_placed = above + in_mine;
+                    }
+                }
+                __syncthreads();
+                if (!sh_crowded) {
+                    const int threshold_slice = sh_cnt;
+                    const int placed = sh_placed;
+                    for_keys([&](int i, uint64_t k) {
+                        if (k != 0) {
+                            const int b = slice_of(k);
+                            if (b >= threshold_slice) {
+                                const int slot = bbase[b] + atomicAdd(&bfill[b], 1);
+                                cand_key[slot] = k;
+                                cand_idx[slot] = (uint32_t)i;
+                            }
+                        }
+                    });
+                    __syncthreads();
+                    bool mine = false;
+                    for (int sl = tid; sl < placed; sl += kTopkThreads) {
+                        const uint64_t k = cand_key[sl];
+                        const uint32_t i = cand_idx[sl];
+                        const int b = slice_of(k);
+                        const int first = bbase[b], n = bcount[b];
+                        int rank = first;
+                        for (int j = 0; j < n; ++j) {
+                            const uint64_t kj = cand_key[first + j];
+                            const uint32_t ij = cand_idx[first + j];
+                            rank += kj > k || (kj == k && ij < i);
+                        }
+                        if (rank < want) {
+                            ids[rank] = i;
+                            mine = mine || i == own;
+                        }
+                    }
+                    if (mine) sh_present = 1;
+                    done = true;
+                }
             }
-        });
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            kmin = min(kmin, (uint64_t)__shfl_xor((unsigned long long)kmin, off, 64));
-            kmax = max(kmax, (uint64_t)__shfl_xor((unsigned long long)kmax, off, 64));
         }
-        if ((tid & 63) == 0) {
-            wave_min[tid >> 6] = kmin;
-            wave_max[tid >> 6] = kmax;
-        }
-        if (tid == 0) sh_done = 0;
-        __syncthreads();
-        for (int w = 0; w < kTopkThreads / 64; ++w) {
-            kmin = min(kmin, wave_min[w]);
-            kmax = max(kmax, wave_max[w]);
-        }
+        if (!done) {
         uint64_t kth = kmax;    // keys greater than kth are selected ...
         int ties_wanted = want; // ... and the first ties_wanted (by index) of those equal to it
         if (kmin != kmax) {
@@ -445,7 +548,7 @@ __global__ __launch_bounds__(kTopkThreads) void topk_blocks_kernel(const TopkPar
             }
         }
 
-        // ---- compaction in index order ---------------------------------------------------
+        // ---- order: descending key, ascending index among equal keys -------------------------
         int ties = 0, greater = 0;
         for_keys([&](int, uint64_t k) {
             ties += k == kth;
@@ -453,6 +556,80 @@ __global__ __launch_bounds__(kTopkThreads) void topk_blocks_kernel(const TopkPar
         });
         int total;
         const int ties_before = block_exclusive_scan(ties, wave_sums, &total);
+        // The keys equal to the threshold are the smallest selected ones and go last, in index order:
+        // their places follow from the scan above.  The n_g keys above the threshold are ordered through
+        // buckets: kBuckets equal slices of the key range (kth, kmax], counted, the counts summed from the
+        // top -- a bucket's keys then own a run of output places -- and every key ranked against the few
+        // others of its bucket.  A handful of barriers instead of a sorting network's stages.  Key ranges
+        // that crowd one bucket (an outlier far above the rest, many equal scores, a selection that spans
+        // both signs) go through the network below.
+        const int n_g = want - ties_wanted;
+        bool ordered = false;
+        {
+            int* const bcount = &hist[0][0];
+            int* const bfill = bcount + kBuckets;
+            int* const bbase = bfill + kBuckets;
+            int sh = 0;
+            if (n_g > 0) {
+                const uint64_t span = kmax - kth - 1;  // some key lies above kth, so kmax does
+                const int bits = span ? 64 - __builtin_clzll(span) : 0;
+                sh = bits > 10 ? bits - 10 : 0;
+            }
+            const auto bucket_of = [&](uint64_t k) { return (int)((k - kth - 1) >> sh); };
+            bcount[tid] = 0;
+            bfill[tid] = 0;
+            if (tid == 0) sh_crowded = 0;
+            __syncthreads();
+            for_keys([&](int, uint64_t k) {
+                if (k > kth) atomicAdd(&bcount[bucket_of(k)], 1);
+            });
+            __syncthreads();
+            const int in_mine = bcount[kBuckets - 1 - tid];  // thread t sums from the top: bucket kBuckets - 1 - t
+            if (in_mine > kBucketCap) sh_crowded = 1;
+            int placed;
+            bbase[kBuckets - 1 - tid] = block_exclusive_scan(in_mine, wave_sums, &placed);
+            __syncthreads();
+            if (!sh_crowded) {
+                for_keys([&](int i, uint64_t k) {
+                    if (k > kth) {
+                        const int b = bucket_of(k);
+                        const int slot = bbase[b] + atomicAdd(&bfill[b], 1);
+                        cand_key[slot] = k;
+                        cand_idx[slot] = (uint32_t)i;
+                    }
+                });
+                __syncthreads();
+                bool mine = false;
+                for (int sl = tid; sl < n_g; sl += kTopkThreads) {
+                    const uint64_t k = cand_key[sl];
+                    const uint32_t i = cand_idx[sl];
+                    const int b = bucket_of(k);
+                    const int first = bbase[b], n = bcount[b];
+                    int rank = 0;
+                    for (int j = 0; j < n; ++j) {
+                        const uint64_t kj = cand_key[first + j];
+                        const uint32_t ij = cand_idx[first + j];
+                        rank += kj > k || (kj == k && ij < i);
+                    }
+                    ids[first + rank] = i;
+                    mine = mine || i == own;
+                }
+                int tie_rank = ties_before;
+                for_keys([&](int i, uint64_t k) {
+                    if (k == kth) {
+                        if (tie_rank < ties_wanted) {
+                            ids[n_g + tie_rank] = (uint32_t)i;
+                            mine = mine || (uint32_t)i == own;
+                        }
+                        ++tie_rank;
+                    }
+                });
+                if (mine) sh_present = 1;
+                ordered = true;
+            }
+        }
+        if (!ordered) {
+        // ---- compaction in index order, then a sorting network ---------------------------------
         const int take = max(0, min(ties, ties_wanted - ties_before));
         int at = block_exclusive_scan(greater + take, wave_sums, &total);
         int tie_rank = ties_before;
@@ -545,18 +722,18 @@ __global__ __launch_bounds__(kTopkThreads) void topk_blocks_kernel(const TopkPar
         }
         }
         __syncthreads();
+        bool mine = false;
+        for (int i = tid; i < want; i += kTopkThreads) {
+            const uint32_t id = cand_idx[i];
+            ids[i] = id;
+            mine = mine || id == own;
+        }
+        if (mine) sh_present = 1;
+        }
+        }
     }
 
-    // ---- emit, then the query's own block when the selection missed it ---------------------
-    if (tid == 0) sh_present = 0;
-    __syncthreads();
-    bool mine = false;
-    for (int i = tid; i < want; i += kTopkThreads) {
-        const uint32_t id = cand_idx[i];
-        ids[i] = id;
-        mine = mine || id == own;
-    }
-    if (mine) sh_present = 1;
+    // ---- the query's own block when the selection missed it ------------------------------------
     __syncthreads();
     if (tid == 0) {
         uint32_t count = (uint32_t)want;

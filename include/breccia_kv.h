@@ -448,8 +448,9 @@ bkv_status bkv_idx_pool(bkv_pool *pool, float *pooled_dev, int32_t max_blocks, f
                         float eps, const float *rope_table_dev, int32_t n_rot, int32_t max_pos,
                         int32_t idx_dim, void *stream);
 /* The top-k alone over f32 scores the caller already holds: Qsa::topk / Qsa::topk_dense on
- * ws.idx_scores [n][n_blocks] (qsa/mod.rs:1264-1376).  A score is live iff it is greater than
- * -1e29 (the shaders' dead marker is -1e30; -inf and NaN are dead too).  The scores are not
+ * ws.idx_scores [n][n_blocks] (qsa/mod.rs:1264-1376).  A score is live iff it is finite and
+ * greater than -1e29 (the shaders' dead marker is -1e30; NaN and both infinities are dead, as
+ * in the CPU path's filter, qsa/cpu.rs:139-143).  The scores are not
  * modified (the reference's serial kernel destroys them).  dense != 0: no scores read, every
  * visible block 0..min(n_blocks, own+1) in ascending order, then the own block if it lies
  * beyond n_blocks. */

@@ -109,6 +109,46 @@ def test_topk_edge_cases():
         assert list(d[2]) == list(range(515))
 
 
+def test_topk_orders_through_buckets_and_through_the_sorting_network():
+    # The kernel selects and orders through one histogram over equal slices of the score range when the
+    # slices at and above the threshold are thinly filled; otherwise by a radix select on the key bits,
+    # then slices of the selected keys' range or, when those are crowded too, a sorting network.  Smooth
+    # scores (thin slices), one outlier far above the rest (every other key in the lowest slice), 200
+    # equal scores above the threshold, a threshold inside a run of equal scores, denormal scores, an
+    # outlier far below (a stretched range, but a tight one among the selected), infinities, a selection
+    # that spans both signs, and lists whose keys are re-read from memory on every pass.
+    rng = np.random.Generator(np.random.PCG64(701))
+    n, k = 5003, 512
+    smooth = rng.standard_normal(n).astype(np.float32)
+    outlier = smooth.copy()
+    outlier[1234] = 1e30
+    both_signs = smooth.copy()
+    many_equal = smooth.copy()
+    many_equal[rng.permutation(n)[:200]] = 2.5
+    run_at_threshold = smooth.copy()
+    order = np.argsort(-smooth, kind="stable")
+    run_at_threshold[order[480:560]] = smooth[order[480]]          # 80 equal scores around rank 512
+    tiny = (rng.standard_normal(n) * 1e-42).astype(np.float32)     # denormal scores of both signs
+    low_outlier = smooth.copy()
+    low_outlier[77] = -1e25                                        # live, and far below: stretches the range
+    with_inf = smooth.copy()
+    with_inf[[5, 4000]] = np.inf                                   # never selected (qsa/cpu.rs:139-143)
+    with_inf[6] = 3.0e38                                           # live: the range overflows f32, not f64
+    rows = [smooth, outlier, many_equal, run_at_threshold, tiny, low_outlier, with_inf]
+    pos = [int(p) for p in rng.integers(0, 4 * n, size=len(rows))]
+    with Pool(n_pages=4, max_seqs=2) as pool:
+        got = gpu_topk(pool, np.stack(rows), pos, k, k + 1)
+        for i, row in enumerate(rows):
+            assert np.array_equal(got[i], oracle_topk_f32(row, k, pos[i] // 4, k + 1)), i
+        got = gpu_topk(pool, both_signs[None, :], [0], 2048, 2049)  # below and above zero
+        assert np.array_equal(got[0], oracle_topk_f32(both_signs, 2048, 0, 2049))
+        big = rng.standard_normal((2, 30011)).astype(np.float32)    # keys re-read from memory per pass
+        big[1, ::7] = 0.125
+        got = gpu_topk(pool, big, [5, 4 * 30011], 2000, 2001)
+        for i, p in enumerate([5, 4 * 30011]):
+            assert np.array_equal(got[i], oracle_topk_f32(big[i], 2000, p // 4, 2001)), i
+
+
 def gpu_select(pool, pos, idx_q, pooled_list, topk, max_ids):
     n = len(pos)
     qd = DeviceBuffer.from_numpy(np.ascontiguousarray(idx_q, dtype=np.float32))
