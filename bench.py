@@ -264,7 +264,7 @@ def main() -> int:
         return 2
 
     from breccia_amd import lib as L
-    from breccia_amd.kv import DeviceBuffer, Stream, device_info, device_sync
+    from breccia_amd.kv import DeviceBuffer, Stream, device_info, device_sync, wait_options
 
     dev_name, n_cu, mem = device_info()
     stream = Stream()
@@ -387,6 +387,9 @@ def main() -> int:
                                "frac_of_hbm_peak_min_max": [round(step_bytes / (max(region_ms) * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
                                                             round(step_bytes / (min(region_ms) * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)]},
              "preheat_ms": round(pre_ms, 1), "preheat_steps": pre_steps,
+             "host_wait": {"timed_regions_end_with": "bkv_stream_sync of the bench library: it polls hipStreamQuery "
+                                                     "(with a pause instruction) for up to 4 ms before it blocks",
+                           "product_wait_options_ms_us": list(wait_options())},
              "contexts": ctx, "pool_pages": pool.desc.n_pages, "device": dev_name, "cus": n_cu,
              "oracle_check_max_abs": checked}
     pool.destroy()
