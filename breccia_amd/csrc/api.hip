@@ -1318,15 +1318,18 @@ bkv_status bkv_prefill_attn(bkv_pool* p, int32_t layer, int32_t n_seqs, const in
         b.pos0[i] = (int32_t)pos0[i];
         b.n_tok[i] = n_tokens[i];
         b.src0[i] = (int32_t)total;
-        b.wg_base[i] = (int32_t)wgs;
         total += n_tokens[i];
-        const int64_t rows = (int64_t)n_tokens[i] * group;
-        const int64_t rows_per_wg = prefill_rows_per_wg(p->g.layout);
-        wgs += (rows + rows_per_wg - 1) / rows_per_wg * p->g.n_kv;
+        wgs += ((int64_t)n_tokens[i] * group + 63) / 64 * p->g.n_kv;  // as 64-row work-groups
         if (total > ((int64_t)1 << 24) || wgs > ((int64_t)1 << 30))
             return fail(BKV_ERR_INVALID, "prefill_attn: more than 2^24 tokens in one call");
     }
     b.n = n_seqs;
+    const int64_t rows_per_wg = prefill_rows_per_wg(p->g.layout, wgs, p->n_cu);
+    wgs = 0;
+    for (int i = 0; i < n_seqs; ++i) {
+        b.wg_base[i] = (int32_t)wgs;
+        wgs += ((int64_t)n_tokens[i] * group + rows_per_wg - 1) / rows_per_wg * p->g.n_kv;
+    }
     b.wg_base[n_seqs] = (int32_t)wgs;
     bkv_status st = need_device(p);
     if (st != BKV_OK) return st;
@@ -1344,7 +1347,7 @@ bkv_status bkv_prefill_attn(bkv_pool* p, int32_t layer, int32_t n_seqs, const in
     a.gate_head_stride = gate_head_stride;
     a.scale = scale;
     a.out = out_dev;
-    BKV_HIP(launch_prefill_attn(p, layer, b, a, S(stream)));
+    BKV_HIP(launch_prefill_attn(p, layer, b, a, (int32_t)rows_per_wg, S(stream)));
     return BKV_OK;
 }
 

@@ -254,9 +254,10 @@ struct PrefillBatch {
     int32_t src0[BKV_MAX_BATCH];    // first token row in q / out
     int32_t wg_base[BKV_MAX_BATCH + 1];
 };
-int32_t prefill_rows_per_wg(int32_t layout);  // query rows one work-group owns
+// query rows one work-group owns, given how many 64-row work-groups the call's chunks would make
+int32_t prefill_rows_per_wg(int32_t layout, int64_t wgs_of_64_rows, int32_t n_cu);
 hipError_t launch_prefill_attn(bkv_pool* p, int32_t layer, const PrefillBatch& b, const AttnArgs& a,
-                               hipStream_t stream);
+                               int32_t rows_per_wg, hipStream_t stream);
 
 hipError_t launch_page_copy(bkv_pool* p, const bkv_page_pair* pairs_dev, int32_t n_pairs,
                             hipStream_t stream);

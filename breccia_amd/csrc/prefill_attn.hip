@@ -105,7 +105,7 @@ template <int LAY>
 struct PageStage;
 template <>
 struct PageStage<BKV_LAYOUT_F16> {
-    v4u k[2], v[2];  // chunks tid and tid + 256 of either image
+    v4u k[2], v[2];  // chunks tid (and, in a work-group of 256 threads, tid + 256) of either image
     int pg;
 };
 // the quantised layouts: thread tid owns row tid / 32, block tid / 4 % 8, codes 8 (tid % 4) .. + 7 of it
@@ -131,13 +131,16 @@ struct PrefillLds {
     float e[LAY == BKV_LAYOUT_Q8V ? 4 : 1][kPage];  // q8_0 V: E of the buffer's cells
 };
 
-template <int LAY>
-__global__ __launch_bounds__(LAY == BKV_LAYOUT_F16 ? 256 : 512, LAY == BKV_LAYOUT_F16 ? 2 : 1) void prefill_attn_kernel(
-    const PrefillKernelParams P) {
+// WAVES: waves of a work-group, 16 query rows each.  Eight share every page image they put into LDS
+// among 128 rows (one work-group per compute unit); four (f16 pools only, two work-groups per
+// compute unit) spread a small chunk over twice as many compute units.
+template <int LAY, int WAVES = 8>
+__global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_attn_kernel(const PrefillKernelParams P) {
+    static_assert(WAVES == 8 || (WAVES == 4 && LAY == BKV_LAYOUT_F16), "the quantised images are dequantised by 512 threads");
     constexpr bool Q8V = LAY == BKV_LAYOUT_Q8V;
     constexpr bool I8H = LAY == BKV_LAYOUT_I8H;
-    constexpr bool WIDE = LAY != BKV_LAYOUT_F16;  // eight waves, V as two f16 images
-    constexpr int kWavesPerWg = WIDE ? 8 : 4;
+    constexpr bool WIDE = LAY != BKV_LAYOUT_F16;  // V (int8 pools: K too) as two f16 images
+    constexpr int kWavesPerWg = WAVES;
     constexpr int kThreads = 64 * kWavesPerWg;
     constexpr int kRowsPerWg = kRowsPerWave * kWavesPerWg;
     // ---- which (entry, kv head, block of 64 query rows) ---------------------------------
@@ -285,7 +288,7 @@ __global__ __launch_bounds__(LAY == BKV_LAYOUT_F16 ? 256 : 512, LAY == BKV_LAYOU
             st.pg = pg;
         } else {
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
+            for (int j = 0; j < 512 / kThreads; ++j) {
                 st.k[j] = *reinterpret_cast<const v4u*>(kp + (size_t)(tid + j * kThreads) * 16);
                 st.v[j] = *reinterpret_cast<const v4u*>(vp + (size_t)(tid + j * kThreads) * 16);
             }
@@ -362,7 +365,7 @@ __global__ __launch_bounds__(LAY == BKV_LAYOUT_F16 ? 256 : 512, LAY == BKV_LAYOU
             // work-group's last page has such rows.
             const bool last_page = st.pg * kPage + kPage - 1 > wg_pos_max;
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
+            for (int j = 0; j < 512 / kThreads; ++j) {
                 const int q = tid + j * kThreads;
                 v4u vv = st.v[j];
                 if (last_page && st.pg * kPage + (q >> 5) > wg_pos_max) vv = v4u{0u, 0u, 0u, 0u};
@@ -568,10 +571,16 @@ __global__ __launch_bounds__(LAY == BKV_LAYOUT_F16 ? 256 : 512, LAY == BKV_LAYOU
 
 }  // namespace
 
-int32_t prefill_rows_per_wg(int32_t layout) { return kRowsPerWave * (layout == BKV_LAYOUT_F16 ? 4 : 8); }
+// Query rows one work-group owns.  f16 pools: 128 when the chunks make more 64-row work-groups than
+// fit the chip at two per compute unit (then sharing the page images among more rows is worth more
+// than spreading out), else 64.
+int32_t prefill_rows_per_wg(int32_t layout, int64_t wgs_of_64_rows, int32_t n_cu) {
+    if (layout != BKV_LAYOUT_F16) return 8 * kRowsPerWave;
+    return wgs_of_64_rows > 2 * (int64_t)(n_cu > 0 ? n_cu : 256) ? 8 * kRowsPerWave : 4 * kRowsPerWave;
+}
 
 hipError_t launch_prefill_attn(bkv_pool* p, int32_t layer, const PrefillBatch& b, const AttnArgs& a,
-                               hipStream_t stream) {
+                               int32_t rows_per_wg, hipStream_t stream) {
     PrefillKernelParams kp;
     kp.b = b;
     kp.kpool = p->k_layer[(size_t)layer];
@@ -593,7 +602,6 @@ hipError_t launch_prefill_attn(bkv_pool* p, int32_t layer, const PrefillBatch& b
     // longest die's share, and work-groups past a shorter die's share leave at once.
     kp.by_xcd = 0;
     {
-        const int rows_per_wg = prefill_rows_per_wg(p->g.layout);
         const int units = b.n * p->g.n_kv;
         int64_t longest = 0;
         if (units >= kXcds) {
@@ -620,8 +628,11 @@ hipError_t launch_prefill_attn(bkv_pool* p, int32_t layer, const PrefillBatch& b
     else if (p->g.layout == BKV_LAYOUT_I8H)
         launch_staged(p, BKV_STAGE_PREFILL_ATTN, prefill_attn_kernel<BKV_LAYOUT_I8H>, dim3((unsigned)grid), dim3(512), 0,
                       stream, kp);
+    else if (rows_per_wg == 8 * kRowsPerWave)
+        launch_staged(p, BKV_STAGE_PREFILL_ATTN, prefill_attn_kernel<BKV_LAYOUT_F16, 8>, dim3((unsigned)grid), dim3(512), 0,
+                      stream, kp);
     else
-        launch_staged(p, BKV_STAGE_PREFILL_ATTN, prefill_attn_kernel<BKV_LAYOUT_F16>, dim3((unsigned)grid), dim3(256), 0,
+        launch_staged(p, BKV_STAGE_PREFILL_ATTN, prefill_attn_kernel<BKV_LAYOUT_F16, 4>, dim3((unsigned)grid), dim3(256), 0,
                       stream, kp);
     return hipGetLastError();
 }
