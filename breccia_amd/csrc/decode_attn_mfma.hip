@@ -1154,7 +1154,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const float w = none_yet ? 0.0f : __builtin_amdgcn_exp2f(tw[r] - m_new);
-            psum += none_yet ? 0.0f : __builtin_amdgcn_exp2f(t4[r] - m_new);
+            psum = fmaf(w, down[r], psum);  // exp2(logit - m_new) = w * 2^-E: no second exponential
             _Float16 hi, lo;
             split_hi_lo(w, hi, lo);
             whi[r] = hi;
