@@ -209,3 +209,26 @@ def test_the_largest_batch_of_chunks_in_one_call(layout):
             tw.pool.prefill_attn(0, ent_seq + [seqs[0]], pos0 + [0], [1] * 65, 16, z, z, 0.0625)
         assert ei.value.status == L.ERR_INVALID
         z.free()
+
+
+def test_work_group_width_does_not_change_a_bit():
+    # On f16 pools a call whose chunks fill the chip runs work-groups of eight waves (128 query rows
+    # share each page image), a smaller one work-groups of four.  A wave's sixteen rows are computed
+    # the same way in both, so three chunks in one call (566 work-groups of 64 rows: eight waves) and
+    # the same chunks one call each (four waves) must agree in every bit; the oracle checks a sample.
+    rng = np.random.Generator(np.random.PCG64(1234))
+    cases = [(100, 700), (37, 650), (515, 900)]
+    with Twin(n_pages=200, max_seqs=4) as tw:
+        tw.pool.set_free_order(rng.permutation(200).astype(np.int32))
+        seqs = [tw.pool.seq_create() for _ in cases]
+        for s, (before, t) in zip(seqs, cases):
+            fill(tw, s, before + t, rng, chunk=1024)
+        qs = [rng.standard_normal((t, 16, 256)).astype(np.float32) for _, t in cases]
+        gates = [rng.standard_normal((t, 16, 256)).astype(np.float32) for _, t in cases]
+        together = prefill(tw, 0, seqs, [b for b, _ in cases], qs, 16, gates)
+        for i, (s, (before, t)) in enumerate(zip(seqs, cases)):
+            alone = prefill(tw, 0, [s], [before], [qs[i]], 16, [gates[i]])[0]
+            assert np.array_equal(alone.view(np.uint32), together[i].view(np.uint32)), i
+            for tok in (0, t - 1, int(rng.integers(0, t))):
+                want = tw.oracle_attend(0, s, before + tok, qs[i][tok], 16, gate=gates[i][tok])
+                check_attn(together[i][tok], want, "chunk %d, token %d" % (i, tok))
