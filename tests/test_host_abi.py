@@ -53,8 +53,9 @@ def test_wait_options_round_trip_and_reject_a_zero_deadline():
 
 
 def test_rust_binding_text_lists_every_declaration_with_its_argument_count():
-    """The Rust `extern "C"` block a maintainer would add (source only, no Rust
-    toolchain here) names every function of the header with as many arguments as the header gives it."""
+    """The Rust `extern "C"` block a maintainer would add (kept with the drop-in notes at the repository
+    root; source only, no Rust toolchain here) names every function of the header with as many arguments
+    as the header gives it."""
     doc = open(os.path.join(os.path.dirname(__file__), "..", "INTEGRATION.md")).read()
     rust = dict((m.group(1), m.group(2)) for m in re.finditer(r"pub fn (bkv_[a-z0-9_]+)\(([^;]*?)\)(?: -> [^;]+)?;", doc, re.S))
     text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
