@@ -32,9 +32,9 @@ struct MoveGeom {
     int32_t n_kv, hd, page_cells, max_pages_per_seq;
 };
 
-// Eight consecutive source values as f32.  Sources are f32 rows, or raw binary16 rows that
-// are widened under the cache's load rule (so an f16 source appends exactly what the f32
-// row of its widened values would).
+// Eight consecutive source values as f32.  Sources are f32 rows, or raw binary16 rows that are
+// read under the cache's load rule (so an f16 source appends exactly what the f32 row of its
+// widened values would): codes8(const uint16_t*) and load8_unflushed / flush8 below.
 __device__ __forceinline__ void load8(const float* p, float (&x)[8]) {
     const v4u a = ld_stream(p), b = ld_stream(p + 4);
     x[0] = __uint_as_float(a.x);
@@ -46,22 +46,6 @@ __device__ __forceinline__ void load8(const float* p, float (&x)[8]) {
     x[6] = __uint_as_float(b.z);
     x[7] = __uint_as_float(b.w);
 }
-// The load rule on the hardware convert: v_cvt_f32_f16 is exact (subnormals included), and a code
-// whose exponent field is 0 -- magnitude below 2^-14 -- reads as a signed zero.
-__device__ __forceinline__ float f16_widen(uint32_t h) {
-    const float x = (float)__builtin_bit_cast(_Float16, (uint16_t)h);
-    return fabsf(x) < 0x1p-14f ? __uint_as_float((h & 0x8000u) << 16) : x;
-}
-__device__ __forceinline__ void load8(const uint16_t* p, float (&x)[8]) {
-    const v4u a = ld_stream(p);
-    const unsigned w[4] = {a.x, a.y, a.z, a.w};
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        x[2 * i] = f16_widen(w[i] & 0xffffu);
-        x[2 * i + 1] = f16_widen(w[i] >> 16);
-    }
-}
-
 // For the quantising kernels: the values as the hardware converts them (subnormal codes keep
 // their value), and the load rule's flush as a separate step.  Where a block's amax is above 2^-6
 // the flush changes neither the amax nor a code (|x| < 2^-14 quantises to 0 against a scale above
