@@ -184,7 +184,9 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const uint32_t at = (uint32_t)i * 4u + (uint32_t)j;
-                const uint32_t id = sel[min(at, n_sel - 1u)];
+                // the slot is read whether or not the list reaches it (the buffer holds max_ids slots per
+                // entry): the read then does not wait for the list's length, one trip to memory less
+                const uint32_t id = sel[min(at, (uint32_t)P.max_ids - 1u)];
                 rr.id[j] = at < n_sel ? id : 0xffffffffu;
                 const uint32_t idc = min(id, (uint32_t)pos >> 2);
                 const size_t off = (size_t)bt[idc >> 2] * page_bytes + head_off + (size_t)(idc & 3u) * 4u * (kHd * 2);
@@ -225,7 +227,9 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_kernel(const AttnK
     int pg = pg0 + wave;
     v4u kf[8], vf[2][4];
     RowRuns<SEL> cur{};
-    if (pg < pg1) {
+    // a selection list's first rows are requested before its length is known (every address is clamped
+    // to the sequence's own blocks, so rows past the list's end are merely unused)
+    if (SEL || pg < pg1) {
         locate(pg, cur);
         const uint8_t* kp_lo = k_row_of(cur, c7);
         const uint8_t* kp_hi = k_row_of(cur, 8 + c7);
@@ -480,13 +484,15 @@ __device__ __forceinline__ const uint8_t* unit_piece(const UnitSrc<SEL>& u, int 
 // `page_bytes` long and whose rows are `row_bytes` long.
 typedef const __attribute__((address_space(4))) uint32_t* sel_list_ptr;
 typedef const __attribute__((address_space(4))) int32_t* block_table_ptr;
-__device__ __forceinline__ void listed_blocks(sel_list_ptr sel, uint32_t n_sel, block_table_ptr bt, int it, int pos,
-                                              size_t page_bytes, size_t head_off, int row_bytes, uint32_t (&id)[4],
-                                              size_t (&off)[4]) {
+__device__ __forceinline__ void listed_blocks(sel_list_ptr sel, uint32_t n_sel, uint32_t max_ids, block_table_ptr bt,
+                                              int it, int pos, size_t page_bytes, size_t head_off, int row_bytes,
+                                              uint32_t (&id)[4], size_t (&off)[4]) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const uint32_t at = (uint32_t)it * 4u + (uint32_t)j;
-        const uint32_t raw = sel[min(at, n_sel - 1u)];
+        // read whether or not the list reaches the slot (the buffer holds max_ids slots per entry): the
+        // read does not wait for the list's length
+        const uint32_t raw = sel[min(at, max_ids - 1u)];
         id[j] = at < n_sel ? raw : 0xffffffffu;
         const uint32_t idc = min(raw, (uint32_t)pos >> 2);
         off[j] = (size_t)bt[idc >> 2] * page_bytes + head_off + (size_t)(idc & 3u) * 4u * (size_t)row_bytes;
@@ -562,16 +568,13 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
     // the K and the V unit of step i (both pools have the same geometry in this layout)
     const auto unit_src = [&](int i, const uint8_t* pool, UnitSrc<SEL>& u) {
         if constexpr (SEL) {
-            if (i < n_steps) {
-                uint32_t id[4];
-                size_t off[4];
-                listed_blocks(sel, n_sel, bt, pg0 + wave + kWaves * i, pos, page_bytes, head_off, kRow, id, off);
+            // whatever the step, listed or past the list's end: every address is clamped to the sequence's
+            // own blocks, and nothing here waits for the list's length
+            uint32_t id[4];
+            size_t off[4];
+            listed_blocks(sel, n_sel, (uint32_t)P.max_ids, bt, pg0 + wave + kWaves * i, pos, page_bytes, head_off, kRow, id, off);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) u.run[j] = pool + off[j];
-            } else {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) u.run[j] = pool;
-            }
+            for (int j = 0; j < 4; ++j) u.run[j] = pool + off[j];
         } else {
             u.run[0] = pool + (n_steps > 0 ? unit_off(i) : 0);
         }
@@ -585,7 +588,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
         unit_src(i, P.vpool, u);
         i8h_unit_fetch<SEL>(u, lane, v_regs);
     };
-    if (n_steps > 0) fetch(0);
+    if (SEL || n_steps > 0) fetch(0);  // a selection list's first units before its length is known
 
     // STEP: the wave that will hold the page of cell pos (in its last step) takes the new rows before the
     // loop, while its first units are on their way: the raw values are requested ahead of the q fragments
@@ -674,7 +677,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_i8h_kernel(const A
         if constexpr (SEL) {
             uint32_t id[4];
             size_t unused[4];
-            listed_blocks(sel, n_sel, bt, pg, pos, page_bytes, head_off, kRow, id, unused);
+            listed_blocks(sel, n_sel, (uint32_t)P.max_ids, bt, pg, pos, page_bytes, head_off, kRow, id, unused);
             const uint32_t mine = pick4(id, g);
 #pragma unroll
             for (int r = 0; r < 4; ++r) live[r] = block_cell_live(mine, r, pos);
@@ -907,17 +910,14 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
     const auto unit_src = [&](int i, bool is_k, UnitSrc<SEL>& u) {
         const uint8_t* pool = is_k ? P.kpool : P.vpool;
         if constexpr (SEL) {
-            if (i < n_steps) {
-                uint32_t id[4];
-                size_t off[4];
-                listed_blocks(sel, n_sel, bt, pg0 + wave + kWaves * i, pos, is_k ? k_page_bytes : v_page_bytes,
-                              is_k ? k_head_off : v_head_off, is_k ? kHd * 2 : kQ8vRow, id, off);
+            // whatever the step, listed or past the list's end: every address is clamped to the sequence's
+            // own blocks, and nothing here waits for the list's length
+            uint32_t id[4];
+            size_t off[4];
+            listed_blocks(sel, n_sel, (uint32_t)P.max_ids, bt, pg0 + wave + kWaves * i, pos, is_k ? k_page_bytes : v_page_bytes,
+                          is_k ? k_head_off : v_head_off, is_k ? kHd * 2 : kQ8vRow, id, off);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) u.run[j] = pool + off[j];
-            } else {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) u.run[j] = pool;
-            }
+            for (int j = 0; j < 4; ++j) u.run[j] = pool + off[j];
         } else {
             u.run[0] = n_steps > 0 ? pool + phys(i) * (is_k ? k_page_bytes : v_page_bytes) + (is_k ? k_head_off : v_head_off)
                                    : pool;
@@ -944,7 +944,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
     // while the page before is multiplied
     v4u kf[8];
     Q8vUnitRegs v_regs;
-    if (n_steps > 0) {
+    if (SEL || n_steps > 0) {  // a selection list's first units before its length is known
         UnitSrc<SEL> u;
         const uint8_t *lo, *hi;
         unit_src(0, true, u);
@@ -1076,7 +1076,7 @@ __global__ __launch_bounds__(kBlock, 2) void decode_attn_mfma_q8v_kernel(const A
         if constexpr (SEL) {
             uint32_t id[4];
             size_t unused[4];
-            listed_blocks(sel, n_sel, bt, pg, pos, k_page_bytes, k_head_off, kHd * 2, id, unused);
+            listed_blocks(sel, n_sel, (uint32_t)P.max_ids, bt, pg, pos, k_page_bytes, k_head_off, kHd * 2, id, unused);
             const uint32_t mine = pick4(id, g);
 #pragma unroll
             for (int r = 0; r < 4; ++r) live[r] = block_cell_live(mine, r, pos);
